@@ -1,0 +1,275 @@
+/*
+ * mi355x_kmeans.h - C ABI of libmi355x_kmeans.so (HIP kernels for gfx950).
+ *
+ * One entry point per kernel family of the reference KMeans engine
+ * (soda-inria/sklearn-numba-dpex).  The reference has no FFI of its own: its kernels are
+ * numba_dpex JIT functions created by `make_*` factories and launched from
+ * sklearn_numba_dpex/kmeans/drivers.py.  Each declaration below cites the factory or driver
+ * code it replaces (paths relative to the reference's sklearn_numba_dpex/ directory).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless its name ends in `_host`.
+ *   - Data layout is the reference's: X_t is (n_features, n_samples) row-major, centroids_t
+ *     is (n_features, n_clusters) row-major (kmeans/drivers.py:43-53, kmeans/engine.py:88-98).
+ *   - `dtype`: KMX_F32 or KMX_F64, the type of every `void*` floating array of the call.
+ *   - Labels are uint32, kmeans++ indices int32, top-k indices int64 (as in the reference).
+ *   - Outputs and workspaces are allocated by the caller; `*_workspace_bytes` give sizes.
+ *     No entry point allocates or frees device memory.
+ *   - `stream` is a hipStream_t (NULL = default stream).  Calls only enqueue work; none
+ *     synchronises except kmx_lloyd_status_read.
+ *   - Return value: 0 on success, a negative KMX_ERR_* for rejected arguments, or a positive
+ *     hipError_t reported by the runtime.  Nothing throws or exits.
+ *   - Calls that share a workspace must be issued on one stream (or otherwise ordered).
+ */
+#ifndef MI355X_KMEANS_H
+#define MI355X_KMEANS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KMX_F32 0
+#define KMX_F64 1
+
+#define KMX_OK 0
+#define KMX_ERR_NULL_POINTER (-1)
+#define KMX_ERR_BAD_SHAPE (-2)      /* n, d, k, rows, cols <= 0 or inconsistent            */
+#define KMX_ERR_BAD_DTYPE (-3)
+#define KMX_ERR_WORKSPACE (-4)      /* workspace smaller than *_workspace_bytes()          */
+#define KMX_ERR_BAD_ARGUMENT (-5)   /* k > n for top-k, unknown op code, ...               */
+#define KMX_ERR_UNSUPPORTED (-6)    /* shape outside what a specialised kernel covers      */
+
+#define KMX_ABI_VERSION 1
+int32_t kmx_abi_version(void);
+const char* kmx_error_string(int32_t code);
+
+/* ------------------------------------------------------------------------------------ *
+ * Lloyd iteration                                                                       *
+ * ------------------------------------------------------------------------------------ */
+
+/* Loop state kept on the device (first bytes of the Lloyd workspace). */
+#define KMX_RUNNING 0
+#define KMX_CONVERGED_STRICT 1   /* no label changed between two successive iterations  */
+#define KMX_CONVERGED_TOL 2      /* shift_sum <= tol                                    */
+#define KMX_MAX_ITER 3
+#define KMX_NEED_RELOCATION 4    /* empty clusters found: host must relocate + finalize */
+
+typedef struct kmx_lloyd_status {
+    int32_t n_iter;       /* iterations completed                                          */
+    int32_t state;        /* KMX_RUNNING ...                                               */
+    int32_t n_empty;      /* empty clusters found by the last reduction                    */
+    uint32_t n_changed;   /* labels that differ from the previous iteration's              */
+    double shift_sum;     /* sum_c ||old_c - new_c||^2 of the last finalised iteration     */
+    double tol;           /* loop runs while shift_sum > tol                               */
+    int32_t max_iter;
+    uint32_t ticket;      /* internal: block counter of the reduction kernel               */
+    double max_sq_dist;   /* scratch for the relocation guard                              */
+    int64_t reserved[2];
+} kmx_lloyd_status;       /* 64 bytes */
+
+size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype);
+
+/* Resets the loop state, packs the initial centroids (+ their half squared norms) and
+ * clears the accumulators.  Replaces the set-up part of lloyd(), kmeans/drivers.py:146-184. */
+int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* centroids_t,
+                       int64_t n, int32_t d, int32_t k, int32_t dtype, int32_t max_iter,
+                       double tol, void* stream);
+
+/* One Lloyd iteration, enqueued as two kernels:
+ *   (1) fused step: pseudo distances 0.5||c||^2 - <x,c>, argmin (lowest index wins ties),
+ *       label write, changed-label count, per-workgroup partial sums of w*x and w;
+ *   (2) reduction of the partial sums, empty-cluster list (ascending), and - when no cluster
+ *       is empty - division by the cluster sizes, centroid shift and convergence test.
+ * Does nothing if the state is not KMX_RUNNING, so iterations may be enqueued ahead of the
+ * host's next look at the status.
+ * Replaces make_lloyd_single_step_fixed_window_kernel (kmeans/kernels/lloyd_single_step.py:35-424),
+ * make_reduce_centroid_data_kernel (kmeans/kernels/utils.py:113-195),
+ * make_half_l2_norm_2d_axis0_kernel, make_initialize_to_zeros_kernel,
+ * make_broadcast_division_1d_2d_axis0_kernel (common/kernels.py:38-145),
+ * make_centroid_shifts_kernel (kmeans/kernels/utils.py:79-110) and the loop body of
+ * lloyd(), kmeans/drivers.py:188-343.
+ *   centroids_t      IN   (d, k)  centroids the labels are computed from
+ *   new_centroids_t  OUT  (d, k)  un-normalised sums if relocation is needed, else new centroids
+ *   labels_prev      IN   (n)     labels of the previous iteration
+ *   labels           OUT  (n)
+ *   cluster_sizes    OUT  (k)     sum of weights per cluster
+ *   empty_clusters   OUT  (k)     ids of empty clusters, ascending, first status.n_empty valid */
+int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* centroids_t,
+                       void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                       void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                       size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                       void* stream);
+
+/* Second half of (2) alone, for the iteration that stopped with KMX_NEED_RELOCATION after
+ * the host has relocated the empty clusters: sums / sizes, shift, convergence test, state
+ * back to KMX_RUNNING (or a terminal state).  kmeans/drivers.py:275,326-343. */
+int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t, const void* cluster_sizes,
+                           void* workspace, size_t workspace_bytes, int32_t d, int32_t k,
+                           int32_t dtype, void* stream);
+
+/* Copies the status to host memory and waits for it (the only synchronising call). */
+int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
+
+/* Which fused-step kernel kmx_lloyd_iter would use for a shape: 0 = generic streaming,
+ * 1 = register-resident samples with LDS accumulators, 2 = register-resident samples with
+ * global accumulators, 3 = MFMA (fp32) with LDS accumulators. */
+int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype);
+
+/* ------------------------------------------------------------------------------------ *
+ * Labels, inertia, distances                                                            *
+ * ------------------------------------------------------------------------------------ */
+
+size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype);
+
+/* labels[i] = argmin_c (0.5||c||^2 - <x_i, c>).  Replaces
+ * make_label_assignment_fixed_window_kernel (kmeans/kernels/compute_labels.py:18-185) and the
+ * half-norm call before it (kmeans/drivers.py:657-669). */
+int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
+                          void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
+                          int32_t k, int32_t dtype, void* stream);
+
+/* out[i] = w_i * sum_f (x_fi - c_f,label_i)^2, features in order; sample_weight may be NULL
+ * for unit weights (the relocation pass).  Replaces make_compute_inertia_kernel
+ * (kmeans/kernels/compute_inertia.py:8-42). */
+int32_t kmx_per_sample_inertia(const void* X_t, const void* sample_weight, const void* centroids_t,
+                               const uint32_t* labels, void* out, int64_t n, int32_t d,
+                               int32_t k, int32_t dtype, void* stream);
+
+/* distances_t (k, n): sqrt(sum_f (c_f - x_f)^2).  Replaces
+ * make_compute_euclidean_distances_fixed_window_kernel
+ * (kmeans/kernels/compute_euclidean_distances.py:15-161). */
+int32_t kmx_euclidean_distances(const void* X_t, const void* centroids_t, void* distances_t,
+                                int64_t n, int32_t d, int32_t k, int32_t dtype, void* stream);
+
+/* Moves each listed empty cluster onto a far sample, on the un-normalised sums:
+ * sums[:, old] -= w*x, sums[:, empty] = w*x, sizes likewise; per_sample_inertia (may be NULL)
+ * of the moved sample is zeroed.  Replaces make_relocate_empty_clusters_kernel
+ * (kmeans/kernels/utils.py:11-76). */
+int32_t kmx_relocate_empty_clusters(const void* X_t, const void* sample_weight,
+                                    const uint32_t* labels, const int64_t* far_samples,
+                                    const uint32_t* empty_clusters, int32_t n_relocated,
+                                    void* per_sample_inertia, void* sums_t, void* cluster_sizes,
+                                    int64_t n, int32_t d, int32_t k, int32_t dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------ *
+ * kmeans++ seeding                                                                      *
+ * ------------------------------------------------------------------------------------ */
+
+size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype);
+
+/* closest[i] = w_i ||x_i - x_start||^2, centers_t[:, 0] = x_start, center_indices[0] = start,
+ * and the per-block partial potentials.  Replaces make_kmeansplusplus_init_kernel
+ * (kmeans/kernels/kmeans_plusplus.py:16-58) + the potential reduction (kmeans/drivers.py:844). */
+int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_index,
+                     void* centers_t, int32_t* center_indices, void* workspace,
+                     size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                     int32_t dtype, void* stream);
+
+/* Candidate t = first j with (inclusive fp64 scan of closest)_j >= uniforms[t] * total,
+ * clipped to [0, n-1].  Replaces make_sample_center_candidates_kernel
+ * (kmeans/kernels/kmeans_plusplus.py:61-103), whose serial scan becomes a two-level search
+ * over the block potentials already held in the workspace.
+ *   uniforms_for_step  IN  (n_trials) doubles in [0, 1)
+ *   candidates         OUT (n_trials) int32, may be NULL (they stay in the workspace) */
+int32_t kmx_kpp_sample_candidates(const double* uniforms_for_step, int32_t* candidates,
+                                  void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
+                                  int32_t k, int32_t n_trials, int32_t dtype, void* stream);
+
+/* For every candidate t and sample i: min(w_i ||x_i - x_cand_t||^2, closest_i), row sums,
+ * argmin over t (lowest t wins ties), closest <- best row, centers_t[:, c] <- x_best,
+ * center_indices[c] <- best candidate.  Replaces
+ * make_kmeansplusplus_single_step_fixed_window_kernel (kmeans/kernels/kmeans_plusplus.py:106-262),
+ * the axis-1 sum and argmin reductions (common/reductions.py) and kmeans/drivers.py:886-908. */
+int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_slot,
+                     void* centers_t, int32_t* center_indices, void* workspace,
+                     size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                     int32_t dtype, void* stream);
+
+/* The whole seeding (init, then k-1 x [sample, step]) with no host round trip.
+ *   uniforms  IN (k-1, n_trials) doubles: row c-1 holds what trial t draws for centre c.
+ * Replaces kmeans_plusplus(), kmeans/drivers.py:735-910. */
+int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* uniforms,
+                    int32_t start_index, void* centers_t, int32_t* center_indices,
+                    void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
+                    int32_t n_trials, int32_t dtype, void* stream);
+
+/* Views into the kmeans++ workspace, for tests: closest (n) in `dtype`, potentials
+ * (n_trials) doubles of the last step, candidates (n_trials) int32. */
+void* kmx_kpp_closest_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype);
+double* kmx_kpp_potentials_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype);
+int32_t* kmx_kpp_candidates_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype);
+
+/* ------------------------------------------------------------------------------------ *
+ * Shared kernels (the reference's common/ directory)                                    *
+ * ------------------------------------------------------------------------------------ */
+
+size_t kmx_sum_workspace_bytes(int64_t rows, int64_t cols);
+
+/* out[r] = sum_c f(in[r, c]) with f = identity or square (first pass only).  Replaces
+ * make_sum_reduction_2d_kernel with axis=1 and the 1-D form (common/reductions.py:214-460,
+ * 643-890).  Accumulates in fp64, fixed order: results are reproducible run to run. */
+int32_t kmx_sum_rows(const void* in, void* out, int64_t rows, int64_t cols, int32_t square,
+                     void* workspace, size_t workspace_bytes, int32_t dtype, void* stream);
+
+/* out[c] = sum_r in[r, c].  Replaces the axis=0 form (common/reductions.py:462-640). */
+int32_t kmx_sum_cols(const void* in, void* out, int64_t rows, int64_t cols, void* workspace,
+                     size_t workspace_bytes, int32_t dtype, void* stream);
+
+/* out[0] = index of the smallest value, lowest index on ties.  Replaces
+ * make_argmin_reduction_1d_kernel (common/reductions.py:17-209). */
+int32_t kmx_argmin(const void* values, int32_t* out, int64_t n, int32_t dtype, void* stream);
+
+/* out[c] = (sum_f a[f, c]^2) / 2.  make_half_l2_norm_2d_axis0_kernel, common/kernels.py:116-145. */
+int32_t kmx_half_sq_norms(const void* a_t, void* out, int32_t rows, int32_t cols, int32_t dtype,
+                          void* stream);
+
+/* a[r, c] = a[r, c] (op) v[r], op 0 = minus, 1 = plus.
+ * make_broadcast_ops_1d_2d_axis1_kernel, common/kernels.py:85-113. */
+int32_t kmx_broadcast_rows(void* a, const void* v, int64_t rows, int64_t cols, int32_t op,
+                           int32_t dtype, void* stream);
+
+/* a[r, c] /= v[c].  make_broadcast_division_1d_2d_axis0_kernel, common/kernels.py:60-82. */
+int32_t kmx_broadcast_div_cols(void* a, const void* v, int64_t rows, int64_t cols, int32_t dtype,
+                               void* stream);
+
+/* data[i] = data[i] / divisor.  make_apply_elementwise_func with _divide_by,
+ * common/kernels.py:11-36, common/_utils.py:17-33. */
+int32_t kmx_divide_by(void* data, int64_t n_items, double divisor, int32_t dtype, void* stream);
+
+/* Zero fill.  make_initialize_to_zeros_kernel, common/kernels.py:38-57. */
+int32_t kmx_fill_zero(void* data, int64_t n_bytes, void* stream);
+
+/* out[c] = sum_f (a[f, c] - b[f, c])^2.  make_centroid_shifts_kernel, kmeans/kernels/utils.py:79-110. */
+int32_t kmx_centroid_shifts(const void* a_t, const void* b_t, void* out, int32_t d, int32_t k,
+                            int32_t dtype, void* stream);
+
+size_t kmx_topk_workspace_bytes(int64_t n, int32_t k);
+
+/* Indices of the k largest values of a 1-D array by radix select (8-bit digits, most
+ * significant first, on the order-preserving unsigned image of the floats), ordered by
+ * descending value then ascending index.  Replaces topk_idx for one row
+ * (common/topk.py:194-270, 273-527, 540-1123, 1250-1365). */
+int32_t kmx_topk_idx(const void* values, int64_t* out_indices, int64_t n, int32_t k,
+                     void* workspace, size_t workspace_bytes, int32_t dtype, void* stream);
+
+/* result[0] = 1 if the two labelings are equal up to a permutation of the labels, else 0.
+ * mapping: scratch of k int32.  make_is_same_clustering_kernel, kmeans/kernels/utils.py:198-253. */
+int32_t kmx_is_same_clustering(const uint32_t* labels1, const uint32_t* labels2, int32_t* mapping,
+                               int32_t* result, int64_t n, int32_t k, void* stream);
+
+/* result[0] = number of distinct labels.  seen: scratch of k int32.
+ * make_get_nb_distinct_clusters_kernel, kmeans/kernels/utils.py:256-279. */
+int32_t kmx_count_distinct_clusters(const uint32_t* labels, int32_t* seen, int32_t* result,
+                                    int64_t n, int32_t k, void* stream);
+
+/* out (m, q) = X (m, p) @ Y_t (q, p)^T.  make_matmul_2d_kernel, common/matmul.py:13-567. */
+int32_t kmx_matmul(const void* X, const void* Y_t, void* out, int32_t m, int32_t p, int32_t q,
+                   int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_KMEANS_H */

@@ -1,0 +1,150 @@
+"""ctypes binding of libmi355x_kmeans.so (declared in include/mi355x_kmeans.h).
+
+The library is the only compute path of this package: if it is missing, importing this
+module raises (there is no CPU or PyTorch fallback).  torch tensors are used strictly as
+device buffers: `ptr(t)` hands their address to the C ABI.
+"""
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_double, c_int32, c_int64, c_size_t, c_void_p
+
+import numpy as np
+
+KMX_F32 = 0
+KMX_F64 = 1
+
+KMX_RUNNING = 0
+KMX_CONVERGED_STRICT = 1
+KMX_CONVERGED_TOL = 2
+KMX_MAX_ITER = 3
+KMX_NEED_RELOCATION = 4
+
+ABI_VERSION = 1
+
+LIB_NAME = "libmi355x_kmeans.so"
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+
+
+class LloydStatus(ctypes.Structure):
+    """Mirror of kmx_lloyd_status."""
+
+    _fields_ = [
+        ("n_iter", c_int32),
+        ("state", c_int32),
+        ("n_empty", c_int32),
+        ("n_changed", ctypes.c_uint32),
+        ("shift_sum", c_double),
+        ("tol", c_double),
+        ("max_iter", c_int32),
+        ("ticket", ctypes.c_uint32),
+        ("max_sq_dist", c_double),
+        ("reserved", c_int64 * 2),
+    ]
+
+
+assert ctypes.sizeof(LloydStatus) == 64
+
+_P = c_void_p
+_I32 = c_int32
+_I64 = c_int64
+_SZ = c_size_t
+
+# name -> (restype, argtypes); must list every function of include/mi355x_kmeans.h
+SIGNATURES = {
+    "kmx_abi_version": (_I32, []),
+    "kmx_error_string": (c_char_p, [_I32]),
+    "kmx_lloyd_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32]),
+    "kmx_lloyd_init": (_I32, [_P, _SZ, _P, _I64, _I32, _I32, _I32, _I32, c_double, _P]),
+    "kmx_lloyd_iter": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
+    "kmx_lloyd_finalize": (_I32, [_P, _P, _P, _P, _SZ, _I32, _I32, _I32, _P]),
+    "kmx_lloyd_status_read": (_I32, [_P, POINTER(LloydStatus), _P]),
+    "kmx_lloyd_kernel_variant": (_I32, [_I64, _I32, _I32, _I32]),
+    "kmx_assign_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "kmx_assign_labels": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
+    "kmx_per_sample_inertia": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "kmx_euclidean_distances": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "kmx_relocate_empty_clusters": (_I32, [_P, _P, _P, _P, _P, _I32, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "kmx_kpp_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
+    "kmx_kpp_init": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
+    "kmx_kpp_sample_candidates": (_I32, [_P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
+    "kmx_kpp_step": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
+    "kmx_kpp_run": (_I32, [_P, _P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
+    "kmx_kpp_closest_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),
+    "kmx_kpp_potentials_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),
+    "kmx_kpp_candidates_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),
+    "kmx_sum_workspace_bytes": (_SZ, [_I64, _I64]),
+    "kmx_sum_rows": (_I32, [_P, _P, _I64, _I64, _I32, _P, _SZ, _I32, _P]),
+    "kmx_sum_cols": (_I32, [_P, _P, _I64, _I64, _P, _SZ, _I32, _P]),
+    "kmx_argmin": (_I32, [_P, _P, _I64, _I32, _P]),
+    "kmx_half_sq_norms": (_I32, [_P, _P, _I32, _I32, _I32, _P]),
+    "kmx_broadcast_rows": (_I32, [_P, _P, _I64, _I64, _I32, _I32, _P]),
+    "kmx_broadcast_div_cols": (_I32, [_P, _P, _I64, _I64, _I32, _P]),
+    "kmx_divide_by": (_I32, [_P, _I64, c_double, _I32, _P]),
+    "kmx_fill_zero": (_I32, [_P, _I64, _P]),
+    "kmx_centroid_shifts": (_I32, [_P, _P, _P, _I32, _I32, _I32, _P]),
+    "kmx_topk_workspace_bytes": (_SZ, [_I64, _I32]),
+    "kmx_topk_idx": (_I32, [_P, _P, _I64, _I32, _P, _SZ, _I32, _P]),
+    "kmx_is_same_clustering": (_I32, [_P, _P, _P, _P, _I64, _I32, _P]),
+    "kmx_count_distinct_clusters": (_I32, [_P, _P, _P, _I64, _I32, _P]),
+    "kmx_matmul": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _P]),
+}
+
+
+class KmxError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = code
+        super().__init__(f"{where} failed with code {code}: {error_string(code)}")
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python sklearn-numba-dpex_amd/_build.py` "
+            "(hipcc, gfx950).  This engine has no fallback path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.kmx_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_NAME} has ABI {lib.kmx_abi_version()}, expected {ABI_VERSION}")
+    return lib
+
+
+lib = _load()
+
+
+def error_string(code):
+    return lib.kmx_error_string(int(code)).decode()
+
+
+def check(code, where):
+    if code != 0:
+        raise KmxError(code, where)
+
+
+def dtype_code(dtype):
+    dtype = np.dtype(dtype) if not hasattr(dtype, "is_floating_point") else dtype
+    name = str(dtype).replace("torch.", "")
+    if name == "float32":
+        return KMX_F32
+    if name == "float64":
+        return KMX_F64
+    raise ValueError(f"unsupported dtype {dtype}; expected float32 or float64")
+
+
+def ptr(tensor):
+    """Device address of a torch tensor (None -> NULL).  The tensor must be contiguous."""
+    if tensor is None:
+        return None
+    if not tensor.is_contiguous():
+        raise ValueError("device buffers handed to the C ABI must be contiguous")
+    return tensor.data_ptr()
+
+
+def current_stream():
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream

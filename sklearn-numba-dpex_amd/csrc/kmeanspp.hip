@@ -1,0 +1,506 @@
+// kmeans++ seeding for gfx950, with no host round trip between centres.
+//
+// State lives in a caller-provided workspace:
+//   header      best row of the last step, total potential of that row
+//   candidates  2 x 16 int32 (two buffers so that a fused select+sample launch can read the
+//               previous candidates while it writes the next ones)
+//   potentials  16 doubles (row sums of the last step)
+//   block_pot   (n_blocks, 16) doubles: per-workgroup partial row sums; workgroup b owns the
+//               samples [b * 1024, (b + 1) * 1024), so these are also the coarse level of the
+//               sampler's two-level search
+//   rows        (n_trials, n) in the compute dtype: min(w * ||x - x_cand||^2, closest) for
+//               every candidate; `closest` IS the best row, updated in place: a thread reads
+//               closest[i] before it writes column i of every row.
+//
+// Per new centre: [select previous best + sample candidates] then [step].  The sampler is a
+// search in the fp64 inclusive scan of `closest`: coarse over the block sums, fine inside one
+// block of 1024 samples, so it never re-reads the whole array.
+#include "kmx_common.h"
+
+namespace {
+
+constexpr int TN_MAX = 16;      // n_local_trials = 2 + floor(ln k) <= 16 for k < 1.2e6
+constexpr int CHUNK = 1024;     // samples per workgroup (256 threads x 4)
+constexpr int FEAT_WINDOW = 128;
+
+struct KppHeader {
+    int32_t best_row;
+    int32_t pad;
+    double total;
+};
+
+struct KppLayout {
+    size_t off_header, off_cand, off_pot, off_block_pot, off_rows, total;
+    int64_t n_blocks;
+};
+
+KppLayout kpp_layout(int64_t n, int n_trials, int dtype) {
+    KppLayout L;
+    L.n_blocks = kmx_cdiv(n, CHUNK);
+    L.off_header = 0;
+    L.off_cand = 256;
+    L.off_pot = 512;
+    L.off_block_pot = 768;
+    L.off_rows = L.off_block_pot + kmx_align256((size_t)L.n_blocks * TN_MAX * sizeof(double));
+    L.total = L.off_rows + kmx_align256((size_t)n_trials * n * kmx_dtype_size(dtype));
+    return L;
+}
+
+// closest = w * ||x - x_start||^2 into row 0; per-block potential; slot 0 of the outputs.
+template <typename T>
+__global__ __launch_bounds__(256) void kpp_init_kernel(
+    const T* __restrict__ X_t, const T* __restrict__ sample_weight, int32_t start,
+    T* __restrict__ centers_t, int32_t* __restrict__ center_indices, T* __restrict__ rows,
+    double* __restrict__ block_pot, KppHeader* __restrict__ header, int64_t n, int d, int k) {
+    const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
+    T acc[4] = {T(0), T(0), T(0), T(0)};
+    for (int f = 0; f < d; ++f) {
+        const T* __restrict__ row = X_t + (size_t)f * n;
+        const T sv = row[start];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (i0 + r < n) {
+                const T diff = row[i0 + r] - sv;
+                acc[r] = fma(diff, diff, acc[r]);
+            }
+        }
+    }
+    double pot = 0.0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (i0 + r < n) {
+            const T v = acc[r] * sample_weight[i0 + r];
+            rows[i0 + r] = v;
+            pot += (double)v;
+        }
+    }
+    __shared__ double scratch[4];
+    const double tot = kmx_block_sum<double>(pot, scratch);
+    if (threadIdx.x == 0) block_pot[(size_t)blockIdx.x * TN_MAX] = tot;
+    if (blockIdx.x == 0) {
+        for (int f = threadIdx.x; f < d; f += 256) centers_t[(size_t)f * k] = X_t[(size_t)f * n + start];
+        if (threadIdx.x == 0) {
+            center_indices[0] = start;
+            header->best_row = 0;
+            header->total = 0.0;
+        }
+    }
+}
+
+// rows[t, i] = min(w_i * ||x_i - x_cand_t||^2, closest_i) and per-block row sums.
+template <typename T>
+__global__ __launch_bounds__(256) void kpp_step_kernel(
+    const T* __restrict__ X_t, const T* __restrict__ sample_weight,
+    const int32_t* __restrict__ candidates, T* __restrict__ rows, double* __restrict__ block_pot,
+    const KppHeader* __restrict__ header, int64_t n, int d, int n_trials, int vec_ok) {
+    __shared__ T cand[TN_MAX][FEAT_WINDOW];
+    __shared__ double scratch[4];
+    const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
+    const int best = header->best_row;
+
+    T acc[TN_MAX][4];
+#pragma unroll
+    for (int t = 0; t < TN_MAX; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[t][r] = T(0);
+
+    for (int f0 = 0; f0 < d; f0 += FEAT_WINDOW) {
+        const int fw = (d - f0 < FEAT_WINDOW) ? d - f0 : FEAT_WINDOW;
+        __syncthreads();
+        for (int j = threadIdx.x; j < n_trials * fw; j += 256) {
+            const int t = j / fw, f = j - t * fw;
+            cand[t][f] = X_t[(size_t)(f0 + f) * n + candidates[t]];
+        }
+        __syncthreads();
+        for (int f = 0; f < fw; ++f) {
+            const T* __restrict__ row = X_t + (size_t)(f0 + f) * n;
+            T xv[4];
+            if (vec_ok && i0 + 4 <= n) {
+                if constexpr (sizeof(T) == 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(row + i0);
+                    xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+                } else {
+                    const double2 a = *reinterpret_cast<const double2*>(row + i0);
+                    const double2 b = *reinterpret_cast<const double2*>(row + i0 + 2);
+                    xv[0] = a.x; xv[1] = a.y; xv[2] = b.x; xv[3] = b.y;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xv[r] = (i0 + r < n) ? row[i0 + r] : T(0);
+            }
+#pragma unroll
+            for (int t = 0; t < TN_MAX; ++t) {
+                if (t < n_trials) {
+                    const T cv = cand[t][f];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const T diff = xv[r] - cv;
+                        acc[t][r] = fma(diff, diff, acc[t][r]);
+                    }
+                }
+            }
+        }
+    }
+
+    T w[4], cl[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const bool ok = i0 + r < n;
+        w[r] = ok ? sample_weight[i0 + r] : T(0);
+        cl[r] = ok ? rows[(size_t)best * n + i0 + r] : T(0);
+    }
+#pragma unroll
+    for (int t = 0; t < TN_MAX; ++t) {
+        if (t < n_trials) {
+            double pot = 0.0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (i0 + r < n) {
+                    const T v = fmin(acc[t][r] * w[r], cl[r]);
+                    rows[(size_t)t * n + i0 + r] = v;
+                    pot += (double)v;
+                }
+            }
+            const double tot = kmx_block_sum<double>(pot, scratch);
+            if (threadIdx.x == 0) block_pot[(size_t)blockIdx.x * TN_MAX + t] = tot;
+        }
+    }
+}
+
+// Block-wide exclusive scan of one double per thread (256 threads); returns the exclusive
+// prefix of the calling thread and the block total.
+__device__ __forceinline__ double block_exclusive_scan(double v, double* wave_tot, double& total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    double incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const double o = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += o;
+    }
+    __syncthreads();
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    double base = 0.0;
+    for (int w2 = 0; w2 < wave; ++w2) base += wave_tot[w2];
+    total = wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+    return base + incl - v;
+}
+
+__device__ __forceinline__ int64_t block_min_i64(int64_t v, int64_t* scratch) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const int64_t o = __shfl_xor(v, off, 64);
+        v = o < v ? o : v;
+    }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    int64_t m = scratch[0];
+    for (int w2 = 1; w2 < 4; ++w2) m = scratch[w2] < m ? scratch[w2] : m;
+    return m;
+}
+
+// One workgroup per trial.
+//   do_select: sum the block potentials of every row of the last step, pick the best row
+//              (lowest index on ties); workgroup 0 records potentials, header, centre slot.
+//   do_sample: candidate t = first j with scan(closest)_j >= uniforms[t] * total.
+template <typename T>
+__global__ __launch_bounds__(256) void kpp_select_sample_kernel(
+    const T* __restrict__ X_t, const double* __restrict__ uniforms,
+    const int32_t* __restrict__ cand_prev, int32_t* __restrict__ cand_next,
+    int32_t* __restrict__ cand_out, T* __restrict__ centers_t,
+    int32_t* __restrict__ center_indices, const T* __restrict__ rows,
+    const double* __restrict__ block_pot, double* __restrict__ potentials,
+    KppHeader* __restrict__ header, int64_t n, int64_t n_blocks, int d, int k, int n_trials,
+    int center_slot, int do_select, int do_sample) {
+    __shared__ double wave_tot[4];
+    __shared__ double dscratch[4];
+    __shared__ int64_t iscratch[4];
+    __shared__ double pot_s[TN_MAX];
+    __shared__ double prefix_s;
+
+    int best = header->best_row;
+    if (do_select) {
+        for (int t = 0; t < n_trials; ++t) {
+            double acc = 0.0;
+            for (int64_t b = threadIdx.x; b < n_blocks; b += 256) acc += block_pot[(size_t)b * TN_MAX + t];
+            const double tot = kmx_block_sum<double>(acc, dscratch);
+            if (threadIdx.x == 0) pot_s[t] = tot;
+        }
+        __syncthreads();
+        best = 0;
+        for (int t = 1; t < n_trials; ++t)
+            if (pot_s[t] < pot_s[best]) best = t;
+        if (blockIdx.x == 0) {
+            const int32_t chosen = cand_prev[best];
+            for (int f = threadIdx.x; f < d; f += 256)
+                centers_t[(size_t)f * k + center_slot] = X_t[(size_t)f * n + chosen];
+            if (threadIdx.x == 0) {
+                for (int t = 0; t < n_trials; ++t) potentials[t] = pot_s[t];
+                center_indices[center_slot] = chosen;
+                header->best_row = best;
+                header->total = pot_s[best];
+            }
+        }
+    }
+    if (!do_sample) return;
+
+    const int trial = blockIdx.x;
+    // ---- coarse level: exclusive scan of the block sums of the best row
+    const int64_t per_thread = (n_blocks + 255) / 256;
+    const int64_t b0 = (int64_t)threadIdx.x * per_thread;
+    int64_t b1 = b0 + per_thread;
+    if (b1 > n_blocks) b1 = n_blocks;
+    double local = 0.0;
+    for (int64_t b = b0; b < b1; ++b) local += block_pot[(size_t)b * TN_MAX + best];
+    double total;
+    const double excl = block_exclusive_scan(local, wave_tot, total);
+    const double rv = uniforms[trial] * total;
+    int64_t found = INT64_MAX;
+    double cum = excl, found_prefix = 0.0;
+    for (int64_t b = b0; b < b1; ++b) {
+        const double before = cum;
+        cum += block_pot[(size_t)b * TN_MAX + best];
+        if (cum >= rv) {
+            found = b;
+            found_prefix = before;
+            break;
+        }
+    }
+    const int64_t bstar_raw = block_min_i64(found, iscratch);
+    const int64_t bstar = bstar_raw == INT64_MAX ? n_blocks - 1 : bstar_raw;
+    if (found == bstar_raw && found != INT64_MAX) prefix_s = found_prefix;
+    if (bstar_raw == INT64_MAX && threadIdx.x == 0) prefix_s = total;  // rounding: rv above every cum
+    __syncthreads();
+    const double prefix = prefix_s;
+
+    // ---- fine level: scan the 1024 samples of block bstar
+    const T* __restrict__ closest = rows + (size_t)best * n;
+    const int64_t j0 = bstar * CHUNK + threadIdx.x * 4;
+    double v[4], s = 0.0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        v[r] = (j0 + r < n) ? (double)closest[j0 + r] : 0.0;
+        s += v[r];
+    }
+    double tot2;
+    double c2 = prefix + block_exclusive_scan(s, wave_tot, tot2);
+    int64_t hit = INT64_MAX;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        c2 += v[r];
+        if (hit == INT64_MAX && j0 + r < n && c2 >= rv) hit = j0 + r;
+    }
+    int64_t cand = block_min_i64(hit, iscratch);
+    if (cand == INT64_MAX) {
+        cand = (bstar + 1) * CHUNK;  // rounding pushed the crossing just past this block
+    }
+    if (cand > n - 1) cand = n - 1;
+    if (threadIdx.x == 0) {
+        cand_next[trial] = (int32_t)cand;
+        if (cand_out) cand_out[trial] = (int32_t)cand;
+    }
+}
+
+struct KppPtrs {
+    KppHeader* header;
+    int32_t* cand;
+    double* potentials;
+    double* block_pot;
+    void* rows;
+};
+
+KppPtrs kpp_ptrs(char* ws, const KppLayout& L) {
+    KppPtrs p;
+    p.header = (KppHeader*)(ws + L.off_header);
+    p.cand = (int32_t*)(ws + L.off_cand);
+    p.potentials = (double*)(ws + L.off_pot);
+    p.block_pot = (double*)(ws + L.off_block_pot);
+    p.rows = ws + L.off_rows;
+    return p;
+}
+
+int32_t kpp_check(const void* X_t, const void* w, void* ws, size_t ws_bytes, int64_t n, int d, int k,
+                  int n_trials, int dtype) {
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(w);
+    KMX_REQUIRE_PTR(ws);
+    if (n <= 0 || d <= 0 || k <= 0 || n > INT32_MAX) return KMX_ERR_BAD_SHAPE;
+    if (n_trials <= 0 || n_trials > TN_MAX) return KMX_ERR_UNSUPPORTED;
+    KMX_REQUIRE_DTYPE(dtype);
+    if (ws_bytes < kpp_layout(n, n_trials, dtype).total) return KMX_ERR_WORKSPACE;
+    return KMX_OK;
+}
+
+template <typename T>
+void launch_init(const void* X_t, const void* w, int32_t start, void* centers_t, int32_t* idx,
+                 const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k, hipStream_t s) {
+    hipLaunchKernelGGL((kpp_init_kernel<T>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
+                       (const T*)X_t, (const T*)w, start, (T*)centers_t, idx, (T*)p.rows,
+                       p.block_pot, p.header, n, d, k);
+}
+
+template <typename T>
+void launch_step(const void* X_t, const void* w, const int32_t* cand, const KppPtrs& p,
+                 const KppLayout& L, int64_t n, int d, int n_trials, hipStream_t s) {
+    const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0);
+    hipLaunchKernelGGL((kpp_step_kernel<T>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
+                       (const T*)X_t, (const T*)w, cand, (T*)p.rows, p.block_pot, p.header, n, d,
+                       n_trials, vec_ok);
+}
+
+template <typename T>
+void launch_select_sample(const void* X_t, const double* uniforms, const int32_t* cand_prev,
+                          int32_t* cand_next, int32_t* cand_out, void* centers_t, int32_t* idx,
+                          const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k,
+                          int n_trials, int slot, int do_select, int do_sample, hipStream_t s) {
+    const unsigned grid = do_sample ? (unsigned)n_trials : 1u;
+    hipLaunchKernelGGL((kpp_select_sample_kernel<T>), dim3(grid), dim3(256), 0, s, (const T*)X_t,
+                       uniforms, cand_prev, cand_next, cand_out, (T*)centers_t, idx,
+                       (const T*)p.rows, p.block_pot, p.potentials, p.header, n, L.n_blocks, d, k,
+                       n_trials, slot, do_select, do_sample);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype) {
+    (void)d;
+    (void)k;
+    if (n <= 0 || n_trials <= 0 || n_trials > TN_MAX || (dtype != KMX_F32 && dtype != KMX_F64))
+        return 0;
+    return kpp_layout(n, n_trials, dtype).total;
+}
+
+int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_index,
+                     void* centers_t, int32_t* center_indices, void* workspace,
+                     size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                     int32_t dtype, void* stream_) {
+    const int32_t rc = kpp_check(X_t, sample_weight, workspace, workspace_bytes, n, d, k, n_trials, dtype);
+    if (rc != KMX_OK) return rc;
+    KMX_REQUIRE_PTR(centers_t);
+    KMX_REQUIRE_PTR(center_indices);
+    if (start_index < 0 || start_index >= n) return KMX_ERR_BAD_ARGUMENT;
+    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppPtrs p = kpp_ptrs((char*)workspace, L);
+    hipStream_t s = (hipStream_t)stream_;
+    if (dtype == KMX_F32)
+        launch_init<float>(X_t, sample_weight, start_index, centers_t, center_indices, p, L, n, d, k, s);
+    else
+        launch_init<double>(X_t, sample_weight, start_index, centers_t, center_indices, p, L, n, d, k, s);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+int32_t kmx_kpp_sample_candidates(const double* uniforms_for_step, int32_t* candidates,
+                                  void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
+                                  int32_t k, int32_t n_trials, int32_t dtype, void* stream_) {
+    KMX_REQUIRE_PTR(uniforms_for_step);
+    const int32_t rc = kpp_check(uniforms_for_step, uniforms_for_step, workspace, workspace_bytes, n, d, k, n_trials, dtype);
+    if (rc != KMX_OK) return rc;
+    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppPtrs p = kpp_ptrs((char*)workspace, L);
+    hipStream_t s = (hipStream_t)stream_;
+    if (dtype == KMX_F32)
+        launch_select_sample<float>(nullptr, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
+                                    nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s);
+    else
+        launch_select_sample<double>(nullptr, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
+                                     nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_slot,
+                     void* centers_t, int32_t* center_indices, void* workspace,
+                     size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                     int32_t dtype, void* stream_) {
+    const int32_t rc = kpp_check(X_t, sample_weight, workspace, workspace_bytes, n, d, k, n_trials, dtype);
+    if (rc != KMX_OK) return rc;
+    KMX_REQUIRE_PTR(centers_t);
+    KMX_REQUIRE_PTR(center_indices);
+    if (center_slot < 1 || center_slot >= k) return KMX_ERR_BAD_ARGUMENT;
+    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppPtrs p = kpp_ptrs((char*)workspace, L);
+    hipStream_t s = (hipStream_t)stream_;
+    if (dtype == KMX_F32) {
+        launch_step<float>(X_t, sample_weight, p.cand, p, L, n, d, n_trials, s);
+        launch_select_sample<float>(X_t, nullptr, p.cand, nullptr, nullptr, centers_t, center_indices,
+                                    p, L, n, d, k, n_trials, center_slot, 1, 0, s);
+    } else {
+        launch_step<double>(X_t, sample_weight, p.cand, p, L, n, d, n_trials, s);
+        launch_select_sample<double>(X_t, nullptr, p.cand, nullptr, nullptr, centers_t,
+                                     center_indices, p, L, n, d, k, n_trials, center_slot, 1, 0, s);
+    }
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* uniforms,
+                    int32_t start_index, void* centers_t, int32_t* center_indices,
+                    void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
+                    int32_t n_trials, int32_t dtype, void* stream_) {
+    int32_t rc = kmx_kpp_init(X_t, sample_weight, start_index, centers_t, center_indices, workspace,
+                              workspace_bytes, n, d, k, n_trials, dtype, stream_);
+    if (rc != KMX_OK) return rc;
+    if (k == 1) return KMX_OK;
+    KMX_REQUIRE_PTR(uniforms);
+    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppPtrs p = kpp_ptrs((char*)workspace, L);
+    hipStream_t s = (hipStream_t)stream_;
+    for (int c = 1; c < k; ++c) {
+        // candidates alternate between two buffers: the fused launch reads the previous
+        // step's candidates (to record its winner) while it writes the next ones
+        int32_t* cand_prev = p.cand + ((c - 1) & 1) * TN_MAX;
+        int32_t* cand_next = p.cand + (c & 1) * TN_MAX;
+        const double* u = uniforms + (size_t)(c - 1) * n_trials;
+        const int do_select = c > 1 ? 1 : 0;
+        if (dtype == KMX_F32) {
+            launch_select_sample<float>(X_t, u, cand_prev, cand_next, nullptr, centers_t,
+                                        center_indices, p, L, n, d, k, n_trials, c - 1, do_select, 1, s);
+            launch_step<float>(X_t, sample_weight, cand_next, p, L, n, d, n_trials, s);
+        } else {
+            launch_select_sample<double>(X_t, u, cand_prev, cand_next, nullptr, centers_t,
+                                         center_indices, p, L, n, d, k, n_trials, c - 1, do_select, 1, s);
+            launch_step<double>(X_t, sample_weight, cand_next, p, L, n, d, n_trials, s);
+        }
+        KMX_LAUNCH_CHECK();
+    }
+    int32_t* cand_last = p.cand + ((k - 1) & 1) * TN_MAX;
+    if (dtype == KMX_F32)
+        launch_select_sample<float>(X_t, nullptr, cand_last, nullptr, nullptr, centers_t,
+                                    center_indices, p, L, n, d, k, n_trials, k - 1, 1, 0, s);
+    else
+        launch_select_sample<double>(X_t, nullptr, cand_last, nullptr, nullptr, centers_t,
+                                     center_indices, p, L, n, d, k, n_trials, k - 1, 1, 0, s);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+void* kmx_kpp_closest_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                          int32_t dtype) {
+    (void)d;
+    (void)k;
+    if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
+    // start of the rows; the caller adds best_row * n elements (best_row from the header)
+    return (char*)workspace + kpp_layout(n, n_trials, dtype).off_rows;
+}
+
+double* kmx_kpp_potentials_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                               int32_t dtype) {
+    (void)d;
+    (void)k;
+    if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
+    return (double*)((char*)workspace + kpp_layout(n, n_trials, dtype).off_pot);
+}
+
+int32_t* kmx_kpp_candidates_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
+                                int32_t dtype) {
+    (void)d;
+    (void)k;
+    if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
+    return (int32_t*)((char*)workspace + kpp_layout(n, n_trials, dtype).off_cand);
+}
+
+}  // extern "C"

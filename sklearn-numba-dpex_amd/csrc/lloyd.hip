@@ -1,0 +1,799 @@
+// Lloyd iteration for gfx950: fused assignment + partial centroid sums, reduction of the
+// partial sums with empty-cluster detection, and the finalisation (division, shift,
+// convergence test).  Public entry points are declared in include/mi355x_kmeans.h.
+//
+// Fused step, vector-ALU variants (this file):
+//   * "register" path: every thread keeps R samples (all features) in registers, read once
+//     from X_t with 128-bit loads; centroids come from a packed (k, dpad) copy through
+//     wave-uniform (scalar) loads, so the inner loop is one v_fma per (sample, feature,
+//     centroid) with the centroid value in an SGPR;
+//   * "streaming" path for wide samples: windows of 8 centroids, features re-read per window.
+// Partial sums of w*x and w go to LDS accumulators private to the workgroup (flushed once
+// per workgroup) when (d + 1) * k values fit, else to a few global copies with hardware
+// float atomics.  The MFMA variant for fp32 lives in lloyd_mfma.hip.
+#include "kmx_common.h"
+#include "lloyd_layout.h"
+
+namespace {
+
+template <typename T, int R>
+struct VecOf;
+template <>
+struct VecOf<float, 1> { using type = float; };
+template <>
+struct VecOf<float, 2> { using type = float2; };
+template <>
+struct VecOf<float, 4> { using type = float4; };
+template <>
+struct VecOf<double, 1> { using type = double; };
+template <>
+struct VecOf<double, 2> { using type = double2; };
+
+// R consecutive samples of one feature row; vector load when the row is aligned.
+template <typename T, int R>
+__device__ __forceinline__ void load_row(const T* __restrict__ row, int64_t i0, int64_t n,
+                                         bool vec_ok, T (&out)[R]) {
+    if (vec_ok && i0 + R <= n) {
+        using V = typename VecOf<T, R>::type;
+        union {
+            V v;
+            T s[R];
+        } u;
+        u.v = *reinterpret_cast<const V*>(row + i0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) out[r] = u.s[r];
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) out[r] = (i0 + r < n) ? row[i0 + r] : T(0);
+    }
+}
+
+constexpr int ACC_NONE = 0;    // labels only
+constexpr int ACC_LDS = 1;     // workgroup-private LDS accumulators, flushed to partial[block]
+constexpr int ACC_GLOBAL = 2;  // hardware float atomics into partial[block % n_copies]
+
+// ------------------------------------------------------------------------------------------
+// Register-resident fused step.
+// ------------------------------------------------------------------------------------------
+template <typename T, int DREG, int R, int ACC>
+__global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
+    const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cpack,
+    const T* __restrict__ half_norms, const uint32_t* __restrict__ labels_prev,
+    uint32_t* __restrict__ labels, T* __restrict__ partial, kmx_lloyd_status* __restrict__ status,
+    int64_t n, int d, int k, int dpad, int n_copies, int vec_ok) {
+    if (ACC != ACC_NONE && status->state != KMX_RUNNING) return;
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* acc = reinterpret_cast<T*>(smem_raw);
+    __shared__ unsigned int changed_block;
+    const int items = (d + 1) * k;
+    if (ACC == ACC_LDS) {
+        for (int j = threadIdx.x; j < items; j += 256) acc[j] = T(0);
+    }
+    if (threadIdx.x == 0) changed_block = 0;
+    __syncthreads();
+
+    T* gacc = (ACC == ACC_GLOBAL) ? partial + (size_t)(blockIdx.x % n_copies) * items : nullptr;
+    unsigned int changed = 0;
+    const int64_t tile_samples = 256 * R;
+    const int64_t n_tiles = (n + tile_samples - 1) / tile_samples;
+
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i0 = tile * tile_samples + (int64_t)threadIdx.x * R;
+        T x[DREG][R];
+#pragma unroll
+        for (int f = 0; f < DREG; ++f) {
+            if (f < d) {
+                load_row<T, R>(X_t + (size_t)f * n, i0, n, vec_ok != 0, x[f]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) x[f][r] = T(0);
+            }
+        }
+
+        T best[R];
+        uint32_t bi[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            best[r] = kmx_inf<T>();
+            bi[r] = 0;
+        }
+
+        for (int c = 0; c < k; ++c) {
+            const T* __restrict__ cp = cpack + (size_t)c * dpad;  // wave-uniform address
+            T dot[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) dot[r] = T(0);
+#pragma unroll
+            for (int f4 = 0; f4 < DREG / 4; ++f4) {
+                if (f4 * 4 < d) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const T cv = cp[f4 * 4 + j];
+#pragma unroll
+                        for (int r = 0; r < R; ++r) dot[r] = fma(x[f4 * 4 + j][r], cv, dot[r]);
+                    }
+                }
+            }
+            const T h = half_norms[c];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const T pd = h - dot[r];
+                if (pd < best[r]) {
+                    best[r] = pd;
+                    bi[r] = (uint32_t)c;
+                }
+            }
+        }
+
+        // labels, changed-label count and accumulation
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t i = i0 + r;
+            if (i < n) {
+                labels[i] = bi[r];
+                if (ACC != ACC_NONE) {
+                    changed += (labels_prev[i] != bi[r]) ? 1u : 0u;
+                    const T wr = sample_weight[i];
+                    T* dst = (ACC == ACC_LDS) ? acc : gacc;
+                    kmx_atomic_add(dst + (size_t)d * k + bi[r], wr);
+#pragma unroll
+                    for (int f = 0; f < DREG; ++f) {
+                        if (f < d) kmx_atomic_add(dst + (size_t)f * k + bi[r], x[f][r] * wr);
+                    }
+                }
+            }
+        }
+    }
+
+    if (ACC != ACC_NONE) {
+        if (changed) atomicAdd(&changed_block, changed);
+        __syncthreads();
+        if (ACC == ACC_LDS) {
+            T* out = partial + (size_t)blockIdx.x * items;
+            for (int j = threadIdx.x; j < items; j += 256) out[j] = acc[j];
+        }
+        if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Streaming fused step for wide samples: windows of KC centroids, features re-read per window.
+// ------------------------------------------------------------------------------------------
+template <typename T, int R, int KC, int ACC>
+__global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
+    const T* __restrict__ X_t, const T* __restrict__ sample_weight,
+    const T* __restrict__ centroids_t, const T* __restrict__ half_norms,
+    const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
+    T* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k,
+    int n_copies) {
+    if (ACC != ACC_NONE && status->state != KMX_RUNNING) return;
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* acc = reinterpret_cast<T*>(smem_raw);
+    __shared__ unsigned int changed_block;
+    const int items = (d + 1) * k;
+    if (ACC == ACC_LDS) {
+        for (int j = threadIdx.x; j < items; j += 256) acc[j] = T(0);
+    }
+    if (threadIdx.x == 0) changed_block = 0;
+    __syncthreads();
+
+    T* gacc = (ACC == ACC_GLOBAL) ? partial + (size_t)(blockIdx.x % n_copies) * items : nullptr;
+    unsigned int changed = 0;
+    const int64_t tile_samples = 256 * R;
+    const int64_t n_tiles = (n + tile_samples - 1) / tile_samples;
+
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        int64_t idx[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) idx[r] = tile * tile_samples + r * 256 + threadIdx.x;
+
+        T best[R];
+        uint32_t bi[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            best[r] = kmx_inf<T>();
+            bi[r] = 0;
+        }
+
+        for (int c0 = 0; c0 < k; c0 += KC) {
+            T dot[R][KC];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int j = 0; j < KC; ++j) dot[r][j] = T(0);
+            for (int f = 0; f < d; ++f) {
+                T xv[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) xv[r] = (idx[r] < n) ? X_t[(size_t)f * n + idx[r]] : T(0);
+                const T* __restrict__ crow = centroids_t + (size_t)f * k;  // wave-uniform
+#pragma unroll
+                for (int j = 0; j < KC; ++j) {
+                    const int c = (c0 + j < k) ? c0 + j : k - 1;
+                    const T cv = crow[c];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) dot[r][j] = fma(xv[r], cv, dot[r][j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < KC; ++j) {
+                if (c0 + j < k) {
+                    const T h = half_norms[c0 + j];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const T pd = h - dot[r][j];
+                        if (pd < best[r]) {
+                            best[r] = pd;
+                            bi[r] = (uint32_t)(c0 + j);
+                        }
+                    }
+                }
+            }
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t i = idx[r];
+            if (i < n) {
+                labels[i] = bi[r];
+                if (ACC != ACC_NONE) {
+                    changed += (labels_prev[i] != bi[r]) ? 1u : 0u;
+                    const T wr = sample_weight[i];
+                    T* dst = (ACC == ACC_LDS) ? acc : gacc;
+                    kmx_atomic_add(dst + (size_t)d * k + bi[r], wr);
+                    for (int f = 0; f < d; ++f)
+                        kmx_atomic_add(dst + (size_t)f * k + bi[r], X_t[(size_t)f * n + i] * wr);
+                }
+            }
+        }
+    }
+
+    if (ACC != ACC_NONE) {
+        if (changed) atomicAdd(&changed_block, changed);
+        __syncthreads();
+        if (ACC == ACC_LDS) {
+            T* out = partial + (size_t)blockIdx.x * items;
+            for (int j = threadIdx.x; j < items; j += 256) out[j] = acc[j];
+        }
+        if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Reduction of the partial copies.  Block = 32 items x 8 copy lanes.  The last block to
+// finish lists the empty clusters in ascending order and finds the heaviest cluster.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void lloyd_reduce_kernel(
+    T* __restrict__ partial, int n_partials, int clear_partials, T* __restrict__ sums_t,
+    T* __restrict__ sizes, uint32_t* __restrict__ empty_clusters,
+    kmx_lloyd_status* __restrict__ status, int d, int k) {
+    if (status->state != KMX_RUNNING) return;
+    const int items = (d + 1) * k;
+    const int it = threadIdx.x & 31;
+    const int cl = threadIdx.x >> 5;
+    const int item = blockIdx.x * 32 + it;
+    __shared__ T red[8][32];
+    T s = T(0);
+    if (item < items) {
+        for (int g = cl; g < n_partials; g += 8) {
+            T* p = partial + (size_t)g * items + item;
+            s += *p;
+            if (clear_partials) *p = T(0);
+        }
+    }
+    red[cl][it] = s;
+    __syncthreads();
+    if (cl == 0 && item < items) {
+        T tot = red[0][it];
+#pragma unroll
+        for (int j = 1; j < 8; ++j) tot += red[j][it];
+        if (item < d * k)
+            sums_t[item] = tot;
+        else
+            sizes[item - d * k] = tot;
+    }
+
+    // ---- last block: empty-cluster list + heaviest cluster
+    __shared__ unsigned int is_last;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned int t = atomicAdd(&status->ticket, 1u);
+        is_last = (t == gridDim.x - 1) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+
+    __shared__ int wave_counts[4];
+    __shared__ T hv_val[4];
+    __shared__ int hv_idx[4];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    int base = 0;
+    T my_max = -kmx_inf<T>();
+    int my_arg = 0x7fffffff;
+    for (int c0 = 0; c0 < k; c0 += 256) {
+        const int c = c0 + threadIdx.x;
+        T sz = T(1);
+        if (c < k) {
+            sz = __builtin_nontemporal_load(sizes + c);
+            if (sz > my_max) {
+                my_max = sz;
+                my_arg = c;
+            }
+        }
+        const bool flag = (c < k) && (sz == T(0));
+        const unsigned long long mask = __ballot(flag);
+        const int prefix = __popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_counts[wave] = __popcll(mask);
+        __syncthreads();
+        int offset = base;
+        for (int w2 = 0; w2 < wave; ++w2) offset += wave_counts[w2];
+        if (flag) empty_clusters[offset + prefix] = (uint32_t)c;
+        base += wave_counts[0] + wave_counts[1] + wave_counts[2] + wave_counts[3];
+        __syncthreads();
+    }
+    // heaviest cluster, lowest index on ties
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const T ov = __shfl_xor(my_max, off, 64);
+        const int oi = __shfl_xor(my_arg, off, 64);
+        if (ov > my_max || (ov == my_max && oi < my_arg)) {
+            my_max = ov;
+            my_arg = oi;
+        }
+    }
+    if (lane == 0) {
+        hv_val[wave] = my_max;
+        hv_idx[wave] = my_arg;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T bv = hv_val[0];
+        int bidx = hv_idx[0];
+        for (int w2 = 1; w2 < 4; ++w2) {
+            if (hv_val[w2] > bv || (hv_val[w2] == bv && hv_idx[w2] < bidx)) {
+                bv = hv_val[w2];
+                bidx = hv_idx[w2];
+            }
+        }
+        status->reserved[0] = bidx;
+        status->n_empty = base;
+        status->ticket = 0;
+        if (base > 0) status->state = KMX_NEED_RELOCATION;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Finalisation: one thread per cluster, features in order (division, packed copy, half
+// squared norm, squared shift); the last block sums the per-block shifts in block order and
+// runs the convergence test.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void lloyd_finalize_kernel(
+    const T* __restrict__ old_centroids_t, T* __restrict__ new_centroids_t,
+    const T* __restrict__ sizes, T* __restrict__ cpack, T* __restrict__ half_norms,
+    double* __restrict__ shift_partial, kmx_lloyd_status* __restrict__ status, int d, int k,
+    int dpad, int force) {
+    const int state = status->state;
+    if (force ? (state != KMX_NEED_RELOCATION && state != KMX_RUNNING) : (state != KMX_RUNNING))
+        return;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    double shift = 0.0;
+    if (c < k) {
+        const T sz = sizes[c];
+        if (sz != T(0)) {
+            T sq = T(0), sh = T(0);
+#pragma unroll 4
+            for (int f = 0; f < d; ++f) {
+                const T nv = new_centroids_t[(size_t)f * k + c] / sz;
+                const T df = old_centroids_t[(size_t)f * k + c] - nv;
+                sh += df * df;
+                sq += nv * nv;
+                cpack[(size_t)c * dpad + f] = nv;
+                new_centroids_t[(size_t)f * k + c] = nv;
+            }
+            for (int f = d; f < dpad; ++f) cpack[(size_t)c * dpad + f] = T(0);
+            half_norms[c] = sq / T(2);
+            shift = (double)sh;
+        }
+    }
+    __shared__ double scratch[4];
+    const double block_shift = kmx_block_sum<double>(shift, scratch);
+    __shared__ unsigned int is_last;
+    if (threadIdx.x == 0) {
+        shift_partial[blockIdx.x] = block_shift;
+        __threadfence();
+        const unsigned int t = atomicAdd(&status->ticket, 1u);
+        is_last = (t == gridDim.x - 1) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+
+    // Clusters that are still empty (more clusters than distinct samples, so nothing could
+    // be relocated) are parked on the finished centroid of the heaviest cluster.
+    double parked_shift = 0.0;
+    if (status->n_empty > 0) {
+        const int heaviest = (int)status->reserved[0];
+        for (int c2 = threadIdx.x; c2 < k; c2 += 256) {
+            if (sizes[c2] == T(0)) {
+                T sq = T(0), sh = T(0);
+                for (int f = 0; f < d; ++f) {
+                    const T nv = __builtin_nontemporal_load(cpack + (size_t)heaviest * dpad + f);
+                    const T df = old_centroids_t[(size_t)f * k + c2] - nv;
+                    sh += df * df;
+                    sq += nv * nv;
+                    cpack[(size_t)c2 * dpad + f] = nv;
+                    new_centroids_t[(size_t)f * k + c2] = nv;
+                }
+                for (int f = d; f < dpad; ++f) cpack[(size_t)c2 * dpad + f] = T(0);
+                half_norms[c2] = sq / T(2);
+                parked_shift += (double)sh;
+            }
+        }
+    }
+    parked_shift = kmx_block_sum<double>(parked_shift, scratch);
+    if (threadIdx.x == 0) {
+        double total = parked_shift;
+        for (unsigned int b = 0; b < gridDim.x; ++b)
+            total += __builtin_nontemporal_load(shift_partial + b);
+        const int n_iter = status->n_iter + 1;
+        const unsigned int changed = status->n_changed;
+        status->n_iter = n_iter;
+        status->shift_sum = total;
+        status->n_changed = 0;
+        status->ticket = 0;
+        int next = KMX_RUNNING;
+        if (n_iter > 1 && changed == 0)
+            next = KMX_CONVERGED_STRICT;
+        else if (!(total > status->tol))
+            next = KMX_CONVERGED_TOL;
+        else if (n_iter >= status->max_iter)
+            next = KMX_MAX_ITER;
+        status->state = next;
+        status->reserved[1] = (int64_t)changed;
+    }
+}
+
+// Packed (k, dpad) copy of the centroids + half squared norms; optional status reset.
+template <typename T>
+__global__ __launch_bounds__(256) void lloyd_pack_kernel(const T* __restrict__ centroids_t,
+                                                         T* __restrict__ cpack,
+                                                         T* __restrict__ half_norms,
+                                                         kmx_lloyd_status* __restrict__ status,
+                                                         int d, int k, int dpad, int max_iter,
+                                                         double tol) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c < k) {
+        T sq = T(0);
+        for (int f = 0; f < d; ++f) {
+            const T v = centroids_t[(size_t)f * k + c];
+            sq += v * v;
+            cpack[(size_t)c * dpad + f] = v;
+        }
+        for (int f = d; f < dpad; ++f) cpack[(size_t)c * dpad + f] = T(0);
+        half_norms[c] = sq / T(2);
+    }
+    if (status != nullptr && c == 0) {
+        status->n_iter = 0;
+        status->state = max_iter > 0 ? KMX_RUNNING : KMX_MAX_ITER;
+        status->n_empty = 0;
+        status->n_changed = 0;
+        status->shift_sum = __builtin_huge_val();
+        status->tol = tol;
+        status->max_iter = max_iter;
+        status->ticket = 0;
+        status->max_sq_dist = 0.0;
+        status->reserved[0] = 0;
+        status->reserved[1] = 0;
+    }
+}
+
+__global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += stride)
+        p[i] = 0u;
+}
+
+// ------------------------------------------------------------------------------------------
+// Host-side launchers
+// ------------------------------------------------------------------------------------------
+
+template <typename T, int DREG, int R, int ACC>
+void launch_reg(const LloydLayout& L, const void* X_t, const void* w, const T* cpack,
+                const T* half_norms, const uint32_t* labels_prev, uint32_t* labels, T* partial,
+                kmx_lloyd_status* status, int64_t n, int d, int k, int grid, hipStream_t stream) {
+    const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(T) : 0;
+    const int vec_ok = (n % R == 0) && (((uintptr_t)X_t) % (R * sizeof(T)) == 0);
+    hipLaunchKernelGGL((lloyd_fused_reg_kernel<T, DREG, R, ACC>), dim3(grid), dim3(256), lds, stream,
+                       (const T*)X_t, (const T*)w, cpack, half_norms, labels_prev, labels, partial,
+                       status, n, d, k, L.dpad, L.n_partials, vec_ok);
+}
+
+template <typename T, int ACC>
+void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
+                  const T* cpack, const T* half_norms, const uint32_t* labels_prev,
+                  uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
+                  hipStream_t stream) {
+    const int cus = kmx_num_cus();
+    if (L.variant == KMX_VARIANT_REGISTER) {
+        const int r = lloyd_reg_samples_per_thread(d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
+        int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
+        int grid = (int)(tiles < (int64_t)L.grid_cap(cus) ? tiles : L.grid_cap(cus));
+        if (grid < 1) grid = 1;
+#define KMX_REG_CASE(DR, RR)                                                                    \
+    launch_reg<T, DR, RR, ACC>(L, X_t, w, cpack, half_norms, labels_prev, labels, partial, status, \
+                               n, d, k, grid, stream)
+        if constexpr (sizeof(T) == 4) {
+            if (d <= 8)
+                KMX_REG_CASE(8, 4);
+            else if (d <= 16)
+                KMX_REG_CASE(16, 4);
+            else if (d <= 32)
+                KMX_REG_CASE(32, 2);
+            else
+                KMX_REG_CASE(64, 1);
+        } else {
+            if (d <= 8)
+                KMX_REG_CASE(8, 2);
+            else if (d <= 16)
+                KMX_REG_CASE(16, 2);
+            else
+                KMX_REG_CASE(32, 1);
+        }
+#undef KMX_REG_CASE
+    } else {
+        constexpr int R = 2, KC = 8;
+        int64_t tiles = kmx_cdiv(n, 256 * (int64_t)R);
+        int grid = (int)(tiles < (int64_t)L.grid_cap(cus) ? tiles : L.grid_cap(cus));
+        if (grid < 1) grid = 1;
+        const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(T) : 0;
+        hipLaunchKernelGGL((lloyd_fused_stream_kernel<T, R, KC, ACC>), dim3(grid), dim3(256), lds,
+                           stream, (const T*)X_t, (const T*)w, (const T*)centroids_t, half_norms,
+                           labels_prev, labels, partial, status, n, d, k, L.n_partials);
+    }
+}
+
+template <typename T>
+int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
+                        const void* centroids_t, void* new_centroids_t,
+                        const uint32_t* labels_prev, uint32_t* labels, void* sizes,
+                        uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
+                        hipStream_t stream) {
+    auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
+    T* cpack = reinterpret_cast<T*>(ws + L.off_cpack);
+    T* half_norms = reinterpret_cast<T*>(ws + L.off_half);
+    T* partial = reinterpret_cast<T*>(ws + L.off_partial);
+    double* shift_partial = reinterpret_cast<double*>(ws + L.off_shift);
+
+    int n_partials_used = L.n_partials;
+    if (L.acc_mode == ACC_LDS) {
+        launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
+                                 partial, status, n, d, k, stream);
+        const int r = (L.variant == KMX_VARIANT_REGISTER)
+                          ? lloyd_reg_samples_per_thread(d, sizeof(T) == 8 ? KMX_F64 : KMX_F32)
+                          : 2;
+        int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
+        const int cap = L.grid_cap(kmx_num_cus());
+        n_partials_used = (int)(tiles < cap ? tiles : cap);
+        if (n_partials_used < 1) n_partials_used = 1;
+    } else {
+        launch_fused<T, ACC_GLOBAL>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
+                                    partial, status, n, d, k, stream);
+    }
+    KMX_LAUNCH_CHECK();
+
+    const int items = (d + 1) * k;
+    hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)kmx_cdiv(items, 32)), dim3(256), 0,
+                       stream, partial, n_partials_used, L.acc_mode == ACC_GLOBAL ? 1 : 0,
+                       (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k);
+    KMX_LAUNCH_CHECK();
+    hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, 256)), dim3(256), 0,
+                       stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
+                       half_norms, shift_partial, status, d, k, L.dpad, 0);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------
+
+int32_t kmx_num_cus() {
+    static int32_t cached = 0;
+    if (cached > 0) return cached;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+        return 256;
+    cached = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    return cached;
+}
+
+extern "C" {
+
+int32_t kmx_abi_version(void) { return KMX_ABI_VERSION; }
+
+const char* kmx_error_string(int32_t code) {
+    switch (code) {
+        case KMX_OK: return "ok";
+        case KMX_ERR_NULL_POINTER: return "null pointer argument";
+        case KMX_ERR_BAD_SHAPE: return "invalid or inconsistent shape";
+        case KMX_ERR_BAD_DTYPE: return "dtype must be KMX_F32 (0) or KMX_F64 (1)";
+        case KMX_ERR_WORKSPACE: return "workspace too small";
+        case KMX_ERR_BAD_ARGUMENT: return "invalid argument";
+        case KMX_ERR_UNSUPPORTED: return "shape not supported by this kernel";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}
+
+size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype) {
+    if (n <= 0 || d <= 0 || k <= 0 || (dtype != KMX_F32 && dtype != KMX_F64)) return 0;
+    return lloyd_layout(n, d, k, dtype).total;
+}
+
+int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype) {
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    return L.variant * 10 + L.acc_mode;
+}
+
+int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* centroids_t, int64_t n,
+                       int32_t d, int32_t k, int32_t dtype, int32_t max_iter, double tol,
+                       void* stream_) {
+    KMX_REQUIRE_PTR(workspace);
+    KMX_REQUIRE_PTR(centroids_t);
+    if (n <= 0 || d <= 0 || k <= 0 || max_iter < 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    if (workspace_bytes < L.total) return KMX_ERR_WORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    char* ws = (char*)workspace;
+    auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
+    const unsigned grid = (unsigned)kmx_cdiv(k, 256);
+    if (dtype == KMX_F32)
+        hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
+                           (const float*)centroids_t, (float*)(ws + L.off_cpack),
+                           (float*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
+    else
+        hipLaunchKernelGGL((lloyd_pack_kernel<double>), dim3(grid), dim3(256), 0, stream,
+                           (const double*)centroids_t, (double*)(ws + L.off_cpack),
+                           (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
+    KMX_LAUNCH_CHECK();
+    if (L.acc_mode == ACC_GLOBAL) {
+        const size_t words = L.partial_bytes / 4;
+        hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1024), dim3(256), 0, stream,
+                           (uint32_t*)(ws + L.off_partial), words);
+        KMX_LAUNCH_CHECK();
+    }
+    return KMX_OK;
+}
+
+int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* centroids_t,
+                       void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                       void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                       size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                       void* stream_) {
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(sample_weight);
+    KMX_REQUIRE_PTR(centroids_t);
+    KMX_REQUIRE_PTR(new_centroids_t);
+    KMX_REQUIRE_PTR(labels_prev);
+    KMX_REQUIRE_PTR(labels);
+    KMX_REQUIRE_PTR(cluster_sizes);
+    KMX_REQUIRE_PTR(empty_clusters);
+    KMX_REQUIRE_PTR(workspace);
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    if (workspace_bytes < L.total) return KMX_ERR_WORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == KMX_F32) {
+        if (L.variant == KMX_VARIANT_MFMA)
+            return kmx_lloyd_iter_mfma_f32(L, X_t, sample_weight, centroids_t, new_centroids_t,
+                                           labels_prev, labels, cluster_sizes, empty_clusters,
+                                           (char*)workspace, n, d, k, stream);
+        return lloyd_iter_impl<float>(L, X_t, sample_weight, centroids_t, new_centroids_t,
+                                      labels_prev, labels, cluster_sizes, empty_clusters,
+                                      (char*)workspace, n, d, k, stream);
+    }
+    return lloyd_iter_impl<double>(L, X_t, sample_weight, centroids_t, new_centroids_t, labels_prev,
+                                   labels, cluster_sizes, empty_clusters, (char*)workspace, n, d, k,
+                                   stream);
+}
+
+int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,
+                           const void* cluster_sizes, void* workspace, size_t workspace_bytes,
+                           int32_t d, int32_t k, int32_t dtype, void* stream_) {
+    KMX_REQUIRE_PTR(centroids_t);
+    KMX_REQUIRE_PTR(new_centroids_t);
+    KMX_REQUIRE_PTR(cluster_sizes);
+    KMX_REQUIRE_PTR(workspace);
+    if (d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    // offsets of the status, packed centroids, half norms and shift slots do not depend on n
+    const LloydLayout L = lloyd_layout(1, d, k, dtype);
+    if (workspace_bytes < L.off_partial) return KMX_ERR_WORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    char* ws = (char*)workspace;
+    auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
+    double* shift_partial = reinterpret_cast<double*>(ws + L.off_shift);
+    const unsigned grid = (unsigned)kmx_cdiv(k, 256);
+    if (dtype == KMX_F32)
+        hipLaunchKernelGGL((lloyd_finalize_kernel<float>), dim3(grid), dim3(256), 0, stream,
+                           (const float*)centroids_t, (float*)new_centroids_t,
+                           (const float*)cluster_sizes, (float*)(ws + L.off_cpack),
+                           (float*)(ws + L.off_half), shift_partial, status, d, k, L.dpad, 1);
+    else
+        hipLaunchKernelGGL((lloyd_finalize_kernel<double>), dim3(grid), dim3(256), 0, stream,
+                           (const double*)centroids_t, (double*)new_centroids_t,
+                           (const double*)cluster_sizes, (double*)(ws + L.off_cpack),
+                           (double*)(ws + L.off_half), shift_partial, status, d, k, L.dpad, 1);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream_) {
+    KMX_REQUIRE_PTR(workspace);
+    KMX_REQUIRE_PTR(status_host);
+    hipStream_t stream = (hipStream_t)stream_;
+    hipError_t e = hipMemcpyAsync(status_host, workspace, sizeof(kmx_lloyd_status),
+                                  hipMemcpyDeviceToHost, stream);
+    if (e != hipSuccess) return (int32_t)e;
+    e = hipStreamSynchronize(stream);
+    return e == hipSuccess ? KMX_OK : (int32_t)e;
+}
+
+size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
+    if (d <= 0 || k <= 0 || (dtype != KMX_F32 && dtype != KMX_F64)) return 0;
+    return lloyd_layout(1, d, k, dtype).off_partial;
+}
+
+int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
+                          void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
+                          int32_t dtype, void* stream_) {
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(centroids_t);
+    KMX_REQUIRE_PTR(labels);
+    KMX_REQUIRE_PTR(workspace);
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    LloydLayout L = lloyd_layout(n, d, k, dtype);
+    if (workspace_bytes < L.off_partial) return KMX_ERR_WORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    char* ws = (char*)workspace;
+    const unsigned grid = (unsigned)kmx_cdiv(k, 256);
+    if (dtype == KMX_F32) {
+        hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
+                           (const float*)centroids_t, (float*)(ws + L.off_cpack),
+                           (float*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
+                           0.0);
+        KMX_LAUNCH_CHECK();
+        if (L.variant == KMX_VARIANT_MFMA)
+            return kmx_assign_labels_mfma_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
+        launch_fused<float, ACC_NONE>(L, X_t, nullptr, centroids_t, (const float*)(ws + L.off_cpack),
+                                      (const float*)(ws + L.off_half), nullptr, labels, nullptr,
+                                      nullptr, n, d, k, stream);
+    } else {
+        hipLaunchKernelGGL((lloyd_pack_kernel<double>), dim3(grid), dim3(256), 0, stream,
+                           (const double*)centroids_t, (double*)(ws + L.off_cpack),
+                           (double*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
+                           0.0);
+        KMX_LAUNCH_CHECK();
+        launch_fused<double, ACC_NONE>(L, X_t, nullptr, centroids_t,
+                                       (const double*)(ws + L.off_cpack),
+                                       (const double*)(ws + L.off_half), nullptr, labels, nullptr,
+                                       nullptr, n, d, k, stream);
+    }
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,115 @@
+"""GPU parity of the Lloyd path (fused step, reduction/finalisation, full run, labels,
+inertia) against the CPU oracle, through the C ABI and through the drivers."""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import datasets
+from oracle import kmeans as ok
+from tests._parity import RTOL, assert_centers_close, assert_labels_match
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, cuda):
+    import torch
+
+    return torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+
+
+def _small_configs():
+    return {
+        "C1": lambda: datasets.config1(n=100_000),
+        "C2": lambda: datasets.config2(n=200_000),
+        "C3": lambda: datasets.config3(n=20_000, d=256, k=1024),
+        "C3s": lambda: datasets.config3(n=30_001, d=70, k=50),
+        "C5": lambda: datasets.config5(n=100_000),
+        "odd": lambda: _odd_config(),
+    }
+
+
+def _odd_config():
+    """Ragged shapes: n not a multiple of anything, d = 3, k = 5, fp64."""
+    rng = np.random.default_rng(7)
+    X = rng.normal(size=(1237, 3))
+    init = X[rng.choice(1237, 5, replace=False)].copy()
+    return dict(X=X, init=init, sample_weight=rng.uniform(0.5, 2, 1237), k=5, max_iter=50, tol=0.0, name="odd")
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C5", "odd"])
+def test_single_iteration_through_c_abi(cuda, name):
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    cfg = _small_configs()[name]()
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    dc = _capi.dtype_code(X.dtype)
+    X_t = _dev(X.T, cuda)
+    w_d = _dev(w, cuda)
+    c_in = _dev(init.T, cuda)
+    c_out = torch.empty_like(c_in)
+    labels_prev = torch.zeros(n, dtype=torch.int32, device=cuda)
+    labels = torch.empty(n, dtype=torch.int32, device=cuda)
+    sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(c_in), n, d, k, dc, 100, 0.0, stream), "init")
+    _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
+                                   ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, dc, stream), "iter")
+    status = _capi.LloydStatus()
+    _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+
+    ref_labels = ok.assign_labels(X, init)
+    n_ties = assert_labels_match(labels.cpu().numpy(), ref_labels, X, init)
+    got_labels = labels.cpu().numpy().astype(np.int64)
+    sums, ref_sizes = ok.weighted_sums(X, w, got_labels, k)
+    n_empty = int(np.count_nonzero(ref_sizes == 0))
+    assert status.n_empty == n_empty
+    np.testing.assert_allclose(sizes.cpu().numpy(), ref_sizes, rtol=RTOL[X.dtype] * 10)
+    if n_empty:
+        assert status.state == _capi.KMX_NEED_RELOCATION
+        assert status.n_iter == 0
+        np.testing.assert_array_equal(empty.cpu().numpy()[:n_empty], np.flatnonzero(ref_sizes == 0))
+        got = c_out.cpu().numpy().T
+        assert_centers_close(got, sums, X.dtype, scale_rtol=RTOL[X.dtype] * 10)
+    else:
+        assert status.state == _capi.KMX_RUNNING
+        assert status.n_iter == 1
+        ref_centers = sums / ref_sizes[:, None]
+        assert_centers_close(c_out.cpu().numpy().T, ref_centers, X.dtype, scale_rtol=RTOL[X.dtype] * 10)
+        shift = float(np.sum((np.asarray(init, np.float64) - ref_centers.astype(np.float64)) ** 2))
+        assert status.shift_sum == pytest.approx(shift, rel=1e-4)
+        expected_changed = int(np.count_nonzero(got_labels != 0))
+        assert status.reserved[1] == expected_changed
+    print(f"{name}: near-tie label differences: {n_ties}")
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C5", "odd"])
+def test_full_lloyd_run_matches_oracle(cuda, name):
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    cfg = _small_configs()[name]()
+    if name == "C2":
+        cfg = datasets.config2(n=50_000)
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    max_iter = min(cfg["max_iter"], 30)
+    Xc = X - X.mean(axis=0).astype(X.dtype)
+    initc = init - X.mean(axis=0).astype(X.dtype)
+    tol = 0.0
+    labels, inertia, centers_t, n_iter = drivers.lloyd(
+        _dev(Xc.T, cuda), _dev(w, cuda), _dev(initc.T, cuda), False, max_iter=max_iter, tol=tol
+    )
+    ref_labels, ref_inertia, ref_centers, ref_n_iter = ok.lloyd(Xc, w, initc, max_iter=max_iter, tol=tol)
+    assert n_iter == ref_n_iter
+    centers = centers_t.cpu().numpy().T
+    # trajectories may separate at near-ties; allow a looser centroid bound after many iterations
+    assert_centers_close(centers, ref_centers, X.dtype, scale_rtol=max(RTOL[X.dtype], 1e-9) * 50)
+    assert_labels_match(labels.cpu().numpy(), ref_labels, Xc, ref_centers)
+    assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-5)
