@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Lloyd throughput of the MI355X KMeans engine on one GPU.
+
+Workload (BASELINE.json configs[1]): fp32 X of shape 5,000,000 x 14 from 127 Gaussian blobs
+(seed 1), k = 127, random-row init, sample weights uniform in [0.5, 1.5], tol = 0.
+A "step" is one Lloyd iteration (fused assignment + partial sums, reduction, finalisation)
+with X, the weights and the centroids already resident in HBM.
+
+Prints ONE JSON line: iterations/s, plus
+  roofline      the fused-step kernel against the roofline that bounds it, from HIP events
+                recorded around that kernel on its stream (kmx_lloyd_iter_timed);
+  roofline_hbm  the same kernel against the HBM roofline;
+  cpu_baseline  scikit-learn's OpenMP/Cython Lloyd on the same data on this host's cores;
+  kmeanspp_ms   kmeans++ seeding time on configs[3] (1,000,000 x 64, k = 256).
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+FP32_PEAK_TFLOPS = 157.3    # MI355X fp32, vector and matrix
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def lloyd_bytes(n, d, s):
+    # read X once, read weight, read previous label, write new label
+    return n * (s * d + s + 4 + 4)
+
+
+def lloyd_flops(n, d, k):
+    return 2.0 * n * d * k + 2.0 * n * d
+
+
+def gpu_lloyd(cfg, steps, warmup):
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    dev = torch.device("cuda:0")
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    dc = _capi.dtype_code(X.dtype)
+    X_t = torch.as_tensor(X, device=dev).T.contiguous()
+    w_d = torch.as_tensor(w, device=dev)
+    cent = [torch.as_tensor(np.ascontiguousarray(init.T), device=dev), None]
+    cent[1] = torch.empty_like(cent[0])
+    labels = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(2)]
+    sizes = torch.empty(k, dtype=X_t.dtype, device=dev)
+    empty = torch.empty(k, dtype=torch.int32, device=dev)
+    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = _capi.current_stream()
+    status = _capi.LloydStatus()
+    total = warmup + 2 * steps + 8
+
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(cent[0]), n, d, k, dc, total, 0.0, stream), "init")
+    it = 0
+
+    def enqueue():
+        nonlocal it
+        a, b = it % 2, (it + 1) % 2
+        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k,
+                                       dc, stream), "iter")
+        it += 1
+
+    for _ in range(warmup):
+        enqueue()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        enqueue()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+    if status.n_iter != warmup + steps:
+        raise RuntimeError(
+            f"only {status.n_iter} of {warmup + steps} iterations did work (state {status.state}): "
+            "the timed region would include no-op launches"
+        )
+
+    # per-kernel durations from HIP events on the launch stream
+    ms = (ctypes.c_float * 3)()
+    acc = np.zeros(3)
+    timed = min(steps, 50)
+    for _ in range(timed):
+        a, b = it % 2, (it + 1) % 2
+        _capi.check(lib.kmx_lloyd_iter_timed(ptr(X_t), ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                             ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d,
+                                             k, dc, stream, ms), "iter_timed")
+        it += 1
+        acc += np.array(list(ms))
+    kernel_ms = acc / timed
+    _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+    if status.n_iter != warmup + steps + timed:
+        raise RuntimeError("timed iterations did not all run")
+
+    # parity gate: labels of the current state against the CPU oracle on a slice
+    from oracle import kmeans as ok
+    from tests._parity import assert_labels_match
+
+    cur = cent[it % 2].T.cpu().numpy()
+    lab = torch.empty(n, dtype=torch.int32, device=dev)
+    aws = lib.kmx_assign_workspace_bytes(d, k, dc)
+    aws_t = torch.empty(aws, dtype=torch.uint8, device=dev)
+    _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(X_t.new_tensor(cur.T.copy())), ptr(lab), ptr(aws_t), aws,
+                                      n, d, k, dc, stream), "assign")
+    m = min(n, 200_000)
+    ties = assert_labels_match(lab[:m].cpu().numpy(), ok.assign_labels(X[:m], cur), X[:m], cur)
+    variant = lib.kmx_lloyd_kernel_variant(n, d, k, dc)
+    return elapsed, kernel_ms, ties, variant
+
+
+def gpu_kmeanspp(cfg):
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    dev = torch.device("cuda:0")
+    X_t = torch.as_tensor(cfg["X"], device=dev).T.contiguous()
+    w = torch.as_tensor(cfg["sample_weight"], device=dev)
+    times = []
+    for rep in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        centers_t, idx = drivers.kmeans_plusplus(X_t, w, cfg["k"], np.random.RandomState(cfg["seed"]))
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    return float(np.median(times)), idx.cpu().numpy()
+
+
+def cpu_lloyd_baseline(cfg, max_iter):
+    """scikit-learn's Lloyd (OpenMP Cython) on the same data, inner routine only."""
+    from sklearn.cluster._kmeans import _kmeans_single_lloyd
+    from sklearn.utils._openmp_helpers import _openmp_effective_n_threads
+
+    X, init, w = cfg["X"], cfg["init"], cfg["sample_weight"]
+    threads = _openmp_effective_n_threads()
+    _kmeans_single_lloyd(X, w, init.copy(), max_iter=1, tol=0, n_threads=threads)  # warm-up
+    t0 = time.perf_counter()
+    _, _, _, n_iter = _kmeans_single_lloyd(X, w, init.copy(), max_iter=max_iter, tol=0, n_threads=threads)
+    elapsed = time.perf_counter() - t0
+    # the routine ends with one extra labelling pass; count it as the work it is
+    return n_iter / elapsed, threads, n_iter, elapsed
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--n", type=int, default=5_000_000, help="samples (default: the full configuration)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-kpp", action="store_true", help="skip the kmeans++ leg")
+    ap.add_argument("--cpu-iters", type=int, default=20)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    from oracle import datasets
+
+    t0 = time.time()
+    cfg = datasets.config2(n=args.n)
+    n, d = cfg["X"].shape
+    k = cfg["k"]
+    log(f"[bench] data {n}x{d} k={k} generated in {time.time() - t0:.1f}s")
+
+    elapsed, kernel_ms, ties, variant = gpu_lloyd(cfg, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1e3
+    iters_per_s = args.steps / elapsed
+    fused_s = kernel_ms[0] * 1e-3
+    flops = lloyd_flops(n, d, k)
+    nbytes = lloyd_bytes(n, d, 4)
+    log(f"[bench] {ms_per_step:.4f} ms/iter; kernels (ms): fused {kernel_ms[0]:.4f} reduce "
+        f"{kernel_ms[1]:.4f} finalize {kernel_ms[2]:.4f}; near-tie label differences on slice: {ties}")
+
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "lloyd_fused_step_c2_traffic.json")
+    if os.path.exists(traffic_file) and n == 5_000_000:
+        with open(traffic_file) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
+    out = {
+        "metric": "lloyd_iterations_per_sec",
+        "value": iters_per_s,
+        "unit": "iter/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"configs[1]: Lloyd n={n} d={d} k={k} fp32, weighted, tol=0",
+                   "kernel_variant": int(variant)},
+        "samples_clusters_per_sec": iters_per_s * n * k,
+        "kernel_ms": {"fused_step": float(kernel_ms[0]), "reduce": float(kernel_ms[1]),
+                      "finalize": float(kernel_ms[2])},
+        "roofline": {
+            "bound": "mfma",
+            "achieved": flops / fused_s / 1e12,
+            "peak": FP32_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": flops / fused_s / 1e12 / FP32_PEAK_TFLOPS,
+            "traffic": traffic,
+            "kernel": "fused Lloyd step",
+            "flops_per_launch": flops,
+        },
+        "roofline_hbm": {
+            "bound": "hbm",
+            "achieved": nbytes / fused_s / 1e9,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": nbytes / fused_s / 1e9 / HBM_PEAK_GBS,
+            "bytes_per_launch": nbytes,
+        },
+        "parity": {"near_tie_label_differences": int(ties), "checked_samples": min(n, 200_000)},
+    }
+
+    if not args.no_kpp:
+        t0 = time.time()
+        c4 = datasets.config4()
+        kpp_ms, _ = gpu_kmeanspp(c4)
+        n4, d4 = c4["X"].shape
+        tn = c4["n_local_trials"]
+        kpp_bytes = (c4["k"] - 1) * (n4 * (4 * d4 + 8) + tn * n4 * 4)
+        out["kmeanspp_ms"] = kpp_ms
+        out["kmeanspp"] = {"workload": f"configs[3]: n={n4} d={d4} k={c4['k']} trials={tn}",
+                           "ms": kpp_ms, "hbm_GBs": kpp_bytes / (kpp_ms * 1e-3) / 1e9,
+                           "hbm_frac": kpp_bytes / (kpp_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        log(f"[bench] kmeans++ {kpp_ms:.1f} ms ({time.time() - t0:.1f}s incl. data)")
+        del c4
+
+    if not args.no_cpu:
+        cpu_ips, threads, cpu_iters, cpu_elapsed = cpu_lloyd_baseline(cfg, args.cpu_iters)
+        out["cpu_baseline"] = {
+            "value": cpu_ips,
+            "unit": "iter/s",
+            "cores": int(threads),
+            "kind": "reference",
+            "impl": "scikit-learn %s _kmeans_single_lloyd (OpenMP Cython), the CPU engine the reference "
+                    "plugin subclasses and falls back to" % __import__("sklearn").__version__,
+            "sample": f"same data and init, {cpu_iters} iterations at full n={n} in {cpu_elapsed:.1f}s "
+                      f"(os.cpu_count()={os.cpu_count()})",
+        }
+        log(f"[bench] sklearn CPU Lloyd: {cpu_ips:.3f} iter/s on {threads} threads")
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

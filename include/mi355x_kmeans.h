@@ -103,6 +103,17 @@ int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* c
                        size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                        void* stream);
 
+/* kmx_lloyd_iter with HIP events recorded on `stream` around each of its kernels.  Waits for
+ * the iteration and writes the three durations in milliseconds (fused step, reduction,
+ * finalisation) to kernel_ms_host[0..2].  For benchmarks and profiling; it has no
+ * counterpart in the reference, whose benchmark only times a whole fit
+ * (benchmark/kmeans.py:163-165). */
+int32_t kmx_lloyd_iter_timed(const void* X_t, const void* sample_weight, const void* centroids_t,
+                             void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                             void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                             size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                             void* stream, float* kernel_ms_host);
+
 /* Second half of (2) alone, for the iteration that stopped with KMX_NEED_RELOCATION after
  * the host has relocated the empty clusters: sums / sizes, shift, convergence test, state
  * back to KMX_RUNNING (or a terminal state).  kmeans/drivers.py:275,326-343. */
@@ -113,9 +124,9 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t, const
 /* Copies the status to host memory and waits for it (the only synchronising call). */
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
 
-/* Which fused-step kernel kmx_lloyd_iter would use for a shape: 0 = generic streaming,
- * 1 = register-resident samples with LDS accumulators, 2 = register-resident samples with
- * global accumulators, 3 = MFMA (fp32) with LDS accumulators. */
+/* Which fused-step kernel kmx_lloyd_iter uses for a shape, as 10 * path + accumulation:
+ * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32);
+ * accumulation 1 = workgroup-private LDS accumulators, 2 = global copies with atomics. */
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype);
 
 /* ------------------------------------------------------------------------------------ *

@@ -563,7 +563,7 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
                         const void* centroids_t, void* new_centroids_t,
                         const uint32_t* labels_prev, uint32_t* labels, void* sizes,
                         uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
-                        hipStream_t stream) {
+                        hipStream_t stream, hipEvent_t* events = nullptr) {
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
     T* cpack = reinterpret_cast<T*>(ws + L.off_cpack);
     T* half_norms = reinterpret_cast<T*>(ws + L.off_half);
@@ -571,6 +571,7 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
     double* shift_partial = reinterpret_cast<double*>(ws + L.off_shift);
 
     int n_partials_used = L.n_partials;
+    if (events) (void)hipEventRecord(events[0], stream);
     if (L.acc_mode == ACC_LDS) {
         launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
                                  partial, status, n, d, k, stream);
@@ -586,16 +587,19 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
                                     partial, status, n, d, k, stream);
     }
     KMX_LAUNCH_CHECK();
+    if (events) (void)hipEventRecord(events[1], stream);
 
     const int items = (d + 1) * k;
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)kmx_cdiv(items, 32)), dim3(256), 0,
                        stream, partial, n_partials_used, L.acc_mode == ACC_GLOBAL ? 1 : 0,
                        (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k);
     KMX_LAUNCH_CHECK();
+    if (events) (void)hipEventRecord(events[2], stream);
     hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, 256)), dim3(256), 0,
                        stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
                        half_norms, shift_partial, status, d, k, L.dpad, 0);
     KMX_LAUNCH_CHECK();
+    if (events) (void)hipEventRecord(events[3], stream);
     return KMX_OK;
 }
 
@@ -676,11 +680,12 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* cent
     return KMX_OK;
 }
 
-int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* centroids_t,
-                       void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
-                       void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
-                       size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
-                       void* stream_) {
+static int32_t lloyd_iter_dispatch(const void* X_t, const void* sample_weight,
+                                   const void* centroids_t, void* new_centroids_t,
+                                   const uint32_t* labels_prev, uint32_t* labels,
+                                   void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                                   size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
+                                   int32_t dtype, void* stream_, hipEvent_t* events) {
     KMX_REQUIRE_PTR(X_t);
     KMX_REQUIRE_PTR(sample_weight);
     KMX_REQUIRE_PTR(centroids_t);
@@ -699,14 +704,48 @@ int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* c
         if (L.variant == KMX_VARIANT_MFMA)
             return kmx_lloyd_iter_mfma_f32(L, X_t, sample_weight, centroids_t, new_centroids_t,
                                            labels_prev, labels, cluster_sizes, empty_clusters,
-                                           (char*)workspace, n, d, k, stream);
+                                           (char*)workspace, n, d, k, stream, events);
         return lloyd_iter_impl<float>(L, X_t, sample_weight, centroids_t, new_centroids_t,
                                       labels_prev, labels, cluster_sizes, empty_clusters,
-                                      (char*)workspace, n, d, k, stream);
+                                      (char*)workspace, n, d, k, stream, events);
     }
     return lloyd_iter_impl<double>(L, X_t, sample_weight, centroids_t, new_centroids_t, labels_prev,
                                    labels, cluster_sizes, empty_clusters, (char*)workspace, n, d, k,
-                                   stream);
+                                   stream, events);
+}
+
+int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* centroids_t,
+                       void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                       void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                       size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                       void* stream_) {
+    return lloyd_iter_dispatch(X_t, sample_weight, centroids_t, new_centroids_t, labels_prev, labels,
+                               cluster_sizes, empty_clusters, workspace, workspace_bytes, n, d, k,
+                               dtype, stream_, nullptr);
+}
+
+int32_t kmx_lloyd_iter_timed(const void* X_t, const void* sample_weight, const void* centroids_t,
+                             void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                             void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                             size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                             void* stream_, float* kernel_ms_host) {
+    KMX_REQUIRE_PTR(kernel_ms_host);
+    hipEvent_t ev[4];
+    for (int i = 0; i < 4; ++i) {
+        const hipError_t e = hipEventCreate(&ev[i]);
+        if (e != hipSuccess) return (int32_t)e;
+    }
+    int32_t rc = lloyd_iter_dispatch(X_t, sample_weight, centroids_t, new_centroids_t, labels_prev,
+                                     labels, cluster_sizes, empty_clusters, workspace,
+                                     workspace_bytes, n, d, k, dtype, stream_, ev);
+    if (rc == KMX_OK) {
+        hipError_t e = hipEventSynchronize(ev[3]);
+        for (int i = 0; i < 3 && e == hipSuccess; ++i)
+            e = hipEventElapsedTime(&kernel_ms_host[i], ev[i], ev[i + 1]);
+        if (e != hipSuccess) rc = (int32_t)e;
+    }
+    for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
+    return rc;
 }
 
 int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,

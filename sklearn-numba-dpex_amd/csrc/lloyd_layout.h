@@ -74,7 +74,7 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
                                 const void* centroids_t, void* new_centroids_t,
                                 const uint32_t* labels_prev, uint32_t* labels, void* sizes,
                                 uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
-                                hipStream_t stream);
+                                hipStream_t stream, hipEvent_t* events);
 int32_t kmx_assign_labels_mfma_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
                                    uint32_t* labels, char* ws, int64_t n, int d, int k,
                                    hipStream_t stream);

@@ -16,7 +16,7 @@ int kmx_forced_variant() {
 
 int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout&, const void*, const void*, const void*, void*,
                                 const uint32_t*, uint32_t*, void*, uint32_t*, char*, int64_t, int,
-                                int, hipStream_t) {
+                                int, hipStream_t, hipEvent_t*) {
     return KMX_ERR_UNSUPPORTED;
 }
 

@@ -91,6 +91,52 @@ def test_single_iteration_through_c_abi(cuda, name):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
+@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "odd"])
+def test_lockstep_iterations_match_oracle(cuda, name):
+    """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
+    iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
+    chaotic, so free-running trajectories may only be compared until the first near-tie)."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    cfg = _small_configs()[name]()
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    dc = _capi.dtype_code(X.dtype)
+    X_t, w_d = _dev(X.T, cuda), _dev(w, cuda)
+    cent = [_dev(init.T, cuda), None]
+    cent[1] = torch.empty_like(cent[0])
+    labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
+    sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+    status = _capi.LloydStatus()
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(cent[0]), n, d, k, dc, 100, 0.0, stream), "init")
+    prev = None
+    for it in range(10):
+        a, b = it % 2, (it + 1) % 2
+        c_in = cent[a].cpu().numpy().T.copy()
+        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k,
+                                       dc, stream), "iter")
+        _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+        got = labels[b].cpu().numpy().astype(np.int64)
+        assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
+        sums, ref_sizes = ok.weighted_sums(X, w, got, k)
+        assert status.n_empty == 0 and status.n_iter == it + 1
+        assert_centers_close(cent[b].cpu().numpy().T, sums / ref_sizes[:, None], X.dtype)
+        if prev is not None:
+            assert status.reserved[1] == int(np.count_nonzero(got != prev))
+        prev = got
+        if status.state != _capi.KMX_RUNNING:
+            assert status.state == _capi.KMX_CONVERGED_STRICT and np.array_equal(got, prev)
+            break
+
+
 @pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C5", "odd"])
 def test_full_lloyd_run_matches_oracle(cuda, name):
     from sklearn_numba_dpex_amd.kmeans import drivers
@@ -109,7 +155,14 @@ def test_full_lloyd_run_matches_oracle(cuda, name):
     ref_labels, ref_inertia, ref_centers, ref_n_iter = ok.lloyd(Xc, w, initc, max_iter=max_iter, tol=tol)
     assert n_iter == ref_n_iter
     centers = centers_t.cpu().numpy().T
-    # trajectories may separate at near-ties; allow a looser centroid bound after many iterations
-    assert_centers_close(centers, ref_centers, X.dtype, scale_rtol=max(RTOL[X.dtype], 1e-9) * 50)
-    assert_labels_match(labels.cpu().numpy(), ref_labels, Xc, ref_centers)
-    assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-5)
+    got = labels.cpu().numpy().astype(np.int64)
+    # the returned labels are the argmin for the returned centroids, whatever the trajectory
+    assert_labels_match(got, ok.assign_labels(Xc, centers), Xc, centers)
+    assert float(inertia) == pytest.approx(float(ok.inertia(Xc, w, centers, got)), rel=1e-5)
+    if np.array_equal(got, ref_labels.astype(np.int64)):
+        # same final partition: centroids must agree to rounding
+        assert_centers_close(centers, ref_centers, X.dtype, scale_rtol=RTOL[X.dtype] * 10)
+        assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-5)
+    else:
+        # a near-tie flipped somewhere along the run: same quality, not the same partition
+        assert float(inertia) == pytest.approx(float(ref_inertia), rel=2e-3)
