@@ -66,7 +66,7 @@ def gpu_lloyd(cfg, steps, warmup):
     status = _capi.LloydStatus()
     total = warmup + 2 * steps + 8
 
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(cent[0]), n, d, k, dc, total, 0.0, stream), "init")
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, total, 0.0, stream), "init")
     it = 0
 
     def enqueue():

@@ -72,13 +72,16 @@ typedef struct kmx_lloyd_status {
 
 size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype);
 
-/* Resets the loop state, packs the initial centroids (+ their half squared norms) and
- * clears the accumulators.  Replaces the set-up part of lloyd(), kmeans/drivers.py:146-184. */
-int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* centroids_t,
-                       int64_t n, int32_t d, int32_t k, int32_t dtype, int32_t max_iter,
-                       double tol, void* stream);
+/* Resets the loop state, packs the initial centroids (+ their half squared norms), clears
+ * the accumulators and, for the fixed-point accumulation of the fp32 matrix-core path, takes
+ * max|x| per feature and max|w| (one pass over X_t and sample_weight).
+ * Replaces the set-up part of lloyd(), kmeans/drivers.py:146-184. */
+int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
+                       const void* sample_weight, const void* centroids_t, int64_t n, int32_t d,
+                       int32_t k, int32_t dtype, int32_t max_iter, double tol, void* stream);
 
-/* One Lloyd iteration, enqueued as two kernels:
+/* One Lloyd iteration, enqueued as two kernels (three for shapes whose partial sums do not
+ * fit in LDS):
  *   (1) fused step: pseudo distances 0.5||c||^2 - <x,c>, argmin (lowest index wins ties),
  *       label write, changed-label count, per-workgroup partial sums of w*x and w;
  *   (2) reduction of the partial sums, empty-cluster list (ascending), and - when no cluster

@@ -13,6 +13,7 @@
 // float atomics.  The MFMA variant for fp32 lives in lloyd_mfma.hip.
 #include "kmx_common.h"
 #include "lloyd_layout.h"
+#include "lloyd_tail.h"
 
 namespace {
 
@@ -503,6 +504,15 @@ __global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words)
 // Host-side launchers
 // ------------------------------------------------------------------------------------------
 
+// Workgroups of a vector-ALU fused step (also the number of partial slots it fills).
+int lloyd_fused_grid(const LloydLayout& L, int64_t n, int d, int dtype) {
+    const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype) : 2;
+    const int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
+    const int cap = L.grid_cap(kmx_num_cus());
+    int grid = (int)(tiles < cap ? tiles : cap);
+    return grid < 1 ? 1 : grid;
+}
+
 template <typename T, int DREG, int R, int ACC>
 void launch_reg(const LloydLayout& L, const void* X_t, const void* w, const T* cpack,
                 const T* half_norms, const uint32_t* labels_prev, uint32_t* labels, T* partial,
@@ -519,12 +529,8 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
                   const T* cpack, const T* half_norms, const uint32_t* labels_prev,
                   uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
                   hipStream_t stream) {
-    const int cus = kmx_num_cus();
+    const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_REGISTER) {
-        const int r = lloyd_reg_samples_per_thread(d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
-        int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
-        int grid = (int)(tiles < (int64_t)L.grid_cap(cus) ? tiles : L.grid_cap(cus));
-        if (grid < 1) grid = 1;
 #define KMX_REG_CASE(DR, RR)                                                                    \
     launch_reg<T, DR, RR, ACC>(L, X_t, w, cpack, half_norms, labels_prev, labels, partial, status, \
                                n, d, k, grid, stream)
@@ -548,9 +554,6 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
 #undef KMX_REG_CASE
     } else {
         constexpr int R = 2, KC = 8;
-        int64_t tiles = kmx_cdiv(n, 256 * (int64_t)R);
-        int grid = (int)(tiles < (int64_t)L.grid_cap(cus) ? tiles : L.grid_cap(cus));
-        if (grid < 1) grid = 1;
         const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(T) : 0;
         hipLaunchKernelGGL((lloyd_fused_stream_kernel<T, R, KC, ACC>), dim3(grid), dim3(256), lds,
                            stream, (const T*)X_t, (const T*)w, (const T*)centroids_t, half_norms,
@@ -570,25 +573,18 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
     T* partial = reinterpret_cast<T*>(ws + L.off_partial);
     double* shift_partial = reinterpret_cast<double*>(ws + L.off_shift);
 
-    int n_partials_used = L.n_partials;
     if (events) (void)hipEventRecord(events[0], stream);
+    int n_partials_used = L.n_partials;
     if (L.acc_mode == ACC_LDS) {
         launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
                                  partial, status, n, d, k, stream);
-        const int r = (L.variant == KMX_VARIANT_REGISTER)
-                          ? lloyd_reg_samples_per_thread(d, sizeof(T) == 8 ? KMX_F64 : KMX_F32)
-                          : 2;
-        int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
-        const int cap = L.grid_cap(kmx_num_cus());
-        n_partials_used = (int)(tiles < cap ? tiles : cap);
-        if (n_partials_used < 1) n_partials_used = 1;
+        n_partials_used = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     } else {
         launch_fused<T, ACC_GLOBAL>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
                                     partial, status, n, d, k, stream);
     }
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[1], stream);
-
     const int items = (d + 1) * k;
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)kmx_cdiv(items, 32)), dim3(256), 0,
                        stream, partial, n_partials_used, L.acc_mode == ACC_GLOBAL ? 1 : 0,
@@ -649,10 +645,12 @@ int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype)
     return L.variant * 10 + L.acc_mode;
 }
 
-int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* centroids_t, int64_t n,
-                       int32_t d, int32_t k, int32_t dtype, int32_t max_iter, double tol,
-                       void* stream_) {
+int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
+                       const void* sample_weight, const void* centroids_t, int64_t n, int32_t d,
+                       int32_t k, int32_t dtype, int32_t max_iter, double tol, void* stream_) {
     KMX_REQUIRE_PTR(workspace);
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(sample_weight);
     KMX_REQUIRE_PTR(centroids_t);
     if (n <= 0 || d <= 0 || k <= 0 || max_iter < 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
@@ -671,6 +669,10 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* cent
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),
                            (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
     KMX_LAUNCH_CHECK();
+    if (L.variant == KMX_VARIANT_MFMA) {
+        const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, stream);
+        if (rc != KMX_OK) return rc;
+    }
     if (L.acc_mode == ACC_GLOBAL) {
         const size_t words = L.partial_bytes / 4;
         hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1024), dim3(256), 0, stream,

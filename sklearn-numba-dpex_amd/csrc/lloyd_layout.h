@@ -15,17 +15,26 @@ constexpr int KMX_MAX_PARTIALS = 1024;          // upper bound on fused-step wor
 constexpr size_t KMX_LDS_ACC_LIMIT = 40000;     // bytes of LDS accumulators per workgroup
 constexpr size_t KMX_GLOBAL_COPIES_BYTES = 64u << 20;
 
+// Environment overrides for experiments: KMX_LLOYD_VARIANT = stream | register | mfma,
+// KMX_LLOYD_WGS_PER_CU = 1..8.
+int kmx_forced_variant();
+int kmx_wgs_per_cu();
+// Shapes the fp32 matrix-core fused step covers (operands and accumulators fit in LDS).
+bool kmx_mfma_supported(int d, int k);
+
 struct LloydLayout {
     int dpad;            // features per packed centroid row (multiple of 4, zero padded)
     int variant;         // KMX_VARIANT_*
     int acc_mode;        // KMX_ACC_*
     int n_partials;      // slots in `partial` (workgroups for LDS mode, copies for global mode)
-    size_t off_status, off_cpack, off_half, off_shift, off_partial;
+    int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
+    size_t off_status, off_scales, off_gsum, off_cpack, off_half, off_shift, off_partial;
     size_t partial_bytes;
     size_t total;
-    // Workgroups of the fused step: four per compute unit, never more than the partial slots.
+    // Workgroups of the fused step: a few per compute unit (KMX_LLOYD_WGS_PER_CU, default 4),
+    // never more than the partial slots.
     int grid_cap(int cus) const {
-        const int g = 4 * cus;
+        const int g = kmx_wgs_per_cu() * cus;
         return g < n_partials ? g : n_partials;
     }
 };
@@ -35,14 +44,13 @@ static inline int lloyd_reg_samples_per_thread(int d, int dtype) {
     return d <= 16 ? 2 : 1;
 }
 
-// Environment override for experiments: KMX_LLOYD_VARIANT = stream | register | mfma.
-int kmx_forced_variant();
 
 static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     (void)n;
     LloydLayout L;
     const size_t s = kmx_dtype_size(dtype);
     L.dpad = (d + 3) & ~3;
+    L.k_for_gsum = k;
     const size_t items = (size_t)(d + 1) * k;
     const bool reg_ok = (dtype == KMX_F32) ? d <= 64 : d <= 32;
     L.variant = reg_ok ? KMX_VARIANT_REGISTER : KMX_VARIANT_STREAM;
@@ -59,17 +67,27 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
         if (copies > 32) copies = 32;
         L.n_partials = (int)copies;
     }
+    if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_supported(d, k) &&
+        (forced < 0 || forced == KMX_VARIANT_MFMA))
+        L.variant = KMX_VARIANT_MFMA;
     L.off_status = 0;
-    L.off_cpack = kmx_align256(sizeof(kmx_lloyd_status));
+    // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
+    L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));
+    L.off_gsum = L.off_scales + kmx_align256(sizeof(float) * 2 * (size_t)(d + 1) + 64);
+    L.off_cpack = L.off_gsum + kmx_align256(items * sizeof(long long));
     L.off_half = L.off_cpack + kmx_align256((size_t)k * L.dpad * s);
     L.off_shift = L.off_half + kmx_align256((size_t)k * s);
     L.off_partial = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 256) * sizeof(double));
-    L.partial_bytes = (size_t)L.n_partials * items * s;
+    // the matrix-core path accumulates into gsum and needs no per-workgroup partials
+    L.partial_bytes = L.variant == KMX_VARIANT_MFMA ? 0 : (size_t)L.n_partials * items * s;
     L.total = L.off_partial + kmx_align256(L.partial_bytes);
     return L;
 }
 
 // fp32 matrix-core implementations (lloyd_mfma.hip)
+// Fixed-point exponents from max|X_t row|, max|w| and n; clears the fixed-point sums.
+int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void* w, char* ws,
+                               int64_t n, int d, hipStream_t stream);
 int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const void* w,
                                 const void* centroids_t, void* new_centroids_t,
                                 const uint32_t* labels_prev, uint32_t* labels, void* sizes,

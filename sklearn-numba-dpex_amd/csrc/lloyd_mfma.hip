@@ -1,6 +1,31 @@
-// fp32 Lloyd step on the matrix cores (v_mfma_f32_32x32x2_f32).  Not selected yet:
-// lloyd_layout() never returns KMX_VARIANT_MFMA, and these entry points refuse to run.
+// fp32 fused Lloyd step on the matrix cores of gfx950 (v_mfma_f32_32x32x2_f32), one launch
+// per iteration.
+//
+// Work decomposition
+//   * A wave owns tiles of 128 consecutive samples.  Lane (j, h) with j = lane % 32,
+//     h = lane / 32 loads, for every pair of features (2s, 2s + 1), the four samples
+//     4j .. 4j + 3 of feature row 2s + h with one 128-bit load: each half-wave reads 512
+//     contiguous bytes of X_t.  Component t of those float4 is exactly the B operand
+//     (K x N = 2 x 32) of MFMA tile t, which holds the samples {4j + t}; no shuffles.
+//   * Centroids are the A operand (M x K = 32 x 2), staged once per workgroup in LDS in
+//     fragment order (conflict-free 4-byte reads, one per MFMA), 32 centroids per block.
+//   * The accumulator of tile t starts at -0.5||c||^2, so after the K loop it holds
+//     <x, c> - 0.5||c||^2 for 16 centroids x 1 sample per lane; the argmax over centroids is
+//     kept per lane in registers (strict '>' in increasing centroid order = lowest index
+//     wins) and the two half-waves are combined once per tile.
+//   * w * x and w are accumulated in 64-bit FIXED POINT: LDS accumulators private to the
+//     workgroup (ds_add_u64 runs ~10x faster than ds_add_f32 on this hardware), flushed once
+//     per workgroup with 64-bit integer global atomics.  Integer addition is associative, so
+//     the sums do not depend on the order in which samples, waves or workgroups arrive: the
+//     iteration is reproducible bit for bit, and the sums are exact to 2^-q (q chosen per
+//     feature from max|x|, max|w| and n so that nothing can overflow).
+//   * A one-workgroup kernel then converts the sums, lists empty clusters and, if there are
+//     none, divides, computes the shift and runs the convergence test (lloyd_tail.h).
+//
+// Arithmetic per sample is the reference's 0.5||c||^2 - <x, c> with another summation
+// order, so labels can differ from a feature-sequential evaluation only at near-ties.
 #include "lloyd_layout.h"
+#include "lloyd_tail.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -14,13 +39,403 @@ int kmx_forced_variant() {
     return -1;
 }
 
-int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout&, const void*, const void*, const void*, void*,
-                                const uint32_t*, uint32_t*, void*, uint32_t*, char*, int64_t, int,
-                                int, hipStream_t, hipEvent_t*) {
-    return KMX_ERR_UNSUPPORTED;
+int kmx_wgs_per_cu() {
+    const char* v = std::getenv("KMX_LLOYD_WGS_PER_CU");
+    if (v == nullptr) return 4;
+    const int x = std::atoi(v);
+    return (x >= 1 && x <= 8) ? x : 4;
 }
 
-int32_t kmx_assign_labels_mfma_f32(const LloydLayout&, const void*, const void*, uint32_t*, char*,
-                                   int64_t, int, int, hipStream_t) {
-    return KMX_ERR_UNSUPPORTED;
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// 1.5 * 2^52: adding it to |v| < 2^51 leaves round-to-nearest(v) in the low mantissa bits.
+constexpr double FIX_MAGIC = 6755399441055744.0;
+constexpr long long FIX_MAGIC_BITS = 0x4338000000000000ll;
+
+__device__ __forceinline__ unsigned long long to_fixed(double scaled_plus_magic) {
+    return (unsigned long long)(__double_as_longlong(scaled_plus_magic) - FIX_MAGIC_BITS);
+}
+
+// ---------------------------------------------------------------------------- scales
+
+__global__ void absmax_zero_kernel(unsigned int* absmax, int count) {
+    for (int i = threadIdx.x; i < count; i += blockDim.x) absmax[i] = 0u;
+}
+
+// Row r < d: max |X_t[r, :]|; row d: max |w|.  Non-negative floats order like their bits.
+__global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ X_t,
+                                                          const float* __restrict__ w,
+                                                          unsigned int* __restrict__ absmax,
+                                                          int64_t n, int d) {
+    const int row = blockIdx.y;
+    const float* __restrict__ p = row < d ? X_t + (size_t)row * n : w;
+    float m = 0.0f;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+        m = fmaxf(m, fabsf(p[i]));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((threadIdx.x & 63) == 0) atomicMax(&absmax[row], __float_as_uint(m));
+}
+
+// q[f] for the sums of w * x_f, q[d] for the sums of w: the largest exponents such that
+// n * max|w| * max|x_f| * 2^q < 2^61 and one sample's contribution stays below 2^50.
+__global__ void fixed_point_exponents_kernel(const unsigned int* __restrict__ absmax,
+                                             int* __restrict__ q, int64_t n, int d) {
+    const int f = threadIdx.x;
+    if (f > d) return;
+    const float wmax = __uint_as_float(absmax[d]);
+    const float xmax = f < d ? __uint_as_float(absmax[f]) : 1.0f;
+    int e = 0;  // log2 upper bound of one contribution
+    if (wmax > 0.0f && isfinite(wmax)) e += ilogbf(wmax) + 1;
+    if (f < d && xmax > 0.0f && isfinite(xmax)) e += ilogbf(xmax) + 1;
+    int en = 1;
+    while (((int64_t)1 << en) < n && en < 62) ++en;  // n <= 2^en
+    int qv = 61 - (e + en);
+    if (qv > 50 - e) qv = 50 - e;
+    if (qv > 100) qv = 100;
+    if (qv < -100) qv = -100;
+    q[f] = qv;
+}
+
+// ---------------------------------------------------------------------------- fused step
+
+template <int NKS, bool UPDATE>
+__global__ __launch_bounds__(256) void lloyd_mfma_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ sample_weight,
+    const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
+    uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
+    const int* __restrict__ q_exp, unsigned long long* __restrict__ gsum, int64_t n, int d, int k,
+    int vec_ok) {
+    if (UPDATE && status->state != KMX_RUNNING) return;
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int nks = (d + 1) >> 1;          // K steps of 2 features
+    const int n_cb = (k + 31) >> 5;        // centroid blocks of 32
+    const int items = (d + 1) * k;
+    unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [(d + 1) * k]
+    float* afrag = reinterpret_cast<float*>(acc + (UPDATE ? items : 0));         // [n_cb][nks][64]
+    float* hneg = afrag + n_cb * nks * 64;  // [n_cb][2][16]  -0.5||c||^2 in accumulator order
+    __shared__ unsigned int changed_block;
+
+    for (int idx = threadIdx.x; idx < n_cb * nks * 64; idx += 256) {
+        const int l = idx & 63;
+        const int s = (idx >> 6) % nks;
+        const int cb = (idx >> 6) / nks;
+        const int c = 32 * cb + (l & 31);
+        const int f = 2 * s + (l >> 5);
+        afrag[idx] = (c < k && f < d) ? centroids_t[(size_t)f * k + c] : 0.0f;
+    }
+    for (int idx = threadIdx.x; idx < n_cb * 32; idx += 256) {
+        const int cb = idx >> 5, h = (idx >> 4) & 1, r = idx & 15;
+        const int c = 32 * cb + 8 * (r >> 2) + 4 * h + (r & 3);
+        float v = -kmx_inf<float>();
+        if (c < k) {
+            float sq = 0.0f;
+            for (int f = 0; f < d; ++f) {
+                const float cv = centroids_t[(size_t)f * k + c];
+                sq += cv * cv;
+            }
+            v = -(sq / 2.0f);
+        }
+        hneg[idx] = v;
+    }
+    if (UPDATE) {
+        for (int jx = threadIdx.x; jx < items; jx += 256) acc[jx] = 0ull;
+        if (threadIdx.x == 0) changed_block = 0;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, j = lane & 31;
+    const int64_t n_wtiles = (n + 127) >> 7;
+    unsigned int changed = 0;
+
+    // 2^q of the feature rows this lane accumulates (row 2s + h), and of the weights
+    float scale[NKS];
+    float scale_w = 1.0f;
+    if (UPDATE) {
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+            const int f = 2 * s + h;
+            scale[s] = (s < nks && f < d) ? ldexpf(1.0f, q_exp[f]) : 0.0f;
+        }
+        scale_w = ldexpf(1.0f, q_exp[d]);
+    }
+
+    for (int64_t wt = (int64_t)blockIdx.x * 4 + wave; wt < n_wtiles; wt += (int64_t)gridDim.x * 4) {
+        const int64_t i0 = wt * 128 + 4 * j;
+        const bool full = vec_ok && (i0 + 4 <= n);
+
+        float4 x[NKS];
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+            x[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int f = 2 * s + h;
+            if (s < nks && f < d) {
+                const float* __restrict__ row = X_t + (size_t)f * n;
+                if (full) {
+                    x[s] = *reinterpret_cast<const float4*>(row + i0);
+                } else {
+                    if (i0 + 0 < n) x[s].x = row[i0 + 0];
+                    if (i0 + 1 < n) x[s].y = row[i0 + 1];
+                    if (i0 + 2 < n) x[s].z = row[i0 + 2];
+                    if (i0 + 3 < n) x[s].w = row[i0 + 3];
+                }
+            }
+        }
+
+        float best[4];
+        int code[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            best[t] = -kmx_inf<float>();
+            code[t] = 0;
+        }
+
+        for (int cb = 0; cb < n_cb; ++cb) {
+            const float* hp = hneg + cb * 32 + h * 16;
+            v16f hv;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) hv[r] = hp[r];
+            const float* ap = afrag + (size_t)cb * nks * 64 + lane;
+            // the first K step reads the accumulator start (-0.5||c||^2) straight from hv
+            float af = ap[0];
+            v16f a0 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].x, hv, 0, 0, 0);
+            v16f a1 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].y, hv, 0, 0, 0);
+            v16f a2 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].z, hv, 0, 0, 0);
+            v16f a3 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].w, hv, 0, 0, 0);
+#pragma unroll
+            for (int s = 1; s < NKS; ++s) {
+                if (s < nks) {
+                    af = ap[s * 64];
+                    a0 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].x, a0, 0, 0, 0);
+                    a1 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].y, a1, 0, 0, 0);
+                    a2 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].z, a2, 0, 0, 0);
+                    a3 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].w, a3, 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int cd = cb * 16 + r;  // wave-uniform
+                if (a0[r] > best[0]) { best[0] = a0[r]; code[0] = cd; }
+                if (a1[r] > best[1]) { best[1] = a1[r]; code[1] = cd; }
+                if (a2[r] > best[2]) { best[2] = a2[r]; code[2] = cd; }
+                if (a3[r] > best[3]) { best[3] = a3[r]; code[3] = cd; }
+            }
+        }
+
+        // decode (block, register) -> centroid index, then combine the two half-waves
+        uint32_t lab[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int c = 32 * (code[t] >> 4) + 8 * ((code[t] & 15) >> 2) + 4 * h + (code[t] & 3);
+            const float ov = __shfl_xor(best[t], 32, 64);
+            const int oc = __shfl_xor(c, 32, 64);
+            if (ov > best[t] || (ov == best[t] && oc < c)) c = oc;
+            lab[t] = (uint32_t)c;
+        }
+
+        if (h == 0) {
+            if (full) {
+                *reinterpret_cast<uint4*>(labels + i0) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (i0 + t < n) labels[i0 + t] = lab[t];
+            }
+        }
+
+        if (UPDATE) {
+            float wv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (full) {
+                const float4 w4 = *reinterpret_cast<const float4*>(sample_weight + i0);
+                wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                if (h == 0) {
+                    const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+                    changed += (p4.x != lab[0]) + (p4.y != lab[1]) + (p4.z != lab[2]) + (p4.w != lab[3]);
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    if (i0 + t < n) {
+                        wv[t] = sample_weight[i0 + t];
+                        if (h == 0) changed += (labels_prev[i0 + t] != lab[t]) ? 1u : 0u;
+                    }
+                }
+            }
+            // samples past the end carry w = 0 and x = 0: they add zero
+            double wd[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) wd[t] = (double)wv[t];
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) {
+                const int f = 2 * s + h;
+                if (s < nks && f < d) {
+                    unsigned long long* rowacc = acc + f * k;
+                    const double sc = (double)scale[s];
+                    const float xs[4] = {x[s].x, x[s].y, x[s].z, x[s].w};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        // x * w is exact in fp64; one rounding, to a multiple of 2^-q
+                        const double v = fma((double)xs[t], wd[t] * sc, FIX_MAGIC);
+                        atomicAdd(rowacc + lab[t], to_fixed(v));
+                    }
+                }
+            }
+            if (h == 0) {
+                unsigned long long* szacc = acc + d * k;
+                const double sc = (double)scale_w;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    atomicAdd(szacc + lab[t], to_fixed(fma(wd[t], sc, FIX_MAGIC)));
+            }
+        }
+    }
+
+    if (UPDATE) {
+        if (changed) atomicAdd(&changed_block, changed);
+        __syncthreads();
+        if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+        for (int jx = threadIdx.x; jx < items; jx += 256) {
+            const unsigned long long v = acc[jx];
+            if (v) atomicAdd(gsum + jx, v);
+        }
+    }
+}
+
+// One workgroup: fixed point -> float sums and sizes (clearing gsum for the next iteration),
+// empty-cluster list, and the finalisation if no cluster is empty.
+__global__ __launch_bounds__(256) void lloyd_mfma_finalize_kernel(
+    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<float> a) {
+    if (a.status->state != KMX_RUNNING) return;
+    const int d = a.d, k = a.k;
+    const int items = (d + 1) * k;
+    for (int jx = threadIdx.x; jx < items; jx += 256) {
+        const long long iv = (long long)gsum[jx];
+        gsum[jx] = 0ull;
+        const int f = jx / k;
+        const float val = (float)ldexp((double)iv, -q_exp[f]);
+        if (f < d)
+            a.sums_t[jx] = val;
+        else
+            a.sizes[jx - d * k] = val;
+    }
+    __syncthreads();
+    int heaviest = 0;
+    const int n_empty = lloyd_list_empty<float>(a.sizes, a.empty_clusters, k, &heaviest);
+    if (threadIdx.x == 0) {
+        a.status->n_empty = n_empty;
+        a.status->reserved[0] = heaviest;
+    }
+    if (n_empty > 0) {
+        if (threadIdx.x == 0) a.status->state = KMX_NEED_RELOCATION;
+        return;
+    }
+    lloyd_finalize_block<float>(a, 0, heaviest);
+}
+
+size_t mfma_lds_bytes(int d, int k, bool update) {
+    const int nks = (d + 1) / 2, n_cb = (k + 31) / 32;
+    size_t bytes = ((size_t)n_cb * nks * 64 + (size_t)n_cb * 32) * sizeof(float);
+    if (update) bytes += (size_t)(d + 1) * k * sizeof(unsigned long long);
+    return bytes;
+}
+
+template <bool UPDATE>
+int32_t launch_mfma(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
+                    const uint32_t* labels_prev, uint32_t* labels, kmx_lloyd_status* status,
+                    const int* q_exp, unsigned long long* gsum, int64_t n, int d, int k,
+                    hipStream_t stream) {
+    const size_t lds = mfma_lds_bytes(d, k, UPDATE);
+    if (lds > 64 * 1024 || d > 64) return KMX_ERR_UNSUPPORTED;
+    const int64_t n_wtiles = kmx_cdiv(n, 128);
+    int64_t grid = kmx_cdiv(n_wtiles, 4);
+    const int cap = L.grid_cap(kmx_num_cus());
+    if (grid > cap) grid = cap;
+    if (grid < 1) grid = 1;
+    auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
+    const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
+                       (!UPDATE || (aligned16(w) && aligned16(labels_prev)));
+#define KMX_MFMA_CASE(NKS)                                                                     \
+    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, UPDATE>), dim3((unsigned)grid), dim3(256), lds, \
+                       stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,  \
+                       labels_prev, labels, status, q_exp, gsum, n, d, k, vec_ok)
+    if (d <= 8)
+        KMX_MFMA_CASE(4);
+    else if (d <= 16)
+        KMX_MFMA_CASE(8);
+    else if (d <= 32)
+        KMX_MFMA_CASE(16);
+    else
+        KMX_MFMA_CASE(32);
+#undef KMX_MFMA_CASE
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+}  // namespace
+
+bool kmx_mfma_supported(int d, int k) {
+    return d <= 64 && k >= 16 && mfma_lds_bytes(d, k, true) <= 64 * 1024;
+}
+
+int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void* w, char* ws,
+                               int64_t n, int d, hipStream_t stream) {
+    unsigned int* absmax = reinterpret_cast<unsigned int*>(ws + L.off_scales);
+    int* q_exp = reinterpret_cast<int*>(absmax + (d + 1));
+    hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(256), 0, stream, absmax, d + 1);
+    int64_t gx = kmx_cdiv(n, 256 * 16);
+    if (gx > 1024) gx = 1024;
+    hipLaunchKernelGGL(absmax_rows_kernel, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
+                       stream, (const float*)X_t, (const float*)w, absmax, n, d);
+    hipLaunchKernelGGL(fixed_point_exponents_kernel, dim3(1), dim3(128), 0, stream, absmax, q_exp, n, d);
+    const size_t words = (size_t)(d + 1) * L.k_for_gsum * 2;
+    hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(1024), 0, stream,
+                       reinterpret_cast<unsigned int*>(ws + L.off_gsum), (int)words);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const void* w,
+                                const void* centroids_t, void* new_centroids_t,
+                                const uint32_t* labels_prev, uint32_t* labels, void* sizes,
+                                uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
+                                hipStream_t stream, hipEvent_t* events) {
+    if (L.acc_mode != KMX_ACC_LDS) return KMX_ERR_UNSUPPORTED;
+    LloydTail<float> tail;
+    tail.sums_t = (float*)new_centroids_t;
+    tail.sizes = (float*)sizes;
+    tail.empty_clusters = empty_clusters;
+    tail.old_centroids_t = (const float*)centroids_t;
+    tail.cpack = reinterpret_cast<float*>(ws + L.off_cpack);
+    tail.half_norms = reinterpret_cast<float*>(ws + L.off_half);
+    tail.status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
+    tail.d = d;
+    tail.k = k;
+    tail.dpad = L.dpad;
+    const int* q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
+    unsigned long long* gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
+    if (events) (void)hipEventRecord(events[0], stream);
+    const int32_t rc = launch_mfma<true>(L, X_t, w, centroids_t, labels_prev, labels, tail.status,
+                                         q_exp, gsum, n, d, k, stream);
+    if (rc != KMX_OK) return rc;
+    if (events) {
+        (void)hipEventRecord(events[1], stream);
+        (void)hipEventRecord(events[2], stream);
+    }
+    hipLaunchKernelGGL(lloyd_mfma_finalize_kernel, dim3(1), dim3(256), 0, stream, gsum, q_exp, tail);
+    KMX_LAUNCH_CHECK();
+    if (events) (void)hipEventRecord(events[3], stream);
+    return KMX_OK;
+}
+
+int32_t kmx_assign_labels_mfma_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
+                                   uint32_t* labels, char* ws, int64_t n, int d, int k,
+                                   hipStream_t stream) {
+    (void)ws;
+    return launch_mfma<false>(L, X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr,
+                              nullptr, n, d, k, stream);
 }

@@ -1,0 +1,150 @@
+// Single-workgroup finalisation of a Lloyd iteration, used when (d + 1) * k is small enough
+// for one workgroup: empty-cluster list (ascending) and heaviest cluster, then division by
+// the cluster sizes, packed centroid copy and half squared norms for the next iteration,
+// centroid shift and the convergence test.  Every sum is taken in a fixed order.
+#pragma once
+
+#include "kmx_common.h"
+
+template <typename T>
+struct LloydTail {
+    T* sums_t;               // (d, k): sums on entry, the new centroids on exit
+    T* sizes;                // OUT (k)
+    uint32_t* empty_clusters;
+    const T* old_centroids_t;
+    T* cpack;
+    T* half_norms;
+    kmx_lloyd_status* status;
+    int d, k, dpad;
+};
+
+// Empty-cluster list (ascending) and heaviest cluster; one workgroup of 256 threads.
+// Returns the number of empty clusters (same value in every thread).
+template <typename T>
+__device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters, int k,
+                                       int* heaviest_out) {
+    __shared__ int wave_counts[4];
+    __shared__ T hv_val[4];
+    __shared__ int hv_idx[4];
+    __shared__ int result_s[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int base = 0;
+    T my_max = -kmx_inf<T>();
+    int my_arg = 0x7fffffff;
+    for (int c0 = 0; c0 < k; c0 += 256) {
+        const int c = c0 + threadIdx.x;
+        T sz = T(1);
+        if (c < k) {
+            sz = sizes[c];
+            if (sz > my_max) {
+                my_max = sz;
+                my_arg = c;
+            }
+        }
+        const bool flag = (c < k) && (sz == T(0));
+        const unsigned long long mask = __ballot(flag);
+        const int prefix = __popcll(mask & ((1ull << lane) - 1ull));
+        __syncthreads();
+        if (lane == 0) wave_counts[wave] = __popcll(mask);
+        __syncthreads();
+        int offset = base;
+        for (int w2 = 0; w2 < wave; ++w2) offset += wave_counts[w2];
+        if (flag) empty_clusters[offset + prefix] = (uint32_t)c;
+        base += wave_counts[0] + wave_counts[1] + wave_counts[2] + wave_counts[3];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const T ov = __shfl_xor(my_max, off, 64);
+        const int oi = __shfl_xor(my_arg, off, 64);
+        if (ov > my_max || (ov == my_max && oi < my_arg)) {
+            my_max = ov;
+            my_arg = oi;
+        }
+    }
+    __syncthreads();
+    if (lane == 0) {
+        hv_val[wave] = my_max;
+        hv_idx[wave] = my_arg;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T bv = hv_val[0];
+        int bidx = hv_idx[0];
+        for (int w2 = 1; w2 < 4; ++w2) {
+            if (hv_val[w2] > bv || (hv_val[w2] == bv && hv_idx[w2] < bidx)) {
+                bv = hv_val[w2];
+                bidx = hv_idx[w2];
+            }
+        }
+        result_s[0] = bidx;
+    }
+    __syncthreads();
+    *heaviest_out = result_s[0];
+    return base;
+}
+
+// Division, packed copy, half norms, shift and convergence test by ONE workgroup of 256
+// threads (thread per cluster, features in order).  `sums_t` becomes the new centroids.
+template <typename T>
+__device__ inline void lloyd_finalize_block(const LloydTail<T>& a, int n_empty, int heaviest) {
+    __shared__ double scratch[4];
+    const int d = a.d, k = a.k, dpad = a.dpad;
+    double shift = 0.0;
+    for (int c = threadIdx.x; c < k; c += 256) {
+        const T sz = a.sizes[c];
+        if (sz != T(0)) {
+            T sq = T(0), sh = T(0);
+#pragma unroll 2
+            for (int f = 0; f < d; ++f) {
+                const T nv = a.sums_t[(size_t)f * k + c] / sz;
+                const T df = a.old_centroids_t[(size_t)f * k + c] - nv;
+                sh += df * df;
+                sq += nv * nv;
+                a.cpack[(size_t)c * dpad + f] = nv;
+                a.sums_t[(size_t)f * k + c] = nv;
+            }
+            for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = T(0);
+            a.half_norms[c] = sq / T(2);
+            shift += (double)sh;
+        }
+    }
+    __syncthreads();
+    if (n_empty > 0) {
+        // still-empty clusters (nothing could be relocated) are parked on the heaviest one
+        for (int c = threadIdx.x; c < k; c += 256) {
+            if (a.sizes[c] == T(0)) {
+                T sq = T(0), sh = T(0);
+                for (int f = 0; f < d; ++f) {
+                    const T nv = a.cpack[(size_t)heaviest * dpad + f];
+                    const T df = a.old_centroids_t[(size_t)f * k + c] - nv;
+                    sh += df * df;
+                    sq += nv * nv;
+                    a.cpack[(size_t)c * dpad + f] = nv;
+                    a.sums_t[(size_t)f * k + c] = nv;
+                }
+                for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = T(0);
+                a.half_norms[c] = sq / T(2);
+                shift += (double)sh;
+            }
+        }
+    }
+    const double total = kmx_block_sum<double>(shift, scratch);
+    if (threadIdx.x == 0) {
+        kmx_lloyd_status* st = a.status;
+        const int n_iter = st->n_iter + 1;
+        const unsigned int changed = st->n_changed;
+        st->n_iter = n_iter;
+        st->shift_sum = total;
+        st->n_changed = 0;
+        int next = KMX_RUNNING;
+        if (n_iter > 1 && changed == 0)
+            next = KMX_CONVERGED_STRICT;
+        else if (!(total > st->tol))
+            next = KMX_CONVERGED_TOL;
+        else if (n_iter >= st->max_iter)
+            next = KMX_MAX_ITER;
+        st->state = next;
+        st->reserved[1] = (int64_t)changed;
+    }
+}
+

@@ -61,7 +61,8 @@ def lloyd(
     empty_list = torch.empty(k, dtype=torch.int32, device=dev)
     verbose = bool(verbose)
 
-    check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(cent[0]), n, d, k, dc, int(max_iter), float(tol), stream),
+    check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), n, d, k, dc, int(max_iter),
+                             float(tol), stream),
           "kmx_lloyd_init")
 
     status = LloydStatus()

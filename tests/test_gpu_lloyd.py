@@ -60,7 +60,7 @@ def test_single_iteration_through_c_abi(cuda, name):
     ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(c_in), n, d, k, dc, 100, 0.0, stream), "init")
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), n, d, k, dc, 100, 0.0, stream), "init")
     _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
                                    ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, dc, stream), "iter")
     status = _capi.LloydStatus()
@@ -115,7 +115,7 @@ def test_lockstep_iterations_match_oracle(cuda, name):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
     status = _capi.LloydStatus()
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(cent[0]), n, d, k, dc, 100, 0.0, stream), "init")
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, 100, 0.0, stream), "init")
     prev = None
     for it in range(10):
         a, b = it % 2, (it + 1) % 2
