@@ -27,6 +27,8 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-munsafe-fp-atomics",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go to architectural VGPRs: the argmax reads them without accvgpr moves
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
 ]
 

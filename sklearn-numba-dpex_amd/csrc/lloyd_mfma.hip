@@ -102,7 +102,11 @@ __global__ void fixed_point_exponents_kernel(const unsigned int* __restrict__ ab
 
 // ---------------------------------------------------------------------------- fused step
 
-template <int NKS, bool UPDATE>
+// NKS = K steps held in registers.  EXACT: the shape has exactly NKS steps, so the K loop has
+// no guards and the body of the centroid-block loop is one basic block (the scheduler can
+// hoist the LDS reads of the A fragments above the MFMAs); otherwise steps s >= nks are
+// skipped with wave-uniform branches.
+template <int NKS, bool EXACT, bool UPDATE>
 __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
@@ -112,7 +116,7 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
     if (UPDATE && status->state != KMX_RUNNING) return;
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const int nks = (d + 1) >> 1;          // K steps of 2 features
+    const int nks = EXACT ? NKS : (d + 1) >> 1;  // K steps of 2 features
     const int n_cb = (k + 31) >> 5;        // centroid blocks of 32
     const int items = (d + 1) * k;
     unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [(d + 1) * k]
@@ -359,18 +363,26 @@ int32_t launch_mfma(const LloydLayout& L, const void* X_t, const void* w, const 
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
                        (!UPDATE || (aligned16(w) && aligned16(labels_prev)));
-#define KMX_MFMA_CASE(NKS)                                                                     \
-    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, UPDATE>), dim3((unsigned)grid), dim3(256), lds, \
-                       stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,  \
-                       labels_prev, labels, status, q_exp, gsum, n, d, k, vec_ok)
-    if (d <= 8)
-        KMX_MFMA_CASE(4);
-    else if (d <= 16)
-        KMX_MFMA_CASE(8);
-    else if (d <= 32)
-        KMX_MFMA_CASE(16);
-    else
-        KMX_MFMA_CASE(32);
+#define KMX_MFMA_CASE(NKS, EXACT)                                                              \
+    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, EXACT, UPDATE>), dim3((unsigned)grid), dim3(256), \
+                       lds, stream, (const float*)X_t, (const float*)w,                          \
+                       (const float*)centroids_t, labels_prev, labels, status, q_exp, gsum, n, d, \
+                       k, vec_ok)
+    switch ((d + 1) / 2) {
+        case 1: KMX_MFMA_CASE(1, true); break;
+        case 2: KMX_MFMA_CASE(2, true); break;
+        case 3: KMX_MFMA_CASE(3, true); break;
+        case 4: KMX_MFMA_CASE(4, true); break;
+        case 5: KMX_MFMA_CASE(5, true); break;
+        case 6: KMX_MFMA_CASE(6, true); break;
+        case 7: KMX_MFMA_CASE(7, true); break;
+        case 8: KMX_MFMA_CASE(8, true); break;
+        default:
+            if (d <= 32)
+                KMX_MFMA_CASE(16, false);
+            else
+                KMX_MFMA_CASE(32, false);
+    }
 #undef KMX_MFMA_CASE
     KMX_LAUNCH_CHECK();
     return KMX_OK;
