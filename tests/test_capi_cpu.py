@@ -1,0 +1,154 @@
+"""The C-ABI library without a GPU: it loads, exports every function the header declares,
+answers the size queries and rejects bad arguments before touching the device."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi355x_kmeans.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kmx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_function():
+    from sklearn_numba_dpex_amd import _capi
+
+    declared = _declared_functions()
+    assert len(declared) >= 35
+    raw = ctypes.CDLL(_capi.LIB_PATH)
+    for name in declared:
+        assert hasattr(raw, name), f"{name} is declared in the header but not exported"
+    assert sorted(_capi.SIGNATURES) == declared, "ctypes signatures and header disagree"
+    assert _capi.lib.kmx_abi_version() == 1
+
+
+def test_header_cites_the_reference_for_every_entry_point():
+    text = open(HEADER).read()
+    # every declaration block mentions the reference file it replaces, or says it has none
+    for name in _declared_functions():
+        if name in ("kmx_abi_version", "kmx_error_string") or name.endswith("_workspace_bytes") \
+                or name.endswith("_ptr") or name in ("kmx_lloyd_status_read", "kmx_lloyd_kernel_variant"):
+            continue
+        idx = text.index(name + "(")
+        comment = text[text.rfind("/*", 0, idx):idx]
+        assert re.search(r"\.py:\d+|no\s+counterpart", comment), f"{name}: no reference citation"
+
+
+def test_error_strings_and_codes():
+    from sklearn_numba_dpex_amd import _capi
+
+    assert _capi.error_string(0) == "ok"
+    assert "null" in _capi.error_string(-1)
+    assert "workspace" in _capi.error_string(-4)
+    with pytest.raises(_capi.KmxError) as e:
+        _capi.check(-2, "somewhere")
+    assert e.value.code == -2 and "somewhere" in str(e.value)
+
+
+def test_workspace_queries():
+    from sklearn_numba_dpex_amd._capi import lib
+
+    small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0)
+    assert 0 < small < 64 << 20
+    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) == small  # independent of n
+    assert lib.kmx_lloyd_workspace_bytes(1_000_000, 256, 1024, 0) > (32 << 20)  # global copies
+    assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0) == 0
+    assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7) == 0
+    assert lib.kmx_assign_workspace_bytes(14, 127, 0) > 127 * 16 * 4
+    assert lib.kmx_kpp_workspace_bytes(1_000_000, 64, 256, 7, 0) >= 7 * 4_000_000
+    assert lib.kmx_kpp_workspace_bytes(1000, 4, 8, 17, 0) == 0  # more trials than supported
+    assert lib.kmx_topk_workspace_bytes(1000, 10) > 0
+    assert lib.kmx_topk_workspace_bytes(5, 10) == 0
+    assert lib.kmx_sum_workspace_bytes(7, 1_000_000) >= 7 * 256 * 8
+
+
+def test_kernel_variant_selection():
+    from sklearn_numba_dpex_amd._capi import lib
+
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 31   # MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 11    # fp64: register + LDS
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 2  # streaming + global copies
+    assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0) == 11           # too few clusters for MFMA
+    assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0) == -2
+    assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4) == -3
+
+
+def test_bad_arguments_are_rejected_without_a_device():
+    from sklearn_numba_dpex_amd._capi import lib
+
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    NULL = None
+    assert lib.kmx_lloyd_init(NULL, 0, p, p, p, 10, 2, 2, 0, 10, 0.0, NULL) == -1
+    assert lib.kmx_lloyd_init(p, 4096, p, p, p, 0, 2, 2, 0, 10, 0.0, NULL) == -2
+    assert lib.kmx_lloyd_init(p, 4096, p, p, p, 10, 2, 2, 9, 10, 0.0, NULL) == -3
+    assert lib.kmx_lloyd_init(p, 16, p, p, p, 10, 2, 2, 0, 10, 0.0, NULL) == -4
+    assert lib.kmx_lloyd_iter(p, p, p, p, p, p, p, p, p, 16, 10, 2, 2, 0, NULL) == -4
+    assert lib.kmx_lloyd_iter(p, NULL, p, p, p, p, p, p, p, 4096, 10, 2, 2, 0, NULL) == -1
+    assert lib.kmx_assign_labels(p, p, NULL, p, 4096, 10, 2, 2, 0, NULL) == -1
+    assert lib.kmx_per_sample_inertia(p, NULL, p, p, p, 0, 2, 2, 0, NULL) == -2
+    assert lib.kmx_euclidean_distances(p, p, p, 10, 2, 2, 5, NULL) == -3
+    assert lib.kmx_topk_idx(p, p, 5, 10, p, 4096, 0, NULL) == -5      # k > n
+    assert lib.kmx_topk_idx(p, p, 50, 10, p, 8, 0, NULL) == -4
+    assert lib.kmx_broadcast_rows(p, p, 2, 2, 3, 0, NULL) == -5       # unknown op
+    assert lib.kmx_kpp_init(p, p, 20, p, p, p, 1 << 20, 10, 2, 2, 2, 0, NULL) in (-4, -5)
+    assert lib.kmx_kpp_run(p, p, p, 0, p, p, p, 16, 10, 2, 2, 2, 0, NULL) == -4
+    assert lib.kmx_kpp_step(p, p, 1, p, p, p, 16, 10, 2, 2, 99, 0, NULL) == -6  # too many trials
+    assert lib.kmx_relocate_empty_clusters(p, p, p, p, p, 3, NULL, p, p, 10, 2, 2, 0, NULL) == -2
+    assert lib.kmx_sum_rows(p, p, 0, 5, 0, p, 4096, 0, NULL) == -2
+    assert lib.kmx_matmul(p, p, NULL, 2, 2, 2, 0, NULL) == -1
+    assert lib.kmx_argmin(p, p, 0, 0, NULL) == -2
+
+
+def test_engine_surface_and_host_checks_without_gpu():
+    from sklearn.cluster import KMeans as SkKMeans
+
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine, NotSupportedByEngineError
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    for method in ["accepts", "prepare_fit", "init_centroids", "kmeans_single", "is_same_clustering",
+                   "count_distinct_clusters", "unshift_centers", "prepare_prediction", "get_labels",
+                   "get_score", "prepare_transform", "get_euclidean_distances", "convert_to_sklearn_types"]:
+        assert callable(getattr(KMeansEngine, method))
+    assert KMeansEngine.engine_name == "kmeans"
+    engine = KMeansEngine(SkKMeans(algorithm="elkan"))
+    assert engine.accepts(np.zeros((3, 2)), None, None) is False
+    engine = KMeansEngine(SkKMeans(algorithm="lloyd"))
+    assert engine.accepts(np.zeros((3, 2)), None, None) is True
+    import scipy.sparse as sp
+
+    assert engine.accepts(sp.csr_matrix(np.eye(3)), None, None) is False
+    assert issubclass(KMeans, SkKMeans)
+    assert issubclass(NotSupportedByEngineError, Exception)
+
+
+def test_testing_mode_env_is_validated(monkeypatch):
+    from sklearn.cluster import KMeans as SkKMeans
+
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine, NotSupportedByEngineError
+
+    monkeypatch.setenv("SKLEARN_NUMBA_DPEX_TESTING_MODE", "2")
+    with pytest.raises(ValueError, match="SKLEARN_NUMBA_DPEX_TESTING_MODE"):
+        KMeansEngine(SkKMeans())
+    monkeypatch.setenv("SKLEARN_NUMBA_DPEX_TESTING_MODE", "1")
+    with pytest.raises(NotSupportedByEngineError):
+        KMeansEngine(SkKMeans(algorithm="elkan")).accepts(np.zeros((3, 2)), None, None)
+
+
+def test_missing_gpu_fails_loudly():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    with pytest.raises(RuntimeError, match="needs a ROCm GPU"):
+        drivers.get_labels_inertia(torch.zeros(2, 3), torch.zeros(2, 2), torch.ones(3), False)

@@ -1,0 +1,176 @@
+"""GPU parity of the shared kernels (sums, argmin, top-k, elementwise, matmul, label helpers),
+restating the reference's common/tests and kmeans/tests cases against numpy."""
+
+import numpy as np
+import pytest
+
+from oracle import kmeans as ok
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+def _dev(a, cuda):
+    import torch
+
+    return torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+
+
+# reference common/tests/test_reductions.py:16-68
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 3), (3, 1), (3, 5), (5, 3), (3, 4), (4, 3), (3, 9), (7, 20011)])
+def test_sum_reduction_2d(cuda, shape, axis, dtype):
+    from sklearn_numba_dpex_amd.common.reductions import sum_reduction
+
+    a = np.arange(shape[0] * shape[1], dtype=dtype).reshape(shape) % 1000
+    got = sum_reduction(_dev(a, cuda), axis=axis).cpu().numpy()
+    np.testing.assert_allclose(got, a.sum(axis=axis, dtype=np.float64), rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sum_reduction_1d_square_and_determinism(cuda, dtype):
+    from sklearn_numba_dpex_amd.common.reductions import sum_reduction
+
+    for length, expected in [(4, 6), (5, 10)]:
+        assert sum_reduction(_dev(np.arange(length, dtype=dtype), cuda)).cpu().numpy()[0] == pytest.approx(expected)
+    rng = np.random.default_rng(0)
+    v = rng.normal(size=3_000_017).astype(dtype)
+    d = _dev(v, cuda)
+    s1 = sum_reduction(d, square=True).cpu().numpy()[0]
+    s2 = sum_reduction(d, square=True).cpu().numpy()[0]
+    assert s1 == s2  # fixed summation order
+    assert s1 == pytest.approx(float(np.sum(v.astype(np.float64) ** 2)), rel=1e-6)
+
+
+# reference common/tests/test_reductions.py:109-133
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("values, expected", [([3.0, 1.0, 0.0, 2.0], 2), ([0.0, 1.0, 3.0, 2.0], 0),
+                                              ([3.0, 1.0, 2.0, -1.0, -2.0], 4), ([5.0, 1.0, 1.0, 7.0], 1)])
+def test_argmin(cuda, values, expected, dtype):
+    import torch
+
+    from sklearn_numba_dpex_amd.common.reductions import argmin_reduction
+
+    out = argmin_reduction(_dev(np.array(values, dtype=dtype), cuda))
+    assert out.dtype == torch.int32
+    assert int(out.cpu()[0]) == expected
+    rng = np.random.default_rng(1)
+    big = rng.normal(size=50_000).astype(dtype)
+    big[[123, 40_000]] = -100.0
+    assert int(argmin_reduction(_dev(big, cuda)).cpu()[0]) == 123
+
+
+TOPK_CASES = [
+    [0, 1, -2, -3, 4, -5, 6, 7, 8, -9, 10],
+    [0, 8, -2, -3, 4, -5, 6, 7, 8, -9, 10],
+    [0, 8, -2, -3, 4, -5, 6, 7, 8, -9, 8],
+    [0, 8, 8, -3, 4, -5, 6, 7, 8, -9, 10],
+    [0, 8, 8, -3, 4, -5, 6, 7, 8, -9, 8],
+    [8, 8, 8, 8, 8, 8, 8, 8, 8, 8, 8],
+]
+
+
+# reference common/tests/test_topk.py:28-59 (+ our deterministic order policy)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [1, 3, 11])
+@pytest.mark.parametrize("case", range(len(TOPK_CASES)))
+def test_topk_handcrafted(cuda, case, k, dtype):
+    from sklearn_numba_dpex_amd.common.topk import topk, topk_idx
+
+    a = np.array(TOPK_CASES[case], dtype=dtype)
+    idx = topk_idx(_dev(a, cuda), k).cpu().numpy()
+    np.testing.assert_array_equal(idx, ok.top_k_indices(a, k))  # descending value, ascending index
+    np.testing.assert_array_equal(np.sort(a[idx]), np.sort(a)[-k:])
+    np.testing.assert_array_equal(np.sort(topk(_dev(a, cuda), k).cpu().numpy()), np.sort(a)[-k:])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_topk_multirow_and_random(cuda, dtype):
+    from sklearn_numba_dpex_amd.common.topk import topk, topk_idx
+
+    a = np.array(TOPK_CASES, dtype=dtype)
+    got = topk(_dev(a, cuda), 3).cpu().numpy()
+    np.testing.assert_array_equal(np.sort(got, axis=1), np.sort(a, axis=1)[:, -3:])
+    rng = np.random.default_rng(123)
+    big = rng.normal(size=(8, 1000)).astype(dtype)  # reference uses (1000, 1000); same per-row path
+    for k in (1, 3):
+        idx = topk_idx(_dev(big, cuda), k).cpu().numpy()
+        for r in range(big.shape[0]):
+            np.testing.assert_array_equal(idx[r], ok.top_k_indices(big[r], k))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_topk_large_with_ties_and_negatives(cuda, dtype):
+    from sklearn_numba_dpex_amd.common.topk import topk_idx
+
+    rng = np.random.default_rng(5)
+    v = rng.normal(size=1_000_003).astype(dtype)
+    v[rng.choice(v.size, 5000, replace=False)] = np.float32(2.5)  # many ties at the threshold
+    v[::7] *= -1
+    for k in (1, 16, 300):
+        idx = topk_idx(_dev(v, cuda), k).cpu().numpy()
+        np.testing.assert_array_equal(idx, ok.top_k_indices(v, k))
+    with pytest.raises(ValueError, match="Expected k to be greater than or equal"):
+        topk_idx(_dev(v[:5], cuda), 6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_elementwise_kernels(cuda, dtype):
+    from sklearn_numba_dpex_amd.common import kernels
+
+    rng = np.random.default_rng(2)
+    a = rng.normal(size=(5, 1003)).astype(dtype)
+    v_rows = rng.normal(size=5).astype(dtype)
+    v_cols = rng.uniform(1, 2, 1003).astype(dtype)
+    d = _dev(a, cuda)
+    np.testing.assert_array_equal(kernels.half_l2_norm(d).cpu().numpy().shape, (1003,))
+    np.testing.assert_allclose(kernels.half_l2_norm(d).cpu().numpy(), ok.half_sq_norms(a.T), rtol=1e-6)
+    kernels.broadcast_rows(d, _dev(v_rows, cuda), "minus")
+    np.testing.assert_array_equal(d.cpu().numpy(), a - v_rows[:, None])
+    kernels.broadcast_rows(d, _dev(v_rows, cuda), "plus")
+    np.testing.assert_allclose(d.cpu().numpy(), a, atol=1e-6)
+    d = _dev(a, cuda)
+    kernels.broadcast_division(d, _dev(v_cols, cuda))
+    np.testing.assert_array_equal(d.cpu().numpy(), a / v_cols[None, :])
+    d = _dev(a, cuda)
+    kernels.divide_by(d, 7.0)
+    np.testing.assert_array_equal(d.cpu().numpy(), a / dtype(7.0))
+    b = rng.normal(size=(5, 1003)).astype(dtype)
+    np.testing.assert_allclose(kernels.centroid_shifts(_dev(a, cuda), _dev(b, cuda)).cpu().numpy(),
+                               ((a - b) ** 2).sum(axis=0), rtol=1e-6)
+    kernels.initialize_to_zeros(d)
+    assert float(d.abs().sum()) == 0.0
+
+
+# reference common/tests/test_matmul.py:71-127
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 2), (16, 16, 16), (65, 17, 130), (1999, 661, 563)])
+def test_matmul(cuda, shape, dtype):
+    from sklearn_numba_dpex_amd.common.matmul import matmul
+
+    m, p, q = shape
+    rng = np.random.default_rng(0)
+    X = rng.normal(size=(m, p)).astype(dtype)
+    Y_t = rng.normal(size=(q, p)).astype(dtype)
+    got = matmul(_dev(X, cuda), _dev(Y_t, cuda)).cpu().numpy()
+    np.testing.assert_allclose(got, X.astype(np.float64) @ Y_t.astype(np.float64).T,
+                               rtol=1e-4 if dtype == np.float32 else 1e-11, atol=1e-4 if dtype == np.float32 else 1e-11)
+
+
+def test_label_helpers(cuda):
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    # reference kmeans/tests/test_kmeans.py:448-457
+    labels = _dev(np.array([0, 1, 0, 2, 2, 7, 6, 5, 3, 3], dtype=np.int32), cuda)
+    assert int(drivers.get_nb_distinct_clusters(labels, 8)) == 7
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 50, 200_000).astype(np.int32)
+    perm = rng.permutation(50).astype(np.int32)
+    b = perm[a]
+    c = b.copy()
+    c[77_777] = (c[77_777] + 1) % 50
+    assert drivers.is_same_clustering(_dev(a, cuda), _dev(b, cuda), 50) is True
+    assert drivers.is_same_clustering(_dev(a, cuda), _dev(c, cuda), 50) is False
+    assert int(drivers.get_nb_distinct_clusters(_dev(a, cuda), 50)) == len(np.unique(a))

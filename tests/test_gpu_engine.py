@@ -1,0 +1,283 @@
+"""The engine behind the estimator, against scikit-learn: the reference's integration tests
+(sklearn_numba_dpex/kmeans/tests/test_kmeans.py) restated for this engine, plus the forced
+empty-cluster configuration and input/ error handling."""
+
+import numpy as np
+import pytest
+from numpy.testing import assert_array_equal
+from sklearn.base import clone
+from sklearn.cluster import KMeans as SkKMeans
+from sklearn.cluster._kmeans import _is_same_clustering
+from sklearn.datasets import make_blobs
+from sklearn.utils._testing import assert_allclose
+
+from oracle import datasets
+from oracle import kmeans as ok
+from tests._parity import assert_centers_close, assert_labels_match
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+def _np(v):
+    return v.cpu().numpy() if hasattr(v, "cpu") else np.asarray(v)
+
+
+def _as_cuda(a, dtype):
+    import torch
+
+    return torch.as_tensor(np.asarray(a, dtype=dtype), device="cuda")
+
+
+# reference test_kmeans.py:28-110
+@pytest.mark.parametrize("kind", ["numpy", "torch_cuda", "torch_cuda+convert", "numpy_fortran"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kmeans_same_results(cuda, dtype, kind):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans, config_context
+
+    X, _ = make_blobs(random_state=42)
+    X = X.astype(dtype)
+    X_array = {"numpy": X, "numpy_fortran": np.asfortranarray(X)}.get(kind)
+    if X_array is None:
+        X_array = _as_cuda(X, dtype)
+    convert = "sklearn_types" if kind.endswith("+convert") else None
+
+    kmeans_truth = SkKMeans(random_state=42, algorithm="lloyd", max_iter=2, n_init=2, init="random")
+    kmeans_engine = KMeans(**kmeans_truth.get_params())
+    kmeans_truth.fit(X)
+    with config_context(engine_attributes=convert):
+        kmeans_engine.fit(X_array)
+    if convert:
+        assert isinstance(kmeans_engine.labels_, np.ndarray) and isinstance(kmeans_engine.cluster_centers_, np.ndarray)
+
+    def same_fit():
+        assert_array_equal(kmeans_truth.labels_, _np(kmeans_engine.labels_))
+        assert_allclose(kmeans_truth.cluster_centers_, _np(kmeans_engine.cluster_centers_))
+        assert_allclose(kmeans_truth.inertia_, kmeans_engine.inertia_)
+        assert kmeans_truth.n_iter_ == kmeans_engine.n_iter_
+
+    same_fit()
+    assert_array_equal(kmeans_truth.fit_predict(X), _np(kmeans_engine.fit_predict(X_array)))
+    same_fit()
+    assert_allclose(kmeans_truth.fit_transform(X), _np(kmeans_engine.fit_transform(X_array)))
+    same_fit()
+    assert_array_equal(kmeans_truth.predict(X), _np(kmeans_engine.predict(X_array)))
+    assert_allclose(kmeans_truth.score(X), kmeans_engine.score(X_array))
+    assert_allclose(kmeans_truth.transform(X), _np(kmeans_engine.transform(X_array)))
+
+
+# reference test_kmeans.py:113-122
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kmeans_predict_centers(cuda, dtype):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    kmeans = KMeans(n_clusters=10)
+    centers = kmeans.cluster_centers_ = _as_cuda(np.arange(100).reshape(10, 10), dtype)
+    kmeans.n_features_in_ = 10
+    assert_array_equal(_np(kmeans.predict(centers)), np.arange(10))
+
+
+# reference test_kmeans.py:125-158
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kmeans_relocated_clusters(cuda, dtype):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X = np.array([[0, 0], [0.5, 0], [0.5, 1], [1, 1]], dtype=dtype)
+    init_centers = np.array([[0.5, 0.5], [3, 3]], dtype=dtype)
+    kmeans = KMeans(n_clusters=2, n_init=1, init=init_centers).fit(X)
+    assert_allclose(kmeans.inertia_, 0.25)
+    assert kmeans.n_iter_ == 3
+    labels, centers = _np(kmeans.labels_), _np(kmeans.cluster_centers_)
+    if labels[0] == 0:
+        assert_array_equal(labels, [0, 0, 1, 1])
+        assert_allclose(centers, [[0.25, 0], [0.75, 1]])
+    else:
+        assert_array_equal(labels, [1, 1, 0, 0])
+        assert_allclose(centers, [[0.75, 1.0], [0.25, 0.0]])
+
+
+# reference test_kmeans.py:161-179
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_euclidean_distance(cuda, dtype):
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine
+
+    rng = np.random.default_rng(42)
+    a = rng.random(size=(1, 100), dtype=dtype)
+    b = rng.standard_normal((1, 100), dtype=dtype)
+    estimator = SkKMeans(n_clusters=len(b))
+    estimator.cluster_centers_ = b
+    estimator.n_features_in_ = 100
+    result = KMeansEngine(estimator).get_euclidean_distances(a)
+    assert tuple(result.shape) == (1, 1)
+    assert_allclose(_np(result), np.sqrt(((a - b) ** 2).sum()), rtol=1e-4 if dtype == np.float32 else 1e-7)
+
+
+# reference test_kmeans.py:182-205 (signed weights)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_inertia(cuda, dtype):
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine
+
+    rng = np.random.default_rng(42)
+    X = rng.random((100, 10), dtype=dtype)
+    sample_weight = rng.standard_normal(100, dtype=dtype)
+    centers = rng.standard_normal((5, 10), dtype=dtype)
+    estimator = SkKMeans(n_clusters=len(centers))
+    estimator.cluster_centers_ = _as_cuda(centers, dtype)
+    estimator.n_features_in_ = 10
+    engine = KMeansEngine(estimator)
+    X_prepared, sw = engine.prepare_prediction(X, sample_weight)
+    labels = _np(engine.get_labels(X_prepared, sw))
+    expected = float(np.sum(((X - centers[labels]) ** 2).sum(axis=1) * sample_weight))
+    inertia = engine.get_score(X_prepared, sw)
+    assert_allclose(float(inertia), expected, rtol=1e-4 if dtype == np.float32 else 1e-6)
+
+
+# reference test_kmeans.py:208-248
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_relocate_empty_clusters(cuda, dtype):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X = np.array([-10.0, -9.5, -9.0, -8.5, -8.0, -1.0, 1.0, 9.0, 9.5, 10.0], dtype=dtype).reshape(-1, 1)
+    init_centers = np.array([-10.0, -10.0, -10.0]).reshape(-1, 1)
+    kmeans_truth = SkKMeans(n_clusters=3, n_init=1, max_iter=1, init=init_centers, algorithm="lloyd")
+    kmeans_engine = KMeans(**kmeans_truth.get_params())
+    kmeans_truth.fit(X)
+    kmeans_engine.fit(X)
+    truth_labels = kmeans_truth.labels_
+    engine_labels = _np(kmeans_engine.labels_).astype(np.int32)
+    assert kmeans_truth.n_iter_ == 1 and kmeans_engine.n_iter_ == 1
+    assert _is_same_clustering(truth_labels, engine_labels, n_clusters=3)
+    assert _is_same_clustering(truth_labels, np.asarray([0, 0, 0, 0, 0, 0, 0, 2, 2, 1], dtype=np.int32), n_clusters=3)
+    assert_allclose(kmeans_truth.cluster_centers_[truth_labels], _np(kmeans_engine.cluster_centers_)[engine_labels])
+    assert_allclose(kmeans_truth.inertia_, kmeans_engine.inertia_)
+
+
+def test_forced_empty_clusters_config5(cuda):
+    """fp64, 16 of 64 initial centroids far away: they empty on iteration 1 and are relocated
+    onto the farthest samples by the radix select; compared with the oracle iteration by
+    iteration until the first relocation is through, then on the final result."""
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    cfg = datasets.config5(n=60_000)
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    mean = X.mean(axis=0)
+    Xc, initc = X - mean, init - mean
+    tol = float(np.mean(np.var(Xc, axis=0)) * cfg["tol"])
+    X_t = torch.as_tensor(np.ascontiguousarray(Xc.T), device=cuda)
+    w_d = torch.as_tensor(w, device=cuda)
+    for relocation in ("sklearn", "literal"):
+        labels, inertia, centers_t, n_iter = drivers.lloyd(
+            X_t, w_d, torch.as_tensor(np.ascontiguousarray(initc.T), device=cuda), True,
+            max_iter=1, tol=tol, relocation=relocation)
+        it = next(ok.lloyd_iterations(Xc, w, initc, max_iter=1, tol=tol, relocation=relocation))
+        assert it["n_empty"] == 16 and n_iter == 1
+        assert_centers_close(centers_t.cpu().numpy().T, it["centers"], np.float64, scale_rtol=1e-11)
+    labels, inertia, centers_t, n_iter = drivers.lloyd(
+        X_t, w_d, torch.as_tensor(np.ascontiguousarray(initc.T), device=cuda), True, max_iter=100, tol=tol)
+    ref_labels, ref_inertia, ref_centers, ref_n_iter = ok.lloyd(Xc, w, initc, max_iter=100, tol=tol)
+    assert n_iter == ref_n_iter
+    assert_labels_match(labels.cpu().numpy(), ref_labels, Xc, ref_centers)
+    assert_centers_close(centers_t.cpu().numpy().T, ref_centers, np.float64, scale_rtol=1e-10)
+    assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-12)
+    assert len(np.unique(labels.cpu().numpy())) == 64
+
+
+def test_more_clusters_than_distinct_points(cuda):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X = np.repeat(np.array([[0.0, 0.0], [1.0, 1.0]]), 5, axis=0)
+    init = np.array([[0.0, 0.0], [1.0, 1.0], [5.0, 5.0]])
+    with pytest.warns(Warning, match="distinct clusters"):
+        km = KMeans(n_clusters=3, n_init=1, init=init).fit(X)
+    assert np.isfinite(_np(km.cluster_centers_)).all()
+    assert km.inertia_ == pytest.approx(0.0, abs=1e-12)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kmeans_plusplus_fit_quality_and_weights(cuda, dtype):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, y = make_blobs(n_samples=3000, n_features=5, centers=6, cluster_std=0.6, random_state=3)
+    X = X.astype(dtype)
+    w = np.random.default_rng(0).uniform(0.5, 1.5, 3000).astype(dtype)
+    km = KMeans(n_clusters=6, init="k-means++", n_init=1, random_state=0).fit(X, sample_weight=w)
+    sk = SkKMeans(n_clusters=6, init="k-means++", n_init=3, random_state=0).fit(X, sample_weight=w)
+    assert km.inertia_ <= sk.inertia_ * 1.05
+    # uniform scalar weight == no weight
+    a = KMeans(n_clusters=6, init=X[:6].copy(), n_init=1).fit(X)
+    b = KMeans(n_clusters=6, init=X[:6].copy(), n_init=1).fit(X, sample_weight=np.full(3000, 1.0))
+    assert_array_equal(_np(a.labels_), _np(b.labels_))
+
+
+def test_verbose_output_and_callable_init(cuda, capsys):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, _ = make_blobs(n_samples=500, centers=4, random_state=0)
+
+    def init(X_, n_clusters, random_state):
+        return X_[:n_clusters]  # rows of the (centred, device-resident) data the engine passes in
+
+    km = KMeans(n_clusters=4, init=init, n_init=1, verbose=1, max_iter=50).fit(X)
+    out = capsys.readouterr().out
+    assert "Iteration 0, inertia" in out
+    assert "Converged at iteration" in out
+    sk = SkKMeans(n_clusters=4, init=X[:4].copy(), n_init=1, max_iter=50).fit(X)
+    assert km.n_iter_ == sk.n_iter_
+    assert_allclose(_np(km.cluster_centers_), sk.cluster_centers_)
+
+
+def test_copy_x_false_restores_a_device_input(cuda):
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, _ = make_blobs(n_samples=400, centers=3, random_state=1)
+    X = X + 50.0
+    X_dev = torch.as_tensor(np.asfortranarray(X).T.copy(), device=cuda).T  # F-ordered device tensor
+    before = X_dev.cpu().numpy().copy()
+    KMeans(n_clusters=3, init=X[:3].copy(), n_init=1, copy_x=False).fit(X_dev)
+    np.testing.assert_allclose(X_dev.cpu().numpy(), before, rtol=1e-12, atol=1e-9)
+    X_np = X.copy()
+    KMeans(n_clusters=3, init=X[:3].copy(), n_init=1, copy_x=True).fit(X_np)
+    assert_array_equal(X_np, X)
+
+
+def test_input_validation_errors(cuda):
+    import scipy.sparse as sp
+
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine, NotSupportedByEngineError
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, _ = make_blobs(n_samples=50, centers=3, random_state=1)
+    with pytest.raises(ValueError, match="should be >= n_clusters"):
+        KMeans(n_clusters=60, n_init=1).fit(X)
+    with pytest.raises(ValueError, match="sample_weight.shape"):
+        KMeans(n_clusters=3, n_init=1).fit(X, sample_weight=np.ones(49))
+    with pytest.raises(ValueError, match="NaN|infinity"):
+        bad = X.copy()
+        bad[3, 1] = np.nan
+        KMeans(n_clusters=3, n_init=1).fit(bad)
+    with pytest.raises(ValueError, match="does not match the number of clusters"):
+        KMeans(n_clusters=3, n_init=1, init=X[:4].copy()).fit(X)
+    km = KMeans(n_clusters=3, n_init=1, random_state=0).fit(X)
+    with pytest.raises(ValueError, match="features"):
+        km.predict(X[:, :1])
+    with pytest.raises(NotSupportedByEngineError):
+        KMeansEngine(SkKMeans())._validate_data(sp.csr_matrix(X))
+    # elkan is not accepted: the estimator falls back to scikit-learn
+    ek = KMeans(n_clusters=3, n_init=1, algorithm="elkan", random_state=0).fit(X)
+    assert isinstance(ek.labels_, np.ndarray)
+
+
+def test_integer_and_float16_inputs_are_converted(cuda):
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, _ = make_blobs(n_samples=300, centers=3, random_state=2)
+    Xi = np.round(X * 10).astype(np.int64)
+    km = KMeans(n_clusters=3, init=Xi[:3].astype(np.float64), n_init=1).fit(Xi)
+    sk = SkKMeans(n_clusters=3, init=Xi[:3].astype(np.float64), n_init=1).fit(Xi)
+    assert_array_equal(_np(km.labels_), sk.labels_)
+    assert_allclose(_np(km.cluster_centers_), sk.cluster_centers_)

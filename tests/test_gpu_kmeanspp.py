@@ -1,0 +1,164 @@
+"""GPU parity of kmeans++ seeding: each kernel family through the C ABI against the oracle's
+exact sampler, the whole seeding against the oracle, and the reference's known answer."""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import datasets
+from oracle import kmeans as ok
+from oracle import rng as orng
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, cuda):
+    import torch
+
+    return torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+
+
+def _cases():
+    rng = np.random.default_rng(11)
+    Xw = rng.normal(size=(5003, 5))
+    return {
+        "C4": (datasets.config4(n=40_000, d=64, k=24)["X"], None, 24, 3),
+        "weighted_f64": (Xw, rng.uniform(0.1, 3.0, 5003), 9, 1),
+        "tiny_f32": (rng.normal(size=(37, 2)).astype(np.float32), None, 4, 0),
+        "wide_f32": (rng.normal(size=(3000, 150)).astype(np.float32), None, 5, 2),
+    }
+
+
+@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32"])
+def test_whole_seeding_matches_oracle(cuda, name):
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    X, w, k, seed = _cases()[name]
+    w = np.ones(len(X), X.dtype) if w is None else w.astype(X.dtype)
+    centers_t, idx = drivers.kmeans_plusplus(_dev(X.T, cuda), _dev(w, cuda), k, np.random.RandomState(seed))
+    seed64 = orng.seed_from_random_state(np.random.RandomState(seed))
+    ref_centers, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact")
+    idx = idx.cpu().numpy()
+    np.testing.assert_array_equal(idx, ref_idx)
+    np.testing.assert_array_equal(centers_t.cpu().numpy().T, X[idx])
+    assert idx.dtype == np.int32 and np.all((idx >= 0) & (idx < len(X)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_step_kernels_through_c_abi(cuda, dtype):
+    """init -> sample -> step with the same uniforms as the oracle: candidates, potentials and
+    the updated closest-distance array all match."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    rng = np.random.default_rng(3)
+    n, d, k, tn = 10_007, 6, 8, 4
+    X = rng.normal(size=(n, d)).astype(dtype)
+    w = rng.uniform(0.5, 1.5, n).astype(dtype)
+    dc = _capi.dtype_code(dtype)
+    X_t, w_d = _dev(X.T, cuda), _dev(w, cuda)
+    centers_t = torch.zeros((d, k), dtype=X_t.dtype, device=cuda)
+    indices = torch.full((k,), -1, dtype=torch.int32, device=cuda)
+    ws_bytes = lib.kmx_kpp_workspace_bytes(n, d, k, tn, dc)
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=cuda)
+    st = _capi.current_stream()
+    start = 4242
+    _capi.check(lib.kmx_kpp_init(ptr(X_t), ptr(w_d), start, ptr(centers_t), ptr(indices), ptr(ws), ws_bytes,
+                                 n, d, k, tn, dc, st), "kpp_init")
+    closest = (((X - X[start]) ** 2).sum(axis=1, dtype=dtype) * w).astype(dtype)
+    rows_ptr = lib.kmx_kpp_closest_ptr(ptr(ws), n, d, k, tn, dc)
+    off = rows_ptr - ws.data_ptr()
+    itemsize = np.dtype(dtype).itemsize
+
+    def row(r):
+        return ws[off + r * n * itemsize: off + (r + 1) * n * itemsize].view(X_t.dtype).cpu().numpy()
+
+    np.testing.assert_allclose(row(0), closest, rtol=1e-5 if dtype == np.float32 else 1e-12)
+    closest = row(0).copy()  # continue from the device's own values: later comparisons are exact
+    assert int(indices.cpu()[0]) == start
+    np.testing.assert_array_equal(centers_t.cpu().numpy()[:, 0], X[start])
+
+    best_row = 0
+    for c in range(1, k):
+        u = rng.random(tn)
+        u[0] = 0.0 if c == 1 else u[0]            # rv == 0 -> first sample (reference would give -1)
+        u[1] = 1.0 - 2.0**-53 if c == 2 else u[1]  # top of the range -> last crossing, clipped to n - 1
+        cand = torch.empty(tn, dtype=torch.int32, device=cuda)
+        _capi.check(lib.kmx_kpp_sample_candidates(ptr(_dev(u, cuda)), ptr(cand), ptr(ws), ws_bytes, n, d, k, tn,
+                                                  dc, st), "kpp_sample")
+        expected = np.array([ok._sample_exact(closest, uu) for uu in u])
+        np.testing.assert_array_equal(cand.cpu().numpy(), expected)
+        _capi.check(lib.kmx_kpp_step(ptr(X_t), ptr(w_d), c, ptr(centers_t), ptr(indices), ptr(ws), ws_bytes,
+                                     n, d, k, tn, dc, st), "kpp_step")
+        rows = np.stack([np.minimum((((X - X[i]) ** 2).sum(axis=1, dtype=dtype) * w).astype(dtype), closest)
+                         for i in expected])
+        pots_ptr = lib.kmx_kpp_potentials_ptr(ptr(ws), n, d, k, tn, dc)
+        poff = pots_ptr - ws.data_ptr()
+        pots = ws[poff: poff + tn * 8].view(torch.float64).cpu().numpy()
+        for t in range(tn):
+            np.testing.assert_allclose(row(t), rows[t], rtol=1e-5 if dtype == np.float32 else 1e-12)
+        got_rows = np.stack([row(t) for t in range(tn)])
+        np.testing.assert_allclose(pots, got_rows.sum(axis=1, dtype=np.float64), rtol=1e-12)
+        best_row = int(np.argmin(pots))
+        assert int(indices.cpu()[c]) == expected[best_row]
+        np.testing.assert_array_equal(centers_t.cpu().numpy()[:, c], X[expected[best_row]])
+        closest = got_rows[best_row].copy()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_known_answer_through_the_engine(cuda, dtype):
+    """reference kmeans/tests/test_kmeans.py:251-325: mean score over seeds 0..9 of the
+    engine's kmeans++ initialisation is -865.257501."""
+    from sklearn.cluster import KMeans as SkKMeans
+    from sklearn.cluster.tests.test_k_means import X as X_sk, n_clusters
+
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine
+
+    X = X_sk.astype(dtype)
+    kmeans = SkKMeans(n_clusters=n_clusters, init="k-means++")
+    kmeans._n_threads = 1
+    scores = []
+    for random_state in range(10):
+        kmeans.set_params(random_state=random_state)
+        engine = KMeansEngine(kmeans)
+        X_prepared, _, sample_weight = engine.prepare_fit(X)
+        centers_t = engine.init_centroids(X_prepared, sample_weight)
+        centers = centers_t.T
+        engine.unshift_centers(X_prepared, centers)
+        kmeans.cluster_centers_ = np.ascontiguousarray(centers.cpu().numpy())
+        scores.append(kmeans.score(X))
+    np.testing.assert_allclose(np.mean(scores), -865.257501, rtol=1e-7)
+
+
+def test_output_sanity_and_data_order(cuda):
+    """reference kmeans/tests/test_kmeans.py:328-392."""
+    from sklearn.cluster import KMeans as SkKMeans
+    from sklearn.cluster.tests.test_k_means import X as X_sk, n_clusters
+
+    from sklearn_numba_dpex_amd.kmeans.engine import KMeansEngine
+
+    for dtype in (np.float32, np.float64):
+        X = X_sk.astype(dtype)
+        sample_weight = np.random.default_rng(42).random(X.shape[0], dtype=dtype)
+        est = SkKMeans(init="k-means++", n_clusters=n_clusters, random_state=42)
+        engine = KMeansEngine(est)
+        X_prepared, _, sw = engine.prepare_fit(X, sample_weight=sample_weight)
+        centers_t, indices = engine._kmeans_plusplus(X_prepared, sw)
+        centers = centers_t.T
+        engine.unshift_centers(X_prepared, centers)
+        centers, indices = centers.cpu().numpy(), indices.cpu().numpy()
+        assert indices.shape[0] == n_clusters and (indices >= 0).all() and (indices < X.shape[0]).all()
+        assert (centers.max(axis=0) <= X.max(axis=0) + 1e-5).all() and (centers.min(axis=0) >= X.min(axis=0) - 1e-5).all()
+        np.testing.assert_allclose(X[indices], centers, rtol=1e-5, atol=1e-6)
+
+    est = SkKMeans(init="k-means++", n_clusters=n_clusters, random_state=42)
+    engine = KMeansEngine(est)
+    Xp, _, sw = engine.prepare_fit(X_sk)
+    centers_c = engine.init_centroids(Xp, sw).T.cpu().numpy()
+    engine = KMeansEngine(est)
+    Xp, _, sw = engine.prepare_fit(np.asfortranarray(X_sk))
+    centers_f = engine.init_centroids(Xp, sw).T.cpu().numpy()
+    np.testing.assert_allclose(centers_c, centers_f)

@@ -1,0 +1,225 @@
+"""Pins the numpy oracle: against scikit-learn's Cython Lloyd (the reference's own oracle,
+sklearn_numba_dpex/kmeans/tests/test_kmeans.py:39-110), against the known answers the
+reference's tests hold, and against closed forms / brute force chosen so that a dropped term,
+a wrong sign or a transposed operand fails."""
+
+import numpy as np
+import pytest
+from sklearn.cluster import KMeans
+from sklearn.cluster._kmeans import _kmeans_single_lloyd, _labels_inertia
+from sklearn.datasets import make_blobs
+from sklearn.utils import check_random_state
+
+from oracle import datasets
+from oracle import kmeans as ok
+from oracle import rng as orng
+
+
+def _blobs(n, d, k, dtype, seed=0):
+    X, _ = make_blobs(n_samples=n, n_features=d, centers=k, random_state=seed)
+    X = X.astype(dtype)
+    X -= X.mean(axis=0)
+    rng = np.random.default_rng(seed)
+    w = rng.uniform(0.5, 1.5, n).astype(dtype)
+    init = X[rng.choice(n, k, replace=False)].copy()
+    return X, w, init
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_lloyd_matches_sklearn(dtype):
+    X, w, init = _blobs(6000, 7, 12, dtype)
+    labels, inertia, centers, n_iter = ok.lloyd(X, w, init, max_iter=100, tol=0)
+    sl, si, sc, sn = _kmeans_single_lloyd(X, w, init.copy(), max_iter=100, tol=0, n_threads=2)
+    assert n_iter == sn
+    np.testing.assert_array_equal(labels, sl)
+    np.testing.assert_allclose(centers, sc, rtol=1e-4 if dtype == np.float32 else 1e-10, atol=1e-5 if dtype == np.float32 else 1e-12)
+    assert inertia == pytest.approx(si, rel=1e-5 if dtype == np.float32 else 1e-12)
+
+
+def test_labels_are_brute_force_argmin_with_lowest_index_ties():
+    rng = np.random.default_rng(1)
+    X = rng.normal(size=(500, 6))
+    C = rng.normal(size=(9, 6))
+    C[5] = C[2]  # exact duplicate: every sample closest to it must get label 2, never 5
+    labels = ok.assign_labels(X, C)
+    d2 = ((X[:, None, :] - C[None, :, :]) ** 2).sum(axis=2)
+    brute = np.argmin(d2, axis=1)
+    assert not np.any(labels == 5)
+    np.testing.assert_array_equal(labels, brute)
+    sk_labels, _ = _labels_inertia(X, np.ones(500), C, n_threads=1)
+    assert np.mean(sk_labels == labels) > 0.99
+
+
+def test_predict_centers_gives_arange():
+    # reference test_kmeans.py:113-122
+    for dtype in (np.float32, np.float64):
+        C = np.arange(100, dtype=dtype).reshape(10, 10)
+        np.testing.assert_array_equal(ok.assign_labels(C, C), np.arange(10))
+
+
+def test_half_sq_norms_closed_form():
+    C = np.arange(12, dtype=np.float64).reshape(3, 4)
+    np.testing.assert_allclose(ok.half_sq_norms(C), (C**2).sum(axis=1) / 2)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_inertia_closed_form_with_signed_weights(dtype):
+    # reference test_kmeans.py:182-205
+    rng = np.random.default_rng(42)
+    X = rng.random((100, 10), dtype=dtype)
+    w = rng.standard_normal(100, dtype=dtype)
+    C = rng.standard_normal((5, 10), dtype=dtype)
+    labels = ok.assign_labels(X, C)
+    expected = float(np.sum(((X - C[labels]) ** 2).sum(axis=1) * w))
+    assert float(ok.inertia(X, w, C, labels)) == pytest.approx(expected, rel=1e-4 if dtype == np.float32 else 1e-10)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_euclidean_distance_closed_form(dtype):
+    # reference test_kmeans.py:161-179
+    from scipy.spatial.distance import cdist
+
+    rng = np.random.default_rng(42)
+    a = rng.random(size=(1, 100), dtype=dtype)
+    b = rng.standard_normal((1, 100), dtype=dtype)
+    assert ok.euclidean_distances(a, b)[0, 0] == pytest.approx(np.sqrt(((a - b) ** 2).sum()), rel=1e-4 if dtype == np.float32 else 1e-7)
+    A = rng.random((30, 7)).astype(dtype)
+    B = rng.random((4, 7)).astype(dtype)
+    np.testing.assert_allclose(ok.euclidean_distances(A, B), cdist(A, B), rtol=1e-5)
+
+
+def test_relocated_clusters_toy():
+    # reference test_kmeans.py:125-158: inertia 0.25, 3 iterations, one of two symmetric answers
+    for dtype in (np.float32, np.float64):
+        X = np.array([[0, 0], [0.5, 0], [0.5, 1], [1, 1]], dtype=dtype)
+        init = np.array([[0.5, 0.5], [3, 3]], dtype=dtype)
+        Xc, mean, initc, tol, _ = ok.prepare_data_for_lloyd(X, init, 1e-4, np.ones(4, dtype))
+        labels, inertia, centers, n_iter = ok.lloyd(Xc, np.ones(4, dtype), initc, 300, tol)
+        centers = ok.restore_data_after_lloyd(centers, mean)
+        assert n_iter == 3
+        assert float(inertia) == pytest.approx(0.25)
+        if labels[0] == 0:
+            np.testing.assert_array_equal(labels, [0, 0, 1, 1])
+            np.testing.assert_allclose(centers, [[0.25, 0], [0.75, 1]])
+        else:
+            np.testing.assert_array_equal(labels, [1, 1, 0, 0])
+            np.testing.assert_allclose(centers, [[0.75, 1], [0.25, 0]])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_relocate_empty_clusters_matches_sklearn(dtype):
+    # reference test_kmeans.py:208-248
+    X = np.array([-10.0, -9.5, -9.0, -8.5, -8.0, -1.0, 1.0, 9.0, 9.5, 10.0], dtype=dtype).reshape(-1, 1)
+    init = np.array([-10.0, -10.0, -10.0], dtype=dtype).reshape(-1, 1)
+    km = KMeans(n_clusters=3, n_init=1, max_iter=1, init=init, algorithm="lloyd").fit(X)
+    Xc, mean, initc, tol, _ = ok.prepare_data_for_lloyd(X, init.copy(), 1e-4, np.ones(10, dtype))
+    labels, inertia, centers, n_iter = ok.lloyd(Xc, np.ones(10, dtype), initc, 1, tol)
+    centers = ok.restore_data_after_lloyd(centers, mean)
+    assert n_iter == 1 and km.n_iter_ == 1
+    assert ok.is_same_clustering(km.labels_, labels, 3)
+    assert ok.is_same_clustering(labels, [0, 0, 0, 0, 0, 0, 0, 2, 2, 1], 3)
+    np.testing.assert_allclose(km.cluster_centers_[km.labels_], centers[labels.astype(int)], rtol=1e-5)
+    assert float(inertia) == pytest.approx(km.inertia_, rel=1e-5)
+
+
+def test_relocation_arithmetic_matches_sklearn_helper():
+    from sklearn.cluster._k_means_common import _relocate_empty_clusters_dense
+
+    rng = np.random.default_rng(3)
+    X = rng.normal(size=(200, 4))
+    w = rng.uniform(0.5, 2.0, 200)
+    centers_old = np.vstack([rng.normal(size=(3, 4)), np.full((2, 4), 50.0)])
+    labels = ok.assign_labels(X, centers_old).astype(np.int32)
+    sums, sizes = ok.weighted_sums(X, w, labels, 5)
+    sk_sums, sk_sizes = sums.copy(), sizes.copy()
+    _relocate_empty_clusters_dense(X, w, centers_old, sk_sums, sk_sizes, labels)
+    sq = ok.sq_dist_to_assigned(X, centers_old, labels)
+    far = ok.relocate_empty_clusters(X, w, sums, sizes, labels, sq)
+    assert set(far.tolist()) == set(np.argsort(sq)[-2:].tolist())
+    # sklearn pairs far samples with empty clusters in argpartition order: compare as sets of rows
+    np.testing.assert_allclose(np.sort(sums[3:], axis=0), np.sort(sk_sums[3:], axis=0))
+    np.testing.assert_allclose(sums[:3], sk_sums[:3])
+    np.testing.assert_allclose(np.sort(sizes), np.sort(sk_sizes))
+
+
+def test_top_k_indices_policy():
+    v = np.array([0, 8, 8, -3, 4, -5, 6, 7, 8, -9, 8], dtype=np.float32)
+    np.testing.assert_array_equal(ok.top_k_indices(v, 3), [1, 2, 8])
+    np.testing.assert_array_equal(ok.top_k_indices(v, 5), [1, 2, 8, 10, 7])
+    with pytest.raises(ValueError):
+        ok.top_k_indices(v, 12)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("sampler", ["literal", "exact"])
+def test_kmeans_plusplus_known_answer(dtype, sampler):
+    # reference test_kmeans.py:251-325: mean score over seeds 0..9 of the engine's kmeans++
+    from sklearn.cluster.tests.test_k_means import X as X_sk, n_clusters
+
+    X = X_sk.astype(dtype)
+    km = KMeans(n_clusters=n_clusters, init="k-means++")
+    km._n_threads = 1
+    scores = []
+    for rs in range(10):
+        w = np.ones(len(X), dtype)
+        Xc, mean, _, _, _ = ok.prepare_data_for_lloyd(X, "k-means++", 1e-4, w)
+        seed = orng.seed_from_random_state(check_random_state(rs))
+        centers, idx = ok.kmeans_plusplus(Xc, w, n_clusters, seed, sampler=sampler)
+        np.testing.assert_array_equal(centers, Xc[idx])
+        assert np.all((idx >= 0) & (idx < len(X)))
+        km.cluster_centers_ = np.ascontiguousarray(ok.restore_data_after_lloyd(centers, mean))
+        scores.append(km.score(X))
+    np.testing.assert_allclose(np.mean(scores), -865.257501, rtol=1e-7)
+
+
+def test_kmeans_plusplus_samplers_agree_and_follow_the_potential():
+    cfg = datasets.config4(n=3000, d=8, k=12)
+    X, w = cfg["X"], cfg["sample_weight"]
+    seed = orng.seed_from_random_state(np.random.RandomState(cfg["seed"]))
+    c1, i1, trace = ok.kmeans_plusplus(X, w, 12, seed, sampler="exact", return_trace=True)
+    c2, i2 = ok.kmeans_plusplus(X, w, 12, seed, sampler="literal")
+    np.testing.assert_array_equal(i1, i2)
+    # the chosen candidate minimises the potential among the trials, potentials never increase
+    pots = [t[1][t[2]] for t in trace]
+    assert all(t[1][t[2]] == t[1].min() for t in trace)
+    assert all(b <= a * (1 + 1e-12) for a, b in zip(pots, pots[1:]))
+
+
+def test_prepare_data_for_lloyd_centering_and_tol():
+    from sklearn.cluster._kmeans import _tolerance
+
+    rng = np.random.default_rng(0)
+    X = rng.normal(3.0, 2.0, size=(400, 5))
+    init = X[:3].copy()
+    Xc, mean, initc, tol, uniform = ok.prepare_data_for_lloyd(X, init, 1e-4, np.ones(400))
+    np.testing.assert_allclose(mean, X.mean(axis=0))
+    np.testing.assert_allclose(Xc, X - X.mean(axis=0))
+    np.testing.assert_allclose(initc, init - X.mean(axis=0))
+    assert tol == pytest.approx(_tolerance(X, 1e-4), rel=1e-10)
+    assert uniform
+    assert not ok.prepare_data_for_lloyd(X, init, 1e-4, rng.uniform(1, 2, 400))[4]
+    # already centred data: no shift recorded
+    Z = np.array([[1.0, -1.0], [-1.0, 1.0]])
+    assert ok.prepare_data_for_lloyd(Z, "random", 0.0, np.ones(2))[1] is None
+
+
+def test_label_helpers():
+    from sklearn.cluster._k_means_common import _is_same_clustering
+
+    a = np.array([0, 1, 0, 2, 2], dtype=np.int32)
+    b = np.array([2, 0, 2, 1, 1], dtype=np.int32)
+    c = np.array([2, 0, 1, 1, 1], dtype=np.int32)
+    assert ok.is_same_clustering(a, b, 3) and _is_same_clustering(a, b, 3)
+    assert not ok.is_same_clustering(a, c, 3) and not _is_same_clustering(a, c, 3)
+    assert ok.count_distinct_clusters([0, 1, 0, 2, 2, 7, 6, 5, 3, 3]) == 7  # reference test_kmeans.py:448-457
+
+
+def test_dataset_generators_are_frozen():
+    c1 = datasets.config1(n=2000)
+    assert c1["X"].shape == (2000, 14) and c1["X"].dtype == np.float32 and c1["init"].shape == (127, 14)
+    assert float(c1["X"][0, 0]) == pytest.approx(float(datasets.config1(n=2000)["X"][0, 0]))
+    c5 = datasets.config5(n=4800)
+    assert c5["X"].dtype == np.float64 and c5["init"].shape == (64, 32)
+    assert np.all(c5["init"][48:] >= 1e3)
+    first = ok.assign_labels(c5["X"], c5["init"])
+    assert set(np.unique(first)).isdisjoint(range(48, 64))  # the far centroids start empty
