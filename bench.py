@@ -166,6 +166,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kpp", action="store_true", help="skip the kmeans++ leg")
     ap.add_argument("--cpu-iters", type=int, default=20)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run five 1 GiB device-to-device copies (calibration of HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -177,6 +179,16 @@ def main():
     n, d = cfg["X"].shape
     k = cfg["k"]
     log(f"[bench] data {n}x{d} k={k} generated in {time.time() - t0:.1f}s")
+
+    if args.copy_probe:
+        import torch
+
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     elapsed, kernel_ms, ties, variant = gpu_lloyd(cfg, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
