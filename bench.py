@@ -72,7 +72,7 @@ def gpu_lloyd(cfg, steps, warmup):
     def enqueue():
         nonlocal it
         a, b = it % 2, (it + 1) % 2
-        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
                                        ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k,
                                        dc, stream), "iter")
         it += 1
@@ -98,7 +98,7 @@ def gpu_lloyd(cfg, steps, warmup):
     timed = min(steps, 50)
     for _ in range(timed):
         a, b = it % 2, (it + 1) % 2
-        _capi.check(lib.kmx_lloyd_iter_timed(ptr(X_t), ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+        _capi.check(lib.kmx_lloyd_iter_timed(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
                                              ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d,
                                              k, dc, stream, ms), "iter_timed")
         it += 1

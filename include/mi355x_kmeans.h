@@ -94,14 +94,18 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
  * make_broadcast_division_1d_2d_axis0_kernel (common/kernels.py:38-145),
  * make_centroid_shifts_kernel (kmeans/kernels/utils.py:79-110) and the loop body of
  * lloyd(), kmeans/drivers.py:188-343.
+ *   X_rowmajor       IN   (n, d)  optional (may be NULL) row-major copy of the same data; used
+ *                                 only by the wide fp32 path (kmx_lloyd_kernel_variant == 42),
+ *                                 which then sums each cluster's rows instead of issuing one
+ *                                 global atomic per (sample, feature)
  *   centroids_t      IN   (d, k)  centroids the labels are computed from
  *   new_centroids_t  OUT  (d, k)  un-normalised sums if relocation is needed, else new centroids
  *   labels_prev      IN   (n)     labels of the previous iteration
  *   labels           OUT  (n)
  *   cluster_sizes    OUT  (k)     sum of weights per cluster
  *   empty_clusters   OUT  (k)     ids of empty clusters, ascending, first status.n_empty valid */
-int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* centroids_t,
-                       void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+int32_t kmx_lloyd_iter(const void* X_t, const void* X_rowmajor, const void* sample_weight,
+                       const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
                        void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                        size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                        void* stream);
@@ -111,8 +115,8 @@ int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* c
  * finalisation) to kernel_ms_host[0..2].  For benchmarks and profiling; it has no
  * counterpart in the reference, whose benchmark only times a whole fit
  * (benchmark/kmeans.py:163-165). */
-int32_t kmx_lloyd_iter_timed(const void* X_t, const void* sample_weight, const void* centroids_t,
-                             void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void* sample_weight,
+                             const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                              size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                              void* stream, float* kernel_ms_host);
@@ -128,8 +132,9 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t, const
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
 
 /* Which fused-step kernel kmx_lloyd_iter uses for a shape, as 10 * path + accumulation:
- * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32);
- * accumulation 1 = workgroup-private LDS accumulators, 2 = global copies with atomics. */
+ * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32) with the
+ * centroids resident in LDS, 4 = MFMA (fp32) with samples in registers and centroids streamed;
+ * accumulation 1 = workgroup-private LDS accumulators, 2 = global sums. */
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype);
 
 /* ------------------------------------------------------------------------------------ *

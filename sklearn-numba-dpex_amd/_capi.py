@@ -56,8 +56,8 @@ SIGNATURES = {
     "kmx_error_string": (c_char_p, [_I32]),
     "kmx_lloyd_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32]),
     "kmx_lloyd_init": (_I32, [_P, _SZ, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, c_double, _P]),
-    "kmx_lloyd_iter": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
-    "kmx_lloyd_iter_timed": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P,
+    "kmx_lloyd_iter": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
+    "kmx_lloyd_iter_timed": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P,
                                     POINTER(ctypes.c_float)]),
     "kmx_lloyd_finalize": (_I32, [_P, _P, _P, _P, _SZ, _I32, _I32, _I32, _P]),
     "kmx_lloyd_status_read": (_I32, [_P, POINTER(LloydStatus), _P]),

@@ -269,31 +269,47 @@ template <typename T>
 __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
     T* __restrict__ partial, int n_partials, int clear_partials, T* __restrict__ sums_t,
     T* __restrict__ sizes, uint32_t* __restrict__ empty_clusters,
-    kmx_lloyd_status* __restrict__ status, int d, int k) {
+    kmx_lloyd_status* __restrict__ status, int d, int k,
+    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp) {
     if (status->state != KMX_RUNNING) return;
     const int items = (d + 1) * k;
-    const int it = threadIdx.x & 31;
-    const int cl = threadIdx.x >> 5;
-    const int item = blockIdx.x * 32 + it;
-    __shared__ T red[8][32];
-    T s = T(0);
-    if (item < items) {
-        for (int g = cl; g < n_partials; g += 8) {
-            T* p = partial + (size_t)g * items + item;
-            s += *p;
-            if (clear_partials) *p = T(0);
+    if (gsum != nullptr) {
+        // 64-bit fixed-point sums of the matrix-core step: one thread per item converts and
+        // clears (launched with items / 256 blocks)
+        const int item = blockIdx.x * 256 + threadIdx.x;
+        if (item < items) {
+            const long long iv = (long long)gsum[item];
+            gsum[item] = 0ull;
+            const T v = (T)ldexp((double)iv, -q_exp[item / k]);
+            if (item < d * k)
+                sums_t[item] = v;
+            else
+                sizes[item - d * k] = v;
         }
-    }
-    red[cl][it] = s;
-    __syncthreads();
-    if (cl == 0 && item < items) {
-        T tot = red[0][it];
+    } else {
+        const int it = threadIdx.x & 31;
+        const int cl = threadIdx.x >> 5;
+        const int item = blockIdx.x * 32 + it;
+        __shared__ T red[8][32];
+        T s = T(0);
+        if (item < items) {
+            for (int g = cl; g < n_partials; g += 8) {
+                T* p = partial + (size_t)g * items + item;
+                s += *p;
+                if (clear_partials) *p = T(0);
+            }
+        }
+        red[cl][it] = s;
+        __syncthreads();
+        if (cl == 0 && item < items) {
+            T tot = red[0][it];
 #pragma unroll
-        for (int j = 1; j < 8; ++j) tot += red[j][it];
-        if (item < d * k)
-            sums_t[item] = tot;
-        else
-            sizes[item - d * k] = tot;
+            for (int j = 1; j < 8; ++j) tot += red[j][it];
+            if (item < d * k)
+                sums_t[item] = tot;
+            else
+                sizes[item - d * k] = tot;
+        }
     }
 
     // ---- last block: empty-cluster list + heaviest cluster
@@ -562,7 +578,7 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
 }
 
 template <typename T>
-int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
+int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_rowmajor, const void* w,
                         const void* centroids_t, void* new_centroids_t,
                         const uint32_t* labels_prev, uint32_t* labels, void* sizes,
                         uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
@@ -575,7 +591,17 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
 
     if (events) (void)hipEventRecord(events[0], stream);
     int n_partials_used = L.n_partials;
-    if (L.acc_mode == ACC_LDS) {
+    unsigned long long* gsum = nullptr;
+    const int* q_exp = nullptr;
+    if (L.variant == KMX_VARIANT_MFMA_WIDE) {
+        if constexpr (sizeof(T) == 4) {
+            const int32_t rc = kmx_lloyd_step_mfma_wide_f32(L, X_t, X_rowmajor, w, centroids_t,
+                                                            labels_prev, labels, ws, n, d, k, stream);
+            if (rc != KMX_OK) return rc;
+        }
+        gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
+        q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
+    } else if (L.acc_mode == ACC_LDS) {
         launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
                                  partial, status, n, d, k, stream);
         n_partials_used = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
@@ -586,9 +612,11 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* w,
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[1], stream);
     const int items = (d + 1) * k;
-    hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)kmx_cdiv(items, 32)), dim3(256), 0,
-                       stream, partial, n_partials_used, L.acc_mode == ACC_GLOBAL ? 1 : 0,
-                       (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k);
+    hipLaunchKernelGGL((lloyd_reduce_kernel<T>),
+                       dim3((unsigned)kmx_cdiv(items, gsum != nullptr ? 256 : 32)), dim3(256), 0,
+                       stream, partial, n_partials_used,
+                       (L.acc_mode == ACC_GLOBAL && gsum == nullptr) ? 1 : 0,
+                       (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k, gsum, q_exp);
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[2], stream);
     hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, 256)), dim3(256), 0,
@@ -669,11 +697,16 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),
                            (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
     KMX_LAUNCH_CHECK();
-    if (L.variant == KMX_VARIANT_MFMA) {
+    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE) {
         const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, stream);
         if (rc != KMX_OK) return rc;
     }
-    if (L.acc_mode == ACC_GLOBAL) {
+    if (L.variant == KMX_VARIANT_MFMA_WIDE) {
+        hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(4), dim3(256), 0, stream,
+                           (uint32_t*)(ws + L.off_bucket), (size_t)k);
+        KMX_LAUNCH_CHECK();
+    }
+    if (L.acc_mode == ACC_GLOBAL && L.partial_bytes > 0) {
         const size_t words = L.partial_bytes / 4;
         hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1024), dim3(256), 0, stream,
                            (uint32_t*)(ws + L.off_partial), words);
@@ -682,8 +715,9 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
     return KMX_OK;
 }
 
-static int32_t lloyd_iter_dispatch(const void* X_t, const void* sample_weight,
-                                   const void* centroids_t, void* new_centroids_t,
+static int32_t lloyd_iter_dispatch(const void* X_t, const void* X_rowmajor,
+                                   const void* sample_weight, const void* centroids_t,
+                                   void* new_centroids_t,
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                                    size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
@@ -707,27 +741,27 @@ static int32_t lloyd_iter_dispatch(const void* X_t, const void* sample_weight,
             return kmx_lloyd_iter_mfma_f32(L, X_t, sample_weight, centroids_t, new_centroids_t,
                                            labels_prev, labels, cluster_sizes, empty_clusters,
                                            (char*)workspace, n, d, k, stream, events);
-        return lloyd_iter_impl<float>(L, X_t, sample_weight, centroids_t, new_centroids_t,
+        return lloyd_iter_impl<float>(L, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t,
                                       labels_prev, labels, cluster_sizes, empty_clusters,
                                       (char*)workspace, n, d, k, stream, events);
     }
-    return lloyd_iter_impl<double>(L, X_t, sample_weight, centroids_t, new_centroids_t, labels_prev,
+    return lloyd_iter_impl<double>(L, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev,
                                    labels, cluster_sizes, empty_clusters, (char*)workspace, n, d, k,
                                    stream, events);
 }
 
-int32_t kmx_lloyd_iter(const void* X_t, const void* sample_weight, const void* centroids_t,
-                       void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+int32_t kmx_lloyd_iter(const void* X_t, const void* X_rowmajor, const void* sample_weight,
+                       const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
                        void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                        size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                        void* stream_) {
-    return lloyd_iter_dispatch(X_t, sample_weight, centroids_t, new_centroids_t, labels_prev, labels,
+    return lloyd_iter_dispatch(X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev, labels,
                                cluster_sizes, empty_clusters, workspace, workspace_bytes, n, d, k,
                                dtype, stream_, nullptr);
 }
 
-int32_t kmx_lloyd_iter_timed(const void* X_t, const void* sample_weight, const void* centroids_t,
-                             void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void* sample_weight,
+                             const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                              size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                              void* stream_, float* kernel_ms_host) {
@@ -737,7 +771,7 @@ int32_t kmx_lloyd_iter_timed(const void* X_t, const void* sample_weight, const v
         const hipError_t e = hipEventCreate(&ev[i]);
         if (e != hipSuccess) return (int32_t)e;
     }
-    int32_t rc = lloyd_iter_dispatch(X_t, sample_weight, centroids_t, new_centroids_t, labels_prev,
+    int32_t rc = lloyd_iter_dispatch(X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev,
                                      labels, cluster_sizes, empty_clusters, workspace,
                                      workspace_bytes, n, d, k, dtype, stream_, ev);
     if (rc == KMX_OK) {
@@ -761,7 +795,7 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,
     KMX_REQUIRE_DTYPE(dtype);
     // offsets of the status, packed centroids, half norms and shift slots do not depend on n
     const LloydLayout L = lloyd_layout(1, d, k, dtype);
-    if (workspace_bytes < L.off_partial) return KMX_ERR_WORKSPACE;
+    if (workspace_bytes < L.off_bucket) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
@@ -794,7 +828,7 @@ int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_ho
 
 size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
     if (d <= 0 || k <= 0 || (dtype != KMX_F32 && dtype != KMX_F64)) return 0;
-    return lloyd_layout(1, d, k, dtype).off_partial;
+    return lloyd_layout(1, d, k, dtype).off_bucket;
 }
 
 int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
@@ -807,7 +841,7 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
     LloydLayout L = lloyd_layout(n, d, k, dtype);
-    if (workspace_bytes < L.off_partial) return KMX_ERR_WORKSPACE;
+    if (workspace_bytes < L.off_bucket) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     const unsigned grid = (unsigned)kmx_cdiv(k, 256);
@@ -819,6 +853,8 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
         KMX_LAUNCH_CHECK();
         if (L.variant == KMX_VARIANT_MFMA)
             return kmx_assign_labels_mfma_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
+        if (L.variant == KMX_VARIANT_MFMA_WIDE)
+            return kmx_assign_labels_mfma_wide_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
         launch_fused<float, ACC_NONE>(L, X_t, nullptr, centroids_t, (const float*)(ws + L.off_cpack),
                                       (const float*)(ws + L.off_half), nullptr, labels, nullptr,
                                       nullptr, n, d, k, stream);

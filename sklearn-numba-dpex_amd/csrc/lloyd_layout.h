@@ -6,7 +6,8 @@
 
 constexpr int KMX_VARIANT_STREAM = 0;    // wide samples: features re-read per centroid window
 constexpr int KMX_VARIANT_REGISTER = 1;  // samples held in registers, centroids in SGPRs
-constexpr int KMX_VARIANT_MFMA = 3;      // fp32 distances on the matrix cores
+constexpr int KMX_VARIANT_MFMA = 3;      // fp32 distances on the matrix cores, LDS accumulators
+constexpr int KMX_VARIANT_MFMA_WIDE = 4; // fp32 matrix cores, samples in registers, global sums
 
 constexpr int KMX_ACC_LDS = 1;
 constexpr int KMX_ACC_GLOBAL = 2;
@@ -19,8 +20,10 @@ constexpr size_t KMX_GLOBAL_COPIES_BYTES = 64u << 20;
 // KMX_LLOYD_WGS_PER_CU = 1..8.
 int kmx_forced_variant();
 int kmx_wgs_per_cu();
-// Shapes the fp32 matrix-core fused step covers (operands and accumulators fit in LDS).
+// Shapes the fp32 matrix-core fused step covers (operands and accumulators fit in LDS), and
+// those its wide-sample variant covers (samples in registers, centroids streamed).
 bool kmx_mfma_supported(int d, int k);
+bool kmx_mfma_wide_supported(int d, int k);
 
 struct LloydLayout {
     int dpad;            // features per packed centroid row (multiple of 4, zero padded)
@@ -28,7 +31,7 @@ struct LloydLayout {
     int acc_mode;        // KMX_ACC_*
     int n_partials;      // slots in `partial` (workgroups for LDS mode, copies for global mode)
     int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
-    size_t off_status, off_scales, off_gsum, off_cpack, off_half, off_shift, off_partial;
+    size_t off_status, off_scales, off_gsum, off_cpack, off_half, off_shift, off_bucket, off_partial;
     size_t partial_bytes;
     size_t total;
     // Workgroups of the fused step: a few per compute unit (KMX_LLOYD_WGS_PER_CU, default 4),
@@ -46,7 +49,6 @@ static inline int lloyd_reg_samples_per_thread(int d, int dtype) {
 
 
 static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
-    (void)n;
     LloydLayout L;
     const size_t s = kmx_dtype_size(dtype);
     L.dpad = (d + 3) & ~3;
@@ -70,6 +72,8 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_supported(d, k) &&
         (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA;
+    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA))
+        L.variant = KMX_VARIANT_MFMA_WIDE;
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
     L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));
@@ -77,9 +81,14 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     L.off_cpack = L.off_gsum + kmx_align256(items * sizeof(long long));
     L.off_half = L.off_cpack + kmx_align256((size_t)k * L.dpad * s);
     L.off_shift = L.off_half + kmx_align256((size_t)k * s);
-    L.off_partial = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 256) * sizeof(double));
+    L.off_bucket = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 256) * sizeof(double));
+    // wide matrix-core path: counts (k), offsets (k + 1), cursors (k), sample order (n) as int32
+    const size_t bucket_bytes =
+        L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)3 * k + 1 + (size_t)n) * sizeof(int) : 0;
+    L.off_partial = L.off_bucket + kmx_align256(bucket_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
-    L.partial_bytes = L.variant == KMX_VARIANT_MFMA ? 0 : (size_t)L.n_partials * items * s;
+    const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE;
+    L.partial_bytes = fixed_point ? 0 : (size_t)L.n_partials * items * s;
     L.total = L.off_partial + kmx_align256(L.partial_bytes);
     return L;
 }
@@ -96,3 +105,12 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
 int32_t kmx_assign_labels_mfma_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
                                    uint32_t* labels, char* ws, int64_t n, int d, int k,
                                    hipStream_t stream);
+// wide-sample variant (lloyd_mfma_wide.hip): the fused step only; the reduction and
+// finalisation kernels of lloyd.hip follow it
+int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, const void* X_rowmajor,
+                                     const void* w, const void* centroids_t,
+                                     const uint32_t* labels_prev, uint32_t* labels, char* ws,
+                                     int64_t n, int d, int k, hipStream_t stream);
+int32_t kmx_assign_labels_mfma_wide_f32(const LloydLayout& L, const void* X_t,
+                                        const void* centroids_t, uint32_t* labels, char* ws,
+                                        int64_t n, int d, int k, hipStream_t stream);

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restric
 // n * max|w| * max|x_f| * 2^q < 2^61 and one sample's contribution stays below 2^50.
 __global__ void fixed_point_exponents_kernel(const unsigned int* __restrict__ absmax,
                                              int* __restrict__ q, int64_t n, int d) {
-    const int f = threadIdx.x;
+    const int f = blockIdx.x * blockDim.x + threadIdx.x;
     if (f > d) return;
     const float wmax = __uint_as_float(absmax[d]);
     const float xmax = f < d ? __uint_as_float(absmax[f]) : 1.0f;
@@ -400,10 +400,11 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
     int* q_exp = reinterpret_cast<int*>(absmax + (d + 1));
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(256), 0, stream, absmax, d + 1);
     int64_t gx = kmx_cdiv(n, 256 * 16);
-    if (gx > 1024) gx = 1024;
+    if (gx > 64) gx = 64;
     hipLaunchKernelGGL(absmax_rows_kernel, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
                        stream, (const float*)X_t, (const float*)w, absmax, n, d);
-    hipLaunchKernelGGL(fixed_point_exponents_kernel, dim3(1), dim3(128), 0, stream, absmax, q_exp, n, d);
+    hipLaunchKernelGGL(fixed_point_exponents_kernel, dim3((unsigned)kmx_cdiv(d + 1, 128)), dim3(128), 0,
+                       stream, absmax, q_exp, n, d);
     const size_t words = (size_t)(d + 1) * L.k_for_gsum * 2;
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(1024), 0, stream,
                        reinterpret_cast<unsigned int*>(ws + L.off_gsum), (int)words);

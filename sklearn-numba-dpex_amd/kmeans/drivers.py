@@ -61,6 +61,10 @@ def lloyd(
     empty_list = torch.empty(k, dtype=torch.int32, device=dev)
     verbose = bool(verbose)
 
+    # the wide fp32 path sums each cluster's rows from a row-major copy of X (one transpose per
+    # run, n * d extra elements of HBM) instead of one global atomic per (sample, feature)
+    X_rm = X_t.T.contiguous() if lib.kmx_lloyd_kernel_variant(n, d, k, dc) == 42 else None
+
     check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), n, d, k, dc, int(max_iter),
                              float(tol), stream),
           "kmx_lloyd_init")
@@ -71,7 +75,7 @@ def lloyd(
     while True:
         for _ in range(lookahead):
             a, b = enqueued % 2, (enqueued + 1) % 2
-            check(lib.kmx_lloyd_iter(ptr(X_t), ptr(sample_weight), ptr(cent[a]), ptr(cent[b]),
+            check(lib.kmx_lloyd_iter(ptr(X_t), ptr(X_rm), ptr(sample_weight), ptr(cent[a]), ptr(cent[b]),
                                      ptr(labels[a]), ptr(labels[b]), ptr(sizes), ptr(empty_list),
                                      ptr(ws), ws_bytes, n, d, k, dc, stream), "kmx_lloyd_iter")
             enqueued += 1

@@ -59,7 +59,7 @@ def test_workspace_queries():
     small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0)
     assert 0 < small < 64 << 20
     assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) == small  # independent of n
-    assert lib.kmx_lloyd_workspace_bytes(1_000_000, 256, 1024, 0) > (32 << 20)  # global copies
+    assert lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0) > (32 << 20)  # global copies
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0) == 0
     assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7) == 0
     assert lib.kmx_assign_workspace_bytes(14, 127, 0) > 127 * 16 * 4
@@ -75,7 +75,8 @@ def test_kernel_variant_selection():
 
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 31   # MFMA + LDS accumulators
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 11    # fp64: register + LDS
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 2  # streaming + global copies
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 42  # wide MFMA + global sums
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0) == 2   # streaming + global copies
     assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0) == 11           # too few clusters for MFMA
     assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0) == -2
     assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4) == -3
@@ -91,8 +92,8 @@ def test_bad_arguments_are_rejected_without_a_device():
     assert lib.kmx_lloyd_init(p, 4096, p, p, p, 0, 2, 2, 0, 10, 0.0, NULL) == -2
     assert lib.kmx_lloyd_init(p, 4096, p, p, p, 10, 2, 2, 9, 10, 0.0, NULL) == -3
     assert lib.kmx_lloyd_init(p, 16, p, p, p, 10, 2, 2, 0, 10, 0.0, NULL) == -4
-    assert lib.kmx_lloyd_iter(p, p, p, p, p, p, p, p, p, 16, 10, 2, 2, 0, NULL) == -4
-    assert lib.kmx_lloyd_iter(p, NULL, p, p, p, p, p, p, p, 4096, 10, 2, 2, 0, NULL) == -1
+    assert lib.kmx_lloyd_iter(p, NULL, p, p, p, p, p, p, p, p, 16, 10, 2, 2, 0, NULL) == -4
+    assert lib.kmx_lloyd_iter(p, NULL, NULL, p, p, p, p, p, p, p, 4096, 10, 2, 2, 0, NULL) == -1
     assert lib.kmx_assign_labels(p, p, NULL, p, 4096, 10, 2, 2, 0, NULL) == -1
     assert lib.kmx_per_sample_inertia(p, NULL, p, p, p, 0, 2, 2, 0, NULL) == -2
     assert lib.kmx_euclidean_distances(p, p, p, 10, 2, 2, 5, NULL) == -3
