@@ -124,6 +124,83 @@ def gpu_lloyd(cfg, steps, warmup):
     return elapsed, kernel_ms, ties, variant
 
 
+def gpu_lloyd_step_time(cfg, reps):
+    """Per-kernel times of ONE Lloyd iteration from the configuration's initial centroids
+    (the state is re-initialised before every repetition, so relocation or convergence never
+    turns a timed launch into a no-op).  Returns mean ms of (fused step, reduce, finalize)."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    dev = torch.device("cuda:0")
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    dc = _capi.dtype_code(X.dtype)
+    variant = lib.kmx_lloyd_kernel_variant(n, d, k, dc)
+    X_rm = torch.as_tensor(X, device=dev)
+    X_t = X_rm.T.contiguous()
+    if variant != 42:
+        X_rm = None
+    w_d = torch.as_tensor(w, device=dev)
+    cent = [torch.as_tensor(np.ascontiguousarray(init.T), device=dev), None]
+    cent[1] = torch.empty_like(cent[0])
+    labels = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(2)]
+    sizes = torch.empty(k, dtype=X_t.dtype, device=dev)
+    empty = torch.empty(k, dtype=torch.int32, device=dev)
+    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = _capi.current_stream()
+    ms = (ctypes.c_float * 3)()
+    acc = np.zeros(3)
+    for rep in range(reps + 2):
+        _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, 10, 0.0,
+                                       stream), "init")
+        _capi.check(lib.kmx_lloyd_iter_timed(ptr(X_t), ptr(X_rm), ptr(w_d), ptr(cent[0]), ptr(cent[1]),
+                                             ptr(labels[0]), ptr(labels[1]), ptr(sizes), ptr(empty), ptr(ws),
+                                             ws_bytes, n, d, k, dc, stream, ms), "iter_timed")
+        if rep >= 2:
+            acc += np.array(list(ms))
+    return acc / reps, int(variant)
+
+
+def extra_configs():
+    """Configs 3 (fp32, d=256, k=1024: matrix-core bound) and 5 (fp64, forced empty clusters)."""
+    from oracle import datasets
+
+    out = {}
+    t0 = time.time()
+    c3 = datasets.config3()
+    n, d = c3["X"].shape
+    kms, variant = gpu_lloyd_step_time(c3, 5)
+    flops = lloyd_flops(n, d, c3["k"])
+    out["config3"] = {
+        "workload": f"configs[2]: Lloyd n={n} d={d} k={c3['k']} fp32", "kernel_variant": variant,
+        "ms_per_iter": float(kms.sum()), "iters_per_sec": 1e3 / float(kms.sum()),
+        "kernel_ms": {"fused_step": float(kms[0]), "reduce": float(kms[1]), "finalize": float(kms[2])},
+        "fused_step_TFLOPs": flops / (kms[0] * 1e-3) / 1e12,
+        "fused_step_frac_of_fp32_peak": flops / (kms[0] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS,
+    }
+    log(f"[bench] config 3: {out['config3']['ms_per_iter']:.3f} ms/iter, fused step "
+        f"{out['config3']['fused_step_frac_of_fp32_peak']:.3f} of fp32 peak ({time.time() - t0:.1f}s incl. data)")
+    del c3
+    t0 = time.time()
+    c5 = datasets.config5()
+    n, d = c5["X"].shape
+    kms, variant = gpu_lloyd_step_time(c5, 5)
+    flops = lloyd_flops(n, d, c5["k"])
+    nbytes = lloyd_bytes(n, d, 8)
+    out["config5"] = {
+        "workload": f"configs[4]: Lloyd n={n} d={d} k={c5['k']} fp64, first iteration (16 empty clusters)",
+        "kernel_variant": variant, "ms_per_iter": float(kms.sum()),
+        "kernel_ms": {"fused_step": float(kms[0]), "reduce": float(kms[1]), "finalize": float(kms[2])},
+        "fused_step_frac_of_fp64_peak": flops / (kms[0] * 1e-3) / 1e12 / 78.6,
+        "fused_step_frac_of_hbm_peak": nbytes / (kms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    }
+    log(f"[bench] config 5: {out['config5']['ms_per_iter']:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
+    return out
+
+
 def gpu_kmeanspp(cfg):
     import torch
 
@@ -166,6 +243,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kpp", action="store_true", help="skip the kmeans++ leg")
     ap.add_argument("--cpu-iters", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="skip the config 3 / config 5 legs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run five 1 GiB device-to-device copies (calibration of HBM traffic counters)")
     args = ap.parse_args()
@@ -258,7 +336,14 @@ def main():
         log(f"[bench] kmeans++ {kpp_ms:.1f} ms ({time.time() - t0:.1f}s incl. data)")
         del c4
 
+    if not args.no_extra:
+        del cfg["X"]  # free host memory before the 1 GB configuration is generated
+        out["other_configs"] = extra_configs()
+        cfg = None
+
     if not args.no_cpu:
+        if cfg is None:
+            cfg = datasets.config2(n=args.n)
         cpu_ips, threads, cpu_iters, cpu_elapsed = cpu_lloyd_baseline(cfg, args.cpu_iters)
         out["cpu_baseline"] = {
             "value": cpu_ips,

@@ -193,9 +193,10 @@ int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_i
  * over the block potentials already held in the workspace.
  *   uniforms_for_step  IN  (n_trials) doubles in [0, 1)
  *   candidates         OUT (n_trials) int32, may be NULL (they stay in the workspace) */
-int32_t kmx_kpp_sample_candidates(const double* uniforms_for_step, int32_t* candidates,
-                                  void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
-                                  int32_t k, int32_t n_trials, int32_t dtype, void* stream);
+int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_step,
+                                  int32_t* candidates, void* workspace, size_t workspace_bytes,
+                                  int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype,
+                                  void* stream);
 
 /* For every candidate t and sample i: min(w_i ||x_i - x_cand_t||^2, closest_i), row sums,
  * argmin over t (lowest t wins ties), closest <- best row, centers_t[:, c] <- x_best,

@@ -69,7 +69,7 @@ SIGNATURES = {
     "kmx_relocate_empty_clusters": (_I32, [_P, _P, _P, _P, _P, _I32, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_kpp_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
     "kmx_kpp_init": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
-    "kmx_kpp_sample_candidates": (_I32, [_P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
+    "kmx_kpp_sample_candidates": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
     "kmx_kpp_step": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
     "kmx_kpp_run": (_I32, [_P, _P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
     "kmx_kpp_closest_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),

@@ -8,6 +8,8 @@
 //   block_pot   (n_blocks, 16) doubles: per-workgroup partial row sums; workgroup b owns the
 //               samples [b * 1024, (b + 1) * 1024), so these are also the coarse level of the
 //               sampler's two-level search
+//   cand_rows   (16, d): the feature rows of the current candidates, copied when they are
+//               sampled so that the step kernel reads them with wave-uniform (scalar) loads
 //   rows        (n_trials, n) in the compute dtype: min(w * ||x - x_cand||^2, closest) for
 //               every candidate; `closest` IS the best row, updated in place: a thread reads
 //               closest[i] before it writes column i of every row.
@@ -21,7 +23,6 @@ namespace {
 
 constexpr int TN_MAX = 16;      // n_local_trials = 2 + floor(ln k) <= 16 for k < 1.2e6
 constexpr int CHUNK = 1024;     // samples per workgroup (256 threads x 4)
-constexpr int FEAT_WINDOW = 128;
 
 struct KppHeader {
     int32_t best_row;
@@ -30,17 +31,18 @@ struct KppHeader {
 };
 
 struct KppLayout {
-    size_t off_header, off_cand, off_pot, off_block_pot, off_rows, total;
+    size_t off_header, off_cand, off_pot, off_cand_rows, off_block_pot, off_rows, total;
     int64_t n_blocks;
 };
 
-KppLayout kpp_layout(int64_t n, int n_trials, int dtype) {
+KppLayout kpp_layout(int64_t n, int d, int n_trials, int dtype) {
     KppLayout L;
     L.n_blocks = kmx_cdiv(n, CHUNK);
     L.off_header = 0;
     L.off_cand = 256;
     L.off_pot = 512;
-    L.off_block_pot = 768;
+    L.off_cand_rows = 768;  // (TN_MAX, d): the candidates' feature rows, read through scalar loads
+    L.off_block_pot = L.off_cand_rows + kmx_align256((size_t)TN_MAX * d * kmx_dtype_size(dtype));
     L.off_rows = L.off_block_pot + kmx_align256((size_t)L.n_blocks * TN_MAX * sizeof(double));
     L.total = L.off_rows + kmx_align256((size_t)n_trials * n * kmx_dtype_size(dtype));
     return L;
@@ -88,54 +90,59 @@ __global__ __launch_bounds__(256) void kpp_init_kernel(
 }
 
 // rows[t, i] = min(w_i * ||x_i - x_cand_t||^2, closest_i) and per-block row sums.
-template <typename T>
+// Candidate rows come from a small (TN, d) buffer through wave-uniform loads (the values sit
+// in SGPRs, no LDS, no barriers in the feature loop); every thread streams 4 consecutive
+// samples of 8 features at a time with 128-bit loads.
+template <typename T, int TN>
 __global__ __launch_bounds__(256) void kpp_step_kernel(
-    const T* __restrict__ X_t, const T* __restrict__ sample_weight,
-    const int32_t* __restrict__ candidates, T* __restrict__ rows, double* __restrict__ block_pot,
-    const KppHeader* __restrict__ header, int64_t n, int d, int n_trials, int vec_ok) {
-    __shared__ T cand[TN_MAX][FEAT_WINDOW];
+    const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cand_rows,
+    T* __restrict__ rows, double* __restrict__ block_pot, const KppHeader* __restrict__ header,
+    int64_t n, int d, int n_trials, int vec_ok) {
     __shared__ double scratch[4];
     const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
     const int best = header->best_row;
+    const bool full = vec_ok && (i0 + 4 <= n);
 
-    T acc[TN_MAX][4];
+    T acc[TN][4];
 #pragma unroll
-    for (int t = 0; t < TN_MAX; ++t)
+    for (int t = 0; t < TN; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[t][r] = T(0);
 
-    for (int f0 = 0; f0 < d; f0 += FEAT_WINDOW) {
-        const int fw = (d - f0 < FEAT_WINDOW) ? d - f0 : FEAT_WINDOW;
-        __syncthreads();
-        for (int j = threadIdx.x; j < n_trials * fw; j += 256) {
-            const int t = j / fw, f = j - t * fw;
-            cand[t][f] = X_t[(size_t)(f0 + f) * n + candidates[t]];
-        }
-        __syncthreads();
-        for (int f = 0; f < fw; ++f) {
-            const T* __restrict__ row = X_t + (size_t)(f0 + f) * n;
-            T xv[4];
-            if (vec_ok && i0 + 4 <= n) {
+    constexpr int FB = 8;  // features per batch of loads
+    for (int f0 = 0; f0 < d; f0 += FB) {
+        T xv[FB][4];
+#pragma unroll
+        for (int j = 0; j < FB; ++j) {
+            const int f = f0 + j < d ? f0 + j : d - 1;  // past the end: a valid row, ignored below
+            const T* __restrict__ row = X_t + (size_t)f * n;
+            if (full) {
                 if constexpr (sizeof(T) == 4) {
                     const float4 v = *reinterpret_cast<const float4*>(row + i0);
-                    xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+                    xv[j][0] = v.x; xv[j][1] = v.y; xv[j][2] = v.z; xv[j][3] = v.w;
                 } else {
                     const double2 a = *reinterpret_cast<const double2*>(row + i0);
                     const double2 b = *reinterpret_cast<const double2*>(row + i0 + 2);
-                    xv[0] = a.x; xv[1] = a.y; xv[2] = b.x; xv[3] = b.y;
+                    xv[j][0] = a.x; xv[j][1] = a.y; xv[j][2] = b.x; xv[j][3] = b.y;
                 }
             } else {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) xv[r] = (i0 + r < n) ? row[i0 + r] : T(0);
+                for (int r = 0; r < 4; ++r) xv[j][r] = (i0 + r < n) ? row[i0 + r] : T(0);
             }
+        }
 #pragma unroll
-            for (int t = 0; t < TN_MAX; ++t) {
-                if (t < n_trials) {
-                    const T cv = cand[t][f];
+        for (int t = 0; t < TN; ++t) {
+            if (t < n_trials) {
+                const T* __restrict__ cr = cand_rows + (size_t)t * d + f0;  // wave-uniform
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const T diff = xv[r] - cv;
-                        acc[t][r] = fma(diff, diff, acc[t][r]);
+                for (int j = 0; j < FB; ++j) {
+                    if (f0 + j < d) {
+                        const T cv = cr[j];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const T diff = xv[j][r] - cv;
+                            acc[t][r] = fma(diff, diff, acc[t][r]);
+                        }
                     }
                 }
             }
@@ -149,19 +156,25 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
         w[r] = ok ? sample_weight[i0 + r] : T(0);
         cl[r] = ok ? rows[(size_t)best * n + i0 + r] : T(0);
     }
+    double pot[TN];
 #pragma unroll
-    for (int t = 0; t < TN_MAX; ++t) {
+    for (int t = 0; t < TN; ++t) {
+        pot[t] = 0.0;
         if (t < n_trials) {
-            double pot = 0.0;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 if (i0 + r < n) {
                     const T v = fmin(acc[t][r] * w[r], cl[r]);
                     rows[(size_t)t * n + i0 + r] = v;
-                    pot += (double)v;
+                    pot[t] += (double)v;
                 }
             }
-            const double tot = kmx_block_sum<double>(pot, scratch);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        if (t < n_trials) {
+            const double tot = kmx_block_sum<double>(pot[t], scratch);
             if (threadIdx.x == 0) block_pot[(size_t)blockIdx.x * TN_MAX + t] = tot;
         }
     }
@@ -211,8 +224,8 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     int32_t* __restrict__ cand_out, T* __restrict__ centers_t,
     int32_t* __restrict__ center_indices, const T* __restrict__ rows,
     const double* __restrict__ block_pot, double* __restrict__ potentials,
-    KppHeader* __restrict__ header, int64_t n, int64_t n_blocks, int d, int k, int n_trials,
-    int center_slot, int do_select, int do_sample) {
+    KppHeader* __restrict__ header, T* __restrict__ cand_rows, int64_t n, int64_t n_blocks, int d,
+    int k, int n_trials, int center_slot, int do_select, int do_sample) {
     __shared__ double wave_tot[4];
     __shared__ double dscratch[4];
     __shared__ int64_t iscratch[4];
@@ -221,11 +234,23 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
 
     int best = header->best_row;
     if (do_select) {
-        for (int t = 0; t < n_trials; ++t) {
-            double acc = 0.0;
-            for (int64_t b = threadIdx.x; b < n_blocks; b += 256) acc += block_pot[(size_t)b * TN_MAX + t];
-            const double tot = kmx_block_sum<double>(acc, dscratch);
-            if (threadIdx.x == 0) pot_s[t] = tot;
+        // all trial sums in one pass over the block potentials (one row of TN_MAX doubles per
+        // block), then one block reduction per trial without memory traffic in between
+        double acc[TN_MAX];
+#pragma unroll
+        for (int t = 0; t < TN_MAX; ++t) acc[t] = 0.0;
+        for (int64_t b = threadIdx.x; b < n_blocks; b += 256) {
+            const double* __restrict__ rowp = block_pot + (size_t)b * TN_MAX;
+#pragma unroll
+            for (int t = 0; t < TN_MAX; ++t)
+                if (t < n_trials) acc[t] += rowp[t];
+        }
+#pragma unroll
+        for (int t = 0; t < TN_MAX; ++t) {
+            if (t < n_trials) {
+                const double tot = kmx_block_sum<double>(acc[t], dscratch);
+                if (threadIdx.x == 0) pot_s[t] = tot;
+            }
         }
         __syncthreads();
         best = 0;
@@ -300,10 +325,13 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
         cand_next[trial] = (int32_t)cand;
         if (cand_out) cand_out[trial] = (int32_t)cand;
     }
+    // the candidate's feature row, for the step kernel's scalar loads
+    for (int f = threadIdx.x; f < d; f += 256) cand_rows[(size_t)trial * d + f] = X_t[(size_t)f * n + cand];
 }
 
 struct KppPtrs {
     KppHeader* header;
+    void* cand_rows;
     int32_t* cand;
     double* potentials;
     double* block_pot;
@@ -314,6 +342,7 @@ KppPtrs kpp_ptrs(char* ws, const KppLayout& L) {
     KppPtrs p;
     p.header = (KppHeader*)(ws + L.off_header);
     p.cand = (int32_t*)(ws + L.off_cand);
+    p.cand_rows = ws + L.off_cand_rows;
     p.potentials = (double*)(ws + L.off_pot);
     p.block_pot = (double*)(ws + L.off_block_pot);
     p.rows = ws + L.off_rows;
@@ -328,7 +357,7 @@ int32_t kpp_check(const void* X_t, const void* w, void* ws, size_t ws_bytes, int
     if (n <= 0 || d <= 0 || k <= 0 || n > INT32_MAX) return KMX_ERR_BAD_SHAPE;
     if (n_trials <= 0 || n_trials > TN_MAX) return KMX_ERR_UNSUPPORTED;
     KMX_REQUIRE_DTYPE(dtype);
-    if (ws_bytes < kpp_layout(n, n_trials, dtype).total) return KMX_ERR_WORKSPACE;
+    if (ws_bytes < kpp_layout(n, d, n_trials, dtype).total) return KMX_ERR_WORKSPACE;
     return KMX_OK;
 }
 
@@ -343,10 +372,16 @@ void launch_init(const void* X_t, const void* w, int32_t start, void* centers_t,
 template <typename T>
 void launch_step(const void* X_t, const void* w, const int32_t* cand, const KppPtrs& p,
                  const KppLayout& L, int64_t n, int d, int n_trials, hipStream_t s) {
+    (void)cand;  // the candidates' rows were copied to p.cand_rows when they were sampled
     const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0);
-    hipLaunchKernelGGL((kpp_step_kernel<T>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
-                       (const T*)X_t, (const T*)w, cand, (T*)p.rows, p.block_pot, p.header, n, d,
-                       n_trials, vec_ok);
+    if (n_trials <= 8)
+        hipLaunchKernelGGL((kpp_step_kernel<T, 8>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
+                           (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,
+                           p.header, n, d, n_trials, vec_ok);
+    else
+        hipLaunchKernelGGL((kpp_step_kernel<T, TN_MAX>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
+                           (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,
+                           p.header, n, d, n_trials, vec_ok);
 }
 
 template <typename T>
@@ -357,8 +392,8 @@ void launch_select_sample(const void* X_t, const double* uniforms, const int32_t
     const unsigned grid = do_sample ? (unsigned)n_trials : 1u;
     hipLaunchKernelGGL((kpp_select_sample_kernel<T>), dim3(grid), dim3(256), 0, s, (const T*)X_t,
                        uniforms, cand_prev, cand_next, cand_out, (T*)centers_t, idx,
-                       (const T*)p.rows, p.block_pot, p.potentials, p.header, n, L.n_blocks, d, k,
-                       n_trials, slot, do_select, do_sample);
+                       (const T*)p.rows, p.block_pot, p.potentials, p.header, (T*)p.cand_rows, n,
+                       L.n_blocks, d, k, n_trials, slot, do_select, do_sample);
 }
 
 }  // namespace
@@ -370,7 +405,7 @@ size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials
     (void)k;
     if (n <= 0 || n_trials <= 0 || n_trials > TN_MAX || (dtype != KMX_F32 && dtype != KMX_F64))
         return 0;
-    return kpp_layout(n, n_trials, dtype).total;
+    return kpp_layout(n, d, n_trials, dtype).total;
 }
 
 int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_index,
@@ -382,7 +417,7 @@ int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_i
     KMX_REQUIRE_PTR(centers_t);
     KMX_REQUIRE_PTR(center_indices);
     if (start_index < 0 || start_index >= n) return KMX_ERR_BAD_ARGUMENT;
-    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppLayout L = kpp_layout(n, d, n_trials, dtype);
     const KppPtrs p = kpp_ptrs((char*)workspace, L);
     hipStream_t s = (hipStream_t)stream_;
     if (dtype == KMX_F32)
@@ -393,20 +428,21 @@ int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_i
     return KMX_OK;
 }
 
-int32_t kmx_kpp_sample_candidates(const double* uniforms_for_step, int32_t* candidates,
-                                  void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
-                                  int32_t k, int32_t n_trials, int32_t dtype, void* stream_) {
+int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_step,
+                                  int32_t* candidates, void* workspace, size_t workspace_bytes,
+                                  int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype,
+                                  void* stream_) {
     KMX_REQUIRE_PTR(uniforms_for_step);
-    const int32_t rc = kpp_check(uniforms_for_step, uniforms_for_step, workspace, workspace_bytes, n, d, k, n_trials, dtype);
+    const int32_t rc = kpp_check(X_t, uniforms_for_step, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
-    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppLayout L = kpp_layout(n, d, n_trials, dtype);
     const KppPtrs p = kpp_ptrs((char*)workspace, L);
     hipStream_t s = (hipStream_t)stream_;
     if (dtype == KMX_F32)
-        launch_select_sample<float>(nullptr, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
+        launch_select_sample<float>(X_t, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
                                     nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s);
     else
-        launch_select_sample<double>(nullptr, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
+        launch_select_sample<double>(X_t, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
                                      nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
@@ -421,7 +457,7 @@ int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_
     KMX_REQUIRE_PTR(centers_t);
     KMX_REQUIRE_PTR(center_indices);
     if (center_slot < 1 || center_slot >= k) return KMX_ERR_BAD_ARGUMENT;
-    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppLayout L = kpp_layout(n, d, n_trials, dtype);
     const KppPtrs p = kpp_ptrs((char*)workspace, L);
     hipStream_t s = (hipStream_t)stream_;
     if (dtype == KMX_F32) {
@@ -446,7 +482,7 @@ int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* un
     if (rc != KMX_OK) return rc;
     if (k == 1) return KMX_OK;
     KMX_REQUIRE_PTR(uniforms);
-    const KppLayout L = kpp_layout(n, n_trials, dtype);
+    const KppLayout L = kpp_layout(n, d, n_trials, dtype);
     const KppPtrs p = kpp_ptrs((char*)workspace, L);
     hipStream_t s = (hipStream_t)stream_;
     for (int c = 1; c < k; ++c) {
@@ -484,7 +520,7 @@ void* kmx_kpp_closest_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int3
     (void)k;
     if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
     // start of the rows; the caller adds best_row * n elements (best_row from the header)
-    return (char*)workspace + kpp_layout(n, n_trials, dtype).off_rows;
+    return (char*)workspace + kpp_layout(n, d, n_trials, dtype).off_rows;
 }
 
 double* kmx_kpp_potentials_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
@@ -492,7 +528,7 @@ double* kmx_kpp_potentials_ptr(void* workspace, int64_t n, int32_t d, int32_t k,
     (void)d;
     (void)k;
     if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
-    return (double*)((char*)workspace + kpp_layout(n, n_trials, dtype).off_pot);
+    return (double*)((char*)workspace + kpp_layout(n, d, n_trials, dtype).off_pot);
 }
 
 int32_t* kmx_kpp_candidates_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
@@ -500,7 +536,7 @@ int32_t* kmx_kpp_candidates_ptr(void* workspace, int64_t n, int32_t d, int32_t k
     (void)d;
     (void)k;
     if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
-    return (int32_t*)((char*)workspace + kpp_layout(n, n_trials, dtype).off_cand);
+    return (int32_t*)((char*)workspace + kpp_layout(n, d, n_trials, dtype).off_cand);
 }
 
 }  // extern "C"

@@ -87,7 +87,7 @@ def test_step_kernels_through_c_abi(cuda, dtype):
         u[0] = 0.0 if c == 1 else u[0]            # rv == 0 -> first sample (reference would give -1)
         u[1] = 1.0 - 2.0**-53 if c == 2 else u[1]  # top of the range -> last crossing, clipped to n - 1
         cand = torch.empty(tn, dtype=torch.int32, device=cuda)
-        _capi.check(lib.kmx_kpp_sample_candidates(ptr(_dev(u, cuda)), ptr(cand), ptr(ws), ws_bytes, n, d, k, tn,
+        _capi.check(lib.kmx_kpp_sample_candidates(ptr(X_t), ptr(_dev(u, cuda)), ptr(cand), ptr(ws), ws_bytes, n, d, k, tn,
                                                   dc, st), "kpp_sample")
         expected = np.array([ok._sample_exact(closest, uu) for uu in u])
         np.testing.assert_array_equal(cand.cpu().numpy(), expected)
