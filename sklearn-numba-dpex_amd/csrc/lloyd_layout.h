@@ -20,6 +20,7 @@ constexpr size_t KMX_GLOBAL_COPIES_BYTES = 64u << 20;
 // KMX_LLOYD_WGS_PER_CU = 1..8.
 int kmx_forced_variant();
 int kmx_wgs_per_cu();
+int kmx_wgs_per_cu_env();
 // Shapes the fp32 matrix-core fused step covers (operands and accumulators fit in LDS), and
 // those its wide-sample variant covers (samples in registers, centroids streamed).
 bool kmx_mfma_supported(int d, int k);

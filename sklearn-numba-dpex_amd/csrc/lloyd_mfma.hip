@@ -28,6 +28,7 @@
 #include "lloyd_tail.h"
 
 #include <cstdlib>
+#include <type_traits>
 #include <cstring>
 
 int kmx_forced_variant() {
@@ -39,11 +40,17 @@ int kmx_forced_variant() {
     return -1;
 }
 
-int kmx_wgs_per_cu() {
+// 0 when KMX_LLOYD_WGS_PER_CU is unset or out of range
+int kmx_wgs_per_cu_env() {
     const char* v = std::getenv("KMX_LLOYD_WGS_PER_CU");
-    if (v == nullptr) return 4;
+    if (v == nullptr) return 0;
     const int x = std::atoi(v);
-    return (x >= 1 && x <= 8) ? x : 4;
+    return (x >= 1 && x <= 8) ? x : 0;
+}
+
+int kmx_wgs_per_cu() {
+    const int x = kmx_wgs_per_cu_env();
+    return x > 0 ? x : 4;
 }
 
 namespace {
@@ -106,8 +113,15 @@ __global__ void fixed_point_exponents_kernel(const unsigned int* __restrict__ ab
 // no guards and the body of the centroid-block loop is one basic block (the scheduler can
 // hoist the LDS reads of the A fragments above the MFMAs); otherwise steps s >= nks are
 // skipped with wave-uniform branches.
+constexpr int ARGMAX_GROUP = 8;  // accumulator registers per argmax group: 1, 2, 4, 8 or 16
+
+// Waves per workgroup: with few K steps the kernel fits two waves per SIMD, and one
+// workgroup of eight waves per compute unit halves the accumulator flushes (the global
+// atomics of all workgroups hit the same (d + 1) * k addresses) and the staging work.
+constexpr int mfma_waves(int nks) { return nks <= 8 ? 8 : 4; }
+
 template <int NKS, bool EXACT, bool UPDATE>
-__global__ __launch_bounds__(256) void lloyd_mfma_kernel(
+__global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
@@ -115,6 +129,7 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
     int vec_ok) {
     if (UPDATE && status->state != KMX_RUNNING) return;
 
+    constexpr int WAVES = mfma_waves(NKS), THREADS = 64 * WAVES;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int nks = EXACT ? NKS : (d + 1) >> 1;  // K steps of 2 features
     const int n_cb = (k + 31) >> 5;        // centroid blocks of 32
@@ -122,9 +137,10 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
     unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [(d + 1) * k]
     float* afrag = reinterpret_cast<float*>(acc + (UPDATE ? items : 0));         // [n_cb][nks][64]
     float* hneg = afrag + n_cb * nks * 64;  // [n_cb][2][16]  -0.5||c||^2 in accumulator order
+    float* qscale = hneg + n_cb * 32;       // [d + 1]  2^q of the fixed-point sums (UPDATE)
     __shared__ unsigned int changed_block;
 
-    for (int idx = threadIdx.x; idx < n_cb * nks * 64; idx += 256) {
+    for (int idx = threadIdx.x; idx < n_cb * nks * 64; idx += THREADS) {
         const int l = idx & 63;
         const int s = (idx >> 6) % nks;
         const int cb = (idx >> 6) / nks;
@@ -132,7 +148,7 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
         const int f = 2 * s + (l >> 5);
         afrag[idx] = (c < k && f < d) ? centroids_t[(size_t)f * k + c] : 0.0f;
     }
-    for (int idx = threadIdx.x; idx < n_cb * 32; idx += 256) {
+    for (int idx = threadIdx.x; idx < n_cb * 32; idx += THREADS) {
         const int cb = idx >> 5, h = (idx >> 4) & 1, r = idx & 15;
         const int c = 32 * cb + 8 * (r >> 2) + 4 * h + (r & 3);
         float v = -kmx_inf<float>();
@@ -147,7 +163,8 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
         hneg[idx] = v;
     }
     if (UPDATE) {
-        for (int jx = threadIdx.x; jx < items; jx += 256) acc[jx] = 0ull;
+        for (int jx = threadIdx.x; jx < items; jx += THREADS) acc[jx] = 0ull;
+        for (int f = threadIdx.x; f <= d; f += THREADS) qscale[f] = ldexpf(1.0f, q_exp[f]);
         if (threadIdx.x == 0) changed_block = 0;
     }
     __syncthreads();
@@ -164,39 +181,32 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
             const int f = 2 * s + h;
-            scale[s] = (s < nks && f < d) ? ldexpf(1.0f, q_exp[f]) : 0.0f;
+            scale[s] = (s < nks && f < d) ? qscale[f] : 0.0f;
         }
-        scale_w = ldexpf(1.0f, q_exp[d]);
+        scale_w = qscale[d];
     }
 
-    for (int64_t wt = (int64_t)blockIdx.x * 4 + wave; wt < n_wtiles; wt += (int64_t)gridDim.x * 4) {
-        const int64_t i0 = wt * 128 + 4 * j;
-        const bool full = vec_ok && (i0 + 4 <= n);
-
-        float4 x[NKS];
-#pragma unroll
-        for (int s = 0; s < NKS; ++s) {
-            x[s] = make_float4(0.f, 0.f, 0.f, 0.f);
-            const int f = 2 * s + h;
-            if (s < nks && f < d) {
-                const float* __restrict__ row = X_t + (size_t)f * n;
-                if (full) {
-                    x[s] = *reinterpret_cast<const float4*>(row + i0);
-                } else {
-                    if (i0 + 0 < n) x[s].x = row[i0 + 0];
-                    if (i0 + 1 < n) x[s].y = row[i0 + 1];
-                    if (i0 + 2 < n) x[s].z = row[i0 + 2];
-                    if (i0 + 3 < n) x[s].w = row[i0 + 3];
-                }
-            }
-        }
-
+    // One 128-sample tile: scores on the matrix cores, argmax, labels and (UPDATE) the
+    // accumulation.  FULL (a std::bool_constant): every lane's four samples exist and 128-bit
+    // accesses are legal.  wv / p4: weights and previous labels of the lane's four samples.
+    auto process = [&](const float4(&x)[NKS], const float(&wv)[4], const uint4 p4, const int64_t i0,
+                       auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        // Running argmax per sample column, by groups of ARGMAX_GROUP accumulator registers:
+        // a group costs one max chain, one compare and the conditional copies of its values
+        // (about 2 VALU instructions per score instead of 3 for a compare and two selects per
+        // score; fp32 MFMA and VALU instructions do not overlap on this hardware, so every
+        // VALU instruction saved is time saved).  The position inside the winning group is
+        // found once per tile.
         float best[4];
         int code[4];
+        float sv[4][ARGMAX_GROUP];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             best[t] = -kmx_inf<float>();
             code[t] = 0;
+#pragma unroll
+            for (int r = 0; r < ARGMAX_GROUP; ++r) sv[t][r] = 0.0f;
         }
 
         for (int cb = 0; cb < n_cb; ++cb) {
@@ -207,35 +217,50 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
             const float* ap = afrag + (size_t)cb * nks * 64 + lane;
             // the first K step reads the accumulator start (-0.5||c||^2) straight from hv
             float af = ap[0];
-            v16f a0 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].x, hv, 0, 0, 0);
-            v16f a1 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].y, hv, 0, 0, 0);
-            v16f a2 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].z, hv, 0, 0, 0);
-            v16f a3 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].w, hv, 0, 0, 0);
+            v16f a[4];
+            a[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].x, hv, 0, 0, 0);
+            a[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].y, hv, 0, 0, 0);
+            a[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].z, hv, 0, 0, 0);
+            a[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].w, hv, 0, 0, 0);
 #pragma unroll
             for (int s = 1; s < NKS; ++s) {
                 if (s < nks) {
                     af = ap[s * 64];
-                    a0 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].x, a0, 0, 0, 0);
-                    a1 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].y, a1, 0, 0, 0);
-                    a2 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].z, a2, 0, 0, 0);
-                    a3 = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].w, a3, 0, 0, 0);
+                    a[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].x, a[0], 0, 0, 0);
+                    a[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].y, a[1], 0, 0, 0);
+                    a[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].z, a[2], 0, 0, 0);
+                    a[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].w, a[3], 0, 0, 0);
                 }
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int cd = cb * 16 + r;  // wave-uniform
-                if (a0[r] > best[0]) { best[0] = a0[r]; code[0] = cd; }
-                if (a1[r] > best[1]) { best[1] = a1[r]; code[1] = cd; }
-                if (a2[r] > best[2]) { best[2] = a2[r]; code[2] = cd; }
-                if (a3[r] > best[3]) { best[3] = a3[r]; code[3] = cd; }
+            for (int g = 0; g < 16 / ARGMAX_GROUP; ++g) {
+                const int cd = cb * (16 / ARGMAX_GROUP) + g;  // wave-uniform
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    float m = a[t][g * ARGMAX_GROUP];
+#pragma unroll
+                    for (int r = 1; r < ARGMAX_GROUP; ++r) m = fmaxf(m, a[t][g * ARGMAX_GROUP + r]);
+                    const bool win = m > best[t];  // strict: the earlier group keeps a tie
+                    best[t] = win ? m : best[t];
+                    code[t] = win ? cd : code[t];
+#pragma unroll
+                    for (int r = 0; r < ARGMAX_GROUP; ++r)
+                        sv[t][r] = win ? a[t][g * ARGMAX_GROUP + r] : sv[t][r];
+                }
             }
         }
 
-        // decode (block, register) -> centroid index, then combine the two half-waves
+        // position inside the winning group (lowest register = lowest centroid of this lane),
+        // (block, register) -> centroid index, then combine the two half-waves
         uint32_t lab[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            int c = 32 * (code[t] >> 4) + 8 * ((code[t] & 15) >> 2) + 4 * h + (code[t] & 3);
+            int pos = ARGMAX_GROUP - 1;
+#pragma unroll
+            for (int r = ARGMAX_GROUP - 2; r >= 0; --r) pos = (sv[t][r] == best[t]) ? r : pos;
+            const int reg = (code[t] % (16 / ARGMAX_GROUP)) * ARGMAX_GROUP + pos;
+            const int blk = code[t] / (16 / ARGMAX_GROUP);
+            int c = 32 * blk + 8 * (reg >> 2) + 4 * h + (reg & 3);
             const float ov = __shfl_xor(best[t], 32, 64);
             const int oc = __shfl_xor(c, 32, 64);
             if (ov > best[t] || (ov == best[t] && oc < c)) c = oc;
@@ -243,7 +268,7 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
         }
 
         if (h == 0) {
-            if (full) {
+            if (FULL) {
                 *reinterpret_cast<uint4*>(labels + i0) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
             } else {
 #pragma unroll
@@ -253,22 +278,11 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
         }
 
         if (UPDATE) {
-            float wv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (full) {
-                const float4 w4 = *reinterpret_cast<const float4*>(sample_weight + i0);
-                wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
-                if (h == 0) {
-                    const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
-                    changed += (p4.x != lab[0]) + (p4.y != lab[1]) + (p4.z != lab[2]) + (p4.w != lab[3]);
-                }
-            } else {
+            if (h == 0) {
+                const uint32_t pl[4] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    if (i0 + t < n) {
-                        wv[t] = sample_weight[i0 + t];
-                        if (h == 0) changed += (labels_prev[i0 + t] != lab[t]) ? 1u : 0u;
-                    }
-                }
+                for (int t = 0; t < 4; ++t)
+                    changed += ((FULL || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
             }
             // samples past the end carry w = 0 and x = 0: they add zero
             double wd[4];
@@ -297,13 +311,93 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
                     atomicAdd(szacc + lab[t], to_fixed(fma(wd[t], sc, FIX_MAGIC)));
             }
         }
+    };
+
+    const int64_t wt_step = (int64_t)gridDim.x * WAVES;
+    const int64_t wt_first = (int64_t)blockIdx.x * WAVES + wave;
+    // Tiles that lie entirely inside the array, when 128-bit accesses are legal: straight-line
+    // loads with the next tile's rows in flight during the current tile (the wave does not
+    // stall on its own loads or on the completion of its label store).
+    const int64_t n_fast = vec_ok ? (n >> 7) : 0;
+    // Rows of the lane's half-wave (2s + h) at the lane's four samples.  The loads are
+    // unconditional, so that the compiler can count them exactly and wait for the older tile
+    // only: a row past d - 1 (odd d, upper half-wave, last K step) reads row d - 1 instead;
+    // its A fragment is zero and the accumulation skips it.
+    const float* __restrict__ xrow_base = X_t + (size_t)h * n + 4 * j;
+    const int last_row = 2 * (nks - 1) + h < d ? 2 * (nks - 1) + h : d - 1;
+    const size_t last_row_off = (size_t)(last_row - h) * n;
+    auto load_rows = [&](const int64_t wt, float4* dst) {
+        const float* __restrict__ p = xrow_base + wt * 128;
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+            if (EXACT || s < nks) {
+                const size_t off = (s == nks - 1) ? last_row_off : (size_t)(2 * s) * n;
+                dst[s] = *reinterpret_cast<const float4*>(p + off);
+            } else {
+                dst[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    };
+    constexpr bool PREFETCH = NKS <= 16;  // the double buffer costs 4 * NKS registers
+    if (wt_first < n_fast) {
+        float4 xn[PREFETCH ? NKS : 1];
+        if constexpr (PREFETCH) load_rows(wt_first, xn);
+        for (int64_t wt = wt_first; wt < n_fast; wt += wt_step) {
+            const int64_t i0 = wt * 128 + 4 * j;
+            float4 x[NKS];
+            if constexpr (PREFETCH) {
+#pragma unroll
+                for (int s = 0; s < NKS; ++s) x[s] = xn[s];
+                // past the last tile the same rows are read again (and not used)
+                load_rows(wt + wt_step < n_fast ? wt + wt_step : wt, xn);
+            } else {
+                load_rows(wt, x);
+            }
+            float wv[4] = {0.f, 0.f, 0.f, 0.f};
+            uint4 p4 = make_uint4(0u, 0u, 0u, 0u);
+            if (UPDATE) {
+                const float4 w4 = *reinterpret_cast<const float4*>(sample_weight + i0);
+                wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+            }
+            process(x, wv, p4, i0, std::true_type{});
+        }
+    }
+    // The rest: a partial last tile, or every tile when 128-bit accesses are not legal
+    for (int64_t wt = n_fast + wt_first; wt < n_wtiles; wt += wt_step) {
+        const int64_t i0 = wt * 128 + 4 * j;
+        float4 x[NKS];
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+            x[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int f = 2 * s + h;
+            if (s < nks && f < d) {
+                const float* __restrict__ row = X_t + (size_t)f * n;
+                if (i0 + 0 < n) x[s].x = row[i0 + 0];
+                if (i0 + 1 < n) x[s].y = row[i0 + 1];
+                if (i0 + 2 < n) x[s].z = row[i0 + 2];
+                if (i0 + 3 < n) x[s].w = row[i0 + 3];
+            }
+        }
+        float wv[4] = {0.f, 0.f, 0.f, 0.f};
+        uint32_t pl[4] = {0u, 0u, 0u, 0u};
+        if (UPDATE) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                if (i0 + t < n) {
+                    wv[t] = sample_weight[i0 + t];
+                    pl[t] = labels_prev[i0 + t];
+                }
+            }
+        }
+        process(x, wv, make_uint4(pl[0], pl[1], pl[2], pl[3]), i0, std::false_type{});
     }
 
     if (UPDATE) {
         if (changed) atomicAdd(&changed_block, changed);
         __syncthreads();
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
-        for (int jx = threadIdx.x; jx < items; jx += 256) {
+        for (int jx = threadIdx.x; jx < items; jx += THREADS) {
             const unsigned long long v = acc[jx];
             if (v) atomicAdd(gsum + jx, v);
         }
@@ -311,25 +405,36 @@ __global__ __launch_bounds__(256) void lloyd_mfma_kernel(
 }
 
 // One workgroup: fixed point -> float sums and sizes (clearing gsum for the next iteration),
-// empty-cluster list, and the finalisation if no cluster is empty.
+// empty-cluster list, and, if no cluster is empty, the finalisation: division by the sizes,
+// packed copy and half norms for the next iteration, centroid shift, convergence test.  The
+// sums stay in LDS between the phases; global memory is read once (fixed-point sums, old
+// centroids) and written once per output.  With an empty cluster the raw sums and sizes are
+// left in global memory for the relocation and the state becomes KMX_NEED_RELOCATION.
 __global__ __launch_bounds__(256) void lloyd_mfma_finalize_kernel(
     unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<float> a) {
+    extern __shared__ __align__(16) unsigned char fin_raw[];
+    __shared__ double scratch[4];
     if (a.status->state != KMX_RUNNING) return;
-    const int d = a.d, k = a.k;
-    const int items = (d + 1) * k;
+    const int d = a.d, k = a.k, dpad = a.dpad;
+    const int items = (d + 1) * k, dk = d * k;
+    float* vals = reinterpret_cast<float*>(fin_raw);  // [(d + 1) * k]: sums, then sizes
+    const float* sizes_s = vals + dk;
+    float* __restrict__ out_t = a.sums_t;
+    const float* __restrict__ old_t = a.old_centroids_t;
     for (int jx = threadIdx.x; jx < items; jx += 256) {
         const long long iv = (long long)gsum[jx];
         gsum[jx] = 0ull;
         const int f = jx / k;
         const float val = (float)ldexp((double)iv, -q_exp[f]);
+        vals[jx] = val;
         if (f < d)
-            a.sums_t[jx] = val;
+            out_t[jx] = val;
         else
-            a.sizes[jx - d * k] = val;
+            a.sizes[jx - dk] = val;
     }
     __syncthreads();
     int heaviest = 0;
-    const int n_empty = lloyd_list_empty<float>(a.sizes, a.empty_clusters, k, &heaviest);
+    const int n_empty = lloyd_list_empty<float>(sizes_s, a.empty_clusters, k, &heaviest);
     if (threadIdx.x == 0) {
         a.status->n_empty = n_empty;
         a.status->reserved[0] = heaviest;
@@ -338,13 +443,32 @@ __global__ __launch_bounds__(256) void lloyd_mfma_finalize_kernel(
         if (threadIdx.x == 0) a.status->state = KMX_NEED_RELOCATION;
         return;
     }
-    lloyd_finalize_block<float>(a, 0, heaviest);
+    double shift = 0.0;
+#pragma unroll 4
+    for (int jx = threadIdx.x; jx < dk; jx += 256) {
+        const int f = jx / k, c = jx - f * k;
+        const float nv = vals[jx] / sizes_s[c];
+        const float df = old_t[jx] - nv;
+        shift += (double)(df * df);
+        vals[jx] = nv;
+        out_t[jx] = nv;
+        a.cpack[(size_t)c * dpad + f] = nv;
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < k; c += 256) {
+        float sq = 0.0f;
+        for (int f = 0; f < d; ++f) sq += vals[f * k + c] * vals[f * k + c];
+        a.half_norms[c] = sq / 2.0f;
+        for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = 0.0f;
+    }
+    const double total = kmx_block_sum<double>(shift, scratch);
+    if (threadIdx.x == 0) lloyd_update_status(a.status, total);
 }
 
 size_t mfma_lds_bytes(int d, int k, bool update) {
     const int nks = (d + 1) / 2, n_cb = (k + 31) / 32;
     size_t bytes = ((size_t)n_cb * nks * 64 + (size_t)n_cb * 32) * sizeof(float);
-    if (update) bytes += (size_t)(d + 1) * k * sizeof(unsigned long long);
+    if (update) bytes += (size_t)(d + 1) * k * sizeof(unsigned long long) + (size_t)(d + 1) * sizeof(float);
     return bytes;
 }
 
@@ -356,18 +480,21 @@ int32_t launch_mfma(const LloydLayout& L, const void* X_t, const void* w, const 
     const size_t lds = mfma_lds_bytes(d, k, UPDATE);
     if (lds > 64 * 1024 || d > 64) return KMX_ERR_UNSUPPORTED;
     const int64_t n_wtiles = kmx_cdiv(n, 128);
-    int64_t grid = kmx_cdiv(n_wtiles, 4);
-    const int cap = L.grid_cap(kmx_num_cus());
+    const int waves = mfma_waves((d + 1) / 2 <= 8 ? (d + 1) / 2 : (d <= 32 ? 16 : 32));
+    int64_t grid = kmx_cdiv(n_wtiles, waves);
+    // resident workgroups only: 8 waves per compute unit in either shape
+    const int per_cu = waves == 8 ? 1 : 2;
+    const int cap = (kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : per_cu) * kmx_num_cus();
     if (grid > cap) grid = cap;
     if (grid < 1) grid = 1;
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
                        (!UPDATE || (aligned16(w) && aligned16(labels_prev)));
 #define KMX_MFMA_CASE(NKS, EXACT)                                                              \
-    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, EXACT, UPDATE>), dim3((unsigned)grid), dim3(256), \
-                       lds, stream, (const float*)X_t, (const float*)w,                          \
-                       (const float*)centroids_t, labels_prev, labels, status, q_exp, gsum, n, d, \
-                       k, vec_ok)
+    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, EXACT, UPDATE>), dim3((unsigned)grid),          \
+                       dim3(64 * mfma_waves(NKS)), lds, stream, (const float*)X_t,             \
+                       (const float*)w, (const float*)centroids_t, labels_prev, labels, status, \
+                       q_exp, gsum, n, d, k, vec_ok)
     switch ((d + 1) / 2) {
         case 1: KMX_MFMA_CASE(1, true); break;
         case 2: KMX_MFMA_CASE(2, true); break;
@@ -439,7 +566,8 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         (void)hipEventRecord(events[1], stream);
         (void)hipEventRecord(events[2], stream);
     }
-    hipLaunchKernelGGL(lloyd_mfma_finalize_kernel, dim3(1), dim3(256), 0, stream, gsum, q_exp, tail);
+    hipLaunchKernelGGL(lloyd_mfma_finalize_kernel, dim3(1), dim3(256),
+                       (size_t)(d + 1) * k * sizeof(float), stream, gsum, q_exp, tail);
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[3], stream);
     return KMX_OK;

@@ -83,6 +83,25 @@ __device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters,
     return base;
 }
 
+// End of an iteration, by one thread: iteration count, shift, and the next state (strict
+// convergence from the second iteration on, then the tolerance, then the iteration limit).
+__device__ inline void lloyd_update_status(kmx_lloyd_status* st, double total_shift) {
+    const int n_iter = st->n_iter + 1;
+    const unsigned int changed = st->n_changed;
+    st->n_iter = n_iter;
+    st->shift_sum = total_shift;
+    st->n_changed = 0;
+    int next = KMX_RUNNING;
+    if (n_iter > 1 && changed == 0)
+        next = KMX_CONVERGED_STRICT;
+    else if (!(total_shift > st->tol))
+        next = KMX_CONVERGED_TOL;
+    else if (n_iter >= st->max_iter)
+        next = KMX_MAX_ITER;
+    st->state = next;
+    st->reserved[1] = (int64_t)changed;
+}
+
 // Division, packed copy, half norms, shift and convergence test by ONE workgroup of 256
 // threads (thread per cluster, features in order).  `sums_t` becomes the new centroids.
 template <typename T>
@@ -129,22 +148,6 @@ __device__ inline void lloyd_finalize_block(const LloydTail<T>& a, int n_empty, 
         }
     }
     const double total = kmx_block_sum<double>(shift, scratch);
-    if (threadIdx.x == 0) {
-        kmx_lloyd_status* st = a.status;
-        const int n_iter = st->n_iter + 1;
-        const unsigned int changed = st->n_changed;
-        st->n_iter = n_iter;
-        st->shift_sum = total;
-        st->n_changed = 0;
-        int next = KMX_RUNNING;
-        if (n_iter > 1 && changed == 0)
-            next = KMX_CONVERGED_STRICT;
-        else if (!(total > st->tol))
-            next = KMX_CONVERGED_TOL;
-        else if (n_iter >= st->max_iter)
-            next = KMX_MAX_ITER;
-        st->state = next;
-        st->reserved[1] = (int64_t)changed;
-    }
+    if (threadIdx.x == 0) lloyd_update_status(a.status, total);
 }
 
