@@ -56,6 +56,7 @@ int kmx_wgs_per_cu() {
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef double v8d __attribute__((ext_vector_type(8)));
 
 // 1.5 * 2^52: adding it to |v| < 2^51 leaves round-to-nearest(v) in the low mantissa bits.
 constexpr double FIX_MAGIC = 6755399441055744.0;
@@ -113,7 +114,7 @@ __global__ void fixed_point_exponents_kernel(const unsigned int* __restrict__ ab
 // no guards and the body of the centroid-block loop is one basic block (the scheduler can
 // hoist the LDS reads of the A fragments above the MFMAs); otherwise steps s >= nks are
 // skipped with wave-uniform branches.
-constexpr int ARGMAX_GROUP = 8;  // accumulator registers per argmax group: 1, 2, 4, 8 or 16
+constexpr int ARGMAX_GROUP = 8;  // accumulator registers per argmax group: 2, 4, 8 or 16
 
 // Waves per workgroup: with few K steps the kernel fits two waves per SIMD, and one
 // workgroup of eight waves per compute unit halves the accumulator flushes (the global
@@ -200,13 +201,13 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
         // found once per tile.
         float best[4];
         int code[4];
-        float sv[4][ARGMAX_GROUP];
+        double svd[4][ARGMAX_GROUP / 2];  // the winning group's registers, as pairs
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             best[t] = -kmx_inf<float>();
             code[t] = 0;
 #pragma unroll
-            for (int r = 0; r < ARGMAX_GROUP; ++r) sv[t][r] = 0.0f;
+            for (int r = 0; r < ARGMAX_GROUP / 2; ++r) svd[t][r] = 0.0;
         }
 
         for (int cb = 0; cb < n_cb; ++cb) {
@@ -237,15 +238,29 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
                 const int cd = cb * (16 / ARGMAX_GROUP) + g;  // wave-uniform
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
+                    // three-operand max: two scores per instruction (fmaxf would also
+                    // canonicalise the matrix-core results first)
                     float m = a[t][g * ARGMAX_GROUP];
 #pragma unroll
-                    for (int r = 1; r < ARGMAX_GROUP; ++r) m = fmaxf(m, a[t][g * ARGMAX_GROUP + r]);
-                    const bool win = m > best[t];  // strict: the earlier group keeps a tie
-                    best[t] = win ? m : best[t];
-                    code[t] = win ? cd : code[t];
+                    for (int r = 1; r + 1 < ARGMAX_GROUP; r += 2)
+                        asm("v_max3_f32 %0, %1, %2, %3"
+                            : "=v"(m)
+                            : "v"(m), "v"(a[t][g * ARGMAX_GROUP + r]), "v"(a[t][g * ARGMAX_GROUP + r + 1]));
+                    if (ARGMAX_GROUP % 2 == 0)
+                        asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(m), "v"(a[t][g * ARGMAX_GROUP + ARGMAX_GROUP - 1]));
+                    // strict: the earlier group keeps a tie.  The winning lanes copy the
+                    // group with 64-bit moves under the execution mask: half the instructions
+                    // of per-register selects.
+                    if (m > best[t]) {
+                        best[t] = m;
+                        code[t] = cd;
+                        const v8d ad = __builtin_bit_cast(v8d, a[t]);
 #pragma unroll
-                    for (int r = 0; r < ARGMAX_GROUP; ++r)
-                        sv[t][r] = win ? a[t][g * ARGMAX_GROUP + r] : sv[t][r];
+                        for (int r = 0; r < ARGMAX_GROUP / 2; ++r)
+                            asm volatile("v_mov_b64 %0, %1"
+                                         : "+v"(svd[t][r])
+                                         : "v"(ad[g * (ARGMAX_GROUP / 2) + r]));
+                    }
                 }
             }
         }
@@ -255,9 +270,16 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
         uint32_t lab[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
+            float sv[ARGMAX_GROUP];
+#pragma unroll
+            for (int r = 0; r < ARGMAX_GROUP / 2; ++r) {
+                const float2 pr = __builtin_bit_cast(float2, svd[t][r]);
+                sv[2 * r] = pr.x;
+                sv[2 * r + 1] = pr.y;
+            }
             int pos = ARGMAX_GROUP - 1;
 #pragma unroll
-            for (int r = ARGMAX_GROUP - 2; r >= 0; --r) pos = (sv[t][r] == best[t]) ? r : pos;
+            for (int r = ARGMAX_GROUP - 2; r >= 0; --r) pos = (sv[r] == best[t]) ? r : pos;
             const int reg = (code[t] % (16 / ARGMAX_GROUP)) * ARGMAX_GROUP + pos;
             const int blk = code[t] / (16 / ARGMAX_GROUP);
             int c = 32 * blk + 8 * (reg >> 2) + 4 * h + (reg & 3);
