@@ -177,6 +177,17 @@ int32_t kmx_relocate_empty_clusters(const void* X_t, const void* sample_weight,
  * kmeans++ seeding                                                                      *
  * ------------------------------------------------------------------------------------ */
 
+/* Host-side generator of the sampler's draws (no device work, callable without a GPU).
+ * kmx_rng_init_states fills `states` (n_states, 2) with xoroshiro128++ states: SplitMix64
+ * seeding of the first one, then `subsequence_start` jumps of 2^64 steps, every further state
+ * one more jump ahead.  kmx_rng_next_raw advances every state n_steps times and writes the raw
+ * 64-bit outputs to `out` (n_steps, n_states), step-major.  Replace create_xoroshiro128pp_states
+ * and the make_rand_uniform_kernel_func stream (common/random.py:124-292); the uint64 -> [0, 1)
+ * conversion (:78-104) stays with the caller. */
+int32_t kmx_rng_init_states(uint64_t seed, int32_t n_states, int32_t subsequence_start,
+                            uint64_t* states);
+int32_t kmx_rng_next_raw(uint64_t* states, int32_t n_states, int32_t n_steps, uint64_t* out);
+
 size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype);
 
 /* closest[i] = w_i ||x_i - x_start||^2, centers_t[:, 0] = x_start, center_indices[0] = start,

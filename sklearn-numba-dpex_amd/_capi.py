@@ -67,6 +67,8 @@ SIGNATURES = {
     "kmx_per_sample_inertia": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_euclidean_distances": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_relocate_empty_clusters": (_I32, [_P, _P, _P, _P, _P, _I32, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
+    "kmx_rng_init_states": (_I32, [ctypes.c_uint64, _I32, _I32, _P]),
+    "kmx_rng_next_raw": (_I32, [_P, _I32, _I32, _P]),
     "kmx_kpp_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
     "kmx_kpp_init": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
     "kmx_kpp_sample_candidates": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),

@@ -281,10 +281,8 @@ def kpp_uniforms(n_clusters, n_local_trials, random_state, dtype):
     the starting centre: common/random.py:29-38, kmeans/drivers.py:799-803, 830)."""
     states = create_xoroshiro128pp_states(n_local_trials, seed=random_state)
     start_raw = get_random_raw(states)
-    table = np.empty((max(n_clusters - 1, 0), n_local_trials), dtype=np.float64)
-    for c in range(n_clusters - 1):
-        table[c] = raw_to_uniform(states.next_raw_all(), dtype).astype(np.float64)
-    return start_raw, table
+    raw = states.next_raw_all(n_steps=max(n_clusters - 1, 0))
+    return start_raw, raw_to_uniform(raw, dtype).astype(np.float64)
 
 
 def kmeans_plusplus(X_t, sample_weight, n_clusters, random_state):
