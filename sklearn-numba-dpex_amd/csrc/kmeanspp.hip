@@ -89,6 +89,40 @@ __global__ __launch_bounds__(256) void kpp_init_kernel(
     }
 }
 
+// Four consecutive values of a row at i0 (one or two 128-bit accesses when `full`), zero past n.
+template <typename T>
+__device__ __forceinline__ void load4(const T* __restrict__ row, int64_t i0, int64_t n, bool full, T (&v)[4]) {
+    if (full) {
+        if constexpr (sizeof(T) == 4) {
+            const float4 q = *reinterpret_cast<const float4*>(row + i0);
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+            const double2 a = *reinterpret_cast<const double2*>(row + i0);
+            const double2 b = *reinterpret_cast<const double2*>(row + i0 + 2);
+            v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = (i0 + r < n) ? row[i0 + r] : T(0);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void store4(T* __restrict__ row, int64_t i0, int64_t n, bool full, const T (&v)[4]) {
+    if (full) {
+        if constexpr (sizeof(T) == 4) {
+            *reinterpret_cast<float4*>(row + i0) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            *reinterpret_cast<double2*>(row + i0) = make_double2(v[0], v[1]);
+            *reinterpret_cast<double2*>(row + i0 + 2) = make_double2(v[2], v[3]);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (i0 + r < n) row[i0 + r] = v[r];
+    }
+}
+
 // rows[t, i] = min(w_i * ||x_i - x_cand_t||^2, closest_i) and per-block row sums.
 // Candidate rows come from a small (TN, d) buffer through wave-uniform loads (the values sit
 // in SGPRs, no LDS, no barriers in the feature loop); every thread streams 4 consecutive
@@ -98,10 +132,16 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cand_rows,
     T* __restrict__ rows, double* __restrict__ block_pot, const KppHeader* __restrict__ header,
     int64_t n, int d, int n_trials, int vec_ok) {
-    __shared__ double scratch[4];
+    __shared__ double wave_pot[4][TN];
     const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
     const int best = header->best_row;
     const bool full = vec_ok && (i0 + 4 <= n);
+
+    // weights and the closest distances so far are needed after the feature loop: in flight
+    // during it
+    T w[4], cl[4];
+    load4<T>(sample_weight, i0, n, full, w);
+    load4<T>(rows + (size_t)best * n, i0, n, full, cl);
 
     T acc[TN][4];
 #pragma unroll
@@ -116,19 +156,7 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
         for (int j = 0; j < FB; ++j) {
             const int f = f0 + j < d ? f0 + j : d - 1;  // past the end: a valid row, ignored below
             const T* __restrict__ row = X_t + (size_t)f * n;
-            if (full) {
-                if constexpr (sizeof(T) == 4) {
-                    const float4 v = *reinterpret_cast<const float4*>(row + i0);
-                    xv[j][0] = v.x; xv[j][1] = v.y; xv[j][2] = v.z; xv[j][3] = v.w;
-                } else {
-                    const double2 a = *reinterpret_cast<const double2*>(row + i0);
-                    const double2 b = *reinterpret_cast<const double2*>(row + i0 + 2);
-                    xv[j][0] = a.x; xv[j][1] = a.y; xv[j][2] = b.x; xv[j][3] = b.y;
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) xv[j][r] = (i0 + r < n) ? row[i0 + r] : T(0);
-            }
+            load4<T>(row, i0, n, full, xv[j]);
         }
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
@@ -149,35 +177,34 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
         }
     }
 
-    T w[4], cl[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const bool ok = i0 + r < n;
-        w[r] = ok ? sample_weight[i0 + r] : T(0);
-        cl[r] = ok ? rows[(size_t)best * n + i0 + r] : T(0);
-    }
     double pot[TN];
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
         pot[t] = 0.0;
         if (t < n_trials) {
+            T v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                if (i0 + r < n) {
-                    const T v = fmin(acc[t][r] * w[r], cl[r]);
-                    rows[(size_t)t * n + i0 + r] = v;
-                    pot[t] += (double)v;
-                }
+                v[r] = fmin(acc[t][r] * w[r], cl[r]);
+                if (i0 + r < n) pot[t] += (double)v[r];
             }
+            store4<T>(rows + (size_t)t * n, i0, n, full, v);
         }
     }
+    // all row sums of the workgroup with one barrier: waves first, then one thread per trial
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
         if (t < n_trials) {
-            const double tot = kmx_block_sum<double>(pot[t], scratch);
-            if (threadIdx.x == 0) block_pot[(size_t)blockIdx.x * TN_MAX + t] = tot;
+            const double ws = kmx_wave_sum<double>(pot[t]);
+            if (lane == 0) wave_pot[wave][t] = ws;
         }
     }
+    __syncthreads();
+    if (threadIdx.x < n_trials)
+        block_pot[(size_t)blockIdx.x * TN_MAX + threadIdx.x] =
+            (wave_pot[0][threadIdx.x] + wave_pot[1][threadIdx.x]) +
+            (wave_pot[2][threadIdx.x] + wave_pot[3][threadIdx.x]);
 }
 
 // Block-wide exclusive scan of one double per thread (256 threads); returns the exclusive
@@ -213,11 +240,17 @@ __device__ __forceinline__ int64_t block_min_i64(int64_t v, int64_t* scratch) {
     return m;
 }
 
-// One workgroup per trial.
+// One workgroup per trial, plus one that records the selection.
 //   do_select: sum the block potentials of every row of the last step, pick the best row
-//              (lowest index on ties); workgroup 0 records potentials, header, centre slot.
-//   do_sample: candidate t = first j with scan(closest)_j >= uniforms[t] * total.
-template <typename T>
+//              (lowest index on ties); the last workgroup records potentials, header and the
+//              centre slot and does not sample.
+//   do_sample: candidate t = first j with scan(closest)_j >= uniforms[t] * total, and the
+//              candidate's feature row for the step kernel.
+// Thread i owns the block sums [i * P, (i + 1) * P); with P <= KPP_OWN they are read once and
+// stay in registers for the row totals, the coarse scan and the search.
+constexpr int KPP_OWN = 4;
+
+template <typename T, int TN>
 __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     const T* __restrict__ X_t, const double* __restrict__ uniforms,
     const int32_t* __restrict__ cand_prev, int32_t* __restrict__ cand_next,
@@ -227,69 +260,127 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     KppHeader* __restrict__ header, T* __restrict__ cand_rows, int64_t n, int64_t n_blocks, int d,
     int k, int n_trials, int center_slot, int do_select, int do_sample) {
     __shared__ double wave_tot[4];
-    __shared__ double dscratch[4];
+    __shared__ double wave_pot[4][TN];
     __shared__ int64_t iscratch[4];
-    __shared__ double pot_s[TN_MAX];
     __shared__ double prefix_s;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-    int best = header->best_row;
+    const int64_t per_thread = (n_blocks + 255) / 256;
+    const bool cached = per_thread <= KPP_OWN;
+    const int64_t b0 = (int64_t)threadIdx.x * per_thread;
+    int64_t b1 = b0 + per_thread;
+    if (b1 > n_blocks) b1 = n_blocks;
+
+    int best;
+    double own_best[KPP_OWN];  // the owned block sums of the best row (cached mode)
+#pragma unroll
+    for (int i = 0; i < KPP_OWN; ++i) own_best[i] = 0.0;
+
     if (do_select) {
-        // all trial sums in one pass over the block potentials (one row of TN_MAX doubles per
-        // block), then one block reduction per trial without memory traffic in between
-        double acc[TN_MAX];
+        double acc[TN];
+        double own[KPP_OWN][TN];
 #pragma unroll
-        for (int t = 0; t < TN_MAX; ++t) acc[t] = 0.0;
-        for (int64_t b = threadIdx.x; b < n_blocks; b += 256) {
-            const double* __restrict__ rowp = block_pot + (size_t)b * TN_MAX;
+        for (int t = 0; t < TN; ++t) acc[t] = 0.0;
+        if (cached) {
 #pragma unroll
-            for (int t = 0; t < TN_MAX; ++t)
-                if (t < n_trials) acc[t] += rowp[t];
+            for (int i = 0; i < KPP_OWN; ++i) {
+                const int64_t b = b0 + i;
+                const double* __restrict__ rowp = block_pot + (size_t)(b < n_blocks ? b : 0) * TN_MAX;
+#pragma unroll
+                for (int t = 0; t < TN; ++t) own[i][t] = (b < b1 && t < n_trials) ? rowp[t] : 0.0;
+            }
+#pragma unroll
+            for (int i = 0; i < KPP_OWN; ++i)
+#pragma unroll
+                for (int t = 0; t < TN; ++t) acc[t] += own[i][t];
+        } else {
+            for (int64_t b = b0; b < b1; ++b) {
+                const double* __restrict__ rowp = block_pot + (size_t)b * TN_MAX;
+#pragma unroll
+                for (int t = 0; t < TN; ++t)
+                    if (t < n_trials) acc[t] += rowp[t];
+            }
         }
 #pragma unroll
-        for (int t = 0; t < TN_MAX; ++t) {
+        for (int t = 0; t < TN; ++t) {
             if (t < n_trials) {
-                const double tot = kmx_block_sum<double>(acc[t], dscratch);
-                if (threadIdx.x == 0) pot_s[t] = tot;
+                const double ws = kmx_wave_sum<double>(acc[t]);
+                if (lane == 0) wave_pot[wave][t] = ws;
             }
         }
         __syncthreads();
+        double best_pot = (wave_pot[0][0] + wave_pot[1][0]) + (wave_pot[2][0] + wave_pot[3][0]);
         best = 0;
-        for (int t = 1; t < n_trials; ++t)
-            if (pot_s[t] < pot_s[best]) best = t;
-        if (blockIdx.x == 0) {
+        for (int t = 1; t < n_trials; ++t) {
+            const double pt = (wave_pot[0][t] + wave_pot[1][t]) + (wave_pot[2][t] + wave_pot[3][t]);
+            if (pt < best_pot) {
+                best_pot = pt;
+                best = t;
+            }
+        }
+        if (cached) {
+#pragma unroll
+            for (int i = 0; i < KPP_OWN; ++i)
+#pragma unroll
+                for (int t = 0; t < TN; ++t) own_best[i] = (t == best) ? own[i][t] : own_best[i];
+        }
+        if (blockIdx.x == gridDim.x - 1) {
             const int32_t chosen = cand_prev[best];
             for (int f = threadIdx.x; f < d; f += 256)
                 centers_t[(size_t)f * k + center_slot] = X_t[(size_t)f * n + chosen];
+            if (threadIdx.x < n_trials)
+                potentials[threadIdx.x] = (wave_pot[0][threadIdx.x] + wave_pot[1][threadIdx.x]) +
+                                          (wave_pot[2][threadIdx.x] + wave_pot[3][threadIdx.x]);
             if (threadIdx.x == 0) {
-                for (int t = 0; t < n_trials; ++t) potentials[t] = pot_s[t];
                 center_indices[center_slot] = chosen;
                 header->best_row = best;
-                header->total = pot_s[best];
+                header->total = best_pot;
             }
+            return;
+        }
+    } else {
+        best = header->best_row;
+        if (cached) {
+#pragma unroll
+            for (int i = 0; i < KPP_OWN; ++i)
+                if (b0 + i < b1) own_best[i] = block_pot[(size_t)(b0 + i) * TN_MAX + best];
         }
     }
     if (!do_sample) return;
 
     const int trial = blockIdx.x;
     // ---- coarse level: exclusive scan of the block sums of the best row
-    const int64_t per_thread = (n_blocks + 255) / 256;
-    const int64_t b0 = (int64_t)threadIdx.x * per_thread;
-    int64_t b1 = b0 + per_thread;
-    if (b1 > n_blocks) b1 = n_blocks;
     double local = 0.0;
-    for (int64_t b = b0; b < b1; ++b) local += block_pot[(size_t)b * TN_MAX + best];
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < KPP_OWN; ++i) local += own_best[i];
+    } else {
+        for (int64_t b = b0; b < b1; ++b) local += block_pot[(size_t)b * TN_MAX + best];
+    }
     double total;
     const double excl = block_exclusive_scan(local, wave_tot, total);
     const double rv = uniforms[trial] * total;
     int64_t found = INT64_MAX;
     double cum = excl, found_prefix = 0.0;
-    for (int64_t b = b0; b < b1; ++b) {
-        const double before = cum;
-        cum += block_pot[(size_t)b * TN_MAX + best];
-        if (cum >= rv) {
-            found = b;
-            found_prefix = before;
-            break;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < KPP_OWN; ++i) {
+            const double before = cum;
+            cum += own_best[i];
+            if (found == INT64_MAX && b0 + i < b1 && cum >= rv) {
+                found = b0 + i;
+                found_prefix = before;
+            }
+        }
+    } else {
+        for (int64_t b = b0; b < b1; ++b) {
+            const double before = cum;
+            cum += block_pot[(size_t)b * TN_MAX + best];
+            if (cum >= rv) {
+                found = b;
+                found_prefix = before;
+                break;
+            }
         }
     }
     const int64_t bstar_raw = block_min_i64(found, iscratch);
@@ -373,7 +464,8 @@ template <typename T>
 void launch_step(const void* X_t, const void* w, const int32_t* cand, const KppPtrs& p,
                  const KppLayout& L, int64_t n, int d, int n_trials, hipStream_t s) {
     (void)cand;  // the candidates' rows were copied to p.cand_rows when they were sampled
-    const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0);
+    const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0) && (((uintptr_t)w) % 16 == 0) &&
+                       (((uintptr_t)p.rows) % 16 == 0);
     if (n_trials <= 8)
         hipLaunchKernelGGL((kpp_step_kernel<T, 8>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
                            (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,
@@ -389,11 +481,19 @@ void launch_select_sample(const void* X_t, const double* uniforms, const int32_t
                           int32_t* cand_next, int32_t* cand_out, void* centers_t, int32_t* idx,
                           const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k,
                           int n_trials, int slot, int do_select, int do_sample, hipStream_t s) {
-    const unsigned grid = do_sample ? (unsigned)n_trials : 1u;
-    hipLaunchKernelGGL((kpp_select_sample_kernel<T>), dim3(grid), dim3(256), 0, s, (const T*)X_t,
-                       uniforms, cand_prev, cand_next, cand_out, (T*)centers_t, idx,
-                       (const T*)p.rows, p.block_pot, p.potentials, p.header, (T*)p.cand_rows, n,
-                       L.n_blocks, d, k, n_trials, slot, do_select, do_sample);
+    // one workgroup per trial when sampling, one more when a selection is recorded
+    const unsigned grid = (do_sample ? (unsigned)n_trials : 0u) + (do_select ? 1u : 0u);
+    if (grid == 0) return;
+#define KMX_KPP_SELECT(TN)                                                                        \
+    hipLaunchKernelGGL((kpp_select_sample_kernel<T, TN>), dim3(grid), dim3(256), 0, s,             \
+                       (const T*)X_t, uniforms, cand_prev, cand_next, cand_out, (T*)centers_t, idx, \
+                       (const T*)p.rows, p.block_pot, p.potentials, p.header, (T*)p.cand_rows, n,   \
+                       L.n_blocks, d, k, n_trials, slot, do_select, do_sample)
+    if (n_trials <= 8)
+        KMX_KPP_SELECT(8);
+    else
+        KMX_KPP_SELECT(TN_MAX);
+#undef KMX_KPP_SELECT
 }
 
 }  // namespace
