@@ -271,28 +271,33 @@ __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint32_t* __r
         order[atomicAdd(cursors + labels[i], 1)] = (int)i;
 }
 
-// One workgroup per (cluster, chunk of ACC_CHUNK samples).  Rows of the ROW-MAJOR copy of X
-// are contiguous: a wave reads one whole row per load instruction (lane l takes features
-// 4l .. 4l + 3 as one 128-bit load, d <= 256), the four waves of the workgroup take
-// different samples, and every lane keeps U loads in flight.  Sums are 64-bit fixed point in
-// registers; each wave adds its totals to the global sums.  Clears counts for the next
+// One workgroup per ACC_CHUNK consecutive positions of `order` (samples sorted by cluster),
+// whatever the cluster sizes: a workgroup walks the cluster segments inside its range and
+// adds one set of totals per segment.  Rows of the ROW-MAJOR copy of X are contiguous: a wave
+// reads one whole row per load instruction (lane l takes features 4l .. 4l + 3 as one 128-bit
+// load, d <= 256), the four waves of the workgroup take different samples, and every lane
+// keeps U loads in flight.  Sums are 64-bit fixed point in registers; the waves' totals are
+// combined in LDS and added to the global sums once per segment.  Clears counts for the next
 // iteration.
-constexpr int ACC_CHUNK = 256;
+constexpr int ACC_CHUNK = 1024;
+constexpr int WIDE_D_MAX = 256;
 
 template <bool VEC>
 __global__ __launch_bounds__(256) void bucket_accumulate_kernel(
     const float* __restrict__ X_rm, const float* __restrict__ sample_weight,
     const int* __restrict__ order, const int* __restrict__ offsets, int* __restrict__ counts,
-    const int* __restrict__ q_exp, unsigned long long* __restrict__ gsum, int d, int k,
-    int chunks_per_cluster) {
-    const int c = blockIdx.x / chunks_per_cluster;
-    const int chunk = blockIdx.x - c * chunks_per_cluster;
-    const int begin = offsets[c], end = offsets[c + 1];
-    const int p0 = begin + chunk * ACC_CHUNK;
-    if (chunk == 0 && threadIdx.x == 0) counts[c] = 0;
-    if (p0 >= end) return;
-    // clusters larger than chunks_per_cluster * ACC_CHUNK: the last chunk takes the remainder
-    const int p1 = (chunk == chunks_per_cluster - 1) ? end : (p0 + ACC_CHUNK < end ? p0 + ACC_CHUNK : end);
+    const int* __restrict__ q_exp, unsigned long long* __restrict__ gsum, int n, int d, int k) {
+    __shared__ long long red[4][WIDE_D_MAX + 1];
+    __shared__ int c_first;
+    const int P0 = blockIdx.x * ACC_CHUNK;
+    const int P1 = P0 + ACC_CHUNK < n ? P0 + ACC_CHUNK : n;
+    for (int c = blockIdx.x * 256 + threadIdx.x; c < k; c += gridDim.x * 256) counts[c] = 0;
+    if (threadIdx.x == 0) c_first = k;
+    __syncthreads();
+    // the (non-empty) cluster that holds position P0
+    for (int c = threadIdx.x; c < k; c += 256)
+        if (offsets[c] <= P0 && P0 < offsets[c + 1]) c_first = c;
+    __syncthreads();
 
     constexpr int U = 8;  // rows in flight per lane
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -302,51 +307,78 @@ __global__ __launch_bounds__(256) void bucket_accumulate_kernel(
     for (int j = 0; j < 4; ++j) sc[j] = f4 + j < d ? (double)ldexpf(1.0f, q_exp[f4 + j]) : 0.0;
     const double sc_w = (double)ldexpf(1.0f, q_exp[d]);
     const float* __restrict__ col = X_rm + (f4 < d ? f4 : 0);
-    long long acc[4] = {0, 0, 0, 0};
-    long long wsum = 0;
 
-    for (int base = p0; base < p1; base += 64) {
-        // each lane fetches one sample index and its weight (one coalesced load + one gather
-        // per 64 samples); lanes past the end hold the last valid sample with weight 0
-        const int pl = base + lane;
-        const int my_idx = order[pl < p1 ? pl : p1 - 1];
-        const float my_w = pl < p1 ? sample_weight[my_idx] : 0.0f;
-        const int n_here = p1 - base < 64 ? p1 - base : 64;
-        for (int u0 = wave; u0 < n_here; u0 += 4 * U) {
-            int idx[U];
-            float wv[U];
-            float xv[U][4];
+    int c = c_first;
+    int pos = P0;
+    while (pos < P1 && c < k) {
+        const int c_end = offsets[c + 1];  // wave-uniform
+        const int p0 = pos, p1 = c_end < P1 ? c_end : P1;
+        if (p1 > p0) {
+            long long acc[4] = {0, 0, 0, 0};
+            long long wsum = 0;
+            // each lane fetches one sample index and its weight (one coalesced load + one
+            // gather per 64 samples), one group ahead of the rows; lanes past the end hold the
+            // last valid sample with weight 0
+            auto fetch = [&](int base, int& idx_out, float& w_out) {
+                const int pl = base + lane;
+                idx_out = order[pl < p1 ? pl : p1 - 1];
+                w_out = pl < p1 ? sample_weight[idx_out] : 0.0f;
+            };
+            int my_idx, next_idx = 0;
+            float my_w, next_w = 0.0f;
+            fetch(p0, my_idx, my_w);
+            for (int base = p0; base < p1; base += 64) {
+                if (base + 64 < p1) fetch(base + 64, next_idx, next_w);
+                const int n_here = p1 - base < 64 ? p1 - base : 64;
+                for (int u0 = wave; u0 < n_here; u0 += 4 * U) {
+                    int idx[U];
+                    float wv[U];
+                    float xv[U][4];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int src = u0 + 4 * u;  // wave-uniform
-                idx[u] = __builtin_amdgcn_readlane(my_idx, src & 63);
-                wv[u] = src < 64 ? __builtin_amdgcn_readlane(my_w, src & 63) : 0.0f;
-            }
+                    for (int u = 0; u < U; ++u) {
+                        const int src = u0 + 4 * u;  // wave-uniform
+                        idx[u] = __builtin_amdgcn_readlane(my_idx, src & 63);
+                        wv[u] = src < 64 ? __builtin_amdgcn_readlane(my_w, src & 63) : 0.0f;
+                    }
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const float* __restrict__ row = col + (size_t)idx[u] * d;
-                if (VEC) {
-                    const float4 v = *reinterpret_cast<const float4*>(row);
-                    xv[u][0] = v.x; xv[u][1] = v.y; xv[u][2] = v.z; xv[u][3] = v.w;
-                } else {
+                    for (int u = 0; u < U; ++u) {
+                        const float* __restrict__ row = col + (size_t)idx[u] * d;
+                        if (VEC) {
+                            const float4 v = *reinterpret_cast<const float4*>(row);
+                            xv[u][0] = v.x; xv[u][1] = v.y; xv[u][2] = v.z; xv[u][3] = v.w;
+                        } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) xv[u][j] = f4 + j < d ? row[j] : 0.0f;
+                            for (int j = 0; j < 4; ++j) xv[u][j] = f4 + j < d ? row[j] : 0.0f;
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const double wd = (double)wv[u];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            acc[j] += (long long)to_fixed(fma((double)xv[u][j], wd * sc[j], FIX_MAGIC));
+                        wsum += (long long)to_fixed(fma(wd, sc_w, FIX_MAGIC));
+                    }
                 }
+                my_idx = next_idx;
+                my_w = next_w;
             }
+            // the four waves' totals meet in LDS; one global atomic per feature and segment
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const double wd = (double)wv[u];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[j] += (long long)to_fixed(fma((double)xv[u][j], wd * sc[j], FIX_MAGIC));
-                wsum += (long long)to_fixed(fma(wd, sc_w, FIX_MAGIC));
+            for (int j = 0; j < 4; ++j)
+                if (f4 + j < WIDE_D_MAX) red[wave][f4 + j] = acc[j];
+            if (lane == 0) red[wave][WIDE_D_MAX] = wsum;
+            __syncthreads();
+            for (int f = threadIdx.x; f <= d; f += 256) {
+                const int slot = f < d ? f : WIDE_D_MAX;
+                const long long tot = (red[0][slot] + red[1][slot]) + (red[2][slot] + red[3][slot]);
+                if (tot != 0) atomicAdd(gsum + (size_t)f * k + c, (unsigned long long)tot);
             }
+            __syncthreads();
+            pos = p1;
         }
+        ++c;
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-        if (f4 + j < d && acc[j] != 0) atomicAdd(gsum + (size_t)(f4 + j) * k + c, (unsigned long long)acc[j]);
-    if (lane == 0 && wsum != 0) atomicAdd(gsum + (size_t)d * k + c, (unsigned long long)wsum);
 }
 
 template <int MODE>
@@ -414,18 +446,15 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
     if (sg > 2048) sg = 2048;
     hipLaunchKernelGGL(bucket_scatter_kernel, dim3((unsigned)sg), dim3(256), 0, stream, labels, cursors,
                        order, n);
-    // enough chunks that a cluster of twice the mean size is split evenly; a bigger cluster's
-    // last chunk takes the rest
-    int chunks = (int)kmx_cdiv(2 * kmx_cdiv(n, k), ACC_CHUNK);
-    if (chunks < 1) chunks = 1;
+    const unsigned ag = (unsigned)kmx_cdiv(n, ACC_CHUNK);
     if (d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0))
-        hipLaunchKernelGGL((bucket_accumulate_kernel<true>), dim3((unsigned)(k * chunks)), dim3(256), 0,
-                           stream, (const float*)X_rowmajor, (const float*)w, order, offsets, counts,
-                           q_exp, gsum, d, k, chunks);
+        hipLaunchKernelGGL((bucket_accumulate_kernel<true>), dim3(ag), dim3(256), 0, stream,
+                           (const float*)X_rowmajor, (const float*)w, order, offsets, counts, q_exp,
+                           gsum, (int)n, d, k);
     else
-        hipLaunchKernelGGL((bucket_accumulate_kernel<false>), dim3((unsigned)(k * chunks)), dim3(256), 0,
-                           stream, (const float*)X_rowmajor, (const float*)w, order, offsets, counts,
-                           q_exp, gsum, d, k, chunks);
+        hipLaunchKernelGGL((bucket_accumulate_kernel<false>), dim3(ag), dim3(256), 0, stream,
+                           (const float*)X_rowmajor, (const float*)w, order, offsets, counts, q_exp,
+                           gsum, (int)n, d, k);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
