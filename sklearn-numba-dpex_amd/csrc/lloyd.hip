@@ -522,6 +522,7 @@ __global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words)
 
 // Workgroups of a vector-ALU fused step (also the number of partial slots it fills).
 int lloyd_fused_grid(const LloydLayout& L, int64_t n, int d, int dtype) {
+    if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n);
     const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype) : 2;
     const int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
     const int cap = L.grid_cap(kmx_num_cus());
@@ -546,7 +547,10 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
                   uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
                   hipStream_t stream) {
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
-    if (L.variant == KMX_VARIANT_REGISTER) {
+    if (L.variant == KMX_VARIANT_MFMA_F64) {
+        (void)kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
+                                      status, n, d, k, ACC != ACC_NONE, stream);
+    } else if (L.variant == KMX_VARIANT_REGISTER) {
 #define KMX_REG_CASE(DR, RR)                                                                    \
     launch_reg<T, DR, RR, ACC>(L, X_t, w, cpack, half_norms, labels_prev, labels, partial, status, \
                                n, d, k, grid, stream)

@@ -8,6 +8,7 @@ constexpr int KMX_VARIANT_STREAM = 0;    // wide samples: features re-read per c
 constexpr int KMX_VARIANT_REGISTER = 1;  // samples held in registers, centroids in SGPRs
 constexpr int KMX_VARIANT_MFMA = 3;      // fp32 distances on the matrix cores, LDS accumulators
 constexpr int KMX_VARIANT_MFMA_WIDE = 4; // fp32 matrix cores, samples in registers, global sums
+constexpr int KMX_VARIANT_MFMA_F64 = 5;  // fp64 distances on the matrix cores, LDS accumulators
 
 constexpr int KMX_ACC_LDS = 1;
 constexpr int KMX_ACC_GLOBAL = 2;
@@ -25,6 +26,7 @@ int kmx_wgs_per_cu_env();
 // those its wide-sample variant covers (samples in registers, centroids streamed).
 bool kmx_mfma_supported(int d, int k);
 bool kmx_mfma_wide_supported(int d, int k);
+bool kmx_mfma_f64_supported(int d, int k);
 
 struct LloydLayout {
     int dpad;            // features per packed centroid row (multiple of 4, zero padded)
@@ -75,6 +77,9 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
         L.variant = KMX_VARIANT_MFMA;
     else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA_WIDE;
+    else if (dtype == KMX_F64 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_f64_supported(d, k) &&
+             (forced < 0 || forced == KMX_VARIANT_MFMA))
+        L.variant = KMX_VARIANT_MFMA_F64;
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
     L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));
@@ -115,3 +120,11 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
 int32_t kmx_assign_labels_mfma_wide_f32(const LloydLayout& L, const void* X_t,
                                         const void* centroids_t, uint32_t* labels, char* ws,
                                         int64_t n, int d, int k, hipStream_t stream);
+
+// fp64 matrix-core fused step (lloyd_mfma_f64.hip): fills partial[0 .. grid) like the
+// vector-ALU kernels with LDS accumulators; `update` false = labels only
+int kmx_mfma_f64_grid(int64_t n);
+int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* centroids_t,
+                                const void* half_norms, const uint32_t* labels_prev,
+                                uint32_t* labels, void* partial, kmx_lloyd_status* status,
+                                int64_t n, int d, int k, bool update, hipStream_t stream);

@@ -1,0 +1,277 @@
+// fp64 fused Lloyd step on the matrix cores (gfx950), for d <= 32 when the (d + 1) * k
+// accumulators fit in LDS.
+//
+// Replaces, for these shapes, the kernel pair fused_lloyd_single_step
+// (sklearn_numba_dpex/kmeans/kernels/lloyd_single_step.py:35-424) + the zero-fill / half-norm
+// helpers (common/kernels.py:38-57, 116-145); the reduction over the workgroups' partial sums
+// and the finalisation stay with lloyd.hip.
+//
+//   * v_mfma_f64_16x16x4_f64: A = 16 centroids x 4 features (lane l: centroid l % 16, feature
+//     l / 16), B = 4 features x 16 samples (lane l: feature l / 16, sample l % 16), D = 16 x 16
+//     with lane l holding rows l / 16 + 4 r (r = 0..3) of column l % 16.
+//   * A wave owns 64 consecutive samples: lane (g, j) = (l / 16, l % 16) loads the four samples
+//     4 j .. 4 j + 3 of feature row 4 s + g with two 128-bit loads (a 16-lane group reads 512
+//     contiguous bytes), and component t of that vector is the B operand of MFMA chain t, so
+//     no shuffles.  Four independent chains per centroid block, accumulators start at
+//     -0.5 ||c||^2, so after the K loop a lane holds <x, c> - 0.5 ||c||^2 for 4 centroids of
+//     each of its 4 samples.
+//   * fp64 MFMA and vector-ALU instructions do not overlap on this hardware (measured), so the
+//     arg-max is kept short: per chain a 3-instruction max of the 4 rows, one compare, and only
+//     the winning lanes copy the rows; the position is resolved once per tile.  Strict `>` in
+//     increasing centroid order: the lowest index wins a tie.
+//   * Partial sums in workgroup-private LDS accumulators (ds_add_f64 is fast on this part),
+//     written to the workgroup's slot of `partial` at the end.
+#include "lloyd_layout.h"
+
+namespace {
+
+typedef double v4d __attribute__((ext_vector_type(4)));
+
+constexpr int F64_WAVES = 8;  // two waves per SIMD, one workgroup per compute unit
+
+// Four consecutive doubles of a row.
+__device__ __forceinline__ void load4d(const double* __restrict__ p, double (&v)[4]) {
+    const double2 a = *reinterpret_cast<const double2*>(p);
+    const double2 b = *reinterpret_cast<const double2*>(p + 2);
+    v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y;
+}
+
+template <int NKS, bool UPDATE>
+__global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
+    const double* __restrict__ X_t, const double* __restrict__ sample_weight,
+    const double* __restrict__ centroids_t, const double* __restrict__ half_norms,
+    const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
+    double* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k,
+    int vec_ok) {
+    if (UPDATE && status->state != KMX_RUNNING) return;
+    constexpr int THREADS = 64 * F64_WAVES;
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int n_cb = (k + 15) >> 4;  // centroid blocks of 16
+    const int items = (d + 1) * k;
+    double* acc = reinterpret_cast<double*>(smem_raw);                   // [(d + 1) * k]
+    double* afrag = acc + (UPDATE ? items : 0);                          // [n_cb][NKS][64]
+    double* hneg = afrag + (size_t)n_cb * NKS * 64;                      // [n_cb * 16]
+    __shared__ unsigned int changed_block;
+
+    for (int idx = threadIdx.x; idx < n_cb * NKS * 64; idx += THREADS) {
+        const int l = idx & 63;
+        const int s = (idx >> 6) % NKS;
+        const int cb = (idx >> 6) / NKS;
+        const int c = 16 * cb + (l & 15);
+        const int f = 4 * s + (l >> 4);
+        afrag[idx] = (c < k && f < d) ? centroids_t[(size_t)f * k + c] : 0.0;
+    }
+    for (int c = threadIdx.x; c < n_cb * 16; c += THREADS)
+        hneg[c] = c < k ? -half_norms[c] : -kmx_inf<double>();
+    if (UPDATE) {
+        for (int jx = threadIdx.x; jx < items; jx += THREADS) acc[jx] = 0.0;
+        if (threadIdx.x == 0) changed_block = 0;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, j = lane & 15;
+    const int64_t n_wtiles = (n + 63) >> 6;
+    unsigned int changed = 0;
+
+    for (int64_t wt = (int64_t)blockIdx.x * F64_WAVES + wave; wt < n_wtiles;
+         wt += (int64_t)gridDim.x * F64_WAVES) {
+        const int64_t i0 = wt * 64 + 4 * j;
+        const bool fast = vec_ok && (wt + 1) * 64 <= n;  // wave-uniform
+
+        double x[NKS][4];
+        double wv[4] = {0.0, 0.0, 0.0, 0.0};
+        uint32_t pl[4] = {0u, 0u, 0u, 0u};
+        if (fast) {
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) {
+                const int f = 4 * s + g;
+                // a row past d - 1 reads row d - 1: its A fragment is zero, the update skips it
+                load4d(X_t + (size_t)(f < d ? f : d - 1) * n + i0, x[s]);
+            }
+            if (UPDATE) {
+                load4d(sample_weight + i0, wv);
+                const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+                pl[0] = p4.x; pl[1] = p4.y; pl[2] = p4.z; pl[3] = p4.w;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) {
+                const int f = 4 * s + g;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    x[s][t] = (f < d && i0 + t < n) ? X_t[(size_t)f * n + i0 + t] : 0.0;
+            }
+            if (UPDATE) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    if (i0 + t < n) {
+                        wv[t] = sample_weight[i0 + t];
+                        pl[t] = labels_prev[i0 + t];
+                    }
+                }
+            }
+        }
+
+        double best[4];
+        int code[4];
+        v4d sv[4];  // the rows of the winning block
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            best[t] = -kmx_inf<double>();
+            code[t] = 0;
+            sv[t] = v4d{0.0, 0.0, 0.0, 0.0};
+        }
+
+        for (int cb = 0; cb < n_cb; ++cb) {
+            const double* hp = hneg + cb * 16 + g;
+            const v4d hv = {hp[0], hp[4], hp[8], hp[12]};
+            const double* ap = afrag + (size_t)cb * NKS * 64 + lane;
+            double af = ap[0];
+            v4d a[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) a[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(af, x[0][t], hv, 0, 0, 0);
+#pragma unroll
+            for (int s = 1; s < NKS; ++s) {
+                af = ap[s * 64];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    a[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(af, x[s][t], a[t], 0, 0, 0);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const double m = fmax(fmax(a[t][0], a[t][1]), fmax(a[t][2], a[t][3]));
+                if (m > best[t]) {  // strict: the earlier block keeps a tie
+                    best[t] = m;
+                    code[t] = cb;
+                    sv[t] = a[t];
+                }
+            }
+        }
+
+        // row inside the winning block (lowest row = lowest centroid of this lane), then the
+        // four lane groups of a column are combined: highest score, lowest centroid on ties
+        uint32_t lab[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int pos = 3;
+#pragma unroll
+            for (int r = 2; r >= 0; --r) pos = (sv[t][r] == best[t]) ? r : pos;
+            int c = 16 * code[t] + g + 4 * pos;
+            double b = best[t];
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const double ob = __shfl_xor(b, off, 64);
+                const int oc = __shfl_xor(c, off, 64);
+                if (ob > b || (ob == b && oc < c)) {
+                    b = ob;
+                    c = oc;
+                }
+            }
+            lab[t] = (uint32_t)c;
+        }
+
+        if (g == 0) {
+            if (fast) {
+                *reinterpret_cast<uint4*>(labels + i0) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (i0 + t < n) labels[i0 + t] = lab[t];
+            }
+        }
+
+        if (UPDATE) {
+            if (g == 0) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    changed += ((fast || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
+                    // samples past the end carry w = 0
+                    if (fast || i0 + t < n) kmx_atomic_add(acc + (size_t)d * k + lab[t], wv[t]);
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) {
+                const int f = 4 * s + g;
+                if (f < d) {
+                    double* rowacc = acc + (size_t)f * k;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (fast || i0 + t < n) kmx_atomic_add(rowacc + lab[t], x[s][t] * wv[t]);
+                }
+            }
+        }
+    }
+
+    if (UPDATE) {
+        if (changed) atomicAdd(&changed_block, changed);
+        __syncthreads();
+        double* out = partial + (size_t)blockIdx.x * items;
+        for (int jx = threadIdx.x; jx < items; jx += THREADS) out[jx] = acc[jx];
+        if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+    }
+}
+
+size_t mfma_f64_lds_bytes(int d, int k, bool update) {
+    const int nks = (d + 3) / 4, n_cb = (k + 15) / 16;
+    size_t bytes = ((size_t)n_cb * nks * 64 + (size_t)n_cb * 16) * sizeof(double);
+    if (update) bytes += (size_t)(d + 1) * k * sizeof(double);
+    return bytes;
+}
+
+}  // namespace
+
+bool kmx_mfma_f64_supported(int d, int k) {
+    return d <= 32 && k >= 16 && mfma_f64_lds_bytes(d, k, true) <= 64 * 1024;
+}
+
+int kmx_mfma_f64_grid(int64_t n) {
+    const int64_t tiles = kmx_cdiv(kmx_cdiv(n, 64), F64_WAVES);
+    const int64_t cap = (int64_t)(kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : 1) * kmx_num_cus();
+    int64_t grid = tiles < cap ? tiles : cap;
+    if (grid > KMX_MAX_PARTIALS) grid = KMX_MAX_PARTIALS;
+    return grid < 1 ? 1 : (int)grid;
+}
+
+int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* centroids_t,
+                                const void* half_norms, const uint32_t* labels_prev,
+                                uint32_t* labels, void* partial, kmx_lloyd_status* status,
+                                int64_t n, int d, int k, bool update, hipStream_t stream) {
+    if (!kmx_mfma_f64_supported(d, k)) return KMX_ERR_UNSUPPORTED;
+    const size_t lds = mfma_f64_lds_bytes(d, k, update);
+    const int grid = kmx_mfma_f64_grid(n);
+    auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
+    // rows start 16-byte aligned when n is even; 4 samples per lane need n % 4 == 0 only for
+    // the 128-bit label accesses
+    const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
+                       (!update || (aligned16(w) && aligned16(labels_prev)));
+#define KMX_F64_CASE(NKS)                                                                        \
+    do {                                                                                         \
+        if (update)                                                                              \
+            hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, true>), dim3((unsigned)grid),          \
+                               dim3(64 * F64_WAVES), lds, stream, (const double*)X_t,             \
+                               (const double*)w, (const double*)centroids_t,                      \
+                               (const double*)half_norms, labels_prev, labels, (double*)partial,  \
+                               status, n, d, k, vec_ok);                                          \
+        else                                                                                     \
+            hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, false>), dim3((unsigned)grid),         \
+                               dim3(64 * F64_WAVES), lds, stream, (const double*)X_t,             \
+                               (const double*)w, (const double*)centroids_t,                      \
+                               (const double*)half_norms, labels_prev, labels, (double*)partial,  \
+                               status, n, d, k, vec_ok);                                          \
+    } while (0)
+    switch ((d + 3) / 4) {
+        case 1: KMX_F64_CASE(1); break;
+        case 2: KMX_F64_CASE(2); break;
+        case 3: KMX_F64_CASE(3); break;
+        case 4: KMX_F64_CASE(4); break;
+        case 5: KMX_F64_CASE(5); break;
+        case 6: KMX_F64_CASE(6); break;
+        case 7: KMX_F64_CASE(7); break;
+        default: KMX_F64_CASE(8); break;
+    }
+#undef KMX_F64_CASE
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}

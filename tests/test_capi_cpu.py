@@ -74,7 +74,8 @@ def test_kernel_variant_selection():
     from sklearn_numba_dpex_amd._capi import lib
 
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 31   # MFMA + LDS accumulators
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 11    # fp64: register + LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 51    # fp64: matrix cores + LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1) in (12, 2)  # accumulators too big for LDS
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 42  # wide MFMA + global sums
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0) == 2   # streaming + global copies
     assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0) == 11           # too few clusters for MFMA
