@@ -226,6 +226,69 @@ def extra_configs():
     return out
 
 
+def gpu_components(cfg):
+    """Times of the other kernels of the path on the same data (configs[1]), each with its
+    algorithmic bytes: labels, inertia, labels + inertia as `predict`/`score` run them,
+    euclidean distances (on a slice: the output is n x k), radix top-k, sums, centering."""
+    import torch
+
+    from sklearn_numba_dpex_amd.common.reductions import sum_reduction
+    from sklearn_numba_dpex_amd.common.topk import topk_idx
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    dev = torch.device("cuda:0")
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    X_t = torch.as_tensor(X, device=dev).T.contiguous()
+    w_d = torch.as_tensor(w, device=dev)
+    cent_t = torch.as_tensor(np.ascontiguousarray(init.T), device=dev)
+    labels = torch.empty(n, dtype=torch.int32, device=dev)
+    s = 4
+
+    def timed(fn, reps=5):
+        fn()
+        ts = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    out = {}
+
+    def put(name, seconds, nbytes, note):
+        out[name] = {"ms": seconds * 1e3, "algorithmic_MB": nbytes / 1e6, "GBps": nbytes / seconds / 1e9,
+                     "hbm_frac": nbytes / seconds / 1e9 / HBM_PEAK_GBS, "what": note}
+
+    t = timed(lambda: drivers._assign(X_t, cent_t, labels))
+    put("assign_labels", t, n * (s * d + 4), "kmx_assign_labels (pack + labels kernel); fp32 contraction bound")
+    out["assign_labels"]["TFLOPs"] = 2.0 * n * d * k / t / 1e12
+    per_sample = torch.empty(n, dtype=X_t.dtype, device=dev)
+    t = timed(lambda: drivers._per_sample_inertia(X_t, w_d, cent_t, labels, out=per_sample))
+    put("per_sample_inertia", t, n * (s * d + 4 + 2 * s), "kmx_per_sample_inertia")
+    t = timed(lambda: sum_reduction(per_sample))
+    put("sum_1d", t, n * s, "kmx_sum_rows over n values (launches + workspace allocation included)")
+    t = timed(lambda: drivers.get_labels_inertia(X_t, cent_t, w_d, True))
+    put("get_labels_inertia", t, n * (2 * s * d + 8 + 3 * s),
+        "labels + inertia + sum + scalar read-back, as score() runs it")
+    m = min(n, 500_000)
+    Xs_t = X_t[:, :m].contiguous()
+    t = timed(lambda: drivers.get_euclidean_distances(Xs_t, cent_t))
+    put("euclidean_distances", t, m * (s * d + s * k),
+        f"kmx_euclidean_distances on {m} samples (output {m}x{k}, allocation included)")
+    t = timed(lambda: topk_idx(per_sample, 16))
+    put("topk_idx_16", t, 4 * n * s, "radix select of the 16 largest of n values: 4 passes of 8 bits over fp32 keys")
+    t = timed(lambda: sum_reduction(X_t, axis=1))
+    put("sum_rows_d_by_n", t, n * d * s, "kmx_sum_rows over X_t (d, n): the feature sums of the centering")
+    Xc = X_t.clone()
+    t = timed(lambda: drivers.prepare_data_for_lloyd(Xc, cent_t.clone(), 1e-4, w_d, copy_x=False))
+    put("prepare_data_for_lloyd", t, 4 * n * d * s,
+        "mean, centering in place, variance for tol, uniform-weight test (3 reads + 1 write of X)")
+    return out
+
+
 def gpu_kmeanspp(cfg):
     import torch
 
@@ -362,6 +425,8 @@ def main():
         del c4
 
     if not args.no_extra:
+        out["components"] = gpu_components(cfg)
+        log("[bench] components (ms): " + ", ".join(f"{k2} {v['ms']:.3f}" for k2, v in out["components"].items()))
         del cfg["X"]  # free host memory before the 1 GB configuration is generated
         out["other_configs"] = extra_configs()
         cfg = None
