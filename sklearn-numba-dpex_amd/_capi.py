@@ -11,6 +11,11 @@ from ctypes import POINTER, c_char_p, c_double, c_int32, c_int64, c_size_t, c_vo
 
 import numpy as np
 
+# torch ships its own copy of the HIP runtime.  It has to be in the process before this
+# library is loaded, so that both bind to the same runtime: with the load order reversed the
+# process holds two runtimes and the second one finds no device.
+import torch  # noqa: F401  (imported for its side effect on the loader)
+
 KMX_F32 = 0
 KMX_F64 = 1
 

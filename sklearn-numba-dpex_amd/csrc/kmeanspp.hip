@@ -512,6 +512,7 @@ int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_i
                      void* centers_t, int32_t* center_indices, void* workspace,
                      size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
                      int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     const int32_t rc = kpp_check(X_t, sample_weight, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
     KMX_REQUIRE_PTR(centers_t);
@@ -532,6 +533,7 @@ int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_st
                                   int32_t* candidates, void* workspace, size_t workspace_bytes,
                                   int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype,
                                   void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(uniforms_for_step);
     const int32_t rc = kpp_check(X_t, uniforms_for_step, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
@@ -552,6 +554,7 @@ int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_
                      void* centers_t, int32_t* center_indices, void* workspace,
                      size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
                      int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     const int32_t rc = kpp_check(X_t, sample_weight, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
     KMX_REQUIRE_PTR(centers_t);
@@ -577,6 +580,7 @@ int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* un
                     int32_t start_index, void* centers_t, int32_t* center_indices,
                     void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
                     int32_t n_trials, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     int32_t rc = kmx_kpp_init(X_t, sample_weight, start_index, centers_t, center_indices, workspace,
                               workspace_bytes, n, d, k, n_trials, dtype, stream_);
     if (rc != KMX_OK) return rc;

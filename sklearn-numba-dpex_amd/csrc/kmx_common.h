@@ -20,6 +20,11 @@
         if ((dt) != KMX_F32 && (dt) != KMX_F64) return KMX_ERR_BAD_DTYPE; \
     } while (0)
 
+// First statement of every entry point that launches kernels: hipGetLastError reports the
+// last error of ANY earlier runtime call of the thread (another library's probe included), so
+// a stale one is dropped here and KMX_LAUNCH_CHECK only sees this library's own launches.
+#define KMX_ENTRY() (void)hipGetLastError()
+
 #define KMX_LAUNCH_CHECK()                    \
     do {                                      \
         hipError_t e_ = hipGetLastError();    \

@@ -680,6 +680,7 @@ int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype)
 int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
                        const void* sample_weight, const void* centroids_t, int64_t n, int32_t d,
                        int32_t k, int32_t dtype, int32_t max_iter, double tol, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(workspace);
     KMX_REQUIRE_PTR(X_t);
     KMX_REQUIRE_PTR(sample_weight);
@@ -759,6 +760,7 @@ int32_t kmx_lloyd_iter(const void* X_t, const void* X_rowmajor, const void* samp
                        void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                        size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                        void* stream_) {
+    KMX_ENTRY();
     return lloyd_iter_dispatch(X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev, labels,
                                cluster_sizes, empty_clusters, workspace, workspace_bytes, n, d, k,
                                dtype, stream_, nullptr);
@@ -769,6 +771,7 @@ int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void
                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                              size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                              void* stream_, float* kernel_ms_host) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(kernel_ms_host);
     hipEvent_t ev[4];
     for (int i = 0; i < 4; ++i) {
@@ -791,6 +794,7 @@ int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void
 int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,
                            const void* cluster_sizes, void* workspace, size_t workspace_bytes,
                            int32_t d, int32_t k, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(centroids_t);
     KMX_REQUIRE_PTR(new_centroids_t);
     KMX_REQUIRE_PTR(cluster_sizes);
@@ -820,6 +824,7 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,
 }
 
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(workspace);
     KMX_REQUIRE_PTR(status_host);
     hipStream_t stream = (hipStream_t)stream_;
@@ -838,6 +843,7 @@ size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
 int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
                           void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
                           int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(X_t);
     KMX_REQUIRE_PTR(centroids_t);
     KMX_REQUIRE_PTR(labels);

@@ -4,22 +4,50 @@
 // block order), so results do not change from run to run.
 #include "kmx_common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int SUM_MAX_BLOCKS_PER_ROW = 256;
 constexpr int SUM_COL_CHUNKS = 64;
 
-template <typename T>
+// VEC: rows start 16-byte aligned and hold a whole number of 16-byte groups; a thread then
+// reads 16 bytes per load and keeps two loads in flight.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void sum_rows_stage1(const T* __restrict__ in,
                                                        double* __restrict__ partial, int64_t cols,
                                                        int square) {
     const int64_t row = blockIdx.y;
     const T* __restrict__ p = in + (size_t)row * cols;
     double acc = 0.0;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += stride) {
-        const double v = (double)p[c];
-        acc += square ? v * v : v;
+    if constexpr (VEC) {
+        constexpr int W = 16 / sizeof(T);
+        using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+        const V* __restrict__ pv = reinterpret_cast<const V*>(p);
+        const int64_t groups = cols / W;
+        const int64_t stride = (int64_t)gridDim.x * 256;
+        int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        auto add = [&](const V& v) {
+            const T* e = reinterpret_cast<const T*>(&v);
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                const double x = (double)e[j];
+                acc += square ? x * x : x;
+            }
+        };
+        for (; g + stride < groups; g += 2 * stride) {
+            const V a = pv[g];
+            const V b = pv[g + stride];
+            add(a);
+            add(b);
+        }
+        if (g < groups) add(pv[g]);
+    } else {
+        const int64_t stride = (int64_t)gridDim.x * 256;
+        for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += stride) {
+            const double v = (double)p[c];
+            acc += square ? v * v : v;
+        }
     }
     __shared__ double scratch[4];
     const double tot = kmx_block_sum<double>(acc, scratch);
@@ -107,16 +135,29 @@ __global__ __launch_bounds__(256) void half_sq_norms_kernel(const T* __restrict_
     out[c] = acc / T(2);
 }
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void broadcast_rows_kernel(T* __restrict__ a,
                                                              const T* __restrict__ v, int64_t rows,
                                                              int64_t cols, int op) {
     const int64_t row = blockIdx.y;
-    const T rv = v[row];
+    const T rv = op == 0 ? -v[row] : v[row];
     T* __restrict__ p = a + (size_t)row * cols;
     const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += stride)
-        p[c] = op == 0 ? p[c] - rv : p[c] + rv;
+    if constexpr (VEC) {
+        constexpr int W = 16 / sizeof(T);
+        using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+        V* __restrict__ pv = reinterpret_cast<V*>(p);
+        const int64_t groups = cols / W;
+        for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += stride) {
+            V x = pv[g];
+            T* e = reinterpret_cast<T*>(&x);
+#pragma unroll
+            for (int j = 0; j < W; ++j) e[j] = e[j] + rv;
+            pv[g] = x;
+        }
+    } else {
+        for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += stride) p[c] = p[c] + rv;
+    }
 }
 
 template <typename T>
@@ -234,6 +275,7 @@ size_t kmx_sum_workspace_bytes(int64_t rows, int64_t cols) {
 
 int32_t kmx_sum_rows(const void* in, void* out, int64_t rows, int64_t cols, int32_t square,
                      void* workspace, size_t workspace_bytes, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(in);
     KMX_REQUIRE_PTR(out);
     KMX_REQUIRE_PTR(workspace);
@@ -243,23 +285,28 @@ int32_t kmx_sum_rows(const void* in, void* out, int64_t rows, int64_t cols, int3
     if (workspace_bytes < (size_t)rows * b * sizeof(double)) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     double* partial = (double*)workspace;
+    const size_t es = kmx_dtype_size(dtype);
+    const bool vec = (((uintptr_t)in) % 16 == 0) && ((cols * es) % 16 == 0);
+#define KMX_SUM_ROWS(T, VEC)                                                                       \
+    do {                                                                                           \
+        hipLaunchKernelGGL((sum_rows_stage1<T, VEC>), dim3(b, (unsigned)rows), dim3(256), 0, stream, \
+                           (const T*)in, partial, cols, square);                                   \
+        hipLaunchKernelGGL((sum_rows_stage2<T>), dim3((unsigned)rows), dim3(256), 0, stream,        \
+                           partial, (T*)out, b);                                                   \
+    } while (0)
     if (dtype == KMX_F32) {
-        hipLaunchKernelGGL((sum_rows_stage1<float>), dim3(b, (unsigned)rows), dim3(256), 0, stream,
-                           (const float*)in, partial, cols, square);
-        hipLaunchKernelGGL((sum_rows_stage2<float>), dim3((unsigned)rows), dim3(256), 0, stream,
-                           partial, (float*)out, b);
+        if (vec) KMX_SUM_ROWS(float, true); else KMX_SUM_ROWS(float, false);
     } else {
-        hipLaunchKernelGGL((sum_rows_stage1<double>), dim3(b, (unsigned)rows), dim3(256), 0, stream,
-                           (const double*)in, partial, cols, square);
-        hipLaunchKernelGGL((sum_rows_stage2<double>), dim3((unsigned)rows), dim3(256), 0, stream,
-                           partial, (double*)out, b);
+        if (vec) KMX_SUM_ROWS(double, true); else KMX_SUM_ROWS(double, false);
     }
+#undef KMX_SUM_ROWS
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
 
 int32_t kmx_sum_cols(const void* in, void* out, int64_t rows, int64_t cols, void* workspace,
                      size_t workspace_bytes, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(in);
     KMX_REQUIRE_PTR(out);
     KMX_REQUIRE_PTR(workspace);
@@ -289,6 +336,7 @@ int32_t kmx_sum_cols(const void* in, void* out, int64_t rows, int64_t cols, void
 }
 
 int32_t kmx_argmin(const void* values, int32_t* out, int64_t n, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(values);
     KMX_REQUIRE_PTR(out);
     if (n <= 0 || n > INT32_MAX) return KMX_ERR_BAD_SHAPE;
@@ -306,6 +354,7 @@ int32_t kmx_argmin(const void* values, int32_t* out, int64_t n, int32_t dtype, v
 
 int32_t kmx_half_sq_norms(const void* a_t, void* out, int32_t rows, int32_t cols, int32_t dtype,
                           void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(a_t);
     KMX_REQUIRE_PTR(out);
     if (rows <= 0 || cols <= 0) return KMX_ERR_BAD_SHAPE;
@@ -324,6 +373,7 @@ int32_t kmx_half_sq_norms(const void* a_t, void* out, int32_t rows, int32_t cols
 
 int32_t kmx_broadcast_rows(void* a, const void* v, int64_t rows, int64_t cols, int32_t op,
                            int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(a);
     KMX_REQUIRE_PTR(v);
     if (rows <= 0 || cols <= 0 || rows > 65535) return KMX_ERR_BAD_SHAPE;
@@ -332,18 +382,24 @@ int32_t kmx_broadcast_rows(void* a, const void* v, int64_t rows, int64_t cols, i
     hipStream_t stream = (hipStream_t)stream_;
     int64_t gx = kmx_cdiv(cols, 256 * 4);
     if (gx > 2048) gx = 2048;
-    if (dtype == KMX_F32)
-        hipLaunchKernelGGL((broadcast_rows_kernel<float>), dim3((unsigned)gx, (unsigned)rows),
-                           dim3(256), 0, stream, (float*)a, (const float*)v, rows, cols, op);
-    else
-        hipLaunchKernelGGL((broadcast_rows_kernel<double>), dim3((unsigned)gx, (unsigned)rows),
-                           dim3(256), 0, stream, (double*)a, (const double*)v, rows, cols, op);
+    const size_t es = kmx_dtype_size(dtype);
+    const bool vec = (((uintptr_t)a) % 16 == 0) && ((cols * es) % 16 == 0);
+#define KMX_BCAST(T, VEC)                                                                       \
+    hipLaunchKernelGGL((broadcast_rows_kernel<T, VEC>), dim3((unsigned)gx, (unsigned)rows),      \
+                       dim3(256), 0, stream, (T*)a, (const T*)v, rows, cols, op)
+    if (dtype == KMX_F32) {
+        if (vec) KMX_BCAST(float, true); else KMX_BCAST(float, false);
+    } else {
+        if (vec) KMX_BCAST(double, true); else KMX_BCAST(double, false);
+    }
+#undef KMX_BCAST
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
 
 int32_t kmx_broadcast_div_cols(void* a, const void* v, int64_t rows, int64_t cols, int32_t dtype,
                                void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(a);
     KMX_REQUIRE_PTR(v);
     if (rows <= 0 || cols <= 0) return KMX_ERR_BAD_SHAPE;
@@ -361,6 +417,7 @@ int32_t kmx_broadcast_div_cols(void* a, const void* v, int64_t rows, int64_t col
 }
 
 int32_t kmx_divide_by(void* data, int64_t n_items, double divisor, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(data);
     if (n_items <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
@@ -377,6 +434,7 @@ int32_t kmx_divide_by(void* data, int64_t n_items, double divisor, int32_t dtype
 }
 
 int32_t kmx_fill_zero(void* data, int64_t n_bytes, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(data);
     if (n_bytes < 0) return KMX_ERR_BAD_SHAPE;
     if (n_bytes == 0) return KMX_OK;
@@ -389,6 +447,7 @@ int32_t kmx_fill_zero(void* data, int64_t n_bytes, void* stream_) {
 
 int32_t kmx_centroid_shifts(const void* a_t, const void* b_t, void* out, int32_t d, int32_t k,
                             int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(a_t);
     KMX_REQUIRE_PTR(b_t);
     KMX_REQUIRE_PTR(out);
@@ -408,6 +467,7 @@ int32_t kmx_centroid_shifts(const void* a_t, const void* b_t, void* out, int32_t
 
 int32_t kmx_is_same_clustering(const uint32_t* labels1, const uint32_t* labels2, int32_t* mapping,
                                int32_t* result, int64_t n, int32_t k, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(labels1);
     KMX_REQUIRE_PTR(labels2);
     KMX_REQUIRE_PTR(mapping);
@@ -427,6 +487,7 @@ int32_t kmx_is_same_clustering(const uint32_t* labels1, const uint32_t* labels2,
 
 int32_t kmx_count_distinct_clusters(const uint32_t* labels, int32_t* seen, int32_t* result,
                                     int64_t n, int32_t k, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(labels);
     KMX_REQUIRE_PTR(seen);
     KMX_REQUIRE_PTR(result);

@@ -246,6 +246,7 @@ size_t kmx_topk_workspace_bytes(int64_t n, int32_t k) {
 
 int32_t kmx_topk_idx(const void* values, int64_t* out_indices, int64_t n, int32_t k,
                      void* workspace, size_t workspace_bytes, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(values);
     KMX_REQUIRE_PTR(out_indices);
     KMX_REQUIRE_PTR(workspace);
