@@ -64,19 +64,44 @@ def gpu_lloyd(cfg, steps, warmup):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     stream = _capi.current_stream()
     status = _capi.LloydStatus()
-    total = warmup + 2 * steps + 8
+    cent_init = cent[0].clone()
+    # At tol = 0 the run stops by itself once no label changes (iteration 851 on configs[1]);
+    # kernels enqueued after that are no-ops.  So that every timed launch does its work for
+    # any --steps, the run restarts from the initial centroids every RESTART iterations (one
+    # tiny copy + kmx_lloyd_init, inside the timed region when it happens).
+    RESTART = 600
+    it = 0          # iterations since the last (re)start
+    done = 0        # iterations that must have done work, over all restarts
+    checked = 0
 
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, total, 0.0, stream), "init")
-    it = 0
+    def restart():
+        nonlocal it, checked
+        if it:
+            _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+            if status.n_iter != it:
+                raise RuntimeError(f"only {status.n_iter} of {it} iterations did work (state {status.state}): "
+                                   "the timed region would include no-op launches")
+            checked += it
+        cent[0].copy_(cent_init)
+        _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc,
+                                       RESTART + 8, 0.0, stream), "init")
+        it = 0
 
-    def enqueue():
-        nonlocal it
+    def enqueue(ms=None):
+        nonlocal it, done
+        if it >= RESTART:
+            restart()
         a, b = it % 2, (it + 1) % 2
-        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
-                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k,
-                                       dc, stream), "iter")
+        args = (ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]), ptr(labels[b]),
+                ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, dc, stream)
+        if ms is None:
+            _capi.check(lib.kmx_lloyd_iter(*args), "iter")
+        else:
+            _capi.check(lib.kmx_lloyd_iter_timed(*args, ms), "iter_timed")
         it += 1
+        done += 1
 
+    restart()
     for _ in range(warmup):
         enqueue()
     torch.cuda.synchronize()
@@ -85,34 +110,28 @@ def gpu_lloyd(cfg, steps, warmup):
         enqueue()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
-    if status.n_iter != warmup + steps:
-        raise RuntimeError(
-            f"only {status.n_iter} of {warmup + steps} iterations did work (state {status.state}): "
-            "the timed region would include no-op launches"
-        )
 
-    # per-kernel durations from HIP events on the launch stream
+    # per-kernel durations from HIP events on the launch stream; three untimed iterations are
+    # enqueued before every timed one, so that the clocks do not sag in the gaps the
+    # synchronising timed call leaves
     ms = (ctypes.c_float * 3)()
     acc = np.zeros(3)
-    timed = min(steps, 50)
+    timed = 25
     for _ in range(timed):
-        a, b = it % 2, (it + 1) % 2
-        _capi.check(lib.kmx_lloyd_iter_timed(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
-                                             ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d,
-                                             k, dc, stream, ms), "iter_timed")
-        it += 1
+        for _ in range(3):
+            enqueue()
+        enqueue(ms)
         acc += np.array(list(ms))
     kernel_ms = acc / timed
     _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
-    if status.n_iter != warmup + steps + timed:
-        raise RuntimeError("timed iterations did not all run")
+    if status.n_iter != it or checked + it != done:
+        raise RuntimeError(f"only {status.n_iter} of {it} iterations did work (state {status.state})")
 
     # parity gate: labels of the current state against the CPU oracle on a slice
     from oracle import kmeans as ok
     from tests._parity import assert_labels_match
 
-    cur = cent[it % 2].T.cpu().numpy()
+    cur = cent[it % 2].T.cpu().numpy()  # the centroids the last iteration produced
     lab = torch.empty(n, dtype=torch.int32, device=dev)
     aws = lib.kmx_assign_workspace_bytes(d, k, dc)
     aws_t = torch.empty(aws, dtype=torch.uint8, device=dev)
@@ -326,7 +345,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed iterations; the default also lets the GPU clocks ramp up (tens of ms)")
     ap.add_argument("--n", type=int, default=5_000_000, help="samples (default: the full configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kpp", action="store_true", help="skip the kmeans++ leg")
