@@ -274,10 +274,9 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
     if (status->state != KMX_RUNNING) return;
     const int items = (d + 1) * k;
     if (gsum != nullptr) {
-        // 64-bit fixed-point sums of the matrix-core step: one thread per item converts and
-        // clears (launched with items / 256 blocks)
-        const int item = blockIdx.x * 256 + threadIdx.x;
-        if (item < items) {
+        // 64-bit fixed-point sums of the matrix-core step: converted and cleared by a grid-stride
+        // loop of few blocks (every block ends with one atomic on the same ticket)
+        for (int item = blockIdx.x * 256 + threadIdx.x; item < items; item += gridDim.x * 256) {
             const long long iv = (long long)gsum[item];
             gsum[item] = 0ull;
             const T v = (T)ldexp((double)iv, -q_exp[item / k]);
@@ -389,6 +388,8 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
 // squared norm, squared shift); the last block sums the per-block shifts in block order and
 // runs the convergence test.
 // ------------------------------------------------------------------------------------------
+constexpr int FIN_CLUSTERS = 32;  // clusters per workgroup of the finalisation kernel
+
 template <typename T>
 __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
     const T* __restrict__ old_centroids_t, T* __restrict__ new_centroids_t,
@@ -398,25 +399,38 @@ __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
     const int state = status->state;
     if (force ? (state != KMX_NEED_RELOCATION && state != KMX_RUNNING) : (state != KMX_RUNNING))
         return;
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    double shift = 0.0;
-    if (c < k) {
-        const T sz = sizes[c];
-        if (sz != T(0)) {
-            T sq = T(0), sh = T(0);
+    // 32 clusters per workgroup; the 8 thread groups of a cluster take every 8th feature and
+    // meet in LDS (fixed order), so that wide samples do not serialise on one thread
+    const int cl = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const int c = blockIdx.x * FIN_CLUSTERS + cl;
+    __shared__ T sq_s[8][FIN_CLUSTERS], sh_s[8][FIN_CLUSTERS];
+    T sq = T(0), sh = T(0);
+    const T sz = c < k ? sizes[c] : T(0);
+    if (sz != T(0)) {
 #pragma unroll 4
-            for (int f = 0; f < d; ++f) {
-                const T nv = new_centroids_t[(size_t)f * k + c] / sz;
-                const T df = old_centroids_t[(size_t)f * k + c] - nv;
-                sh += df * df;
-                sq += nv * nv;
-                cpack[(size_t)c * dpad + f] = nv;
-                new_centroids_t[(size_t)f * k + c] = nv;
-            }
-            for (int f = d; f < dpad; ++f) cpack[(size_t)c * dpad + f] = T(0);
-            half_norms[c] = sq / T(2);
-            shift = (double)sh;
+        for (int f = grp; f < d; f += 8) {
+            const T nv = new_centroids_t[(size_t)f * k + c] / sz;
+            const T df = old_centroids_t[(size_t)f * k + c] - nv;
+            sh += df * df;
+            sq += nv * nv;
+            cpack[(size_t)c * dpad + f] = nv;
+            new_centroids_t[(size_t)f * k + c] = nv;
         }
+        for (int f = d + grp; f < dpad; f += 8) cpack[(size_t)c * dpad + f] = T(0);
+    }
+    sq_s[grp][cl] = sq;
+    sh_s[grp][cl] = sh;
+    __syncthreads();
+    double shift = 0.0;
+    if (grp == 0 && sz != T(0)) {
+        T sq_t = sq_s[0][cl], sh_t = sh_s[0][cl];
+#pragma unroll
+        for (int g2 = 1; g2 < 8; ++g2) {
+            sq_t += sq_s[g2][cl];
+            sh_t += sh_s[g2][cl];
+        }
+        half_norms[c] = sq_t / T(2);
+        shift = (double)sh_t;
     }
     __shared__ double scratch[4];
     const double block_shift = kmx_block_sum<double>(shift, scratch);
@@ -616,14 +630,15 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[1], stream);
     const int items = (d + 1) * k;
-    hipLaunchKernelGGL((lloyd_reduce_kernel<T>),
-                       dim3((unsigned)kmx_cdiv(items, gsum != nullptr ? 256 : 32)), dim3(256), 0,
+    const int64_t reduce_grid =
+        gsum != nullptr ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128) : kmx_cdiv(items, 32);
+    hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)reduce_grid), dim3(256), 0,
                        stream, partial, n_partials_used,
                        (L.acc_mode == ACC_GLOBAL && gsum == nullptr) ? 1 : 0,
                        (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k, gsum, q_exp);
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[2], stream);
-    hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, 256)), dim3(256), 0,
+    hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, FIN_CLUSTERS)), dim3(256), 0,
                        stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
                        half_norms, shift_partial, status, d, k, L.dpad, 0);
     KMX_LAUNCH_CHECK();
@@ -808,7 +823,7 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,
     char* ws = (char*)workspace;
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
     double* shift_partial = reinterpret_cast<double*>(ws + L.off_shift);
-    const unsigned grid = (unsigned)kmx_cdiv(k, 256);
+    const unsigned grid = (unsigned)kmx_cdiv(k, FIN_CLUSTERS);
     if (dtype == KMX_F32)
         hipLaunchKernelGGL((lloyd_finalize_kernel<float>), dim3(grid), dim3(256), 0, stream,
                            (const float*)centroids_t, (float*)new_centroids_t,

@@ -84,8 +84,8 @@ __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
     const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     kmx_lloyd_status* __restrict__ status, const int* __restrict__ q_exp,
-    unsigned long long* __restrict__ gsum, int* __restrict__ counts, int64_t n, int d, int k,
-    int vec_ok) {
+    unsigned long long* __restrict__ gsum, int* __restrict__ counts, int* __restrict__ ranks,
+    int64_t n, int d, int k, int vec_ok) {
     constexpr bool UPDATE = MODE != MODE_LABELS;
     if (UPDATE && status->state != KMX_RUNNING) return;
 
@@ -201,7 +201,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
         if (valid && h == 0) {
             labels[i] = lab;
             if (UPDATE) changed += (labels_prev[i] != lab) ? 1u : 0u;
-            if (MODE == MODE_COUNT) atomicAdd(counts + lab, 1);
+            // the returned count is the sample's rank inside its cluster: the scatter that
+            // follows needs no atomics of its own
+            if (MODE == MODE_COUNT) ranks[i] = atomicAdd(counts + lab, 1);
         }
         if (MODE == MODE_ATOMICS && valid) {
             const double wd = (double)sample_weight[i];
@@ -264,11 +266,12 @@ __global__ __launch_bounds__(1024) void bucket_offsets_kernel(const int* __restr
 }
 
 __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint32_t* __restrict__ labels,
-                                                             int* __restrict__ cursors,
+                                                             const int* __restrict__ offsets,
+                                                             const int* __restrict__ ranks,
                                                              int* __restrict__ order, int64_t n) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-        order[atomicAdd(cursors + labels[i], 1)] = (int)i;
+        order[offsets[labels[i]] + ranks[i]] = (int)i;
 }
 
 // One workgroup per ACC_CHUNK consecutive positions of `order` (samples sorted by cluster),
@@ -385,7 +388,7 @@ template <int MODE>
 int32_t launch_wide(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
                     const float* half_norms, const uint32_t* labels_prev, uint32_t* labels,
                     kmx_lloyd_status* status, const int* q_exp, unsigned long long* gsum,
-                    int* counts, int64_t n, int d, int k, hipStream_t stream) {
+                    int* counts, int* ranks, int64_t n, int d, int k, hipStream_t stream) {
     if (!kmx_mfma_wide_supported(d, k)) return KMX_ERR_UNSUPPORTED;
     const int n_cg = (k + CG - 1) / CG;
     const size_t lds = (size_t)n_cg * CG * sizeof(float);
@@ -398,7 +401,7 @@ int32_t launch_wide(const LloydLayout& L, const void* X_t, const void* w, const 
 #define KMX_WIDE_CASE(NKC)                                                                      \
     hipLaunchKernelGGL((lloyd_mfma_wide_kernel<NKC, MODE>), dim3((unsigned)grid), dim3(256), lds, \
                        stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,     \
-                       half_norms, labels_prev, labels, status, q_exp, gsum, counts, n, d, k, vec_ok)
+                       half_norms, labels_prev, labels, status, q_exp, gsum, counts, ranks, n, d, k, vec_ok)
     switch ((d + KC - 1) / KC) {
         case 1: KMX_WIDE_CASE(1); break;
         case 2: KMX_WIDE_CASE(2); break;
@@ -432,19 +435,20 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
     const float* half_norms = reinterpret_cast<const float*>(ws + L.off_half);
     if (X_rowmajor == nullptr || n > INT32_MAX)
         return launch_wide<MODE_ATOMICS>(L, X_t, w, centroids_t, half_norms, labels_prev, labels,
-                                         status, q_exp, gsum, nullptr, n, d, k, stream);
+                                         status, q_exp, gsum, nullptr, nullptr, n, d, k, stream);
     // labels + counts, then bucket the samples by label and sum each bucket's rows
     int* counts = reinterpret_cast<int*>(ws + L.off_bucket);
     int* offsets = counts + k;
     int* cursors = offsets + (k + 1);
     int* order = cursors + k;
+    int* ranks = order + n;
     int32_t rc = launch_wide<MODE_COUNT>(L, X_t, w, centroids_t, half_norms, labels_prev, labels,
-                                         status, q_exp, gsum, counts, n, d, k, stream);
+                                         status, q_exp, gsum, counts, ranks, n, d, k, stream);
     if (rc != KMX_OK) return rc;
     hipLaunchKernelGGL(bucket_offsets_kernel, dim3(1), dim3(1024), 0, stream, counts, offsets, cursors, k);
     int64_t sg = kmx_cdiv(n, 256 * 4);
     if (sg > 2048) sg = 2048;
-    hipLaunchKernelGGL(bucket_scatter_kernel, dim3((unsigned)sg), dim3(256), 0, stream, labels, cursors,
+    hipLaunchKernelGGL(bucket_scatter_kernel, dim3((unsigned)sg), dim3(256), 0, stream, labels, offsets, ranks,
                        order, n);
     const unsigned ag = (unsigned)kmx_cdiv(n, ACC_CHUNK);
     if (d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0))
@@ -464,5 +468,5 @@ int32_t kmx_assign_labels_mfma_wide_f32(const LloydLayout& L, const void* X_t,
                                         int64_t n, int d, int k, hipStream_t stream) {
     return launch_wide<MODE_LABELS>(L, X_t, nullptr, centroids_t,
                                     reinterpret_cast<const float*>(ws + L.off_half), nullptr, labels,
-                                    nullptr, nullptr, nullptr, nullptr, n, d, k, stream);
+                                    nullptr, nullptr, nullptr, nullptr, nullptr, n, d, k, stream);
 }
