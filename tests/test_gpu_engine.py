@@ -281,3 +281,15 @@ def test_integer_and_float16_inputs_are_converted(cuda):
     sk = SkKMeans(n_clusters=3, init=Xi[:3].astype(np.float64), n_init=1).fit(Xi)
     assert_array_equal(_np(km.labels_), sk.labels_)
     assert_allclose(_np(km.cluster_centers_), sk.cluster_centers_)
+
+
+# reference benchmark/kmeans.py:137-207: every provider runs max_iter iterations from the same
+# centroids and returns the same clustering
+def test_benchmark_cli_consistency(cuda, capsys):
+    from sklearn_numba_dpex_amd.benchmark import kmeans as bench_cli
+
+    rc = bench_cli.main(["--dataset", "config1", "--n-data-samples", "30000", "--n-clusters", "31",
+                         "--max-iter", "5", "--run-consistency-checks"])
+    assert rc == 0
+    out = capsys.readouterr().out
+    assert "KMeansEngine ... done" in out and "consistency:" in out
