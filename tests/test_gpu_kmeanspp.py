@@ -27,10 +27,14 @@ def _cases():
         "weighted_f64": (Xw, rng.uniform(0.1, 3.0, 5003), 9, 1),
         "tiny_f32": (rng.normal(size=(37, 2)).astype(np.float32), None, 4, 0),
         "wide_f32": (rng.normal(size=(3000, 150)).astype(np.float32), None, 5, 2),
+        # 2 + floor(ln 3000) = 10 local trials: the 16-trial instantiation of the kernels
+        "many_trials_f32": (rng.normal(size=(6001, 7)).astype(np.float32), None, 3000, 4),
+        # more than 4 x 256 blocks of 1024 samples: the sampler re-reads its block sums
+        "many_blocks_f64": (rng.normal(size=(1_100_003, 2)), None, 6, 5),
     }
 
 
-@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32"])
+@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32", "many_trials_f32", "many_blocks_f64"])
 def test_whole_seeding_matches_oracle(cuda, name):
     from sklearn_numba_dpex_amd.kmeans import drivers
 

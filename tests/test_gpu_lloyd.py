@@ -29,7 +29,28 @@ def _small_configs():
         "C3w": lambda: datasets.config3(n=9_000, d=300, k=70),
         "C5": lambda: datasets.config5(n=100_000),
         "odd": lambda: _odd_config(),
+        # shapes off the fast paths of the matrix-core kernels: n not a multiple of the tile or
+        # of 4 (no 128-bit accesses), odd d, k not a multiple of the centroid block
+        "F64a": lambda: _blob_config(10_007, 13, 37, np.float64, 11),
+        "F64b": lambda: _blob_config(4_100, 30, 100, np.float64, 12),
+        "F64c": lambda: _blob_config(50, 32, 16, np.float64, 13),
+        "M32a": lambda: _blob_config(10_003, 9, 45, np.float32, 14),
+        "M32b": lambda: _blob_config(5_000, 40, 20, np.float32, 15),
+        "M32c": lambda: _blob_config(33, 14, 16, np.float32, 16),
+        # wide fp32 path with very unequal clusters (bucket sizes from 0 to a third of n)
+        "C3k": lambda: _blob_config(40_000, 128, 64, np.float32, 17, skew=True),
     }
+
+
+def _blob_config(n, d, k, dtype, seed, skew=False):
+    rng = np.random.default_rng(seed)
+    centers = rng.uniform(-10, 10, (k, d))
+    p = rng.dirichlet(np.full(k, 0.15)) if skew else np.full(k, 1.0 / k)
+    y = rng.choice(k, size=n, p=p)
+    X = (centers[y] + rng.standard_normal((n, d))).astype(dtype)
+    init = X[rng.choice(n, k, replace=False)].copy()
+    w = rng.uniform(0.5, 1.5, n).astype(dtype)
+    return dict(X=X, init=init, sample_weight=w, k=k, max_iter=20, tol=0.0, name=f"blob{seed}")
 
 
 def _odd_config():
@@ -41,7 +62,8 @@ def _odd_config():
 
 
 @pytest.mark.parametrize("rowmajor", [False, True])
-@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
+                                  "M32a", "M32b", "M32c", "C3k"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -97,7 +119,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
-@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
