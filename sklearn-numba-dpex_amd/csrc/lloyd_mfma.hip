@@ -187,23 +187,27 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
         scale_w = qscale[d];
     }
 
-    // One 128-sample tile: scores on the matrix cores, argmax, labels and (UPDATE) the
-    // accumulation.  FULL (a std::bool_constant): every lane's four samples exist and 128-bit
-    // accesses are legal.  wv / p4: weights and previous labels of the lane's four samples.
-    auto process = [&](const float4(&x)[NKS], const float(&wv)[4], const uint4 p4, const int64_t i0,
-                       auto full_tag) {
+    // One tile of NC sample columns per lane: scores on the matrix cores, argmax, labels and
+    // (UPDATE) the accumulation.  NC = 4: 128 samples, the lane's samples are i0 .. i0 + 3;
+    // NC = 1: 32 samples (a quarter tile), the lane's sample is i0.  FULL: every sample of the
+    // tile exists and (NC = 4) 128-bit accesses are legal.  wv / pl: weights and previous
+    // labels of the lane's samples.
+    auto process = [&](auto nc_tag, auto full_tag, const float(&x)[NKS][decltype(nc_tag)::value],
+                       const float(&wv)[decltype(nc_tag)::value],
+                       const uint32_t(&pl)[decltype(nc_tag)::value], const int64_t i0) {
+        constexpr int NC = decltype(nc_tag)::value;
         constexpr bool FULL = decltype(full_tag)::value;
         // Running argmax per sample column, by groups of ARGMAX_GROUP accumulator registers:
         // a group costs one max chain, one compare and the conditional copies of its values
-        // (about 2 VALU instructions per score instead of 3 for a compare and two selects per
-        // score; fp32 MFMA and VALU instructions do not overlap on this hardware, so every
+        // (about 1.4 VALU instructions per score instead of 3 for a compare and two selects
+        // per score; fp32 MFMA and VALU instructions do not overlap on this hardware, so every
         // VALU instruction saved is time saved).  The position inside the winning group is
         // found once per tile.
-        float best[4];
-        int code[4];
-        double svd[4][ARGMAX_GROUP / 2];  // the winning group's registers, as pairs
+        float best[NC];
+        int code[NC];
+        double svd[NC][ARGMAX_GROUP / 2];  // the winning group's registers, as pairs
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < NC; ++t) {
             best[t] = -kmx_inf<float>();
             code[t] = 0;
 #pragma unroll
@@ -218,26 +222,23 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
             const float* ap = afrag + (size_t)cb * nks * 64 + lane;
             // the first K step reads the accumulator start (-0.5||c||^2) straight from hv
             float af = ap[0];
-            v16f a[4];
-            a[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].x, hv, 0, 0, 0);
-            a[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].y, hv, 0, 0, 0);
-            a[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].z, hv, 0, 0, 0);
-            a[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0].w, hv, 0, 0, 0);
+            v16f a[NC];
+#pragma unroll
+            for (int t = 0; t < NC; ++t) a[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[0][t], hv, 0, 0, 0);
 #pragma unroll
             for (int s = 1; s < NKS; ++s) {
                 if (s < nks) {
                     af = ap[s * 64];
-                    a[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].x, a[0], 0, 0, 0);
-                    a[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].y, a[1], 0, 0, 0);
-                    a[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].z, a[2], 0, 0, 0);
-                    a[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s].w, a[3], 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < NC; ++t)
+                        a[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(af, x[s][t], a[t], 0, 0, 0);
                 }
             }
 #pragma unroll
             for (int g = 0; g < 16 / ARGMAX_GROUP; ++g) {
                 const int cd = cb * (16 / ARGMAX_GROUP) + g;  // wave-uniform
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
+                for (int t = 0; t < NC; ++t) {
                     // three-operand max: two scores per instruction (fmaxf would also
                     // canonicalise the matrix-core results first)
                     float m = a[t][g * ARGMAX_GROUP];
@@ -267,9 +268,9 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
 
         // position inside the winning group (lowest register = lowest centroid of this lane),
         // (block, register) -> centroid index, then combine the two half-waves
-        uint32_t lab[4];
+        uint32_t lab[NC];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < NC; ++t) {
             float sv[ARGMAX_GROUP];
 #pragma unroll
             for (int r = 0; r < ARGMAX_GROUP / 2; ++r) {
@@ -290,37 +291,35 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
         }
 
         if (h == 0) {
-            if (FULL) {
+            if constexpr (FULL && NC == 4) {
                 *reinterpret_cast<uint4*>(labels + i0) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
             } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (i0 + t < n) labels[i0 + t] = lab[t];
+                for (int t = 0; t < NC; ++t)
+                    if (FULL || i0 + t < n) labels[i0 + t] = lab[t];
             }
         }
 
         if (UPDATE) {
             if (h == 0) {
-                const uint32_t pl[4] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < NC; ++t)
                     changed += ((FULL || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
             }
             // samples past the end carry w = 0 and x = 0: they add zero
-            double wd[4];
+            double wd[NC];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) wd[t] = (double)wv[t];
+            for (int t = 0; t < NC; ++t) wd[t] = (double)wv[t];
 #pragma unroll
             for (int s = 0; s < NKS; ++s) {
                 const int f = 2 * s + h;
                 if (s < nks && f < d) {
                     unsigned long long* rowacc = acc + f * k;
                     const double sc = (double)scale[s];
-                    const float xs[4] = {x[s].x, x[s].y, x[s].z, x[s].w};
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
+                    for (int t = 0; t < NC; ++t) {
                         // x * w is exact in fp64; one rounding, to a multiple of 2^-q
-                        const double v = fma((double)xs[t], wd[t] * sc, FIX_MAGIC);
+                        const double v = fma((double)x[s][t], wd[t] * sc, FIX_MAGIC);
                         atomicAdd(rowacc + lab[t], to_fixed(v));
                     }
                 }
@@ -329,11 +328,13 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
                 unsigned long long* szacc = acc + d * k;
                 const double sc = (double)scale_w;
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < NC; ++t)
                     atomicAdd(szacc + lab[t], to_fixed(fma(wd[t], sc, FIX_MAGIC)));
             }
         }
     };
+    using Cols4 = std::integral_constant<int, 4>;
+    using Cols1 = std::integral_constant<int, 1>;
 
     const int64_t wt_step = (int64_t)gridDim.x * WAVES;
     const int64_t wt_first = (int64_t)blockIdx.x * WAVES + wave;
@@ -341,6 +342,13 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
     // loads with the next tile's rows in flight during the current tile (the wave does not
     // stall on its own loads or on the completion of its label store).
     const int64_t n_fast = vec_ok ? (n >> 7) : 0;
+    // The last round of full tiles would keep only n_fast % wt_step of the waves busy for a
+    // whole tile time.  When it is at most three quarters full it is cut into quarter tiles of
+    // 32 samples instead (one MFMA chain per wave), spread over all the waves.
+    const int64_t n_rounds = n_fast / wt_step;
+    const int64_t n_left = n_fast - n_rounds * wt_step;
+    const bool quarters = n_left > 0 && 4 * n_left <= 3 * wt_step;
+    const int64_t n_main = quarters ? n_rounds * wt_step : n_fast;
     // Rows of the lane's half-wave (2s + h) at the lane's four samples.  The loads are
     // unconditional, so that the compiler can count them exactly and wait for the older tile
     // only: a row past d - 1 (odd d, upper half-wave, last K step) reads row d - 1 instead;
@@ -361,45 +369,66 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
         }
     };
     constexpr bool PREFETCH = NKS <= 16;  // the double buffer costs 4 * NKS registers
-    if (wt_first < n_fast) {
+    if (wt_first < n_main) {
         float4 xn[PREFETCH ? NKS : 1];
         if constexpr (PREFETCH) load_rows(wt_first, xn);
-        for (int64_t wt = wt_first; wt < n_fast; wt += wt_step) {
+        for (int64_t wt = wt_first; wt < n_main; wt += wt_step) {
             const int64_t i0 = wt * 128 + 4 * j;
-            float4 x[NKS];
+            float4 xv[NKS];
             if constexpr (PREFETCH) {
 #pragma unroll
-                for (int s = 0; s < NKS; ++s) x[s] = xn[s];
+                for (int s = 0; s < NKS; ++s) xv[s] = xn[s];
                 // past the last tile the same rows are read again (and not used)
-                load_rows(wt + wt_step < n_fast ? wt + wt_step : wt, xn);
+                load_rows(wt + wt_step < n_main ? wt + wt_step : wt, xn);
             } else {
-                load_rows(wt, x);
+                load_rows(wt, xv);
             }
             float wv[4] = {0.f, 0.f, 0.f, 0.f};
-            uint4 p4 = make_uint4(0u, 0u, 0u, 0u);
+            uint32_t pl[4] = {0u, 0u, 0u, 0u};
             if (UPDATE) {
                 const float4 w4 = *reinterpret_cast<const float4*>(sample_weight + i0);
                 wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
-                p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+                const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+                pl[0] = p4.x; pl[1] = p4.y; pl[2] = p4.z; pl[3] = p4.w;
             }
-            process(x, wv, p4, i0, std::true_type{});
+            float x[NKS][4];
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) {
+                x[s][0] = xv[s].x; x[s][1] = xv[s].y; x[s][2] = xv[s].z; x[s][3] = xv[s].w;
+            }
+            process(Cols4{}, std::true_type{}, x, wv, pl, i0);
+        }
+    }
+    if (quarters) {
+        // quarter q of the left-over tiles: samples [n_main * 128 + 32 q, + 32), lane j takes
+        // sample j of it (128 contiguous bytes per half-wave and row)
+        for (int64_t q = wt_first; q < 4 * n_left; q += wt_step) {
+            const int64_t i0 = n_main * 128 + 32 * q + j;
+            float x[NKS][1];
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) {
+                const int f = 2 * s + h;
+                x[s][0] = (s < nks && f < d) ? X_t[(size_t)f * n + i0] : 0.0f;
+            }
+            float wv[1] = {0.f};
+            uint32_t pl[1] = {0u};
+            if (UPDATE) {
+                wv[0] = sample_weight[i0];
+                pl[0] = labels_prev[i0];
+            }
+            process(Cols1{}, std::true_type{}, x, wv, pl, i0);
         }
     }
     // The rest: a partial last tile, or every tile when 128-bit accesses are not legal
     for (int64_t wt = n_fast + wt_first; wt < n_wtiles; wt += wt_step) {
         const int64_t i0 = wt * 128 + 4 * j;
-        float4 x[NKS];
+        float x[NKS][4];
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
-            x[s] = make_float4(0.f, 0.f, 0.f, 0.f);
             const int f = 2 * s + h;
-            if (s < nks && f < d) {
-                const float* __restrict__ row = X_t + (size_t)f * n;
-                if (i0 + 0 < n) x[s].x = row[i0 + 0];
-                if (i0 + 1 < n) x[s].y = row[i0 + 1];
-                if (i0 + 2 < n) x[s].z = row[i0 + 2];
-                if (i0 + 3 < n) x[s].w = row[i0 + 3];
-            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                x[s][t] = (s < nks && f < d && i0 + t < n) ? X_t[(size_t)f * n + i0 + t] : 0.0f;
         }
         float wv[4] = {0.f, 0.f, 0.f, 0.f};
         uint32_t pl[4] = {0u, 0u, 0u, 0u};
@@ -412,7 +441,7 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
                 }
             }
         }
-        process(x, wv, make_uint4(pl[0], pl[1], pl[2], pl[3]), i0, std::false_type{});
+        process(Cols4{}, std::false_type{}, x, wv, pl, i0);
     }
 
     if (UPDATE) {
