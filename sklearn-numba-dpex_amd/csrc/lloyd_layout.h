@@ -88,10 +88,10 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     L.off_half = L.off_cpack + kmx_align256((size_t)k * L.dpad * s);
     L.off_shift = L.off_half + kmx_align256((size_t)k * s);
     L.off_bucket = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 32) * sizeof(double));  // one per finalisation workgroup
-    // wide matrix-core path: counts (k), offsets (k + 1), cursors (k), sample order (n) and
-    // ranks inside the cluster (n) as int32
+    // wide matrix-core path: counts (k), offsets (k + 1), sample order (n) and ranks inside the
+    // cluster (n) as int32
     const size_t bucket_bytes =
-        L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)3 * k + 1 + 2 * (size_t)n) * sizeof(int) : 0;
+        L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int) : 0;
     L.off_partial = L.off_bucket + kmx_align256(bucket_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
     const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE;

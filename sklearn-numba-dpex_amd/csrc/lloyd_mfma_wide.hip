@@ -230,12 +230,12 @@ __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
 }
 
 // ---- bucketed accumulation ---------------------------------------------------------------
-// counts[c] samples carry label c.  offsets = exclusive scan of counts (one workgroup),
-// order[offsets[c] ..] = the samples of cluster c (any order: the sums below are integers).
+// counts[c] samples carry label c and ranks[i] is the position of sample i among them (the
+// value its counting atomic returned).  offsets = exclusive scan of counts (one workgroup),
+// order[offsets[c] + rank] = the samples of cluster c (any order: the sums below are integers).
 
 __global__ __launch_bounds__(1024) void bucket_offsets_kernel(const int* __restrict__ counts,
-                                                             int* __restrict__ offsets,
-                                                             int* __restrict__ cursors, int k) {
+                                                             int* __restrict__ offsets, int k) {
     __shared__ int wave_tot[16];
     __shared__ int carry_s;
     if (threadIdx.x == 0) carry_s = 0;
@@ -254,10 +254,7 @@ __global__ __launch_bounds__(1024) void bucket_offsets_kernel(const int* __restr
         __syncthreads();
         int base = carry_s;
         for (int w2 = 0; w2 < wave; ++w2) base += wave_tot[w2];
-        if (c < k) {
-            offsets[c] = base + incl - v;
-            cursors[c] = base + incl - v;
-        }
+        if (c < k) offsets[c] = base + incl - v;
         __syncthreads();
         if (threadIdx.x == 1023) carry_s = base + incl;
         __syncthreads();
@@ -439,13 +436,12 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
     // labels + counts, then bucket the samples by label and sum each bucket's rows
     int* counts = reinterpret_cast<int*>(ws + L.off_bucket);
     int* offsets = counts + k;
-    int* cursors = offsets + (k + 1);
-    int* order = cursors + k;
+    int* order = offsets + (k + 1);
     int* ranks = order + n;
     int32_t rc = launch_wide<MODE_COUNT>(L, X_t, w, centroids_t, half_norms, labels_prev, labels,
                                          status, q_exp, gsum, counts, ranks, n, d, k, stream);
     if (rc != KMX_OK) return rc;
-    hipLaunchKernelGGL(bucket_offsets_kernel, dim3(1), dim3(1024), 0, stream, counts, offsets, cursors, k);
+    hipLaunchKernelGGL(bucket_offsets_kernel, dim3(1), dim3(1024), 0, stream, counts, offsets, k);
     int64_t sg = kmx_cdiv(n, 256 * 4);
     if (sg > 2048) sg = 2048;
     hipLaunchKernelGGL(bucket_scatter_kernel, dim3((unsigned)sg), dim3(256), 0, stream, labels, offsets, ranks,
