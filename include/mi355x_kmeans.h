@@ -98,7 +98,10 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
  *                                 only by the wide fp32 path (kmx_lloyd_kernel_variant == 42),
  *                                 which then sums each cluster's rows instead of issuing one
  *                                 global atomic per (sample, feature)
- *   centroids_t      IN   (d, k)  centroids the labels are computed from
+ *   centroids_t      IN   (d, k)  centroids the labels are computed from: the array given to
+ *                                 kmx_lloyd_init for the first iteration, then the
+ *                                 new_centroids_t of the previous one (the workspace holds a
+ *                                 packed copy and the half squared norms of exactly those)
  *   new_centroids_t  OUT  (d, k)  un-normalised sums if relocation is needed, else new centroids
  *   labels_prev      IN   (n)     labels of the previous iteration
  *   labels           OUT  (n)

@@ -265,6 +265,8 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
 // Reduction of the partial copies.  Block = 32 items x 8 copy lanes.  The last block to
 // finish lists the empty clusters in ascending order and finds the heaviest cluster.
 // ------------------------------------------------------------------------------------------
+constexpr int RED_ITEMS = 16, RED_GROUPS = 16;  // 256 threads of the reduction kernel
+
 template <typename T>
 __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
     T* __restrict__ partial, int n_partials, int clear_partials, T* __restrict__ sums_t,
@@ -286,13 +288,15 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
                 sizes[item - d * k] = v;
         }
     } else {
-        const int it = threadIdx.x & 31;
-        const int cl = threadIdx.x >> 5;
-        const int item = blockIdx.x * 32 + it;
-        __shared__ T red[8][32];
+        // RED_ITEMS items per workgroup, RED_GROUPS thread groups over the partial slots
+        // (fixed order: slot g + RED_GROUPS * i in thread group g, then the groups in order)
+        const int it = threadIdx.x % RED_ITEMS;
+        const int cl = threadIdx.x / RED_ITEMS;
+        const int item = blockIdx.x * RED_ITEMS + it;
+        __shared__ T red[RED_GROUPS][RED_ITEMS];
         T s = T(0);
         if (item < items) {
-            for (int g = cl; g < n_partials; g += 8) {
+            for (int g = cl; g < n_partials; g += RED_GROUPS) {
                 T* p = partial + (size_t)g * items + item;
                 s += *p;
                 if (clear_partials) *p = T(0);
@@ -303,7 +307,7 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
         if (cl == 0 && item < items) {
             T tot = red[0][it];
 #pragma unroll
-            for (int j = 1; j < 8; ++j) tot += red[j][it];
+            for (int j = 1; j < RED_GROUPS; ++j) tot += red[j][it];
             if (item < d * k)
                 sums_t[item] = tot;
             else
@@ -631,7 +635,7 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     if (events) (void)hipEventRecord(events[1], stream);
     const int items = (d + 1) * k;
     const int64_t reduce_grid =
-        gsum != nullptr ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128) : kmx_cdiv(items, 32);
+        gsum != nullptr ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128) : kmx_cdiv(items, RED_ITEMS);
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)reduce_grid), dim3(256), 0,
                        stream, partial, n_partials_used,
                        (L.acc_mode == ACC_GLOBAL && gsum == nullptr) ? 1 : 0,

@@ -23,28 +23,43 @@
 //     written to the workgroup's slot of `partial` at the end.
 #include "lloyd_layout.h"
 
+#include <cstdlib>
+#include <type_traits>
+
 namespace {
 
 typedef double v4d __attribute__((ext_vector_type(4)));
 
-constexpr int F64_WAVES = 8;  // two waves per SIMD, one workgroup per compute unit
+// waves per workgroup (one workgroup per compute unit): two per SIMD with four sample columns
+// per lane, three with two columns (fewer registers)
+constexpr int f64_waves(int nc) { return nc == 2 ? 12 : 8; }
 
-// Four consecutive doubles of a row.
-__device__ __forceinline__ void load4d(const double* __restrict__ p, double (&v)[4]) {
-    const double2 a = *reinterpret_cast<const double2*>(p);
-    const double2 b = *reinterpret_cast<const double2*>(p + 2);
-    v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y;
+// NC (2 or 4) consecutive doubles of a row, as 128-bit loads.
+template <int NC>
+__device__ __forceinline__ void load_cols(const double* __restrict__ p, double (&v)[NC]) {
+#pragma unroll
+    for (int c = 0; c < NC; c += 2) {
+        const double2 a = *reinterpret_cast<const double2*>(p + c);
+        v[c] = a.x;
+        v[c + 1] = a.y;
+    }
 }
 
-template <int NKS, bool UPDATE>
-__global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
+// NC = sample columns per lane: a wave tile is 16 * NC samples and runs NC MFMA chains per
+// centroid block.  NC = 2 leaves registers for the next tile's rows to be in flight during the
+// current tile and for a third wave per SIMD.
+template <int NKS, int NC, bool UPDATE>
+__global__ __launch_bounds__(64 * f64_waves(NC)) void lloyd_mfma_f64_kernel(
     const double* __restrict__ X_t, const double* __restrict__ sample_weight,
     const double* __restrict__ centroids_t, const double* __restrict__ half_norms,
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     double* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k,
     int vec_ok) {
     if (UPDATE && status->state != KMX_RUNNING) return;
+    constexpr int F64_WAVES = f64_waves(NC);
     constexpr int THREADS = 64 * F64_WAVES;
+    constexpr int TILE = 16 * NC;
+    constexpr bool PREFETCH = NC == 2;
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int n_cb = (k + 15) >> 4;  // centroid blocks of 16
@@ -72,53 +87,19 @@ __global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, j = lane & 15;
-    const int64_t n_wtiles = (n + 63) >> 6;
+    const int64_t n_wtiles = (n + TILE - 1) / TILE;
     unsigned int changed = 0;
 
-    for (int64_t wt = (int64_t)blockIdx.x * F64_WAVES + wave; wt < n_wtiles;
-         wt += (int64_t)gridDim.x * F64_WAVES) {
-        const int64_t i0 = wt * 64 + 4 * j;
-        const bool fast = vec_ok && (wt + 1) * 64 <= n;  // wave-uniform
-
-        double x[NKS][4];
-        double wv[4] = {0.0, 0.0, 0.0, 0.0};
-        uint32_t pl[4] = {0u, 0u, 0u, 0u};
-        if (fast) {
+    // One tile: scores, arg-max, labels and (UPDATE) the accumulation.  FULL: every sample of
+    // the tile exists and 128-bit accesses are legal.
+    auto process = [&](auto full_tag, const double(&x)[NKS][NC], const double(&wv)[NC],
+                       const uint32_t(&pl)[NC], const int64_t i0) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        double best[NC];
+        int code[NC];
+        v4d sv[NC];  // the rows of the winning block
 #pragma unroll
-            for (int s = 0; s < NKS; ++s) {
-                const int f = 4 * s + g;
-                // a row past d - 1 reads row d - 1: its A fragment is zero, the update skips it
-                load4d(X_t + (size_t)(f < d ? f : d - 1) * n + i0, x[s]);
-            }
-            if (UPDATE) {
-                load4d(sample_weight + i0, wv);
-                const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
-                pl[0] = p4.x; pl[1] = p4.y; pl[2] = p4.z; pl[3] = p4.w;
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < NKS; ++s) {
-                const int f = 4 * s + g;
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    x[s][t] = (f < d && i0 + t < n) ? X_t[(size_t)f * n + i0 + t] : 0.0;
-            }
-            if (UPDATE) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    if (i0 + t < n) {
-                        wv[t] = sample_weight[i0 + t];
-                        pl[t] = labels_prev[i0 + t];
-                    }
-                }
-            }
-        }
-
-        double best[4];
-        int code[4];
-        v4d sv[4];  // the rows of the winning block
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < NC; ++t) {
             best[t] = -kmx_inf<double>();
             code[t] = 0;
             sv[t] = v4d{0.0, 0.0, 0.0, 0.0};
@@ -129,18 +110,18 @@ __global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
             const v4d hv = {hp[0], hp[4], hp[8], hp[12]};
             const double* ap = afrag + (size_t)cb * NKS * 64 + lane;
             double af = ap[0];
-            v4d a[4];
+            v4d a[NC];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) a[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(af, x[0][t], hv, 0, 0, 0);
+            for (int t = 0; t < NC; ++t) a[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(af, x[0][t], hv, 0, 0, 0);
 #pragma unroll
             for (int s = 1; s < NKS; ++s) {
                 af = ap[s * 64];
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < NC; ++t)
                     a[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(af, x[s][t], a[t], 0, 0, 0);
             }
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < NC; ++t) {
                 const double m = fmax(fmax(a[t][0], a[t][1]), fmax(a[t][2], a[t][3]));
                 if (m > best[t]) {  // strict: the earlier block keeps a tie
                     best[t] = m;
@@ -152,9 +133,9 @@ __global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
 
         // row inside the winning block (lowest row = lowest centroid of this lane), then the
         // four lane groups of a column are combined: highest score, lowest centroid on ties
-        uint32_t lab[4];
+        uint32_t lab[NC];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < NC; ++t) {
             int pos = 3;
 #pragma unroll
             for (int r = 2; r >= 0; --r) pos = (sv[t][r] == best[t]) ? r : pos;
@@ -173,11 +154,13 @@ __global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
         }
 
         if (g == 0) {
-            if (fast) {
+            if constexpr (FULL && NC == 4) {
                 *reinterpret_cast<uint4*>(labels + i0) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
+            } else if constexpr (FULL && NC == 2) {
+                *reinterpret_cast<uint2*>(labels + i0) = make_uint2(lab[0], lab[1]);
             } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < NC; ++t)
                     if (i0 + t < n) labels[i0 + t] = lab[t];
             }
         }
@@ -185,10 +168,10 @@ __global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
         if (UPDATE) {
             if (g == 0) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    changed += ((fast || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
+                for (int t = 0; t < NC; ++t) {
+                    changed += ((FULL || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
                     // samples past the end carry w = 0
-                    if (fast || i0 + t < n) kmx_atomic_add(acc + (size_t)d * k + lab[t], wv[t]);
+                    if (FULL || i0 + t < n) kmx_atomic_add(acc + (size_t)d * k + lab[t], wv[t]);
                 }
             }
 #pragma unroll
@@ -197,11 +180,84 @@ __global__ __launch_bounds__(64 * F64_WAVES) void lloyd_mfma_f64_kernel(
                 if (f < d) {
                     double* rowacc = acc + (size_t)f * k;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        if (fast || i0 + t < n) kmx_atomic_add(rowacc + lab[t], x[s][t] * wv[t]);
+                    for (int t = 0; t < NC; ++t)
+                        if (FULL || i0 + t < n) kmx_atomic_add(rowacc + lab[t], x[s][t] * wv[t]);
                 }
             }
         }
+    };
+
+    const int64_t wt_step = (int64_t)gridDim.x * F64_WAVES;
+    const int64_t wt_first = (int64_t)blockIdx.x * F64_WAVES + wave;
+    const int64_t n_fast = vec_ok ? n / TILE : 0;  // tiles entirely inside the array
+    // rows 4 s + g of the lane's samples; a row past d - 1 reads row d - 1 (its A fragment is
+    // zero and the update skips it), so that the loads are unconditional
+    auto load_rows = [&](const int64_t wt, double(&dst)[NKS][NC]) {
+        const double* __restrict__ p = X_t + wt * TILE + NC * j;
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+            const int f = 4 * s + g;
+            load_cols<NC>(p + (size_t)(f < d ? f : d - 1) * n, dst[s]);
+        }
+    };
+    if (wt_first < n_fast) {
+        double xn[PREFETCH ? NKS : 1][NC];
+        if constexpr (PREFETCH) load_rows(wt_first, xn);
+        for (int64_t wt = wt_first; wt < n_fast; wt += wt_step) {
+            const int64_t i0 = wt * TILE + NC * j;
+            double x[NKS][NC];
+            if constexpr (PREFETCH) {
+#pragma unroll
+                for (int s = 0; s < NKS; ++s)
+#pragma unroll
+                    for (int t = 0; t < NC; ++t) x[s][t] = xn[s][t];
+                load_rows(wt + wt_step < n_fast ? wt + wt_step : wt, xn);
+            } else {
+                load_rows(wt, x);
+            }
+            double wv[NC];
+            uint32_t pl[NC];
+#pragma unroll
+            for (int t = 0; t < NC; ++t) {
+                wv[t] = 0.0;
+                pl[t] = 0u;
+            }
+            if (UPDATE) {
+                load_cols<NC>(sample_weight + i0, wv);
+                if constexpr (NC == 4) {
+                    const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+                    pl[0] = p4.x; pl[1] = p4.y; pl[2] = p4.z; pl[3] = p4.w;
+                } else {
+                    const uint2 p2 = *reinterpret_cast<const uint2*>(labels_prev + i0);
+                    pl[0] = p2.x; pl[1] = p2.y;
+                }
+            }
+            process(std::true_type{}, x, wv, pl, i0);
+        }
+    }
+    // The rest: a partial last tile, or every tile when 128-bit accesses are not legal
+    for (int64_t wt = n_fast + wt_first; wt < n_wtiles; wt += wt_step) {
+        const int64_t i0 = wt * TILE + NC * j;
+        double x[NKS][NC];
+        double wv[NC];
+        uint32_t pl[NC];
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+            const int f = 4 * s + g;
+#pragma unroll
+            for (int t = 0; t < NC; ++t)
+                x[s][t] = (f < d && i0 + t < n) ? X_t[(size_t)f * n + i0 + t] : 0.0;
+        }
+#pragma unroll
+        for (int t = 0; t < NC; ++t) {
+            wv[t] = 0.0;
+            pl[t] = 0u;
+            if (UPDATE && i0 + t < n) {
+                wv[t] = sample_weight[i0 + t];
+                pl[t] = labels_prev[i0 + t];
+            }
+        }
+        process(std::false_type{}, x, wv, pl, i0);
     }
 
     if (UPDATE) {
@@ -226,8 +282,17 @@ bool kmx_mfma_f64_supported(int d, int k) {
     return d <= 32 && k >= 16 && mfma_f64_lds_bytes(d, k, true) <= 64 * 1024;
 }
 
+// Sample columns per lane: two (three waves per SIMD, next tile in flight) once there are
+// several tiles per wave, four for small inputs.  KMX_F64_COLS = 2 | 4 overrides this for
+// experiments.
+static int f64_cols(int64_t n) {
+    const char* v = std::getenv("KMX_F64_COLS");
+    if (v != nullptr && (v[0] == '2' || v[0] == '4') && v[1] == 0) return v[0] - '0';
+    return n >= (int64_t)1 << 19 ? 2 : 4;
+}
+
 int kmx_mfma_f64_grid(int64_t n) {
-    const int64_t tiles = kmx_cdiv(kmx_cdiv(n, 64), F64_WAVES);
+    const int64_t tiles = kmx_cdiv(kmx_cdiv(n, 16 * f64_cols(n)), f64_waves(f64_cols(n)));
     const int64_t cap = (int64_t)(kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : 1) * kmx_num_cus();
     int64_t grid = tiles < cap ? tiles : cap;
     if (grid > KMX_MAX_PARTIALS) grid = KMX_MAX_PARTIALS;
@@ -246,20 +311,21 @@ int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* cent
     // the 128-bit label accesses
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
                        (!update || (aligned16(w) && aligned16(labels_prev)));
-#define KMX_F64_CASE(NKS)                                                                        \
-    do {                                                                                         \
-        if (update)                                                                              \
-            hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, true>), dim3((unsigned)grid),          \
-                               dim3(64 * F64_WAVES), lds, stream, (const double*)X_t,             \
-                               (const double*)w, (const double*)centroids_t,                      \
-                               (const double*)half_norms, labels_prev, labels, (double*)partial,  \
-                               status, n, d, k, vec_ok);                                          \
-        else                                                                                     \
-            hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, false>), dim3((unsigned)grid),         \
-                               dim3(64 * F64_WAVES), lds, stream, (const double*)X_t,             \
-                               (const double*)w, (const double*)centroids_t,                      \
-                               (const double*)half_norms, labels_prev, labels, (double*)partial,  \
-                               status, n, d, k, vec_ok);                                          \
+    const int cols = f64_cols(n);
+#define KMX_F64_LAUNCH(NKS, NC, UPD)                                                              \
+    hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, NC, UPD>), dim3((unsigned)grid),                 \
+                       dim3(64 * f64_waves(NC)), lds, stream, (const double*)X_t, (const double*)w, \
+                       (const double*)centroids_t, (const double*)half_norms, labels_prev, labels,  \
+                       (double*)partial, status, n, d, k, vec_ok)
+#define KMX_F64_CASE(NKS)                                    \
+    do {                                                     \
+        if (cols == 2) {                                     \
+            if (update) KMX_F64_LAUNCH(NKS, 2, true);        \
+            else KMX_F64_LAUNCH(NKS, 2, false);              \
+        } else {                                             \
+            if (update) KMX_F64_LAUNCH(NKS, 4, true);        \
+            else KMX_F64_LAUNCH(NKS, 4, false);              \
+        }                                                    \
     } while (0)
     switch ((d + 3) / 4) {
         case 1: KMX_F64_CASE(1); break;
@@ -271,6 +337,7 @@ int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* cent
         case 7: KMX_F64_CASE(7); break;
         default: KMX_F64_CASE(8); break;
     }
+#undef KMX_F64_LAUNCH
 #undef KMX_F64_CASE
     KMX_LAUNCH_CHECK();
     return KMX_OK;
