@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
     T* __restrict__ partial, int n_partials, int clear_partials, T* __restrict__ sums_t,
     T* __restrict__ sizes, uint32_t* __restrict__ empty_clusters,
     kmx_lloyd_status* __restrict__ status, int d, int k,
-    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp) {
+    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, int with_tail) {
     if (status->state != KMX_RUNNING) return;
     const int items = (d + 1) * k;
     if (gsum != nullptr) {
@@ -315,7 +315,9 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
         }
     }
 
-    // ---- last block: empty-cluster list + heaviest cluster
+    // ---- last block: empty-cluster list + heaviest cluster (left to the one-workgroup
+    // finalisation kernel when that one follows)
+    if (!with_tail) return;
     __shared__ unsigned int is_last;
     __threadfence();
     __syncthreads();
@@ -636,15 +638,34 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     const int items = (d + 1) * k;
     const int64_t reduce_grid =
         gsum != nullptr ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128) : kmx_cdiv(items, RED_ITEMS);
+    // sums that fit in LDS are finished by one workgroup (no device-wide fences or tickets)
+    const bool small_tail = gsum == nullptr && (size_t)items * sizeof(T) <= 48 * 1024;
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)reduce_grid), dim3(256), 0,
                        stream, partial, n_partials_used,
                        (L.acc_mode == ACC_GLOBAL && gsum == nullptr) ? 1 : 0,
-                       (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k, gsum, q_exp);
+                       (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k, gsum, q_exp,
+                       small_tail ? 0 : 1);
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[2], stream);
-    hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, FIN_CLUSTERS)), dim3(256), 0,
-                       stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
-                       half_norms, shift_partial, status, d, k, L.dpad, 0);
+    if (small_tail) {
+        LloydTail<T> tail;
+        tail.sums_t = (T*)new_centroids_t;
+        tail.sizes = (T*)sizes;
+        tail.empty_clusters = empty_clusters;
+        tail.old_centroids_t = (const T*)centroids_t;
+        tail.cpack = cpack;
+        tail.half_norms = half_norms;
+        tail.status = status;
+        tail.d = d;
+        tail.k = k;
+        tail.dpad = L.dpad;
+        hipLaunchKernelGGL((lloyd_small_finalize_kernel<T, false>), dim3(1), dim3(256),
+                           (size_t)items * sizeof(T), stream, nullptr, nullptr, tail);
+    } else {
+        hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, FIN_CLUSTERS)), dim3(256), 0,
+                           stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
+                           half_norms, shift_partial, status, d, k, L.dpad, 0);
+    }
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[3], stream);
     return KMX_OK;

@@ -455,67 +455,6 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
     }
 }
 
-// One workgroup: fixed point -> float sums and sizes (clearing gsum for the next iteration),
-// empty-cluster list, and, if no cluster is empty, the finalisation: division by the sizes,
-// packed copy and half norms for the next iteration, centroid shift, convergence test.  The
-// sums stay in LDS between the phases; global memory is read once (fixed-point sums, old
-// centroids) and written once per output.  With an empty cluster the raw sums and sizes are
-// left in global memory for the relocation and the state becomes KMX_NEED_RELOCATION.
-__global__ __launch_bounds__(256) void lloyd_mfma_finalize_kernel(
-    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<float> a) {
-    extern __shared__ __align__(16) unsigned char fin_raw[];
-    __shared__ double scratch[4];
-    if (a.status->state != KMX_RUNNING) return;
-    const int d = a.d, k = a.k, dpad = a.dpad;
-    const int items = (d + 1) * k, dk = d * k;
-    float* vals = reinterpret_cast<float*>(fin_raw);  // [(d + 1) * k]: sums, then sizes
-    const float* sizes_s = vals + dk;
-    float* __restrict__ out_t = a.sums_t;
-    const float* __restrict__ old_t = a.old_centroids_t;
-    for (int jx = threadIdx.x; jx < items; jx += 256) {
-        const long long iv = (long long)gsum[jx];
-        gsum[jx] = 0ull;
-        const int f = jx / k;
-        const float val = (float)ldexp((double)iv, -q_exp[f]);
-        vals[jx] = val;
-        if (f < d)
-            out_t[jx] = val;
-        else
-            a.sizes[jx - dk] = val;
-    }
-    __syncthreads();
-    int heaviest = 0;
-    const int n_empty = lloyd_list_empty<float>(sizes_s, a.empty_clusters, k, &heaviest);
-    if (threadIdx.x == 0) {
-        a.status->n_empty = n_empty;
-        a.status->reserved[0] = heaviest;
-    }
-    if (n_empty > 0) {
-        if (threadIdx.x == 0) a.status->state = KMX_NEED_RELOCATION;
-        return;
-    }
-    double shift = 0.0;
-#pragma unroll 4
-    for (int jx = threadIdx.x; jx < dk; jx += 256) {
-        const int f = jx / k, c = jx - f * k;
-        const float nv = vals[jx] / sizes_s[c];
-        const float df = old_t[jx] - nv;
-        shift += (double)(df * df);
-        vals[jx] = nv;
-        out_t[jx] = nv;
-        a.cpack[(size_t)c * dpad + f] = nv;
-    }
-    __syncthreads();
-    for (int c = threadIdx.x; c < k; c += 256) {
-        float sq = 0.0f;
-        for (int f = 0; f < d; ++f) sq += vals[f * k + c] * vals[f * k + c];
-        a.half_norms[c] = sq / 2.0f;
-        for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = 0.0f;
-    }
-    const double total = kmx_block_sum<double>(shift, scratch);
-    if (threadIdx.x == 0) lloyd_update_status(a.status, total);
-}
-
 size_t mfma_lds_bytes(int d, int k, bool update) {
     const int nks = (d + 1) / 2, n_cb = (k + 31) / 32;
     size_t bytes = ((size_t)n_cb * nks * 64 + (size_t)n_cb * 32) * sizeof(float);
@@ -617,7 +556,7 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         (void)hipEventRecord(events[1], stream);
         (void)hipEventRecord(events[2], stream);
     }
-    hipLaunchKernelGGL(lloyd_mfma_finalize_kernel, dim3(1), dim3(256),
+    hipLaunchKernelGGL((lloyd_small_finalize_kernel<float, true>), dim3(1), dim3(256),
                        (size_t)(d + 1) * k * sizeof(float), stream, gsum, q_exp, tail);
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[3], stream);

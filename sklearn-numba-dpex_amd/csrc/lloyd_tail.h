@@ -151,3 +151,73 @@ __device__ inline void lloyd_finalize_block(const LloydTail<T>& a, int n_empty, 
     if (threadIdx.x == 0) lloyd_update_status(a.status, total);
 }
 
+
+// One workgroup finishes an iteration whose (d + 1) * k sums fit in LDS: empty-cluster list
+// and, if no cluster is empty, division by the sizes, packed copy and half norms for the next
+// iteration, centroid shift, convergence test.  The sums stay in LDS between the phases;
+// global memory is read once and written once per output, and no device-wide fence is needed
+// (the kernel boundary orders it after the producers).
+//   FROM_GSUM: the sums arrive as 64-bit fixed point (`gsum`, binary point q_exp[f]) and are
+//              converted, stored to sums_t / sizes and cleared here;
+//   otherwise: sums_t / sizes already hold the reduced sums.
+// With an empty cluster the raw sums and sizes stay in global memory for the relocation and
+// the state becomes KMX_NEED_RELOCATION.
+template <typename T, bool FROM_GSUM>
+__global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
+    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<T> a) {
+    extern __shared__ __align__(16) unsigned char fin_raw[];
+    __shared__ double scratch[4];
+    if (a.status->state != KMX_RUNNING) return;
+    const int d = a.d, k = a.k, dpad = a.dpad;
+    const int items = (d + 1) * k, dk = d * k;
+    T* vals = reinterpret_cast<T*>(fin_raw);  // [(d + 1) * k]: sums, then sizes
+    const T* sizes_s = vals + dk;
+    T* __restrict__ out_t = a.sums_t;
+    const T* __restrict__ old_t = a.old_centroids_t;
+    for (int jx = threadIdx.x; jx < items; jx += 256) {
+        if constexpr (FROM_GSUM) {
+            const long long iv = (long long)gsum[jx];
+            gsum[jx] = 0ull;
+            const int f = jx / k;
+            const T val = (T)ldexp((double)iv, -q_exp[f]);
+            vals[jx] = val;
+            if (f < d)
+                out_t[jx] = val;
+            else
+                a.sizes[jx - dk] = val;
+        } else {
+            vals[jx] = jx < dk ? out_t[jx] : a.sizes[jx - dk];
+        }
+    }
+    __syncthreads();
+    int heaviest = 0;
+    const int n_empty = lloyd_list_empty<T>(sizes_s, a.empty_clusters, k, &heaviest);
+    if (threadIdx.x == 0) {
+        a.status->n_empty = n_empty;
+        a.status->reserved[0] = heaviest;
+    }
+    if (n_empty > 0) {
+        if (threadIdx.x == 0) a.status->state = KMX_NEED_RELOCATION;
+        return;
+    }
+    double shift = 0.0;
+#pragma unroll 4
+    for (int jx = threadIdx.x; jx < dk; jx += 256) {
+        const int f = jx / k, c = jx - f * k;
+        const T nv = vals[jx] / sizes_s[c];
+        const T df = old_t[jx] - nv;
+        shift += (double)(df * df);
+        vals[jx] = nv;
+        out_t[jx] = nv;
+        a.cpack[(size_t)c * dpad + f] = nv;
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < k; c += 256) {
+        T sq = T(0);
+        for (int f = 0; f < d; ++f) sq += vals[f * k + c] * vals[f * k + c];
+        a.half_norms[c] = sq / T(2);
+        for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = T(0);
+    }
+    const double total = kmx_block_sum<double>(shift, scratch);
+    if (threadIdx.x == 0) lloyd_update_status(a.status, total);
+}
