@@ -229,6 +229,8 @@ class KMeansEngine(_EngineBase):
     # ------------------------------------------------------------------ validation (private)
 
     def _as_device(self, array, dtype):
+        if not isinstance(array, (torch.Tensor, np.ndarray)) and hasattr(array, "__dlpack__"):
+            array = torch.from_dlpack(array)
         if isinstance(array, torch.Tensor):
             return array.to(device=self.device, dtype=dtype)
         return torch.as_tensor(np.asarray(array), device=self.device).to(dtype)
@@ -240,6 +242,11 @@ class KMeansEngine(_EngineBase):
         estimator = self.estimator
         if sp.issparse(X):
             raise NotSupportedByEngineError("A sparse matrix was passed, but dense data is required.")
+
+        if not isinstance(X, (torch.Tensor, np.ndarray)) and hasattr(X, "__dlpack__"):
+            # any array library that speaks DLPack (the counterpart of the reference taking
+            # dpctl / dpnp arrays, engine.py:293-302): device arrays are used without a copy
+            X = torch.from_dlpack(X)
 
         if isinstance(X, torch.Tensor):
             if X.dim() != 2:
@@ -321,6 +328,8 @@ class KMeansEngine(_EngineBase):
             return torch.ones(n_samples, dtype=X.dtype, device=X.device)
         if isinstance(sample_weight, numbers.Number):
             return torch.full((n_samples,), float(sample_weight), dtype=X.dtype, device=X.device)
+        if not isinstance(sample_weight, (torch.Tensor, np.ndarray)) and hasattr(sample_weight, "__dlpack__"):
+            sample_weight = torch.from_dlpack(sample_weight)
         if isinstance(sample_weight, torch.Tensor):
             sample_weight = sample_weight.to(device=X.device, dtype=X.dtype).contiguous()
         else:

@@ -293,3 +293,41 @@ def test_benchmark_cli_consistency(cuda, capsys):
     assert rc == 0
     out = capsys.readouterr().out
     assert "KMeansEngine ... done" in out and "consistency:" in out
+
+
+class _DLPackOnly:
+    """An array that offers nothing but the DLPack protocol (stands for dpnp / cupy arrays)."""
+
+    def __init__(self, tensor):
+        self._t = tensor
+
+    def __dlpack__(self, stream=None):
+        return self._t.__dlpack__()
+
+    def __dlpack_device__(self):
+        return self._t.__dlpack_device__()
+
+
+# reference test_kmeans.py:28-37: the engine takes device arrays of another library
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_dlpack_inputs_give_the_same_fit(cuda, dtype):
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans, config_context
+
+    rng = np.random.default_rng(5)
+    X = rng.normal(size=(500, 6)).astype(dtype)
+    w = rng.uniform(0.5, 2.0, 500).astype(dtype)
+    init = X[:7].copy()
+    with config_context(engine_attributes="sklearn_types"):
+        a = KMeans(n_clusters=7, init=init, n_init=1, max_iter=20, tol=0).fit(X, sample_weight=w)
+        b = KMeans(n_clusters=7, init=init, n_init=1, max_iter=20, tol=0).fit(
+            _DLPackOnly(torch.as_tensor(X, device=cuda)), sample_weight=_DLPackOnly(torch.as_tensor(w, device=cuda)))
+    np.testing.assert_array_equal(a.labels_, b.labels_)
+    if dtype == np.float32:
+        # fixed-point sums: the fit is bit-reproducible
+        np.testing.assert_array_equal(a.cluster_centers_, b.cluster_centers_)
+    else:
+        # fp64 sums go through floating-point LDS atomics, whose order varies from run to run
+        np.testing.assert_allclose(a.cluster_centers_, b.cluster_centers_, rtol=1e-12, atol=1e-13)
+    assert a.n_iter_ == b.n_iter_
