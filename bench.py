@@ -317,6 +317,15 @@ def gpu_components(cfg):
     put("topk_idx_16", t, 4 * n * s, "radix select of the 16 largest of n values: 4 passes of 8 bits over fp32 keys")
     t = timed(lambda: sum_reduction(X_t, axis=1))
     put("sum_rows_d_by_n", t, n * d * s, "kmx_sum_rows over X_t (d, n): the feature sums of the centering")
+    from sklearn_numba_dpex_amd.common.matmul import matmul
+
+    A = torch.randn(4096, 4096, device=dev)
+    B = torch.randn(4096, 4096, device=dev)
+    t = timed(lambda: matmul(A, B))
+    put("matmul_4096", t, 3 * 4096 * 4096 * s, "kmx_matmul fp32 4096 x 4096 x 4096 on the matrix cores (contraction bound)")
+    out["matmul_4096"]["TFLOPs"] = 2.0 * 4096**3 / t / 1e12
+    out["matmul_4096"]["fp32_peak_frac"] = out["matmul_4096"]["TFLOPs"] / FP32_PEAK_TFLOPS
+    del A, B
     Xc = X_t.clone()
     t = timed(lambda: drivers.prepare_data_for_lloyd(Xc, cent_t.clone(), 1e-4, w_d, copy_x=False))
     put("prepare_data_for_lloyd", t, 4 * n * d * s,

@@ -1,11 +1,126 @@
-// out (m, q) = X (m, p) @ Y_t (q, p)^T for gfx950: LDS-tiled, 64 x 64 output tile per
-// workgroup of 256 threads, 4 x 4 register block per thread, K staged 16 at a time.  LDS
-// tiles are stored K-major with a one-element pad so that the 4-wide reads of a register
-// block do not collide on banks.  Not on the KMeans call path (the reference only calls it
-// from its own test); kept for parity of the shared-kernel surface.
+// out (m, q) = X (m, p) @ Y_t (q, p)^T for gfx950.  Not on the KMeans call path (the reference
+// only calls make_matmul_2d_kernel, common/matmul.py:13-567, from its own test); kept for
+// parity of the shared-kernel surface.
+//
+//   * fp32: matrix cores (v_mfma_f32_32x32x2_f32).  A workgroup of four waves owns a 128 x 128
+//     output tile, a wave a 64 x 64 quarter of it (2 x 2 MFMA tiles, 64 accumulator registers).
+//     Both operands have K innermost in memory; a thread reads four consecutive K values of
+//     one row with a 128-bit load and stores them K-major into LDS ([kk][row], double
+//     buffered, 16 K values per stage), so that the fragment reads of a half-wave are 32
+//     consecutive words.  The next stage's global loads are in flight during the MFMAs.
+//   * fp64 and tiny shapes: LDS-tiled vector-ALU kernel, 64 x 64 output tile per workgroup of
+//     256 threads, 4 x 4 register block per thread, K staged 16 at a time.
 #include "kmx_common.h"
 
 namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int MM = 128, MN = 128, MK = 16;  // MFMA kernel: workgroup tile and K stage
+
+// Stage loads: the 128 x 16 tile of an operand is 512 groups of four K values; thread t takes
+// groups t and t + 256: row (g / 4), K offset 4 (g % 4).
+__device__ __forceinline__ void mm_stage_load(float4 (&r)[2], const float* __restrict__ base, int rows,
+                                              int row0, int p, int k0, bool vec_ok) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        const int row = row0 + (g >> 2), kk = k0 + 4 * (g & 3);
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row < rows) {
+            const float* __restrict__ src = base + (size_t)row * p + kk;
+            if (vec_ok && kk + 4 <= p) {
+                v = *reinterpret_cast<const float4*>(src);
+            } else {
+                if (kk + 0 < p) v.x = src[0];
+                if (kk + 1 < p) v.y = src[1];
+                if (kk + 2 < p) v.z = src[2];
+                if (kk + 3 < p) v.w = src[3];
+            }
+        }
+        r[l] = v;
+    }
+}
+
+__device__ __forceinline__ void mm_stage_store(float (*tile)[MM], const float4 (&r)[2]) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        const int row = g >> 2, kk = 4 * (g & 3);
+        tile[kk + 0][row] = r[l].x;
+        tile[kk + 1][row] = r[l].y;
+        tile[kk + 2][row] = r[l].z;
+        tile[kk + 3][row] = r[l].w;
+    }
+}
+
+__global__ __launch_bounds__(256) void matmul_mfma_f32_kernel(const float* __restrict__ X,
+                                                              const float* __restrict__ Y_t,
+                                                              float* __restrict__ out, int m, int p,
+                                                              int q, int vec_ok) {
+    __shared__ float xs[2][MK][MM];
+    __shared__ float ys[2][MK][MN];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, j = lane & 31;
+    const int row0 = blockIdx.y * MM, col0 = blockIdx.x * MN;
+    const int wr = 64 * (wave >> 1), wc = 64 * (wave & 1);  // the wave's quarter of the tile
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    float4 rx[2], ry[2];
+    mm_stage_load(rx, X, m, row0, p, 0, vec_ok != 0);
+    mm_stage_load(ry, Y_t, q, col0, p, 0, vec_ok != 0);
+    mm_stage_store(xs[0], rx);
+    mm_stage_store(ys[0], ry);
+    __syncthreads();
+
+    const int n_stages = (p + MK - 1) / MK;
+    for (int st = 0; st < n_stages; ++st) {
+        const int cur = st & 1;
+        if (st + 1 < n_stages) {
+            mm_stage_load(rx, X, m, row0, p, (st + 1) * MK, vec_ok != 0);
+            mm_stage_load(ry, Y_t, q, col0, p, (st + 1) * MK, vec_ok != 0);
+        }
+#pragma unroll
+        for (int s = 0; s < MK / 2; ++s) {
+            // MFMA operands: lane (i, h) supplies K index 2 s + h of row / column i
+            float af[2], bf[2];
+#pragma unroll
+            for (int a = 0; a < 2; ++a) af[a] = xs[cur][2 * s + h][wr + 32 * a + j];
+#pragma unroll
+            for (int b = 0; b < 2; ++b) bf[b] = ys[cur][2 * s + h][wc + 32 * b + j];
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[a], bf[b], acc[a][b], 0, 0, 0);
+        }
+        if (st + 1 < n_stages) {
+            mm_stage_store(xs[cur ^ 1], rx);
+            mm_stage_store(ys[cur ^ 1], ry);
+        }
+        __syncthreads();
+    }
+
+    // accumulator register r of lane (j, h): row 8 (r / 4) + 4 h + r % 4, column j of the tile
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int gc = col0 + wc + 32 * b + j;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int gr = row0 + wr + 32 * a + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (gr < m && gc < q) out[(size_t)gr * q + gc] = acc[a][b][r];
+            }
+        }
+}
 
 constexpr int TM = 64, TN = 64, TK = 16;
 
@@ -67,12 +182,21 @@ __global__ __launch_bounds__(256) void matmul_kernel(const T* __restrict__ X,
 
 extern "C" int32_t kmx_matmul(const void* X, const void* Y_t, void* out, int32_t m, int32_t p,
                               int32_t q, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
     KMX_REQUIRE_PTR(X);
     KMX_REQUIRE_PTR(Y_t);
     KMX_REQUIRE_PTR(out);
     if (m <= 0 || p <= 0 || q <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
     hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == KMX_F32 && (int64_t)m * q >= 128 * 128) {
+        const dim3 mgrid((unsigned)kmx_cdiv(q, MN), (unsigned)kmx_cdiv(m, MM));
+        const int vec_ok = (p % 4 == 0) && ((((uintptr_t)X) & 15) == 0) && ((((uintptr_t)Y_t) & 15) == 0);
+        hipLaunchKernelGGL(matmul_mfma_f32_kernel, mgrid, dim3(256), 0, stream, (const float*)X,
+                           (const float*)Y_t, (float*)out, m, p, q, vec_ok);
+        KMX_LAUNCH_CHECK();
+        return KMX_OK;
+    }
     const dim3 grid((unsigned)kmx_cdiv(q, TN), (unsigned)kmx_cdiv(m, TM));
     if (dtype == KMX_F32)
         hipLaunchKernelGGL((matmul_kernel<float>), grid, dim3(256), 0, stream, (const float*)X,

@@ -146,7 +146,8 @@ def test_elementwise_kernels(cuda, dtype):
 
 # reference common/tests/test_matmul.py:71-127
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 2), (16, 16, 16), (65, 17, 130), (1999, 661, 563)])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 2), (16, 16, 16), (65, 17, 130), (1999, 661, 563), (128, 4, 128),
+                                   (257, 33, 129), (300, 70, 200), (1024, 256, 512)])
 def test_matmul(cuda, shape, dtype):
     from sklearn_numba_dpex_amd.common.matmul import matmul
 
