@@ -147,3 +147,21 @@ def test_kmeanspp_contract_at_full_size(cuda):
     # 256 well separated blobs: seeding must reach (nearly) all of them
     dist = drivers.get_euclidean_distances(X_t[:, :50_000].contiguous(), runs[0][0])
     assert float(dist.min(dim=1).values.max()) < 30.0
+
+
+def test_kmeanspp_first_centres_match_oracle_at_full_n(cuda):
+    """The first 12 centres on the full 1,000,000 x 64 data against the oracle's sampler fed
+    with the same uniform draws (the whole 256-centre seeding would take the oracle minutes)."""
+    import torch
+
+    from oracle import rng as orng
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    cfg = datasets.config4()
+    X, k = cfg["X"], 12
+    w = cfg["sample_weight"]
+    X_t = torch.as_tensor(X, device=cuda).T.contiguous()
+    _, idx = drivers.kmeans_plusplus(X_t, torch.as_tensor(w, device=cuda), k, np.random.RandomState(cfg["seed"]))
+    seed64 = orng.seed_from_random_state(np.random.RandomState(cfg["seed"]))
+    _, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact")
+    np.testing.assert_array_equal(idx.cpu().numpy(), ref_idx)
