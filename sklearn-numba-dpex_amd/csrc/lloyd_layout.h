@@ -75,8 +75,10 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_supported(d, k) &&
         (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA;
-    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA))
+    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA)) {
         L.variant = KMX_VARIANT_MFMA_WIDE;
+        L.acc_mode = KMX_ACC_GLOBAL;  // always the global fixed-point sums (variant code 42)
+    }
     else if (dtype == KMX_F64 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_f64_supported(d, k) &&
              (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA_F64;

@@ -338,7 +338,7 @@ __global__ __launch_bounds__(256) void bucket_accumulate_kernel(
                     for (int u = 0; u < U; ++u) {
                         const int src = u0 + 4 * u;  // wave-uniform
                         idx[u] = __builtin_amdgcn_readlane(my_idx, src & 63);
-                        wv[u] = src < 64 ? __builtin_amdgcn_readlane(my_w, src & 63) : 0.0f;
+                        wv[u] = src < 64 ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), src & 63)) : 0.0f;
                     }
 #pragma unroll
                     for (int u = 0; u < U; ++u) {

@@ -39,6 +39,10 @@ def _small_configs():
         "M32c": lambda: _blob_config(33, 14, 16, np.float32, 16),
         # wide fp32 path with very unequal clusters (bucket sizes from 0 to a third of n)
         "C3k": lambda: _blob_config(40_000, 128, 64, np.float32, 17, skew=True),
+        # few features but too many clusters for LDS accumulators: the wide path with one chunk
+        "M32d": lambda: _blob_config(20_000, 14, 600, np.float32, 18),
+        # fp64 whose accumulators do not fit LDS: vector-ALU kernel with global copies
+        "F64d": lambda: _blob_config(20_000, 32, 300, np.float64, 19),
     }
 
 
@@ -63,7 +67,7 @@ def _odd_config():
 
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
-                                  "M32a", "M32b", "M32c", "C3k"])
+                                  "M32a", "M32b", "M32c", "C3k", "M32d", "F64d"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -119,7 +123,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
-@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "F64d"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
