@@ -175,3 +175,39 @@ def test_label_helpers(cuda):
     assert drivers.is_same_clustering(_dev(a, cuda), _dev(b, cuda), 50) is True
     assert drivers.is_same_clustering(_dev(a, cuda), _dev(c, cuda), 50) is False
     assert int(drivers.get_nb_distinct_clusters(_dev(a, cuda), 50)) == len(np.unique(a))
+
+
+# every instantiation of the distance and inertia kernels (register / windowed distances,
+# centroids in LDS or not, 128-bit or scalar accesses) against numpy in fp64
+@pytest.mark.parametrize("shape", [(1003, 14, 127, np.float32), (4096, 32, 7, np.float32), (777, 33, 5, np.float32),
+                                   (1001, 16, 9, np.float64), (500, 17, 3, np.float64), (1000, 300, 50, np.float32),
+                                   (3, 2, 2, np.float64)])
+def test_distances_and_inertia_kernels(cuda, shape):
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    n, d, k, dtype = shape
+    rng = np.random.default_rng(n + d)
+    X = rng.normal(size=(n, d)).astype(dtype)
+    C = rng.normal(size=(k, d)).astype(dtype)
+    w = rng.uniform(0.5, 2.0, n).astype(dtype)
+    labels = rng.integers(0, k, n).astype(np.int32)
+    X_t, C_t = _dev(X.T, cuda), _dev(C.T, cuda)
+    rtol = 2e-5 if dtype == np.float32 else 1e-12
+    exact = np.sqrt(((X.astype(np.float64)[:, None, :] - C.astype(np.float64)[None, :, :]) ** 2).sum(axis=2))
+    got = drivers.get_euclidean_distances(X_t, C_t).cpu().numpy()
+    assert got.shape == (n, k)
+    np.testing.assert_allclose(got, exact, rtol=rtol, atol=rtol)
+    per_sample = (exact[np.arange(n), labels] ** 2)
+    lab_d = torch.as_tensor(labels, device=cuda)
+    got_w = drivers._per_sample_inertia(X_t, _dev(w, cuda), C_t, lab_d).cpu().numpy()
+    np.testing.assert_allclose(got_w, per_sample * w.astype(np.float64), rtol=rtol * 5, atol=rtol)
+    # unit weights through the NULL-weights entry (what the relocation ranks samples by)
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    out = torch.empty(n, dtype=X_t.dtype, device=cuda)
+    _capi.check(lib.kmx_per_sample_inertia(ptr(X_t), None, ptr(C_t), ptr(lab_d), ptr(out), n, d, k,
+                                           _capi.dtype_code(X.dtype), _capi.current_stream()), "inertia")
+    np.testing.assert_allclose(out.cpu().numpy(), per_sample, rtol=rtol * 5, atol=rtol)

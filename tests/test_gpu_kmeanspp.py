@@ -26,6 +26,7 @@ def _cases():
         "C4": (datasets.config4(n=40_000, d=64, k=24)["X"], None, 24, 3),
         "weighted_f64": (Xw, rng.uniform(0.1, 3.0, 5003), 9, 1),
         "tiny_f32": (rng.normal(size=(37, 2)).astype(np.float32), None, 4, 0),
+        "weighted_f32": (rng.normal(size=(4099, 9)).astype(np.float32), rng.uniform(0.1, 3.0, 4099), 17, 6),
         "wide_f32": (rng.normal(size=(3000, 150)).astype(np.float32), None, 5, 2),
         # 2 + floor(ln 3000) = 10 local trials: the 16-trial instantiation of the kernels
         "many_trials_f32": (rng.normal(size=(6001, 7)).astype(np.float32), None, 3000, 4),
@@ -34,7 +35,7 @@ def _cases():
     }
 
 
-@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32", "many_trials_f32", "many_blocks_f64"])
+@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32", "many_trials_f32", "many_blocks_f64", "weighted_f32"])
 def test_whole_seeding_matches_oracle(cuda, name):
     from sklearn_numba_dpex_amd.kmeans import drivers
 
