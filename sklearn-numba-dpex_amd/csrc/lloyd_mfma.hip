@@ -76,13 +76,22 @@ __global__ void absmax_zero_kernel(unsigned int* absmax, int count) {
 __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ X_t,
                                                           const float* __restrict__ w,
                                                           unsigned int* __restrict__ absmax,
-                                                          int64_t n, int d) {
+                                                          int64_t n, int d, int vec_ok) {
     const int row = blockIdx.y;
     const float* __restrict__ p = row < d ? X_t + (size_t)row * n : w;
     float m = 0.0f;
     const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-        m = fmaxf(m, fabsf(p[i]));
+    if (vec_ok) {
+        // rows start 16-byte aligned and n is a multiple of 4: 128-bit loads
+        const float4* __restrict__ p4 = reinterpret_cast<const float4*>(p);
+        for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < (n >> 2); g += stride) {
+            const float4 v = p4[g];
+            m = fmaxf(fmaxf(m, fabsf(v.x)), fmaxf(fabsf(v.y), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    } else {
+        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+            m = fmaxf(m, fabsf(p[i]));
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     if ((threadIdx.x & 63) == 0) atomicMax(&absmax[row], __float_as_uint(m));
@@ -517,9 +526,10 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
     int* q_exp = reinterpret_cast<int*>(absmax + (d + 1));
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(256), 0, stream, absmax, d + 1);
     int64_t gx = kmx_cdiv(n, 256 * 16);
-    if (gx > 64) gx = 64;
+    if (gx > 128) gx = 128;
+    const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0) && ((((uintptr_t)w) & 15) == 0);
     hipLaunchKernelGGL(absmax_rows_kernel, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
-                       stream, (const float*)X_t, (const float*)w, absmax, n, d);
+                       stream, (const float*)X_t, (const float*)w, absmax, n, d, vec_ok);
     hipLaunchKernelGGL(fixed_point_exponents_kernel, dim3((unsigned)kmx_cdiv(d + 1, 128)), dim3(128), 0,
                        stream, absmax, q_exp, n, d);
     const size_t words = (size_t)(d + 1) * L.k_for_gsum * 2;
