@@ -2,15 +2,16 @@
 // per iteration.
 //
 // Work decomposition
-//   * A wave owns tiles of 128 consecutive samples.  Lane (j, h) with j = lane % 32,
-//     h = lane / 32 loads, for every pair of features (2s, 2s + 1), the four samples
-//     4j .. 4j + 3 of feature row 2s + h with one 128-bit load: each half-wave reads 512
-//     contiguous bytes of X_t.  Component t of those float4 is exactly the B operand
-//     (K x N = 2 x 32) of MFMA tile t, which holds the samples {4j + t}; no shuffles.
+//   * A wave owns tiles of 32 * MC consecutive samples, MC = 2 or 4 sample columns per lane.
+//     Lane (j, h) with j = lane % 32, h = lane / 32 loads, for every pair of features
+//     (2s, 2s + 1), the samples MC j .. MC j + MC - 1 of feature row 2s + h with one 64- or
+//     128-bit load: each half-wave reads 256 or 512 contiguous bytes of X_t.  Component t of
+//     that vector is exactly the B operand (K x N = 2 x 32) of MFMA chain t, which holds the
+//     samples {MC j + t}; no shuffles.
 //   * Centroids are the A operand (M x K = 32 x 2), staged once per workgroup in LDS in
 //     fragment order (conflict-free 4-byte reads, one per MFMA), 32 centroids per block.
 //   * The accumulator of tile t starts at -0.5||c||^2, so after the K loop it holds
-//     <x, c> - 0.5||c||^2 for 16 centroids x 1 sample per lane; the argmax over centroids is
+//     <x, c> - 0.5||c||^2 for 16 centroids x 1 sample per lane and chain; the argmax over centroids is
 //     kept per lane in registers (strict '>' in increasing centroid order = lowest index
 //     wins) and the two half-waves are combined once per tile.
 //   * w * x and w are accumulated in 64-bit FIXED POINT: LDS accumulators private to the
@@ -125,13 +126,17 @@ __global__ void fixed_point_exponents_kernel(const unsigned int* __restrict__ ab
 // skipped with wave-uniform branches.
 constexpr int ARGMAX_GROUP = 8;  // accumulator registers per argmax group: 2, 4, 8 or 16
 
-// Waves per workgroup: with few K steps the kernel fits two waves per SIMD, and one
-// workgroup of eight waves per compute unit halves the accumulator flushes (the global
-// atomics of all workgroups hit the same (d + 1) * k addresses) and the staging work.
-constexpr int mfma_waves(int nks) { return nks <= 8 ? 8 : 4; }
+// Waves per workgroup: with few K steps the kernel fits two (four sample columns per lane) or
+// three (two columns) waves per SIMD, and ONE workgroup per compute unit keeps the accumulator
+// flushes (the global atomics of all workgroups hit the same (d + 1) * k addresses) and the
+// staging work at their minimum.
+#ifndef KMX_MC2_WAVES
+#define KMX_MC2_WAVES 12
+#endif
+constexpr int mfma_waves(int nks, int mc) { return nks <= 8 ? (mc == 2 ? KMX_MC2_WAVES : 8) : 4; }
 
-template <int NKS, bool EXACT, bool UPDATE>
-__global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
+template <int NKS, bool EXACT, bool UPDATE, int MC>
+__global__ __launch_bounds__(64 * mfma_waves(NKS, MC)) void lloyd_mfma_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
@@ -139,7 +144,7 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
     int vec_ok) {
     if (UPDATE && status->state != KMX_RUNNING) return;
 
-    constexpr int WAVES = mfma_waves(NKS), THREADS = 64 * WAVES;
+    constexpr int WAVES = mfma_waves(NKS, MC), THREADS = 64 * WAVES;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int nks = EXACT ? NKS : (d + 1) >> 1;  // K steps of 2 features
     const int n_cb = (k + 31) >> 5;        // centroid blocks of 32
@@ -181,7 +186,7 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, j = lane & 31;
-    const int64_t n_wtiles = (n + 127) >> 7;
+    const int64_t n_wtiles = (n + 32 * MC - 1) / (32 * MC);
     unsigned int changed = 0;
 
     // 2^q of the feature rows this lane accumulates (row 2s + h), and of the weights
@@ -302,6 +307,8 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
         if (h == 0) {
             if constexpr (FULL && NC == 4) {
                 *reinterpret_cast<uint4*>(labels + i0) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
+            } else if constexpr (FULL && NC == 2) {
+                *reinterpret_cast<uint2*>(labels + i0) = make_uint2(lab[0], lab[1]);
             } else {
 #pragma unroll
                 for (int t = 0; t < NC; ++t)
@@ -342,77 +349,94 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
             }
         }
     };
-    using Cols4 = std::integral_constant<int, 4>;
+    using ColsM = std::integral_constant<int, MC>;
     using Cols1 = std::integral_constant<int, 1>;
+    constexpr int TILE = 32 * MC;  // samples of a full wave tile
 
     const int64_t wt_step = (int64_t)gridDim.x * WAVES;
     const int64_t wt_first = (int64_t)blockIdx.x * WAVES + wave;
-    // Tiles that lie entirely inside the array, when 128-bit accesses are legal: straight-line
+    // Tiles that lie entirely inside the array, when vector accesses are legal: straight-line
     // loads with the next tile's rows in flight during the current tile (the wave does not
     // stall on its own loads or on the completion of its label store).
-    const int64_t n_fast = vec_ok ? (n >> 7) : 0;
+    const int64_t n_fast = vec_ok ? n / TILE : 0;
     // The last round of full tiles would keep only n_fast % wt_step of the waves busy for a
-    // whole tile time.  When it is at most three quarters full it is cut into quarter tiles of
-    // 32 samples instead (one MFMA chain per wave), spread over all the waves.
+    // whole tile time.  When it is at most three quarters full it is cut into single-column
+    // tiles of 32 samples instead (one MFMA chain per wave), spread over all the waves.
     const int64_t n_rounds = n_fast / wt_step;
     const int64_t n_left = n_fast - n_rounds * wt_step;
-    const bool quarters = n_left > 0 && 4 * n_left <= 3 * wt_step;
+    const bool quarters = MC > 1 && n_left > 0 && 4 * n_left <= 3 * wt_step;
     const int64_t n_main = quarters ? n_rounds * wt_step : n_fast;
-    // Rows of the lane's half-wave (2s + h) at the lane's four samples.  The loads are
+    // Rows of the lane's half-wave (2s + h) at the lane's MC samples.  The loads are
     // unconditional, so that the compiler can count them exactly and wait for the older tile
     // only: a row past d - 1 (odd d, upper half-wave, last K step) reads row d - 1 instead;
     // its A fragment is zero and the accumulation skips it.
-    const float* __restrict__ xrow_base = X_t + (size_t)h * n + 4 * j;
+    const float* __restrict__ xrow_base = X_t + (size_t)h * n + MC * j;
     const int last_row = 2 * (nks - 1) + h < d ? 2 * (nks - 1) + h : d - 1;
     const size_t last_row_off = (size_t)(last_row - h) * n;
-    auto load_rows = [&](const int64_t wt, float4* dst) {
-        const float* __restrict__ p = xrow_base + wt * 128;
+    auto load_cols = [&](const float* __restrict__ p, float(&v)[MC]) {
+        if constexpr (MC == 4) {
+            const float4 q = *reinterpret_cast<const float4*>(p);
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+            const float2 q = *reinterpret_cast<const float2*>(p);
+            v[0] = q.x; v[1] = q.y;
+        }
+    };
+    auto load_rows = [&](const int64_t wt, float(&dst)[NKS][MC]) {
+        const float* __restrict__ p = xrow_base + wt * TILE;
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
             if (EXACT || s < nks) {
                 const size_t off = (s == nks - 1) ? last_row_off : (size_t)(2 * s) * n;
-                dst[s] = *reinterpret_cast<const float4*>(p + off);
+                load_cols(p + off, dst[s]);
             } else {
-                dst[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int t = 0; t < MC; ++t) dst[s][t] = 0.0f;
             }
         }
     };
-    constexpr bool PREFETCH = NKS <= 16;  // the double buffer costs 4 * NKS registers
+    constexpr bool PREFETCH = NKS <= 16;  // the double buffer costs MC * NKS registers
     if (wt_first < n_main) {
-        float4 xn[PREFETCH ? NKS : 1];
+        float xn[PREFETCH ? NKS : 1][MC];
         if constexpr (PREFETCH) load_rows(wt_first, xn);
         for (int64_t wt = wt_first; wt < n_main; wt += wt_step) {
-            const int64_t i0 = wt * 128 + 4 * j;
-            float4 xv[NKS];
+            const int64_t i0 = wt * TILE + MC * j;
+            float x[NKS][MC];
             if constexpr (PREFETCH) {
 #pragma unroll
-                for (int s = 0; s < NKS; ++s) xv[s] = xn[s];
+                for (int s = 0; s < NKS; ++s)
+#pragma unroll
+                    for (int t = 0; t < MC; ++t) x[s][t] = xn[s][t];
                 // past the last tile the same rows are read again (and not used)
                 load_rows(wt + wt_step < n_main ? wt + wt_step : wt, xn);
             } else {
-                load_rows(wt, xv);
+                load_rows(wt, x);
             }
-            float wv[4] = {0.f, 0.f, 0.f, 0.f};
-            uint32_t pl[4] = {0u, 0u, 0u, 0u};
-            if (UPDATE) {
-                const float4 w4 = *reinterpret_cast<const float4*>(sample_weight + i0);
-                wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
-                const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
-                pl[0] = p4.x; pl[1] = p4.y; pl[2] = p4.z; pl[3] = p4.w;
-            }
-            float x[NKS][4];
+            float wv[MC];
+            uint32_t pl[MC];
 #pragma unroll
-            for (int s = 0; s < NKS; ++s) {
-                x[s][0] = xv[s].x; x[s][1] = xv[s].y; x[s][2] = xv[s].z; x[s][3] = xv[s].w;
+            for (int t = 0; t < MC; ++t) {
+                wv[t] = 0.f;
+                pl[t] = 0u;
             }
-            process(Cols4{}, std::true_type{}, x, wv, pl, i0);
+            if (UPDATE) {
+                load_cols(sample_weight + i0, wv);
+                if constexpr (MC == 4) {
+                    const uint4 p4 = *reinterpret_cast<const uint4*>(labels_prev + i0);
+                    pl[0] = p4.x; pl[1] = p4.y; pl[2] = p4.z; pl[3] = p4.w;
+                } else {
+                    const uint2 p2 = *reinterpret_cast<const uint2*>(labels_prev + i0);
+                    pl[0] = p2.x; pl[1] = p2.y;
+                }
+            }
+            process(ColsM{}, std::true_type{}, x, wv, pl, i0);
         }
     }
     if (quarters) {
-        // quarter q of the left-over tiles: samples [n_main * 128 + 32 q, + 32), lane j takes
-        // sample j of it (128 contiguous bytes per half-wave and row)
-        for (int64_t q = wt_first; q < 4 * n_left; q += wt_step) {
-            const int64_t i0 = n_main * 128 + 32 * q + j;
+        // single-column tile q of the left-over tiles: samples [n_main * TILE + 32 q, + 32),
+        // lane j takes sample j of it (128 contiguous bytes per half-wave and row)
+        for (int64_t q = wt_first; q < MC * n_left; q += wt_step) {
+            const int64_t i0 = n_main * TILE + 32 * q + j;
             float x[NKS][1];
 #pragma unroll
             for (int s = 0; s < NKS; ++s) {
@@ -428,29 +452,29 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS)) void lloyd_mfma_kernel(
             process(Cols1{}, std::true_type{}, x, wv, pl, i0);
         }
     }
-    // The rest: a partial last tile, or every tile when 128-bit accesses are not legal
+    // The rest: a partial last tile, or every tile when vector accesses are not legal
     for (int64_t wt = n_fast + wt_first; wt < n_wtiles; wt += wt_step) {
-        const int64_t i0 = wt * 128 + 4 * j;
-        float x[NKS][4];
+        const int64_t i0 = wt * TILE + MC * j;
+        float x[NKS][MC];
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
             const int f = 2 * s + h;
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < MC; ++t)
                 x[s][t] = (s < nks && f < d && i0 + t < n) ? X_t[(size_t)f * n + i0 + t] : 0.0f;
         }
-        float wv[4] = {0.f, 0.f, 0.f, 0.f};
-        uint32_t pl[4] = {0u, 0u, 0u, 0u};
-        if (UPDATE) {
+        float wv[MC];
+        uint32_t pl[MC];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                if (i0 + t < n) {
-                    wv[t] = sample_weight[i0 + t];
-                    pl[t] = labels_prev[i0 + t];
-                }
+        for (int t = 0; t < MC; ++t) {
+            wv[t] = 0.f;
+            pl[t] = 0u;
+            if (UPDATE && i0 + t < n) {
+                wv[t] = sample_weight[i0 + t];
+                pl[t] = labels_prev[i0 + t];
             }
         }
-        process(Cols4{}, std::false_type{}, x, wv, pl, i0);
+        process(ColsM{}, std::false_type{}, x, wv, pl, i0);
     }
 
     if (UPDATE) {
@@ -478,22 +502,36 @@ int32_t launch_mfma(const LloydLayout& L, const void* X_t, const void* w, const 
                     hipStream_t stream) {
     const size_t lds = mfma_lds_bytes(d, k, UPDATE);
     if (lds > 64 * 1024 || d > 64) return KMX_ERR_UNSUPPORTED;
-    const int64_t n_wtiles = kmx_cdiv(n, 128);
-    const int waves = mfma_waves((d + 1) / 2 <= 8 ? (d + 1) / 2 : (d <= 32 ? 16 : 32));
+    const int nks_t = (d + 1) / 2 <= 8 ? (d + 1) / 2 : (d <= 32 ? 16 : 32);
+    // Sample columns per lane.  Two (64 samples per wave tile, two MFMA chains) leave
+    // registers for three waves per SIMD and run about 4 % faster than four columns with two
+    // waves; KMX_MFMA_COLS = 4 restores the latter for experiments.  Shapes with more than 8 K
+    // steps keep four columns and four waves per workgroup.
+    const char* cols_env = std::getenv("KMX_MFMA_COLS");
+    const int mc = (nks_t <= 8 && !(cols_env != nullptr && cols_env[0] == '4')) ? 2 : 4;
+    const int64_t n_wtiles = kmx_cdiv(n, 32 * mc);
+    const int waves = mfma_waves(nks_t, mc);
     int64_t grid = kmx_cdiv(n_wtiles, waves);
-    // resident workgroups only: 8 waves per compute unit in either shape
-    const int per_cu = waves == 8 ? 1 : 2;
+    // resident workgroups only: one workgroup per compute unit, or two of four waves
+    const int per_cu = waves >= 8 ? 1 : 2;
     const int cap = (kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : per_cu) * kmx_num_cus();
     if (grid > cap) grid = cap;
     if (grid < 1) grid = 1;
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
                        (!UPDATE || (aligned16(w) && aligned16(labels_prev)));
-#define KMX_MFMA_CASE(NKS, EXACT)                                                              \
-    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, EXACT, UPDATE>), dim3((unsigned)grid),          \
-                       dim3(64 * mfma_waves(NKS)), lds, stream, (const float*)X_t,             \
-                       (const float*)w, (const float*)centroids_t, labels_prev, labels, status, \
+#define KMX_MFMA_LAUNCH(NKS, EXACT, MC)                                                           \
+    hipLaunchKernelGGL((lloyd_mfma_kernel<NKS, EXACT, UPDATE, MC>), dim3((unsigned)grid),          \
+                       dim3(64 * mfma_waves(NKS, MC)), lds, stream, (const float*)X_t,             \
+                       (const float*)w, (const float*)centroids_t, labels_prev, labels, status,    \
                        q_exp, gsum, n, d, k, vec_ok)
+#define KMX_MFMA_CASE(NKS, EXACT)                    \
+    do {                                             \
+        if (mc == 2 && NKS <= 8)                     \
+            KMX_MFMA_LAUNCH(NKS, EXACT, 2);          \
+        else                                         \
+            KMX_MFMA_LAUNCH(NKS, EXACT, 4);          \
+    } while (0)
     switch ((d + 1) / 2) {
         case 1: KMX_MFMA_CASE(1, true); break;
         case 2: KMX_MFMA_CASE(2, true); break;
@@ -510,6 +548,7 @@ int32_t launch_mfma(const LloydLayout& L, const void* X_t, const void* w, const 
                 KMX_MFMA_CASE(32, false);
     }
 #undef KMX_MFMA_CASE
+#undef KMX_MFMA_LAUNCH
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
