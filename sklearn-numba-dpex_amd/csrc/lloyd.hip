@@ -497,6 +497,7 @@ __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
 }
 
 // Packed (k, dpad) copy of the centroids + half squared norms; optional status reset.
+constexpr int PACK_CLUSTERS = 32;
 template <typename T>
 __global__ __launch_bounds__(256) void lloyd_pack_kernel(const T* __restrict__ centroids_t,
                                                          T* __restrict__ cpack,
@@ -504,18 +505,22 @@ __global__ __launch_bounds__(256) void lloyd_pack_kernel(const T* __restrict__ c
                                                          kmx_lloyd_status* __restrict__ status,
                                                          int d, int k, int dpad, int max_iter,
                                                          double tol) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
+    // 32 clusters x 8 feature lanes per workgroup: lane g of a cluster takes features g, g+8, ...
+    const int g = threadIdx.x & 7;
+    const int c = blockIdx.x * PACK_CLUSTERS + (threadIdx.x >> 3);
+    T sq = T(0);
     if (c < k) {
-        T sq = T(0);
-        for (int f = 0; f < d; ++f) {
-            const T v = centroids_t[(size_t)f * k + c];
+        for (int f = g; f < dpad; f += 8) {
+            const T v = f < d ? centroids_t[(size_t)f * k + c] : T(0);
             sq += v * v;
             cpack[(size_t)c * dpad + f] = v;
         }
-        for (int f = d; f < dpad; ++f) cpack[(size_t)c * dpad + f] = T(0);
-        half_norms[c] = sq / T(2);
     }
-    if (status != nullptr && c == 0) {
+    sq += __shfl_xor(sq, 1, 64);
+    sq += __shfl_xor(sq, 2, 64);
+    sq += __shfl_xor(sq, 4, 64);
+    if (c < k && g == 0) half_norms[c] = sq / T(2);
+    if (status != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         status->n_iter = 0;
         status->state = max_iter > 0 ? KMX_RUNNING : KMX_MAX_ITER;
         status->n_empty = 0;
@@ -732,7 +737,7 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
-    const unsigned grid = (unsigned)kmx_cdiv(k, 256);
+    const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32)
         hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
                            (const float*)centroids_t, (float*)(ws + L.off_cpack),
@@ -894,7 +899,7 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     if (workspace_bytes < L.off_bucket) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
-    const unsigned grid = (unsigned)kmx_cdiv(k, 256);
+    const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32) {
         hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
                            (const float*)centroids_t, (float*)(ws + L.off_cpack),

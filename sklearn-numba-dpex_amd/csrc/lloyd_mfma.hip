@@ -85,10 +85,17 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restric
     if (vec_ok) {
         // rows start 16-byte aligned and n is a multiple of 4: 128-bit loads
         const float4* __restrict__ p4 = reinterpret_cast<const float4*>(p);
-        for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < (n >> 2); g += stride) {
-            const float4 v = p4[g];
-            m = fmaxf(fmaxf(m, fabsf(v.x)), fmaxf(fabsf(v.y), fmaxf(fabsf(v.z), fabsf(v.w))));
+        auto amax4 = [](float a, const float4& v) {
+            return fmaxf(fmaxf(a, fabsf(v.x)), fmaxf(fabsf(v.y), fmaxf(fabsf(v.z), fabsf(v.w))));
+        };
+        const int64_t n4 = n >> 2;
+        int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        for (; g + 3 * stride < n4; g += 4 * stride) {  // four loads in flight per lane
+            const float4 v0 = p4[g], v1 = p4[g + stride], v2 = p4[g + 2 * stride],
+                         v3 = p4[g + 3 * stride];
+            m = amax4(amax4(amax4(amax4(m, v0), v1), v2), v3);
         }
+        for (; g < n4; g += stride) m = amax4(m, p4[g]);
     } else {
         for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
             m = fmaxf(m, fabsf(p[i]));
@@ -564,7 +571,7 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
     unsigned int* absmax = reinterpret_cast<unsigned int*>(ws + L.off_scales);
     int* q_exp = reinterpret_cast<int*>(absmax + (d + 1));
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(256), 0, stream, absmax, d + 1);
-    int64_t gx = kmx_cdiv(n, 256 * 16);
+    int64_t gx = kmx_cdiv(n, 256 * 32);
     if (gx > 128) gx = 128;
     const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0) && ((((uintptr_t)w) & 15) == 0);
     hipLaunchKernelGGL(absmax_rows_kernel, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
