@@ -134,6 +134,13 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t, const
 /* Copies the status to host memory and waits for it (the only synchronising call). */
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
 
+/* Kernel variant 61 only (fp32 labels screened on the fp16 matrix cores): number of list
+ * entries - samples, plus a few unused slots - that the last completed iteration re-evaluated
+ * in plain fp32 because the screen could not certify their label; 0 for the other variants.
+ * Synchronises the stream.  It has no counterpart in the reference (diagnostics). */
+int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int32_t k,
+                                int32_t dtype, uint32_t* count_host, void* stream);
+
 /* Which fused-step kernel kmx_lloyd_iter uses for a shape, as 10 * path + accumulation:
  * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32) with the
  * centroids resident in LDS, 4 = MFMA (fp32) with samples in registers and centroids streamed;

@@ -719,7 +719,7 @@ int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype)
     if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
     const LloydLayout L = lloyd_layout(n, d, k, dtype);
-    return L.variant * 10 + L.acc_mode;
+    return L.screen ? 61 : L.variant * 10 + L.acc_mode;
 }
 
 int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
@@ -751,9 +751,11 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
         const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, stream);
         if (rc != KMX_OK) return rc;
     }
-    if (L.variant == KMX_VARIANT_MFMA_WIDE) {
+    if (L.variant == KMX_VARIANT_MFMA_WIDE || L.screen) {
+        // cluster counts of the wide path / the counter of uncertain samples of the screened one
         hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(4), dim3(256), 0, stream,
-                           (uint32_t*)(ws + L.off_bucket), (size_t)k);
+                           (uint32_t*)(ws + L.off_bucket),
+                           L.screen ? (size_t)64 : (size_t)k);
         KMX_LAUNCH_CHECK();
     }
     if (L.acc_mode == ACC_GLOBAL && L.partial_bytes > 0) {
@@ -875,6 +877,24 @@ int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_ho
     hipStream_t stream = (hipStream_t)stream_;
     hipError_t e = hipMemcpyAsync(status_host, workspace, sizeof(kmx_lloyd_status),
                                   hipMemcpyDeviceToHost, stream);
+    if (e != hipSuccess) return (int32_t)e;
+    e = hipStreamSynchronize(stream);
+    return e == hipSuccess ? KMX_OK : (int32_t)e;
+}
+
+int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int32_t k,
+                                int32_t dtype, uint32_t* count_host, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(workspace);
+    KMX_REQUIRE_PTR(count_host);
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    *count_host = 0;
+    if (!L.screen) return KMX_OK;
+    hipStream_t stream = (hipStream_t)stream_;
+    hipError_t e = hipMemcpyAsync(count_host, (const char*)workspace + L.off_bucket + sizeof(uint32_t),
+                                  sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
     if (e != hipSuccess) return (int32_t)e;
     e = hipStreamSynchronize(stream);
     return e == hipSuccess ? KMX_OK : (int32_t)e;

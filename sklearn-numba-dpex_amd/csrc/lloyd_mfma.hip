@@ -605,12 +605,25 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
     const int* q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
     unsigned long long* gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
     if (events) (void)hipEventRecord(events[0], stream);
-    const int32_t rc = launch_mfma<true>(L, X_t, w, centroids_t, labels_prev, labels, tail.status,
-                                         q_exp, gsum, n, d, k, stream);
-    if (rc != KMX_OK) return rc;
-    if (events) {
-        (void)hipEventRecord(events[1], stream);
-        (void)hipEventRecord(events[2], stream);
+    if (L.screen) {
+        // bf16-screened labels; the samples it cannot certify are redone in fp32 by a second
+        // kernel (timed in the slot the other variants use for their reduction)
+        uint32_t* recheck = reinterpret_cast<uint32_t*>(ws + L.off_bucket);
+        tail.clear_word = recheck;
+        const int32_t rc = kmx_lloyd_step_mfma_screen(
+            X_t, w, centroids_t, tail.cpack, tail.half_norms, labels_prev, labels, tail.status,
+            reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, recheck, n, d, k,
+            L.dpad, stream, events ? events[1] : nullptr);
+        if (rc != KMX_OK) return rc;
+        if (events) (void)hipEventRecord(events[2], stream);
+    } else {
+        const int32_t rc = launch_mfma<true>(L, X_t, w, centroids_t, labels_prev, labels,
+                                             tail.status, q_exp, gsum, n, d, k, stream);
+        if (rc != KMX_OK) return rc;
+        if (events) {
+            (void)hipEventRecord(events[1], stream);
+            (void)hipEventRecord(events[2], stream);
+        }
     }
     hipLaunchKernelGGL((lloyd_small_finalize_kernel<float, true>), dim3(1), dim3(256),
                        (size_t)(d + 1) * k * sizeof(float), stream, gsum, q_exp, tail);

@@ -16,6 +16,7 @@ struct LloydTail {
     T* half_norms;
     kmx_lloyd_status* status;
     int d, k, dpad;
+    uint32_t* clear_word = nullptr;  // a counter to copy to the next word and zero, or null
 };
 
 // Empty-cluster list (ascending) and heaviest cluster; one workgroup of 256 threads.
@@ -168,6 +169,10 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
     extern __shared__ __align__(16) unsigned char fin_raw[];
     __shared__ double scratch[4];
     if (a.status->state != KMX_RUNNING) return;
+    if (a.clear_word != nullptr && threadIdx.x == 0) {
+        a.clear_word[1] = a.clear_word[0];  // kept for kmx_lloyd_recheck_count
+        a.clear_word[0] = 0u;
+    }
     const int d = a.d, k = a.k, dpad = a.dpad;
     const int items = (d + 1) * k, dk = d * k;
     T* vals = reinterpret_cast<T*>(fin_raw);  // [(d + 1) * k]: sums, then sizes

@@ -58,7 +58,9 @@ def test_workspace_queries():
 
     small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0)
     assert 0 < small < 64 << 20
-    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) == small  # independent of n
+    # the screened fp32 step lists its uncertain samples: 4 bytes per sample
+    assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) - small - 4 * 4_900_000) < 256
+    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1)
     assert lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0) > (32 << 20)  # global copies
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0) == 0
     assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7) == 0
@@ -73,7 +75,8 @@ def test_workspace_queries():
 def test_kernel_variant_selection():
     from sklearn_numba_dpex_amd._capi import lib
 
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 31   # MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 61   # bf16-screened MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0) == 31   # fp32 MFMA + LDS accumulators
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 51    # fp64: matrix cores + LDS
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1) in (12, 2)  # accumulators too big for LDS
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 42  # wide MFMA + global sums
