@@ -146,17 +146,25 @@ def gpu_lloyd(cfg, steps, warmup):
     if status.n_iter != it or checked + it != done:
         raise RuntimeError(f"only {status.n_iter} of {it} iterations did work (state {status.state})")
 
-    # parity gate: labels for the current centroids against exact fp64 distances on a slice
-    cur = cent[it % 2].T.cpu().numpy()  # the centroids the last iteration produced
+    # samples the last iteration evaluated in fp32 because its fp16 screen could not certify them
+    rechecked = ctypes.c_uint32(0)
+    _capi.check(lib.kmx_lloyd_recheck_count(ptr(ws), n, d, k, dc, ctypes.byref(rechecked), stream), "recheck_count")
+
+    # parity gate 1: the labels the last Lloyd iteration wrote, against exact fp64 distances to
+    # the centroids it started from, on a slice
+    m = min(n, 200_000)
+    prev_c = cent[(it - 1) % 2].T.cpu().numpy()
+    ties_iter = check_labels(labels[it % 2][:m].cpu().numpy(), X[:m], prev_c)
+    # parity gate 2: kmx_assign_labels for the centroids the last iteration produced
+    cur = cent[it % 2].T.cpu().numpy()
     lab = torch.empty(n, dtype=torch.int32, device=dev)
     aws = lib.kmx_assign_workspace_bytes(d, k, dc)
     aws_t = torch.empty(aws, dtype=torch.uint8, device=dev)
     _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(X_t.new_tensor(cur.T.copy())), ptr(lab), ptr(aws_t), aws,
                                       n, d, k, dc, stream), "assign")
-    m = min(n, 200_000)
-    ties = check_labels(lab[:m].cpu().numpy(), X[:m], cur)
+    ties = ties_iter + check_labels(lab[:m].cpu().numpy(), X[:m], cur)
     variant = lib.kmx_lloyd_kernel_variant(n, d, k, dc)
-    return elapsed, kernel_ms, ties, variant
+    return elapsed, kernel_ms, ties, variant, int(rechecked.value)
 
 
 def gpu_lloyd_step_time(cfg, reps, consecutive=False):
@@ -401,14 +409,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    elapsed, kernel_ms, ties, variant = gpu_lloyd(cfg, args.steps, args.warmup)
+    elapsed, kernel_ms, ties, variant, rechecked = gpu_lloyd(cfg, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     iters_per_s = args.steps / elapsed
     fused_s = kernel_ms[0] * 1e-3
     flops = lloyd_flops(n, d, k)
     nbytes = lloyd_bytes(n, d, 4)
     log(f"[bench] {ms_per_step:.4f} ms/iter; kernels (ms): fused {kernel_ms[0]:.4f} reduce "
-        f"{kernel_ms[1]:.4f} finalize {kernel_ms[2]:.4f}; near-tie label differences on slice: {ties}")
+        f"{kernel_ms[1]:.4f} finalize {kernel_ms[2]:.4f}; near-tie label differences on slices: {ties}; "
+        f"samples evaluated in fp32 by the last iteration: {rechecked} ({rechecked / n:.2e} of n)")
 
     traffic = None
     traffic_file = os.path.join(ROOT, "profiles", "lloyd_fused_step_c2_traffic.json")

@@ -134,10 +134,10 @@ int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t, const
 /* Copies the status to host memory and waits for it (the only synchronising call). */
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
 
-/* Kernel variant 61 only (fp32 labels screened on the fp16 matrix cores): number of list
- * entries - samples, plus a few unused slots - that the last completed iteration re-evaluated
- * in plain fp32 because the screen could not certify their label; 0 for the other variants.
- * Synchronises the stream.  It has no counterpart in the reference (diagnostics). */
+/* Kernel variant 61 only (fp32 labels screened on the fp16 matrix cores): number of samples
+ * whose label the screen of the last completed iteration could not certify and that were
+ * evaluated in plain fp32 instead; 0 for the other variants.  Synchronises the stream.
+ * It has no counterpart in the reference (diagnostics). */
 int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int32_t k,
                                 int32_t dtype, uint32_t* count_host, void* stream);
 

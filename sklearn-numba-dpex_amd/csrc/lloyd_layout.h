@@ -16,9 +16,6 @@ constexpr int KMX_ACC_GLOBAL = 2;
 constexpr int KMX_MAX_PARTIALS = 1024;          // upper bound on fused-step workgroups
 constexpr size_t KMX_LDS_ACC_LIMIT = 40000;     // bytes of LDS accumulators per workgroup
 constexpr size_t KMX_GLOBAL_COPIES_BYTES = 64u << 20;
-// list of uncertain samples of the screened step: entries beyond n (each workgroup may leave
-// a hole of fewer than 128 entries)
-constexpr size_t KMX_SCREEN_LIST_SLACK = 128 * 2048;
 
 // Environment overrides for experiments: KMX_LLOYD_VARIANT = stream | register | mfma,
 // KMX_LLOYD_WGS_PER_CU = 1..8.
@@ -99,10 +96,10 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     L.off_bucket = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 32) * sizeof(double));  // one per finalisation workgroup
     // wide matrix-core path: counts (k), offsets (k + 1), sample order (n) and ranks inside the
     // cluster (n) as int32
-    // screened path: the counter of uncertain samples (64 words), then up to n sample indices
+    // screened path: the counter of samples evaluated in fp32 and its copy for the host
     const size_t bucket_bytes =
         L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int)
-        : L.screen                         ? ((size_t)64 + KMX_SCREEN_LIST_SLACK + (size_t)n) * sizeof(int)
+        : L.screen                         ? (size_t)64 * sizeof(int)
                                            : 0;
     L.off_partial = L.off_bucket + kmx_align256(bucket_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
@@ -124,15 +121,14 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
 int32_t kmx_assign_labels_mfma_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
                                    uint32_t* labels, char* ws, int64_t n, int d, int k,
                                    hipStream_t stream);
-// screened fused step + recheck kernel (lloyd_mfma_screen.hip); `recheck` = counter word, then
-// 64 words on, the list; mid_event (or null) is recorded between the two kernels
+// screened fused step (lloyd_mfma_screen.hip); `uncertain_count`: one word for the number of
+// samples evaluated in fp32
 int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
-                                   const void* cpack, const void* half_norms,
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    kmx_lloyd_status* status, const unsigned int* absmax,
-                                   const int* q_exp, unsigned long long* gsum, uint32_t* recheck,
-                                   int64_t n, int d, int k, int dpad, hipStream_t stream,
-                                   hipEvent_t mid_event);
+                                   const int* q_exp, unsigned long long* gsum,
+                                   uint32_t* uncertain_count, int64_t n, int d, int k,
+                                   hipStream_t stream);
 // wide-sample variant (lloyd_mfma_wide.hip): the fused step only; the reduction and
 // finalisation kernels of lloyd.hip follow it
 int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, const void* X_rowmajor,

@@ -606,16 +606,18 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
     unsigned long long* gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
     if (events) (void)hipEventRecord(events[0], stream);
     if (L.screen) {
-        // bf16-screened labels; the samples it cannot certify are redone in fp32 by a second
-        // kernel (timed in the slot the other variants use for their reduction)
-        uint32_t* recheck = reinterpret_cast<uint32_t*>(ws + L.off_bucket);
-        tail.clear_word = recheck;
+        // labels screened on the fp16 matrix cores (lloyd_mfma_screen.hip)
+        uint32_t* uncertain = reinterpret_cast<uint32_t*>(ws + L.off_bucket);
+        tail.clear_word = uncertain;
         const int32_t rc = kmx_lloyd_step_mfma_screen(
-            X_t, w, centroids_t, tail.cpack, tail.half_norms, labels_prev, labels, tail.status,
-            reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, recheck, n, d, k,
-            L.dpad, stream, events ? events[1] : nullptr);
+            X_t, w, centroids_t, labels_prev, labels, tail.status,
+            reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain, n, d, k,
+            stream);
         if (rc != KMX_OK) return rc;
-        if (events) (void)hipEventRecord(events[2], stream);
+        if (events) {
+            (void)hipEventRecord(events[1], stream);
+            (void)hipEventRecord(events[2], stream);
+        }
     } else {
         const int32_t rc = launch_mfma<true>(L, X_t, w, centroids_t, labels_prev, labels,
                                              tail.status, q_exp, gsum, n, d, k, stream);

@@ -15,12 +15,13 @@
 //   E(x) = 6.93e-6 ||x|| C + 6.2e-6 H + 6.2e-5 sqrt(d) (||x|| + C),  C = max ||c||, H = max 0.5||c||^2
 // (scaled units).  If the best approximate score beats the second best by more than 2 E(x),
 // the arg-max of the approximate scores IS the arg-max of the exact real-valued scores: the
-// label is certain.  Otherwise (about 2 samples in 1000 on blob data) the sample is put on a
-// list and left out of the sums, and `lloyd_recheck_kernel` evaluates it in plain fp32
-// (feature-sequential fused multiply-adds, lowest index wins a tie) and adds it to the sums.
-// Labels therefore meet the same bar as an all-fp32 evaluation (they can differ from it only
-// where fp32's own rounding decides), and the sums are taken from the fp32 inputs in 64-bit
-// fixed point exactly as in lloyd_mfma.hip.  Non-finite scores make a sample uncertain.
+// label is certain.  Otherwise (about 2 samples in 1000 on blob data) the wave evaluates the
+// sample in plain fp32 on the spot: every lane takes the centroids lane, lane + 64, ... with
+// feature-sequential fused multiply-adds from -0.5||c||^2, and the wave combines the results
+// with the lowest index winning a tie.  Labels therefore meet the same bar as an all-fp32
+// evaluation (they can differ from it only where fp32's own rounding decides), and the sums
+// are taken from the fp32 inputs in 64-bit fixed point exactly as in lloyd_mfma.hip.
+// Non-finite scores make a sample uncertain.
 //
 // Work decomposition: as in lloyd_mfma.hip with two sample columns per lane.  Lane (j, h) of a
 // wave owns features 16 s + 2 i + h (i < 8) of samples 2 j, 2 j + 1 of the wave's 64-sample
@@ -51,7 +52,6 @@ __device__ __forceinline__ unsigned long long to_fixed(double scaled_plus_magic)
 constexpr float SCR_ERR_X = 6.93e-6f;
 constexpr float SCR_ERR_H = 6.2e-6f;
 constexpr float SCR_ERR_ABS = 6.2e-5f;
-constexpr int SCR_QUEUE = 1024;  // uncertain samples a workgroup buffers in LDS
 constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
 
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
@@ -61,7 +61,8 @@ constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
 
 struct ScreenLds {
-    size_t off_afh, off_afl, off_hneg, off_queue, total;
+    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, total;
+    int kp;  // centroids rounded up to a multiple of 64
 };
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
@@ -70,8 +71,10 @@ __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool updat
     s.off_afh = acc;
     s.off_afl = s.off_afh + n_cb * nk * 64 * 16;
     s.off_hneg = s.off_afl + n_cb * nk * 64 * 16;
-    s.off_queue = s.off_hneg + n_cb * 32 * 4;
-    s.total = s.off_queue + (size_t)SCR_QUEUE * 4;
+    s.kp = (k + 63) & ~63;
+    s.off_ct = s.off_hneg + n_cb * 32 * 4;             // fp32 centroids, (d, kp)
+    s.off_hx = s.off_ct + (size_t)d * s.kp * 4;        // fp32 0.5||c||^2, (kp), +inf past k
+    s.total = s.off_hx + (size_t)s.kp * 4;
     return s;
 }
 
@@ -93,8 +96,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
     const unsigned int* __restrict__ absmax, const int* __restrict__ q_exp,
-    unsigned long long* __restrict__ gsum, uint32_t* __restrict__ recheck_list,
-    uint32_t* __restrict__ recheck_count, int64_t n, int d, int k, int vec_ok) {
+    unsigned long long* __restrict__ gsum, uint32_t* __restrict__ uncertain_count, int64_t n,
+    int d, int k, int vec_ok) {
     if (UPDATE && status->state != KMX_RUNNING) return;
 
     constexpr int WAVES = scr_waves(NK), THREADS = 64 * WAVES;
@@ -108,19 +111,19 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     v8h* afh = reinterpret_cast<v8h*>(smem_raw + lay.off_afh);                  // [n_cb][NK][64]
     v8h* afl = reinterpret_cast<v8h*>(smem_raw + lay.off_afl);
     float* hneg = reinterpret_cast<float*>(smem_raw + lay.off_hneg);            // [n_cb][2][16]
-    uint32_t* queue = reinterpret_cast<uint32_t*>(smem_raw + lay.off_queue);    // [SCR_QUEUE]
+    float* ct = reinterpret_cast<float*>(smem_raw + lay.off_ct);                // [d][kp]
+    float* hx = reinterpret_cast<float*>(smem_raw + lay.off_hx);                // [kp]
+    const int kp = lay.kp;
     __shared__ unsigned int changed_block;
     __shared__ unsigned int hmax_bits;
-    __shared__ unsigned int queue_count;
-    __shared__ unsigned int queue_base;
+    __shared__ unsigned int uncertain_block;
+    __shared__ unsigned long long wave_key[WAVES];
 
     if (threadIdx.x == 0) {
         changed_block = 0;
         hmax_bits = 0;
-        queue_count = 0;
+        uncertain_block = 0;
     }
-    // a batch that does not fit the queue goes to the global list and leaves a hole here
-    for (int q = threadIdx.x; q < SCR_QUEUE; q += THREADS) queue[q] = 0xffffffffu;
     // 2^-a with max|x| * 2^-a in [2^14, 2^15) (1 for all-zero or non-finite data)
     float xmax = 0.0f;
     for (int f = 0; f < d; ++f) xmax = fmaxf(xmax, __uint_as_float(absmax[f]));
@@ -161,6 +164,23 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         }
         hneg[idx] = v;
     }
+    // unscaled fp32 copies for the samples the screen cannot certify
+    for (int idx = threadIdx.x; idx < d * kp; idx += THREADS) {
+        const int f = idx / kp, c = idx - f * kp;
+        ct[idx] = c < k ? centroids_t[(size_t)f * k + c] : 0.0f;
+    }
+    for (int c = threadIdx.x; c < kp; c += THREADS) {
+        float v = kmx_inf<float>();
+        if (c < k) {
+            float sq = 0.0f;
+            for (int f = 0; f < d; ++f) {
+                const float cv = centroids_t[(size_t)f * k + c];
+                sq += cv * cv;
+            }
+            v = sq / 2.0f;
+        }
+        hx[c] = v;
+    }
     if (UPDATE)
         for (int jx = threadIdx.x; jx < items; jx += THREADS) acc[jx] = 0ull;
     __syncthreads();
@@ -169,6 +189,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     const int h = lane >> 5, j = lane & 31;
     const int64_t n_wtiles = (n + TILE - 1) / TILE;
     unsigned int changed = 0;
+    unsigned int n_uncertain = 0;  // wave-uniform
 
     // uncertain when best - second <= thr_x * ||x|| + thr_0: twice the error bound, with a
     // margin for the rounding of the bound itself and of the hardware square root
@@ -237,14 +258,17 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         unsigned int code[NC];
         // the winning group's registers, as pairs; whatever the registers hold until the first
         // group with a score above -inf overwrites them (no instruction spent on a reset)
-        double svd[NC][G / 2];
+        // (named scalars, not an array: they are written by inline assembly at several inlined
+        // sites, and only scalars are certain to stay in registers then)
+        static_assert(G == 8 && NC <= 2, "four register pairs per column, two columns");
+        double s00, s01, s02, s03, s10, s11, s12, s13;
+        asm volatile("" : "=v"(s00), "=v"(s01), "=v"(s02), "=v"(s03));
+        asm volatile("" : "=v"(s10), "=v"(s11), "=v"(s12), "=v"(s13));
 #pragma unroll
         for (int t = 0; t < NC; ++t) {
             best[t] = neg_inf;
             second[t] = neg_inf;
             code[t] = 0;
-#pragma unroll
-            for (int r = 0; r < G / 2; ++r) asm volatile("" : "=v"(svd[t][r]));
         }
 
         // approximate scores of centroid block cb for the NC columns
@@ -296,17 +320,43 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                         best[t] = m;
                         code[t] = cd;
                         const v8d ad = __builtin_bit_cast(v8d, a[t]);
-#pragma unroll
-                        for (int r = 0; r < G / 2; ++r)
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(svd[t][r]) : "v"(ad[g * (G / 2) + r]));
+                        if (t == 0) {
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s00) : "v"(ad[g * 4]));
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s01) : "v"(ad[g * 4 + 1]));
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s02) : "v"(ad[g * 4 + 2]));
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s03) : "v"(ad[g * 4 + 3]));
+                        } else {
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s10) : "v"(ad[g * 4]));
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s11) : "v"(ad[g * 4 + 1]));
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s12) : "v"(ad[g * 4 + 2]));
+                            asm volatile("v_mov_b64 %0, %1" : "+v"(s13) : "v"(ad[g * 4 + 3]));
+                        }
                     }
                 }
             }
         };
-        for (int cb = 0; cb < n_cb; ++cb) {
-            v16f a[NC];
-            scores(cb, a);
-            argmax_block(cb, a);
+        // the scores of the next block are issued before the arg-max of the current one, so
+        // that the vector ALU does not wait for a matrix-core result
+        {
+            v16f a0[NC], a1[NC];
+            scores(0, a0);
+            int cb = 0;
+            for (; cb + 2 < n_cb; cb += 2) {  // both accumulators are rewritten unconditionally
+                scores(cb + 1, a1);
+                __builtin_amdgcn_sched_barrier(0);
+                argmax_block(cb, a0);
+                scores(cb + 2, a0);
+                __builtin_amdgcn_sched_barrier(0);
+                argmax_block(cb + 1, a1);
+            }
+            if (cb + 1 < n_cb) {
+                scores(cb + 1, a1);
+                __builtin_amdgcn_sched_barrier(0);
+                argmax_block(cb, a0);
+                argmax_block(cb + 1, a1);
+            } else {
+                argmax_block(cb, a0);
+            }
         }
 
         // position inside the winning group, second largest inside it, then both half-waves
@@ -317,7 +367,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             float sv[G];
 #pragma unroll
             for (int r = 0; r < G / 2; ++r) {
-                const float2 pr = __builtin_bit_cast(float2, svd[t][r]);
+                const double pair = t == 0 ? (r == 0 ? s00 : r == 1 ? s01 : r == 2 ? s02 : s03)
+                                           : (r == 0 ? s10 : r == 1 ? s11 : r == 2 ? s12 : s13);
+                const float2 pr = __builtin_bit_cast(float2, pair);
                 sv[2 * r] = pr.x;
                 sv[2 * r + 1] = pr.y;
             }
@@ -358,6 +410,53 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             unsure[t] = !(b - s2 > thr) && (FULL || i0 + t < n);
         }
 
+        // Samples the screen cannot certify: plain fp32, the whole wave on one sample at a
+        // time.  Lane l takes the centroids l, l + 64, ... (fused multiply-adds in feature
+        // order from -0.5||c||^2, strict '>' in increasing order), then the wave combines.
+#pragma unroll
+        for (int t = 0; t < NC; ++t) {
+            unsigned long long todo = __ballot(h == 0 && unsure[t]);  // wave-uniform
+            n_uncertain += (unsigned int)__popcll(todo);
+            while (todo) {
+                const int js = __builtin_ctzll(todo);
+                todo &= todo - 1;
+                float xf[16 * NK];
+#pragma unroll
+                for (int s = 0; s < NK; ++s)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int bits = __float_as_int(x[s][i][t]);
+                        xf[16 * s + 2 * i] = __int_as_float(__builtin_amdgcn_readlane(bits, js));
+                        xf[16 * s + 2 * i + 1] = __int_as_float(__builtin_amdgcn_readlane(bits, js + 32));
+                    }
+                float bs = neg_inf;
+                int bc = 0x7fffffff;
+                for (int c = lane; c < kp; c += 64) {
+                    float sc = -hx[c];
+#pragma unroll
+                    for (int f = 0; f < 16 * NK; ++f)
+                        if (f < d) sc = fmaf(xf[f], ct[f * kp + c], sc);  // wave-uniform guard
+                    if (sc > bs) {
+                        bs = sc;
+                        bc = c;
+                    }
+                }
+                // one 64-bit key per lane, (score in an order-preserving integer form, ~index):
+                // the largest key is the best score, the lowest index among equal scores; the
+                // wave's LDS word takes the maximum (LDS operations of a wave execute in order)
+                const unsigned int sb = __float_as_uint(bs);
+                const unsigned int ordered = sb ^ ((sb >> 31) ? 0xffffffffu : 0x80000000u);
+                const unsigned long long key = ((unsigned long long)ordered << 32) | (unsigned int)~bc;
+                if (lane == 0) wave_key[wave] = 0ull;
+                __builtin_amdgcn_wave_barrier();  // keeps the three accesses in this order
+                atomicMax(&wave_key[wave], key);
+                __builtin_amdgcn_wave_barrier();
+                bc = (int)~(unsigned int)*(volatile unsigned long long*)&wave_key[wave];
+                if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
+                if (j == js) lab[t] = (uint32_t)bc;
+            }
+        }
+
         if (h == 0) {
             if constexpr (FULL && NC == 2) {
                 *reinterpret_cast<uint2*>(labels + i0) = make_uint2(lab[0], lab[1]);
@@ -368,43 +467,16 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             }
         }
 
-        // uncertain samples go on the list (lower half-wave only: both halves hold the same flags)
-        unsigned long long um[NC];
-        int n_unsure = 0;
-#pragma unroll
-        for (int t = 0; t < NC; ++t) {
-            um[t] = __ballot(h == 0 && unsure[t]);
-            n_unsure += __popcll(um[t]);
-        }
-        if (n_unsure) {  // wave-uniform
-            // into the workgroup's queue, or straight to the global list when that is full
-            unsigned int base = 0;
-            if (lane == 0) base = atomicAdd(&queue_count, (unsigned int)n_unsure);
-            base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
-            uint32_t* dst = queue;
-            if (base + (unsigned int)n_unsure > (unsigned int)SCR_QUEUE) {
-                if (lane == 0) base = atomicAdd(recheck_count, (unsigned int)n_unsure);
-                base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
-                dst = recheck_list;
-            }
-            const unsigned long long below = (1ull << lane) - 1ull;
-#pragma unroll
-            for (int t = 0; t < NC; ++t) {
-                if (h == 0 && unsure[t]) dst[base + __popcll(um[t] & below)] = (uint32_t)(i0 + t);
-                base += __popcll(um[t]);
-            }
-        }
-
         if (UPDATE) {
             if (h == 0) {
 #pragma unroll
                 for (int t = 0; t < NC; ++t)
-                    changed += ((FULL || i0 + t < n) && !unsure[t] && pl[t] != lab[t]) ? 1u : 0u;
+                    changed += ((FULL || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
             }
-            // uncertain samples and samples past the end add zero
+            // samples past the end carry w = 0: they add zero
             double wd[NC];
 #pragma unroll
-            for (int t = 0; t < NC; ++t) wd[t] = unsure[t] ? 0.0 : (double)wv[t];
+            for (int t = 0; t < NC; ++t) wd[t] = (double)wv[t];
 #pragma unroll
             for (int s = 0; s < NK; ++s)
 #pragma unroll
@@ -455,17 +527,26 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             lane_off[s][i] = (uint32_t)(MC * j) * 4u + ((16 * s + 2 * i + 1 < d) ? (uint32_t)h * (uint32_t)n * 4u : 0u);
+    // The row addresses are rebuilt with scalar additions for every tile (the asm hides the
+    // base from loop-invariant hoisting: eight or sixteen precomputed 64-bit row pointers
+    // would not fit the scalar registers and would be spilled and reloaded around every load).
+    const size_t pair_stride = (size_t)n * 8u;  // two rows
+    const char* const tail_row = xbytes + (size_t)(d - 1) * (size_t)n * 4u;
     auto load_rows = [&](const int64_t wt, float(&dst)[NK][8][MC]) {
         const uint32_t tile_off = (uint32_t)wt * (uint32_t)(TILE * 4);
+        size_t hidden_zero = 0;
+        asm volatile("" : "+s"(hidden_zero));
+        const char* row = xbytes + hidden_zero;
 #pragma unroll
         for (int s = 0; s < NK; ++s)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int p0 = 16 * s + 2 * i;
-                const char* row = xbytes + (size_t)(p0 + 1 < d ? p0 : d - 1) * (size_t)n * 4u;
-                const float2 q = *reinterpret_cast<const float2*>(row + (tile_off + lane_off[s][i]));
+                const char* src = p0 + 1 < d ? row : tail_row;
+                const float2 q = *reinterpret_cast<const float2*>(src + (tile_off + lane_off[s][i]));
                 dst[s][i][0] = q.x;
                 dst[s][i][1] = q.y;
+                row += pair_stride;
             }
     };
 
@@ -544,12 +625,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     }
 
     if (UPDATE && changed) atomicAdd(&changed_block, changed);
+    if (lane == 0 && n_uncertain) atomicAdd(&uncertain_block, n_uncertain);
     __syncthreads();
-    // the queue (holes included: the recheck skips them) moves to the global list
-    const unsigned int q_n = queue_count < (unsigned int)SCR_QUEUE ? queue_count : (unsigned int)SCR_QUEUE;
-    if (threadIdx.x == 0 && q_n) queue_base = atomicAdd(recheck_count, q_n);
-    __syncthreads();
-    for (unsigned int q = threadIdx.x; q < q_n; q += THREADS) recheck_list[queue_base + q] = queue[q];
+    if (threadIdx.x == 0 && uncertain_block) atomicAdd(uncertain_count, uncertain_block);
     if (UPDATE) {
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
         for (int jx = threadIdx.x; jx < items; jx += THREADS) {
@@ -559,146 +637,28 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     }
 }
 
-// ---------------------------------------------------------------------------- recheck
-
-constexpr int RECHECK_THREADS = 256;
-constexpr int RECHECK_PARTS = 4;  // lanes per sample, each takes every fourth centroid
-constexpr int RECHECK_CHUNK = RECHECK_THREADS / RECHECK_PARTS;  // samples per block and pass
-constexpr int RECHECK_BLOCKS = 1024;
-
-__host__ __device__ inline size_t recheck_lds_bytes(int d, int k, int dpad, bool update) {
-    size_t b = update ? (((size_t)(d + 1) * k * 8 + 15) & ~(size_t)15) : 0;
-    b += (size_t)k * dpad * 4 + (size_t)k * 4 + (size_t)(d + 1) * 4;
-    return b;
-}
-
-// The listed samples in plain fp32: score = -0.5||c||^2 + sum_f x_f c_f by fused multiply-adds
-// in feature order, strict '>' in increasing centroid order.  Four neighbouring lanes share a
-// sample (centroids p, p + 4, ... each, combined with the lowest index winning a tie); block b
-// takes the chunks b, b + gridDim.x, ... of the list, and blocks without a chunk leave at once.
-// Entries 0xffffffff are holes.
-template <int NK, bool UPDATE>
-__global__ __launch_bounds__(RECHECK_THREADS) void lloyd_recheck_kernel(
-    const float* __restrict__ X_t, const float* __restrict__ sample_weight,
-    const float* __restrict__ cpack, const float* __restrict__ half_norms,
-    const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
-    const uint32_t* __restrict__ recheck_list, const uint32_t* __restrict__ recheck_count,
-    kmx_lloyd_status* __restrict__ status, const int* __restrict__ q_exp,
-    unsigned long long* __restrict__ gsum, int64_t n, int d, int k, int dpad) {
-    if (UPDATE && status->state != KMX_RUNNING) return;
-    const uint32_t cnt = *recheck_count;
-    if ((uint64_t)blockIdx.x * RECHECK_CHUNK >= cnt) return;
-
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    const int items = (d + 1) * k;
-    unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);
-    float* cp = reinterpret_cast<float*>(smem_raw + (UPDATE ? (((size_t)items * 8 + 15) & ~(size_t)15) : 0));
-    float* hn = cp + (size_t)k * dpad;
-    float* qscale = hn + k;
-    __shared__ unsigned int changed_block;
-    for (int idx = threadIdx.x; idx < k * dpad; idx += RECHECK_THREADS) cp[idx] = cpack[idx];
-    for (int c = threadIdx.x; c < k; c += RECHECK_THREADS) hn[c] = half_norms[c];
-    if (UPDATE) {
-        for (int jx = threadIdx.x; jx < items; jx += RECHECK_THREADS) acc[jx] = 0ull;
-        for (int f = threadIdx.x; f <= d; f += RECHECK_THREADS) qscale[f] = ldexpf(1.0f, q_exp[f]);
-        if (threadIdx.x == 0) changed_block = 0;
-    }
-    __syncthreads();
-
-    const int part = threadIdx.x & (RECHECK_PARTS - 1), slot = threadIdx.x / RECHECK_PARTS;
-    unsigned int changed = 0;
-    for (uint64_t base = (uint64_t)blockIdx.x * RECHECK_CHUNK; base < cnt;
-         base += (uint64_t)gridDim.x * RECHECK_CHUNK) {
-        const uint64_t e = base + slot;
-        const uint32_t entry = e < cnt ? recheck_list[e] : 0xffffffffu;
-        const bool active = entry != 0xffffffffu;
-        const int64_t i = active ? (int64_t)entry : 0;
-        float x[16 * NK];
-#pragma unroll
-        for (int f = 0; f < 16 * NK; ++f) x[f] = f < d ? X_t[(size_t)f * n + i] : 0.0f;
-        float best = -kmx_inf<float>();
-        int bl = 0x7fffffff;
-        for (int c = part; c < k; c += RECHECK_PARTS) {
-            const float4* __restrict__ row = reinterpret_cast<const float4*>(cp + (size_t)c * dpad);
-            float s = -hn[c];
-#pragma unroll
-            for (int f4 = 0; f4 < 4 * NK; ++f4)
-                if (4 * f4 < dpad) {  // wave-uniform; the padding of the packed rows is zero
-                    const float4 q = row[f4];
-                    s = fmaf(x[4 * f4], q.x, s);
-                    s = fmaf(x[4 * f4 + 1], q.y, s);
-                    s = fmaf(x[4 * f4 + 2], q.z, s);
-                    s = fmaf(x[4 * f4 + 3], q.w, s);
-                }
-            if (s > best) {
-                best = s;
-                bl = c;
-            }
-        }
-#pragma unroll
-        for (int off = 1; off < RECHECK_PARTS; off <<= 1) {
-            const float ov = __shfl_xor(best, off, 64);
-            const int oc = __shfl_xor(bl, off, 64);
-            if (ov > best || (ov == best && oc < bl)) {
-                best = ov;
-                bl = oc;
-            }
-        }
-        if (bl == 0x7fffffff) bl = 0;  // every score NaN: the reference's running arg-min keeps 0
-        if (active) {
-            if (part == 0) {
-                labels[i] = (uint32_t)bl;
-                if (UPDATE) changed += labels_prev[i] != (uint32_t)bl ? 1u : 0u;
-            }
-            if (UPDATE) {
-                const double wd = (double)sample_weight[i];
-#pragma unroll
-                for (int f = 0; f < 16 * NK; ++f)
-                    if (f < d && (f & (RECHECK_PARTS - 1)) == part) {
-                        const double v = fma((double)x[f], wd * (double)qscale[f], FIX_MAGIC);
-                        atomicAdd(acc + f * k + bl, to_fixed(v));
-                    }
-                if (part == RECHECK_PARTS - 1)
-                    atomicAdd(acc + d * k + bl, to_fixed(fma(wd, (double)qscale[d], FIX_MAGIC)));
-            }
-        }
-    }
-    if (UPDATE) {
-        if (changed) atomicAdd(&changed_block, changed);
-        __syncthreads();
-        if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
-        for (int jx = threadIdx.x; jx < items; jx += RECHECK_THREADS) {
-            const unsigned long long v = acc[jx];
-            if (v) atomicAdd(gsum + jx, v);
-        }
-    }
-}
-
 }  // namespace
 
-// Shapes the screened step covers: d <= 32, the operands of both kernels within 64 KB of LDS,
-// byte offsets inside two rows of X_t within 32 bits.  KMX_LLOYD_ASSIGN = f32 switches it off (all-fp32 scores).
+// Shapes the screened step covers: d <= 32, everything within 64 KB of LDS, byte offsets
+// inside two rows of X_t within 32 bits.  KMX_LLOYD_ASSIGN = f32 switches it off (all-fp32
+// scores on the matrix cores, lloyd_mfma.hip).
 bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
     if (d < 1 || d > 32 || k < 16 || n >= ((int64_t)1 << 29)) return false;
     const char* v = std::getenv("KMX_LLOYD_ASSIGN");
     if (v != nullptr && std::strcmp(v, "f32") == 0) return false;
-    const int nk = (d + 15) / 16, dpad = (d + 3) & ~3;
-    return screen_lds(d, k, nk, true).total <= 64 * 1024 &&
-           recheck_lds_bytes(d, k, dpad, true) <= 64 * 1024;
+    return screen_lds(d, k, (d + 15) / 16, true).total <= 64 * 1024;
 }
 
-// Screened fused step + recheck of the uncertain samples.  `recheck` points at the counter
-// (one word, zero on entry; the finalisation that follows clears it again) followed, 64 words
-// later, by room for n + KMX_SCREEN_LIST_SLACK entries (sample indices and the holes of the
-// workgroup queues).  `absmax`: bits of max|X_t row| per feature, as kmx_lloyd_mfma_prepare
-// leaves them.
+// Screened fused step.  `uncertain_count`: one word the kernel adds the number of samples it
+// evaluated in fp32 to (zero on entry; the finalisation that follows moves it to the next word
+// and clears it).  `absmax`: bits of max|X_t row| per feature, as kmx_lloyd_mfma_prepare leaves
+// them.
 int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
-                                   const void* cpack, const void* half_norms,
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    kmx_lloyd_status* status, const unsigned int* absmax,
-                                   const int* q_exp, unsigned long long* gsum, uint32_t* recheck,
-                                   int64_t n, int d, int k, int dpad, hipStream_t stream,
-                                   hipEvent_t mid_event) {
+                                   const int* q_exp, unsigned long long* gsum,
+                                   uint32_t* uncertain_count, int64_t n, int d, int k,
+                                   hipStream_t stream) {
     if (!kmx_mfma_screen_supported(n, d, k)) return KMX_ERR_UNSUPPORTED;
     const int nk = (d + 15) / 16;
     const int waves = scr_waves(nk);
@@ -712,29 +672,16 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) && aligned16(w) &&
                        aligned16(labels_prev);
     const size_t lds = screen_lds(d, k, nk, true).total;
-    uint32_t* count = recheck;
-    uint32_t* list = recheck + 64;
     if (nk == 1)
         hipLaunchKernelGGL((lloyd_screen_kernel<1, true>), dim3((unsigned)grid), dim3(64 * scr_waves(1)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
-                           labels_prev, labels, status, absmax, q_exp, gsum, list, count, n, d, k, vec_ok);
+                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, n, d, k,
+                           vec_ok);
     else
         hipLaunchKernelGGL((lloyd_screen_kernel<2, true>), dim3((unsigned)grid), dim3(64 * scr_waves(2)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
-                           labels_prev, labels, status, absmax, q_exp, gsum, list, count, n, d, k, vec_ok);
-    KMX_LAUNCH_CHECK();
-    if (mid_event) (void)hipEventRecord(mid_event, stream);
-    const size_t lds2 = recheck_lds_bytes(d, k, dpad, true);
-    if (nk == 1)
-        hipLaunchKernelGGL((lloyd_recheck_kernel<1, true>), dim3(RECHECK_BLOCKS), dim3(RECHECK_THREADS),
-                           lds2, stream, (const float*)X_t, (const float*)w, (const float*)cpack,
-                           (const float*)half_norms, labels_prev, labels, list, count, status, q_exp,
-                           gsum, n, d, k, dpad);
-    else
-        hipLaunchKernelGGL((lloyd_recheck_kernel<2, true>), dim3(RECHECK_BLOCKS), dim3(RECHECK_THREADS),
-                           lds2, stream, (const float*)X_t, (const float*)w, (const float*)cpack,
-                           (const float*)half_norms, labels_prev, labels, list, count, status, q_exp,
-                           gsum, n, d, k, dpad);
+                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, n, d, k,
+                           vec_ok);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
