@@ -375,20 +375,20 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             }
             // registers equal to the best: the lowest is the label's; a second one makes the
             // second best equal to the best
-            unsigned int pos = G - 1, pos_hi = 0;
+            unsigned int pos = G - 1, n_eq = 0;
             float rest[G];
 #pragma unroll
             for (int r = G - 1; r >= 0; --r) {
                 const bool eq = sv[r] == best[t];
                 pos = eq ? (unsigned int)r : pos;
-                pos_hi = eq ? (unsigned int)(G - 1 - r) : pos_hi;  // ends as the highest match, mirrored
+                n_eq += eq ? 1u : 0u;
                 rest[r] = eq ? neg_inf : sv[r];
             }
             float sec = second[t];
 #pragma unroll
             for (int r = 0; r + 1 < G; r += 2)
                 asm("v_max3_f32 %0, %1, %2, %3" : "=v"(sec) : "v"(sec), "v"(rest[r]), "v"(rest[r + 1]));
-            sec = (pos + pos_hi != (unsigned int)(G - 1)) ? best[t] : sec;
+            sec = n_eq > 1u ? best[t] : sec;
             const unsigned int reg = (code[t] % NG) * G + pos;
             const unsigned int blk = code[t] / NG;
             int c = (int)(32 * blk + 8 * (reg >> 2) + 4 * h + (reg & 3));

@@ -1,0 +1,248 @@
+"""GPU tests of the fp32 Lloyd step whose labels are screened on the fp16 matrix cores
+(kernel variant 61): inputs chosen so that the certification fails for many, all or none of
+the samples, exact ties, features of very different scale, offsets far from the origin.
+Everything is compared with the CPU oracle (labels: exact except fp64 near-ties; exact ties
+must go to the lowest index, as in the reference's running arg-min,
+sklearn_numba_dpex/kmeans/kernels/_base_kmeans_kernel_funcs.py:228-267)."""
+
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from oracle import kmeans as ok
+from tests._parity import assert_centers_close, assert_labels_match
+
+pytestmark = pytest.mark.gpu
+
+
+def _one_iteration(X, w, init, cuda):
+    """kmx_lloyd_init + one kmx_lloyd_iter through the C ABI; returns labels, new centroids
+    (or the sums when a cluster is empty), sizes, status, variant, samples evaluated in fp32."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    n, d = X.shape
+    k = init.shape[0]
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+    X_t, w_d, c_in = dev(X.T), dev(w), dev(init.T)
+    c_out = torch.empty_like(c_in)
+    labels_prev = torch.zeros(n, dtype=torch.int32, device=cuda)
+    labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
+    sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+    variant = lib.kmx_lloyd_kernel_variant(n, d, k, 0)
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), n, d, k, 0, 10, 0.0, stream), "init")
+    _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
+                                   ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, 0, stream), "iter")
+    status = _capi.LloydStatus()
+    _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+    rechecked = ctypes.c_uint32(0)
+    _capi.check(lib.kmx_lloyd_recheck_count(ptr(ws), n, d, k, 0, ctypes.byref(rechecked), stream), "recheck")
+    return (labels.cpu().numpy().astype(np.int64), c_out.cpu().numpy().T, sizes.cpu().numpy(), status, variant,
+            int(rechecked.value))
+
+
+def _check_against_oracle(X, w, init, labels, c_out, sizes, status):
+    k = init.shape[0]
+    assert labels.min() >= 0 and labels.max() < k
+    assert_labels_match(labels, ok.assign_labels(X, init), X, init)
+    sums, ref_sizes = ok.weighted_sums(X, w, labels, k)
+    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-4)
+    assert status.n_empty == int(np.count_nonzero(ref_sizes == 0))
+    if status.n_empty == 0:
+        assert_centers_close(c_out, sums / ref_sizes[:, None], np.float32, scale_rtol=1e-4)
+    else:
+        assert_centers_close(c_out, sums, np.float32, scale_rtol=1e-4)
+
+
+def _blobs(n, d, k, seed, offset=0.0, scale=1.0):
+    rng = np.random.default_rng(seed)
+    centers = rng.uniform(-10, 10, (k, d))
+    X = ((centers[rng.integers(0, k, n)] + rng.standard_normal((n, d))) * scale + offset).astype(np.float32)
+    init = X[rng.choice(n, k, replace=False)].copy()
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    return X, w, init
+
+
+@pytest.mark.parametrize("shape", [(20_000, 14, 127), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40),
+                                   (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16)])
+def test_screened_step_matches_oracle(cuda, shape):
+    n, d, k = shape
+    X, w, init = _blobs(n, d, k, seed=n + d)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+    # on blob data only a small fraction of the labels needs the fp32 evaluation
+    assert rechecked <= 8 + n // 20
+
+
+def test_fp32_matrix_core_step_selected_by_environment(cuda):
+    """KMX_LLOYD_ASSIGN=f32 selects the all-fp32 kernel (variant 31); both give the oracle's labels."""
+    X, w, init = _blobs(30_000, 14, 127, seed=5)
+    got = {}
+    for mode in ("screen", "f32"):
+        if mode == "f32":
+            os.environ["KMX_LLOYD_ASSIGN"] = "f32"
+        try:
+            labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+        finally:
+            os.environ.pop("KMX_LLOYD_ASSIGN", None)
+        assert variant == (61 if mode == "screen" else 31)
+        if mode == "f32":
+            assert rechecked == 0
+        _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+        got[mode] = labels
+    # the two kernels may only differ at fp64 near-ties
+    assert_labels_match(got["screen"], got["f32"], X, init)
+
+
+def test_duplicate_centroids_take_the_lowest_index(cuda):
+    """Two pairs of identical centroids: exact ties, none of them certifiable; the reference's
+    strict '<' in increasing centroid order keeps the lower index."""
+    X, w, init = _blobs(20_000, 14, 64, seed=21)
+    init[40] = init[3]
+    init[63] = init[17]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    assert not np.any(labels == 40) and not np.any(labels == 63)
+    ref = ok.assign_labels(X, init)
+    assert_labels_match(labels, ref, X, init)
+    # every sample of the duplicated clusters went through the fp32 evaluation
+    assert rechecked >= int(np.count_nonzero((ref == 3) | (ref == 17)))
+    assert status.n_empty == 2 and status.state == 4
+
+
+def test_all_centroids_identical(cuda):
+    """No sample can be certified: every label comes from the fp32 evaluation and is 0."""
+    X, w, init = _blobs(5_000, 14, 16, seed=22)
+    init[:] = init[0]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    assert np.all(labels == 0)
+    assert rechecked == X.shape[0]
+    assert status.n_empty == 15
+
+
+def test_samples_on_the_bisector(cuda):
+    """Samples at exactly the same fp32 distance from two centroids (mirror images in the
+    first coordinate): the lower index wins; the other samples follow the oracle."""
+    rng = np.random.default_rng(23)
+    n, d, k = 8_192, 14, 32
+    init = rng.uniform(-4, 4, (k, d)).astype(np.float32)
+    init[1] = init[0]
+    init[1, 0] = -init[0, 0]                       # centroid 1 mirrors centroid 0
+    X = (init[rng.integers(0, k, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32)
+    on = np.arange(0, n, 7)
+    X[on] = init[0] + 0.05 * rng.standard_normal((on.size, d)).astype(np.float32)
+    X[on, 0] = 0.0                                 # on the bisector of centroids 0 and 1
+    w = np.ones(n, dtype=np.float32)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    ref = ok.assign_labels(X, init)
+    assert np.all(ref[on] <= 1)
+    assert np.all(labels[on] == 0)
+    assert_labels_match(labels, ref, X, init)
+    assert rechecked >= on.size
+
+
+def test_features_of_very_different_scale(cuda):
+    """One feature 1e6 times larger than the one that separates the clusters: the fp16 parts
+    of the small feature are far below those of the large one."""
+    rng = np.random.default_rng(24)
+    n, d, k = 20_000, 6, 24
+    centers = rng.uniform(-1, 1, (k, d))
+    X = centers[rng.integers(0, k, n)] + 0.05 * rng.standard_normal((n, d))
+    scales = np.array([1e3, 1e-3, 1.0, 30.0, 1e-2, 5.0])
+    X = (X * scales).astype(np.float32)
+    init = X[rng.choice(n, k, replace=False)].copy()
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+
+
+@pytest.mark.parametrize("offset,scale", [(1000.0, 1.0), (-3.0e4, 10.0), (0.0, 1e-12), (0.0, 1e12)])
+def test_offsets_and_extreme_magnitudes(cuda, offset, scale):
+    """Data far from the origin (the gaps between scores are tiny next to ||x|| ||c||, so many
+    samples need the fp32 evaluation) and data near the ends of the fp32 range."""
+    X, w, init = _blobs(10_000, 8, 20, seed=25, offset=offset, scale=scale)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    k = init.shape[0]
+    assert labels.min() >= 0 and labels.max() < k
+    # fp32 itself cannot separate clusters whose distance differences drown in ||x||^2: the
+    # oracle evaluates the same fp32 formula, and labels may differ where fp64 says near-tie
+    ref = ok.assign_labels(X, init)
+    dist_scale = 1.0
+    if offset != 0.0:
+        # accept the labels the fp32 formula can justify: compare through fp64 distances with
+        # the fp32 resolution of 0.5||c||^2 - <x, c> as tolerance
+        X64, C64 = X.astype(np.float64), init.astype(np.float64)
+        dd = ((X64[:, None, :] - C64[None, :, :]) ** 2).sum(axis=2)
+        got_d = dd[np.arange(len(labels)), labels]
+        best_d = dd.min(axis=1)
+        resolution = 64 * np.finfo(np.float32).eps * (np.abs(X64).max() ** 2) * X.shape[1]
+        assert np.all(got_d - best_d <= resolution * dist_scale)
+    else:
+        assert_labels_match(labels, ref, X, init)
+    sums, ref_sizes = ok.weighted_sums(X, w, labels, k)
+    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-4)
+
+
+def test_all_zero_data(cuda):
+    X = np.zeros((4_096, 14), dtype=np.float32)
+    w = np.ones(4_096, dtype=np.float32)
+    init = np.zeros((16, 14), dtype=np.float32)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    assert np.all(labels == 0)
+    assert sizes[0] == 4_096 and status.n_empty == 15
+
+
+def test_ten_iterations_stay_in_lockstep_with_the_oracle(cuda):
+    """Ten iterations through the driver-level loop of the C ABI; every iteration is compared
+    from the centroids the GPU started it with, and the count of fp32 evaluations stays small."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    X, w, init = _blobs(50_000, 14, 127, seed=26)
+    n, d = X.shape
+    k = init.shape[0]
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+    X_t, w_d = dev(X.T), dev(w)
+    cent = [dev(init.T), torch.empty(d, k, dtype=torch.float32, device=cuda)]
+    labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
+    sizes = torch.empty(k, dtype=torch.float32, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+    assert lib.kmx_lloyd_kernel_variant(n, d, k, 0) == 61
+    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, 0, 100, 0.0, stream), "init")
+    status = _capi.LloydStatus()
+    rechecked = ctypes.c_uint32(0)
+    for it in range(10):
+        a, b = it % 2, (it + 1) % 2
+        c_in = cent[a].cpu().numpy().T.copy()
+        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, 0,
+                                       stream), "iter")
+        _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+        _capi.check(lib.kmx_lloyd_recheck_count(ptr(ws), n, d, k, 0, ctypes.byref(rechecked), stream), "recheck")
+        got = labels[b].cpu().numpy().astype(np.int64)
+        assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
+        assert rechecked.value <= n // 50
+        if status.n_empty:
+            break
+        sums, ref_sizes = ok.weighted_sums(X, w, got, k)
+        assert_centers_close(cent[b].cpu().numpy().T, sums / ref_sizes[:, None], np.float32)
+        assert status.n_iter == it + 1
