@@ -335,28 +335,10 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 }
             }
         };
-        // the scores of the next block are issued before the arg-max of the current one, so
-        // that the vector ALU does not wait for a matrix-core result
-        {
-            v16f a0[NC], a1[NC];
-            scores(0, a0);
-            int cb = 0;
-            for (; cb + 2 < n_cb; cb += 2) {  // both accumulators are rewritten unconditionally
-                scores(cb + 1, a1);
-                __builtin_amdgcn_sched_barrier(0);
-                argmax_block(cb, a0);
-                scores(cb + 2, a0);
-                __builtin_amdgcn_sched_barrier(0);
-                argmax_block(cb + 1, a1);
-            }
-            if (cb + 1 < n_cb) {
-                scores(cb + 1, a1);
-                __builtin_amdgcn_sched_barrier(0);
-                argmax_block(cb, a0);
-                argmax_block(cb + 1, a1);
-            } else {
-                argmax_block(cb, a0);
-            }
+        for (int cb = 0; cb < n_cb; ++cb) {
+            v16f a[NC];
+            scores(cb, a);
+            argmax_block(cb, a);
         }
 
         // position inside the winning group, second largest inside it, then both half-waves
@@ -518,9 +500,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 
     // Rows of the lane: feature 2 p + h for the pairs p = 8 s + i.  Every load is a uniform
     // row address plus a 32-bit byte offset of the lane (n < 2^29), and unconditional, so
-    // that the compiler counts the loads and waits for the older tile only: a pair that is
-    // not entirely below d reads row d - 1 in both half-waves.
+    // that the compiler counts the loads and waits for the older tile only.
     const char* const xbytes = reinterpret_cast<const char*>(X_t);
+    // A pair that is not entirely below d reads row d - 1 in both half-waves.
     uint32_t lane_off[NK][8];
 #pragma unroll
     for (int s = 0; s < NK; ++s)
