@@ -56,7 +56,10 @@ constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
 
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
 #ifndef KMX_SCR_WAVES
-#define KMX_SCR_WAVES 8
+#define KMX_SCR_WAVES 12
+#endif
+#ifndef KMX_SCR_PREFETCH
+#define KMX_SCR_PREFETCH false
 #endif
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
 
@@ -533,19 +536,24 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     };
 
     if (wt_first < n_main) {
-        float xn[NK][8][MC];
-        load_rows(wt_first, xn);
+        constexpr bool PREFETCH = KMX_SCR_PREFETCH;
+        float xn[PREFETCH ? NK : 1][8][MC];
+        if constexpr (PREFETCH) load_rows(wt_first, xn);
         for (int64_t wt = wt_first; wt < n_main; wt += wt_step) {
             const int64_t i0 = wt * TILE + MC * j;
             float x[NK][8][MC];
+            if constexpr (PREFETCH) {
 #pragma unroll
-            for (int s = 0; s < NK; ++s)
+                for (int s = 0; s < NK; ++s)
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
+                    for (int i = 0; i < 8; ++i)
 #pragma unroll
-                    for (int t = 0; t < MC; ++t) x[s][i][t] = xn[s][i][t];
-            // past the last tile the same rows are read again (and not used)
-            load_rows(wt + wt_step < n_main ? wt + wt_step : wt, xn);
+                        for (int t = 0; t < MC; ++t) x[s][i][t] = xn[s][i][t];
+                // past the last tile the same rows are read again (and not used)
+                load_rows(wt + wt_step < n_main ? wt + wt_step : wt, xn);
+            } else {
+                load_rows(wt, x);
+            }
             float wv[MC] = {0.f, 0.f};
             uint32_t pl[MC] = {0u, 0u};
             if (UPDATE) {
