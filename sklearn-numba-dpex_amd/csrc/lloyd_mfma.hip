@@ -102,7 +102,14 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restric
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-    if ((threadIdx.x & 63) == 0) atomicMax(&absmax[row], __float_as_uint(m));
+    // one atomic per workgroup: thousands of waves on the same few words serialise in L2
+    __shared__ float wave_max[4];
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+        atomicMax(&absmax[row], __float_as_uint(m));
+    }
 }
 
 // q[f] for the sums of w * x_f, q[d] for the sums of w: the largest exponents such that
@@ -571,8 +578,9 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
     unsigned int* absmax = reinterpret_cast<unsigned int*>(ws + L.off_scales);
     int* q_exp = reinterpret_cast<int*>(absmax + (d + 1));
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(256), 0, stream, absmax, d + 1);
-    int64_t gx = kmx_cdiv(n, 256 * 32);
-    if (gx > 128) gx = 128;
+    int64_t gx = kmx_cdiv(n, 256 * 64);
+    if (gx > 64) gx = 64;
+    if (gx * (d + 1) < 1024) gx = kmx_cdiv(1024, d + 1) < kmx_cdiv(n, 1024) ? kmx_cdiv(1024, d + 1) : kmx_cdiv(n, 1024);
     const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0) && ((((uintptr_t)w) & 15) == 0);
     hipLaunchKernelGGL(absmax_rows_kernel, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
                        stream, (const float*)X_t, (const float*)w, absmax, n, d, vec_ok);
