@@ -141,6 +141,18 @@ int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_ho
 int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int32_t k,
                                 int32_t dtype, uint32_t* count_host, void* stream);
 
+/* Diagnostics of kernel variant 61, for tests of its certificate: the approximate scores
+ * <x, c> - 0.5||c||^2 exactly as the fused step forms them on the fp16 matrix cores (same
+ * power-of-two scaling, same two-part fp16 split, same MFMA sequence), in scaled units
+ * (x * scale, c * scale): scores (k, n), the per-sample error bound bounds (n) the step
+ * compares half the best-to-second gap with, the fp32 0.5||c * scale||^2 it starts from
+ * half_norms (k), and scale (1).  fp32 only; shapes variant 61 covers, else
+ * KMX_ERR_UNSUPPORTED; scratch: 256 bytes of device memory.
+ * It has no counterpart in the reference (diagnostics). */
+int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* scores, float* bounds,
+                          float* half_norms, float* scale, void* scratch, int64_t n, int32_t d,
+                          int32_t k, void* stream);
+
 /* Which fused-step kernel kmx_lloyd_iter uses for a shape, as 10 * path + accumulation:
  * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32) with the
  * centroids resident in LDS, 4 = MFMA (fp32) with samples in registers and centroids streamed;

@@ -67,6 +67,7 @@ SIGNATURES = {
     "kmx_lloyd_finalize": (_I32, [_P, _P, _P, _P, _SZ, _I32, _I32, _I32, _P]),
     "kmx_lloyd_status_read": (_I32, [_P, POINTER(LloydStatus), _P]),
     "kmx_lloyd_recheck_count": (_I32, [_P, _I64, _I32, _I32, _I32, POINTER(ctypes.c_uint32), _P]),
+    "kmx_screen_scores": (_I32, [_P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _P]),
     "kmx_lloyd_kernel_variant": (_I32, [_I64, _I32, _I32, _I32]),
     "kmx_assign_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kmx_assign_labels": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),

@@ -900,6 +900,22 @@ int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int
     return e == hipSuccess ? KMX_OK : (int32_t)e;
 }
 
+int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* scores, float* bounds,
+                          float* half_norms, float* scale, void* scratch, int64_t n, int32_t d,
+                          int32_t k, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(centroids_t);
+    KMX_REQUIRE_PTR(scores);
+    KMX_REQUIRE_PTR(bounds);
+    KMX_REQUIRE_PTR(half_norms);
+    KMX_REQUIRE_PTR(scale);
+    KMX_REQUIRE_PTR(scratch);
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    return kmx_screen_scores_impl((const float*)X_t, (const float*)centroids_t, scores, bounds, half_norms,
+                                  scale, (unsigned int*)scratch, n, d, k, (hipStream_t)stream_);
+}
+
 size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
     if (d <= 0 || k <= 0 || (dtype != KMX_F32 && dtype != KMX_F64)) return 0;
     return lloyd_layout(1, d, k, dtype).off_bucket;

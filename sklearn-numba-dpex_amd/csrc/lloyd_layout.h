@@ -129,6 +129,9 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, int64_t n, int d, int k,
                                    hipStream_t stream);
+int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
+                               float* bounds, float* half_norms, float* scale, unsigned int* scratch,
+                               int64_t n, int d, int k, hipStream_t stream);
 // wide-sample variant (lloyd_mfma_wide.hip): the fused step only; the reduction and
 // finalisation kernels of lloyd.hip follow it
 int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, const void* X_rowmajor,

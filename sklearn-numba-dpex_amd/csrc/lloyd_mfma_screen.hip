@@ -627,6 +627,130 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------- diagnostics
+
+__global__ void absmax_fill_zero(unsigned int* p) {
+    if (threadIdx.x == 0) *p = 0u;
+}
+
+// max |X_t| over all features into *xmax_bits (zero on entry), one workgroup per 1024 values.
+__global__ __launch_bounds__(256) void screen_absmax_kernel(const float* __restrict__ X_t,
+                                                            unsigned int* __restrict__ xmax_bits,
+                                                            int64_t count) {
+    float m = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256)
+        m = fmaxf(m, fabsf(X_t[i]));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((threadIdx.x & 63) == 0) atomicMax(xmax_bits, __float_as_uint(m));
+}
+
+// The approximate scores exactly as lloyd_screen_kernel forms them (same scaling, same split,
+// same MFMA sequence), written out with the error bound the kernel would use: one wave per 32
+// samples.  scores (k, n) and half_norms (k) are in scaled units (x * scale, c * scale).
+template <int NK>
+__global__ __launch_bounds__(64) void screen_scores_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ centroids_t,
+    const unsigned int* __restrict__ xmax_bits, float* __restrict__ scores,
+    float* __restrict__ bounds, float* __restrict__ half_norms, float* __restrict__ scale_out,
+    int64_t n, int d, int k) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int n_cb = (k + 31) >> 5;
+    v8h* afh = reinterpret_cast<v8h*>(smem_raw);
+    v8h* afl = afh + n_cb * NK * 64;
+    float* hneg = reinterpret_cast<float*>(afl + n_cb * NK * 64);
+    __shared__ unsigned int hmax_bits;
+    const float xmax = __uint_as_float(*xmax_bits);
+    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, 14 - ilogbf(xmax)) : 1.0f;
+    if (threadIdx.x == 0) hmax_bits = 0;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < n_cb * NK * 64; idx += 64) {
+        const int l = idx & 63, s = (idx >> 6) % NK, cb = (idx >> 6) / NK;
+        const int c = 32 * cb + (l & 31);
+        v8h hi, lo;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int f = 16 * s + 2 * i + (l >> 5);
+            const float v = (c < k && f < d) ? centroids_t[(size_t)f * k + c] * xs : 0.0f;
+            const _Float16 hb = (_Float16)v;
+            hi[i] = hb;
+            lo[i] = (_Float16)(v - (float)hb);
+        }
+        afh[idx] = hi;
+        afl[idx] = lo;
+    }
+    for (int idx = threadIdx.x; idx < n_cb * 32; idx += 64) {
+        const int cb = idx >> 5, hh = (idx >> 4) & 1, r = idx & 15;
+        const int c = 32 * cb + 8 * (r >> 2) + 4 * hh + (r & 3);
+        float v = -kmx_inf<float>();
+        if (c < k) {
+            float sq = 0.0f;
+            for (int f = 0; f < d; ++f) {
+                const float cv = centroids_t[(size_t)f * k + c] * xs;
+                sq += cv * cv;
+            }
+            v = -(sq / 2.0f);
+            atomicMax(&hmax_bits, __float_as_uint(sq / 2.0f));
+            if (blockIdx.x == 0) half_norms[c] = sq / 2.0f;
+        }
+        hneg[idx] = v;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x, h = lane >> 5, j = lane & 31;
+    const int64_t i0 = (int64_t)blockIdx.x * 32 + j;
+    const float hmax = __uint_as_float(hmax_bits);
+    const float cmax = sqrtf(2.0f * hmax), abs_term = SCR_ERR_ABS * sqrtf((float)d);
+    v8h xh[NK], xl[NK];
+    float ss = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NK; ++s)
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            const int f = 16 * s + 2 * i + h;
+            const float x0 = (f < d && i0 < n) ? X_t[(size_t)f * n + i0] : 0.0f;
+            const float x1 = (f + 2 < d && i0 < n) ? X_t[(size_t)(f + 2) * n + i0] : 0.0f;
+            const v2f p = {x0 * xs, x1 * xs};
+            const v2h hh = __builtin_convertvector(p, v2h);
+            const v2f r = p - __builtin_convertvector(hh, v2f);
+            const v2h ll = __builtin_convertvector(r, v2h);
+            xh[s][i] = hh[0];
+            xh[s][i + 1] = hh[1];
+            xl[s][i] = ll[0];
+            xl[s][i + 1] = ll[1];
+            ss = fmaf(p[0], p[0], ss);
+            ss = fmaf(p[1], p[1], ss);
+        }
+    const float nrm = ss + __shfl_xor(ss, 32, 64);
+    if (h == 0 && i0 < n)
+        bounds[i0] = fmaf(SCR_ERR_X * cmax + abs_term, __builtin_amdgcn_sqrtf(nrm), SCR_ERR_H * hmax + abs_term * cmax);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = xs;
+    for (int cb = 0; cb < n_cb; ++cb) {
+        const float4* hp = reinterpret_cast<const float4*>(hneg + cb * 32 + h * 16);
+        v16f a;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 v4 = hp[q];
+            a[4 * q] = v4.x;
+            a[4 * q + 1] = v4.y;
+            a[4 * q + 2] = v4.z;
+            a[4 * q + 3] = v4.w;
+        }
+#pragma unroll
+        for (int s = 0; s < NK; ++s) {
+            const v8h ah = afh[(cb * NK + s) * 64 + lane];
+            const v8h al = afl[(cb * NK + s) * 64 + lane];
+            a = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xh[s], a, 0, 0, 0);
+            a = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xl[s], a, 0, 0, 0);
+            a = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, xh[s], a, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int c = 32 * cb + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (c < k && i0 < n) scores[(size_t)c * n + i0] = a[r];
+        }
+    }
+}
+
 }  // namespace
 
 // Shapes the screened step covers: d <= 32, everything within 64 KB of LDS, byte offsets
@@ -672,6 +796,27 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
                            labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, n, d, k,
                            vec_ok);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+// Diagnostics of the screen: approximate scores and error bounds as the fused step forms them.
+int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
+                               float* bounds, float* half_norms, float* scale, unsigned int* scratch,
+                               int64_t n, int d, int k, hipStream_t stream) {
+    if (!kmx_mfma_screen_supported(n, d, k)) return KMX_ERR_UNSUPPORTED;
+    const int nk = (d + 15) / 16, n_cb = (k + 31) / 32;
+    const size_t lds = (size_t)n_cb * nk * 64 * 32 + (size_t)n_cb * 32 * 4;
+    if (lds > 64 * 1024) return KMX_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(absmax_fill_zero, dim3(1), dim3(64), 0, stream, scratch);
+    hipLaunchKernelGGL(screen_absmax_kernel, dim3(256), dim3(256), 0, stream, X_t, scratch, (int64_t)d * n);
+    const unsigned grid = (unsigned)kmx_cdiv(n, 32);
+    if (nk == 1)
+        hipLaunchKernelGGL((screen_scores_kernel<1>), dim3(grid), dim3(64), lds, stream, X_t, centroids_t,
+                           scratch, scores, bounds, half_norms, scale, n, d, k);
+    else
+        hipLaunchKernelGGL((screen_scores_kernel<2>), dim3(grid), dim3(64), lds, stream, X_t, centroids_t,
+                           scratch, scores, bounds, half_norms, scale, n, d, k);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

@@ -246,3 +246,71 @@ def test_ten_iterations_stay_in_lockstep_with_the_oracle(cuda):
         sums, ref_sizes = ok.weighted_sums(X, w, got, k)
         assert_centers_close(cent[b].cpu().numpy().T, sums / ref_sizes[:, None], np.float32)
         assert status.n_iter == it + 1
+
+
+def _screen_scores(X, C, cuda):
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    n, d = X.shape
+    k = C.shape[0]
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+    X_t, C_t = dev(X.T), dev(C.T)
+    scores = torch.empty(k, n, dtype=torch.float32, device=cuda)
+    bounds = torch.empty(n, dtype=torch.float32, device=cuda)
+    half = torch.empty(k, dtype=torch.float32, device=cuda)
+    scale = torch.empty(1, dtype=torch.float32, device=cuda)
+    scratch = torch.zeros(64, dtype=torch.int32, device=cuda)
+    _capi.check(lib.kmx_screen_scores(ptr(X_t), ptr(C_t), ptr(scores), ptr(bounds), ptr(half), ptr(scale),
+                                      ptr(scratch), n, d, k, _capi.current_stream()), "screen_scores")
+    torch.cuda.synchronize()
+    return scores.cpu().numpy(), bounds.cpu().numpy(), half.cpu().numpy(), float(scale.cpu().numpy()[0])
+
+
+def _screen_cases():
+    rng = np.random.default_rng(31)
+    cases = {}
+    X, _, C = _blobs(4_000, 14, 127, seed=32)
+    cases["blobs d=14 k=127"] = (X, C)
+    X, _, C = _blobs(3_000, 32, 64, seed=33)
+    cases["blobs d=32 k=64"] = (X, C)
+    # centroids are samples: <x, c> - 0.5||c||^2 cancels to 0.5||x||^2 - 0.5||x - c||^2
+    X = rng.standard_normal((2_048, 16)).astype(np.float32) * 3 + 50
+    cases["offset 50, centroids = samples"] = (X, X[:64].copy())
+    # every mantissa bit in use, alternating signs, wide range of magnitudes inside a row
+    X = (rng.uniform(1, 2, (2_048, 31)) * rng.choice([-1, 1], (2_048, 31)) *
+         np.exp2(rng.integers(-12, 12, (2_048, 31)))).astype(np.float32)
+    C = (rng.uniform(1, 2, (48, 31)) * rng.choice([-1, 1], (48, 31)) *
+         np.exp2(rng.integers(-12, 12, (48, 31)))).astype(np.float32)
+    cases["random exponents d=31"] = (X, C)
+    # one feature only, tiny and huge data
+    cases["d=1"] = (rng.standard_normal((1_000, 1)).astype(np.float32), rng.standard_normal((16, 1)).astype(np.float32))
+    cases["tiny values"] = ((rng.standard_normal((1_000, 8)) * 1e-18).astype(np.float32),
+                            (rng.standard_normal((20, 8)) * 1e-18).astype(np.float32))
+    cases["huge values"] = ((rng.standard_normal((1_000, 8)) * 1e16).astype(np.float32),
+                            (rng.standard_normal((20, 8)) * 1e16).astype(np.float32))
+    return cases
+
+
+@pytest.mark.parametrize("name", list(_screen_cases().keys()))
+def test_error_bound_of_the_screen_holds_on_the_hardware(cuda, name):
+    """The certificate of variant 61 rests on |approximate score - exact score| <= E(x).  The
+    scores the matrix cores really produce are compared with fp64 here (the bound assumes at
+    most one ulp of error per accumulation inside an MFMA, which no document guarantees)."""
+    X, C = _screen_cases()[name]
+    scores, bounds, half, scale = _screen_scores(X, C, cuda)
+    assert np.log2(scale) == np.round(np.log2(scale))            # a power of two
+    assert 2.0 ** 14 <= np.abs(X).max() * scale < 2.0 ** 15
+    Xs, Cs = X.astype(np.float64) * scale, C.astype(np.float64) * scale
+    np.testing.assert_allclose(half, 0.5 * (Cs ** 2).sum(axis=1), rtol=1e-5)
+    exact = Cs @ Xs.T - half.astype(np.float64)[:, None]           # from the fp32 half norms the step uses
+    err = np.abs(scores.astype(np.float64) - exact)
+    assert np.all(np.isfinite(scores))
+    ratio = (err / bounds[None, :].astype(np.float64)).max()
+    print(f"{name}: largest error / bound = {ratio:.3f}")
+    assert ratio <= 1.0
+    # and the bound is not vacuous: far below the typical score
+    typical = np.median(np.abs(exact))
+    assert np.median(bounds) <= 1e-3 * max(typical, np.abs(exact).max() * 1e-3)
