@@ -758,6 +758,11 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
                            L.screen ? (size_t)64 : (size_t)k);
         KMX_LAUNCH_CHECK();
     }
+    if (L.variant == KMX_VARIANT_MFMA_WIDE) {
+        hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1), dim3(64), 0, stream,
+                           (uint32_t*)(ws + L.off_wscreen), (size_t)64);
+        KMX_LAUNCH_CHECK();
+    }
     if (L.acc_mode == ACC_GLOBAL && L.partial_bytes > 0) {
         const size_t words = L.partial_bytes / 4;
         hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1024), dim3(256), 0, stream,
@@ -891,10 +896,14 @@ int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int
     KMX_REQUIRE_DTYPE(dtype);
     const LloydLayout L = lloyd_layout(n, d, k, dtype);
     *count_host = 0;
-    if (!L.screen) return KMX_OK;
+    const void* src = nullptr;
+    if (L.screen)
+        src = (const char*)workspace + L.off_bucket + sizeof(uint32_t);
+    else if (L.variant == KMX_VARIANT_MFMA_WIDE && kmx_wide_screen_enabled(n, d, k))
+        src = kmx_wide_screen_counter((const char*)workspace + L.off_wscreen);
+    if (src == nullptr) return KMX_OK;
     hipStream_t stream = (hipStream_t)stream_;
-    hipError_t e = hipMemcpyAsync(count_host, (const char*)workspace + L.off_bucket + sizeof(uint32_t),
-                                  sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
+    hipError_t e = hipMemcpyAsync(count_host, src, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
     if (e != hipSuccess) return (int32_t)e;
     e = hipStreamSynchronize(stream);
     return e == hipSuccess ? KMX_OK : (int32_t)e;

@@ -29,6 +29,11 @@ bool kmx_mfma_wide_supported(int d, int k);
 bool kmx_mfma_f64_supported(int d, int k);
 // fp32 matrix-core step with bf16 screening of the labels (lloyd_mfma_screen.hip)
 bool kmx_mfma_screen_supported(int64_t n, int d, int k);
+// screened label step of the wide path (lloyd_mfma_wide_screen.hip)
+size_t kmx_wide_screen_bytes(int64_t n, int d, int k);
+const int* kmx_wide_screen_list(const char* area, int d, int k);
+bool kmx_wide_screen_enabled(int64_t n, int d, int k);
+const uint32_t* kmx_wide_screen_counter(const char* area);
 
 struct LloydLayout {
     int dpad;            // features per packed centroid row (multiple of 4, zero padded)
@@ -37,7 +42,7 @@ struct LloydLayout {
     int n_partials;      // slots in `partial` (workgroups for LDS mode, copies for global mode)
     int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
     bool screen;         // KMX_VARIANT_MFMA with bf16-screened labels (variant code 61)
-    size_t off_status, off_scales, off_gsum, off_cpack, off_half, off_shift, off_bucket, off_partial;
+    size_t off_status, off_scales, off_gsum, off_cpack, off_half, off_shift, off_bucket, off_wscreen, off_partial;
     size_t partial_bytes;
     size_t total;
     // Workgroups of the fused step: a few per compute unit (KMX_LLOYD_WGS_PER_CU, default 4),
@@ -101,7 +106,11 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
         L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int)
         : L.screen                         ? (size_t)64 * sizeof(int)
                                            : 0;
-    L.off_partial = L.off_bucket + kmx_align256(bucket_bytes);
+    // wide matrix-core path: header, scaled half norms and fp16 parts of the centroids for the
+    // screened label step (lloyd_mfma_wide_screen.hip)
+    L.off_wscreen = L.off_bucket + kmx_align256(bucket_bytes);
+    const size_t wscreen_bytes = L.variant == KMX_VARIANT_MFMA_WIDE ? kmx_wide_screen_bytes(n, d, k) : 0;
+    L.off_partial = L.off_wscreen + kmx_align256(wscreen_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
     const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE;
     L.partial_bytes = fixed_point ? 0 : (size_t)L.n_partials * items * s;
@@ -132,6 +141,11 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,
                                int64_t n, int d, int k, hipStream_t stream);
+int32_t kmx_lloyd_wide_screen_count(const void* X_t, const void* centroids_t,
+                                    const unsigned int* absmax, char* area,
+                                    const uint32_t* labels_prev, uint32_t* labels,
+                                    kmx_lloyd_status* status, int* counts, int* ranks, int64_t n,
+                                    int d, int k, hipStream_t stream);
 // wide-sample variant (lloyd_mfma_wide.hip): the fused step only; the reduction and
 // finalisation kernels of lloyd.hip follow it
 int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, const void* X_rowmajor,

@@ -190,7 +190,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, j = lane & 31;
-    const int64_t n_wtiles = (n + TILE - 1) / TILE;
+    const int n_wtiles = (int)((n + TILE - 1) / TILE);  // n < 2^29: tile and sample indices fit 32 bits
     unsigned int changed = 0;
     unsigned int n_uncertain = 0;  // wave-uniform
 
@@ -491,15 +491,15 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     using Cols2 = std::integral_constant<int, MC>;
     using Cols1 = std::integral_constant<int, 1>;
 
-    const int64_t wt_step = (int64_t)gridDim.x * WAVES;
-    const int64_t wt_first = (int64_t)blockIdx.x * WAVES + wave;
-    const int64_t n_fast = vec_ok ? n / TILE : 0;
+    const int wt_step = (int)gridDim.x * WAVES;
+    const int wt_first = (int)blockIdx.x * WAVES + wave;
+    const int n_fast = vec_ok ? (int)(n / TILE) : 0;
     // a last round of full tiles that is at most three quarters full is cut into
     // single-column tiles of 32 samples, spread over all the waves
-    const int64_t n_rounds = n_fast / wt_step;
-    const int64_t n_left = n_fast - n_rounds * wt_step;
-    const bool halves = n_left > 0 && 4 * n_left <= 3 * wt_step;
-    const int64_t n_main = halves ? n_rounds * wt_step : n_fast;
+    const int n_rounds = n_fast / wt_step;
+    const int n_left = n_fast - n_rounds * wt_step;
+    const bool halves = n_left > 0 && 4 * (int64_t)n_left <= 3 * (int64_t)wt_step;
+    const int n_main = halves ? n_rounds * wt_step : n_fast;
 
     // Rows of the lane: feature 2 p + h for the pairs p = 8 s + i.  Every load is a uniform
     // row address plus a 32-bit byte offset of the lane (n < 2^29), and unconditional, so
@@ -517,17 +517,19 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     // would not fit the scalar registers and would be spilled and reloaded around every load).
     const size_t pair_stride = (size_t)n * 8u;  // two rows
     const char* const tail_row = xbytes + (size_t)(d - 1) * (size_t)n * 4u;
-    auto load_rows = [&](const int64_t wt, float(&dst)[NK][8][MC]) {
+    auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) {
         const uint32_t tile_off = (uint32_t)wt * (uint32_t)(TILE * 4);
         size_t hidden_zero = 0;
         asm volatile("" : "+s"(hidden_zero));
         const char* row = xbytes + hidden_zero;
+        int d_now = d;  // compared afresh with scalar instructions: no lane masks kept per row
+        asm volatile("" : "+s"(d_now));
 #pragma unroll
         for (int s = 0; s < NK; ++s)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int p0 = 16 * s + 2 * i;
-                const char* src = p0 + 1 < d ? row : tail_row;
+                const char* src = p0 + 1 < d_now ? row : tail_row;
                 const float2 q = *reinterpret_cast<const float2*>(src + (tile_off + lane_off[s][i]));
                 dst[s][i][0] = q.x;
                 dst[s][i][1] = q.y;
@@ -539,8 +541,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         constexpr bool PREFETCH = KMX_SCR_PREFETCH;
         float xn[PREFETCH ? NK : 1][8][MC];
         if constexpr (PREFETCH) load_rows(wt_first, xn);
-        for (int64_t wt = wt_first; wt < n_main; wt += wt_step) {
-            const int64_t i0 = wt * TILE + MC * j;
+        for (int wt = wt_first; wt < n_main; wt += wt_step) {
+            const int64_t i0 = (int64_t)wt * TILE + MC * j;
             float x[NK][8][MC];
             if constexpr (PREFETCH) {
 #pragma unroll
@@ -582,8 +584,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     };
     if (halves) {
         // single-column tile q of the left-over tiles: samples [n_main * TILE + 32 q, + 32)
-        for (int64_t q = wt_first; q < MC * n_left; q += wt_step) {
-            const int64_t i0 = n_main * TILE + 32 * q + j;
+        for (int q = wt_first; q < MC * n_left; q += wt_step) {
+            const int64_t i0 = (int64_t)n_main * TILE + 32 * q + j;
             float x[NK][8][1];
             load_scalar(Cols1{}, i0, x);
             float wv[1] = {0.f};
@@ -596,8 +598,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         }
     }
     // The rest: a partial last tile, or every tile when vector accesses are not legal
-    for (int64_t wt = n_fast + wt_first; wt < n_wtiles; wt += wt_step) {
-        const int64_t i0 = wt * TILE + MC * j;
+    for (int wt = n_fast + wt_first; wt < n_wtiles; wt += wt_step) {
+        const int64_t i0 = (int64_t)wt * TILE + MC * j;
         float x[NK][8][MC];
         load_scalar(Cols2{}, i0, x);
         float wv[MC];

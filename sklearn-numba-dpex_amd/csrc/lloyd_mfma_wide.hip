@@ -78,16 +78,22 @@ constexpr int MODE_ATOMICS = 1;  // labels + one global fixed-point atomic per (
 constexpr int MODE_COUNT = 2;    // labels + changed count + per-cluster sample counts; the sums
                                  // are taken afterwards by the bucketed accumulation below
 
-template <int NKC, int MODE>
+// LISTED: the kernel works on the samples list[0 .. *list_count) instead of 0 .. n - 1 (the
+// samples the fp16 screen of lloyd_mfma_wide_screen.hip could not certify) and reads their
+// features from the row-major copy X_rm.
+template <int NKC, int MODE, bool LISTED = false>
 __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     kmx_lloyd_status* __restrict__ status, const int* __restrict__ q_exp,
     unsigned long long* __restrict__ gsum, int* __restrict__ counts, int* __restrict__ ranks,
-    int64_t n, int d, int k, int vec_ok) {
+    int64_t n, int d, int k, int vec_ok, const float* __restrict__ X_rm = nullptr,
+    const int* __restrict__ list = nullptr, const unsigned int* __restrict__ list_count = nullptr) {
     constexpr bool UPDATE = MODE != MODE_LABELS;
     if (UPDATE && status->state != KMX_RUNNING) return;
+    const int64_t n_work = LISTED ? (int64_t)*list_count : n;
+    if (LISTED && (int64_t)blockIdx.x * 128 >= n_work) return;
 
     __shared__ __align__(16) float ctile[2][KC][CG];
     extern __shared__ __align__(16) float hneg_s[];  // [n_cg * CG]: -0.5||c||^2, -inf past k
@@ -103,17 +109,22 @@ __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, j = lane & 31;
-    const int64_t n_tiles = (n + 127) >> 7;
+    const int64_t n_tiles = (n_work + 127) >> 7;
     unsigned int changed = 0;
     constexpr int NKS = NKC * 16;
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        const int64_t i = tile * 128 + wave * 32 + j;
-        const bool valid = i < n;
+        const int64_t slot = tile * 128 + wave * 32 + j;
+        const bool valid = slot < n_work;
+        const int64_t i = LISTED ? (int64_t)list[valid ? slot : 0] : slot;
 
         // row 2s + h of X_t, advanced by two rows per K step (no per-row offsets kept alive)
         float x[NKS];
-        {
+        if constexpr (LISTED) {
+            const float* __restrict__ xp = X_rm + (size_t)i * d + h;
+#pragma unroll
+            for (int s = 0; s < NKS; ++s) x[s] = (valid && 2 * s + h < d) ? xp[2 * s] : 0.0f;
+        } else {
             // branch-free: out-of-range rows/samples read element 0 of X_t and are zeroed
             const float* __restrict__ xp = X_t + (size_t)h * n + (valid ? i : 0);
             const size_t two_rows = 2 * (size_t)n;
@@ -415,6 +426,42 @@ int32_t launch_wide(const LloydLayout& L, const void* X_t, const void* w, const 
     return KMX_OK;
 }
 
+// The counting mode on the listed samples only; the grid is fixed because the length of the
+// list is only known on the device (blocks without a tile leave at once).
+int32_t launch_wide_listed(const void* X_t, const void* X_rm, const void* w, const void* centroids_t,
+                           const float* half_norms, const uint32_t* labels_prev, uint32_t* labels,
+                           kmx_lloyd_status* status, const int* q_exp, unsigned long long* gsum,
+                           int* counts, int* ranks, const int* list, const unsigned int* list_count,
+                           int64_t n, int d, int k, hipStream_t stream) {
+    if (!kmx_mfma_wide_supported(d, k)) return KMX_ERR_UNSUPPORTED;
+    const int n_cg = (k + CG - 1) / CG;
+    const size_t lds = (size_t)n_cg * CG * sizeof(float);
+    int64_t grid = kmx_cdiv(n, 128);
+    const int64_t cap = 2 * (int64_t)kmx_num_cus();
+    if (grid > cap) grid = cap;
+    if (grid < 1) grid = 1;
+    const int vec_ok = (k % 4 == 0) && ((((uintptr_t)centroids_t) & 15) == 0);
+#define KMX_WIDE_CASE(NKC)                                                                             \
+    hipLaunchKernelGGL((lloyd_mfma_wide_kernel<NKC, MODE_COUNT, true>), dim3((unsigned)grid), dim3(256), \
+                       lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,       \
+                       half_norms, labels_prev, labels, status, q_exp, gsum, counts, ranks, n, d, k,     \
+                       vec_ok, (const float*)X_rm, list, list_count)
+    switch ((d + KC - 1) / KC) {
+        case 1: KMX_WIDE_CASE(1); break;
+        case 2: KMX_WIDE_CASE(2); break;
+        case 3: KMX_WIDE_CASE(3); break;
+        case 4: KMX_WIDE_CASE(4); break;
+        case 5: KMX_WIDE_CASE(5); break;
+        case 6: KMX_WIDE_CASE(6); break;
+        case 7: KMX_WIDE_CASE(7); break;
+        case 8: KMX_WIDE_CASE(8); break;
+        default: return KMX_ERR_UNSUPPORTED;
+    }
+#undef KMX_WIDE_CASE
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
 }  // namespace
 
 bool kmx_mfma_wide_supported(int d, int k) {
@@ -438,8 +485,21 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
     int* offsets = counts + k;
     int* order = offsets + (k + 1);
     int* ranks = order + n;
-    int32_t rc = launch_wide<MODE_COUNT>(L, X_t, w, centroids_t, half_norms, labels_prev, labels,
-                                         status, q_exp, gsum, counts, ranks, n, d, k, stream);
+    int32_t rc;
+    if (kmx_wide_screen_enabled(n, d, k)) {
+        // labels screened on the fp16 matrix cores; what the screen cannot certify is listed
+        // and goes through the all-fp32 kernel
+        char* area = ws + L.off_wscreen;
+        rc = kmx_lloyd_wide_screen_count(X_t, centroids_t,
+                                         reinterpret_cast<const unsigned int*>(ws + L.off_scales), area,
+                                         labels_prev, labels, status, counts, ranks, n, d, k, stream);
+        if (rc != KMX_OK) return rc;
+        rc = launch_wide_listed(X_t, X_rowmajor, w, centroids_t, half_norms, labels_prev, labels, status,
+                                q_exp, gsum, counts, ranks, kmx_wide_screen_list(area, d, k),
+                                kmx_wide_screen_counter(area), n, d, k, stream);
+    } else
+        rc = launch_wide<MODE_COUNT>(L, X_t, w, centroids_t, half_norms, labels_prev, labels, status,
+                                     q_exp, gsum, counts, ranks, n, d, k, stream);
     if (rc != KMX_OK) return rc;
     hipLaunchKernelGGL(bucket_offsets_kernel, dim3(1), dim3(1024), 0, stream, counts, offsets, k);
     int64_t sg = kmx_cdiv(n, 256 * 4);

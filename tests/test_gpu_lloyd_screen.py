@@ -39,7 +39,8 @@ def _one_iteration(X, w, init, cuda):
     stream = _capi.current_stream()
     variant = lib.kmx_lloyd_kernel_variant(n, d, k, 0)
     _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), n, d, k, 0, 10, 0.0, stream), "init")
-    _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
+    X_rm = dev(X) if variant == 42 else None  # the wide path sums (and screens) with a row-major copy
+    _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
                                    ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, 0, stream), "iter")
     status = _capi.LloydStatus()
     _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
@@ -314,3 +315,49 @@ def test_error_bound_of_the_screen_holds_on_the_hardware(cuda, name):
     # and the bound is not vacuous: far below the typical score
     typical = np.median(np.abs(exact))
     assert np.median(bounds) <= 1e-3 * max(typical, np.abs(exact).max() * 1e-3)
+
+
+@pytest.mark.parametrize("shape", [(6_000, 128, 64), (3_000, 256, 200), (4_097, 40, 400), (2_500, 70, 1024)])
+def test_wide_screened_step_matches_oracle(cuda, shape):
+    """The wide fp32 path (variant 42) screens its labels the same way; what it cannot certify
+    goes through the all-fp32 matrix-core kernel."""
+    n, d, k = shape
+    X, w, init = _blobs(n, d, k, seed=n + d)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 42
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+    assert rechecked <= 8 + n // 10
+
+
+def test_wide_duplicate_centroids_take_the_lowest_index(cuda):
+    X, w, init = _blobs(8_000, 128, 96, seed=41)
+    init[70] = init[5]
+    init[95] = init[64]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 42
+    assert not np.any(labels == 70) and not np.any(labels == 95)
+    ref = ok.assign_labels(X, init)
+    assert_labels_match(labels, ref, X, init)
+    assert rechecked >= int(np.count_nonzero((ref == 5) | (ref == 64)))
+    assert status.n_empty == 2
+
+
+def test_wide_all_centroids_identical(cuda):
+    X, w, init = _blobs(3_000, 96, 64, seed=42)
+    init[:] = init[0]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 42
+    assert np.all(labels == 0)
+    assert rechecked == X.shape[0]
+    assert status.n_empty == 63
+
+
+def test_wide_screen_switched_off_by_environment(cuda):
+    X, w, init = _blobs(5_000, 128, 64, seed=43)
+    os.environ["KMX_LLOYD_ASSIGN"] = "f32"
+    try:
+        labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    finally:
+        os.environ.pop("KMX_LLOYD_ASSIGN", None)
+    assert variant == 42 and rechecked == 0
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
