@@ -184,14 +184,14 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
         v8h xh[NS], xl[NS];
         float ss = 0.0f;
         {
-            // Loaded in batches of two K steps, 16 values in flight per lane, then converted.  The
+            // Loaded in batches of four K steps, 32 values in flight per lane, then converted.  The
             // loads are inline assembly: at this register pressure the compiler would otherwise
             // funnel every value through one register and wait for each load in turn, paying the
             // memory latency 128 times per tile.  The values are valid after the wait statement,
             // which takes them as operands.
             const float* __restrict__ xp = X_t + (size_t)h * n + (valid ? i : 0);
             const size_t two_rows = 2 * (size_t)n;
-            constexpr int BATCH = NS < 2 ? NS : 2;
+            constexpr int BATCH = NS < 4 ? 2 : 4;  // NS is even
 #pragma unroll
             for (int S0 = 0; S0 < NS; S0 += BATCH) {
                 float raw[BATCH * 8];
@@ -203,16 +203,14 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                     asm volatile("global_load_dword %0, %1, off" : "=v"(raw[u]) : "v"(src));
                     xp += two_rows;
                 }
-                if constexpr (BATCH == 2)
+                // one wait for the whole batch; the statements take 16 values each (operand limit)
+#pragma unroll
+                for (int g = 0; g < BATCH * 8; g += 16)
                     asm volatile("s_waitcnt vmcnt(0)"
-                                 : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]), "+v"(raw[4]),
-                                   "+v"(raw[5]), "+v"(raw[6]), "+v"(raw[7]), "+v"(raw[8]), "+v"(raw[9]),
-                                   "+v"(raw[10]), "+v"(raw[11]), "+v"(raw[12]), "+v"(raw[13]),
-                                   "+v"(raw[14]), "+v"(raw[15]));
-                else
-                    asm volatile("s_waitcnt vmcnt(0)"
-                                 : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]), "+v"(raw[4]),
-                                   "+v"(raw[5]), "+v"(raw[6]), "+v"(raw[7]));
+                                 : "+v"(raw[g + 0]), "+v"(raw[g + 1]), "+v"(raw[g + 2]), "+v"(raw[g + 3]),
+                                   "+v"(raw[g + 4]), "+v"(raw[g + 5]), "+v"(raw[g + 6]), "+v"(raw[g + 7]),
+                                   "+v"(raw[g + 8]), "+v"(raw[g + 9]), "+v"(raw[g + 10]), "+v"(raw[g + 11]),
+                                   "+v"(raw[g + 12]), "+v"(raw[g + 13]), "+v"(raw[g + 14]), "+v"(raw[g + 15]));
 #pragma unroll
                 for (int u = 0; u < BATCH * 8; u += 2) {
                     const int S = S0 + u / 8, q = u % 8;
