@@ -146,8 +146,9 @@ int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int
  * power-of-two scaling, same two-part fp16 split, same MFMA sequence), in scaled units
  * (x * scale, c * scale): scores (k, n), the per-sample error bound bounds (n) the step
  * compares half the best-to-second gap with, the fp32 0.5||c * scale||^2 it starts from
- * half_norms (k), and scale (1).  fp32 only; shapes variant 61 covers, else
- * KMX_ERR_UNSUPPORTED; scratch: 256 bytes of device memory.
+ * half_norms (k), and scale (1).  fp32 only; d <= 256 and k small enough for the operands of
+ * all centroids to fit 64 KB of LDS (the wide path, variant 42, uses the same arithmetic),
+ * else KMX_ERR_UNSUPPORTED; scratch: 256 bytes of device memory.
  * It has no counterpart in the reference (diagnostics). */
 int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* scores, float* bounds,
                           float* half_norms, float* scale, void* scratch, int64_t n, int32_t d,

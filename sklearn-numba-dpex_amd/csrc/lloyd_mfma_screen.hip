@@ -12,8 +12,8 @@
 // and the fp32 accumulation of the 48 exact products adds at most 51 roundings of one ulp of a
 // partial sum each (6.1e-6 relative to 0.5||c||^2 + sum_f |x_f c_f|).  With Cauchy-Schwarz the
 // error of every score of sample x is bounded by
-//   E(x) = 6.93e-6 ||x|| C + 6.2e-6 H + 6.2e-5 sqrt(d) (||x|| + C),  C = max ||c||, H = max 0.5||c||^2
-// (scaled units).  If the best approximate score beats the second best by more than 2 E(x),
+//   E(x) = (7.2e-7 + r) ||x|| C + r H + 6.2e-5 sqrt(d) (||x|| + C),  r = 6.1e-6 ceil(d / 16),
+// C = max ||c||, H = max 0.5||c||^2 (scaled units).  If the best approximate score beats the second best by more than 2 E(x),
 // the arg-max of the approximate scores IS the arg-max of the exact real-valued scores: the
 // label is certain.  Otherwise (about 2 samples in 1000 on blob data) the wave evaluates the
 // sample in plain fp32 on the spot: every lane takes the centroids lane, lane + 64, ... with
@@ -48,10 +48,11 @@ __device__ __forceinline__ unsigned long long to_fixed(double scaled_plus_magic)
 }
 
 // Error bound of one approximate score, in scaled units:
-//   SCR_ERR_X ||x|| C + SCR_ERR_H H + SCR_ERR_ABS sqrt(d) (||x|| + C)
-constexpr float SCR_ERR_X = 6.93e-6f;
-constexpr float SCR_ERR_H = 6.2e-6f;
-constexpr float SCR_ERR_ABS = 6.2e-5f;
+//   (SCR_ERR_SPLIT + r) ||x|| C + r H + SCR_ERR_ABS sqrt(d) (||x|| + C),
+// r = SCR_ERR_ROUND * 51 * (K steps of 16 features): one ulp per addition of the accumulation
+constexpr float SCR_ERR_SPLIT = 7.2e-7f;  // 3.01 * 2^-22, rounded up
+constexpr float SCR_ERR_ROUND = 1.2e-7f;  // 2^-23, rounded up
+constexpr float SCR_ERR_ABS = 6.2e-5f;    // 2^-14, rounded up
 constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
 
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
@@ -198,8 +199,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     // margin for the rounding of the bound itself and of the hardware square root
     const float hmax = __uint_as_float(hmax_bits);
     const float cmax = sqrtf(2.0f * hmax), abs_term = SCR_ERR_ABS * sqrtf((float)d);
-    const float thr_x = 2.01f * (SCR_ERR_X * cmax + abs_term);
-    const float thr_0 = 2.01f * (SCR_ERR_H * hmax + abs_term * cmax);
+    const float round_term = SCR_ERR_ROUND * 51.0f * (float)NK;
+    const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term);
+    const float thr_0 = 2.01f * (round_term * hmax + abs_term * cmax);
     // +inf the optimiser cannot see through (it would turn the median below into a maximum
     // with two canonicalising instructions in front)
     float pos_inf = kmx_inf<float>();
@@ -702,6 +704,7 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
     const int64_t i0 = (int64_t)blockIdx.x * 32 + j;
     const float hmax = __uint_as_float(hmax_bits);
     const float cmax = sqrtf(2.0f * hmax), abs_term = SCR_ERR_ABS * sqrtf((float)d);
+    const float round_term = SCR_ERR_ROUND * 51.0f * (float)((d + 15) / 16);
     v8h xh[NK], xl[NK];
     float ss = 0.0f;
 #pragma unroll
@@ -724,7 +727,8 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
         }
     const float nrm = ss + __shfl_xor(ss, 32, 64);
     if (h == 0 && i0 < n)
-        bounds[i0] = fmaf(SCR_ERR_X * cmax + abs_term, __builtin_amdgcn_sqrtf(nrm), SCR_ERR_H * hmax + abs_term * cmax);
+        bounds[i0] = fmaf((SCR_ERR_SPLIT + round_term) * cmax + abs_term, __builtin_amdgcn_sqrtf(nrm),
+                          round_term * hmax + abs_term * cmax);
     if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = xs;
     for (int cb = 0; cb < n_cb; ++cb) {
         const float4* hp = reinterpret_cast<const float4*>(hneg + cb * 32 + h * 16);
@@ -806,19 +810,26 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,
                                int64_t n, int d, int k, hipStream_t stream) {
-    if (!kmx_mfma_screen_supported(n, d, k)) return KMX_ERR_UNSUPPORTED;
-    const int nk = (d + 15) / 16, n_cb = (k + 31) / 32;
+    if (d < 1 || d > 256 || k < 1 || n >= ((int64_t)1 << 29)) return KMX_ERR_UNSUPPORTED;
+    const int nk16 = (d + 15) / 16;
+    const int nk = nk16 <= 1 ? 1 : nk16 <= 2 ? 2 : nk16 <= 4 ? 4 : nk16 <= 8 ? 8 : 16;
+    const int n_cb = (k + 31) / 32;
     const size_t lds = (size_t)n_cb * nk * 64 * 32 + (size_t)n_cb * 32 * 4;
     if (lds > 64 * 1024) return KMX_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(absmax_fill_zero, dim3(1), dim3(64), 0, stream, scratch);
     hipLaunchKernelGGL(screen_absmax_kernel, dim3(256), dim3(256), 0, stream, X_t, scratch, (int64_t)d * n);
     const unsigned grid = (unsigned)kmx_cdiv(n, 32);
-    if (nk == 1)
-        hipLaunchKernelGGL((screen_scores_kernel<1>), dim3(grid), dim3(64), lds, stream, X_t, centroids_t,
-                           scratch, scores, bounds, half_norms, scale, n, d, k);
-    else
-        hipLaunchKernelGGL((screen_scores_kernel<2>), dim3(grid), dim3(64), lds, stream, X_t, centroids_t,
-                           scratch, scores, bounds, half_norms, scale, n, d, k);
+#define KMX_DIAG_CASE(NK)                                                                               \
+    hipLaunchKernelGGL((screen_scores_kernel<NK>), dim3(grid), dim3(64), lds, stream, X_t, centroids_t, \
+                       scratch, scores, bounds, half_norms, scale, n, d, k)
+    switch (nk) {
+        case 1: KMX_DIAG_CASE(1); break;
+        case 2: KMX_DIAG_CASE(2); break;
+        case 4: KMX_DIAG_CASE(4); break;
+        case 8: KMX_DIAG_CASE(8); break;
+        default: KMX_DIAG_CASE(16); break;
+    }
+#undef KMX_DIAG_CASE
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

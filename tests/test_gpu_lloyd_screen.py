@@ -292,6 +292,12 @@ def _screen_cases():
                             (rng.standard_normal((20, 8)) * 1e-18).astype(np.float32))
     cases["huge values"] = ((rng.standard_normal((1_000, 8)) * 1e16).astype(np.float32),
                             (rng.standard_normal((20, 8)) * 1e16).astype(np.float32))
+    # the wide path's shapes: 16 K steps, centroids = samples (maximal cancellation), and noise
+    X = (rng.standard_normal((1_024, 256)) * 2 + rng.standard_normal(256) * 5).astype(np.float32)
+    cases["d=256, centroids = samples"] = (X, X[:32].copy())
+    cases["d=200 random"] = (rng.standard_normal((1_024, 200)).astype(np.float32) * 7,
+                             rng.standard_normal((32, 200)).astype(np.float32) * 7)
+    cases["d=70"] = (rng.standard_normal((1_024, 70)).astype(np.float32), rng.standard_normal((64, 70)).astype(np.float32))
     return cases
 
 
