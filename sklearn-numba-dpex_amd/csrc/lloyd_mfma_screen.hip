@@ -54,6 +54,7 @@ constexpr float SCR_ERR_SPLIT = 7.2e-7f;  // 3.01 * 2^-22, rounded up
 constexpr float SCR_ERR_ROUND = 1.2e-7f;  // 2^-23, rounded up
 constexpr float SCR_ERR_ABS = 6.2e-5f;    // 2^-14, rounded up
 constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
+constexpr int SCR_REDO_COLUMN = 3;  // uncertain samples from which a 32-sample column is redone in fp32
 
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
 #ifndef KMX_SCR_WAVES
@@ -92,6 +93,45 @@ __device__ __forceinline__ unsigned long long to_fixed_q(double v_plus_magic, do
     unsigned int hi;
     asm("v_sub_u32 %0, %1, %2" : "=v"(hi) : "v"(__double2hiint(v_plus_magic)), "v"(__double2hiint(magic)));
     return ((unsigned long long)hi << 32) | (unsigned int)__double2loint(v_plus_magic);
+}
+
+// One column of 32 samples against all centroids in plain fp32 on the matrix cores
+// (v_mfma_f32_32x32x2_f32 from -0.5||c||^2, lowest index wins a tie): the route for columns with
+// several samples the screen cannot certify.  rows.v[8 s + i] = feature 16 s + 2 i + h of the
+// lane's sample; ct (d, kp) and hx (kp) are the fp32 centroids and half norms in LDS.
+struct ColumnRows {
+    float v[16];
+};
+__device__ __forceinline__ uint32_t redo_column_fp32(ColumnRows rows, const float* ct, const float* hx,
+                                                  int nk, int n_cb, int d, int kp, int h, int j) {
+    float bv = -kmx_inf<float>();
+    int bc = 0x7fffffff;
+    for (int cb = 0; cb < n_cb; ++cb) {
+        v16f a;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) a[r] = -hx[32 * cb + 8 * (r >> 2) + 4 * h + (r & 3)];
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const int p0 = 2 * p;  // features p0 + h; wave-uniform guards
+            if (p < 8 * nk && p0 < d) {
+                const bool ok = p0 + h < d;
+                const float af = ok ? ct[(p0 + h) * kp + 32 * cb + j] : 0.0f;
+                const float xv = ok ? rows.v[p] : 0.0f;
+                a = __builtin_amdgcn_mfma_f32_32x32x2f32(af, xv, a, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r)  // increasing centroid index inside the lane
+            if (a[r] > bv) {
+                bv = a[r];
+                bc = 32 * cb + 8 * (r >> 2) + 4 * h + (r & 3);
+            }
+    }
+    const float ov = __shfl_xor(bv, 32, 64);
+    const int oc = __shfl_xor(bc, 32, 64);
+    if (ov > bv || (ov == bv && oc < bc)) bc = oc;
+    if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
+    return (uint32_t)bc;
 }
 
 template <int NK, bool UPDATE>
@@ -400,11 +440,24 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         // Samples the screen cannot certify: plain fp32, the whole wave on one sample at a
         // time.  Lane l takes the centroids l, l + 64, ... (fused multiply-adds in feature
         // order from -0.5||c||^2, strict '>' in increasing order), then the wave combines.
+        // A column with several such samples (ties between duplicate centroids, degenerate
+        // data) is instead redone as a whole in fp32 on the matrix cores, which bounds the cost
+        // of a tile at about three times the usual one however many samples fail the screen.
 #pragma unroll
         for (int t = 0; t < NC; ++t) {
             unsigned long long todo = __ballot(h == 0 && unsure[t]);  // wave-uniform
-            n_uncertain += (unsigned int)__popcll(todo);
-            while (todo) {
+            const int n_todo = __popcll(todo);
+            n_uncertain += (unsigned int)n_todo;
+            if (__builtin_expect(n_todo >= SCR_REDO_COLUMN, 0)) {  // cold: spills belong in here
+                ColumnRows rows;
+#pragma unroll
+                for (int s = 0; s < NK; ++s)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = x[s][i][t];
+                lab[t] = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
+                todo = 0ull;
+            }
+            while (__builtin_expect(todo != 0ull, 0)) {
                 const int js = __builtin_ctzll(todo);
                 todo &= todo - 1;
                 float xf[16 * NK];

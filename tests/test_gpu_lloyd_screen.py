@@ -367,3 +367,45 @@ def test_wide_screen_switched_off_by_environment(cuda):
         os.environ.pop("KMX_LLOYD_ASSIGN", None)
     assert variant == 42 and rechecked == 0
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+
+
+def test_many_ties_stay_affordable(cuda):
+    """Columns with several uncertifiable samples are redone on the fp32 matrix cores: with every
+    sample of a large input failing the screen, an iteration must stay within a small multiple
+    of the usual time (the per-sample route alone would take tens of times longer)."""
+    import time
+
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    n, d, k = 1_000_000, 14, 127
+    X_t = torch.randn(d, n, device=cuda)
+    w = torch.ones(n, device=cuda)
+
+    def one_iteration_ms(c_in):
+        c_out = torch.empty_like(c_in)
+        lab0 = torch.zeros(n, dtype=torch.int32, device=cuda)
+        lab1 = torch.empty(n, dtype=torch.int32, device=cuda)
+        sizes = torch.empty(k, device=cuda)
+        empty = torch.empty(k, dtype=torch.int32, device=cuda)
+        wsb = lib.kmx_lloyd_workspace_bytes(n, d, k, 0)
+        ws = torch.empty(wsb, dtype=torch.uint8, device=cuda)
+        st = _capi.current_stream()
+        best = 1e9
+        for _ in range(3):
+            _capi.check(lib.kmx_lloyd_init(ptr(ws), wsb, ptr(X_t), ptr(w), ptr(c_in), n, d, k, 0, 10, 0.0, st), "init")
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w), ptr(c_in), ptr(c_out), ptr(lab0), ptr(lab1),
+                                           ptr(sizes), ptr(empty), ptr(ws), wsb, n, d, k, 0, st), "iter")
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        return best, lab1
+
+    usual, _ = one_iteration_ms(torch.randn(d, k, device=cuda))
+    tied, labels = one_iteration_ms(torch.randn(d, 1, device=cuda).repeat(1, k).contiguous())
+    assert int(labels.max()) == 0
+    print(f"usual {usual:.3f} ms, every sample tied {tied:.3f} ms")
+    assert tied < 10 * usual + 0.5
