@@ -101,10 +101,11 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     L.off_bucket = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 32) * sizeof(double));  // one per finalisation workgroup
     // wide matrix-core path: counts (k), offsets (k + 1), sample order (n) and ranks inside the
     // cluster (n) as int32
-    // screened path: the counter of samples evaluated in fp32 and its copy for the host
+    // screened path: the counter of samples evaluated in fp32 and its copy for the host (256
+    // bytes), then ||x_i|| per sample
     const size_t bucket_bytes =
         L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int)
-        : L.screen                         ? (size_t)64 * sizeof(int)
+        : L.screen                         ? (size_t)256 + (size_t)n * sizeof(float)
                                            : 0;
     // wide matrix-core path: header, scaled half norms and fp16 parts of the centroids for the
     // screened label step (lloyd_mfma_wide_screen.hip)
@@ -136,8 +137,9 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    kmx_lloyd_status* status, const unsigned int* absmax,
                                    const int* q_exp, unsigned long long* gsum,
-                                   uint32_t* uncertain_count, int64_t n, int d, int k,
-                                   hipStream_t stream);
+                                   uint32_t* uncertain_count, const float* norms, int64_t n, int d,
+                                   int k, hipStream_t stream);
+int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream);
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,
                                int64_t n, int d, int k, hipStream_t stream);

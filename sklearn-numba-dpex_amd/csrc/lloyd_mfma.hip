@@ -590,6 +590,10 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(1024), 0, stream,
                        reinterpret_cast<unsigned int*>(ws + L.off_gsum), (int)words);
     KMX_LAUNCH_CHECK();
+    // the screened step compares score gaps with a bound proportional to ||x_i||
+    if (L.screen)
+        return kmx_sample_norms((const float*)X_t, reinterpret_cast<float*>(ws + L.off_bucket + 256), n, d,
+                                stream);
     return KMX_OK;
 }
 
@@ -619,8 +623,8 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         tail.clear_word = uncertain;
         const int32_t rc = kmx_lloyd_step_mfma_screen(
             X_t, w, centroids_t, labels_prev, labels, tail.status,
-            reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain, n, d, k,
-            stream);
+            reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain,
+            reinterpret_cast<const float*>(ws + L.off_bucket + 256), n, d, k, stream);
         if (rc != KMX_OK) return rc;
         if (events) {
             (void)hipEventRecord(events[1], stream);

@@ -140,8 +140,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
     const unsigned int* __restrict__ absmax, const int* __restrict__ q_exp,
-    unsigned long long* __restrict__ gsum, uint32_t* __restrict__ uncertain_count, int64_t n,
-    int d, int k, int vec_ok) {
+    unsigned long long* __restrict__ gsum, uint32_t* __restrict__ uncertain_count,
+    const float* __restrict__ norms, int64_t n, int d, int k, int vec_ok) {
     if (UPDATE && status->state != KMX_RUNNING) return;
 
     constexpr int WAVES = scr_waves(NK), THREADS = 64 * WAVES;
@@ -240,7 +240,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     const float hmax = __uint_as_float(hmax_bits);
     const float cmax = sqrtf(2.0f * hmax), abs_term = SCR_ERR_ABS * sqrtf((float)d);
     const float round_term = SCR_ERR_ROUND * 51.0f * (float)NK;
-    const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term);
+    // (||x|| comes unscaled from kmx_lloyd_init, hence the factor xs)
+    const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term) * xs;
     const float thr_0 = 2.01f * (round_term * hmax + abs_term * cmax);
     // +inf the optimiser cannot see through (it would turn the median below into a maximum
     // with two canonicalising instructions in front)
@@ -269,16 +270,15 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     auto process = [&](auto nc_tag, auto full_tag,
                        const float(&x)[NK][8][decltype(nc_tag)::value],
                        const float(&wv)[decltype(nc_tag)::value],
-                       const uint32_t(&pl)[decltype(nc_tag)::value], const int64_t i0) {
+                       const uint32_t(&pl)[decltype(nc_tag)::value],
+                       const float(&xnorm)[decltype(nc_tag)::value], const int64_t i0) {
         constexpr int NC = decltype(nc_tag)::value;
         constexpr bool FULL = decltype(full_tag)::value;
 
-        // scaled fp16 split of the B operand and ||x||^2
+        // scaled fp16 split of the B operand
         v8h xh[NK][NC], xl[NK][NC];
-        float nrm[NC];
 #pragma unroll
         for (int t = 0; t < NC; ++t) {
-            float ss = 0.0f;
 #pragma unroll
             for (int s = 0; s < NK; ++s)
 #pragma unroll
@@ -291,10 +291,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                     xh[s][t][i + 1] = hh[1];
                     xl[s][t][i] = ll[0];
                     xl[s][t][i + 1] = ll[1];
-                    ss = fmaf(p[0], p[0], ss);
-                    ss = fmaf(p[1], p[1], ss);
                 }
-            nrm[t] = ss + __shfl_xor(ss, 32, 64);
         }
 
         // Running arg-max by groups of G accumulator registers, plus the second largest of
@@ -433,7 +430,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             }
             lab[t] = (uint32_t)c;
             // written so that a NaN anywhere makes the sample uncertain
-            const float thr = fmaf(thr_x, __builtin_amdgcn_sqrtf(nrm[t]), thr_0);
+            const float thr = fmaf(thr_x, xnorm[t], thr_0);
             unsure[t] = !(b - s2 > thr) && (FULL || i0 + t < n);
         }
 
@@ -613,6 +610,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             }
             float wv[MC] = {0.f, 0.f};
             uint32_t pl[MC] = {0u, 0u};
+            const float2 n2 = *reinterpret_cast<const float2*>(norms + i0);
+            const float xnorm[MC] = {n2.x, n2.y};
             if (UPDATE) {
                 const float2 w2 = *reinterpret_cast<const float2*>(sample_weight + i0);
                 wv[0] = w2.x;
@@ -621,7 +620,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 pl[0] = p2.x;
                 pl[1] = p2.y;
             }
-            process(Cols2{}, std::true_type{}, x, wv, pl, i0);
+            process(Cols2{}, std::true_type{}, x, wv, pl, xnorm, i0);
         }
     }
     // scalar loads of the lane's rows (row d - 1 where the feature does not exist)
@@ -645,11 +644,12 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             load_scalar(Cols1{}, i0, x);
             float wv[1] = {0.f};
             uint32_t pl[1] = {0u};
+            const float xnorm[1] = {norms[i0]};
             if (UPDATE) {
                 wv[0] = sample_weight[i0];
                 pl[0] = labels_prev[i0];
             }
-            process(Cols1{}, std::true_type{}, x, wv, pl, i0);
+            process(Cols1{}, std::true_type{}, x, wv, pl, xnorm, i0);
         }
     }
     // The rest: a partial last tile, or every tile when vector accesses are not legal
@@ -659,16 +659,18 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         load_scalar(Cols2{}, i0, x);
         float wv[MC];
         uint32_t pl[MC];
+        float xnorm[MC];
 #pragma unroll
         for (int t = 0; t < MC; ++t) {
             wv[t] = 0.f;
             pl[t] = 0u;
+            xnorm[t] = i0 + t < n ? norms[i0 + t] : 0.0f;
             if (UPDATE && i0 + t < n) {
                 wv[t] = sample_weight[i0 + t];
                 pl[t] = labels_prev[i0 + t];
             }
         }
-        process(Cols2{}, std::false_type{}, x, wv, pl, i0);
+        process(Cols2{}, std::false_type{}, x, wv, pl, xnorm, i0);
     }
 
     if (UPDATE && changed) atomicAdd(&changed_block, changed);
@@ -825,13 +827,13 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
 // Screened fused step.  `uncertain_count`: one word the kernel adds the number of samples it
 // evaluated in fp32 to (zero on entry; the finalisation that follows moves it to the next word
 // and clears it).  `absmax`: bits of max|X_t row| per feature, as kmx_lloyd_mfma_prepare leaves
-// them.
+// them; `norms`: ||x_i|| per sample (kmx_sample_norms).
 int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    kmx_lloyd_status* status, const unsigned int* absmax,
                                    const int* q_exp, unsigned long long* gsum,
-                                   uint32_t* uncertain_count, int64_t n, int d, int k,
-                                   hipStream_t stream) {
+                                   uint32_t* uncertain_count, const float* norms, int64_t n, int d,
+                                   int k, hipStream_t stream) {
     if (!kmx_mfma_screen_supported(n, d, k)) return KMX_ERR_UNSUPPORTED;
     const int nk = (d + 15) / 16;
     const int waves = scr_waves(nk);
@@ -848,13 +850,13 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
     if (nk == 1)
         hipLaunchKernelGGL((lloyd_screen_kernel<1, true>), dim3((unsigned)grid), dim3(64 * scr_waves(1)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
-                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, n, d, k,
-                           vec_ok);
+                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, norms, n, d,
+                           k, vec_ok);
     else
         hipLaunchKernelGGL((lloyd_screen_kernel<2, true>), dim3((unsigned)grid), dim3(64 * scr_waves(2)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
-                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, n, d, k,
-                           vec_ok);
+                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, norms, n, d,
+                           k, vec_ok);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
@@ -883,6 +885,29 @@ int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float
         default: KMX_DIAG_CASE(16); break;
     }
 #undef KMX_DIAG_CASE
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+namespace {
+// ||x_i|| in fp32, features in order; one thread per sample (consecutive threads, consecutive
+// addresses in every feature row).
+__global__ __launch_bounds__(256) void sample_norms_kernel(const float* __restrict__ X_t,
+                                                           float* __restrict__ norms, int64_t n, int d) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float sq = 0.0f;
+#pragma unroll 8
+    for (int f = 0; f < d; ++f) {
+        const float v = X_t[(size_t)f * n + i];
+        sq = fmaf(v, v, sq);
+    }
+    norms[i] = sqrtf(sq);
+}
+}  // namespace
+
+int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream) {
+    hipLaunchKernelGGL(sample_norms_kernel, dim3((unsigned)kmx_cdiv(n, 256)), dim3(256), 0, stream, X_t, norms, n, d);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

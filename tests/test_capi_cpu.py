@@ -58,7 +58,8 @@ def test_workspace_queries():
 
     small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0)
     assert 0 < small < 64 << 20
-    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) == small  # independent of n
+    # the screened fp32 step keeps ||x_i|| per sample: 4 bytes per sample
+    assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) - small - 4 * 4_900_000) < 256
     assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1)
     assert lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0) > (32 << 20)  # global copies
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0) == 0

@@ -324,10 +324,11 @@ def test_dlpack_inputs_give_the_same_fit(cuda, dtype):
         b = KMeans(n_clusters=7, init=init, n_init=1, max_iter=20, tol=0).fit(
             _DLPackOnly(torch.as_tensor(X, device=cuda)), sample_weight=_DLPackOnly(torch.as_tensor(w, device=cuda)))
     np.testing.assert_array_equal(a.labels_, b.labels_)
+    # this small shape runs the vector-ALU kernel, whose sums go through floating-point LDS
+    # atomics in an order that varies from run to run (only the matrix-core fp32 kernels, with
+    # their fixed-point sums, are bit-reproducible: tests/test_gpu_full_size.py checks that)
     if dtype == np.float32:
-        # fixed-point sums: the fit is bit-reproducible
-        np.testing.assert_array_equal(a.cluster_centers_, b.cluster_centers_)
+        np.testing.assert_allclose(a.cluster_centers_, b.cluster_centers_, rtol=2e-6, atol=1e-6)
     else:
-        # fp64 sums go through floating-point LDS atomics, whose order varies from run to run
         np.testing.assert_allclose(a.cluster_centers_, b.cluster_centers_, rtol=1e-12, atol=1e-13)
     assert a.n_iter_ == b.n_iter_
