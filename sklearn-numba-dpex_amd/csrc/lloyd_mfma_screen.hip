@@ -397,22 +397,28 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 sv[2 * r] = pr.x;
                 sv[2 * r + 1] = pr.y;
             }
-            // registers equal to the best: the lowest is the label's; a second one makes the
-            // second best equal to the best
-            unsigned int pos = G - 1, n_eq = 0;
-            float rest[G];
+            // the lowest register equal to the best is the label's
+            unsigned int pos = G - 1;
 #pragma unroll
-            for (int r = G - 1; r >= 0; --r) {
-                const bool eq = sv[r] == best[t];
-                pos = eq ? (unsigned int)r : pos;
-                n_eq += eq ? 1u : 0u;
-                rest[r] = eq ? neg_inf : sv[r];
-            }
-            float sec = second[t];
-#pragma unroll
-            for (int r = 0; r + 1 < G; r += 2)
-                asm("v_max3_f32 %0, %1, %2, %3" : "=v"(sec) : "v"(sec), "v"(rest[r]), "v"(rest[r + 1]));
-            sec = n_eq > 1u ? best[t] : sec;
+            for (int r = G - 2; r >= 0; --r) pos = (sv[r] == best[t]) ? (unsigned int)r : pos;
+            // Second largest of the eight (equal to the largest if that occurs twice), by a
+            // tournament of (largest, second) pairs: triples give max3 / med3, and two pairs
+            // merge into (max(m, m'), max3(min(m, m'), s, s')).
+            float mA, sA, mB, sB, mC, sC, mL, mAB, sAB, sG;
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mA) : "v"(sv[0]), "v"(sv[1]), "v"(sv[2]));
+            asm("v_med3_f32 %0, %1, %2, %3" : "=v"(sA) : "v"(sv[0]), "v"(sv[1]), "v"(sv[2]));
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mB) : "v"(sv[3]), "v"(sv[4]), "v"(sv[5]));
+            asm("v_med3_f32 %0, %1, %2, %3" : "=v"(sB) : "v"(sv[3]), "v"(sv[4]), "v"(sv[5]));
+            asm("v_max_f32 %0, %1, %2" : "=v"(mC) : "v"(sv[6]), "v"(sv[7]));
+            asm("v_min_f32 %0, %1, %2" : "=v"(sC) : "v"(sv[6]), "v"(sv[7]));
+            asm("v_min_f32 %0, %1, %2" : "=v"(mL) : "v"(mA), "v"(mB));
+            asm("v_max_f32 %0, %1, %2" : "=v"(mAB) : "v"(mA), "v"(mB));
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(sAB) : "v"(mL), "v"(sA), "v"(sB));
+            asm("v_min_f32 %0, %1, %2" : "=v"(mL) : "v"(mAB), "v"(mC));
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(sG) : "v"(mL), "v"(sAB), "v"(sC));
+            // and the second largest of the other groups' maxima
+            float sec;
+            asm("v_max_f32 %0, %1, %2" : "=v"(sec) : "v"(sG), "v"(second[t]));
             const unsigned int reg = (code[t] % NG) * G + pos;
             const unsigned int blk = code[t] / NG;
             int c = (int)(32 * blk + 8 * (reg >> 2) + 4 * h + (reg & 3));
