@@ -72,7 +72,8 @@ struct ScreenLds {
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
     const size_t n_cb = (size_t)(k + 31) / 32;
-    const size_t acc = update ? (((size_t)(d + 1) * k * 8 + 15) & ~(size_t)15) : 0;
+    // sums: the feature rows, a spare row when d is odd, then the row of the cluster sizes
+    const size_t acc = update ? (((size_t)(((d + 1) & ~1) + 1) * k * 8 + 15) & ~(size_t)15) : 0;
     s.off_afh = acc;
     s.off_afl = s.off_afh + n_cb * nk * 64 * 16;
     s.off_hneg = s.off_afl + n_cb * nk * 64 * 16;
@@ -149,9 +150,13 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     constexpr int G = SCR_GROUP, NG = 16 / SCR_GROUP;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int n_cb = (k + 31) >> 5;
-    const int items = (d + 1) * k;
+    // Accumulator rows: feature f in row f, the cluster sizes in row d_even.  For odd d the row
+    // between them takes what the upper half-wave adds for the feature that does not exist
+    // (never read), so that the update needs neither a select nor a guard per lane.
+    const int d_even = (d + 1) & ~1;
+    const int items = (d_even + 1) * k;
     const ScreenLds lay = screen_lds(d, k, NK, UPDATE);
-    unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [(d + 1) * k]
+    unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [(d_even + 1) * k]
     v8h* afh = reinterpret_cast<v8h*>(smem_raw + lay.off_afh);                  // [n_cb][NK][64]
     v8h* afl = reinterpret_cast<v8h*>(smem_raw + lay.off_afl);
     float* hneg = reinterpret_cast<float*>(smem_raw + lay.off_hneg);            // [n_cb][2][16]
@@ -231,6 +236,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, j = lane & 31;
+    const unsigned int h4 = 4u * (unsigned int)h;
     const int n_wtiles = (int)((n + TILE - 1) / TILE);  // n < 2^29: tile and sample indices fit 32 bits
     unsigned int changed = 0;
     unsigned int n_uncertain = 0;  // wave-uniform
@@ -397,10 +403,14 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 sv[2 * r] = pr.x;
                 sv[2 * r + 1] = pr.y;
             }
-            // the lowest register equal to the best is the label's
-            unsigned int pos = G - 1;
+            // The lowest register equal to the best is the label's.  Register r of group g of
+            // block b holds centroid 32 b + 16 g + 8 (r / 4) + 4 h + r % 4 (G = 8): the chain
+            // selects 8 (r / 4) + r % 4 directly.
+            static_assert(G == 8 && NG == 2, "centroid index below assumes two groups of eight");
+            unsigned int pos = 8 * ((G - 1) >> 2) + ((G - 1) & 3);
 #pragma unroll
-            for (int r = G - 2; r >= 0; --r) pos = (sv[r] == best[t]) ? (unsigned int)r : pos;
+            for (int r = G - 2; r >= 0; --r)
+                pos = (sv[r] == best[t]) ? (unsigned int)(8 * (r >> 2) + (r & 3)) : pos;
             // Second largest of the eight (equal to the largest if that occurs twice), by a
             // tournament of (largest, second) pairs: triples give max3 / med3, and two pairs
             // merge into (max(m, m'), max3(min(m, m'), s, s')).
@@ -419,22 +429,23 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             // and the second largest of the other groups' maxima
             float sec;
             asm("v_max_f32 %0, %1, %2" : "=v"(sec) : "v"(sG), "v"(second[t]));
-            const unsigned int reg = (code[t] % NG) * G + pos;
-            const unsigned int blk = code[t] / NG;
-            int c = (int)(32 * blk + 8 * (reg >> 2) + 4 * h + (reg & 3));
-            const float ov = __shfl_xor(best[t], 32, 64);
-            const float o2 = __shfl_xor(sec, 32, 64);
-            const int oc = __shfl_xor(c, 32, 64);
+            const unsigned int c_mine = (code[t] << 4) + pos + h4;
+            // Both half-waves see both halves' results (one register swap each, no LDS traffic
+            // that would queue behind the accumulator atomics) and combine them identically.
+            const auto bb = __builtin_amdgcn_permlane32_swap(__float_as_uint(best[t]),
+                                                             __float_as_uint(best[t]), false, false);
+            const auto ss = __builtin_amdgcn_permlane32_swap(__float_as_uint(sec), __float_as_uint(sec),
+                                                             false, false);
+            const auto cc = __builtin_amdgcn_permlane32_swap(c_mine, c_mine, false, false);
+            const float b_lo = __uint_as_float(bb[0]), b_hi = __uint_as_float(bb[1]);
             // second best over both halves: the loser of the two bests or a half's own second
-            float s2 = sec > o2 ? sec : o2;
-            const float lo_best = ov < best[t] ? ov : best[t];
-            s2 = lo_best > s2 ? lo_best : s2;
-            float b = best[t];
-            if (ov > b || (ov == b && oc < c)) {
-                c = oc;
-                b = ov;
-            }
-            lab[t] = (uint32_t)c;
+            float s2, b;
+            asm("v_min_f32 %0, %1, %2" : "=v"(s2) : "v"(b_lo), "v"(b_hi));
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(s2) : "v"(s2), "v"(__uint_as_float(ss[0])), "v"(__uint_as_float(ss[1])));
+            asm("v_max_f32 %0, %1, %2" : "=v"(b) : "v"(b_lo), "v"(b_hi));
+            // the lower centroid index wins a tie between the halves
+            const bool take_hi = b_hi > b_lo || (b_hi == b_lo && cc[1] < cc[0]);
+            lab[t] = take_hi ? cc[1] : cc[0];
             // written so that a NaN anywhere makes the sample uncertain
             const float thr = fmaf(thr_x, xnorm[t], thr_0);
             unsure[t] = !(b - s2 > thr) && (FULL || i0 + t < n);
@@ -526,12 +537,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 for (int i = 0; i < 8; ++i) {
                     const int p0 = 16 * s + 2 * i;  // the pair's even feature
                     if (p0 < d) {                   // wave-uniform
-                        // odd d, last pair: the upper half-wave adds zero to row d - 1
-                        const bool odd_tail = p0 + 1 == d;
-                        unsigned long long* rowacc = acc + (odd_tail ? p0 : p0 + h) * k;
+                        // (odd d, last pair: the upper half-wave adds to the spare row)
+                        unsigned long long* rowacc = acc + (p0 + h) * k;
 #pragma unroll
                         for (int t = 0; t < NC; ++t) {
-                            const double xd = (double)((odd_tail && h) ? 0.0f : x[s][i][t]);
+                            const double xd = (double)x[s][i][t];
                             // x * w is exact in fp64; one rounding, to a multiple of 2^-q
                             const double v = fma(xd, wd[t], magic[s][i]);
                             atomicAdd(rowacc + lab[t], to_fixed_q(v, magic[s][i]));
@@ -539,7 +549,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                     }
                 }
             if (h == 0) {
-                unsigned long long* szacc = acc + d * k;
+                unsigned long long* szacc = acc + d_even * k;
 #pragma unroll
                 for (int t = 0; t < NC; ++t)
                     atomicAdd(szacc + lab[t], to_fixed_q(wd[t] + magic_w, magic_w));
@@ -685,8 +695,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     if (threadIdx.x == 0 && uncertain_block) atomicAdd(uncertain_count, uncertain_block);
     if (UPDATE) {
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
-        for (int jx = threadIdx.x; jx < items; jx += THREADS) {
-            const unsigned long long v = acc[jx];
+        const int n_out = (d + 1) * k, skip = (d_even - d) * k;  // gsum has no spare row
+        for (int jx = threadIdx.x; jx < n_out; jx += THREADS) {
+            const unsigned long long v = acc[jx < d * k ? jx : jx + skip];
             if (v) atomicAdd(gsum + jx, v);
         }
     }
