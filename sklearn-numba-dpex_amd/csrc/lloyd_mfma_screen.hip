@@ -66,9 +66,13 @@ constexpr int SCR_REDO_COLUMN = 3;  // uncertain samples from which a 32-sample 
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
 
 struct ScreenLds {
-    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, total;
-    int kp;  // centroids rounded up to a multiple of 64
+    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, off_queue, total;
+    int kp;       // centroids rounded up to a multiple of 64
+    int q_cap;    // entries of the queue of samples the screen could not certify
+    int q_words;  // 32-bit words per entry: 16 nk feature values, weight, sample index, old label
 };
+constexpr int SCR_QUEUE_MAX = 256;
+constexpr size_t SCR_LDS_MAX = 64 * 1024;
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
     const size_t n_cb = (size_t)(k + 31) / 32;
@@ -80,7 +84,13 @@ __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool updat
     s.kp = (k + 63) & ~63;
     s.off_ct = s.off_hneg + n_cb * 32 * 4;             // fp32 centroids, (d, kp)
     s.off_hx = s.off_ct + (size_t)d * s.kp * 4;        // fp32 0.5||c||^2, (kp), +inf past k
-    s.total = s.off_hx + (size_t)s.kp * 4;
+    s.off_queue = s.off_hx + (size_t)s.kp * 4;
+    // the queue takes what is left of the 64 KB, up to SCR_QUEUE_MAX entries (none: every
+    // uncertain sample is then handled where it turns up)
+    s.q_words = 16 * nk + 4;
+    const size_t room = s.off_queue < SCR_LDS_MAX ? (SCR_LDS_MAX - s.off_queue) / ((size_t)s.q_words * 4) : 0;
+    s.q_cap = (int)(room < (size_t)SCR_QUEUE_MAX ? room : (size_t)SCR_QUEUE_MAX);
+    s.total = s.off_queue + (size_t)s.q_cap * s.q_words * 4;
     return s;
 }
 
@@ -163,6 +173,14 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     float* ct = reinterpret_cast<float*>(smem_raw + lay.off_ct);                // [d][kp]
     float* hx = reinterpret_cast<float*>(smem_raw + lay.off_hx);                // [kp]
     const int kp = lay.kp;
+    // Queue of the samples the screen could not certify, evaluated in fp32 by the whole
+    // workgroup after the last tile: per entry the 16 NK feature values in feature order, the
+    // weight, the sample index (QUEUE_FREE: never written) and the previous label.
+    uint32_t* queue = reinterpret_cast<uint32_t*>(smem_raw + lay.off_queue);    // [q_cap][q_words]
+    const int q_cap = lay.q_cap;
+    constexpr int QW = 16 * NK + 4, Q_WEIGHT = 16 * NK, Q_INDEX = 16 * NK + 1, Q_PREV = 16 * NK + 2;
+    constexpr uint32_t QUEUE_FREE = 0xffffffffu;
+    __shared__ unsigned int queue_count;
     __shared__ unsigned int changed_block;
     __shared__ unsigned int hmax_bits;
     __shared__ unsigned int uncertain_block;
@@ -170,6 +188,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 
     if (threadIdx.x == 0) {
         changed_block = 0;
+        queue_count = 0;
         hmax_bits = 0;
         uncertain_block = 0;
     }
@@ -232,6 +251,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     }
     if (UPDATE)
         for (int jx = threadIdx.x; jx < items; jx += THREADS) acc[jx] = 0ull;
+    for (int e = threadIdx.x; e < q_cap; e += THREADS) queue[e * QW + Q_INDEX] = QUEUE_FREE;
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -451,63 +471,52 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             unsure[t] = !(b - s2 > thr) && (FULL || i0 + t < n);
         }
 
-        // Samples the screen cannot certify: plain fp32, the whole wave on one sample at a
-        // time.  Lane l takes the centroids l, l + 64, ... (fused multiply-adds in feature
-        // order from -0.5||c||^2, strict '>' in increasing order), then the wave combines.
-        // A column with several such samples (ties between duplicate centroids, degenerate
-        // data) is instead redone as a whole in fp32 on the matrix cores, which bounds the cost
-        // of a tile at about three times the usual one however many samples fail the screen.
+        // Samples the screen cannot certify go to the workgroup's queue with weight zero here
+        // (their label below is provisional and adds nothing); the queue is worked off in
+        // plain fp32 after the last tile, by all waves alike, so that no wave is held up by
+        // the samples it happens to meet.  A column with several such samples (ties between
+        // duplicate centroids, degenerate data), or one that finds the queue full, is instead
+        // redone as a whole in fp32 on the matrix cores, which bounds the cost of a tile at
+        // about three times the usual one however many samples fail the screen.
+        float wl[NC];
+        bool counted[NC];
 #pragma unroll
         for (int t = 0; t < NC; ++t) {
-            unsigned long long todo = __ballot(h == 0 && unsure[t]);  // wave-uniform
-            const int n_todo = __popcll(todo);
-            n_uncertain += (unsigned int)n_todo;
-            if (__builtin_expect(n_todo >= SCR_REDO_COLUMN, 0)) {  // cold: spills belong in here
-                ColumnRows rows;
-#pragma unroll
-                for (int s = 0; s < NK; ++s)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = x[s][i][t];
-                lab[t] = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
-                todo = 0ull;
-            }
-            while (__builtin_expect(todo != 0ull, 0)) {
-                const int js = __builtin_ctzll(todo);
-                todo &= todo - 1;
-                float xf[16 * NK];
-#pragma unroll
-                for (int s = 0; s < NK; ++s)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        const int bits = __float_as_int(x[s][i][t]);
-                        xf[16 * s + 2 * i] = __int_as_float(__builtin_amdgcn_readlane(bits, js));
-                        xf[16 * s + 2 * i + 1] = __int_as_float(__builtin_amdgcn_readlane(bits, js + 32));
-                    }
-                float bs = neg_inf;
-                int bc = 0x7fffffff;
-                for (int c = lane; c < kp; c += 64) {
-                    float sc = -hx[c];
-#pragma unroll
-                    for (int f = 0; f < 16 * NK; ++f)
-                        if (f < d) sc = fmaf(xf[f], ct[f * kp + c], sc);  // wave-uniform guard
-                    if (sc > bs) {
-                        bs = sc;
-                        bc = c;
-                    }
+            wl[t] = wv[t];
+            counted[t] = FULL || i0 + t < n;
+            const unsigned long long todo = __ballot(h == 0 && unsure[t]);  // wave-uniform
+            if (__builtin_expect(todo != 0ull, 0)) {  // cold: spills belong in here
+                const int n_todo = __popcll(todo);
+                n_uncertain += (unsigned int)n_todo;
+                bool redo = n_todo >= SCR_REDO_COLUMN;
+                unsigned int base = 0;
+                if (!redo) {
+                    if (lane == 0) base = atomicAdd(&queue_count, (unsigned int)n_todo);
+                    base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
+                    redo = base + (unsigned int)n_todo > (unsigned int)q_cap;
                 }
-                // one 64-bit key per lane, (score in an order-preserving integer form, ~index):
-                // the largest key is the best score, the lowest index among equal scores; the
-                // wave's LDS word takes the maximum (LDS operations of a wave execute in order)
-                const unsigned int sb = __float_as_uint(bs);
-                const unsigned int ordered = sb ^ ((sb >> 31) ? 0xffffffffu : 0x80000000u);
-                const unsigned long long key = ((unsigned long long)ordered << 32) | (unsigned int)~bc;
-                if (lane == 0) wave_key[wave] = 0ull;
-                __builtin_amdgcn_wave_barrier();  // keeps the three accesses in this order
-                atomicMax(&wave_key[wave], key);
-                __builtin_amdgcn_wave_barrier();
-                bc = (int)~(unsigned int)*(volatile unsigned long long*)&wave_key[wave];
-                if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
-                if (j == js) lab[t] = (uint32_t)bc;
+                if (redo) {
+                    ColumnRows rows;
+#pragma unroll
+                    for (int s = 0; s < NK; ++s)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = x[s][i][t];
+                    lab[t] = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
+                } else if (((unsigned int)todo >> j) & 1u) {  // both lanes of the sample
+                    const unsigned int slot = base + (unsigned int)__popc((unsigned int)todo & ((1u << j) - 1u));
+                    uint32_t* entry = queue + slot * QW;
+#pragma unroll
+                    for (int s = 0; s < NK; ++s)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) entry[16 * s + 2 * i + h] = __float_as_uint(x[s][i][t]);
+                    if (h == 0) {
+                        entry[Q_WEIGHT] = __float_as_uint(wv[t]);
+                        entry[Q_INDEX] = (uint32_t)(i0 + t);
+                        entry[Q_PREV] = pl[t];
+                    }
+                    wl[t] = 0.0f;
+                    counted[t] = false;
+                }
             }
         }
 
@@ -525,12 +534,12 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             if (h == 0) {
 #pragma unroll
                 for (int t = 0; t < NC; ++t)
-                    changed += ((FULL || i0 + t < n) && pl[t] != lab[t]) ? 1u : 0u;
+                    changed += (counted[t] && pl[t] != lab[t]) ? 1u : 0u;
             }
             // samples past the end carry w = 0: they add zero
             double wd[NC];
 #pragma unroll
-            for (int t = 0; t < NC; ++t) wd[t] = (double)wv[t];
+            for (int t = 0; t < NC; ++t) wd[t] = (double)wl[t];
 #pragma unroll
             for (int s = 0; s < NK; ++s)
 #pragma unroll
@@ -689,6 +698,90 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         process(Cols2{}, std::false_type{}, x, wv, pl, xnorm, i0);
     }
 
+    // The queue: one wave per entry, lane l on the centroids l, l + 64, ... (fused multiply-adds
+    // in feature order from -0.5||c||^2, strict '>' in increasing order), then the wave combines.
+    __syncthreads();  // entries complete; provisional labels have reached memory
+    {
+        const int n_queued = (int)min(queue_count, (unsigned int)q_cap);
+        double magic_lane = 0.0;  // lane f: of feature f; lane d: of the weights
+        if (UPDATE && n_queued > 0) magic_lane = fix_magic(q_exp[lane < d ? lane : d]);
+        for (int e = wave; e < n_queued; e += WAVES) {
+            const uint32_t* entry = queue + e * QW;
+            const uint32_t sample = entry[Q_INDEX];
+            if (sample == QUEUE_FREE) continue;  // reserved by a column that was redone instead
+            const float* xe = reinterpret_cast<const float*>(entry);
+            float bs = neg_inf;
+            int bc = 0x7fffffff;
+            // Two centroids per lane and pass, the features in batches of 8, 4, 2, 1 whose LDS
+            // reads are in flight together; the additions stay in feature order.
+            for (int c = lane; c < kp; c += 128) {
+                const bool two = c + 64 < kp;  // wave-uniform: kp is a multiple of 64
+                const int c1 = two ? c + 64 : c;
+                const float* col0 = ct + c;
+                const float* col1 = ct + c1;
+                float s0 = -hx[c], s1 = -hx[c1];
+                auto batch = [&](auto nb_tag, const int f0) {
+                    constexpr int NB = decltype(nb_tag)::value;
+                    float xv[NB], a0[NB], a1[NB];
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        xv[i] = xe[f0 + i];
+                        a0[i] = col0[(f0 + i) * kp];
+                        a1[i] = col1[(f0 + i) * kp];
+                    }
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        s0 = fmaf(xv[i], a0[i], s0);
+                        s1 = fmaf(xv[i], a1[i], s1);
+                    }
+                };
+                int f = 0;
+                for (; f + 8 <= d; f += 8) batch(std::integral_constant<int, 8>{}, f);
+                if (f + 4 <= d) {
+                    batch(std::integral_constant<int, 4>{}, f);
+                    f += 4;
+                }
+                if (f + 2 <= d) {
+                    batch(std::integral_constant<int, 2>{}, f);
+                    f += 2;
+                }
+                if (f < d) batch(std::integral_constant<int, 1>{}, f);
+                if (s0 > bs) {
+                    bs = s0;
+                    bc = c;
+                }
+                if (two && s1 > bs) {
+                    bs = s1;
+                    bc = c1;
+                }
+            }
+            // one 64-bit key per lane, (score in an order-preserving integer form, ~index):
+            // the largest key is the best score, the lowest index among equal scores; the
+            // wave's LDS word takes the maximum (LDS operations of a wave execute in order)
+            const unsigned int sb = __float_as_uint(bs);
+            const unsigned int ordered = sb ^ ((sb >> 31) ? 0xffffffffu : 0x80000000u);
+            const unsigned long long key = ((unsigned long long)ordered << 32) | (unsigned int)~bc;
+            if (lane == 0) wave_key[wave] = 0ull;
+            __builtin_amdgcn_wave_barrier();  // keeps the three accesses in this order
+            atomicMax(&wave_key[wave], key);
+            __builtin_amdgcn_wave_barrier();
+            bc = (int)~(unsigned int)*(volatile unsigned long long*)&wave_key[wave];
+            if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
+            if (lane == 0) {
+                labels[sample] = (uint32_t)bc;
+                if (UPDATE) changed += entry[Q_PREV] != (uint32_t)bc ? 1u : 0u;
+            }
+            if (UPDATE) {
+                // lane f adds feature f, lane d the weight: the same fixed-point terms as above
+                const double wq = (double)__uint_as_float(entry[Q_WEIGHT]);
+                if (lane <= d) {
+                    const double term = lane < d ? fma((double)xe[lane], wq, magic_lane) : wq + magic_lane;
+                    atomicAdd(acc + (lane < d ? lane : d_even) * k + bc, to_fixed_q(term, magic_lane));
+                }
+            }
+        }
+    }
+
     if (UPDATE && changed) atomicAdd(&changed_block, changed);
     if (lane == 0 && n_uncertain) atomicAdd(&uncertain_block, n_uncertain);
     __syncthreads();
@@ -838,7 +931,7 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
     if (d < 1 || d > 32 || k < 16 || n >= ((int64_t)1 << 29)) return false;
     const char* v = std::getenv("KMX_LLOYD_ASSIGN");
     if (v != nullptr && std::strcmp(v, "f32") == 0) return false;
-    return screen_lds(d, k, (d + 15) / 16, true).total <= 64 * 1024;
+    return screen_lds(d, k, (d + 15) / 16, true).off_queue <= SCR_LDS_MAX;
 }
 
 // Screened fused step.  `uncertain_count`: one word the kernel adds the number of samples it
