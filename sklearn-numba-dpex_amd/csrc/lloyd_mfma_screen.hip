@@ -60,9 +60,6 @@ constexpr int SCR_REDO_COLUMN = 3;  // uncertain samples from which a 32-sample 
 #ifndef KMX_SCR_WAVES
 #define KMX_SCR_WAVES 12
 #endif
-#ifndef KMX_SCR_PREFETCH
-#define KMX_SCR_PREFETCH false
-#endif
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
 
 struct ScreenLds {
@@ -186,28 +183,43 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     __shared__ unsigned int uncertain_block;
     __shared__ unsigned long long wave_key[WAVES];
 
+    __shared__ unsigned int xmax_bits;
+    __shared__ unsigned int tile_ticket;
     if (threadIdx.x == 0) {
+        tile_ticket = 0;
         changed_block = 0;
         queue_count = 0;
         hmax_bits = 0;
         uncertain_block = 0;
+        xmax_bits = 0;
     }
-    // 2^-a with max|x| * 2^-a in [2^14, 2^15) (1 for all-zero or non-finite data)
-    float xmax = 0.0f;
-    for (int f = 0; f < d; ++f) xmax = fmaxf(xmax, __uint_as_float(absmax[f]));
-    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, 14 - ilogbf(xmax)) : 1.0f;
+    // Everything below is derived from one pass over the centroids in memory: row f goes to
+    // wave f % WAVES, all its loads are in flight together, and the fragments and norms are
+    // then computed from the copy in LDS.
+    {
+        const int lane_ = threadIdx.x & 63, wave_ = threadIdx.x >> 6;
+        const unsigned int my_absmax = threadIdx.x < d ? absmax[threadIdx.x] : 0u;
+        for (int f = wave_; f < d; f += WAVES)
+            for (int c = lane_; c < kp; c += 64) ct[f * kp + c] = c < k ? centroids_t[(size_t)f * k + c] : 0.0f;
+        __syncthreads();  // the shared words above are zero
+        // (non-negative floats order like their bits)
+        if (threadIdx.x < d) atomicMax(&xmax_bits, my_absmax);
+    }
     __syncthreads();
+    // 2^-a with max|x| * 2^-a in [2^14, 2^15) (1 for all-zero or non-finite data)
+    const float xmax = __uint_as_float(xmax_bits);
+    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, 14 - ilogbf(xmax)) : 1.0f;
     // A operand: hi and lo parts of 32 centroids x 16 features per block and K step
     for (int idx = threadIdx.x; idx < n_cb * NK * 64; idx += THREADS) {
         const int l = idx & 63;
         const int s = (idx >> 6) % NK;
         const int cb = (idx >> 6) / NK;
-        const int c = 32 * cb + (l & 31);
+        const int c = 32 * cb + (l & 31);  // < kp; zero in ct from k on
         v8h hi, lo;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int f = 16 * s + 2 * i + (l >> 5);
-            const float v = (c < k && f < d) ? centroids_t[(size_t)f * k + c] * xs : 0.0f;
+            const float v = f < d ? ct[f * kp + c] * xs : 0.0f;
             const _Float16 hb = (_Float16)v;
             hi[i] = hb;
             lo[i] = (_Float16)(v - (float)hb);
@@ -222,7 +234,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         if (c < k) {
             float sq = 0.0f;
             for (int f = 0; f < d; ++f) {
-                const float cv = centroids_t[(size_t)f * k + c] * xs;
+                const float cv = ct[f * kp + c] * xs;
                 sq += cv * cv;
             }
             v = -(sq / 2.0f);
@@ -232,17 +244,13 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         }
         hneg[idx] = v;
     }
-    // unscaled fp32 copies for the samples the screen cannot certify
-    for (int idx = threadIdx.x; idx < d * kp; idx += THREADS) {
-        const int f = idx / kp, c = idx - f * kp;
-        ct[idx] = c < k ? centroids_t[(size_t)f * k + c] : 0.0f;
-    }
+    // unscaled half norms for the samples the screen cannot certify
     for (int c = threadIdx.x; c < kp; c += THREADS) {
         float v = kmx_inf<float>();
         if (c < k) {
             float sq = 0.0f;
             for (int f = 0; f < d; ++f) {
-                const float cv = centroids_t[(size_t)f * k + c];
+                const float cv = ct[f * kp + c];
                 sq += cv * cv;
             }
             v = sq / 2.0f;
@@ -614,25 +622,25 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             }
     };
 
-    if (wt_first < n_main) {
-        constexpr bool PREFETCH = KMX_SCR_PREFETCH;
-        float xn[PREFETCH ? NK : 1][8][MC];
-        if constexpr (PREFETCH) load_rows(wt_first, xn);
-        for (int wt = wt_first; wt < n_main; wt += wt_step) {
+    // The workgroup's full tiles (tile WAVES * blockIdx.x + q % WAVES of round q / WAVES) are
+    // handed out through a ticket counter in LDS: the waves of a workgroup do not advance at
+    // the same pace, and with fixed shares the fastest would wait a fifth of the time for the
+    // slowest at the end.  The next ticket is drawn before the current tile is worked on.
+    if (n_main > 0) {
+        auto draw = [&]() {
+            unsigned int ticket = 0;
+            if (lane == 0) ticket = atomicAdd(&tile_ticket, 1u);
+            return ticket;  // valid in lane 0
+        };
+        unsigned int ticket = draw();
+        for (;;) {
+            const int q = __builtin_amdgcn_readfirstlane((int)ticket);
+            const int wt = (int)blockIdx.x * WAVES + q % WAVES + (q / WAVES) * wt_step;
+            if (wt >= n_main) break;  // every wave gets here: the counter only grows
+            ticket = draw();
             const int64_t i0 = (int64_t)wt * TILE + MC * j;
             float x[NK][8][MC];
-            if constexpr (PREFETCH) {
-#pragma unroll
-                for (int s = 0; s < NK; ++s)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i)
-#pragma unroll
-                        for (int t = 0; t < MC; ++t) x[s][i][t] = xn[s][i][t];
-                // past the last tile the same rows are read again (and not used)
-                load_rows(wt + wt_step < n_main ? wt + wt_step : wt, xn);
-            } else {
-                load_rows(wt, x);
-            }
+            load_rows(wt, x);
             float wv[MC] = {0.f, 0.f};
             uint32_t pl[MC] = {0u, 0u};
             const float2 n2 = *reinterpret_cast<const float2*>(norms + i0);
@@ -789,7 +797,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     if (UPDATE) {
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
         const int n_out = (d + 1) * k, skip = (d_even - d) * k;  // gsum has no spare row
-        for (int jx = threadIdx.x; jx < n_out; jx += THREADS) {
+        // every workgroup starts at another word: the workgroups finish together and would
+        // otherwise queue up on the same addresses
+        const int rot = (int)(((int64_t)blockIdx.x * n_out) / gridDim.x);
+        for (int jy = threadIdx.x; jy < n_out; jy += THREADS) {
+            const int jx = jy + rot < n_out ? jy + rot : jy + rot - n_out;
             const unsigned long long v = acc[jx < d * k ? jx : jx + skip];
             if (v) atomicAdd(gsum + jx, v);
         }
