@@ -153,6 +153,28 @@ def test_samples_on_the_bisector(cuda):
     assert rechecked >= on.size
 
 
+def test_more_uncertain_samples_than_the_queue_holds(cuda):
+    """Two samples of every 32-sample column lie on the bisector of centroids 0 and 1: too few
+    for the column to be redone as a whole, so they go to the workgroup's queue, and with
+    512 of them per workgroup the queue (256 entries at most) overflows.  Labels, weighted sums
+    and sizes must come out the same whichever route a sample took."""
+    rng = np.random.default_rng(29)
+    n, d, k = 1 << 21, 4, 16
+    init = rng.uniform(-4, 4, (k, d)).astype(np.float32)
+    init[1] = init[0]
+    init[1, 0] = -init[0, 0]
+    X = (init[rng.integers(0, k, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32)
+    on = np.arange(0, n, 16)
+    X[on] = init[0] + 0.05 * rng.standard_normal((on.size, d)).astype(np.float32)
+    X[on, 0] = 0.0
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 61
+    assert np.all(labels[on] == 0)
+    assert rechecked >= on.size
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+
+
 def test_features_of_very_different_scale(cuda):
     """One feature 1e6 times larger than the one that separates the clusters: the fp16 parts
     of the small feature are far below those of the large one."""
