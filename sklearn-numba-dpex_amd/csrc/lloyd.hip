@@ -946,6 +946,8 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     char* ws = (char*)workspace;
     const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32) {
+        // labels screened on the fp16 matrix cores: one kernel, straight from the centroids
+        if (L.screen) return kmx_assign_labels_mfma_screen(X_t, centroids_t, labels, n, d, k, stream);
         hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
                            (const float*)centroids_t, (float*)(ws + L.off_cpack),
                            (float*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,

@@ -139,6 +139,9 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, const float* norms, int64_t n, int d,
                                    int k, hipStream_t stream);
+// labels only, screened the same way (scale from the centroids, norms taken per tile)
+int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
+                                      int64_t n, int d, int k, hipStream_t stream);
 int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream);
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,

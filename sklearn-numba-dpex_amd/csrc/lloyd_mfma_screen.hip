@@ -198,12 +198,19 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     // then computed from the copy in LDS.
     {
         const int lane_ = threadIdx.x & 63, wave_ = threadIdx.x >> 6;
-        const unsigned int my_absmax = threadIdx.x < d ? absmax[threadIdx.x] : 0u;
+        // Labels only: max|x| is not known and any scale is a correct one (a sample that overflows
+        // fp16 gives infinite or NaN scores, fails the test and is evaluated in fp32), so four
+        // times max|c| stands in for it: samples lie around the centroids they are assigned to.
+        unsigned int my_absmax = (UPDATE && threadIdx.x < d) ? absmax[threadIdx.x] : 0u;
         for (int f = wave_; f < d; f += WAVES)
-            for (int c = lane_; c < kp; c += 64) ct[f * kp + c] = c < k ? centroids_t[(size_t)f * k + c] : 0.0f;
+            for (int c = lane_; c < kp; c += 64) {
+                const float v = c < k ? centroids_t[(size_t)f * k + c] : 0.0f;
+                ct[f * kp + c] = v;
+                if (!UPDATE) my_absmax = max(my_absmax, __float_as_uint(fabsf(v) * 4.0f));
+            }
         __syncthreads();  // the shared words above are zero
         // (non-negative floats order like their bits)
-        if (threadIdx.x < d) atomicMax(&xmax_bits, my_absmax);
+        if (UPDATE ? threadIdx.x < d : my_absmax != 0u) atomicMax(&xmax_bits, my_absmax);
     }
     __syncthreads();
     // 2^-a with max|x| * 2^-a in [2^14, 2^15) (1 for all-zero or non-finite data)
@@ -275,7 +282,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     const float cmax = sqrtf(2.0f * hmax), abs_term = SCR_ERR_ABS * sqrtf((float)d);
     const float round_term = SCR_ERR_ROUND * 51.0f * (float)NK;
     // (||x|| comes unscaled from kmx_lloyd_init, hence the factor xs)
-    const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term) * xs;
+    // (and a norm the kernel takes itself, from the scaled values: no factor)
+    const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term) * (UPDATE ? xs : 1.0f);
     const float thr_0 = 2.01f * (round_term * hmax + abs_term * cmax);
     // +inf the optimiser cannot see through (it would turn the median below into a maximum
     // with two canonicalising instructions in front)
@@ -311,13 +319,16 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 
         // scaled fp16 split of the B operand
         v8h xh[NK][NC], xl[NK][NC];
+        float own_sq[NC];  // labels only: the lane's part of ||x||^2, scaled
 #pragma unroll
         for (int t = 0; t < NC; ++t) {
+            own_sq[t] = 0.0f;
 #pragma unroll
             for (int s = 0; s < NK; ++s)
 #pragma unroll
                 for (int i = 0; i < 8; i += 2) {
                     const v2f p = {x[s][i][t] * xsr[s][i], x[s][i + 1][t] * xsr[s][i + 1]};
+                    if (!UPDATE) own_sq[t] = fmaf(p[1], p[1], fmaf(p[0], p[0], own_sq[t]));
                     const v2h hh = __builtin_convertvector(p, v2h);
                     const v2f r = p - __builtin_convertvector(hh, v2f);
                     const v2h ll = __builtin_convertvector(r, v2h);
@@ -475,7 +486,13 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             const bool take_hi = b_hi > b_lo || (b_hi == b_lo && cc[1] < cc[0]);
             lab[t] = take_hi ? cc[1] : cc[0];
             // written so that a NaN anywhere makes the sample uncertain
-            const float thr = fmaf(thr_x, xnorm[t], thr_0);
+            float norm_t = xnorm[t];
+            if (!UPDATE) {
+                const auto qq = __builtin_amdgcn_permlane32_swap(__float_as_uint(own_sq[t]),
+                                                                 __float_as_uint(own_sq[t]), false, false);
+                norm_t = sqrtf(__uint_as_float(qq[0]) + __uint_as_float(qq[1]));
+            }
+            const float thr = fmaf(thr_x, norm_t, thr_0);
             unsure[t] = !(b - s2 > thr) && (FULL || i0 + t < n);
         }
 
@@ -643,9 +660,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             load_rows(wt, x);
             float wv[MC] = {0.f, 0.f};
             uint32_t pl[MC] = {0u, 0u};
-            const float2 n2 = *reinterpret_cast<const float2*>(norms + i0);
-            const float xnorm[MC] = {n2.x, n2.y};
+            float xnorm[MC] = {0.f, 0.f};  // labels only: taken from the tile itself
             if (UPDATE) {
+                const float2 n2 = *reinterpret_cast<const float2*>(norms + i0);
+                xnorm[0] = n2.x;
+                xnorm[1] = n2.y;
                 const float2 w2 = *reinterpret_cast<const float2*>(sample_weight + i0);
                 wv[0] = w2.x;
                 wv[1] = w2.y;
@@ -677,8 +696,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             load_scalar(Cols1{}, i0, x);
             float wv[1] = {0.f};
             uint32_t pl[1] = {0u};
-            const float xnorm[1] = {norms[i0]};
+            float xnorm[1] = {0.f};
             if (UPDATE) {
+                xnorm[0] = norms[i0];
                 wv[0] = sample_weight[i0];
                 pl[0] = labels_prev[i0];
             }
@@ -697,8 +717,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         for (int t = 0; t < MC; ++t) {
             wv[t] = 0.f;
             pl[t] = 0u;
-            xnorm[t] = i0 + t < n ? norms[i0 + t] : 0.0f;
+            xnorm[t] = 0.0f;
             if (UPDATE && i0 + t < n) {
+                xnorm[t] = norms[i0 + t];
                 wv[t] = sample_weight[i0 + t];
                 pl[t] = labels_prev[i0 + t];
             }
@@ -793,7 +814,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     if (UPDATE && changed) atomicAdd(&changed_block, changed);
     if (lane == 0 && n_uncertain) atomicAdd(&uncertain_block, n_uncertain);
     __syncthreads();
-    if (threadIdx.x == 0 && uncertain_block) atomicAdd(uncertain_count, uncertain_block);
+    if (threadIdx.x == 0 && uncertain_block && uncertain_count != nullptr)
+        atomicAdd(uncertain_count, uncertain_block);
     if (UPDATE) {
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
         const int n_out = (d + 1) * k, skip = (d_even - d) * k;  // gsum has no spare row
@@ -946,16 +968,12 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
     return screen_lds(d, k, (d + 15) / 16, true).off_queue <= SCR_LDS_MAX;
 }
 
-// Screened fused step.  `uncertain_count`: one word the kernel adds the number of samples it
-// evaluated in fp32 to (zero on entry; the finalisation that follows moves it to the next word
-// and clears it).  `absmax`: bits of max|X_t row| per feature, as kmx_lloyd_mfma_prepare leaves
-// them; `norms`: ||x_i|| per sample (kmx_sample_norms).
-int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
-                                   const uint32_t* labels_prev, uint32_t* labels,
-                                   kmx_lloyd_status* status, const unsigned int* absmax,
-                                   const int* q_exp, unsigned long long* gsum,
-                                   uint32_t* uncertain_count, const float* norms, int64_t n, int d,
-                                   int k, hipStream_t stream) {
+namespace {
+template <bool UPDATE>
+int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, const uint32_t* labels_prev,
+                      uint32_t* labels, kmx_lloyd_status* status, const unsigned int* absmax,
+                      const int* q_exp, unsigned long long* gsum, uint32_t* uncertain_count,
+                      const float* norms, int64_t n, int d, int k, hipStream_t stream) {
     if (!kmx_mfma_screen_supported(n, d, k)) return KMX_ERR_UNSUPPORTED;
     const int nk = (d + 15) / 16;
     const int waves = scr_waves(nk);
@@ -968,19 +986,42 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) && aligned16(w) &&
                        aligned16(labels_prev);
-    const size_t lds = screen_lds(d, k, nk, true).total;
+    const size_t lds = screen_lds(d, k, nk, UPDATE).total;
     if (nk == 1)
-        hipLaunchKernelGGL((lloyd_screen_kernel<1, true>), dim3((unsigned)grid), dim3(64 * scr_waves(1)),
+        hipLaunchKernelGGL((lloyd_screen_kernel<1, UPDATE>), dim3((unsigned)grid), dim3(64 * scr_waves(1)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
                            labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, norms, n, d,
                            k, vec_ok);
     else
-        hipLaunchKernelGGL((lloyd_screen_kernel<2, true>), dim3((unsigned)grid), dim3(64 * scr_waves(2)),
+        hipLaunchKernelGGL((lloyd_screen_kernel<2, UPDATE>), dim3((unsigned)grid), dim3(64 * scr_waves(2)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
                            labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, norms, n, d,
                            k, vec_ok);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
+}
+}  // namespace
+
+// Screened fused step.  `uncertain_count`: one word the kernel adds the number of samples it
+// evaluated in fp32 to (zero on entry; the finalisation that follows moves it to the next word
+// and clears it).  `absmax`: bits of max|X_t row| per feature, as kmx_lloyd_mfma_prepare leaves
+// them; `norms`: ||x_i|| per sample (kmx_sample_norms).
+int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
+                                   const uint32_t* labels_prev, uint32_t* labels,
+                                   kmx_lloyd_status* status, const unsigned int* absmax,
+                                   const int* q_exp, unsigned long long* gsum,
+                                   uint32_t* uncertain_count, const float* norms, int64_t n, int d,
+                                   int k, hipStream_t stream) {
+    return launch_screen<true>(X_t, w, centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,
+                               uncertain_count, norms, n, d, k, stream);
+}
+
+// Labels only, screened the same way: nothing but X and the centroids is needed (the scale comes
+// from the centroids, each tile takes the norms of its samples itself).
+int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
+                                      int64_t n, int d, int k, hipStream_t stream) {
+    return launch_screen<false>(X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr, nullptr,
+                                nullptr, nullptr, nullptr, n, d, k, stream);
 }
 
 // Diagnostics of the screen: approximate scores and error bounds as the fused step forms them.

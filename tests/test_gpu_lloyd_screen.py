@@ -84,6 +84,63 @@ def test_screened_step_matches_oracle(cuda, shape):
     assert rechecked <= 8 + n // 20
 
 
+def _labels_only(X, C, cuda):
+    """kmx_assign_labels through the C ABI (the screened label kernel for these shapes)."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    n, d = X.shape
+    k = C.shape[0]
+    X_t = torch.as_tensor(np.ascontiguousarray(X.T), device=cuda)
+    c_t = torch.as_tensor(np.ascontiguousarray(C.T), device=cuda)
+    labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
+    ws_bytes = lib.kmx_assign_workspace_bytes(d, k, 0)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
+    _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(c_t), ptr(labels), ptr(ws), ws_bytes, n, d, k, 0,
+                                      _capi.current_stream()), "assign")
+    return labels.cpu().numpy().astype(np.int64)
+
+
+@pytest.mark.parametrize("shape", [(20_000, 14, 127), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40),
+                                   (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16)])
+def test_screened_labels_only_match_oracle(cuda, shape):
+    n, d, k = shape
+    X, _, init = _blobs(n, d, k, seed=n + d + 1)
+    labels = _labels_only(X, init, cuda)
+    assert labels.min() >= 0 and labels.max() < k
+    assert_labels_match(labels, ok.assign_labels(X, init), X, init)
+
+
+@pytest.mark.parametrize("factor", [1e-6, 0.3, 7.0, 300.0, 1e6])
+def test_labels_only_with_samples_of_another_magnitude_than_the_centroids(cuda, factor):
+    """The labels-only kernel takes its scale from the centroids: samples far larger overflow
+    fp16 (and must then be evaluated in fp32), samples far smaller lose all their bits; the
+    labels must be the oracle's either way."""
+    rng = np.random.default_rng(31)
+    n, d, k = 6_000, 14, 40
+    C = rng.uniform(-4, 4, (k, d)).astype(np.float32)
+    X = (rng.uniform(-4, 4, (n, d)) * factor).astype(np.float32)
+    labels = _labels_only(X, C, cuda)
+    assert_labels_match(labels, ok.assign_labels(X, C), X, C)
+
+
+def test_labels_only_ties_and_zero_centroids(cuda):
+    rng = np.random.default_rng(37)
+    n, d, k = 5_000, 8, 24
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    C = rng.standard_normal((k, d)).astype(np.float32)
+    C[5] = C[2]                                    # duplicates: the lower index wins
+    C[9] = C[2]
+    labels = _labels_only(X, C, cuda)
+    ref = ok.assign_labels(X, C)
+    assert not np.any(labels == 5) and not np.any(labels == 9)
+    assert_labels_match(labels, ref, X, C)
+    zeros = _labels_only(X, np.zeros((k, d), dtype=np.float32), cuda)
+    assert np.all(zeros == 0)
+
+
 def test_fp32_matrix_core_step_selected_by_environment(cuda):
     """KMX_LLOYD_ASSIGN=f32 selects the all-fp32 kernel (variant 31); both give the oracle's labels."""
     X, w, init = _blobs(30_000, 14, 127, seed=5)
