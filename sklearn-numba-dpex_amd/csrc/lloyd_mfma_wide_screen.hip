@@ -26,6 +26,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 namespace {
 
@@ -57,6 +58,10 @@ __device__ __forceinline__ v4f lds_read16(unsigned int addr) {
 }
 __device__ __forceinline__ void lds_wait(v4f& a, v4f& b, v4f& c, v4f& d) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+// the same with the four most recent reads still in flight (a, b, c, d were issued before them)
+__device__ __forceinline__ void lds_wait_but4(v4f& a, v4f& b, v4f& c, v4f& d) {
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 
 // header words in the workspace
@@ -275,43 +280,62 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                 __syncthreads();
                 if (step + 2 < n_chunks) chunk_issue(step + 2, (step + 2) % 3);
                 const unsigned int fa = tile_addr + (unsigned int)(step % 3) * (CHUNK_VEC * 16u);
+                // Entry ((b * 2 + s2) * 2 + part) * 64 + lane of the chunk, 16 bytes each.  The
+                // four blocks are independent chains: their MFMAs are interleaved so that none
+                // waits for the result of the one before it.  The LDS reads run one group of
+                // MFMAs ahead (LDS reads of a wave complete in order): the hi parts of a K
+                // step are used while its lo parts arrive, the lo parts while the next hi parts
+                // arrive; a register is reloaded once the MFMAs reading it have been issued.
+                v4f rh[4], rl[4];
+                auto read_hi = [&](auto s_tag) {
+                    constexpr int S2 = decltype(s_tag)::value;
+                    rh[0] = lds_read16<(0 + 2 * S2) * 1024>(fa);
+                    rh[1] = lds_read16<(4 + 2 * S2) * 1024>(fa);
+                    rh[2] = lds_read16<(8 + 2 * S2) * 1024>(fa);
+                    rh[3] = lds_read16<(12 + 2 * S2) * 1024>(fa);
+                };
+                auto read_lo = [&](auto s_tag) {
+                    constexpr int S2 = decltype(s_tag)::value;
+                    rl[0] = lds_read16<(1 + 2 * S2) * 1024>(fa);
+                    rl[1] = lds_read16<(5 + 2 * S2) * 1024>(fa);
+                    rl[2] = lds_read16<(9 + 2 * S2) * 1024>(fa);
+                    rl[3] = lds_read16<(13 + 2 * S2) * 1024>(fa);
+                };
+                auto mfma_hi = [&](const int S) {  // hi * hi, hi * lo
+                    v8h ah[4];
 #pragma unroll
-                for (int s2i = 0; s2i < 2; ++s2i) {
-                    const int S = 2 * kc + s2i;
-                    // the four blocks are independent chains: their MFMAs are interleaved so that
-                    // none waits for the result of the one before it
-                    // entry ((b * 2 + s2) * 2 + part) * 64 + lane of the chunk, 16 bytes each
-                    v4f rh[4], rl[4];
-                    if (s2i == 0) {
-                        rh[0] = lds_read16<0 * 1024>(fa); rl[0] = lds_read16<1 * 1024>(fa);
-                        rh[1] = lds_read16<4 * 1024>(fa); rl[1] = lds_read16<5 * 1024>(fa);
-                        rh[2] = lds_read16<8 * 1024>(fa); rl[2] = lds_read16<9 * 1024>(fa);
-                        rh[3] = lds_read16<12 * 1024>(fa); rl[3] = lds_read16<13 * 1024>(fa);
-                    } else {
-                        rh[0] = lds_read16<2 * 1024>(fa); rl[0] = lds_read16<3 * 1024>(fa);
-                        rh[1] = lds_read16<6 * 1024>(fa); rl[1] = lds_read16<7 * 1024>(fa);
-                        rh[2] = lds_read16<10 * 1024>(fa); rl[2] = lds_read16<11 * 1024>(fa);
-                        rh[3] = lds_read16<14 * 1024>(fa); rl[3] = lds_read16<15 * 1024>(fa);
-                    }
-                    lds_wait(rh[0], rh[1], rh[2], rh[3]);
-                    lds_wait(rl[0], rl[1], rl[2], rl[3]);
-                    v8h ah[4], al[4];
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        ah[b] = __builtin_bit_cast(v8h, rh[b]);
-                        al[b] = __builtin_bit_cast(v8h, rl[b]);
-                    }
+                    for (int b = 0; b < 4; ++b) ah[b] = __builtin_bit_cast(v8h, rh[b]);
 #pragma unroll
                     for (int b = 0; b < 4; ++b)
                         acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[b], xh[S], acc[b], 0, 0, 0);
 #pragma unroll
                     for (int b = 0; b < 4; ++b)
                         acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[b], xl[S], acc[b], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+                auto mfma_lo = [&](const int S) {  // lo * hi
+                    v8h al[4];
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) al[b] = __builtin_bit_cast(v8h, rl[b]);
 #pragma unroll
                     for (int b = 0; b < 4; ++b)
                         acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[b], xh[S], acc[b], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
-                }
+                };
+                using Step0 = std::integral_constant<int, 0>;
+                using Step1 = std::integral_constant<int, 1>;
+                read_hi(Step0{});
+                read_lo(Step0{});
+                lds_wait_but4(rh[0], rh[1], rh[2], rh[3]);
+                mfma_hi(2 * kc);
+                lds_wait(rl[0], rl[1], rl[2], rl[3]);
+                read_hi(Step1{});
+                mfma_lo(2 * kc);
+                read_lo(Step1{});
+                lds_wait_but4(rh[0], rh[1], rh[2], rh[3]);
+                mfma_hi(2 * kc + 1);
+                lds_wait(rl[0], rl[1], rl[2], rl[3]);
+                mfma_lo(2 * kc + 1);
             }
 
             // arg-max by groups of 8 registers with the second largest of the group maxima
