@@ -216,6 +216,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     // 2^-a with max|x| * 2^-a in [2^14, 2^15) (1 for all-zero or non-finite data)
     const float xmax = __uint_as_float(xmax_bits);
     const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, 14 - ilogbf(xmax)) : 1.0f;
+    // The four pieces of work below start at different waves (thread index rotated by a third,
+    // a half, two thirds of the workgroup): each is a chain of LDS round trips too short to
+    // fill the workgroup, and one after the other on the same threads they took 3.7 us.
+    auto rotated = [&](const int by) { return (int)((threadIdx.x + THREADS - by) % THREADS); };
+    constexpr int ROT_HNEG = (THREADS / 3) & ~63, ROT_HX = THREADS / 2, ROT_ZERO = (2 * THREADS / 3) & ~63;
     // A operand: hi and lo parts of 32 centroids x 16 features per block and K step
     for (int idx = threadIdx.x; idx < n_cb * NK * 64; idx += THREADS) {
         const int l = idx & 63;
@@ -234,12 +239,13 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         afh[idx] = hi;
         afl[idx] = lo;
     }
-    for (int idx = threadIdx.x; idx < n_cb * 32; idx += THREADS) {
+    for (int idx = rotated(ROT_HNEG); idx < n_cb * 32; idx += THREADS) {
         const int cb = idx >> 5, hh = (idx >> 4) & 1, r = idx & 15;
         const int c = 32 * cb + 8 * (r >> 2) + 4 * hh + (r & 3);
         float v = -kmx_inf<float>();
         if (c < k) {
             float sq = 0.0f;
+#pragma unroll 8
             for (int f = 0; f < d; ++f) {
                 const float cv = ct[f * kp + c] * xs;
                 sq += cv * cv;
@@ -252,10 +258,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         hneg[idx] = v;
     }
     // unscaled half norms for the samples the screen cannot certify
-    for (int c = threadIdx.x; c < kp; c += THREADS) {
+    for (int c = rotated(ROT_HX); c < kp; c += THREADS) {
         float v = kmx_inf<float>();
         if (c < k) {
             float sq = 0.0f;
+#pragma unroll 8
             for (int f = 0; f < d; ++f) {
                 const float cv = ct[f * kp + c];
                 sq += cv * cv;
@@ -265,8 +272,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         hx[c] = v;
     }
     if (UPDATE)
-        for (int jx = threadIdx.x; jx < items; jx += THREADS) acc[jx] = 0ull;
-    for (int e = threadIdx.x; e < q_cap; e += THREADS) queue[e * QW + Q_INDEX] = QUEUE_FREE;
+        for (int jx = rotated(ROT_ZERO); jx < items; jx += THREADS) acc[jx] = 0ull;
+    for (int e = rotated(ROT_ZERO); e < q_cap; e += THREADS) queue[e * QW + Q_INDEX] = QUEUE_FREE;
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
