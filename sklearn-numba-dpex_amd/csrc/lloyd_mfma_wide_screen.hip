@@ -189,23 +189,34 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
         v8h xh[NS], xl[NS];
         float ss = 0.0f;
         {
-            // Loaded in batches of four K steps, 32 values in flight per lane, then converted.  The
-            // loads are inline assembly: at this register pressure the compiler would otherwise
-            // funnel every value through one register and wait for each load in turn, paying the
-            // memory latency 128 times per tile.  The values are valid after the wait statement,
-            // which takes them as operands.
+            // Loaded in batches of eight K steps, 64 values in flight per lane, then converted.
+            // The loads are inline assembly: at this register pressure the compiler would
+            // otherwise funnel every value through one register and wait for each load in turn,
+            // paying the memory latency 128 times per tile.  The values are valid after the wait
+            // statement, which takes them as operands.  Which rows exist is the same for the whole
+            // wave (scalar branches, no per-lane selects); of a last pair that is half there
+            // (odd d) both half-waves read row d - 1 and the upper one drops the value.  A lane
+            // past the end works on sample 0 and its results are not used.
             const float* __restrict__ xp = X_t + (size_t)h * n + (valid ? i : 0);
             const size_t two_rows = 2 * (size_t)n;
-            constexpr int BATCH = NS < 4 ? 2 : 4;  // NS is even
-#pragma unroll
-            for (int S0 = 0; S0 < NS; S0 += BATCH) {
+            auto load_batch = [&](auto s0_tag, auto batch_tag) {
+                constexpr int S0 = decltype(s0_tag)::value, BATCH = decltype(batch_tag)::value;
+                static_assert(BATCH % 2 == 0, "the wait statements take 16 values each");
                 float raw[BATCH * 8];
-                bool ok[BATCH * 8];
+                // (d compared afresh with scalar instructions: the compiler would otherwise keep
+                // one lane mask per row in scalar registers across the tile loop and spill them)
+                int d_now = d;
+                asm volatile("" : "+s"(d_now));
 #pragma unroll
                 for (int u = 0; u < BATCH * 8; ++u) {
-                    ok[u] = valid && (16 * S0 + 2 * u + h < d);
-                    const float* src = ok[u] ? xp : X_t;  // branch-free: element 0 instead, zeroed below
-                    asm volatile("global_load_dword %0, %1, off" : "=v"(raw[u]) : "v"(src));
+                    const int f0 = 16 * S0 + 2 * u;  // the pair's even feature
+                    raw[u] = 0.0f;
+                    if (f0 + 1 < d_now) {
+                        asm volatile("global_load_dword %0, %1, off" : "=v"(raw[u]) : "v"(xp));
+                    } else if (f0 + 1 == d_now) {
+                        const float* last_row = xp - (size_t)h * n;
+                        asm volatile("global_load_dword %0, %1, off" : "=v"(raw[u]) : "v"(last_row));
+                    }
                     xp += two_rows;
                 }
                 // one wait for the whole batch; the statements take 16 values each (operand limit)
@@ -217,9 +228,12 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                                    "+v"(raw[g + 8]), "+v"(raw[g + 9]), "+v"(raw[g + 10]), "+v"(raw[g + 11]),
                                    "+v"(raw[g + 12]), "+v"(raw[g + 13]), "+v"(raw[g + 14]), "+v"(raw[g + 15]));
 #pragma unroll
+                for (int u = 0; u < BATCH * 8; ++u)
+                    if (16 * S0 + 2 * u + 1 == d_now && h) raw[u] = 0.0f;  // scalar test first
+#pragma unroll
                 for (int u = 0; u < BATCH * 8; u += 2) {
                     const int S = S0 + u / 8, q = u % 8;
-                    const v2f p = {ok[u] ? raw[u] * xs : 0.0f, ok[u + 1] ? raw[u + 1] * xs : 0.0f};
+                    const v2f p = {raw[u] * xs, raw[u + 1] * xs};
                     const v2h hh = __builtin_convertvector(p, v2h);
                     const v2f r = p - __builtin_convertvector(hh, v2f);
                     const v2h ll = __builtin_convertvector(r, v2h);
@@ -230,7 +244,13 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                     ss = fmaf(p[0], p[0], ss);
                     ss = fmaf(p[1], p[1], ss);
                 }
-            }
+            };
+            constexpr int FULL8 = NS / 8, REST = NS % 8;  // NS is even
+            if constexpr (FULL8 >= 1) load_batch(std::integral_constant<int, 0>{}, std::integral_constant<int, 8>{});
+            if constexpr (FULL8 >= 2) load_batch(std::integral_constant<int, 8>{}, std::integral_constant<int, 8>{});
+            static_assert(FULL8 <= 2, "d <= 256");
+            if constexpr (REST > 0)
+                load_batch(std::integral_constant<int, 8 * FULL8>{}, std::integral_constant<int, REST>{});
         }
         const float nrm = ss + __shfl_xor(ss, 32, 64);
 
