@@ -193,31 +193,37 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
             // The loads are inline assembly: at this register pressure the compiler would
             // otherwise funnel every value through one register and wait for each load in turn,
             // paying the memory latency 128 times per tile.  The values are valid after the wait
-            // statement, which takes them as operands.  Which rows exist is the same for the whole
-            // wave (scalar branches, no per-lane selects); of a last pair that is half there
-            // (odd d) both half-waves read row d - 1 and the upper one drops the value.  A lane
-            // past the end works on sample 0 and its results are not used.
-            const float* __restrict__ xp = X_t + (size_t)h * n + (valid ? i : 0);
-            const size_t two_rows = 2 * (size_t)n;
+            // statement, which takes them as operands.
+            // Every load is a scalar row address plus a 32-bit byte offset of the lane (n < 2^29):
+            // no vector instruction goes into addresses.  Which rows exist is the same for the
+            // whole wave and decided by scalar branches (the assembly in their bodies keeps the
+            // compiler from turning them into per-lane selects): a pair below d reads rows f0
+            // and f0 + 1; of a last pair that is half there (odd d) both half-waves read row
+            // d - 1 and the upper one drops the value; a pair past d reads row 0 and is scaled
+            // by zero.  A lane past the end works on sample 0 and its results are not used.
+            const uint32_t off_0 = (uint32_t)(valid ? i : 0) * 4u;
+            const uint32_t off_h = off_0 + (uint32_t)h * (uint32_t)n * 4u;
+            const size_t pair_stride = (size_t)n * 8u;  // two rows
             auto load_batch = [&](auto s0_tag, auto batch_tag) {
                 constexpr int S0 = decltype(s0_tag)::value, BATCH = decltype(batch_tag)::value;
                 static_assert(BATCH % 2 == 0, "the wait statements take 16 values each");
                 float raw[BATCH * 8];
-                // (d compared afresh with scalar instructions: the compiler would otherwise keep
-                // one lane mask per row in scalar registers across the tile loop and spill them)
+                // (d and the base are hidden from loop-invariant hoisting: one lane mask and one
+                // 64-bit pointer per row kept across the tile loop would all be spilled)
                 int d_now = d;
-                asm volatile("" : "+s"(d_now));
+                size_t hidden_zero = 0;
+                asm volatile("" : "+s"(d_now), "+s"(hidden_zero));
+                const char* row = reinterpret_cast<const char*>(X_t) + hidden_zero + (size_t)(8 * S0) * pair_stride;
 #pragma unroll
                 for (int u = 0; u < BATCH * 8; ++u) {
                     const int f0 = 16 * S0 + 2 * u;  // the pair's even feature
-                    raw[u] = 0.0f;
                     if (f0 + 1 < d_now) {
-                        asm volatile("global_load_dword %0, %1, off" : "=v"(raw[u]) : "v"(xp));
-                    } else if (f0 + 1 == d_now) {
-                        const float* last_row = xp - (size_t)h * n;
-                        asm volatile("global_load_dword %0, %1, off" : "=v"(raw[u]) : "v"(last_row));
+                        asm volatile("global_load_dword %0, %1, %2" : "=v"(raw[u]) : "v"(off_h), "s"(row));
+                    } else {
+                        const char* one_row = f0 < d_now ? row : reinterpret_cast<const char*>(X_t);
+                        asm volatile("global_load_dword %0, %1, %2" : "=v"(raw[u]) : "v"(off_0), "s"(one_row));
                     }
-                    xp += two_rows;
+                    row += pair_stride;
                 }
                 // one wait for the whole batch; the statements take 16 values each (operand limit)
 #pragma unroll
@@ -227,13 +233,22 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                                    "+v"(raw[g + 4]), "+v"(raw[g + 5]), "+v"(raw[g + 6]), "+v"(raw[g + 7]),
                                    "+v"(raw[g + 8]), "+v"(raw[g + 9]), "+v"(raw[g + 10]), "+v"(raw[g + 11]),
                                    "+v"(raw[g + 12]), "+v"(raw[g + 13]), "+v"(raw[g + 14]), "+v"(raw[g + 15]));
+                float scaled[BATCH * 8];
+                int d_then = d;  // compared afresh again: nothing kept from the loads above
+                asm volatile("" : "+s"(d_then));
 #pragma unroll
-                for (int u = 0; u < BATCH * 8; ++u)
-                    if (16 * S0 + 2 * u + 1 == d_now && h) raw[u] = 0.0f;  // scalar test first
+                for (int u = 0; u < BATCH * 8; ++u) {
+                    const int f0 = 16 * S0 + 2 * u;
+                    scaled[u] = raw[u] * xs;
+                    if (f0 + 1 >= d_then) {  // the last pair of an odd d, or padding
+                        asm volatile("" : "+v"(scaled[u]));
+                        if (f0 >= d_then || h) scaled[u] = 0.0f;
+                    }
+                }
 #pragma unroll
                 for (int u = 0; u < BATCH * 8; u += 2) {
                     const int S = S0 + u / 8, q = u % 8;
-                    const v2f p = {raw[u] * xs, raw[u + 1] * xs};
+                    const v2f p = {scaled[u], scaled[u + 1]};
                     const v2h hh = __builtin_convertvector(p, v2h);
                     const v2f r = p - __builtin_convertvector(hh, v2f);
                     const v2h ll = __builtin_convertvector(r, v2h);
@@ -455,7 +470,8 @@ size_t kmx_wide_screen_bytes(int64_t n, int d, int k) {
 
 // KMX_LLOYD_ASSIGN = f32 switches the screen off (all-fp32 scores, lloyd_mfma_wide.hip).
 bool kmx_wide_screen_enabled(int64_t n, int d, int k) {
-    if (!kmx_mfma_wide_supported(d, k) || n > INT32_MAX) return false;
+    // (the label kernel addresses a lane's samples with 32-bit byte offsets into two rows)
+    if (!kmx_mfma_wide_supported(d, k) || n >= ((int64_t)1 << 29)) return false;
     const char* v = std::getenv("KMX_LLOYD_ASSIGN");
     return !(v != nullptr && std::strcmp(v, "f32") == 0);
 }

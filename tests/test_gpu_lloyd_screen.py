@@ -402,7 +402,8 @@ def test_error_bound_of_the_screen_holds_on_the_hardware(cuda, name):
     assert np.median(bounds) <= 1e-3 * max(typical, np.abs(exact).max() * 1e-3)
 
 
-@pytest.mark.parametrize("shape", [(6_000, 128, 64), (3_000, 256, 200), (4_097, 40, 400), (2_500, 70, 1024)])
+@pytest.mark.parametrize("shape", [(6_000, 128, 64), (3_000, 256, 200), (4_097, 40, 400), (2_500, 70, 1024),
+                                   (3_001, 67, 300), (2_000, 33, 300), (1_500, 255, 96)])
 def test_wide_screened_step_matches_oracle(cuda, shape):
     """The wide fp32 path (variant 42) screens its labels the same way; what it cannot certify
     goes through the all-fp32 matrix-core kernel."""
