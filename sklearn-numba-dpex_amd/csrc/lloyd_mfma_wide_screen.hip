@@ -149,7 +149,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
     for (int c = threadIdx.x; c < n_cg * CG; c += 256) hneg_s[c] = hneg[c];
     if (threadIdx.x == 0) changed_block = 0;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // (the wave index as a scalar: what is derived from it, such as the LDS base of the chunk
+    // copies, then needs no vector instructions)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int h = lane >> 5, j = lane & 31;
     const int64_t n_tiles = (n + 127) >> 7;
     unsigned int changed = 0;
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
     const unsigned int tile_addr = (unsigned int)(uintptr_t)(&ctile[0][0]) + (unsigned int)lane * 16u;
     const unsigned int hneg_addr = (unsigned int)(uintptr_t)(&hneg_s[0]);
     auto chunk_issue = [&](int chunk, int buf) {
-        const uint4* __restrict__ src = split + (size_t)chunk * CHUNK_VEC + threadIdx.x;
+        const uint4* __restrict__ src = split + (size_t)chunk * CHUNK_VEC + 64 * wave + lane;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             __builtin_amdgcn_global_load_lds(
