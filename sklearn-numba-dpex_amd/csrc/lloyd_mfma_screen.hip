@@ -15,13 +15,19 @@
 //   E(x) = (7.2e-7 + r) ||x|| C + r H + 6.2e-5 sqrt(d) (||x|| + C),  r = 6.1e-6 ceil(d / 16),
 // C = max ||c||, H = max 0.5||c||^2 (scaled units).  If the best approximate score beats the second best by more than 2 E(x),
 // the arg-max of the approximate scores IS the arg-max of the exact real-valued scores: the
-// label is certain.  Otherwise (about 2 samples in 1000 on blob data) the wave evaluates the
-// sample in plain fp32 on the spot: every lane takes the centroids lane, lane + 64, ... with
-// feature-sequential fused multiply-adds from -0.5||c||^2, and the wave combines the results
-// with the lowest index winning a tie.  Labels therefore meet the same bar as an all-fp32
-// evaluation (they can differ from it only where fp32's own rounding decides), and the sums
-// are taken from the fp32 inputs in 64-bit fixed point exactly as in lloyd_mfma.hip.
-// Non-finite scores make a sample uncertain.
+// label is certain.  Otherwise (about 2 samples in 1000 on blob data) the sample is put on a
+// queue of the workgroup in LDS and evaluated in plain fp32 after the last tile, one wave per
+// entry: every lane takes the centroids lane, lane + 64, ... with feature-sequential fused
+// multiply-adds from -0.5||c||^2, and the wave combines the results with the lowest index
+// winning a tie.  A 32-sample column with several such samples, or one that finds the queue
+// full, is redone as a whole in fp32 on the matrix cores instead.  Labels therefore meet the
+// same bar as an all-fp32 evaluation (they can differ from it only where fp32's own rounding
+// decides), and the sums are taken from the fp32 inputs in 64-bit fixed point exactly as in
+// lloyd_mfma.hip.  Non-finite scores make a sample uncertain.
+//
+// The same kernel without the update assigns labels only (kmx_assign_labels): there the scale
+// comes from the centroids (any scale is correct, a sample that overflows fp16 merely fails the
+// test) and each tile takes the norms of its samples itself.
 //
 // Work decomposition: as in lloyd_mfma.hip with two sample columns per lane.  Lane (j, h) of a
 // wave owns features 16 s + 2 i + h (i < 8) of samples 2 j, 2 j + 1 of the wave's 64-sample
@@ -40,12 +46,6 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef double v8d __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-
-constexpr double FIX_MAGIC = 6755399441055744.0;  // 1.5 * 2^52
-constexpr long long FIX_MAGIC_BITS = 0x4338000000000000ll;
-__device__ __forceinline__ unsigned long long to_fixed(double scaled_plus_magic) {
-    return (unsigned long long)(__double_as_longlong(scaled_plus_magic) - FIX_MAGIC_BITS);
-}
 
 // Error bound of one approximate score, in scaled units:
 //   (SCR_ERR_SPLIT + r) ||x|| C + r H + SCR_ERR_ABS sqrt(d) (||x|| + C),
