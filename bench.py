@@ -160,7 +160,7 @@ def gpu_lloyd(cfg, steps, warmup):
     # parity gate 2: kmx_assign_labels for the centroids the last iteration produced
     cur = cent[it % 2].T.cpu().numpy()
     lab = torch.empty(n, dtype=torch.int32, device=dev)
-    aws = lib.kmx_assign_workspace_bytes(d, k, dc)
+    aws = lib.kmx_assign_workspace_bytes_for(n, d, k, dc)
     aws_t = torch.empty(aws, dtype=torch.uint8, device=dev)
     _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(X_t.new_tensor(cur.T.copy())), ptr(lab), ptr(aws_t), aws,
                                       n, d, k, dc, stream), "assign")

@@ -166,6 +166,12 @@ int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype)
 
 size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype);
 
+/* The workspace with which kmx_assign_labels takes its fastest path for n samples: wide fp32
+ * shapes screen the labels on the fp16 matrix cores and need room for a list of samples.  Never
+ * smaller than kmx_assign_workspace_bytes, which always suffices.  It has no counterpart in the
+ * reference (workspaces belong to this library). */
+size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype);
+
 /* labels[i] = argmin_c (0.5||c||^2 - <x_i, c>).  Replaces
  * make_label_assignment_fixed_window_kernel (kmeans/kernels/compute_labels.py:18-185) and the
  * half-norm call before it (kmeans/drivers.py:657-669). */

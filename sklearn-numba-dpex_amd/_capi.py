@@ -70,6 +70,7 @@ SIGNATURES = {
     "kmx_screen_scores": (_I32, [_P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _P]),
     "kmx_lloyd_kernel_variant": (_I32, [_I64, _I32, _I32, _I32]),
     "kmx_assign_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "kmx_assign_workspace_bytes_for": (_SZ, [_I64, _I32, _I32, _I32]),
     "kmx_assign_labels": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
     "kmx_per_sample_inertia": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_euclidean_distances": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _P]),

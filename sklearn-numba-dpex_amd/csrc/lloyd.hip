@@ -930,6 +930,14 @@ size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
     return lloyd_layout(1, d, k, dtype).off_bucket;
 }
 
+size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype) {
+    const size_t base = kmx_assign_workspace_bytes(d, k, dtype);
+    if (base == 0 || n <= 0 || dtype != KMX_F32) return base;
+    if (lloyd_layout(n, d, k, dtype).variant != KMX_VARIANT_MFMA_WIDE) return base;
+    const size_t extra = kmx_assign_wide_screen_bytes(n, d, k);
+    return extra ? kmx_align256(base) + extra : base;
+}
+
 int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
                           void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
                           int32_t dtype, void* stream_) {
@@ -955,8 +963,15 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
         KMX_LAUNCH_CHECK();
         if (L.variant == KMX_VARIANT_MFMA)
             return kmx_assign_labels_mfma_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
-        if (L.variant == KMX_VARIANT_MFMA_WIDE)
+        if (L.variant == KMX_VARIANT_MFMA_WIDE) {
+            // with the larger workspace of kmx_assign_workspace_bytes_for: labels screened in fp16
+            const size_t extra = kmx_assign_wide_screen_bytes(n, d, k);
+            const size_t extra_off = kmx_align256(L.off_bucket);
+            if (extra != 0 && workspace_bytes >= extra_off + extra)
+                return kmx_assign_labels_wide_screen_f32(L, X_t, centroids_t, labels, ws, ws + extra_off, n, d,
+                                                         k, stream);
             return kmx_assign_labels_mfma_wide_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
+        }
         launch_fused<float, ACC_NONE>(L, X_t, nullptr, centroids_t, (const float*)(ws + L.off_cpack),
                                       (const float*)(ws + L.off_half), nullptr, labels, nullptr,
                                       nullptr, n, d, k, stream);

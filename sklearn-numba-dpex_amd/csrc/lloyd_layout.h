@@ -146,6 +146,14 @@ int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipSt
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,
                                int64_t n, int d, int k, hipStream_t stream);
+int32_t kmx_wide_screen_scale_from_centroids(const void* centroids_t, unsigned int* absmax, int d, int k,
+                                             hipStream_t stream);
+// labels only through the wide screen: bytes of extra workspace (0: not available), and the pass
+size_t kmx_assign_wide_screen_bytes(int64_t n, int d, int k);
+int32_t kmx_assign_labels_wide_screen_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
+                                          uint32_t* labels, char* ws, char* extra, int64_t n, int d,
+                                          int k, hipStream_t stream);
+// (labels_prev, status, counts, ranks all null: labels only)
 int32_t kmx_lloyd_wide_screen_count(const void* X_t, const void* centroids_t,
                                     const unsigned int* absmax, char* area,
                                     const uint32_t* labels_prev, uint32_t* labels,

@@ -80,7 +80,7 @@ constexpr int MODE_COUNT = 2;    // labels + changed count + per-cluster sample 
 
 // LISTED: the kernel works on the samples list[0 .. *list_count) instead of 0 .. n - 1 (the
 // samples the fp16 screen of lloyd_mfma_wide_screen.hip could not certify) and reads their
-// features from the row-major copy X_rm.
+// features from the row-major copy X_rm, or gathers them from X_t where there is none.
 template <int NKC, int MODE, bool LISTED = false>
 __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
 
         // row 2s + h of X_t, advanced by two rows per K step (no per-row offsets kept alive)
         float x[NKS];
-        if constexpr (LISTED) {
+        if (LISTED && X_rm != nullptr) {
             const float* __restrict__ xp = X_rm + (size_t)i * d + h;
 #pragma unroll
             for (int s = 0; s < NKS; ++s) x[s] = (valid && 2 * s + h < d) ? xp[2 * s] : 0.0f;
@@ -426,8 +426,9 @@ int32_t launch_wide(const LloydLayout& L, const void* X_t, const void* w, const 
     return KMX_OK;
 }
 
-// The counting mode on the listed samples only; the grid is fixed because the length of the
-// list is only known on the device (blocks without a tile leave at once).
+// One mode on the listed samples only; the grid is fixed because the length of the list is only
+// known on the device (blocks without a tile leave at once).
+template <int MODE>
 int32_t launch_wide_listed(const void* X_t, const void* X_rm, const void* w, const void* centroids_t,
                            const float* half_norms, const uint32_t* labels_prev, uint32_t* labels,
                            kmx_lloyd_status* status, const int* q_exp, unsigned long long* gsum,
@@ -442,7 +443,7 @@ int32_t launch_wide_listed(const void* X_t, const void* X_rm, const void* w, con
     if (grid < 1) grid = 1;
     const int vec_ok = (k % 4 == 0) && ((((uintptr_t)centroids_t) & 15) == 0);
 #define KMX_WIDE_CASE(NKC)                                                                             \
-    hipLaunchKernelGGL((lloyd_mfma_wide_kernel<NKC, MODE_COUNT, true>), dim3((unsigned)grid), dim3(256), \
+    hipLaunchKernelGGL((lloyd_mfma_wide_kernel<NKC, MODE, true>), dim3((unsigned)grid), dim3(256),       \
                        lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,       \
                        half_norms, labels_prev, labels, status, q_exp, gsum, counts, ranks, n, d, k,     \
                        vec_ok, (const float*)X_rm, list, list_count)
@@ -494,9 +495,9 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
                                          reinterpret_cast<const unsigned int*>(ws + L.off_scales), area,
                                          labels_prev, labels, status, counts, ranks, n, d, k, stream);
         if (rc != KMX_OK) return rc;
-        rc = launch_wide_listed(X_t, X_rowmajor, w, centroids_t, half_norms, labels_prev, labels, status,
-                                q_exp, gsum, counts, ranks, kmx_wide_screen_list(area, d, k),
-                                kmx_wide_screen_counter(area), n, d, k, stream);
+        rc = launch_wide_listed<MODE_COUNT>(X_t, X_rowmajor, w, centroids_t, half_norms, labels_prev, labels,
+                                            status, q_exp, gsum, counts, ranks, kmx_wide_screen_list(area, d, k),
+                                            kmx_wide_screen_counter(area), n, d, k, stream);
     } else
         rc = launch_wide<MODE_COUNT>(L, X_t, w, centroids_t, half_norms, labels_prev, labels, status,
                                      q_exp, gsum, counts, ranks, n, d, k, stream);
@@ -517,6 +518,30 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
                            gsum, (int)n, d, k);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
+}
+
+size_t kmx_assign_wide_screen_bytes(int64_t n, int d, int k) {
+    if (!kmx_wide_screen_enabled(n, d, k)) return 0;
+    return kmx_align256((size_t)d * sizeof(unsigned int)) + kmx_wide_screen_bytes(n, d, k);
+}
+
+// Labels only with the fp16 screen: `extra` holds kmx_assign_wide_screen_bytes.  The scale comes
+// from the centroids (any scale is a correct one), the listed samples are gathered from X_t.
+int32_t kmx_assign_labels_wide_screen_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
+                                          uint32_t* labels, char* ws, char* extra, int64_t n, int d,
+                                          int k, hipStream_t stream) {
+    unsigned int* absmax = reinterpret_cast<unsigned int*>(extra);
+    char* area = extra + kmx_align256((size_t)d * sizeof(unsigned int));
+    int32_t rc = kmx_wide_screen_scale_from_centroids(centroids_t, absmax, d, k, stream);
+    if (rc != KMX_OK) return rc;
+    rc = kmx_lloyd_wide_screen_count(X_t, centroids_t, absmax, area, nullptr, labels, nullptr, nullptr,
+                                     nullptr, n, d, k, stream);
+    if (rc != KMX_OK) return rc;
+    return launch_wide_listed<MODE_LABELS>(X_t, nullptr, nullptr, centroids_t,
+                                           reinterpret_cast<const float*>(ws + L.off_half), nullptr, labels,
+                                           nullptr, nullptr, nullptr, nullptr, nullptr,
+                                           kmx_wide_screen_list(area, d, k), kmx_wide_screen_counter(area),
+                                           n, d, k, stream);
 }
 
 int32_t kmx_assign_labels_mfma_wide_f32(const LloydLayout& L, const void* X_t,

@@ -138,7 +138,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     kmx_lloyd_status* __restrict__ status, int* __restrict__ counts, int* __restrict__ ranks,
     int64_t n, int d, int k) {
-    if (status->state != KMX_RUNNING) return;
+    // labels only: no status, previous labels, counts or ranks
+    const bool update = status != nullptr;
+    if (update && status->state != KMX_RUNNING) return;
 
     constexpr int NS = 2 * NKC;  // K steps of 16 features
     __shared__ __align__(16) uint4 ctile[3][CHUNK_VEC];
@@ -452,18 +454,45 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
 
         if (valid && h == 0 && !unsure) {
             labels[i] = lab;
-            changed += (labels_prev[i] != lab) ? 1u : 0u;
-            // the returned count is the sample's rank inside its cluster (for the scatter)
-            ranks[i] = atomicAdd(counts + lab, 1);
+            if (update) {
+                changed += (labels_prev[i] != lab) ? 1u : 0u;
+                // the returned count is the sample's rank inside its cluster (for the scatter)
+                ranks[i] = atomicAdd(counts + lab, 1);
+            }
         }
     }
 
     if (changed) atomicAdd(&changed_block, changed);
     __syncthreads();
-    if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+    if (update && threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+}
+
+// absmax[f] = bits of 4 max|c| for every feature: the stand-in for max|x| where only the
+// centroids are at hand (labels only); one workgroup.
+__global__ __launch_bounds__(1024) void wide_scale_from_centroids_kernel(const float* __restrict__ centroids_t,
+                                                                        unsigned int* __restrict__ absmax,
+                                                                        int d, int k) {
+    __shared__ unsigned int m_bits;
+    if (threadIdx.x == 0) m_bits = 0u;
+    __syncthreads();
+    float m = 0.0f;
+    for (int idx = threadIdx.x; idx < d * k; idx += 1024) m = fmaxf(m, fabsf(centroids_t[idx]));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((threadIdx.x & 63) == 0) atomicMax(&m_bits, __float_as_uint(4.0f * m));  // non-negative: ordered like the bits
+    __syncthreads();
+    for (int f = threadIdx.x; f < d; f += 1024) absmax[f] = m_bits;
 }
 
 }  // namespace
+
+int32_t kmx_wide_screen_scale_from_centroids(const void* centroids_t, unsigned int* absmax, int d, int k,
+                                             hipStream_t stream) {
+    hipLaunchKernelGGL(wide_scale_from_centroids_kernel, dim3(1), dim3(1024), 0, stream,
+                       (const float*)centroids_t, absmax, d, k);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
 
 size_t kmx_wide_screen_bytes(int64_t n, int d, int k) {
     const size_t n_cg = (size_t)(k + CG - 1) / CG, nkc = (size_t)(d + KC - 1) / KC;

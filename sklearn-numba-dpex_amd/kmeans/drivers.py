@@ -126,7 +126,7 @@ def _assign(X_t, centroids_t, labels_out):
     d, n = X_t.shape
     k = centroids_t.shape[1]
     dc = dcode(X_t)
-    ws_bytes = lib.kmx_assign_workspace_bytes(d, k, dc)
+    ws_bytes = lib.kmx_assign_workspace_bytes_for(n, d, k, dc)
     ws = workspace(ws_bytes, X_t.device)
     check(lib.kmx_assign_labels(ptr(X_t), ptr(centroids_t), ptr(labels_out), ptr(ws), ws_bytes, n, d, k,
                                 dc, _capi.current_stream()), "kmx_assign_labels")

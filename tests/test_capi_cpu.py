@@ -65,6 +65,11 @@ def test_workspace_queries():
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0) == 0
     assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7) == 0
     assert lib.kmx_assign_workspace_bytes(14, 127, 0) > 127 * 16 * 4
+    # the roomy variant only grows for wide fp32 shapes (a list of sample indices)
+    assert lib.kmx_assign_workspace_bytes_for(1000, 14, 127, 0) == lib.kmx_assign_workspace_bytes(14, 127, 0)
+    assert lib.kmx_assign_workspace_bytes_for(1000, 256, 1024, 1) == lib.kmx_assign_workspace_bytes(256, 1024, 1)
+    assert (lib.kmx_assign_workspace_bytes_for(1000, 256, 1024, 0)
+            >= lib.kmx_assign_workspace_bytes(256, 1024, 0) + 1000 * 4)
     assert lib.kmx_kpp_workspace_bytes(1_000_000, 64, 256, 7, 0) >= 7 * 4_000_000
     assert lib.kmx_kpp_workspace_bytes(1000, 4, 8, 17, 0) == 0  # more trials than supported
     assert lib.kmx_topk_workspace_bytes(1000, 10) > 0

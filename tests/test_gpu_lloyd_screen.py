@@ -84,8 +84,9 @@ def test_screened_step_matches_oracle(cuda, shape):
     assert rechecked <= 8 + n // 20
 
 
-def _labels_only(X, C, cuda):
-    """kmx_assign_labels through the C ABI (the screened label kernel for these shapes)."""
+def _labels_only(X, C, cuda, roomy=True):
+    """kmx_assign_labels through the C ABI (the screened label kernels; with roomy=False the
+    minimal workspace, with which wide shapes take the all-fp32 kernel)."""
     import torch
 
     from sklearn_numba_dpex_amd import _capi
@@ -96,7 +97,7 @@ def _labels_only(X, C, cuda):
     X_t = torch.as_tensor(np.ascontiguousarray(X.T), device=cuda)
     c_t = torch.as_tensor(np.ascontiguousarray(C.T), device=cuda)
     labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_assign_workspace_bytes(d, k, 0)
+    ws_bytes = lib.kmx_assign_workspace_bytes_for(n, d, k, 0) if roomy else lib.kmx_assign_workspace_bytes(d, k, 0)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
     _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(c_t), ptr(labels), ptr(ws), ws_bytes, n, d, k, 0,
                                       _capi.current_stream()), "assign")
@@ -413,6 +414,37 @@ def test_wide_screened_step_matches_oracle(cuda, shape):
     assert variant == 42
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
     assert rechecked <= 8 + n // 10
+
+
+@pytest.mark.parametrize("shape", [(6_000, 128, 64), (3_000, 256, 200), (4_097, 40, 400), (2_500, 70, 1024),
+                                   (3_001, 67, 300), (1_500, 255, 96)])
+def test_wide_screened_labels_only_match_oracle(cuda, shape):
+    """kmx_assign_labels for wide shapes: screened in fp16 when the workspace has room for the list
+    of uncertified samples (kmx_assign_workspace_bytes_for), all fp32 with the minimal workspace;
+    both must give the oracle's labels."""
+    from sklearn_numba_dpex_amd._capi import lib
+
+    n, d, k = shape
+    X, _, init = _blobs(n, d, k, seed=n + d + 2)
+    assert lib.kmx_assign_workspace_bytes_for(n, d, k, 0) > lib.kmx_assign_workspace_bytes(d, k, 0)
+    ref = ok.assign_labels(X, init)
+    for roomy in (True, False):
+        labels = _labels_only(X, init, cuda, roomy=roomy)
+        assert labels.min() >= 0 and labels.max() < k
+        assert_labels_match(labels, ref, X, init)
+
+
+def test_wide_labels_only_with_samples_far_from_the_centroids(cuda):
+    """Scale taken from the centroids: samples a thousand times larger overflow fp16, are all
+    listed and evaluated in fp32; duplicated centroids give the lowest index."""
+    rng = np.random.default_rng(41)
+    n, d, k = 3_000, 96, 128
+    C = rng.standard_normal((k, d)).astype(np.float32)
+    C[7] = C[3]
+    X = (1000.0 * rng.standard_normal((n, d))).astype(np.float32)
+    labels = _labels_only(X, C, cuda)
+    assert not np.any(labels == 7)
+    assert_labels_match(labels, ok.assign_labels(X, C), X, C)
 
 
 def test_wide_duplicate_centroids_take_the_lowest_index(cuda):
