@@ -19,6 +19,8 @@
 // block of 1024 samples, so it never re-reads the whole array.
 #include "kmx_common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int TN_MAX = 16;      // n_local_trials = 2 + floor(ln k) <= 16 for k < 1.2e6
@@ -135,13 +137,15 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
     __shared__ double wave_pot[4][TN];
     const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
     const int best = header->best_row;
-    const bool full = vec_ok && (i0 + 4 <= n);
+    // Whether the 128-bit accesses are legal is decided once per workgroup and known at compile
+    // time inside the body: with a test per access every load sat in a branch of its own and
+    // was waited for before the next one was issued.
+    auto body = [&](auto full_tag) {
+    constexpr bool full = decltype(full_tag)::value;
 
-    // weights and the closest distances so far are needed after the feature loop: in flight
-    // during it
+    // weights and the closest distances so far are needed after the feature loop: requested
+    // with its last batch
     T w[4], cl[4];
-    load4<T>(sample_weight, i0, n, full, w);
-    load4<T>(rows + (size_t)best * n, i0, n, full, cl);
 
     T acc[TN][4];
 #pragma unroll
@@ -149,7 +153,9 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[t][r] = T(0);
 
-    constexpr int FB = 8;  // features per batch of loads
+    // Features in batches of FB rows: 16 loads of 16 bytes per lane in flight at a time in fp32
+    // (a wave has 64 KB to stream and only four of them share a SIMD).
+    constexpr int FB = sizeof(T) == 4 ? 16 : 8;
     for (int f0 = 0; f0 < d; f0 += FB) {
         T xv[FB][4];
 #pragma unroll
@@ -157,6 +163,10 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
             const int f = f0 + j < d ? f0 + j : d - 1;  // past the end: a valid row, ignored below
             const T* __restrict__ row = X_t + (size_t)f * n;
             load4<T>(row, i0, n, full, xv[j]);
+        }
+        if (f0 + FB >= d) {
+            load4<T>(sample_weight, i0, n, full, w);
+            load4<T>(rows + (size_t)best * n, i0, n, full, cl);
         }
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
@@ -205,6 +215,11 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
         block_pot[(size_t)blockIdx.x * TN_MAX + threadIdx.x] =
             (wave_pot[0][threadIdx.x] + wave_pot[1][threadIdx.x]) +
             (wave_pot[2][threadIdx.x] + wave_pot[3][threadIdx.x]);
+    };
+    if (vec_ok && (int64_t)(blockIdx.x + 1) * CHUNK <= n)
+        body(std::true_type{});
+    else
+        body(std::false_type{});
 }
 
 // Block-wide exclusive scan of one double per thread (256 threads); returns the exclusive
