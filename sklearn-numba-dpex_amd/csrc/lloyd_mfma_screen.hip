@@ -966,13 +966,19 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 }  // namespace
 
 // Shapes the screened step covers: d <= 32, everything within 64 KB of LDS, byte offsets
-// inside two rows of X_t within 32 bits.  KMX_LLOYD_ASSIGN = f32 switches it off (all-fp32
-// scores on the matrix cores, lloyd_mfma.hip).
+// inside two rows of X_t within 32 bits.  It is chosen where it is the faster one: the all-fp32
+// step pays d / 2 fp32 MFMAs per block of 32 centroids, the screen three fp16 ones plus the
+// split and the certificate whatever d is; measured on 2e6 samples the screen wins from d = 10
+// on, from d = 8 for k >= 64 and from d = 6 for k >= 128 (at d = 2 it is 30 % slower, at d = 16,
+// k = 128 36 % faster).  KMX_LLOYD_ASSIGN = f32 switches it off (all-fp32 scores on the matrix
+// cores, lloyd_mfma.hip), KMX_LLOYD_ASSIGN = screen selects it wherever it is possible.
 bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
     if (d < 1 || d > 32 || k < 16 || n >= ((int64_t)1 << 29)) return false;
     const char* v = std::getenv("KMX_LLOYD_ASSIGN");
     if (v != nullptr && std::strcmp(v, "f32") == 0) return false;
-    return screen_lds(d, k, (d + 15) / 16, true).off_queue <= SCR_LDS_MAX;
+    if (screen_lds(d, k, (d + 15) / 16, true).off_queue > SCR_LDS_MAX) return false;
+    if (v != nullptr && std::strcmp(v, "screen") == 0) return true;
+    return d >= 10 || (d >= 8 && k >= 64) || (d >= 6 && k >= 128);
 }
 
 namespace {

@@ -82,6 +82,9 @@ def test_kernel_variant_selection():
 
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 61   # bf16-screened MFMA + LDS accumulators
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0) == 31   # fp32 MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 4, 127, 0) == 31    # too few features for the screen to pay
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 64, 0) == 61
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 32, 0) == 31
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 51    # fp64: matrix cores + LDS
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1) in (12, 2)  # accumulators too big for LDS
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 42  # wide MFMA + global sums

@@ -17,6 +17,15 @@ from tests._parity import assert_centers_close, assert_labels_match
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _screen_wherever_possible():
+    """The library screens the labels only where that is the faster kernel (from about ten
+    features on); the tests here want the screened kernel on every shape it can run."""
+    os.environ["KMX_LLOYD_ASSIGN"] = "screen"
+    yield
+    os.environ.pop("KMX_LLOYD_ASSIGN", None)
+
+
 def _one_iteration(X, w, init, cuda):
     """kmx_lloyd_init + one kmx_lloyd_iter through the C ABI; returns labels, new centroids
     (or the sums when a cluster is empty), sizes, status, variant, samples evaluated in fp32."""
@@ -142,6 +151,19 @@ def test_labels_only_ties_and_zero_centroids(cuda):
     assert np.all(zeros == 0)
 
 
+def test_default_choice_between_screened_and_fp32_step(cuda):
+    """Without the environment switch the screen is used where it is the faster kernel."""
+    from sklearn_numba_dpex_amd._capi import lib
+
+    os.environ.pop("KMX_LLOYD_ASSIGN", None)
+    for (d, k), variant in {(14, 127): 61, (2, 16): 31, (8, 32): 31, (8, 64): 61, (6, 128): 61, (32, 64): 61}.items():
+        assert lib.kmx_lloyd_kernel_variant(100_000, d, k, 0) == variant, (d, k)
+    X, w, init = _blobs(5_000, 4, 20, seed=11)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    assert variant == 31 and rechecked == 0
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+
+
 def test_fp32_matrix_core_step_selected_by_environment(cuda):
     """KMX_LLOYD_ASSIGN=f32 selects the all-fp32 kernel (variant 31); both give the oracle's labels."""
     X, w, init = _blobs(30_000, 14, 127, seed=5)
@@ -152,7 +174,7 @@ def test_fp32_matrix_core_step_selected_by_environment(cuda):
         try:
             labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
         finally:
-            os.environ.pop("KMX_LLOYD_ASSIGN", None)
+            os.environ["KMX_LLOYD_ASSIGN"] = "screen"
         assert variant == (61 if mode == "screen" else 31)
         if mode == "f32":
             assert rechecked == 0
@@ -476,7 +498,7 @@ def test_wide_screen_switched_off_by_environment(cuda):
     try:
         labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
     finally:
-        os.environ.pop("KMX_LLOYD_ASSIGN", None)
+        os.environ["KMX_LLOYD_ASSIGN"] = "screen"
     assert variant == 42 and rechecked == 0
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
 
