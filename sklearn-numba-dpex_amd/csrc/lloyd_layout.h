@@ -80,7 +80,10 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
         if (copies > 32) copies = 32;
         L.n_partials = (int)copies;
     }
-    if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_supported(d, k) &&
+    // (the screened step has the whole LDS of a compute unit and covers shapes the all-fp32
+    // step, which stays within 64 KB, does not)
+    if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS &&
+        (kmx_mfma_supported(d, k) || kmx_mfma_screen_supported(n, d, k)) &&
         (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA;
     else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA)) {

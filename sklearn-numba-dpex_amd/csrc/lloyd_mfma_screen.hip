@@ -69,7 +69,10 @@ struct ScreenLds {
     int q_words;  // 32-bit words per entry: 16 nk feature values, weight, sample index, old label
 };
 constexpr int SCR_QUEUE_MAX = 256;
-constexpr size_t SCR_LDS_MAX = 64 * 1024;
+// LDS a workgroup may take: the compute unit has 160 KB; one workgroup of twelve waves per
+// compute unit (one K step) can have nearly all of it, two workgroups of four waves (two K
+// steps) half each.  Above 64 KB the kernel needs hipFuncAttributeMaxDynamicSharedMemorySize.
+__host__ __device__ constexpr size_t scr_lds_max(int nk) { return nk == 1 ? 156 * 1024 : 78 * 1024; }
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
     const size_t n_cb = (size_t)(k + 31) / 32;
@@ -82,10 +85,11 @@ __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool updat
     s.off_ct = s.off_hneg + n_cb * 32 * 4;             // fp32 centroids, (d, kp)
     s.off_hx = s.off_ct + (size_t)d * s.kp * 4;        // fp32 0.5||c||^2, (kp), +inf past k
     s.off_queue = s.off_hx + (size_t)s.kp * 4;
-    // the queue takes what is left of the 64 KB, up to SCR_QUEUE_MAX entries (none: every
-    // uncertain sample is then handled where it turns up)
+    // the queue takes what is left of the workgroup's LDS, up to SCR_QUEUE_MAX entries (none:
+    // every uncertain sample is then handled where it turns up)
     s.q_words = 16 * nk + 4;
-    const size_t room = s.off_queue < SCR_LDS_MAX ? (SCR_LDS_MAX - s.off_queue) / ((size_t)s.q_words * 4) : 0;
+    const size_t cap = scr_lds_max(nk);
+    const size_t room = s.off_queue < cap ? (cap - s.off_queue) / ((size_t)s.q_words * 4) : 0;
     s.q_cap = (int)(room < (size_t)SCR_QUEUE_MAX ? room : (size_t)SCR_QUEUE_MAX);
     s.total = s.off_queue + (size_t)s.q_cap * s.q_words * 4;
     return s;
@@ -965,7 +969,7 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 
 }  // namespace
 
-// Shapes the screened step covers: d <= 32, everything within 64 KB of LDS, byte offsets
+// Shapes the screened step covers: d <= 32, everything within the workgroup's LDS, byte offsets
 // inside two rows of X_t within 32 bits.  It is chosen where it is the faster one: the all-fp32
 // step pays d / 2 fp32 MFMAs per block of 32 centroids, the screen three fp16 ones plus the
 // split and the certificate whatever d is; measured on 2e6 samples the screen wins from d = 10
@@ -976,7 +980,7 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
     if (d < 1 || d > 32 || k < 16 || n >= ((int64_t)1 << 29)) return false;
     const char* v = std::getenv("KMX_LLOYD_ASSIGN");
     if (v != nullptr && std::strcmp(v, "f32") == 0) return false;
-    if (screen_lds(d, k, (d + 15) / 16, true).off_queue > SCR_LDS_MAX) return false;
+    if (screen_lds(d, k, (d + 15) / 16, true).off_queue > scr_lds_max((d + 15) / 16)) return false;
     if (v != nullptr && std::strcmp(v, "screen") == 0) return true;
     return d >= 10 || (d >= 8 && k >= 64) || (d >= 6 && k >= 128);
 }
@@ -1000,6 +1004,12 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) && aligned16(w) &&
                        aligned16(labels_prev);
     const size_t lds = screen_lds(d, k, nk, UPDATE).total;
+    if (lds > 64 * 1024) {
+        const void* kernel = nk == 1 ? reinterpret_cast<const void*>(&lloyd_screen_kernel<1, UPDATE>)
+                                     : reinterpret_cast<const void*>(&lloyd_screen_kernel<2, UPDATE>);
+        const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int32_t)e;
+    }
     if (nk == 1)
         hipLaunchKernelGGL((lloyd_screen_kernel<1, UPDATE>), dim3((unsigned)grid), dim3(64 * scr_waves(1)),
                            lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,

@@ -82,7 +82,9 @@ def _blobs(n, d, k, seed, offset=0.0, scale=1.0):
 
 
 @pytest.mark.parametrize("shape", [(20_000, 14, 127), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40),
-                                   (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16)])
+                                   (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16),
+                                   # more than 64 KB of LDS per workgroup
+                                   (20_000, 16, 512), (9_000, 14, 600), (6_000, 8, 512), (5_000, 32, 128)])
 def test_screened_step_matches_oracle(cuda, shape):
     n, d, k = shape
     X, w, init = _blobs(n, d, k, seed=n + d)
@@ -114,7 +116,8 @@ def _labels_only(X, C, cuda, roomy=True):
 
 
 @pytest.mark.parametrize("shape", [(20_000, 14, 127), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40),
-                                   (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16)])
+                                   (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16),
+                                   (20_000, 16, 512), (9_000, 14, 600), (5_000, 32, 128)])
 def test_screened_labels_only_match_oracle(cuda, shape):
     n, d, k = shape
     X, _, init = _blobs(n, d, k, seed=n + d + 1)
