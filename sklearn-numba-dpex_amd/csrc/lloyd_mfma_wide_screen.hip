@@ -68,6 +68,7 @@ __device__ __forceinline__ void lds_wait_but4(v4f& a, v4f& b, v4f& c, v4f& d) {
 constexpr int HDR_HMAX = 0;       // bits of max 0.5||c * scale||^2
 constexpr int HDR_SCALE = 1;      // bits of the scale
 constexpr int HDR_UNCERTAIN = 2;  // samples evaluated in fp32 by the last label step
+constexpr int HDR_TILE = 3;       // tiles handed out beyond the first one of every workgroup
 
 // fp16 parts of the scaled centroids in consumption order, scaled -0.5||c||^2, and the header.
 // One thread per (chunk, block, K step, lane); launched with enough blocks of 256 threads.
@@ -128,6 +129,7 @@ __global__ void wide_header_reset_kernel(unsigned int* header) {
     if (threadIdx.x == 0) {
         header[HDR_HMAX] = 0u;
         header[HDR_UNCERTAIN] = 0u;
+        header[HDR_TILE] = 0u;
     }
 }
 
@@ -185,7 +187,14 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                 src + 256 * q, (__attribute__((address_space(3))) void*)(&ctile[buf][256 * q + 64 * wave]), 16, 0, 0);
     };
 
-    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    // Tiles beyond the first are drawn from a counter in memory (a tile takes tens of
+    // microseconds, the draw is requested during the X loads and published by the barrier the
+    // tile needs anyway): with fixed shares the workgroups with one tile more than the others
+    // set the time.
+    __shared__ unsigned int next_tile_s;
+    for (int64_t tile = blockIdx.x; tile < n_tiles;) {
+        unsigned int drawn = 0;
+        if (threadIdx.x == 0) drawn = atomicAdd(header + HDR_TILE, 1u);
         const int64_t i = tile * 128 + wave * 32 + j;
         const bool valid = i < n;
 
@@ -278,7 +287,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
         double s0, s1, s2, s3;  // the winning group's registers, as pairs
         asm volatile("" : "=v"(s0), "=v"(s1), "=v"(s2), "=v"(s3));
 
+        if (threadIdx.x == 0) next_tile_s = gridDim.x + drawn;
         __syncthreads();  // every wave is done with the LDS buffers (previous tile); hneg_s is set
+        const int64_t tile_after = (int64_t)next_tile_s;  // rewritten only after the barriers of this tile
         chunk_issue(0, 0);
         if (n_chunks > 1) chunk_issue(1, 1);
 
@@ -460,6 +471,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_wide_screen_kernel(
                 ranks[i] = atomicAdd(counts + lab, 1);
             }
         }
+        tile = tile_after;
     }
 
     if (changed) atomicAdd(&changed_block, changed);
