@@ -76,7 +76,7 @@ __host__ __device__ constexpr size_t scr_lds_max(int nk) { return nk == 1 ? 156 
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
     const size_t n_cb = (size_t)(k + 31) / 32;
-    // sums: the feature rows, a spare row when d is odd, then the row of the cluster sizes
+    // sums, cluster-major: per cluster the features, a spare word when d is odd, then the size
     const size_t acc = update ? (((size_t)(((d + 1) & ~1) + 1) * k * 8 + 15) & ~(size_t)15) : 0;
     s.off_afh = acc;
     s.off_afl = s.off_afh + n_cb * nk * 64 * 16;
@@ -161,13 +161,16 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     constexpr int G = SCR_GROUP, NG = 16 / SCR_GROUP;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int n_cb = (k + 31) >> 5;
-    // Accumulator rows: feature f in row f, the cluster sizes in row d_even.  For odd d the row
-    // between them takes what the upper half-wave adds for the feature that does not exist
-    // (never read), so that the update needs neither a select nor a guard per lane.
+    // Accumulators: cluster-major, acc_stride = d_even + 1 words per cluster: feature f in word f,
+    // the cluster size in word d_even.  For odd d the word between them takes what the upper
+    // half-wave adds for the feature that does not exist (never read), so that the update needs
+    // neither a select nor a guard per lane; and with the cluster's words next to each other the
+    // atomics of a lane differ by compile-time offsets only.
     const int d_even = (d + 1) & ~1;
-    const int items = (d_even + 1) * k;
+    const int acc_stride = d_even + 1;
+    const int items = acc_stride * k;
     const ScreenLds lay = screen_lds(d, k, NK, UPDATE);
-    unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [(d_even + 1) * k]
+    unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [k][d_even + 1]
     v8h* afh = reinterpret_cast<v8h*>(smem_raw + lay.off_afh);                  // [n_cb][NK][64]
     v8h* afl = reinterpret_cast<v8h*>(smem_raw + lay.off_afl);
     float* hneg = reinterpret_cast<float*>(smem_raw + lay.off_hneg);            // [n_cb][2][16]
@@ -574,30 +577,32 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             }
             // samples past the end carry w = 0: they add zero
             double wd[NC];
+            unsigned long long* mine[NC];  // word h of the label's cluster
 #pragma unroll
-            for (int t = 0; t < NC; ++t) wd[t] = (double)wl[t];
+            for (int t = 0; t < NC; ++t) {
+                wd[t] = (double)wl[t];
+                mine[t] = acc + lab[t] * (uint32_t)acc_stride + h;
+            }
 #pragma unroll
             for (int s = 0; s < NK; ++s)
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int p0 = 16 * s + 2 * i;  // the pair's even feature
                     if (p0 < d) {                   // wave-uniform
-                        // (odd d, last pair: the upper half-wave adds to the spare row)
-                        unsigned long long* rowacc = acc + (p0 + h) * k;
+                        // (odd d, last pair: the upper half-wave adds to the spare word)
 #pragma unroll
                         for (int t = 0; t < NC; ++t) {
                             const double xd = (double)x[s][i][t];
                             // x * w is exact in fp64; one rounding, to a multiple of 2^-q
                             const double v = fma(xd, wd[t], magic[s][i]);
-                            atomicAdd(rowacc + lab[t], to_fixed_q(v, magic[s][i]));
+                            atomicAdd(mine[t] + p0, to_fixed_q(v, magic[s][i]));
                         }
                     }
                 }
             if (h == 0) {
-                unsigned long long* szacc = acc + d_even * k;
 #pragma unroll
                 for (int t = 0; t < NC; ++t)
-                    atomicAdd(szacc + lab[t], to_fixed_q(wd[t] + magic_w, magic_w));
+                    atomicAdd(mine[t] + d_even, to_fixed_q(wd[t] + magic_w, magic_w));
             }
         }
     };
@@ -816,7 +821,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 const double wq = (double)__uint_as_float(entry[Q_WEIGHT]);
                 if (lane <= d) {
                     const double term = lane < d ? fma((double)xe[lane], wq, magic_lane) : wq + magic_lane;
-                    atomicAdd(acc + (lane < d ? lane : d_even) * k + bc, to_fixed_q(term, magic_lane));
+                    atomicAdd(acc + bc * acc_stride + (lane < d ? lane : d_even), to_fixed_q(term, magic_lane));
                 }
             }
         }
@@ -829,13 +834,14 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         atomicAdd(uncertain_count, uncertain_block);
     if (UPDATE) {
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
-        const int n_out = (d + 1) * k, skip = (d_even - d) * k;  // gsum has no spare row
+        const int n_out = (d + 1) * k;  // gsum is feature-major, (d + 1, k), and has no spare row
         // every workgroup starts at another word: the workgroups finish together and would
         // otherwise queue up on the same addresses
         const int rot = (int)(((int64_t)blockIdx.x * n_out) / gridDim.x);
         for (int jy = threadIdx.x; jy < n_out; jy += THREADS) {
             const int jx = jy + rot < n_out ? jy + rot : jy + rot - n_out;
-            const unsigned long long v = acc[jx < d * k ? jx : jx + skip];
+            const int f = jx / k, c = jx - f * k;
+            const unsigned long long v = acc[c * acc_stride + (f < d ? f : d_even)];
             if (v) atomicAdd(gsum + jx, v);
         }
     }
