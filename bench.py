@@ -10,7 +10,7 @@ Prints ONE JSON line: iterations/s, plus
   roofline      the fused-step kernel against the roofline it has to approach, from HIP events
                 recorded around that kernel on its stream (kmx_lloyd_iter_timed): HBM for the
                 kernel that screens the labels on the fp16 matrix cores (variant 61), the fp32
-                MFMA peak for the all-fp32 kernel (variant 31, KMX_LLOYD_ASSIGN=f32);
+                MFMA peak for the all-fp32 kernel (variant 31, KMX_FLAG_LABELS_F32);
   roofline_other_bound  the same kernel against the other of the two;
   cpu_baseline  scikit-learn's OpenMP/Cython Lloyd on the same data on this host's cores;
   kmeanspp_ms   kmeans++ seeding time on configs[3] (1,000,000 x 64, k = 256).
@@ -30,6 +30,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3    # MI355X fp32, vector and matrix
+RAMP_MS = 60.0              # untimed iterations before every timed region, for the GPU clocks
+FLAG_LABELS_F32 = 0x10      # KMX_FLAG_LABELS_F32: every product of the fp32 paths in fp32
 
 
 def log(*a):
@@ -64,7 +66,11 @@ def check_labels(labels, X, centers, chunk=20_000):
     return ties
 
 
-def gpu_lloyd(cfg, steps, warmup):
+def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
+    """Times `steps` Lloyd iterations of one fit: a throw-away run first brings the GPU clocks
+    up (at least RAMP_MS of iterations, whatever --warmup says), then the fit restarts from the
+    initial centroids, runs `warmup` untimed iterations and `steps` timed ones, i.e. the timed
+    region is iterations warmup + 1 .. warmup + steps of a fit."""
     import torch
 
     from sklearn_numba_dpex_amd import _capi
@@ -81,7 +87,8 @@ def gpu_lloyd(cfg, steps, warmup):
     labels = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(2)]
     sizes = torch.empty(k, dtype=X_t.dtype, device=dev)
     empty = torch.empty(k, dtype=torch.int32, device=dev)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    plan = _capi.lloyd_plan(n, d, k, dc, flags)
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     stream = _capi.current_stream()
     status = _capi.LloydStatus()
@@ -104,7 +111,7 @@ def gpu_lloyd(cfg, steps, warmup):
                                    "the timed region would include no-op launches")
             checked += it
         cent[0].copy_(cent_init)
-        _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc,
+        _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]),
                                        RESTART + 8, 0.0, stream), "init")
         it = 0
 
@@ -113,8 +120,8 @@ def gpu_lloyd(cfg, steps, warmup):
         if it >= RESTART:
             restart()
         a, b = it % 2, (it + 1) % 2
-        args = (ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]), ptr(labels[b]),
-                ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, dc, stream)
+        args = (plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]), ptr(labels[b]),
+                ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream)
         if ms is None:
             _capi.check(lib.kmx_lloyd_iter(*args), "iter")
         else:
@@ -122,6 +129,16 @@ def gpu_lloyd(cfg, steps, warmup):
         it += 1
         done += 1
 
+    # clock ramp: the GPU clocks need tens of milliseconds of load to come up; a throw-away
+    # run provides them, then the fit proper starts over from the initial centroids
+    restart()
+    ramp_iters = 0
+    t_ramp = time.perf_counter()
+    while (time.perf_counter() - t_ramp) * 1e3 < RAMP_MS and ramp_iters < RESTART - 50:
+        for _ in range(50):
+            enqueue()
+        ramp_iters += 50
+        torch.cuda.synchronize()
     restart()
     for _ in range(warmup):
         enqueue()
@@ -150,7 +167,9 @@ def gpu_lloyd(cfg, steps, warmup):
 
     # samples the last iteration evaluated in fp32 because its fp16 screen could not certify them
     rechecked = ctypes.c_uint32(0)
-    _capi.check(lib.kmx_lloyd_recheck_count(ptr(ws), n, d, k, dc, ctypes.byref(rechecked), stream), "recheck_count")
+    _capi.check(lib.kmx_lloyd_recheck_count(plan, ptr(ws), ctypes.byref(rechecked), stream), "recheck_count")
+    if not gates:
+        return elapsed, kernel_ms, 0, plan.variant, int(rechecked.value), ramp_iters
 
     # parity gate 1: the labels the last Lloyd iteration wrote, against exact fp64 distances to
     # the centroids it started from, on a slice
@@ -160,16 +179,56 @@ def gpu_lloyd(cfg, steps, warmup):
     # parity gate 2: kmx_assign_labels for the centroids the last iteration produced
     cur = cent[it % 2].T.cpu().numpy()
     lab = torch.empty(n, dtype=torch.int32, device=dev)
-    aws = lib.kmx_assign_workspace_bytes_for(n, d, k, dc)
+    aws = lib.kmx_assign_workspace_bytes_for(n, d, k, dc, flags)
     aws_t = torch.empty(aws, dtype=torch.uint8, device=dev)
     _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(X_t.new_tensor(cur.T.copy())), ptr(lab), ptr(aws_t), aws,
-                                      n, d, k, dc, stream), "assign")
+                                      n, d, k, dc, flags, stream), "assign")
     ties = ties_iter + check_labels(lab[:m].cpu().numpy(), X[:m], cur)
-    variant = lib.kmx_lloyd_kernel_variant(n, d, k, dc)
-    return elapsed, kernel_ms, ties, variant, int(rechecked.value)
+    return elapsed, kernel_ms, ties, plan.variant, int(rechecked.value), ramp_iters
 
 
-def gpu_lloyd_step_time(cfg, reps, consecutive=False):
+def gpu_measured_peaks():
+    """What this GPU reaches on the simplest kernels (probe kernels of the library, HIP events on
+    the launch stream): a 1 GiB device-to-device copy, a read-only pass over 1 GiB, and streams
+    of independent fp32 / fp16 / fp64 matrix-core instructions."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    dev = torch.device("cuda:0")
+    stream = _capi.current_stream()
+    nbytes = 1 << 30
+    src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    scratch = torch.zeros(1 << 20, dtype=torch.uint8, device=dev)
+
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    t_copy = timed(lambda: _capi.check(lib.kmx_probe_copy(ptr(src), ptr(dst), nbytes, stream), "probe_copy"), 10)
+    t_read = timed(lambda: _capi.check(lib.kmx_probe_read(ptr(src), nbytes, ptr(scratch), stream), "probe_read"), 10)
+    out = {"what": "probe kernels of the library on this GPU: 1 GiB copy (read + written bytes), 1 GiB read-only "
+                   "stream, independent MFMA chains (two waves per SIMD)",
+           "copy_GBps": 2 * nbytes / t_copy / 1e9, "read_GBps": nbytes / t_read / 1e9}
+    flops = ctypes.c_double(0.0)
+    for kind, name in ((0, "mfma_f32_TFLOPs"), (1, "mfma_f16_TFLOPs"), (2, "mfma_f64_TFLOPs")):
+        t = timed(lambda: _capi.check(lib.kmx_probe_mfma(kind, 20000, ptr(scratch), ctypes.byref(flops), stream),
+                                      "probe_mfma"), 3)
+        out[name] = flops.value / t / 1e12
+    del src, dst
+    return out
+
+
+def gpu_lloyd_step_time(cfg, reps, consecutive=False, flags=0):
     """Per-kernel times of a Lloyd iteration, mean ms of (fused step, reduce, finalize).
 
     ONE iteration from the configuration's initial centroids, the state re-initialised before
@@ -186,7 +245,8 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False):
     X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
     n, d = X.shape
     dc = _capi.dtype_code(X.dtype)
-    variant = lib.kmx_lloyd_kernel_variant(n, d, k, dc)
+    plan = _capi.lloyd_plan(n, d, k, dc, flags)
+    variant = plan.variant
     X_rm = torch.as_tensor(X, device=dev)
     X_t = X_rm.T.contiguous()
     if variant != 42:
@@ -197,7 +257,7 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False):
     labels = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(2)]
     sizes = torch.empty(k, dtype=X_t.dtype, device=dev)
     empty = torch.empty(k, dtype=torch.int32, device=dev)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     stream = _capi.current_stream()
     ms = (ctypes.c_float * 3)()
@@ -210,7 +270,7 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False):
         def run(max_iter):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            n_iter = drivers.lloyd(X_t, w_d, cent[0], max_iter=max_iter, tol=0.0)[3]
+            n_iter = drivers.lloyd(X_t, w_d, cent[0], max_iter=max_iter, tol=0.0, flags=flags)[3]
             torch.cuda.synchronize()
             return time.perf_counter() - t0, int(n_iter)
 
@@ -221,11 +281,11 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False):
             raise RuntimeError(f"the run converged after {it_long} iterations: nothing to time")
         wall_ms = (t_long - t_short) / (it_long - it_short) * 1e3
     for rep in range(reps + 2):
-        _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, 10, 0.0,
+        _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 10, 0.0,
                                        stream), "init")
-        _capi.check(lib.kmx_lloyd_iter_timed(ptr(X_t), ptr(X_rm), ptr(w_d), ptr(cent[0]), ptr(cent[1]),
+        _capi.check(lib.kmx_lloyd_iter_timed(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(cent[0]), ptr(cent[1]),
                                              ptr(labels[0]), ptr(labels[1]), ptr(sizes), ptr(empty), ptr(ws),
-                                             ws_bytes, n, d, k, dc, stream, ms), "iter_timed")
+                                             ws_bytes, stream, ms), "iter_timed")
         if rep >= 2:
             acc += np.array(list(ms))
     if consecutive:
@@ -244,11 +304,7 @@ def extra_configs():
     kms, variant, wall_ms = gpu_lloyd_step_time(c3, 10, consecutive=True)
     # the same step with every product in fp32 on the matrix cores (the label kernel the default
     # path falls back to for the samples its fp16 screen cannot certify): MFMA utilisation
-    os.environ["KMX_LLOYD_ASSIGN"] = "f32"
-    try:
-        kms32, _ = gpu_lloyd_step_time(c3, 5)
-    finally:
-        os.environ.pop("KMX_LLOYD_ASSIGN", None)
+    kms32, _ = gpu_lloyd_step_time(c3, 5, flags=FLAG_LABELS_F32)
     flops = lloyd_flops(n, d, c3["k"])
     out["config3"] = {
         "workload": f"configs[2]: Lloyd n={n} d={d} k={c3['k']} fp32; ms_per_iter over iterations 6-15 of the "
@@ -257,7 +313,7 @@ def extra_configs():
         "labels": "fp16 matrix-core screen, certified per sample, all-fp32 matrix-core kernel where not certified",
         "kernel_ms": {"fused_step": float(kms[0]), "reduce": float(kms[1]), "finalize": float(kms[2])},
         "fused_step_fp32_equivalent_TFLOPs": flops / (kms[0] * 1e-3) / 1e12,
-        "all_fp32": {"switch": "KMX_LLOYD_ASSIGN=f32", "fused_step_ms": float(kms32[0]),
+        "all_fp32": {"switch": "KMX_FLAG_LABELS_F32", "fused_step_ms": float(kms32[0]),
                      "fused_step_TFLOPs": flops / (kms32[0] * 1e-3) / 1e12,
                      "fused_step_frac_of_fp32_peak": flops / (kms32[0] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS},
     }
@@ -391,8 +447,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=100,
-                    help="untimed iterations; the default also lets the GPU clocks ramp up (tens of ms)")
+    ap.add_argument("--warmup", type=int, default=5,
+                    help="untimed iterations of the fit before the timed ones (the GPU clocks are brought up "
+                         "by a separate throw-away run, whatever this is)")
     ap.add_argument("--n", type=int, default=5_000_000, help="samples (default: the full configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kpp", action="store_true", help="skip the kmeans++ leg")
@@ -422,7 +479,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    elapsed, kernel_ms, ties, variant, rechecked = gpu_lloyd(cfg, args.steps, args.warmup)
+    elapsed, kernel_ms, ties, variant, rechecked, ramp_iters = gpu_lloyd(cfg, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     iters_per_s = args.steps / elapsed
     fused_s = kernel_ms[0] * 1e-3
@@ -460,11 +517,28 @@ def main():
     }
     # Variant 61 screens the labels on the fp16 matrix cores: the fp32 contraction that bounded
     # variant 31 is gone, and what is left to approach is the HBM time of the algorithmic bytes.
-    # Variant 31 (KMX_LLOYD_ASSIGN=f32) multiplies in fp32 and is priced against the fp32 MFMA peak.
+    # Variant 31 (KMX_FLAG_LABELS_F32) multiplies in fp32 and is priced against the fp32 MFMA peak.
     roofline, roofline_other = (hbm_roof, mfma_roof) if int(variant) == 61 else (mfma_roof, hbm_roof)
     if int(variant) == 61:
         mfma_roof["note"] = ("2 n d k flops of the exact contraction over the fp32 MFMA peak, for comparison "
                              "with the all-fp32 kernel; this kernel runs 3 fp16 products per fp32 one instead")
+
+    # the same fit with every product taken in fp32 (variant 31), timed the same way
+    e32, kms32, _, variant32, _, _ = gpu_lloyd(cfg, args.steps, args.warmup, flags=FLAG_LABELS_F32, gates=False)
+    all_fp32 = {
+        "switch": "KMX_FLAG_LABELS_F32", "kernel_variant": int(variant32),
+        "ms_per_step": e32 / args.steps * 1e3, "iters_per_sec": args.steps / e32,
+        "fused_step_ms": float(kms32[0]),
+        "fused_step_TFLOPs": flops / (kms32[0] * 1e-3) / 1e12,
+        "frac_of_fp32_peak": flops / (kms32[0] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS,
+    }
+    log(f"[bench] every product in fp32: {all_fp32['ms_per_step']:.4f} ms/iter, fused step "
+        f"{kms32[0]:.4f} ms = {all_fp32['frac_of_fp32_peak']:.3f} of fp32 peak")
+    peaks = gpu_measured_peaks()
+    log("[bench] measured peaks: " + ", ".join(f"{k2} {v:.1f}" for k2, v in peaks.items() if k2 != "what"))
+    hbm_roof["frac_of_measured_peak"] = hbm_roof["achieved"] / peaks["read_GBps"]
+    mfma_roof["frac_of_measured_peak"] = mfma_roof["achieved"] / peaks["mfma_f32_TFLOPs"]
+    all_fp32["frac_of_measured_fp32_peak"] = all_fp32["fused_step_TFLOPs"] / peaks["mfma_f32_TFLOPs"]
 
     out = {
         "metric": "lloyd_iterations_per_sec",
@@ -473,6 +547,8 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "clock_ramp_iters": int(ramp_iters),
+        "timed_iterations": f"{args.warmup + 1}..{args.warmup + args.steps} of a fit from the initial centroids",
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -489,6 +565,8 @@ def main():
                       "finalize": float(kernel_ms[2])},
         "roofline": roofline,
         "roofline_other_bound": roofline_other,
+        "all_fp32": all_fp32,
+        "measured_peaks": peaks,
         "fp32_evaluated_samples": {"count": int(rechecked), "fraction_of_n": rechecked / n},
         "parity": {"near_tie_label_differences": int(ties), "checked_samples": min(n, 200_000)},
     }

@@ -20,6 +20,8 @@
  *   - Return value: 0 on success, a negative KMX_ERR_* for rejected arguments, or a positive
  *     hipError_t reported by the runtime.  Nothing throws or exits.
  *   - Calls that share a workspace must be issued on one stream (or otherwise ordered).
+ *   - The library keeps no selection state and reads no environment variable: which kernel
+ *     runs follows from the shape and from the caller's `flags` (KMX_FLAG_*) alone.
  */
 #ifndef MI355X_KMEANS_H
 #define MI355X_KMEANS_H
@@ -42,7 +44,9 @@ extern "C" {
 #define KMX_ERR_BAD_ARGUMENT (-5)   /* k > n for top-k, unknown op code, ...               */
 #define KMX_ERR_UNSUPPORTED (-6)    /* shape outside what a specialised kernel covers      */
 
-#define KMX_ABI_VERSION 1
+#define KMX_ERR_BAD_PLAN (-7)       /* kmx_lloyd_plan not made by kmx_lloyd_plan_init, or edited */
+
+#define KMX_ABI_VERSION 2
 int32_t kmx_abi_version(void);
 const char* kmx_error_string(int32_t code);
 
@@ -70,15 +74,58 @@ typedef struct kmx_lloyd_status {
     int64_t reserved[2];
 } kmx_lloyd_status;       /* 64 bytes */
 
-size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype);
+/* Kernel selection: `flags` of kmx_lloyd_plan_init and kmx_assign_labels.  0 leaves every
+ * choice to the library (the fastest kernel it has for the shape).  The reference has no
+ * counterpart: its kernels are specialised by the JIT from the shape alone
+ * (kmeans/drivers.py:103-135). */
+#define KMX_FLAG_PATH_MASK 0x0000000fu
+#define KMX_FLAG_PATH_AUTO 0x0u
+#define KMX_FLAG_PATH_STREAM 0x1u      /* features re-read per centroid window                */
+#define KMX_FLAG_PATH_REGISTER 0x2u    /* samples in registers, vector ALU                    */
+#define KMX_FLAG_PATH_MFMA 0x3u        /* matrix cores wherever the shape allows              */
+#define KMX_FLAG_LABELS_MASK 0x00000030u
+#define KMX_FLAG_LABELS_AUTO 0x00u
+#define KMX_FLAG_LABELS_F32 0x10u      /* every product of the fp32 paths taken in fp32       */
+#define KMX_FLAG_LABELS_SCREEN 0x20u   /* fp16 screen + fp32 certificate wherever it fits     */
+#define KMX_FLAG_WGS_PER_CU(x) (((uint32_t)(x) & 0xfu) << 8)  /* 1..8 workgroups per CU; 0: default */
+#define KMX_FLAG_COLS(x) (((uint32_t)(x) & 0x7u) << 12)       /* 2 | 4 sample columns per lane; 0: default */
+
+/* What kmx_lloyd_init / kmx_lloyd_iter / kmx_lloyd_finalize run for one problem: the shape, the
+ * caller's flags, the kernel variant chosen from them and the workspace the variant needs.
+ * Plain host memory owned by the caller, filled by kmx_lloyd_plan_init and passed unchanged to
+ * the other calls: the workspace layout is a function of the plan, so the calls of one fit
+ * cannot disagree about it.  A plan that was not made by kmx_lloyd_plan_init of this library
+ * version, or whose fields were edited afterwards, is rejected with KMX_ERR_BAD_PLAN. */
+typedef struct kmx_lloyd_plan {
+    uint32_t magic;
+    int32_t abi_version;
+    int64_t n;
+    int32_t d;
+    int32_t k;
+    int32_t dtype;
+    uint32_t flags;
+    int32_t variant;           /* 10 * path + accumulation, see kmx_lloyd_kernel_variant      */
+    int32_t reserved;
+    uint64_t workspace_bytes;  /* bytes of device memory kmx_lloyd_init and the others need   */
+    uint64_t check;            /* over the fields above                                       */
+} kmx_lloyd_plan;              /* 56 bytes */
+
+/* Fills `plan` for n samples, d features, k clusters.  KMX_ERR_BAD_SHAPE, KMX_ERR_BAD_DTYPE or
+ * KMX_ERR_BAD_ARGUMENT (flags that name no choice).  Host only: no device work.
+ * Replaces the kernel factories' specialisation on the shape, kmeans/drivers.py:103-135. */
+int32_t kmx_lloyd_plan_init(kmx_lloyd_plan* plan, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                            uint32_t flags);
+
+/* plan.workspace_bytes / plan.variant without a plan (0 / a negative code for bad arguments). */
+size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* Resets the loop state, packs the initial centroids (+ their half squared norms), clears
  * the accumulators and, for the fixed-point accumulation of the fp32 matrix-core path, takes
  * max|x| per feature and max|w| (one pass over X_t and sample_weight).
  * Replaces the set-up part of lloyd(), kmeans/drivers.py:146-184. */
-int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
-                       const void* sample_weight, const void* centroids_t, int64_t n, int32_t d,
-                       int32_t k, int32_t dtype, int32_t max_iter, double tol, void* stream);
+int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t workspace_bytes,
+                       const void* X_t, const void* sample_weight, const void* centroids_t,
+                       int32_t max_iter, double tol, void* stream);
 
 /* One Lloyd iteration, enqueued as two kernels (three for shapes whose partial sums do not
  * fit in LDS):
@@ -95,7 +142,7 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
  * make_centroid_shifts_kernel (kmeans/kernels/utils.py:79-110) and the loop body of
  * lloyd(), kmeans/drivers.py:188-343.
  *   X_rowmajor       IN   (n, d)  optional (may be NULL) row-major copy of the same data; used
- *                                 only by the wide fp32 path (kmx_lloyd_kernel_variant == 42),
+ *                                 only by the wide fp32 path (plan.variant == 42),
  *                                 which then sums each cluster's rows instead of issuing one
  *                                 global atomic per (sample, feature)
  *   centroids_t      IN   (d, k)  centroids the labels are computed from: the array given to
@@ -107,10 +154,10 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
  *   labels           OUT  (n)
  *   cluster_sizes    OUT  (k)     sum of weights per cluster
  *   empty_clusters   OUT  (k)     ids of empty clusters, ascending, first status.n_empty valid */
-int32_t kmx_lloyd_iter(const void* X_t, const void* X_rowmajor, const void* sample_weight,
-                       const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
-                       void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
-                       size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+int32_t kmx_lloyd_iter(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
+                       const void* sample_weight, const void* centroids_t, void* new_centroids_t,
+                       const uint32_t* labels_prev, uint32_t* labels, void* cluster_sizes,
+                       uint32_t* empty_clusters, void* workspace, size_t workspace_bytes,
                        void* stream);
 
 /* kmx_lloyd_iter with HIP events recorded on `stream` around each of its kernels.  Waits for
@@ -118,18 +165,18 @@ int32_t kmx_lloyd_iter(const void* X_t, const void* X_rowmajor, const void* samp
  * finalisation) to kernel_ms_host[0..2].  For benchmarks and profiling; it has no
  * counterpart in the reference, whose benchmark only times a whole fit
  * (benchmark/kmeans.py:163-165). */
-int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void* sample_weight,
-                             const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+int32_t kmx_lloyd_iter_timed(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
+                             const void* sample_weight, const void* centroids_t,
+                             void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
-                             size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
-                             void* stream, float* kernel_ms_host);
+                             size_t workspace_bytes, void* stream, float* kernel_ms_host);
 
 /* Second half of (2) alone, for the iteration that stopped with KMX_NEED_RELOCATION after
  * the host has relocated the empty clusters: sums / sizes, shift, convergence test, state
  * back to KMX_RUNNING (or a terminal state).  kmeans/drivers.py:275,326-343. */
-int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t, const void* cluster_sizes,
-                           void* workspace, size_t workspace_bytes, int32_t d, int32_t k,
-                           int32_t dtype, void* stream);
+int32_t kmx_lloyd_finalize(const kmx_lloyd_plan* plan, const void* centroids_t,
+                           void* new_centroids_t, const void* cluster_sizes, void* workspace,
+                           size_t workspace_bytes, void* stream);
 
 /* Copies the status to host memory and waits for it (the only synchronising call). */
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
@@ -138,8 +185,8 @@ int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_ho
  * whose label the screen of the last completed iteration could not certify and that were
  * evaluated in plain fp32 instead; 0 for the other variants.  Synchronises the stream.
  * It has no counterpart in the reference (diagnostics). */
-int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int32_t k,
-                                int32_t dtype, uint32_t* count_host, void* stream);
+int32_t kmx_lloyd_recheck_count(const kmx_lloyd_plan* plan, const void* workspace,
+                                uint32_t* count_host, void* stream);
 
 /* Diagnostics of kernel variant 61, for tests of its certificate: the approximate scores
  * <x, c> - 0.5||c||^2 exactly as the fused step forms them on the fp16 matrix cores (same
@@ -154,11 +201,12 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
                           float* half_norms, float* scale, void* scratch, int64_t n, int32_t d,
                           int32_t k, void* stream);
 
-/* Which fused-step kernel kmx_lloyd_iter uses for a shape, as 10 * path + accumulation:
+/* Which fused-step kernel kmx_lloyd_iter uses for a shape and flags, as 10 * path + accumulation:
  * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32) with the
- * centroids resident in LDS, 4 = MFMA (fp32) with samples in registers and centroids streamed;
+ * centroids resident in LDS, 4 = MFMA (fp32) with samples in registers and centroids streamed,
+ * 5 = MFMA (fp64), 6 = path 3 with the labels screened on the fp16 matrix cores;
  * accumulation 1 = workgroup-private LDS accumulators, 2 = global sums. */
-int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype);
+int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* ------------------------------------------------------------------------------------ *
  * Labels, inertia, distances                                                            *
@@ -170,14 +218,14 @@ size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype);
  * shapes screen the labels on the fp16 matrix cores and need room for a list of samples.  Never
  * smaller than kmx_assign_workspace_bytes, which always suffices.  It has no counterpart in the
  * reference (workspaces belong to this library). */
-size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype);
+size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* labels[i] = argmin_c (0.5||c||^2 - <x_i, c>).  Replaces
  * make_label_assignment_fixed_window_kernel (kmeans/kernels/compute_labels.py:18-185) and the
  * half-norm call before it (kmeans/drivers.py:657-669). */
 int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
                           void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
-                          int32_t k, int32_t dtype, void* stream);
+                          int32_t k, int32_t dtype, uint32_t flags, void* stream);
 
 /* out[i] = w_i * sum_f (x_fi - c_f,label_i)^2, features in order; sample_weight may be NULL
  * for unit weights (the relocation pass).  Replaces make_compute_inertia_kernel
@@ -328,6 +376,22 @@ int32_t kmx_count_distinct_clusters(const uint32_t* labels, int32_t* seen, int32
 /* out (m, q) = X (m, p) @ Y_t (q, p)^T.  make_matmul_2d_kernel, common/matmul.py:13-567. */
 int32_t kmx_matmul(const void* X, const void* Y_t, void* out, int32_t m, int32_t p, int32_t q,
                    int32_t dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------ *
+ * Machine probes (benchmarks only)                                                      *
+ * ------------------------------------------------------------------------------------ */
+
+/* What this GPU reaches on the simplest kernels, so that a benchmark can price the KMeans
+ * kernels against measured ceilings next to the datasheet ones: a device-to-device copy
+ * (n_bytes read + n_bytes written), a read-only pass over n_bytes, and a stream of independent
+ * matrix-core instructions (kind 0: v_mfma_f32_32x32x2_f32, 1: v_mfma_f32_32x32x16_f16,
+ * 2: v_mfma_f64_16x16x4_f64; *flops_host receives the flops of the launch).  The caller times
+ * them on `stream`.  n_bytes: a multiple of 16, pointers 16-byte aligned; scratch: 1 MiB of
+ * device memory.  They have no counterpart in the reference, which publishes no roofline
+ * figures (benchmark/kmeans.py only times whole fits). */
+int32_t kmx_probe_copy(const void* src, void* dst, size_t n_bytes, void* stream);
+int32_t kmx_probe_read(const void* src, size_t n_bytes, void* scratch, void* stream);
+int32_t kmx_probe_mfma(int32_t kind, int32_t iters, void* scratch, double* flops_host, void* stream);
 
 #ifdef __cplusplus
 }

@@ -25,7 +25,25 @@ KMX_CONVERGED_TOL = 2
 KMX_MAX_ITER = 3
 KMX_NEED_RELOCATION = 4
 
-ABI_VERSION = 1
+KMX_ERR_BAD_PLAN = -7
+
+# kernel selection flags (KMX_FLAG_* of the header)
+FLAG_PATH_STREAM = 0x1
+FLAG_PATH_REGISTER = 0x2
+FLAG_PATH_MFMA = 0x3
+FLAG_LABELS_F32 = 0x10
+FLAG_LABELS_SCREEN = 0x20
+
+
+def flag_wgs_per_cu(x):
+    return (int(x) & 0xF) << 8
+
+
+def flag_cols(x):
+    return (int(x) & 0x7) << 12
+
+
+ABI_VERSION = 2
 
 LIB_NAME = "libmi355x_kmeans.so"
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
@@ -50,28 +68,52 @@ class LloydStatus(ctypes.Structure):
 
 assert ctypes.sizeof(LloydStatus) == 64
 
+
+class LloydPlan(ctypes.Structure):
+    """Mirror of kmx_lloyd_plan: shape, flags, chosen kernel variant, workspace size."""
+
+    _fields_ = [
+        ("magic", ctypes.c_uint32),
+        ("abi_version", c_int32),
+        ("n", c_int64),
+        ("d", c_int32),
+        ("k", c_int32),
+        ("dtype", c_int32),
+        ("flags", ctypes.c_uint32),
+        ("variant", c_int32),
+        ("reserved", c_int32),
+        ("workspace_bytes", ctypes.c_uint64),
+        ("check", ctypes.c_uint64),
+    ]
+
+
+assert ctypes.sizeof(LloydPlan) == 56
+
 _P = c_void_p
 _I32 = c_int32
 _I64 = c_int64
 _SZ = c_size_t
+_U32 = ctypes.c_uint32
+_PLAN = POINTER(LloydPlan)
 
 # name -> (restype, argtypes); must list every function of include/mi355x_kmeans.h
 SIGNATURES = {
     "kmx_abi_version": (_I32, []),
     "kmx_error_string": (c_char_p, [_I32]),
-    "kmx_lloyd_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32]),
-    "kmx_lloyd_init": (_I32, [_P, _SZ, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, c_double, _P]),
-    "kmx_lloyd_iter": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
-    "kmx_lloyd_iter_timed": (_I32, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P,
+    "kmx_lloyd_plan_init": (_I32, [_PLAN, _I64, _I32, _I32, _I32, _U32]),
+    "kmx_lloyd_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _U32]),
+    "kmx_lloyd_init": (_I32, [_PLAN, _P, _SZ, _P, _P, _P, _I32, c_double, _P]),
+    "kmx_lloyd_iter": (_I32, [_PLAN, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "kmx_lloyd_iter_timed": (_I32, [_PLAN, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P,
                                     POINTER(ctypes.c_float)]),
-    "kmx_lloyd_finalize": (_I32, [_P, _P, _P, _P, _SZ, _I32, _I32, _I32, _P]),
+    "kmx_lloyd_finalize": (_I32, [_PLAN, _P, _P, _P, _P, _SZ, _P]),
     "kmx_lloyd_status_read": (_I32, [_P, POINTER(LloydStatus), _P]),
-    "kmx_lloyd_recheck_count": (_I32, [_P, _I64, _I32, _I32, _I32, POINTER(ctypes.c_uint32), _P]),
+    "kmx_lloyd_recheck_count": (_I32, [_PLAN, _P, POINTER(ctypes.c_uint32), _P]),
     "kmx_screen_scores": (_I32, [_P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _P]),
-    "kmx_lloyd_kernel_variant": (_I32, [_I64, _I32, _I32, _I32]),
+    "kmx_lloyd_kernel_variant": (_I32, [_I64, _I32, _I32, _I32, _U32]),
     "kmx_assign_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
-    "kmx_assign_workspace_bytes_for": (_SZ, [_I64, _I32, _I32, _I32]),
-    "kmx_assign_labels": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
+    "kmx_assign_workspace_bytes_for": (_SZ, [_I64, _I32, _I32, _I32, _U32]),
+    "kmx_assign_labels": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _U32, _P]),
     "kmx_per_sample_inertia": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_euclidean_distances": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_relocate_empty_clusters": (_I32, [_P, _P, _P, _P, _P, _I32, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
@@ -100,6 +142,9 @@ SIGNATURES = {
     "kmx_is_same_clustering": (_I32, [_P, _P, _P, _P, _I64, _I32, _P]),
     "kmx_count_distinct_clusters": (_I32, [_P, _P, _P, _I64, _I32, _P]),
     "kmx_matmul": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _P]),
+    "kmx_probe_copy": (_I32, [_P, _P, _SZ, _P]),
+    "kmx_probe_read": (_I32, [_P, _SZ, _P, _P]),
+    "kmx_probe_mfma": (_I32, [_I32, _I32, _P, POINTER(c_double), _P]),
 }
 
 
@@ -135,6 +180,35 @@ def error_string(code):
 def check(code, where):
     if code != 0:
         raise KmxError(code, where)
+
+
+def _flags_from_environment():
+    """Kernel selection for callers that pass no flags, from KMX_LLOYD_ASSIGN = f32 | screen,
+    KMX_LLOYD_VARIANT = stream | register | mfma, KMX_LLOYD_WGS_PER_CU = 1..8 and
+    KMX_LLOYD_COLS = 2 | 4.  Read ONCE, when this module is imported: the library itself never
+    looks at the environment, and later changes of these variables have no effect."""
+    flags = 0
+    flags |= {"f32": FLAG_LABELS_F32, "screen": FLAG_LABELS_SCREEN}.get(os.environ.get("KMX_LLOYD_ASSIGN", ""), 0)
+    flags |= {"stream": FLAG_PATH_STREAM, "register": FLAG_PATH_REGISTER,
+              "mfma": FLAG_PATH_MFMA}.get(os.environ.get("KMX_LLOYD_VARIANT", ""), 0)
+    wgs = os.environ.get("KMX_LLOYD_WGS_PER_CU", "")
+    if wgs.isdigit() and 1 <= int(wgs) <= 8:
+        flags |= flag_wgs_per_cu(int(wgs))
+    cols = os.environ.get("KMX_LLOYD_COLS", "")
+    if cols in ("2", "4"):
+        flags |= flag_cols(int(cols))
+    return flags
+
+
+DEFAULT_FLAGS = _flags_from_environment()
+
+
+def lloyd_plan(n, d, k, dtype_code_, flags=None):
+    """A filled kmx_lloyd_plan (flags=None: the import-time defaults)."""
+    plan = LloydPlan()
+    check(lib.kmx_lloyd_plan_init(ctypes.byref(plan), int(n), int(d), int(k), int(dtype_code_),
+                                  DEFAULT_FLAGS if flags is None else int(flags)), "kmx_lloyd_plan_init")
+    return plan
 
 
 def dtype_code(dtype):

@@ -547,7 +547,7 @@ __global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words)
 
 // Workgroups of a vector-ALU fused step (also the number of partial slots it fills).
 int lloyd_fused_grid(const LloydLayout& L, int64_t n, int d, int dtype) {
-    if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n);
+    if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n, L.wgs_per_cu, L.cols);
     const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype) : 2;
     const int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
     const int cap = L.grid_cap(kmx_num_cus());
@@ -574,7 +574,7 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_MFMA_F64) {
         (void)kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
-                                      status, n, d, k, ACC != ACC_NONE, stream);
+                                      status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, stream);
     } else if (L.variant == KMX_VARIANT_REGISTER) {
 #define KMX_REG_CASE(DR, RR)                                                                    \
     launch_reg<T, DR, RR, ACC>(L, X_t, w, cpack, half_norms, labels_prev, labels, partial, status, \
@@ -706,33 +706,95 @@ const char* kmx_error_string(int32_t code) {
         case KMX_ERR_WORKSPACE: return "workspace too small";
         case KMX_ERR_BAD_ARGUMENT: return "invalid argument";
         case KMX_ERR_UNSUPPORTED: return "shape not supported by this kernel";
+        case KMX_ERR_BAD_PLAN: return "kmx_lloyd_plan not made by kmx_lloyd_plan_init of this library, or edited";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }
 
-size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype) {
-    if (n <= 0 || d <= 0 || k <= 0 || (dtype != KMX_F32 && dtype != KMX_F64)) return 0;
-    return lloyd_layout(n, d, k, dtype).total;
-}
+// ---- plan: shape + flags + what follows from them; validated by every call that takes one
 
-int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype) {
+static uint64_t plan_check_value(const kmx_lloyd_plan& p) {
+    // FNV-1a over the fields in declaration order (not over padding)
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&h](uint64_t v) {
+        for (int i = 0; i < 8; ++i) {
+            h ^= (v >> (8 * i)) & 0xffu;
+            h *= 1099511628211ull;
+        }
+    };
+    mix(p.magic);
+    mix((uint64_t)(uint32_t)p.abi_version);
+    mix((uint64_t)p.n);
+    mix((uint64_t)(uint32_t)p.d);
+    mix((uint64_t)(uint32_t)p.k);
+    mix((uint64_t)(uint32_t)p.dtype);
+    mix(p.flags);
+    mix((uint64_t)(uint32_t)p.variant);
+    mix((uint64_t)(uint32_t)p.reserved);
+    mix(p.workspace_bytes);
+    return h;
+}
+constexpr uint32_t KMX_PLAN_MAGIC = 0x50584d4bu;  // "KMXP"
+
+static int32_t plan_validate(const kmx_lloyd_plan* p) {
+    if (p == nullptr) return KMX_ERR_NULL_POINTER;
+    if (p->magic != KMX_PLAN_MAGIC || p->abi_version != KMX_ABI_VERSION || p->check != plan_check_value(*p))
+        return KMX_ERR_BAD_PLAN;
+    return KMX_OK;
+}
+#define KMX_REQUIRE_PLAN(p)                     \
+    do {                                        \
+        const int32_t rc_ = plan_validate(p);   \
+        if (rc_ != KMX_OK) return rc_;          \
+    } while (0)
+
+static int32_t layout_variant_code(const LloydLayout& L) { return L.screen ? 61 : L.variant * 10 + L.acc_mode; }
+
+int32_t kmx_lloyd_plan_init(kmx_lloyd_plan* plan, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                            uint32_t flags) {
+    KMX_REQUIRE_PTR(plan);
     if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
-    const LloydLayout L = lloyd_layout(n, d, k, dtype);
-    return L.screen ? 61 : L.variant * 10 + L.acc_mode;
+    if (!kmx_flags_valid(flags)) return KMX_ERR_BAD_ARGUMENT;
+    const LloydLayout L = lloyd_layout(n, d, k, dtype, flags);
+    plan->magic = KMX_PLAN_MAGIC;
+    plan->abi_version = KMX_ABI_VERSION;
+    plan->n = n;
+    plan->d = d;
+    plan->k = k;
+    plan->dtype = dtype;
+    plan->flags = flags;
+    plan->variant = layout_variant_code(L);
+    plan->reserved = 0;
+    plan->workspace_bytes = L.total;
+    plan->check = plan_check_value(*plan);
+    return KMX_OK;
 }
 
-int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
-                       const void* sample_weight, const void* centroids_t, int64_t n, int32_t d,
-                       int32_t k, int32_t dtype, int32_t max_iter, double tol, void* stream_) {
+size_t kmx_lloyd_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags) {
+    kmx_lloyd_plan plan;
+    return kmx_lloyd_plan_init(&plan, n, d, k, dtype, flags) == KMX_OK ? (size_t)plan.workspace_bytes : 0;
+}
+
+int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags) {
+    kmx_lloyd_plan plan;
+    const int32_t rc = kmx_lloyd_plan_init(&plan, n, d, k, dtype, flags);
+    return rc == KMX_OK ? plan.variant : rc;
+}
+
+int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t workspace_bytes,
+                       const void* X_t, const void* sample_weight, const void* centroids_t,
+                       int32_t max_iter, double tol, void* stream_) {
     KMX_ENTRY();
+    KMX_REQUIRE_PLAN(plan);
     KMX_REQUIRE_PTR(workspace);
     KMX_REQUIRE_PTR(X_t);
     KMX_REQUIRE_PTR(sample_weight);
     KMX_REQUIRE_PTR(centroids_t);
-    if (n <= 0 || d <= 0 || k <= 0 || max_iter < 0) return KMX_ERR_BAD_SHAPE;
-    KMX_REQUIRE_DTYPE(dtype);
-    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    if (max_iter < 0) return KMX_ERR_BAD_SHAPE;
+    const int64_t n = plan->n;
+    const int32_t d = plan->d, k = plan->k, dtype = plan->dtype;
+    const LloydLayout L = lloyd_layout(n, d, k, dtype, plan->flags);
     if (workspace_bytes < L.total) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
@@ -772,13 +834,13 @@ int32_t kmx_lloyd_init(void* workspace, size_t workspace_bytes, const void* X_t,
     return KMX_OK;
 }
 
-static int32_t lloyd_iter_dispatch(const void* X_t, const void* X_rowmajor,
+static int32_t lloyd_iter_dispatch(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
                                    const void* sample_weight, const void* centroids_t,
                                    void* new_centroids_t,
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
-                                   size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
-                                   int32_t dtype, void* stream_, hipEvent_t* events) {
+                                   size_t workspace_bytes, void* stream_, hipEvent_t* events) {
+    KMX_REQUIRE_PLAN(plan);
     KMX_REQUIRE_PTR(X_t);
     KMX_REQUIRE_PTR(sample_weight);
     KMX_REQUIRE_PTR(centroids_t);
@@ -788,9 +850,9 @@ static int32_t lloyd_iter_dispatch(const void* X_t, const void* X_rowmajor,
     KMX_REQUIRE_PTR(cluster_sizes);
     KMX_REQUIRE_PTR(empty_clusters);
     KMX_REQUIRE_PTR(workspace);
-    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
-    KMX_REQUIRE_DTYPE(dtype);
-    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    const int64_t n = plan->n;
+    const int32_t d = plan->d, k = plan->k, dtype = plan->dtype;
+    const LloydLayout L = lloyd_layout(n, d, k, dtype, plan->flags);
     if (workspace_bytes < L.total) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     if (dtype == KMX_F32) {
@@ -807,32 +869,33 @@ static int32_t lloyd_iter_dispatch(const void* X_t, const void* X_rowmajor,
                                    stream, events);
 }
 
-int32_t kmx_lloyd_iter(const void* X_t, const void* X_rowmajor, const void* sample_weight,
-                       const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
-                       void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
-                       size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+int32_t kmx_lloyd_iter(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
+                       const void* sample_weight, const void* centroids_t, void* new_centroids_t,
+                       const uint32_t* labels_prev, uint32_t* labels, void* cluster_sizes,
+                       uint32_t* empty_clusters, void* workspace, size_t workspace_bytes,
                        void* stream_) {
     KMX_ENTRY();
-    return lloyd_iter_dispatch(X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev, labels,
-                               cluster_sizes, empty_clusters, workspace, workspace_bytes, n, d, k,
-                               dtype, stream_, nullptr);
+    return lloyd_iter_dispatch(plan, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev,
+                               labels, cluster_sizes, empty_clusters, workspace, workspace_bytes, stream_,
+                               nullptr);
 }
 
-int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void* sample_weight,
-                             const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+int32_t kmx_lloyd_iter_timed(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
+                             const void* sample_weight, const void* centroids_t,
+                             void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
-                             size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
-                             void* stream_, float* kernel_ms_host) {
+                             size_t workspace_bytes, void* stream_, float* kernel_ms_host) {
     KMX_ENTRY();
     KMX_REQUIRE_PTR(kernel_ms_host);
+    KMX_REQUIRE_PLAN(plan);
     hipEvent_t ev[4];
     for (int i = 0; i < 4; ++i) {
         const hipError_t e = hipEventCreate(&ev[i]);
         if (e != hipSuccess) return (int32_t)e;
     }
-    int32_t rc = lloyd_iter_dispatch(X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev,
-                                     labels, cluster_sizes, empty_clusters, workspace,
-                                     workspace_bytes, n, d, k, dtype, stream_, ev);
+    int32_t rc = lloyd_iter_dispatch(plan, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t,
+                                     labels_prev, labels, cluster_sizes, empty_clusters, workspace,
+                                     workspace_bytes, stream_, ev);
     if (rc == KMX_OK) {
         hipError_t e = hipEventSynchronize(ev[3]);
         for (int i = 0; i < 3 && e == hipSuccess; ++i)
@@ -843,19 +906,18 @@ int32_t kmx_lloyd_iter_timed(const void* X_t, const void* X_rowmajor, const void
     return rc;
 }
 
-int32_t kmx_lloyd_finalize(const void* centroids_t, void* new_centroids_t,
-                           const void* cluster_sizes, void* workspace, size_t workspace_bytes,
-                           int32_t d, int32_t k, int32_t dtype, void* stream_) {
+int32_t kmx_lloyd_finalize(const kmx_lloyd_plan* plan, const void* centroids_t,
+                           void* new_centroids_t, const void* cluster_sizes, void* workspace,
+                           size_t workspace_bytes, void* stream_) {
     KMX_ENTRY();
+    KMX_REQUIRE_PLAN(plan);
     KMX_REQUIRE_PTR(centroids_t);
     KMX_REQUIRE_PTR(new_centroids_t);
     KMX_REQUIRE_PTR(cluster_sizes);
     KMX_REQUIRE_PTR(workspace);
-    if (d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
-    KMX_REQUIRE_DTYPE(dtype);
-    // offsets of the status, packed centroids, half norms and shift slots do not depend on n
-    const LloydLayout L = lloyd_layout(1, d, k, dtype);
-    if (workspace_bytes < L.off_bucket) return KMX_ERR_WORKSPACE;
+    const int32_t d = plan->d, k = plan->k, dtype = plan->dtype;
+    const LloydLayout L = lloyd_layout(plan->n, d, k, dtype, plan->flags);
+    if (workspace_bytes < L.total) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
@@ -887,19 +949,20 @@ int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_ho
     return e == hipSuccess ? KMX_OK : (int32_t)e;
 }
 
-int32_t kmx_lloyd_recheck_count(const void* workspace, int64_t n, int32_t d, int32_t k,
-                                int32_t dtype, uint32_t* count_host, void* stream_) {
+int32_t kmx_lloyd_recheck_count(const kmx_lloyd_plan* plan, const void* workspace,
+                                uint32_t* count_host, void* stream_) {
     KMX_ENTRY();
+    KMX_REQUIRE_PLAN(plan);
     KMX_REQUIRE_PTR(workspace);
     KMX_REQUIRE_PTR(count_host);
-    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
-    KMX_REQUIRE_DTYPE(dtype);
-    const LloydLayout L = lloyd_layout(n, d, k, dtype);
+    const int64_t n = plan->n;
+    const int32_t d = plan->d, k = plan->k;
+    const LloydLayout L = lloyd_layout(n, d, k, plan->dtype, plan->flags);
     *count_host = 0;
     const void* src = nullptr;
     if (L.screen)
         src = (const char*)workspace + L.off_bucket + sizeof(uint32_t);
-    else if (L.variant == KMX_VARIANT_MFMA_WIDE && kmx_wide_screen_enabled(n, d, k))
+    else if (L.variant == KMX_VARIANT_MFMA_WIDE && kmx_wide_screen_enabled(n, d, k, L.flags))
         src = kmx_wide_screen_counter((const char*)workspace + L.off_wscreen);
     if (src == nullptr) return KMX_OK;
     hipStream_t stream = (hipStream_t)stream_;
@@ -927,20 +990,20 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
 
 size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
     if (d <= 0 || k <= 0 || (dtype != KMX_F32 && dtype != KMX_F64)) return 0;
-    return lloyd_layout(1, d, k, dtype).off_bucket;
+    return lloyd_layout(1, d, k, dtype, 0).off_bucket;
 }
 
-size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype) {
+size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags) {
     const size_t base = kmx_assign_workspace_bytes(d, k, dtype);
-    if (base == 0 || n <= 0 || dtype != KMX_F32) return base;
-    if (lloyd_layout(n, d, k, dtype).variant != KMX_VARIANT_MFMA_WIDE) return base;
-    const size_t extra = kmx_assign_wide_screen_bytes(n, d, k);
+    if (base == 0 || n <= 0 || dtype != KMX_F32 || !kmx_flags_valid(flags)) return base;
+    if (lloyd_layout(n, d, k, dtype, flags).variant != KMX_VARIANT_MFMA_WIDE) return base;
+    const size_t extra = kmx_assign_wide_screen_bytes(n, d, k, flags);
     return extra ? kmx_align256(base) + extra : base;
 }
 
 int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* labels,
                           void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
-                          int32_t dtype, void* stream_) {
+                          int32_t dtype, uint32_t flags, void* stream_) {
     KMX_ENTRY();
     KMX_REQUIRE_PTR(X_t);
     KMX_REQUIRE_PTR(centroids_t);
@@ -948,14 +1011,15 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     KMX_REQUIRE_PTR(workspace);
     if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
-    LloydLayout L = lloyd_layout(n, d, k, dtype);
+    if (!kmx_flags_valid(flags)) return KMX_ERR_BAD_ARGUMENT;
+    LloydLayout L = lloyd_layout(n, d, k, dtype, flags);
     if (workspace_bytes < L.off_bucket) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32) {
         // labels screened on the fp16 matrix cores: one kernel, straight from the centroids
-        if (L.screen) return kmx_assign_labels_mfma_screen(X_t, centroids_t, labels, n, d, k, stream);
+        if (L.screen) return kmx_assign_labels_mfma_screen(X_t, centroids_t, labels, n, d, k, L.wgs_per_cu, stream);
         hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
                            (const float*)centroids_t, (float*)(ws + L.off_cpack),
                            (float*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
@@ -965,7 +1029,7 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
             return kmx_assign_labels_mfma_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
         if (L.variant == KMX_VARIANT_MFMA_WIDE) {
             // with the larger workspace of kmx_assign_workspace_bytes_for: labels screened in fp16
-            const size_t extra = kmx_assign_wide_screen_bytes(n, d, k);
+            const size_t extra = kmx_assign_wide_screen_bytes(n, d, k, flags);
             const size_t extra_off = kmx_align256(L.off_bucket);
             if (extra != 0 && workspace_bytes >= extra_off + extra)
                 return kmx_assign_labels_wide_screen_f32(L, X_t, centroids_t, labels, ws, ws + extra_off, n, d,

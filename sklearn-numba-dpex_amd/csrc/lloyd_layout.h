@@ -17,22 +17,47 @@ constexpr int KMX_MAX_PARTIALS = 1024;          // upper bound on fused-step wor
 constexpr size_t KMX_LDS_ACC_LIMIT = 40000;     // bytes of LDS accumulators per workgroup
 constexpr size_t KMX_GLOBAL_COPIES_BYTES = 64u << 20;
 
-// Environment overrides for experiments: KMX_LLOYD_VARIANT = stream | register | mfma,
-// KMX_LLOYD_WGS_PER_CU = 1..8.
-int kmx_forced_variant();
-int kmx_wgs_per_cu();
-int kmx_wgs_per_cu_env();
+// Kernel selection comes from the caller's `flags` (KMX_FLAG_* of the public header) and from
+// nothing else: the library reads no environment variable and keeps no selection state.
+// Forced path (KMX_VARIANT_* or -1), workgroups per compute unit (0 = the kernel's default)
+// and sample columns per lane of the matrix-core kernels (0 = default) out of the flags:
+static inline int kmx_flags_forced_variant(uint32_t flags) {
+    switch (flags & KMX_FLAG_PATH_MASK) {
+        case KMX_FLAG_PATH_STREAM: return 0;
+        case KMX_FLAG_PATH_REGISTER: return 1;
+        case KMX_FLAG_PATH_MFMA: return 3;
+        default: return -1;
+    }
+}
+static inline int kmx_flags_wgs_per_cu(uint32_t flags) {
+    const int x = (int)((flags >> 8) & 0xfu);
+    return (x >= 1 && x <= 8) ? x : 0;
+}
+static inline int kmx_flags_cols(uint32_t flags) {
+    const int x = (int)((flags >> 12) & 0x7u);
+    return (x == 2 || x == 4) ? x : 0;
+}
+static inline bool kmx_flags_valid(uint32_t flags) {
+    if (flags & ~(uint32_t)0x7f3f) return false;
+    if ((flags & KMX_FLAG_PATH_MASK) > KMX_FLAG_PATH_MFMA) return false;
+    if ((flags & KMX_FLAG_LABELS_MASK) == KMX_FLAG_LABELS_MASK) return false;
+    const uint32_t w = (flags >> 8) & 0xfu, c = (flags >> 12) & 0x7u;
+    return w <= 8 && (c == 0 || c == 2 || c == 4);
+}
 // Shapes the fp32 matrix-core fused step covers (operands and accumulators fit in LDS), and
 // those its wide-sample variant covers (samples in registers, centroids streamed).
 bool kmx_mfma_supported(int d, int k);
 bool kmx_mfma_wide_supported(int d, int k);
 bool kmx_mfma_f64_supported(int d, int k);
-// fp32 matrix-core step with bf16 screening of the labels (lloyd_mfma_screen.hip)
-bool kmx_mfma_screen_supported(int64_t n, int d, int k);
+// fp32 matrix-core step with fp16 screening of the labels (lloyd_mfma_screen.hip): whether the
+// shape fits the kernel at all, and whether the flags (or, left to the library, the measured
+// break-even) select it
+bool kmx_mfma_screen_fits(int64_t n, int d, int k);
+bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags);
 // screened label step of the wide path (lloyd_mfma_wide_screen.hip)
 size_t kmx_wide_screen_bytes(int64_t n, int d, int k);
 const int* kmx_wide_screen_list(const char* area, int d, int k);
-bool kmx_wide_screen_enabled(int64_t n, int d, int k);
+bool kmx_wide_screen_enabled(int64_t n, int d, int k, uint32_t flags);
 const uint32_t* kmx_wide_screen_counter(const char* area);
 
 struct LloydLayout {
@@ -41,14 +66,17 @@ struct LloydLayout {
     int acc_mode;        // KMX_ACC_*
     int n_partials;      // slots in `partial` (workgroups for LDS mode, copies for global mode)
     int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
-    bool screen;         // KMX_VARIANT_MFMA with bf16-screened labels (variant code 61)
+    bool screen;         // KMX_VARIANT_MFMA with fp16-screened labels (variant code 61)
+    uint32_t flags;      // the caller's KMX_FLAG_* selection
+    int wgs_per_cu;      // workgroups per compute unit asked for (0: the kernel's default)
+    int cols;            // sample columns per lane asked for (0: the kernel's default)
     size_t off_status, off_scales, off_gsum, off_cpack, off_half, off_shift, off_bucket, off_wscreen, off_partial;
     size_t partial_bytes;
     size_t total;
-    // Workgroups of the fused step: a few per compute unit (KMX_LLOYD_WGS_PER_CU, default 4),
-    // never more than the partial slots.
+    // Workgroups of the fused step: a few per compute unit (default 4), never more than the
+    // partial slots.
     int grid_cap(int cus) const {
-        const int g = kmx_wgs_per_cu() * cus;
+        const int g = (wgs_per_cu > 0 ? wgs_per_cu : 4) * cus;
         return g < n_partials ? g : n_partials;
     }
 };
@@ -59,15 +87,18 @@ static inline int lloyd_reg_samples_per_thread(int d, int dtype) {
 }
 
 
-static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
+static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint32_t flags) {
     LloydLayout L;
+    L.flags = flags;
+    L.wgs_per_cu = kmx_flags_wgs_per_cu(flags);
+    L.cols = kmx_flags_cols(flags);
     const size_t s = kmx_dtype_size(dtype);
     L.dpad = (d + 3) & ~3;
     L.k_for_gsum = k;
     const size_t items = (size_t)(d + 1) * k;
     const bool reg_ok = (dtype == KMX_F32) ? d <= 64 : d <= 32;
     L.variant = reg_ok ? KMX_VARIANT_REGISTER : KMX_VARIANT_STREAM;
-    const int forced = kmx_forced_variant();
+    const int forced = kmx_flags_forced_variant(flags);
     if (forced == KMX_VARIANT_STREAM) L.variant = KMX_VARIANT_STREAM;
     if (forced == KMX_VARIANT_REGISTER && reg_ok) L.variant = KMX_VARIANT_REGISTER;
     if (items * s <= KMX_LDS_ACC_LIMIT) {
@@ -83,7 +114,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     // (the screened step has the whole LDS of a compute unit and covers shapes the all-fp32
     // step, which stays within 64 KB, does not)
     if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS &&
-        (kmx_mfma_supported(d, k) || kmx_mfma_screen_supported(n, d, k)) &&
+        (kmx_mfma_supported(d, k) || kmx_mfma_screen_supported(n, d, k, flags)) &&
         (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA;
     else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA)) {
@@ -93,7 +124,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     else if (dtype == KMX_F64 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_f64_supported(d, k) &&
              (forced < 0 || forced == KMX_VARIANT_MFMA))
         L.variant = KMX_VARIANT_MFMA_F64;
-    L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k);
+    L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
     L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));
@@ -113,7 +144,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype) {
     // wide matrix-core path: header, scaled half norms and fp16 parts of the centroids for the
     // screened label step (lloyd_mfma_wide_screen.hip)
     L.off_wscreen = L.off_bucket + kmx_align256(bucket_bytes);
-    const size_t wscreen_bytes = L.variant == KMX_VARIANT_MFMA_WIDE ? kmx_wide_screen_bytes(n, d, k) : 0;
+    const size_t wscreen_bytes = L.variant == KMX_VARIANT_MFMA_WIDE ? kmx_wide_screen_bytes(n, d, k) : 0;  // (reserved whatever the flags say: the layout does not move with them)
     L.off_partial = L.off_wscreen + kmx_align256(wscreen_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
     const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE;
@@ -141,10 +172,10 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    kmx_lloyd_status* status, const unsigned int* absmax,
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, const float* norms, int64_t n, int d,
-                                   int k, hipStream_t stream);
+                                   int k, int wgs_per_cu, hipStream_t stream);
 // labels only, screened the same way (scale from the centroids, norms taken per tile)
 int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
-                                      int64_t n, int d, int k, hipStream_t stream);
+                                      int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);
 int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream);
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,
@@ -152,7 +183,7 @@ int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float
 int32_t kmx_wide_screen_scale_from_centroids(const void* centroids_t, unsigned int* absmax, int d, int k,
                                              hipStream_t stream);
 // labels only through the wide screen: bytes of extra workspace (0: not available), and the pass
-size_t kmx_assign_wide_screen_bytes(int64_t n, int d, int k);
+size_t kmx_assign_wide_screen_bytes(int64_t n, int d, int k, uint32_t flags);
 int32_t kmx_assign_labels_wide_screen_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
                                           uint32_t* labels, char* ws, char* extra, int64_t n, int d,
                                           int k, hipStream_t stream);
@@ -174,8 +205,9 @@ int32_t kmx_assign_labels_mfma_wide_f32(const LloydLayout& L, const void* X_t,
 
 // fp64 matrix-core fused step (lloyd_mfma_f64.hip): fills partial[0 .. grid) like the
 // vector-ALU kernels with LDS accumulators; `update` false = labels only
-int kmx_mfma_f64_grid(int64_t n);
+int kmx_mfma_f64_grid(int64_t n, int wgs_per_cu, int cols);
 int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* centroids_t,
                                 const void* half_norms, const uint32_t* labels_prev,
                                 uint32_t* labels, void* partial, kmx_lloyd_status* status,
-                                int64_t n, int d, int k, bool update, hipStream_t stream);
+                                int64_t n, int d, int k, bool update, int wgs_per_cu, int cols,
+                                hipStream_t stream);

@@ -28,31 +28,7 @@
 #include "lloyd_layout.h"
 #include "lloyd_tail.h"
 
-#include <cstdlib>
 #include <type_traits>
-#include <cstring>
-
-int kmx_forced_variant() {
-    const char* v = std::getenv("KMX_LLOYD_VARIANT");
-    if (v == nullptr) return -1;
-    if (std::strcmp(v, "stream") == 0) return KMX_VARIANT_STREAM;
-    if (std::strcmp(v, "register") == 0) return KMX_VARIANT_REGISTER;
-    if (std::strcmp(v, "mfma") == 0) return KMX_VARIANT_MFMA;
-    return -1;
-}
-
-// 0 when KMX_LLOYD_WGS_PER_CU is unset or out of range
-int kmx_wgs_per_cu_env() {
-    const char* v = std::getenv("KMX_LLOYD_WGS_PER_CU");
-    if (v == nullptr) return 0;
-    const int x = std::atoi(v);
-    return (x >= 1 && x <= 8) ? x : 0;
-}
-
-int kmx_wgs_per_cu() {
-    const int x = kmx_wgs_per_cu_env();
-    return x > 0 ? x : 4;
-}
 
 namespace {
 
@@ -220,6 +196,10 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS, MC)) void lloyd_mfma_kernel(
     // NC = 1: 32 samples (a quarter tile), the lane's sample is i0.  FULL: every sample of the
     // tile exists and (NC = 4) 128-bit accesses are legal.  wv / pl: weights and previous
     // labels of the lane's samples.
+    // +inf the optimiser cannot see through (it would turn the median in the arg-max into a
+    // maximum with two canonicalising instructions in front)
+    float pos_inf = kmx_inf<float>();
+    asm volatile("" : "+s"(pos_inf));
     auto process = [&](auto nc_tag, auto full_tag, const float(&x)[NKS][decltype(nc_tag)::value],
                        const float(&wv)[decltype(nc_tag)::value],
                        const uint32_t(&pl)[decltype(nc_tag)::value], const int64_t i0) {
@@ -268,15 +248,19 @@ __global__ __launch_bounds__(64 * mfma_waves(NKS, MC)) void lloyd_mfma_kernel(
 #pragma unroll
                 for (int t = 0; t < NC; ++t) {
                     // three-operand max: two scores per instruction (fmaxf would also
-                    // canonicalise the matrix-core results first)
-                    float m = a[t][g * ARGMAX_GROUP];
+                    // canonicalise the matrix-core results first).  The FIRST read of a
+                    // matrix-core result must be an instruction the compiler knows (the median
+                    // of a, b and +inf is max(a, b)): it inserts the wait states an MFMA result
+                    // needs before a vector-ALU read, which it does not do for operands of
+                    // inline assembly.  Once that instruction has issued the whole MFMA is
+                    // complete, so the rest of the chain may be assembly.
+                    static_assert(ARGMAX_GROUP % 2 == 0, "pairs of registers");
+                    float m = __builtin_amdgcn_fmed3f(a[t][g * ARGMAX_GROUP], a[t][g * ARGMAX_GROUP + 1], pos_inf);
 #pragma unroll
-                    for (int r = 1; r + 1 < ARGMAX_GROUP; r += 2)
+                    for (int r = 2; r + 1 < ARGMAX_GROUP; r += 2)
                         asm("v_max3_f32 %0, %1, %2, %3"
                             : "=v"(m)
                             : "v"(m), "v"(a[t][g * ARGMAX_GROUP + r]), "v"(a[t][g * ARGMAX_GROUP + r + 1]));
-                    if (ARGMAX_GROUP % 2 == 0)
-                        asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(m), "v"(a[t][g * ARGMAX_GROUP + ARGMAX_GROUP - 1]));
                     // strict: the earlier group keeps a tie.  The winning lanes copy the
                     // group with 64-bit moves under the execution mask: half the instructions
                     // of per-register selects.
@@ -519,16 +503,15 @@ int32_t launch_mfma(const LloydLayout& L, const void* X_t, const void* w, const 
     const int nks_t = (d + 1) / 2 <= 8 ? (d + 1) / 2 : (d <= 32 ? 16 : 32);
     // Sample columns per lane.  Two (64 samples per wave tile, two MFMA chains) leave
     // registers for three waves per SIMD and run about 4 % faster than four columns with two
-    // waves; KMX_MFMA_COLS = 4 restores the latter for experiments.  Shapes with more than 8 K
+    // waves; KMX_FLAG_COLS(4) restores the latter for experiments.  Shapes with more than 8 K
     // steps keep four columns and four waves per workgroup.
-    const char* cols_env = std::getenv("KMX_MFMA_COLS");
-    const int mc = (nks_t <= 8 && !(cols_env != nullptr && cols_env[0] == '4')) ? 2 : 4;
+    const int mc = (nks_t <= 8 && L.cols != 4) ? 2 : 4;
     const int64_t n_wtiles = kmx_cdiv(n, 32 * mc);
     const int waves = mfma_waves(nks_t, mc);
     int64_t grid = kmx_cdiv(n_wtiles, waves);
     // resident workgroups only: one workgroup per compute unit, or two of four waves
     const int per_cu = waves >= 8 ? 1 : 2;
-    const int cap = (kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : per_cu) * kmx_num_cus();
+    const int cap = (L.wgs_per_cu > 0 ? L.wgs_per_cu : per_cu) * kmx_num_cus();
     if (grid > cap) grid = cap;
     if (grid < 1) grid = 1;
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
@@ -624,7 +607,7 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         const int32_t rc = kmx_lloyd_step_mfma_screen(
             X_t, w, centroids_t, labels_prev, labels, tail.status,
             reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain,
-            reinterpret_cast<const float*>(ws + L.off_bucket + 256), n, d, k, stream);
+            reinterpret_cast<const float*>(ws + L.off_bucket + 256), n, d, k, L.wgs_per_cu, stream);
         if (rc != KMX_OK) return rc;
         if (events) {
             (void)hipEventRecord(events[1], stream);

@@ -23,7 +23,6 @@
 //     written to the workgroup's slot of `partial` at the end.
 #include "lloyd_layout.h"
 
-#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -283,17 +282,17 @@ bool kmx_mfma_f64_supported(int d, int k) {
 }
 
 // Sample columns per lane: two (three waves per SIMD, next tile in flight) once there are
-// several tiles per wave, four for small inputs.  KMX_F64_COLS = 2 | 4 overrides this for
+// several tiles per wave, four for small inputs.  KMX_FLAG_COLS(2 | 4) overrides this for
 // experiments.
-static int f64_cols(int64_t n) {
-    const char* v = std::getenv("KMX_F64_COLS");
-    if (v != nullptr && (v[0] == '2' || v[0] == '4') && v[1] == 0) return v[0] - '0';
+static int f64_cols(int64_t n, int cols) {
+    if (cols == 2 || cols == 4) return cols;
     return n >= (int64_t)1 << 19 ? 2 : 4;
 }
 
-int kmx_mfma_f64_grid(int64_t n) {
-    const int64_t tiles = kmx_cdiv(kmx_cdiv(n, 16 * f64_cols(n)), f64_waves(f64_cols(n)));
-    const int64_t cap = (int64_t)(kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : 1) * kmx_num_cus();
+int kmx_mfma_f64_grid(int64_t n, int wgs_per_cu, int cols_asked) {
+    const int nc = f64_cols(n, cols_asked);
+    const int64_t tiles = kmx_cdiv(kmx_cdiv(n, 16 * nc), f64_waves(nc));
+    const int64_t cap = (int64_t)(wgs_per_cu > 0 ? wgs_per_cu : 1) * kmx_num_cus();
     int64_t grid = tiles < cap ? tiles : cap;
     if (grid > KMX_MAX_PARTIALS) grid = KMX_MAX_PARTIALS;
     return grid < 1 ? 1 : (int)grid;
@@ -302,16 +301,17 @@ int kmx_mfma_f64_grid(int64_t n) {
 int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* centroids_t,
                                 const void* half_norms, const uint32_t* labels_prev,
                                 uint32_t* labels, void* partial, kmx_lloyd_status* status,
-                                int64_t n, int d, int k, bool update, hipStream_t stream) {
+                                int64_t n, int d, int k, bool update, int wgs_per_cu, int cols_asked,
+                                hipStream_t stream) {
     if (!kmx_mfma_f64_supported(d, k)) return KMX_ERR_UNSUPPORTED;
     const size_t lds = mfma_f64_lds_bytes(d, k, update);
-    const int grid = kmx_mfma_f64_grid(n);
+    const int grid = kmx_mfma_f64_grid(n, wgs_per_cu, cols_asked);
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     // rows start 16-byte aligned when n is even; 4 samples per lane need n % 4 == 0 only for
     // the 128-bit label accesses
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
                        (!update || (aligned16(w) && aligned16(labels_prev)));
-    const int cols = f64_cols(n);
+    const int cols = f64_cols(n, cols_asked);
 #define KMX_F64_LAUNCH(NKS, NC, UPD)                                                              \
     hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, NC, UPD>), dim3((unsigned)grid),                 \
                        dim3(64 * f64_waves(NC)), lds, stream, (const double*)X_t, (const double*)w, \

@@ -35,8 +35,6 @@
 #include "lloyd_layout.h"
 #include "lloyd_tail.h"
 
-#include <cstdlib>
-#include <cstring>
 #include <type_traits>
 
 namespace {
@@ -976,18 +974,22 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 }  // namespace
 
 // Shapes the screened step covers: d <= 32, everything within the workgroup's LDS, byte offsets
-// inside two rows of X_t within 32 bits.  It is chosen where it is the faster one: the all-fp32
-// step pays d / 2 fp32 MFMAs per block of 32 centroids, the screen three fp16 ones plus the
-// split and the certificate whatever d is; measured on 2e6 samples the screen wins from d = 10
-// on, from d = 8 for k >= 64 and from d = 6 for k >= 128 (at d = 2 it is 30 % slower, at d = 16,
-// k = 128 36 % faster).  KMX_LLOYD_ASSIGN = f32 switches it off (all-fp32 scores on the matrix
-// cores, lloyd_mfma.hip), KMX_LLOYD_ASSIGN = screen selects it wherever it is possible.
-bool kmx_mfma_screen_supported(int64_t n, int d, int k) {
+// inside two rows of X_t within 32 bits.
+bool kmx_mfma_screen_fits(int64_t n, int d, int k) {
     if (d < 1 || d > 32 || k < 16 || n >= ((int64_t)1 << 29)) return false;
-    const char* v = std::getenv("KMX_LLOYD_ASSIGN");
-    if (v != nullptr && std::strcmp(v, "f32") == 0) return false;
-    if (screen_lds(d, k, (d + 15) / 16, true).off_queue > scr_lds_max((d + 15) / 16)) return false;
-    if (v != nullptr && std::strcmp(v, "screen") == 0) return true;
+    return screen_lds(d, k, (d + 15) / 16, true).off_queue <= scr_lds_max((d + 15) / 16);
+}
+
+// Left to the library it is chosen where it is the faster one: the all-fp32 step pays d / 2 fp32
+// MFMAs per block of 32 centroids, the screen three fp16 ones plus the split and the certificate
+// whatever d is; measured on 2e6 samples the screen wins from d = 10 on, from d = 8 for k >= 64
+// and from d = 6 for k >= 128 (at d = 2 it is 30 % slower, at d = 16, k = 128 36 % faster).
+// KMX_FLAG_LABELS_F32 switches it off (all-fp32 scores on the matrix cores, lloyd_mfma.hip),
+// KMX_FLAG_LABELS_SCREEN selects it wherever it is possible.
+bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags) {
+    if ((flags & KMX_FLAG_LABELS_MASK) == KMX_FLAG_LABELS_F32) return false;
+    if (!kmx_mfma_screen_fits(n, d, k)) return false;
+    if ((flags & KMX_FLAG_LABELS_MASK) == KMX_FLAG_LABELS_SCREEN) return true;
     return d >= 10 || (d >= 8 && k >= 64) || (d >= 6 && k >= 128);
 }
 
@@ -996,14 +998,14 @@ template <bool UPDATE>
 int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, const uint32_t* labels_prev,
                       uint32_t* labels, kmx_lloyd_status* status, const unsigned int* absmax,
                       const int* q_exp, unsigned long long* gsum, uint32_t* uncertain_count,
-                      const float* norms, int64_t n, int d, int k, hipStream_t stream) {
-    if (!kmx_mfma_screen_supported(n, d, k)) return KMX_ERR_UNSUPPORTED;
+                      const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
+    if (!kmx_mfma_screen_fits(n, d, k)) return KMX_ERR_UNSUPPORTED;
     const int nk = (d + 15) / 16;
     const int waves = scr_waves(nk);
     const int64_t n_wtiles = kmx_cdiv(n, 64);
     int64_t grid = kmx_cdiv(n_wtiles, waves);
     const int per_cu = waves >= 8 ? 1 : 2;
-    const int cap = (kmx_wgs_per_cu_env() > 0 ? kmx_wgs_per_cu_env() : per_cu) * kmx_num_cus();
+    const int cap = (wgs_per_cu > 0 ? wgs_per_cu : per_cu) * kmx_num_cus();
     if (grid > cap) grid = cap;
     if (grid < 1) grid = 1;
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
@@ -1040,17 +1042,17 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    kmx_lloyd_status* status, const unsigned int* absmax,
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, const float* norms, int64_t n, int d,
-                                   int k, hipStream_t stream) {
+                                   int k, int wgs_per_cu, hipStream_t stream) {
     return launch_screen<true>(X_t, w, centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,
-                               uncertain_count, norms, n, d, k, stream);
+                               uncertain_count, norms, n, d, k, wgs_per_cu, stream);
 }
 
 // Labels only, screened the same way: nothing but X and the centroids is needed (the scale comes
 // from the centroids, each tile takes the norms of its samples itself).
 int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
-                                      int64_t n, int d, int k, hipStream_t stream) {
+                                      int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
     return launch_screen<false>(X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr, nullptr,
-                                nullptr, nullptr, nullptr, n, d, k, stream);
+                                nullptr, nullptr, nullptr, n, d, k, wgs_per_cu, stream);
 }
 
 // Diagnostics of the screen: approximate scores and error bounds as the fused step forms them.

@@ -487,7 +487,7 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
     int* order = offsets + (k + 1);
     int* ranks = order + n;
     int32_t rc;
-    if (kmx_wide_screen_enabled(n, d, k)) {
+    if (kmx_wide_screen_enabled(n, d, k, L.flags)) {
         // labels screened on the fp16 matrix cores; what the screen cannot certify is listed
         // and goes through the all-fp32 kernel
         char* area = ws + L.off_wscreen;
@@ -520,8 +520,8 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
     return KMX_OK;
 }
 
-size_t kmx_assign_wide_screen_bytes(int64_t n, int d, int k) {
-    if (!kmx_wide_screen_enabled(n, d, k)) return 0;
+size_t kmx_assign_wide_screen_bytes(int64_t n, int d, int k, uint32_t flags) {
+    if (!kmx_wide_screen_enabled(n, d, k, flags)) return 0;
     return kmx_align256((size_t)d * sizeof(unsigned int)) + kmx_wide_screen_bytes(n, d, k);
 }
 

@@ -24,8 +24,6 @@
 // and ranks; the sums are taken by the bucketed accumulation from the row-major copy of X).
 #include "lloyd_layout.h"
 
-#include <cstdlib>
-#include <cstring>
 #include <type_traits>
 
 namespace {
@@ -511,12 +509,11 @@ size_t kmx_wide_screen_bytes(int64_t n, int d, int k) {
     return 256 + n_cg * CG * sizeof(float) + n_cg * nkc * CHUNK_VEC * sizeof(uint4) + (size_t)n * sizeof(int);
 }
 
-// KMX_LLOYD_ASSIGN = f32 switches the screen off (all-fp32 scores, lloyd_mfma_wide.hip).
-bool kmx_wide_screen_enabled(int64_t n, int d, int k) {
+// KMX_FLAG_LABELS_F32 switches the screen off (all-fp32 scores, lloyd_mfma_wide.hip).
+bool kmx_wide_screen_enabled(int64_t n, int d, int k, uint32_t flags) {
     // (the label kernel addresses a lane's samples with 32-bit byte offsets into two rows)
     if (!kmx_mfma_wide_supported(d, k) || n >= ((int64_t)1 << 29)) return false;
-    const char* v = std::getenv("KMX_LLOYD_ASSIGN");
-    return !(v != nullptr && std::strcmp(v, "f32") == 0);
+    return (flags & KMX_FLAG_LABELS_MASK) != KMX_FLAG_LABELS_F32;
 }
 
 const uint32_t* kmx_wide_screen_counter(const char* area) {

@@ -31,6 +31,7 @@ def lloyd(
     verbose=False,
     tol=1e-4,
     relocation="sklearn",
+    flags=None,
 ):
     """Single Lloyd run (reference: kmeans/drivers.py:43-393).
 
@@ -44,6 +45,9 @@ def lloyd(
     relocation: which centroids the distances that rank samples for empty-cluster relocation
     are measured to: "sklearn" = the centroids the labels were computed from (what
     scikit-learn does), "literal" = the un-normalised sums (kmeans/drivers.py:252-259).
+
+    flags: kernel selection (KMX_FLAG_* of the C header); None = the defaults `_capi` took from
+    the environment when it was imported.
     """
     require_cuda()
     X_t = contiguous(X_t)
@@ -53,7 +57,8 @@ def lloyd(
     dev, dt, dc = X_t.device, X_t.dtype, dcode(X_t)
     stream = _capi.current_stream()
 
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    plan = _capi.lloyd_plan(n, d, k, dc, flags)
+    ws_bytes = plan.workspace_bytes
     ws = workspace(ws_bytes, dev)
     cent = [contiguous(centroids_t).clone(), torch.empty((d, k), dtype=dt, device=dev)]
     labels = [torch.empty(n, dtype=torch.int32, device=dev) for _ in range(2)]
@@ -63,9 +68,9 @@ def lloyd(
 
     # the wide fp32 path sums each cluster's rows from a row-major copy of X (one transpose per
     # run, n * d extra elements of HBM) instead of one global atomic per (sample, feature)
-    X_rm = X_t.T.contiguous() if lib.kmx_lloyd_kernel_variant(n, d, k, dc) == 42 else None
+    X_rm = X_t.T.contiguous() if plan.variant == 42 else None
 
-    check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), n, d, k, dc, int(max_iter),
+    check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), int(max_iter),
                              float(tol), stream),
           "kmx_lloyd_init")
 
@@ -75,9 +80,9 @@ def lloyd(
     while True:
         for _ in range(lookahead):
             a, b = enqueued % 2, (enqueued + 1) % 2
-            check(lib.kmx_lloyd_iter(ptr(X_t), ptr(X_rm), ptr(sample_weight), ptr(cent[a]), ptr(cent[b]),
+            check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(sample_weight), ptr(cent[a]), ptr(cent[b]),
                                      ptr(labels[a]), ptr(labels[b]), ptr(sizes), ptr(empty_list),
-                                     ptr(ws), ws_bytes, n, d, k, dc, stream), "kmx_lloyd_iter")
+                                     ptr(ws), ws_bytes, stream), "kmx_lloyd_iter")
             enqueued += 1
         check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "kmx_lloyd_status_read")
 
@@ -88,8 +93,8 @@ def lloyd(
                 status.n_empty, X_t, sample_weight, cent[b], sizes, labels[b], empty_list,
                 cent[a] if relocation == "sklearn" else cent[b],
             )
-            check(lib.kmx_lloyd_finalize(ptr(cent[a]), ptr(cent[b]), ptr(sizes), ptr(ws), ws_bytes, d, k,
-                                         dc, stream), "kmx_lloyd_finalize")
+            check(lib.kmx_lloyd_finalize(plan, ptr(cent[a]), ptr(cent[b]), ptr(sizes), ptr(ws), ws_bytes,
+                                         stream), "kmx_lloyd_finalize")
             enqueued = j + 1
             lookahead = 1
             check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "kmx_lloyd_status_read")
@@ -117,19 +122,20 @@ def lloyd(
     # labels for the final centroids and the exact inertia (kmeans/drivers.py:356-391)
     best = cent[n_iteration % 2]
     assignments_idx = labels[0]
-    _assign(X_t, best, assignments_idx)
+    _assign(X_t, best, assignments_idx, flags)
     inertia = _inertia(X_t, sample_weight, best, assignments_idx)
     return assignments_idx, inertia, best, n_iteration
 
 
-def _assign(X_t, centroids_t, labels_out):
+def _assign(X_t, centroids_t, labels_out, flags=None):
     d, n = X_t.shape
     k = centroids_t.shape[1]
     dc = dcode(X_t)
-    ws_bytes = lib.kmx_assign_workspace_bytes_for(n, d, k, dc)
+    flags = _capi.DEFAULT_FLAGS if flags is None else int(flags)
+    ws_bytes = lib.kmx_assign_workspace_bytes_for(n, d, k, dc, flags)
     ws = workspace(ws_bytes, X_t.device)
     check(lib.kmx_assign_labels(ptr(X_t), ptr(centroids_t), ptr(labels_out), ptr(ws), ws_bytes, n, d, k,
-                                dc, _capi.current_stream()), "kmx_assign_labels")
+                                dc, flags, _capi.current_stream()), "kmx_assign_labels")
 
 
 def _per_sample_inertia(X_t, sample_weight, centroids_t, labels, out=None):

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_function():
     for name in declared:
         assert hasattr(raw, name), f"{name} is declared in the header but not exported"
     assert sorted(_capi.SIGNATURES) == declared, "ctypes signatures and header disagree"
-    assert _capi.lib.kmx_abi_version() == 1
+    assert _capi.lib.kmx_abi_version() == 2
 
 
 def test_header_cites_the_reference_for_every_entry_point():
@@ -56,19 +56,19 @@ def test_error_strings_and_codes():
 def test_workspace_queries():
     from sklearn_numba_dpex_amd._capi import lib
 
-    small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0)
+    small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0, 0)
     assert 0 < small < 64 << 20
     # the screened fp32 step keeps ||x_i|| per sample: 4 bytes per sample
-    assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0) - small - 4 * 4_900_000) < 256
-    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1)
-    assert lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0) > (32 << 20)  # global copies
-    assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0) == 0
-    assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7) == 0
+    assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0, 0) - small - 4 * 4_900_000) < 256
+    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0)
+    assert lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) > (32 << 20)  # global copies
+    assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0, 0) == 0
+    assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7, 0) == 0
     assert lib.kmx_assign_workspace_bytes(14, 127, 0) > 127 * 16 * 4
     # the roomy variant only grows for wide fp32 shapes (a list of sample indices)
-    assert lib.kmx_assign_workspace_bytes_for(1000, 14, 127, 0) == lib.kmx_assign_workspace_bytes(14, 127, 0)
-    assert lib.kmx_assign_workspace_bytes_for(1000, 256, 1024, 1) == lib.kmx_assign_workspace_bytes(256, 1024, 1)
-    assert (lib.kmx_assign_workspace_bytes_for(1000, 256, 1024, 0)
+    assert lib.kmx_assign_workspace_bytes_for(1000, 14, 127, 0, 0) == lib.kmx_assign_workspace_bytes(14, 127, 0)
+    assert lib.kmx_assign_workspace_bytes_for(1000, 256, 1024, 1, 0) == lib.kmx_assign_workspace_bytes(256, 1024, 1)
+    assert (lib.kmx_assign_workspace_bytes_for(1000, 256, 1024, 0, 0)
             >= lib.kmx_assign_workspace_bytes(256, 1024, 0) + 1000 * 4)
     assert lib.kmx_kpp_workspace_bytes(1_000_000, 64, 256, 7, 0) >= 7 * 4_000_000
     assert lib.kmx_kpp_workspace_bytes(1000, 4, 8, 17, 0) == 0  # more trials than supported
@@ -80,18 +80,80 @@ def test_workspace_queries():
 def test_kernel_variant_selection():
     from sklearn_numba_dpex_amd._capi import lib
 
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0) == 61   # bf16-screened MFMA + LDS accumulators
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0) == 31   # fp32 MFMA + LDS accumulators
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 4, 127, 0) == 31    # too few features for the screen to pay
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 64, 0) == 61
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 32, 0) == 31
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1) == 51    # fp64: matrix cores + LDS
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1) in (12, 2)  # accumulators too big for LDS
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0) == 42  # wide MFMA + global sums
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0) == 2   # streaming + global copies
-    assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0) == 11           # too few clusters for MFMA
-    assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0) == -2
-    assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4) == -3
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0) == 61   # fp16-screened MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0, 0) == 31   # fp32 MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 4, 127, 0, 0) == 31    # too few features for the screen to pay
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 64, 0, 0) == 61
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 32, 0, 0) == 31
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0) == 51    # fp64: matrix cores + LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0) in (12, 2)  # accumulators too big for LDS
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0, 0) == 42  # wide MFMA + global sums
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 2   # streaming + global copies
+    assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0, 0) == 11           # too few clusters for MFMA
+    assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0, 0) == -2
+    assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4, 0) == -3
+    # the caller's flags, and nothing else, move the choice
+    F32, SCREEN, REGISTER, STREAM = 0x10, 0x20, 0x2, 0x1
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, F32) == 31
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 4, 127, 0, SCREEN) == 61
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, REGISTER) == 11
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, STREAM) == 1
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0, F32) == 42   # same path, labels all fp32
+    assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 0, 0x30) == -5    # both label switches
+    assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 0, 0x8000) == -5  # unknown bit
+    assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 0, 0x3000) == -5  # three sample columns
+
+
+def test_environment_does_not_reach_the_library(monkeypatch):
+    """The library reads no environment variable: only the flags select a kernel.  (The Python
+    binding turns the variables into default flags once, when it is imported.)"""
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib
+
+    before = lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0)
+    monkeypatch.setenv("KMX_LLOYD_ASSIGN", "f32")
+    monkeypatch.setenv("KMX_LLOYD_VARIANT", "stream")
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0) == before == 61
+    assert _capi.lloyd_plan(5_000_000, 14, 127, 0, 0).variant == 61
+    assert _capi._flags_from_environment() == (_capi.FLAG_LABELS_F32 | _capi.FLAG_PATH_STREAM)
+    # no getenv in any source of the library
+    import glob
+    import os
+    for path in glob.glob(os.path.join(os.path.dirname(_capi.__file__), "csrc", "*")):
+        assert "getenv" not in open(path).read(), path
+
+
+def test_lloyd_plan_is_validated():
+    """A plan carries shape, flags, variant and workspace size; the calls that take one reject a
+    plan they did not make, an edited one, and a workspace smaller than the plan's."""
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib
+
+    buf = ctypes.create_string_buffer(1 << 16)
+    p = ctypes.addressof(buf)
+    plan = _capi.lloyd_plan(1000, 14, 127, 0, 0)
+    assert (plan.n, plan.d, plan.k, plan.dtype, plan.flags) == (1000, 14, 127, 0, 0)
+    assert plan.variant == 61 and plan.workspace_bytes == lib.kmx_lloyd_workspace_bytes(1000, 14, 127, 0, 0)
+    f32 = _capi.lloyd_plan(1000, 14, 127, 0, _capi.FLAG_LABELS_F32)
+    assert f32.variant == 31 and f32.workspace_bytes < plan.workspace_bytes   # no per-sample norms
+    # a workspace sized for the other variant is too small for this plan
+    assert lib.kmx_lloyd_init(plan, p, f32.workspace_bytes, p, p, p, 10, 0.0, None) == -4
+    assert lib.kmx_lloyd_iter(plan, p, None, p, p, p, p, p, p, p, p, f32.workspace_bytes, None) == -4
+    # flags changed behind the library's back: variant and layout would no longer match
+    edited = _capi.LloydPlan.from_buffer_copy(plan)
+    edited.flags = _capi.FLAG_LABELS_F32
+    assert lib.kmx_lloyd_iter(edited, p, None, p, p, p, p, p, p, p, p, 1 << 16, None) == _capi.KMX_ERR_BAD_PLAN
+    edited = _capi.LloydPlan.from_buffer_copy(plan)
+    edited.variant = 31
+    assert lib.kmx_lloyd_init(edited, p, 1 << 16, p, p, p, 10, 0.0, None) == _capi.KMX_ERR_BAD_PLAN
+    edited = _capi.LloydPlan.from_buffer_copy(plan)
+    edited.n = 2000
+    assert lib.kmx_lloyd_finalize(edited, p, p, p, p, 1 << 16, None) == _capi.KMX_ERR_BAD_PLAN
+    assert lib.kmx_lloyd_iter(_capi.LloydPlan(), p, None, p, p, p, p, p, p, p, p, 1 << 16, None) == _capi.KMX_ERR_BAD_PLAN
+    assert lib.kmx_lloyd_iter(None, p, None, p, p, p, p, p, p, p, p, 1 << 16, None) == -1
+    rechecked = ctypes.c_uint32(7)
+    assert lib.kmx_lloyd_recheck_count(edited, p, ctypes.byref(rechecked), None) == _capi.KMX_ERR_BAD_PLAN
+    assert "plan" in _capi.error_string(_capi.KMX_ERR_BAD_PLAN)
 
 
 def test_bad_arguments_are_rejected_without_a_device():
@@ -100,13 +162,20 @@ def test_bad_arguments_are_rejected_without_a_device():
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     NULL = None
-    assert lib.kmx_lloyd_init(NULL, 0, p, p, p, 10, 2, 2, 0, 10, 0.0, NULL) == -1
-    assert lib.kmx_lloyd_init(p, 4096, p, p, p, 0, 2, 2, 0, 10, 0.0, NULL) == -2
-    assert lib.kmx_lloyd_init(p, 4096, p, p, p, 10, 2, 2, 9, 10, 0.0, NULL) == -3
-    assert lib.kmx_lloyd_init(p, 16, p, p, p, 10, 2, 2, 0, 10, 0.0, NULL) == -4
-    assert lib.kmx_lloyd_iter(p, NULL, p, p, p, p, p, p, p, p, 16, 10, 2, 2, 0, NULL) == -4
-    assert lib.kmx_lloyd_iter(p, NULL, NULL, p, p, p, p, p, p, p, 4096, 10, 2, 2, 0, NULL) == -1
-    assert lib.kmx_assign_labels(p, p, NULL, p, 4096, 10, 2, 2, 0, NULL) == -1
+    from sklearn_numba_dpex_amd import _capi
+
+    plan = _capi.LloydPlan()
+    assert lib.kmx_lloyd_plan_init(plan, 0, 2, 2, 0, 0) == -2
+    assert lib.kmx_lloyd_plan_init(plan, 10, 2, 2, 9, 0) == -3
+    assert lib.kmx_lloyd_plan_init(None, 10, 2, 2, 0, 0) == -1
+    assert lib.kmx_lloyd_plan_init(plan, 10, 2, 2, 0, 0) == 0
+    assert lib.kmx_lloyd_init(plan, NULL, 0, p, p, p, 10, 0.0, NULL) == -1
+    assert lib.kmx_lloyd_init(plan, p, 4096, p, p, p, -1, 0.0, NULL) == -2
+    assert lib.kmx_lloyd_init(plan, p, 16, p, p, p, 10, 0.0, NULL) == -4
+    assert lib.kmx_lloyd_iter(plan, p, NULL, p, p, p, p, p, p, p, p, 16, NULL) == -4
+    assert lib.kmx_lloyd_iter(plan, p, NULL, NULL, p, p, p, p, p, p, p, 4096, NULL) == -1
+    assert lib.kmx_assign_labels(p, p, NULL, p, 4096, 10, 2, 2, 0, 0, NULL) == -1
+    assert lib.kmx_assign_labels(p, p, p, p, 4096, 10, 2, 2, 0, 0x30, NULL) == -5
     assert lib.kmx_per_sample_inertia(p, NULL, p, p, p, 0, 2, 2, 0, NULL) == -2
     assert lib.kmx_euclidean_distances(p, p, p, 10, 2, 2, 5, NULL) == -3
     assert lib.kmx_topk_idx(p, p, 5, 10, p, 4096, 0, NULL) == -5      # k > n

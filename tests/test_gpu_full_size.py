@@ -26,7 +26,8 @@ def _run_iterations(cuda, cfg, n_iter):
     dc = _capi.dtype_code(X.dtype)
     X_rm = torch.as_tensor(X, device=cuda)
     X_t = X_rm.T.contiguous()
-    if lib.kmx_lloyd_kernel_variant(n, d, k, dc) != 42:
+    plan = _capi.lloyd_plan(n, d, k, dc, 0)
+    if plan.variant != 42:
         X_rm = None
     w_d = torch.as_tensor(w, device=cuda)
     cent = [torch.as_tensor(np.ascontiguousarray(init.T), device=cuda), None]
@@ -34,17 +35,17 @@ def _run_iterations(cuda, cfg, n_iter):
     labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
     sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
     empty = torch.empty(k, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
     status = _capi.LloydStatus()
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, 1000, 0.0,
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 1000, 0.0,
                                    stream), "init")
     out = []
     for it in range(n_iter):
         a, b = it % 2, (it + 1) % 2
-        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(X_rm), ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
-                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, dc,
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(cent[a]), ptr(cent[b]),
+                                       ptr(labels[a]), ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes,
                                        stream), "iter")
         _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
         out.append(dict(inp=cent[a].clone(), new=cent[b].clone(), labels=labels[b].clone(), sizes=sizes.clone(),

@@ -39,8 +39,13 @@ def _small_configs():
         "M32c": lambda: _blob_config(33, 14, 16, np.float32, 16),
         # wide fp32 path with very unequal clusters (bucket sizes from 0 to a third of n)
         "C3k": lambda: _blob_config(40_000, 128, 64, np.float32, 17, skew=True),
-        # few features but too many clusters for LDS accumulators: the wide path with one chunk
-        "M32d": lambda: _blob_config(20_000, 14, 600, np.float32, 18),
+        # few features, many clusters: accumulators and centroid copies need more than 64 KB of
+        # LDS, which only the screened step (one workgroup per compute unit) may take
+        "M32d": lambda: dict(_blob_config(20_000, 14, 600, np.float32, 18), variant=61),
+        # the same with the screen switched off, and a shape whose accumulators exceed what any
+        # kernel keeps in LDS: the wide path with one chunk of features (d <= 32)
+        "M32e": lambda: dict(_blob_config(20_000, 14, 600, np.float32, 18), flags=0x10, variant=42),
+        "M32f": lambda: dict(_blob_config(20_000, 14, 700, np.float32, 20), variant=42),
         # fp64 whose accumulators do not fit LDS: vector-ALU kernel with global copies
         "F64d": lambda: _blob_config(20_000, 32, 300, np.float64, 19),
     }
@@ -67,7 +72,7 @@ def _odd_config():
 
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
-                                  "M32a", "M32b", "M32c", "C3k", "M32d", "F64d"])
+                                  "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -86,15 +91,18 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     labels = torch.empty(n, dtype=torch.int32, device=cuda)
     sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
     empty = torch.empty(k, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    plan = _capi.lloyd_plan(n, d, k, dc, cfg.get("flags", 0))
+    if "variant" in cfg:
+        assert plan.variant == cfg["variant"]
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), n, d, k, dc, 100, 0.0, stream), "init")
-    if rowmajor and lib.kmx_lloyd_kernel_variant(n, d, k, dc) != 42:
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), 100, 0.0, stream), "init")
+    if rowmajor and plan.variant != 42:
         pytest.skip("the row-major copy is only used by the wide fp32 path")
     X_rm = _dev(X, cuda) if rowmajor else None
-    _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
-                                   ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, dc, stream), "iter")
+    _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev),
+                                   ptr(labels), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
     status = _capi.LloydStatus()
     _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
 
@@ -104,18 +112,18 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     sums, ref_sizes = ok.weighted_sums(X, w, got_labels, k)
     n_empty = int(np.count_nonzero(ref_sizes == 0))
     assert status.n_empty == n_empty
-    np.testing.assert_allclose(sizes.cpu().numpy(), ref_sizes, rtol=RTOL[X.dtype] * 10)
+    np.testing.assert_allclose(sizes.cpu().numpy(), ref_sizes, rtol=RTOL[X.dtype])
     if n_empty:
         assert status.state == _capi.KMX_NEED_RELOCATION
         assert status.n_iter == 0
         np.testing.assert_array_equal(empty.cpu().numpy()[:n_empty], np.flatnonzero(ref_sizes == 0))
         got = c_out.cpu().numpy().T
-        assert_centers_close(got, sums, X.dtype, scale_rtol=RTOL[X.dtype] * 10)
+        assert_centers_close(got, sums, X.dtype)
     else:
         assert status.state == _capi.KMX_RUNNING
         assert status.n_iter == 1
         ref_centers = sums / ref_sizes[:, None]
-        assert_centers_close(c_out.cpu().numpy().T, ref_centers, X.dtype, scale_rtol=RTOL[X.dtype] * 10)
+        assert_centers_close(c_out.cpu().numpy().T, ref_centers, X.dtype)
         shift = float(np.sum((np.asarray(init, np.float64) - ref_centers.astype(np.float64)) ** 2))
         assert status.shift_sum == pytest.approx(shift, rel=1e-4)
         expected_changed = int(np.count_nonzero(got_labels != 0))
@@ -123,7 +131,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
-@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "F64d"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
@@ -143,18 +151,19 @@ def test_lockstep_iterations_match_oracle(cuda, name):
     labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
     sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
     empty = torch.empty(k, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, dc)
+    plan = _capi.lloyd_plan(n, d, k, dc, cfg.get("flags", 0))
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
     status = _capi.LloydStatus()
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, dc, 100, 0.0, stream), "init")
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 100, 0.0, stream), "init")
     prev = None
     for it in range(10):
         a, b = it % 2, (it + 1) % 2
         c_in = cent[a].cpu().numpy().T.copy()
-        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
-                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k,
-                                       dc, stream), "iter")
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream),
+                    "iter")
         _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
         got = labels[b].cpu().numpy().astype(np.int64)
         assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
@@ -198,8 +207,16 @@ def test_full_lloyd_run_matches_oracle(cuda, name):
     assert float(inertia) == pytest.approx(float(ok.inertia(Xc, w, centers, got)), rel=1e-5)
     if np.array_equal(got, ref_labels.astype(np.int64)):
         # same final partition: centroids must agree to rounding
+        # (ten roundings of 1e-5 / 1e-12: the two runs agree iteration by iteration, each
+        # within the per-iteration tolerance, and the iterations contract towards the fixed point)
         assert_centers_close(centers, ref_centers, X.dtype, scale_rtol=RTOL[X.dtype] * 10)
         assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-5)
     else:
-        # a near-tie flipped somewhere along the run: same quality, not the same partition
-        assert float(inertia) == pytest.approx(float(ref_inertia), rel=2e-3)
+        # a near-tie flipped somewhere along the run: a few samples at a boundary, not another
+        # clustering (per-iteration parity is what the lockstep test above asserts)
+        assert np.count_nonzero(got != ref_labels.astype(np.int64)) <= max(1, n_samples_differ_cap(X))
+        assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-4)
+
+
+def n_samples_differ_cap(X):
+    return X.shape[0] // 1000

@@ -6,7 +6,6 @@ must go to the lowest index, as in the reference's running arg-min,
 sklearn_numba_dpex/kmeans/kernels/_base_kmeans_kernel_funcs.py:228-267)."""
 
 import ctypes
-import os
 
 import numpy as np
 import pytest
@@ -17,16 +16,13 @@ from tests._parity import assert_centers_close, assert_labels_match
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True)
-def _screen_wherever_possible():
-    """The library screens the labels only where that is the faster kernel (from about ten
-    features on); the tests here want the screened kernel on every shape it can run."""
-    os.environ["KMX_LLOYD_ASSIGN"] = "screen"
-    yield
-    os.environ.pop("KMX_LLOYD_ASSIGN", None)
+# The library screens the labels only where that is the faster kernel (from about ten features
+# on); the tests here want the screened kernel on every shape it can run.
+SCREEN = 0x20   # KMX_FLAG_LABELS_SCREEN
+ALL_F32 = 0x10  # KMX_FLAG_LABELS_F32
 
 
-def _one_iteration(X, w, init, cuda):
+def _one_iteration(X, w, init, cuda, flags=SCREEN):
     """kmx_lloyd_init + one kmx_lloyd_iter through the C ABI; returns labels, new centroids
     (or the sums when a cluster is empty), sizes, status, variant, samples evaluated in fp32."""
     import torch
@@ -43,18 +39,19 @@ def _one_iteration(X, w, init, cuda):
     labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
     sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
     empty = torch.empty(k, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, 0)
+    plan = _capi.lloyd_plan(n, d, k, 0, flags)
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
-    variant = lib.kmx_lloyd_kernel_variant(n, d, k, 0)
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), n, d, k, 0, 10, 0.0, stream), "init")
+    variant = plan.variant
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), 10, 0.0, stream), "init")
     X_rm = dev(X) if variant == 42 else None  # the wide path sums (and screens) with a row-major copy
-    _capi.check(lib.kmx_lloyd_iter(ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev), ptr(labels),
-                                   ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, 0, stream), "iter")
+    _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev),
+                                   ptr(labels), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
     status = _capi.LloydStatus()
     _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
     rechecked = ctypes.c_uint32(0)
-    _capi.check(lib.kmx_lloyd_recheck_count(ptr(ws), n, d, k, 0, ctypes.byref(rechecked), stream), "recheck")
+    _capi.check(lib.kmx_lloyd_recheck_count(plan, ptr(ws), ctypes.byref(rechecked), stream), "recheck")
     return (labels.cpu().numpy().astype(np.int64), c_out.cpu().numpy().T, sizes.cpu().numpy(), status, variant,
             int(rechecked.value))
 
@@ -64,12 +61,12 @@ def _check_against_oracle(X, w, init, labels, c_out, sizes, status):
     assert labels.min() >= 0 and labels.max() < k
     assert_labels_match(labels, ok.assign_labels(X, init), X, init)
     sums, ref_sizes = ok.weighted_sums(X, w, labels, k)
-    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-4)
+    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-5)
     assert status.n_empty == int(np.count_nonzero(ref_sizes == 0))
     if status.n_empty == 0:
-        assert_centers_close(c_out, sums / ref_sizes[:, None], np.float32, scale_rtol=1e-4)
+        assert_centers_close(c_out, sums / ref_sizes[:, None], np.float32)
     else:
-        assert_centers_close(c_out, sums, np.float32, scale_rtol=1e-4)
+        assert_centers_close(c_out, sums, np.float32)
 
 
 def _blobs(n, d, k, seed, offset=0.0, scale=1.0):
@@ -95,7 +92,7 @@ def test_screened_step_matches_oracle(cuda, shape):
     assert rechecked <= 8 + n // 20
 
 
-def _labels_only(X, C, cuda, roomy=True):
+def _labels_only(X, C, cuda, roomy=True, flags=SCREEN):
     """kmx_assign_labels through the C ABI (the screened label kernels; with roomy=False the
     minimal workspace, with which wide shapes take the all-fp32 kernel)."""
     import torch
@@ -108,9 +105,10 @@ def _labels_only(X, C, cuda, roomy=True):
     X_t = torch.as_tensor(np.ascontiguousarray(X.T), device=cuda)
     c_t = torch.as_tensor(np.ascontiguousarray(C.T), device=cuda)
     labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_assign_workspace_bytes_for(n, d, k, 0) if roomy else lib.kmx_assign_workspace_bytes(d, k, 0)
+    ws_bytes = (lib.kmx_assign_workspace_bytes_for(n, d, k, 0, flags) if roomy
+                else lib.kmx_assign_workspace_bytes(d, k, 0))
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
-    _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(c_t), ptr(labels), ptr(ws), ws_bytes, n, d, k, 0,
+    _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(c_t), ptr(labels), ptr(ws), ws_bytes, n, d, k, 0, flags,
                                       _capi.current_stream()), "assign")
     return labels.cpu().numpy().astype(np.int64)
 
@@ -155,29 +153,24 @@ def test_labels_only_ties_and_zero_centroids(cuda):
 
 
 def test_default_choice_between_screened_and_fp32_step(cuda):
-    """Without the environment switch the screen is used where it is the faster kernel."""
+    """With flags = 0 the screen is used where it is the faster kernel."""
     from sklearn_numba_dpex_amd._capi import lib
 
-    os.environ.pop("KMX_LLOYD_ASSIGN", None)
     for (d, k), variant in {(14, 127): 61, (2, 16): 31, (8, 32): 31, (8, 64): 61, (6, 128): 61, (32, 64): 61}.items():
-        assert lib.kmx_lloyd_kernel_variant(100_000, d, k, 0) == variant, (d, k)
+        assert lib.kmx_lloyd_kernel_variant(100_000, d, k, 0, 0) == variant, (d, k)
     X, w, init = _blobs(5_000, 4, 20, seed=11)
-    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=0)
     assert variant == 31 and rechecked == 0
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
 
 
-def test_fp32_matrix_core_step_selected_by_environment(cuda):
-    """KMX_LLOYD_ASSIGN=f32 selects the all-fp32 kernel (variant 31); both give the oracle's labels."""
+def test_fp32_matrix_core_step_selected_by_flag(cuda):
+    """KMX_FLAG_LABELS_F32 selects the all-fp32 kernel (variant 31); both give the oracle's labels."""
     X, w, init = _blobs(30_000, 14, 127, seed=5)
     got = {}
     for mode in ("screen", "f32"):
-        if mode == "f32":
-            os.environ["KMX_LLOYD_ASSIGN"] = "f32"
-        try:
-            labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
-        finally:
-            os.environ["KMX_LLOYD_ASSIGN"] = "screen"
+        labels, c_out, sizes, status, variant, rechecked = _one_iteration(
+            X, w, init, cuda, flags=SCREEN if mode == "screen" else ALL_F32)
         assert variant == (61 if mode == "screen" else 31)
         if mode == "f32":
             assert rechecked == 0
@@ -299,7 +292,7 @@ def test_offsets_and_extreme_magnitudes(cuda, offset, scale):
     else:
         assert_labels_match(labels, ref, X, init)
     sums, ref_sizes = ok.weighted_sums(X, w, labels, k)
-    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-4)
+    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-5)
 
 
 def test_all_zero_data(cuda):
@@ -329,21 +322,21 @@ def test_ten_iterations_stay_in_lockstep_with_the_oracle(cuda):
     labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
     sizes = torch.empty(k, dtype=torch.float32, device=cuda)
     empty = torch.empty(k, dtype=torch.int32, device=cuda)
-    ws_bytes = lib.kmx_lloyd_workspace_bytes(n, d, k, 0)
+    plan = _capi.lloyd_plan(n, d, k, 0, SCREEN)
+    ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
-    assert lib.kmx_lloyd_kernel_variant(n, d, k, 0) == 61
-    _capi.check(lib.kmx_lloyd_init(ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), n, d, k, 0, 100, 0.0, stream), "init")
+    assert plan.variant == 61
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 100, 0.0, stream), "init")
     status = _capi.LloydStatus()
     rechecked = ctypes.c_uint32(0)
     for it in range(10):
         a, b = it % 2, (it + 1) % 2
         c_in = cent[a].cpu().numpy().T.copy()
-        _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
-                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, n, d, k, 0,
-                                       stream), "iter")
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
         _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
-        _capi.check(lib.kmx_lloyd_recheck_count(ptr(ws), n, d, k, 0, ctypes.byref(rechecked), stream), "recheck")
+        _capi.check(lib.kmx_lloyd_recheck_count(plan, ptr(ws), ctypes.byref(rechecked), stream), "recheck")
         got = labels[b].cpu().numpy().astype(np.int64)
         assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
         assert rechecked.value <= n // 50
@@ -451,7 +444,7 @@ def test_wide_screened_labels_only_match_oracle(cuda, shape):
 
     n, d, k = shape
     X, _, init = _blobs(n, d, k, seed=n + d + 2)
-    assert lib.kmx_assign_workspace_bytes_for(n, d, k, 0) > lib.kmx_assign_workspace_bytes(d, k, 0)
+    assert lib.kmx_assign_workspace_bytes_for(n, d, k, 0, SCREEN) > lib.kmx_assign_workspace_bytes(d, k, 0)
     ref = ok.assign_labels(X, init)
     for roomy in (True, False):
         labels = _labels_only(X, init, cuda, roomy=roomy)
@@ -495,13 +488,9 @@ def test_wide_all_centroids_identical(cuda):
     assert status.n_empty == 63
 
 
-def test_wide_screen_switched_off_by_environment(cuda):
+def test_wide_screen_switched_off_by_flag(cuda):
     X, w, init = _blobs(5_000, 128, 64, seed=43)
-    os.environ["KMX_LLOYD_ASSIGN"] = "f32"
-    try:
-        labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
-    finally:
-        os.environ["KMX_LLOYD_ASSIGN"] = "screen"
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=ALL_F32)
     assert variant == 42 and rechecked == 0
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
 
@@ -527,16 +516,17 @@ def test_many_ties_stay_affordable(cuda):
         lab1 = torch.empty(n, dtype=torch.int32, device=cuda)
         sizes = torch.empty(k, device=cuda)
         empty = torch.empty(k, dtype=torch.int32, device=cuda)
-        wsb = lib.kmx_lloyd_workspace_bytes(n, d, k, 0)
+        plan = _capi.lloyd_plan(n, d, k, 0, SCREEN)
+        wsb = plan.workspace_bytes
         ws = torch.empty(wsb, dtype=torch.uint8, device=cuda)
         st = _capi.current_stream()
         best = 1e9
         for _ in range(3):
-            _capi.check(lib.kmx_lloyd_init(ptr(ws), wsb, ptr(X_t), ptr(w), ptr(c_in), n, d, k, 0, 10, 0.0, st), "init")
+            _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), wsb, ptr(X_t), ptr(w), ptr(c_in), 10, 0.0, st), "init")
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            _capi.check(lib.kmx_lloyd_iter(ptr(X_t), None, ptr(w), ptr(c_in), ptr(c_out), ptr(lab0), ptr(lab1),
-                                           ptr(sizes), ptr(empty), ptr(ws), wsb, n, d, k, 0, st), "iter")
+            _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w), ptr(c_in), ptr(c_out), ptr(lab0), ptr(lab1),
+                                           ptr(sizes), ptr(empty), ptr(ws), wsb, st), "iter")
             torch.cuda.synchronize()
             best = min(best, (time.perf_counter() - t0) * 1e3)
         return best, lab1
