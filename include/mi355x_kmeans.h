@@ -322,6 +322,17 @@ size_t kmx_sum_workspace_bytes(int64_t rows, int64_t cols);
 int32_t kmx_sum_rows(const void* in, void* out, int64_t rows, int64_t cols, int32_t square,
                      void* workspace, size_t workspace_bytes, int32_t dtype, void* stream);
 
+/* kmx_sum_rows for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same kernels and the same result,
+ * with the per-workgroup partial sums in a 128 KiB array that is part of the library's device
+ * image instead of a caller-provided workspace.  It has no counterpart in the reference.
+ * Calls no hipMalloc / hipFree or any allocating routine.  Limit: rows <= 64 (else
+ * KMX_ERR_UNSUPPORTED); cols unlimited.  Each GPU has ONE such array, shared by every call
+ * on that GPU: calls that overlap in time on one GPU (different streams, different threads)
+ * race on it and must be ordered by the caller.  Nothing in it needs to start at zero. */
+int32_t kmx_sum_rows_static(const void* in, void* out, int64_t rows, int64_t cols, int32_t square,
+                            int32_t dtype, void* stream);
+
 /* out[c] = sum_r in[r, c].  Replaces the axis=0 form (common/reductions.py:462-640). */
 int32_t kmx_sum_cols(const void* in, void* out, int64_t rows, int64_t cols, void* workspace,
                      size_t workspace_bytes, int32_t dtype, void* stream);

@@ -129,6 +129,7 @@ SIGNATURES = {
     "kmx_kpp_candidates_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),
     "kmx_sum_workspace_bytes": (_SZ, [_I64, _I64]),
     "kmx_sum_rows": (_I32, [_P, _P, _I64, _I64, _I32, _P, _SZ, _I32, _P]),
+    "kmx_sum_rows_static": (_I32, [_P, _P, _I64, _I64, _I32, _I32, _P]),
     "kmx_sum_cols": (_I32, [_P, _P, _I64, _I64, _P, _SZ, _I32, _P]),
     "kmx_argmin": (_I32, [_P, _P, _I64, _I32, _P]),
     "kmx_half_sq_norms": (_I32, [_P, _P, _I32, _I32, _I32, _P]),

@@ -4,6 +4,7 @@
 // block order), so results do not change from run to run.
 #include "kmx_common.h"
 
+#include <mutex>
 #include <type_traits>
 
 namespace {
@@ -302,6 +303,57 @@ int32_t kmx_sum_rows(const void* in, void* out, int64_t rows, int64_t cols, int3
 #undef KMX_SUM_ROWS
     KMX_LAUNCH_CHECK();
     return KMX_OK;
+}
+
+// ---- kmx_sum_rows without any allocation: the per-workgroup partial sums live in a
+// file-scope device array instead of a caller-provided workspace.
+}  // extern "C"
+
+namespace {
+constexpr int SUM_STATIC_MAX_ROWS = 64;
+__device__ __align__(256) double sum_static_scratch[SUM_STATIC_MAX_ROWS * SUM_MAX_BLOCKS_PER_ROW];  // 128 KiB
+
+// Device address of sum_static_scratch on the current device (every GPU holds its own copy of
+// the array at its own address; the array's name is only a host-side handle and must never be
+// handed to a kernel).  Looked up once per device; no allocation.
+constexpr int SUM_STATIC_MAX_DEVICES = 64;
+int32_t sum_static_scratch_ptr(double** out) {
+    static double* ptrs[SUM_STATIC_MAX_DEVICES] = {};
+    static std::mutex lock;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int32_t)e;
+    if (dev < 0 || dev >= SUM_STATIC_MAX_DEVICES) return KMX_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> guard(lock);
+    if (ptrs[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(sum_static_scratch));
+        if (e != hipSuccess) return (int32_t)e;
+        if (p == nullptr) return KMX_ERR_UNSUPPORTED;
+        ptrs[dev] = static_cast<double*>(p);
+    }
+    *out = ptrs[dev];
+    return KMX_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int32_t kmx_sum_rows_static(const void* in, void* out, int64_t rows, int64_t cols, int32_t square,
+                            int32_t dtype, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(in);
+    KMX_REQUIRE_PTR(out);
+    if (rows <= 0 || cols <= 0) return KMX_ERR_BAD_SHAPE;
+    if (rows > SUM_STATIC_MAX_ROWS) return KMX_ERR_UNSUPPORTED;  // beyond the static scratch
+    KMX_REQUIRE_DTYPE(dtype);
+    double* partial = nullptr;
+    const int32_t rc = sum_static_scratch_ptr(&partial);
+    if (rc != KMX_OK) return rc;
+    // stage 1 writes every slot stage 2 reads (rows * b of them), so nothing has to start at
+    // zero and the previous call's contents do not matter
+    return kmx_sum_rows(in, out, rows, cols, square, partial,
+                        sizeof(double) * SUM_STATIC_MAX_ROWS * SUM_MAX_BLOCKS_PER_ROW, dtype, stream_);
 }
 
 int32_t kmx_sum_cols(const void* in, void* out, int64_t rows, int64_t cols, void* workspace,
