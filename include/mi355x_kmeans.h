@@ -150,7 +150,12 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
  *                                 new_centroids_t of the previous one (the workspace holds a
  *                                 packed copy and the half squared norms of exactly those)
  *   new_centroids_t  OUT  (d, k)  un-normalised sums if relocation is needed, else new centroids
- *   labels_prev      IN   (n)     labels of the previous iteration
+ *   labels_prev      IN   (n)     labels of the previous iteration: from the second iteration on
+ *                                 exactly the array the previous kmx_lloyd_iter of this workspace
+ *                                 wrote as `labels` (the callers ping-pong two arrays).  Besides
+ *                                 the count of changed labels, variant 61 builds on it: once few
+ *                                 labels change it no longer rebuilds its integer sums but moves
+ *                                 every sample that changes cluster from the old sum to the new one
  *   labels           OUT  (n)
  *   cluster_sizes    OUT  (k)     sum of weights per cluster
  *   empty_clusters   OUT  (k)     ids of empty clusters, ascending, first status.n_empty valid */

@@ -46,7 +46,8 @@ def flag_cols(x):
 ABI_VERSION = 2
 
 LIB_NAME = "libmi355x_kmeans.so"
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+# (KMX_LIBRARY_PATH: another build of the same library, for experiments; read when this module is imported)
+LIB_PATH = os.environ.get("KMX_LIBRARY_PATH") or os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 
 class LloydStatus(ctypes.Structure):

@@ -604,6 +604,10 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         // labels screened on the fp16 matrix cores (lloyd_mfma_screen.hip)
         uint32_t* uncertain = reinterpret_cast<uint32_t*>(ws + L.off_bucket);
         tail.clear_word = uncertain;
+        // sums corrected instead of rebuilt once an iteration changes at most one label in 64
+        // (above that nearly every 64-sample tile holds a change and rebuilding is cheaper)
+        tail.n_samples = n;
+        tail.delta_divisor = 64;
         const int32_t rc = kmx_lloyd_step_mfma_screen(
             X_t, w, centroids_t, labels_prev, labels, tail.status,
             reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain,

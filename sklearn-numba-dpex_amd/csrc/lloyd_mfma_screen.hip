@@ -51,12 +51,33 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 constexpr float SCR_ERR_SPLIT = 7.2e-7f;  // 3.01 * 2^-22, rounded up
 constexpr float SCR_ERR_ROUND = 1.2e-7f;  // 2^-23, rounded up
 constexpr float SCR_ERR_ABS = 6.2e-5f;    // 2^-14, rounded up
+// Scaled data lie in [2^(SCR_SCALE_EXP - 1), 2^SCR_SCALE_EXP): low enough for -0.5||c||^2 / SCR_HK_X1
+// to stay inside fp16 for every d <= 31 (0.5 * 31 * 2^26 / 2^15 < 2^15), high enough for the
+// absolute term of the bound to stay a few percent of the relative one.
+constexpr int SCR_SCALE_EXP = 13;
+// When the last K step has a feature slot to spare (d not a multiple of 16), -0.5||c||^2 rides in
+// it instead of in the accumulator's start value: the samples carry the constant SCR_HK_X1 there
+// (hi part; lo part zero) and the centroids the two fp16 parts of -0.5||c||^2 / SCR_HK_X1, so
+// that hi*hi + lo*hi add it up to 2^-22 relative (SCR_ERR_HNEG), or 2^-14 * SCR_HK_X1 absolute
+// should the lo part be flushed.  The accumulators then start from the constant zero: no read
+// of sixteen start values per block and column, no registers for them.
+constexpr float SCR_HK_X1 = 32768.0f;
+constexpr float SCR_ERR_HNEG = 3.0e-7f;  // 2^-22 for the two-part value, 2^-24 for its fp32 original, rounded up
 constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
 constexpr int SCR_REDO_COLUMN = 3;  // uncertain samples from which a 32-sample column is redone in fp32
+// Words of the step's counter block in the workspace (`uncertain_count`): samples evaluated in
+// fp32 by the running iteration, the same of the last finished one, and whether the next step
+// may correct the sums for the label changes only (written by the finalisation).
+constexpr int SCR_WORD_DELTA = 2;
 
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
 #ifndef KMX_SCR_WAVES
 #define KMX_SCR_WAVES 12
+#endif
+// Matrix-core and vector work of one wave interleaved (software pipeline over the centroid
+// blocks); 0 restores blockwise scoring for comparison.
+#ifndef KMX_SCR_PIPE
+#define KMX_SCR_PIPE 1
 #endif
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
 
@@ -73,7 +94,9 @@ constexpr int SCR_QUEUE_MAX = 256;
 __host__ __device__ constexpr size_t scr_lds_max(int nk) { return nk == 1 ? 156 * 1024 : 78 * 1024; }
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
-    const size_t n_cb = (size_t)(k + 31) / 32;
+    // (an even number of centroid blocks: the scoring loop takes them in pairs; a block past
+    // the last one holds padding only, whose scores are -inf)
+    const size_t n_cb = (((size_t)(k + 31) / 32) + 1) & ~(size_t)1;
     // sums, cluster-major: per cluster the features, a spare word when d is odd, then the size
     const size_t acc = update ? (((size_t)(((d + 1) & ~1) + 1) * k * 8 + 15) & ~(size_t)15) : 0;
     s.off_afh = acc;
@@ -144,8 +167,8 @@ __device__ __forceinline__ uint32_t redo_column_fp32(ColumnRows rows, const floa
     return (uint32_t)bc;
 }
 
-template <int NK, bool UPDATE>
-__global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
+template <int NK, bool UPDATE, bool HK>
+__global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2) void lloyd_screen_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
@@ -157,8 +180,15 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     constexpr int WAVES = scr_waves(NK), THREADS = 64 * WAVES;
     constexpr int MC = 2, TILE = 64;
     constexpr int G = SCR_GROUP, NG = 16 / SCR_GROUP;
+    // HK: the feature slot that carries -0.5||c||^2: the last K index of the last K step (it
+    // holds no feature, d being no multiple of 16), i.e. pair 7 of that step in the upper half-wave
+    constexpr int SPARE = 16 * NK - 1;
+    using Cols0 = std::integral_constant<int, 0>;  // column tags of the arg-max, column counts of a tile
+    using Cols1 = std::integral_constant<int, 1>;
+    using Cols2 = std::integral_constant<int, MC>;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int n_cb = (k + 31) >> 5;
+    const int n_cbe = (n_cb + 1) & ~1;  // blocks in the operand arrays: an even number, padding at the end
     // Accumulators: cluster-major, acc_stride = d_even + 1 words per cluster: feature f in word f,
     // the cluster size in word d_even.  For odd d the word between them takes what the upper
     // half-wave adds for the feature that does not exist (never read), so that the update needs
@@ -190,6 +220,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 
     __shared__ unsigned int xmax_bits;
     __shared__ unsigned int tile_ticket;
+    __shared__ int q_lds[36];  // binary points of the fixed-point sums: features, then the weights
+    if (UPDATE && threadIdx.x <= d) q_lds[threadIdx.x] = q_exp[threadIdx.x];
     if (threadIdx.x == 0) {
         tile_ticket = 0;
         changed_block = 0;
@@ -218,16 +250,16 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         if (UPDATE ? threadIdx.x < d : my_absmax != 0u) atomicMax(&xmax_bits, my_absmax);
     }
     __syncthreads();
-    // 2^-a with max|x| * 2^-a in [2^14, 2^15) (1 for all-zero or non-finite data)
+    // 2^-a with max|x| * 2^-a in [2^(SCR_SCALE_EXP - 1), 2^SCR_SCALE_EXP) (1 for all-zero or non-finite data)
     const float xmax = __uint_as_float(xmax_bits);
-    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, 14 - ilogbf(xmax)) : 1.0f;
+    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, SCR_SCALE_EXP - 1 - ilogbf(xmax)) : 1.0f;
     // The four pieces of work below start at different waves (thread index rotated by a third,
     // a half, two thirds of the workgroup): each is a chain of LDS round trips too short to
     // fill the workgroup, and one after the other on the same threads they took 3.7 us.
     auto rotated = [&](const int by) { return (int)((threadIdx.x + THREADS - by) % THREADS); };
     constexpr int ROT_HNEG = (THREADS / 3) & ~63, ROT_HX = THREADS / 2, ROT_ZERO = (2 * THREADS / 3) & ~63;
     // A operand: hi and lo parts of 32 centroids x 16 features per block and K step
-    for (int idx = threadIdx.x; idx < n_cb * NK * 64; idx += THREADS) {
+    for (int idx = threadIdx.x; idx < n_cbe * NK * 64; idx += THREADS) {
         const int l = idx & 63;
         const int s = (idx >> 6) % NK;
         const int cb = (idx >> 6) / NK;
@@ -236,15 +268,35 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int f = 16 * s + 2 * i + (l >> 5);
-            const float v = f < d ? ct[f * kp + c] * xs : 0.0f;
+            float v = f < d ? ct[f * kp + c] * xs : 0.0f;
+            if (HK && f == SPARE) {
+                // the spare slot: -0.5||c||^2 / SCR_HK_X1, summed exactly as for hneg below;
+                // -inf for the padding past k, whose scores then never win
+                v = -kmx_inf<float>();
+                if (c < k) {
+                    float sq = 0.0f;
+#pragma unroll 8
+                    for (int g = 0; g < d; ++g) {
+                        const float cv = ct[g * kp + c] * xs;
+                        sq += cv * cv;
+                    }
+                    v = -(sq / 2.0f) * (1.0f / SCR_HK_X1);
+                }
+            }
             const _Float16 hb = (_Float16)v;
             hi[i] = hb;
             lo[i] = (_Float16)(v - (float)hb);
+            if (HK && f == SPARE && !(c < k)) {
+                // the -inf of the padding goes into the lo part alone: it then only meets the
+                // sample's constant (hi part) and never a zero, which would give NaN
+                hi[i] = (_Float16)0.0f;
+                lo[i] = hb;
+            }
         }
         afh[idx] = hi;
         afl[idx] = lo;
     }
-    for (int idx = rotated(ROT_HNEG); idx < n_cb * 32; idx += THREADS) {
+    for (int idx = rotated(ROT_HNEG); idx < n_cbe * 32; idx += THREADS) {  // (-inf for the padding)
         const int cb = idx >> 5, hh = (idx >> 4) & 1, r = idx & 15;
         const int c = 32 * cb + 8 * (r >> 2) + 4 * hh + (r & 3);
         float v = -kmx_inf<float>();
@@ -296,60 +348,102 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     // (||x|| comes unscaled from kmx_lloyd_init, hence the factor xs)
     // (and a norm the kernel takes itself, from the scaled values: no factor)
     const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term) * (UPDATE ? xs : 1.0f);
-    const float thr_0 = 2.01f * (round_term * hmax + abs_term * cmax);
+    const float thr_0 = 2.01f * (round_term * hmax + abs_term * cmax +
+                                 (HK ? SCR_ERR_HNEG * hmax + SCR_ERR_ABS * SCR_HK_X1 : 0.0f));
+    // what a sample carries in the spare slot: its scaled value is SCR_HK_X1
+    const float hk_x = SCR_HK_X1 / xs;
     // +inf the optimiser cannot see through (it would turn the median below into a maximum
     // with two canonicalising instructions in front)
     float pos_inf = kmx_inf<float>();
     asm volatile("" : "+s"(pos_inf));
     const float neg_inf = -kmx_inf<float>();
+    // the scale as a scalar operand of the conversions
+    const float xs_s = __uint_as_float((unsigned int)__builtin_amdgcn_readfirstlane((int)__float_as_uint(xs)));
 
-    // The lane's features: pair p = 8 s + i, feature 2 p + h.  xsr: 2^-a, or 0 for a feature
-    // that does not exist (its loads read row d - 1); magic: see fix_magic.
-    float xsr[NK][8];
-    double magic[NK][8];
-    double magic_w = 0.0;
-#pragma unroll
-    for (int s = 0; s < NK; ++s)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int f = 16 * s + 2 * i + h;
-            xsr[s][i] = f < d ? xs : 0.0f;
-            magic[s][i] = 0.0;
-            if (UPDATE) magic[s][i] = fix_magic(f < d ? q_exp[f] : 0);
-        }
-    if (UPDATE) magic_w = fix_magic(q_exp[d]);
+    // Fused step: whether the sums are rebuilt from every sample (first iteration, or after one
+    // that changed many labels) or only corrected for the samples whose label changes: the
+    // fixed-point sums are integers, so taking a sample's terms off its old cluster and adding
+    // them to the new one leaves exactly the sums a full pass would produce.
+    const bool full_mode = UPDATE ? (uncertain_count[SCR_WORD_DELTA] == 0u) : false;  // wave-uniform
 
-    // One tile of NC sample columns per lane (NC = 2: samples i0, i0 + 1; NC = 1: sample i0).
-    // x holds the lane's rows at its samples (row d - 1 where the feature does not exist).
-    auto process = [&](auto nc_tag, auto full_tag,
-                       const float(&x)[NK][8][decltype(nc_tag)::value],
-                       const float(&wv)[decltype(nc_tag)::value],
-                       const uint32_t(&pl)[decltype(nc_tag)::value],
-                       const float(&xnorm)[decltype(nc_tag)::value], const int64_t i0) {
+    // One tile of NC sample columns per lane.  NC = 2: 64 samples, lane (j, h) scores samples
+    // i0 and i0 + 1 (i0 = first + 2 j) against its half of every centroid block and, once the
+    // two half-waves have exchanged their results, OWNS sample i0 + h (threshold test, label,
+    // bookkeeping).  NC = 1: 32 samples, sample i0 = first + j, owned by the lower half-wave.
+    // `load` fills the lane's rows x[s][i][t] = feature 16 s + 2 i + h of sample i0 + t (row
+    // d - 1 where the feature does not exist: the centroid operand is zero there); it is called
+    // again by the rare paths that need the fp32 values once more, so that they do not occupy
+    // registers across the scoring.
+    // `x`, `norm_in`, `pl_in`: the lane's rows, the owner's norm and previous label, loaded by the
+    // caller (for full tiles: while the previous tile was being scored); `refill` is called once
+    // they have been consumed and may load the next tile's into the same variables.
+    auto process = [&](auto nc_tag, auto full_tag, auto&& load, auto&& refill,
+                       float(&x)[NK][8][decltype(nc_tag)::value], float& norm_in, uint32_t& pl_in,
+                       const int64_t i0) __attribute__((always_inline)) {
         constexpr int NC = decltype(nc_tag)::value;
         constexpr bool FULL = decltype(full_tag)::value;
+        const int64_t my_idx = NC == 2 ? i0 + h : i0;
+        const bool owner = NC == 2 ? true : h == 0;
+        const bool in_range = FULL || my_idx < n;
 
-        // scaled fp16 split of the B operand
+        // the owner's norm and previous label
+        float norm_mine = norm_in;
+        const uint32_t pl_mine = pl_in;
+
+        // scaled fp16 split of the B operand: hi = fp16(x * 2^-a), lo = fp16(x * 2^-a - hi), each
+        // one mixed-precision fused multiply-add with a single rounding (the product with a power
+        // of two and the difference are exact)
         v8h xh[NK][NC], xl[NK][NC];
         float own_sq[NC];  // labels only: the lane's part of ||x||^2, scaled
+        {
+            const float xs_sc = xs_s;  // (a local: operands of inline assembly must be the lambda's own)
 #pragma unroll
-        for (int t = 0; t < NC; ++t) {
-            own_sq[t] = 0.0f;
+            for (int t = 0; t < NC; ++t) {
+                own_sq[t] = 0.0f;
 #pragma unroll
-            for (int s = 0; s < NK; ++s)
+                for (int s = 0; s < NK; ++s) {
+                    unsigned int hw[4], lw[4];
+                    // Sixteen instructions in ONE statement: between separate statements the
+                    // compiler pads every dependency on an assembly result with a wait state
+                    // (it must assume a partial register write).  The real rule - a 16-bit write
+                    // needs one instruction between it and a read of that register - is kept
+                    // by the order: the four registers are written in rotation.  The closing
+                    // s_nop gives a vector-ALU result the two wait states it needs before a
+                    // matrix instruction may read it.
+                    asm("v_fma_mixlo_f16 %0, %8, %16, 0\n\t"
+                        "v_fma_mixlo_f16 %1, %10, %16, 0\n\t"
+                        "v_fma_mixlo_f16 %2, %12, %16, 0\n\t"
+                        "v_fma_mixlo_f16 %3, %14, %16, 0\n\t"
+                        "v_fma_mixhi_f16 %0, %9, %16, 0\n\t"
+                        "v_fma_mixhi_f16 %1, %11, %16, 0\n\t"
+                        "v_fma_mixhi_f16 %2, %13, %16, 0\n\t"
+                        "v_fma_mixhi_f16 %3, %15, %16, 0\n\t"
+                        "v_fma_mixlo_f16 %4, %8, %16, -%0 op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixlo_f16 %5, %10, %16, -%1 op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixlo_f16 %6, %12, %16, -%2 op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixlo_f16 %7, %14, %16, -%3 op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixhi_f16 %4, %9, %16, -%0 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixhi_f16 %5, %11, %16, -%1 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixhi_f16 %6, %13, %16, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+                        "v_fma_mixhi_f16 %7, %15, %16, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+                        "s_nop 1"
+                        : "=&v"(hw[0]), "=&v"(hw[1]), "=&v"(hw[2]), "=&v"(hw[3]), "=&v"(lw[0]), "=&v"(lw[1]),
+                          "=&v"(lw[2]), "=&v"(lw[3])
+                        : "v"(x[s][0][t]), "v"(x[s][1][t]), "v"(x[s][2][t]), "v"(x[s][3][t]), "v"(x[s][4][t]),
+                          "v"(x[s][5][t]), "v"(x[s][6][t]), "v"(x[s][7][t]), "s"(xs_sc));
+                    if (!UPDATE) {
 #pragma unroll
-                for (int i = 0; i < 8; i += 2) {
-                    const v2f p = {x[s][i][t] * xsr[s][i], x[s][i + 1][t] * xsr[s][i + 1]};
-                    if (!UPDATE) own_sq[t] = fmaf(p[1], p[1], fmaf(p[0], p[0], own_sq[t]));
-                    const v2h hh = __builtin_convertvector(p, v2h);
-                    const v2f r = p - __builtin_convertvector(hh, v2f);
-                    const v2h ll = __builtin_convertvector(r, v2h);
-                    xh[s][t][i] = hh[0];
-                    xh[s][t][i + 1] = hh[1];
-                    xl[s][t][i] = ll[0];
-                    xl[s][t][i + 1] = ll[1];
+                        for (int i = 0; i < 8; ++i) {
+                            const float pv = (16 * s + 2 * i + h < d) ? x[s][i][t] * xs : 0.0f;
+                            own_sq[t] = fmaf(pv, pv, own_sq[t]);
+                        }
+                    }
+                    xh[s][t] = __builtin_bit_cast(v8h, make_uint4(hw[0], hw[1], hw[2], hw[3]));
+                    xl[s][t] = __builtin_bit_cast(v8h, make_uint4(lw[0], lw[1], lw[2], lw[3]));
                 }
+            }
         }
+        refill();
 
         // Running arg-max by groups of G accumulator registers, plus the second largest of
         // the group maxima (the median of best, second and the new maximum).
@@ -370,10 +464,50 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             code[t] = 0;
         }
 
-        // approximate scores of centroid block cb for the NC columns
-        auto scores = [&](const int cb, v16f(&a)[NC]) __attribute__((always_inline)) {
+        // One arg-max group: registers g * G .. g * G + G - 1 of the accumulator `acc` of one
+        // column (centroid block cb); bst / sec / cde and the four register pairs sa .. sd are
+        // that column's running state.  g is a literal at every call.
+        auto argmax_group_of = [&](const int cb, const int g, const v16f& av, float& bst, float& sec,
+                                   unsigned int& cde, double& sa, double& sb, double& sc, double& sd)
+                                   __attribute__((always_inline)) {
+            const unsigned int cd = (unsigned int)(cb * NG + g);  // wave-uniform
+            // The first read of the matrix-core result is an instruction the compiler
+            // knows (the median of a, b and +inf is max(a, b)): it inserts the wait
+            // states an MFMA result needs before a vector-ALU read, which it does not
+            // do for operands of inline assembly.
+            float m = __builtin_amdgcn_fmed3f(av[g * G], av[g * G + 1], pos_inf);
+            // (one statement: see the conversion above)
+            static_assert(G == 8, "three three-operand maxima after the first pair");
+            asm("v_max3_f32 %0, %0, %2, %3\n\t"
+                "v_max3_f32 %0, %0, %4, %5\n\t"
+                "v_max3_f32 %0, %0, %6, %7\n\t"
+                "v_med3_f32 %1, %8, %1, %0"
+                : "+v"(m), "+v"(sec)
+                : "v"(av[g * G + 2]), "v"(av[g * G + 3]), "v"(av[g * G + 4]), "v"(av[g * G + 5]), "v"(av[g * G + 6]),
+                  "v"(av[g * G + 7]), "v"(bst));
+            // strict: the earlier group keeps a tie
+            if (m > bst) {
+                bst = m;
+                cde = cd;
+                const v8d ad = __builtin_bit_cast(v8d, av);
+                asm volatile("v_mov_b64 %0, %1" : "+v"(sa) : "v"(ad[g * 4]));
+                asm volatile("v_mov_b64 %0, %1" : "+v"(sb) : "v"(ad[g * 4 + 1]));
+                asm volatile("v_mov_b64 %0, %1" : "+v"(sc) : "v"(ad[g * 4 + 2]));
+                asm volatile("v_mov_b64 %0, %1" : "+v"(sd) : "v"(ad[g * 4 + 3]));
+            }
+        };
+        auto argmax_group = [&](const int cb, auto g_tag, auto t_tag, const v16f& av) __attribute__((always_inline)) {
+            constexpr int g = decltype(g_tag)::value, t = decltype(t_tag)::value;
+            if constexpr (t == 0)
+                argmax_group_of(cb, g, av, best[0], second[0], code[0], s00, s01, s02, s03);
+            else
+                argmax_group_of(cb, g, av, best[NC - 1], second[NC - 1], code[NC - 1], s10, s11, s12, s13);
+        };
+        using G0 = std::integral_constant<int, 0>;
+        using G1 = std::integral_constant<int, 1>;
+        static_assert(NG == 2, "two arg-max groups per accumulator");
+        auto load_hneg = [&](const int cb, v16f& hv) __attribute__((always_inline)) {
             const float4* hp = reinterpret_cast<const float4*>(hneg + cb * 32 + h * 16);
-            v16f hv;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float4 v4 = hp[q];
@@ -382,67 +516,93 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 hv[4 * q + 2] = v4.z;
                 hv[4 * q + 3] = v4.w;
             }
-#pragma unroll
-            for (int s = 0; s < NK; ++s) {
-                const v8h ah = afh[(cb * NK + s) * 64 + lane];
-                const v8h al = afl[(cb * NK + s) * 64 + lane];
-#pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    a[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xh[s][t], s == 0 ? hv : a[t], 0, 0, 0);
-#pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    a[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xl[s][t], a[t], 0, 0, 0);
-#pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    a[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, xh[s][t], a[t], 0, 0, 0);
-            }
         };
-        auto argmax_block = [&](const int cb, const v16f(&a)[NC]) __attribute__((always_inline)) {
+
+        if constexpr (KMX_SCR_PIPE && NK == 1 && NC == 2) {
+            // Software pipeline over the stages (block cb, column t), t fastest: while the vector
+            // ALU works through the scores of one stage, the matrix core already forms those of
+            // the next (the other column's accumulator), one MFMA of its chain of three issued
+            // ahead of each arg-max group.  fp16 MFMAs run beside vector instructions on this
+            // hardware, but only if a wave has both kinds to issue: with all MFMAs of a block
+            // first and all of its arg-max after, the waves of a SIMD fall into step and the two
+            // units take turns.
+            v16f a0, a1, hv;  // hv: the accumulators' start, -0.5||c||^2 of the block or (HK) zero
+            v8h ahA, alA, ahB, alB;  // A operands of the block at hand and of the next one
+            ahA = afh[lane];
+            alA = afl[lane];
+            if constexpr (HK) {
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                const unsigned int cd = (unsigned int)(cb * NG + g);  // wave-uniform
-#pragma unroll
-                for (int t = 0; t < NC; ++t) {
-                    // The first read of the matrix-core result is an instruction the compiler
-                    // knows (the median of a, b and +inf is max(a, b)): it inserts the wait
-                    // states an MFMA result needs before a vector-ALU read, which it does not
-                    // do for operands of inline assembly.
-                    float m = __builtin_amdgcn_fmed3f(a[t][g * G], a[t][g * G + 1], pos_inf);
-#pragma unroll
-                    for (int r = 2; r + 1 < G; r += 2)
-                        asm("v_max3_f32 %0, %1, %2, %3"
-                            : "=v"(m)
-                            : "v"(m), "v"(a[t][g * G + r]), "v"(a[t][g * G + r + 1]));
-                    asm("v_med3_f32 %0, %1, %2, %3" : "=v"(second[t]) : "v"(best[t]), "v"(second[t]), "v"(m));
-                    // strict: the earlier group keeps a tie
-                    if (m > best[t]) {
-                        best[t] = m;
-                        code[t] = cd;
-                        const v8d ad = __builtin_bit_cast(v8d, a[t]);
-                        if (t == 0) {
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s00) : "v"(ad[g * 4]));
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s01) : "v"(ad[g * 4 + 1]));
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s02) : "v"(ad[g * 4 + 2]));
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s03) : "v"(ad[g * 4 + 3]));
-                        } else {
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s10) : "v"(ad[g * 4]));
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s11) : "v"(ad[g * 4 + 1]));
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s12) : "v"(ad[g * 4 + 2]));
-                            asm volatile("v_mov_b64 %0, %1" : "+v"(s13) : "v"(ad[g * 4 + 3]));
-                        }
-                    }
+                for (int r = 0; r < 16; ++r) hv[r] = 0.0f;
+            } else {
+                load_hneg(0, hv);
+            }
+            a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahA, xh[0][0], hv, 0, 0, 0);
+            a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahA, xl[0][0], a0, 0, 0, 0);
+            a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(alA, xh[0][0], a0, 0, 0, 0);
+            // stages (cb, 0) and (cb, 1); (ahC, alC) hold block cb, (ahN, alN) receive block cb + 1
+            // when there is one (MORE)
+            auto block_pair = [&](auto more_tag, const int cb, const v8h& ahC, const v8h& alC, v8h& ahN, v8h& alN)
+                                  __attribute__((always_inline)) {
+                constexpr bool MORE = decltype(more_tag)::value;
+                a1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahC, xh[0][1], hv, 0, 0, 0);
+                if constexpr (MORE) {
+                    ahN = afh[(cb + 1) * 64 + lane];
+                    alN = afl[(cb + 1) * 64 + lane];
                 }
+                argmax_group(cb, G0{}, Cols0{}, a0);
+                if constexpr (MORE && !HK) load_hneg(cb + 1, hv);  // its last reader, the MFMA above, has long finished
+                a1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahC, xl[0][1], a1, 0, 0, 0);
+                argmax_group(cb, G1{}, Cols0{}, a0);
+                a1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(alC, xh[0][1], a1, 0, 0, 0);
+                if constexpr (MORE) a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahN, xh[0][0], hv, 0, 0, 0);
+                argmax_group(cb, G0{}, Cols1{}, a1);
+                if constexpr (MORE) a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahN, xl[0][0], a0, 0, 0, 0);
+                argmax_group(cb, G1{}, Cols1{}, a1);
+                if constexpr (MORE) a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(alN, xh[0][0], a0, 0, 0, 0);
+            };
+            // (n_cbe is even: an odd number of real blocks is followed by one of padding, whose
+            // scores are -inf; one straight-line tail, so that no registers change place at a join)
+            int cb = 0;
+            for (; cb + 2 < n_cbe; cb += 2) {
+                block_pair(std::true_type{}, cb, ahA, alA, ahB, alB);
+                block_pair(std::true_type{}, cb + 1, ahB, alB, ahA, alA);
             }
-        };
-        for (int cb = 0; cb < n_cb; ++cb) {
-            v16f a[NC];
-            scores(cb, a);
-            argmax_block(cb, a);
+            block_pair(std::true_type{}, cb, ahA, alA, ahB, alB);
+            block_pair(std::false_type{}, cb + 1, ahB, alB, ahA, alA);
+        } else {
+            for (int cb = 0; cb < n_cb; ++cb) {
+                v16f a[NC], hv;
+                if constexpr (HK) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) hv[r] = 0.0f;
+                } else {
+                    load_hneg(cb, hv);
+                }
+#pragma unroll
+                for (int s = 0; s < NK; ++s) {
+                    const v8h ah = afh[(cb * NK + s) * 64 + lane];
+                    const v8h al = afl[(cb * NK + s) * 64 + lane];
+#pragma unroll
+                    for (int t = 0; t < NC; ++t)
+                        a[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xh[s][t], s == 0 ? hv : a[t], 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < NC; ++t)
+                        a[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xl[s][t], a[t], 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < NC; ++t)
+                        a[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, xh[s][t], a[t], 0, 0, 0);
+                }
+                argmax_group(cb, G0{}, Cols0{}, a[0]);
+                if constexpr (NC == 2) argmax_group(cb, G0{}, Cols1{}, a[1]);
+                argmax_group(cb, G1{}, Cols0{}, a[0]);
+                if constexpr (NC == 2) argmax_group(cb, G1{}, Cols1{}, a[1]);
+            }
         }
 
-        // position inside the winning group, second largest inside it, then both half-waves
-        uint32_t lab[NC];
-        bool unsure[NC];
+        // Per column and half-wave: position inside the winning group and the second largest
+        // inside it.
+        float sec_c[NC];
+        unsigned int cen_c[NC];
 #pragma unroll
         for (int t = 0; t < NC; ++t) {
             float sv[G];
@@ -465,65 +625,72 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             // Second largest of the eight (equal to the largest if that occurs twice), by a
             // tournament of (largest, second) pairs: triples give max3 / med3, and two pairs
             // merge into (max(m, m'), max3(min(m, m'), s, s')).
-            float mA, sA, mB, sB, mC, sC, mL, mAB, sAB, sG;
-            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mA) : "v"(sv[0]), "v"(sv[1]), "v"(sv[2]));
-            asm("v_med3_f32 %0, %1, %2, %3" : "=v"(sA) : "v"(sv[0]), "v"(sv[1]), "v"(sv[2]));
-            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mB) : "v"(sv[3]), "v"(sv[4]), "v"(sv[5]));
-            asm("v_med3_f32 %0, %1, %2, %3" : "=v"(sB) : "v"(sv[3]), "v"(sv[4]), "v"(sv[5]));
-            asm("v_max_f32 %0, %1, %2" : "=v"(mC) : "v"(sv[6]), "v"(sv[7]));
-            asm("v_min_f32 %0, %1, %2" : "=v"(sC) : "v"(sv[6]), "v"(sv[7]));
-            asm("v_min_f32 %0, %1, %2" : "=v"(mL) : "v"(mA), "v"(mB));
-            asm("v_max_f32 %0, %1, %2" : "=v"(mAB) : "v"(mA), "v"(mB));
-            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(sAB) : "v"(mL), "v"(sA), "v"(sB));
-            asm("v_min_f32 %0, %1, %2" : "=v"(mL) : "v"(mAB), "v"(mC));
-            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(sG) : "v"(mL), "v"(sAB), "v"(sC));
-            // and the second largest of the other groups' maxima
-            float sec;
-            asm("v_max_f32 %0, %1, %2" : "=v"(sec) : "v"(sG), "v"(second[t]));
-            const unsigned int c_mine = (code[t] << 4) + pos + h4;
-            // Both half-waves see both halves' results (one register swap each, no LDS traffic
-            // that would queue behind the accumulator atomics) and combine them identically.
-            const auto bb = __builtin_amdgcn_permlane32_swap(__float_as_uint(best[t]),
-                                                             __float_as_uint(best[t]), false, false);
-            const auto ss = __builtin_amdgcn_permlane32_swap(__float_as_uint(sec), __float_as_uint(sec),
-                                                             false, false);
-            const auto cc = __builtin_amdgcn_permlane32_swap(c_mine, c_mine, false, false);
-            const float b_lo = __uint_as_float(bb[0]), b_hi = __uint_as_float(bb[1]);
-            // second best over both halves: the loser of the two bests or a half's own second
-            float s2, b;
-            asm("v_min_f32 %0, %1, %2" : "=v"(s2) : "v"(b_lo), "v"(b_hi));
-            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(s2) : "v"(s2), "v"(__uint_as_float(ss[0])), "v"(__uint_as_float(ss[1])));
-            asm("v_max_f32 %0, %1, %2" : "=v"(b) : "v"(b_lo), "v"(b_hi));
-            // the lower centroid index wins a tie between the halves
-            const bool take_hi = b_hi > b_lo || (b_hi == b_lo && cc[1] < cc[0]);
-            lab[t] = take_hi ? cc[1] : cc[0];
-            // written so that a NaN anywhere makes the sample uncertain
-            float norm_t = xnorm[t];
-            if (!UPDATE) {
-                const auto qq = __builtin_amdgcn_permlane32_swap(__float_as_uint(own_sq[t]),
-                                                                 __float_as_uint(own_sq[t]), false, false);
-                norm_t = sqrtf(__uint_as_float(qq[0]) + __uint_as_float(qq[1]));
-            }
-            const float thr = fmaf(thr_x, norm_t, thr_0);
-            unsure[t] = !(b - s2 > thr) && (FULL || i0 + t < n);
+            // (temporaries %1 .. %4; one statement: see the conversion above)
+            float tA, tB, tC, tD;
+            asm("v_max3_f32 %1, %5, %6, %7\n\t"     // mA
+                "v_max3_f32 %2, %8, %9, %10\n\t"    // mB
+                "v_med3_f32 %3, %5, %6, %7\n\t"     // sA
+                "v_med3_f32 %4, %8, %9, %10\n\t"    // sB
+                "v_min_f32 %0, %1, %2\n\t"          // min(mA, mB)
+                "v_max_f32 %1, %1, %2\n\t"          // mAB
+                "v_max3_f32 %0, %0, %3, %4\n\t"     // sAB
+                "v_max_f32 %2, %11, %12\n\t"        // mC
+                "v_min_f32 %3, %11, %12\n\t"        // sC
+                "v_min_f32 %1, %1, %2\n\t"          // min(mAB, mC)
+                "v_max3_f32 %0, %1, %0, %3\n\t"     // second largest of the eight
+                "v_max_f32 %0, %0, %13"               // or of the other groups' maxima
+                : "=&v"(sec_c[t]), "=&v"(tA), "=&v"(tB), "=&v"(tC), "=&v"(tD)
+                : "v"(sv[0]), "v"(sv[1]), "v"(sv[2]), "v"(sv[3]), "v"(sv[4]), "v"(sv[5]), "v"(sv[6]), "v"(sv[7]),
+                  "v"(second[t]));
+            cen_c[t] = (code[t] << 4) + pos + h4;
         }
 
-        // Samples the screen cannot certify go to the workgroup's queue with weight zero here
-        // (their label below is provisional and adds nothing); the queue is worked off in
-        // plain fp32 after the last tile, by all waves alike, so that no wave is held up by
-        // the samples it happens to meet.  A column with several such samples (ties between
-        // duplicate centroids, degenerate data), or one that finds the queue full, is instead
-        // redone as a whole in fp32 on the matrix cores, which bounds the cost of a tile at
-        // about three times the usual one however many samples fail the screen.
-        float wl[NC];
-        bool counted[NC];
+        // The half-waves exchange results: one register swap per quantity gives the lower
+        // half-wave both halves' results for column 0 and the upper one those for column 1
+        // (NC = 1: both get column 0), so that each lane finishes ONE sample.  No LDS traffic
+        // that would queue behind the accumulator atomics.
+        const auto bb = __builtin_amdgcn_permlane32_swap(__float_as_uint(best[0]), __float_as_uint(best[NC - 1]),
+                                                         false, false);
+        const auto ss = __builtin_amdgcn_permlane32_swap(__float_as_uint(sec_c[0]), __float_as_uint(sec_c[NC - 1]),
+                                                         false, false);
+        const auto cc = __builtin_amdgcn_permlane32_swap(cen_c[0], cen_c[NC - 1], false, false);
+        const float b_lo = __uint_as_float(bb[0]), b_hi = __uint_as_float(bb[1]);
+        // second best over both halves: the loser of the two bests or a half's own second
+        float s2, b;
+        asm("v_min_f32 %0, %2, %3\n\t"
+            "v_max_f32 %1, %2, %3\n\t"
+            "v_max3_f32 %0, %0, %4, %5"
+            : "=&v"(s2), "=&v"(b)
+            : "v"(b_lo), "v"(b_hi), "v"(__uint_as_float(ss[0])), "v"(__uint_as_float(ss[1])));
+        // the lower centroid index wins a tie between the halves
+        const bool take_hi = b_hi > b_lo || (b_hi == b_lo && cc[1] < cc[0]);
+        uint32_t lab_mine = take_hi ? cc[1] : cc[0];
+        if (!UPDATE) {
+            const auto qq = __builtin_amdgcn_permlane32_swap(__float_as_uint(own_sq[0]),
+                                                             __float_as_uint(own_sq[NC - 1]), false, false);
+            norm_mine = sqrtf(__uint_as_float(qq[0]) + __uint_as_float(qq[1]));
+        }
+        // written so that a NaN anywhere makes the sample uncertain
+        const float thr = fmaf(thr_x, norm_mine, thr_0);
+        const bool unsure_mine = !(b - s2 > thr) && in_range && owner;
+
+        // Samples the screen cannot certify go to the workgroup's queue (their label below is
+        // provisional and they take no part in the sums here); the queue is worked off in plain
+        // fp32 after the last tile, by all waves alike, so that no wave is held up by the samples
+        // it happens to meet.  A column with several such samples (ties between duplicate
+        // centroids, degenerate data), or one that finds the queue full, is instead redone as a
+        // whole in fp32 on the matrix cores, which bounds the cost of a tile at about three times
+        // the usual one however many samples fail the screen.
+        bool queued_mine = false;
+        const unsigned long long todo_all = __ballot(unsure_mine);  // bit 32 t + j: sample j of column t
+        if (__builtin_expect(todo_all != 0ull, 0)) {                // cold: spills belong in here
+            float xr[NK][8][NC];
+            load(xr);
 #pragma unroll
-        for (int t = 0; t < NC; ++t) {
-            wl[t] = wv[t];
-            counted[t] = FULL || i0 + t < n;
-            const unsigned long long todo = __ballot(h == 0 && unsure[t]);  // wave-uniform
-            if (__builtin_expect(todo != 0ull, 0)) {  // cold: spills belong in here
-                const int n_todo = __popcll(todo);
+            for (int t = 0; t < NC; ++t) {
+                const unsigned int todo = (unsigned int)(todo_all >> (32 * t));  // wave-uniform
+                if (todo == 0u) continue;
+                const int n_todo = __popc(todo);
                 n_uncertain += (unsigned int)n_todo;
                 bool redo = n_todo >= SCR_REDO_COLUMN;
                 unsigned int base = 0;
@@ -532,80 +699,91 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                     base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
                     redo = base + (unsigned int)n_todo > (unsigned int)q_cap;
                 }
+                const bool col_mine = NC == 2 ? h == t : true;  // whether the lane's own sample is in column t
                 if (redo) {
                     ColumnRows rows;
 #pragma unroll
                     for (int s = 0; s < NK; ++s)
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = x[s][i][t];
-                    lab[t] = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
-                } else if (((unsigned int)todo >> j) & 1u) {  // both lanes of the sample
-                    const unsigned int slot = base + (unsigned int)__popc((unsigned int)todo & ((1u << j) - 1u));
+                        for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = xr[s][i][t];
+                    const uint32_t r = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
+                    if (col_mine) lab_mine = r;
+                } else if ((todo >> j) & 1u) {  // both lanes of the sample
+                    const unsigned int slot = base + (unsigned int)__popc(todo & ((1u << j) - 1u));
                     uint32_t* entry = queue + slot * QW;
 #pragma unroll
                     for (int s = 0; s < NK; ++s)
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) entry[16 * s + 2 * i + h] = __float_as_uint(x[s][i][t]);
+                        for (int i = 0; i < 8; ++i) entry[16 * s + 2 * i + h] = __float_as_uint(xr[s][i][t]);
                     if (h == 0) {
-                        entry[Q_WEIGHT] = __float_as_uint(wv[t]);
-                        entry[Q_INDEX] = (uint32_t)(i0 + t);
-                        entry[Q_PREV] = pl[t];
+                        const int64_t idx_t = i0 + t;
+                        entry[Q_WEIGHT] = UPDATE ? __float_as_uint(sample_weight[idx_t]) : 0u;
+                        entry[Q_INDEX] = (uint32_t)idx_t;
+                        entry[Q_PREV] = UPDATE ? labels_prev[idx_t] : 0u;
                     }
-                    wl[t] = 0.0f;
-                    counted[t] = false;
+                    if (col_mine) queued_mine = true;
                 }
             }
         }
 
-        if (h == 0) {
-            if constexpr (FULL && NC == 2) {
-                *reinterpret_cast<uint2*>(labels + i0) = make_uint2(lab[0], lab[1]);
-            } else {
-#pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    if (FULL || i0 + t < n) labels[i0 + t] = lab[t];
-            }
-        }
+        if (in_range && owner) labels[my_idx] = lab_mine;
 
         if (UPDATE) {
-            if (h == 0) {
+            const bool counted_mine = in_range && owner && !queued_mine;
+            const bool chg_mine = counted_mine && pl_mine != lab_mine;
+            changed += chg_mine ? 1u : 0u;
+            // which samples the sums have to hear of: all of them when the sums are rebuilt,
+            // those that change cluster otherwise (bit 32 t + j: sample j of column t)
+            const unsigned long long act_all = __ballot(full_mode ? counted_mine : chg_mine);
+            if (act_all != 0ull) {
+                float xr[NK][8][NC];
+                load(xr);
+                // both columns' labels in every lane (the lane adds its features of both samples)
+                uint32_t lab[NC], pl[NC];
+                const auto ll = __builtin_amdgcn_permlane32_swap(lab_mine, lab_mine, false, false);
+                const auto pp = __builtin_amdgcn_permlane32_swap(pl_mine, pl_mine, false, false);
+                lab[0] = ll[0];
+                pl[0] = pp[0];
+                if (NC == 2) {
+                    lab[NC - 1] = ll[1];
+                    pl[NC - 1] = pp[1];
+                }
 #pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    changed += (counted[t] && pl[t] != lab[t]) ? 1u : 0u;
-            }
-            // samples past the end carry w = 0: they add zero
-            double wd[NC];
-            unsigned long long* mine[NC];  // word h of the label's cluster
+                for (int t = 0; t < NC; ++t) {
+                    const unsigned int act_col = (unsigned int)(act_all >> (32 * t));  // wave-uniform
+                    if (act_col == 0u) continue;
+                    const bool act = (act_col >> j) & 1u;
+                    // samples past the end and samples that stay put are not in the mask
+                    const double wd = act ? (double)sample_weight[i0 + t] : 0.0;
+                    unsigned long long* to = acc + lab[t] * (uint32_t)acc_stride + h;    // word h of the new cluster
+                    unsigned long long* from = acc + pl[t] * (uint32_t)acc_stride + h;   // and of the old one
 #pragma unroll
-            for (int t = 0; t < NC; ++t) {
-                wd[t] = (double)wl[t];
-                mine[t] = acc + lab[t] * (uint32_t)acc_stride + h;
-            }
+                    for (int s = 0; s < NK; ++s)
 #pragma unroll
-            for (int s = 0; s < NK; ++s)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int p0 = 16 * s + 2 * i;  // the pair's even feature
-                    if (p0 < d) {                   // wave-uniform
-                        // (odd d, last pair: the upper half-wave adds to the spare word)
-#pragma unroll
-                        for (int t = 0; t < NC; ++t) {
-                            const double xd = (double)x[s][i][t];
-                            // x * w is exact in fp64; one rounding, to a multiple of 2^-q
-                            const double v = fma(xd, wd[t], magic[s][i]);
-                            atomicAdd(mine[t] + p0, to_fixed_q(v, magic[s][i]));
+                        for (int i = 0; i < 8; ++i) {
+                            const int p0 = 16 * s + 2 * i;  // the pair's even feature
+                            if (p0 < d) {                   // wave-uniform
+                                // (odd d, last pair: the upper half-wave adds to the spare word)
+                                const double magic = fix_magic(q_lds[p0 + h]);
+                                // x * w is exact in fp64; one rounding, to a multiple of 2^-q
+                                const double v = fma((double)xr[s][i][t], wd, magic);
+                                const unsigned long long term = to_fixed_q(v, magic);
+                                if (act) {
+                                    atomicAdd(to + p0, term);
+                                    if (!full_mode) atomicSub(from + p0, term);
+                                }
+                            }
                         }
+                    if (h == 0 && act) {
+                        const double magic_w = fix_magic(q_lds[d]);
+                        const unsigned long long term = to_fixed_q(wd + magic_w, magic_w);
+                        atomicAdd(to + d_even, term);
+                        if (!full_mode) atomicSub(from + d_even, term);
                     }
                 }
-            if (h == 0) {
-#pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    atomicAdd(mine[t] + d_even, to_fixed_q(wd[t] + magic_w, magic_w));
             }
         }
     };
-    using Cols2 = std::integral_constant<int, MC>;
-    using Cols1 = std::integral_constant<int, 1>;
 
     const int wt_step = (int)gridDim.x * WAVES;
     const int wt_first = (int)blockIdx.x * WAVES + wave;
@@ -617,40 +795,35 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     const bool halves = n_left > 0 && 4 * (int64_t)n_left <= 3 * (int64_t)wt_step;
     const int n_main = halves ? n_rounds * wt_step : n_fast;
 
-    // Rows of the lane: feature 2 p + h for the pairs p = 8 s + i.  Every load is a uniform
-    // row address plus a 32-bit byte offset of the lane (n < 2^29), and unconditional, so
-    // that the compiler counts the loads and waits for the older tile only.
+    // Rows of the lane: feature 2 p + h for the pairs p = 8 s + i, row d - 1 where that feature
+    // does not exist (the centroid operand is zero there, so any finite value will do).  A load
+    // is the scalar address of the tile in row 0 plus a 32-bit byte offset of the lane that does
+    // not change from tile to tile (d * n * 4 < 2^32 is a condition of this path): no vector
+    // arithmetic and no branch per tile.
     const char* const xbytes = reinterpret_cast<const char*>(X_t);
-    // A pair that is not entirely below d reads row d - 1 in both half-waves.
-    uint32_t lane_off[NK][8];
+    uint32_t row_off[NK][8];
 #pragma unroll
     for (int s = 0; s < NK; ++s)
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            lane_off[s][i] = (uint32_t)(MC * j) * 4u + ((16 * s + 2 * i + 1 < d) ? (uint32_t)h * (uint32_t)n * 4u : 0u);
-    // The row addresses are rebuilt with scalar additions for every tile (the asm hides the
-    // base from loop-invariant hoisting: eight or sixteen precomputed 64-bit row pointers
-    // would not fit the scalar registers and would be spilled and reloaded around every load).
-    const size_t pair_stride = (size_t)n * 8u;  // two rows
-    const char* const tail_row = xbytes + (size_t)(d - 1) * (size_t)n * 4u;
-    auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) {
-        const uint32_t tile_off = (uint32_t)wt * (uint32_t)(TILE * 4);
-        size_t hidden_zero = 0;
-        asm volatile("" : "+s"(hidden_zero));
-        const char* row = xbytes + hidden_zero;
-        int d_now = d;  // compared afresh with scalar instructions: no lane masks kept per row
-        asm volatile("" : "+s"(d_now));
+        for (int i = 0; i < 8; ++i) {
+            const int f = 16 * s + 2 * i + h;
+            row_off[s][i] = (uint32_t)(f < d ? f : d - 1) * (uint32_t)n * 4u + (uint32_t)(MC * j) * 4u;
+        }
+    auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
+        const char* const tile = xbytes + (size_t)wt * (size_t)(TILE * 4);  // wave-uniform
 #pragma unroll
         for (int s = 0; s < NK; ++s)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int p0 = 16 * s + 2 * i;
-                const char* src = p0 + 1 < d_now ? row : tail_row;
-                const float2 q = *reinterpret_cast<const float2*>(src + (tile_off + lane_off[s][i]));
+                const float2 q = *reinterpret_cast<const float2*>(tile + row_off[s][i]);
                 dst[s][i][0] = q.x;
                 dst[s][i][1] = q.y;
-                row += pair_stride;
             }
+        if (HK) {
+            // the spare slot carries the constant whose scaled value is SCR_HK_X1
+#pragma unroll
+            for (int t = 0; t < MC; ++t) dst[NK - 1][7][t] = h ? hk_x : dst[NK - 1][7][t];
+        }
     };
 
     // The workgroup's full tiles (tile WAVES * blockIdx.x + q % WAVES of round q / WAVES) are
@@ -658,39 +831,53 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
     // the same pace, and with fixed shares the fastest would wait a fifth of the time for the
     // slowest at the end.  The next ticket is drawn before the current tile is worked on.
     if (n_main > 0) {
-        auto draw = [&]() {
+        auto draw = [&]() __attribute__((always_inline)) {
             unsigned int ticket = 0;
             if (lane == 0) ticket = atomicAdd(&tile_ticket, 1u);
             return ticket;  // valid in lane 0
         };
-        unsigned int ticket = draw();
-        for (;;) {
-            const int q = __builtin_amdgcn_readfirstlane((int)ticket);
-            const int wt = (int)blockIdx.x * WAVES + q % WAVES + (q / WAVES) * wt_step;
-            if (wt >= n_main) break;  // every wave gets here: the counter only grows
-            ticket = draw();
-            const int64_t i0 = (int64_t)wt * TILE + MC * j;
-            float x[NK][8][MC];
-            load_rows(wt, x);
-            float wv[MC] = {0.f, 0.f};
-            uint32_t pl[MC] = {0u, 0u};
-            float xnorm[MC] = {0.f, 0.f};  // labels only: taken from the tile itself
-            if (UPDATE) {
-                const float2 n2 = *reinterpret_cast<const float2*>(norms + i0);
-                xnorm[0] = n2.x;
-                xnorm[1] = n2.y;
-                const float2 w2 = *reinterpret_cast<const float2*>(sample_weight + i0);
-                wv[0] = w2.x;
-                wv[1] = w2.y;
-                const uint2 p2 = *reinterpret_cast<const uint2*>(labels_prev + i0);
-                pl[0] = p2.x;
-                pl[1] = p2.y;
+        auto tile_of = [&](const unsigned int ticket_) __attribute__((always_inline)) {
+            const int q = __builtin_amdgcn_readfirstlane((int)ticket_);
+            return (int)blockIdx.x * WAVES + q % WAVES + (q / WAVES) * wt_step;
+        };
+        // The rows, norm and previous label of a tile are requested while the tile before it
+        // is scored (they are consumed at the very start of a tile, and nothing else of a tile
+        // can start before them): a wave's own loads then cost it no waiting.
+        float x[NK][8][MC];
+        float norm_next = 0.0f;
+        uint32_t pl_next = 0u;
+        auto request = [&](const int wt_) __attribute__((always_inline)) {
+            if (wt_ < n_main) {  // wave-uniform
+                load_rows(wt_, x);
+                if (UPDATE) {
+                    const int64_t idx = (int64_t)wt_ * TILE + MC * j + h;
+                    norm_next = norms[idx];
+                    pl_next = labels_prev[idx];
+                }
             }
-            process(Cols2{}, std::true_type{}, x, wv, pl, xnorm, i0);
+        };
+        // (two K steps: the registers do not allow it, the tile's data are requested when it starts)
+        constexpr bool AHEAD = NK == 1;
+        int wt = tile_of(draw());
+        if (AHEAD) request(wt);
+        while (wt < n_main) {  // every wave gets out: the counter only grows
+            const int wt_next = tile_of(draw());
+            const int64_t i0 = (int64_t)wt * TILE + MC * j;
+            const int wt_now = wt;
+            if (!AHEAD) request(wt_now);
+            process(
+                Cols2{}, std::true_type{},
+                [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_rows(wt_now, xr); },
+                [&]() __attribute__((always_inline)) {
+                    if (AHEAD) request(wt_next);
+                },
+                x, norm_next, pl_next, i0);
+            wt = wt_next;
         }
     }
     // scalar loads of the lane's rows (row d - 1 where the feature does not exist)
-    auto load_scalar = [&](auto nc_tag, const int64_t i0, float(&dst)[NK][8][decltype(nc_tag)::value]) {
+    auto load_scalar = [&](auto nc_tag, const int64_t i0, float(&dst)[NK][8][decltype(nc_tag)::value])
+                           __attribute__((always_inline)) {
         constexpr int NC = decltype(nc_tag)::value;
 #pragma unroll
         for (int s = 0; s < NK; ++s)
@@ -698,8 +885,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             for (int i = 0; i < 8; ++i) {
                 const int f = 16 * s + 2 * i + h;
                 const float* row = X_t + (size_t)(f < d ? f : d - 1) * n;
+                const float absent = (HK && f == SPARE) ? hk_x : 0.0f;  // the spare slot, or no feature at all
 #pragma unroll
-                for (int t = 0; t < NC; ++t) dst[s][i][t] = i0 + t < n ? row[i0 + t] : 0.0f;
+                for (int t = 0; t < NC; ++t) dst[s][i][t] = f < d ? (i0 + t < n ? row[i0 + t] : 0.0f) : absent;
             }
     };
     if (halves) {
@@ -708,15 +896,12 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
             const int64_t i0 = (int64_t)n_main * TILE + 32 * q + j;
             float x[NK][8][1];
             load_scalar(Cols1{}, i0, x);
-            float wv[1] = {0.f};
-            uint32_t pl[1] = {0u};
-            float xnorm[1] = {0.f};
-            if (UPDATE) {
-                xnorm[0] = norms[i0];
-                wv[0] = sample_weight[i0];
-                pl[0] = labels_prev[i0];
-            }
-            process(Cols1{}, std::true_type{}, x, wv, pl, xnorm, i0);
+            float norm_now = UPDATE ? norms[i0] : 0.0f;
+            uint32_t pl_now = UPDATE ? labels_prev[i0] : 0u;
+            process(
+                Cols1{}, std::true_type{},
+                [&](float(&xr)[NK][8][1]) __attribute__((always_inline)) { load_scalar(Cols1{}, i0, xr); }, [] {}, x,
+                norm_now, pl_now, i0);
         }
     }
     // The rest: a partial last tile, or every tile when vector accesses are not legal
@@ -724,21 +909,13 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
         const int64_t i0 = (int64_t)wt * TILE + MC * j;
         float x[NK][8][MC];
         load_scalar(Cols2{}, i0, x);
-        float wv[MC];
-        uint32_t pl[MC];
-        float xnorm[MC];
-#pragma unroll
-        for (int t = 0; t < MC; ++t) {
-            wv[t] = 0.f;
-            pl[t] = 0u;
-            xnorm[t] = 0.0f;
-            if (UPDATE && i0 + t < n) {
-                xnorm[t] = norms[i0 + t];
-                wv[t] = sample_weight[i0 + t];
-                pl[t] = labels_prev[i0 + t];
-            }
-        }
-        process(Cols2{}, std::false_type{}, x, wv, pl, xnorm, i0);
+        const bool mine_exists = i0 + h < n;
+        float norm_now = (UPDATE && mine_exists) ? norms[i0 + h] : 0.0f;
+        uint32_t pl_now = (UPDATE && mine_exists) ? labels_prev[i0 + h] : 0u;
+        process(
+            Cols2{}, std::false_type{},
+            [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_scalar(Cols2{}, i0, xr); }, [] {}, x,
+            norm_now, pl_now, i0);
     }
 
     // The queue: one wave per entry, lane l on the centroids l, l + 64, ... (fused multiply-adds
@@ -815,11 +992,17 @@ __global__ __launch_bounds__(64 * scr_waves(NK)) void lloyd_screen_kernel(
                 if (UPDATE) changed += entry[Q_PREV] != (uint32_t)bc ? 1u : 0u;
             }
             if (UPDATE) {
-                // lane f adds feature f, lane d the weight: the same fixed-point terms as above
+                // lane f adds feature f, lane d the weight: the same fixed-point terms as above;
+                // when the sums are only corrected, a sample that stays in its cluster adds
+                // nothing and one that moves is taken off the old cluster
+                const uint32_t prev = entry[Q_PREV];
                 const double wq = (double)__uint_as_float(entry[Q_WEIGHT]);
-                if (lane <= d) {
+                if (lane <= d && (full_mode || prev != (uint32_t)bc)) {
                     const double term = lane < d ? fma((double)xe[lane], wq, magic_lane) : wq + magic_lane;
-                    atomicAdd(acc + bc * acc_stride + (lane < d ? lane : d_even), to_fixed_q(term, magic_lane));
+                    const unsigned long long fixed = to_fixed_q(term, magic_lane);
+                    const int word = lane < d ? lane : d_even;
+                    atomicAdd(acc + bc * acc_stride + word, fixed);
+                    if (!full_mode) atomicSub(acc + prev * (uint32_t)acc_stride + word, fixed);
                 }
             }
         }
@@ -879,7 +1062,15 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
     float* hneg = reinterpret_cast<float*>(afl + n_cb * NK * 64);
     __shared__ unsigned int hmax_bits;
     const float xmax = __uint_as_float(*xmax_bits);
-    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, 14 - ilogbf(xmax)) : 1.0f;
+    // d <= 32: the arithmetic of lloyd_screen_kernel (its scale; -0.5||c||^2 in the spare feature
+    // slot d when there is one); wider: that of the wide path's label kernel (data scaled into
+    // [2^14, 2^15), -0.5||c||^2 as the accumulators' start)
+    const bool narrow = d <= 32;
+    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>())
+                         ? ldexpf(1.0f, (narrow ? SCR_SCALE_EXP - 1 : 14) - ilogbf(xmax))
+                         : 1.0f;
+    const bool hk = narrow && d % 16 != 0;
+    const int spare = 16 * ((d + 15) / 16) - 1;  // the feature slot that then carries -0.5||c||^2
     if (threadIdx.x == 0) hmax_bits = 0;
     __syncthreads();
     for (int idx = threadIdx.x; idx < n_cb * NK * 64; idx += 64) {
@@ -889,10 +1080,25 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int f = 16 * s + 2 * i + (l >> 5);
-            const float v = (c < k && f < d) ? centroids_t[(size_t)f * k + c] * xs : 0.0f;
+            float v = (c < k && f < d) ? centroids_t[(size_t)f * k + c] * xs : 0.0f;
+            if (hk && f == spare) {
+                v = -kmx_inf<float>();
+                if (c < k) {
+                    float sq = 0.0f;
+                    for (int g = 0; g < d; ++g) {
+                        const float cv = centroids_t[(size_t)g * k + c] * xs;
+                        sq += cv * cv;
+                    }
+                    v = -(sq / 2.0f) * (1.0f / SCR_HK_X1);
+                }
+            }
             const _Float16 hb = (_Float16)v;
             hi[i] = hb;
             lo[i] = (_Float16)(v - (float)hb);
+            if (hk && f == spare && !(c < k)) {
+                hi[i] = (_Float16)0.0f;
+                lo[i] = hb;
+            }
         }
         afh[idx] = hi;
         afl[idx] = lo;
@@ -928,7 +1134,9 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
             const int f = 16 * s + 2 * i + h;
             const float x0 = (f < d && i0 < n) ? X_t[(size_t)f * n + i0] : 0.0f;
             const float x1 = (f + 2 < d && i0 < n) ? X_t[(size_t)(f + 2) * n + i0] : 0.0f;
-            const v2f p = {x0 * xs, x1 * xs};
+            v2f p = {x0 * xs, x1 * xs};
+            if (hk && f == spare) p[0] = SCR_HK_X1;
+            if (hk && f + 2 == spare) p[1] = SCR_HK_X1;
             const v2h hh = __builtin_convertvector(p, v2h);
             const v2f r = p - __builtin_convertvector(hh, v2f);
             const v2h ll = __builtin_convertvector(r, v2h);
@@ -936,13 +1144,14 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
             xh[s][i + 1] = hh[1];
             xl[s][i] = ll[0];
             xl[s][i + 1] = ll[1];
-            ss = fmaf(p[0], p[0], ss);
-            ss = fmaf(p[1], p[1], ss);
+            if (f < d) ss = fmaf(p[0], p[0], ss);
+            if (f + 2 < d) ss = fmaf(p[1], p[1], ss);
         }
     const float nrm = ss + __shfl_xor(ss, 32, 64);
     if (h == 0 && i0 < n)
         bounds[i0] = fmaf((SCR_ERR_SPLIT + round_term) * cmax + abs_term, __builtin_amdgcn_sqrtf(nrm),
-                          round_term * hmax + abs_term * cmax);
+                          round_term * hmax + abs_term * cmax +
+                              (hk ? SCR_ERR_HNEG * hmax + SCR_ERR_ABS * SCR_HK_X1 : 0.0f));
     if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = xs;
     for (int cb = 0; cb < n_cb; ++cb) {
         const float4* hp = reinterpret_cast<const float4*>(hneg + cb * 32 + h * 16);
@@ -950,10 +1159,10 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 v4 = hp[q];
-            a[4 * q] = v4.x;
-            a[4 * q + 1] = v4.y;
-            a[4 * q + 2] = v4.z;
-            a[4 * q + 3] = v4.w;
+            a[4 * q] = hk ? 0.0f : v4.x;
+            a[4 * q + 1] = hk ? 0.0f : v4.y;
+            a[4 * q + 2] = hk ? 0.0f : v4.z;
+            a[4 * q + 3] = hk ? 0.0f : v4.w;
         }
 #pragma unroll
         for (int s = 0; s < NK; ++s) {
@@ -1009,25 +1218,32 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
     if (grid > cap) grid = cap;
     if (grid < 1) grid = 1;
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
-    const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) && aligned16(w) &&
+    // (the fast path addresses a lane's rows with 32-bit byte offsets from the tile's address in row 0)
+    const int vec_ok = ((uint64_t)d * (uint64_t)n * 4u < ((uint64_t)1 << 32)) && (n % 4 == 0) && aligned16(X_t) &&
+                       aligned16(labels) && aligned16(w) &&
                        aligned16(labels_prev);
     const size_t lds = screen_lds(d, k, nk, UPDATE).total;
-    if (lds > 64 * 1024) {
-        const void* kernel = nk == 1 ? reinterpret_cast<const void*>(&lloyd_screen_kernel<1, UPDATE>)
-                                     : reinterpret_cast<const void*>(&lloyd_screen_kernel<2, UPDATE>);
-        const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int32_t)e;
+    // -0.5||c||^2 in a spare feature slot of the last K step whenever there is one
+    const bool hk = d % 16 != 0;
+#define KMX_SCR_LAUNCH(NK_, HK_)                                                                            \
+    do {                                                                                                    \
+        if (lds > 64 * 1024) {                                                                              \
+            const hipError_t e = hipFuncSetAttribute(                                                       \
+                reinterpret_cast<const void*>(&lloyd_screen_kernel<NK_, UPDATE, HK_>),                      \
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                      \
+            if (e != hipSuccess) return (int32_t)e;                                                         \
+        }                                                                                                   \
+        hipLaunchKernelGGL((lloyd_screen_kernel<NK_, UPDATE, HK_>), dim3((unsigned)grid),                   \
+                           dim3(64 * scr_waves(NK_)), lds, stream, (const float*)X_t, (const float*)w,      \
+                           (const float*)centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,     \
+                           uncertain_count, norms, n, d, k, vec_ok);                                        \
+    } while (0)
+    if (nk == 1) {
+        if (hk) KMX_SCR_LAUNCH(1, true); else KMX_SCR_LAUNCH(1, false);
+    } else {
+        if (hk) KMX_SCR_LAUNCH(2, true); else KMX_SCR_LAUNCH(2, false);
     }
-    if (nk == 1)
-        hipLaunchKernelGGL((lloyd_screen_kernel<1, UPDATE>), dim3((unsigned)grid), dim3(64 * scr_waves(1)),
-                           lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
-                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, norms, n, d,
-                           k, vec_ok);
-    else
-        hipLaunchKernelGGL((lloyd_screen_kernel<2, UPDATE>), dim3((unsigned)grid), dim3(64 * scr_waves(2)),
-                           lds, stream, (const float*)X_t, (const float*)w, (const float*)centroids_t,
-                           labels_prev, labels, status, absmax, q_exp, gsum, uncertain_count, norms, n, d,
-                           k, vec_ok);
+#undef KMX_SCR_LAUNCH
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

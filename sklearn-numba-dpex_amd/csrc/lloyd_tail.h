@@ -17,6 +17,12 @@ struct LloydTail {
     kmx_lloyd_status* status;
     int d, k, dpad;
     uint32_t* clear_word = nullptr;  // a counter to copy to the next word and zero, or null
+    // Screened fused step only: word clear_word[2] tells the next step whether it may correct the
+    // fixed-point sums for the samples that change cluster instead of rebuilding them; the sums
+    // then stay in `gsum` instead of being cleared.  Chosen when the iteration just finished
+    // changed at most n_samples / delta_divisor labels (0: always rebuild).
+    int64_t n_samples = 0;
+    int delta_divisor = 0;
 };
 
 // Empty-cluster list (ascending) and heaviest cluster; one workgroup of 256 threads.
@@ -179,10 +185,14 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
     const T* sizes_s = vals + dk;
     T* __restrict__ out_t = a.sums_t;
     const T* __restrict__ old_t = a.old_centroids_t;
+    // (the label changes of the iteration at hand; every thread reads the same word before
+    // thread 0 resets it at the end of the kernel)
+    const bool keep_sums = FROM_GSUM && a.clear_word != nullptr && a.delta_divisor > 0 &&
+                           (int64_t)a.status->n_changed * a.delta_divisor <= a.n_samples;
     for (int jx = threadIdx.x; jx < items; jx += 256) {
         if constexpr (FROM_GSUM) {
             const long long iv = (long long)gsum[jx];
-            gsum[jx] = 0ull;
+            if (!keep_sums) gsum[jx] = 0ull;
             const int f = jx / k;
             const T val = (T)ldexp((double)iv, -q_exp[f]);
             vals[jx] = val;
@@ -202,9 +212,18 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
         a.status->reserved[0] = heaviest;
     }
     if (n_empty > 0) {
-        if (threadIdx.x == 0) a.status->state = KMX_NEED_RELOCATION;
+        // the host relocates and finishes the iteration; the next step rebuilds the sums
+        if constexpr (FROM_GSUM) {
+            if (keep_sums)
+                for (int jx = threadIdx.x; jx < items; jx += 256) gsum[jx] = 0ull;
+        }
+        if (threadIdx.x == 0) {
+            a.status->state = KMX_NEED_RELOCATION;
+            if (a.clear_word != nullptr) a.clear_word[2] = 0u;
+        }
         return;
     }
+    if (a.clear_word != nullptr && threadIdx.x == 0) a.clear_word[2] = keep_sums ? 1u : 0u;
     double shift = 0.0;
 #pragma unroll 4
     for (int jx = threadIdx.x; jx < dk; jx += 256) {
