@@ -36,7 +36,7 @@ except ImportError:  # stock scikit-learn
             self.estimator = estimator
 
 
-from ..common._buffers import require_cuda
+from ..common._buffers import require_cuda, upload
 from .drivers import (
     get_euclidean_distances,
     get_labels_inertia,
@@ -278,8 +278,8 @@ class KMeansEngine(_EngineBase):
             )
             n_features = X_np.shape[1]
             # upload, then transpose on the device: (d, n) contiguous
-            X_t = torch.as_tensor(np.ascontiguousarray(X_np.T) if X_np.flags.f_contiguous
-                                  else X_np, device=self.device)
+            # (through pinned staging buffers when the array is large)
+            X_t = upload(np.ascontiguousarray(X_np.T) if X_np.flags.f_contiguous else X_np, self.device)
             X_t = X_t if X_np.flags.f_contiguous else X_t.T.contiguous()
 
         if reset:
@@ -344,7 +344,7 @@ class KMeansEngine(_EngineBase):
                 estimator=self.estimator,
                 input_name="sample_weight",
             )
-            sample_weight = torch.as_tensor(sample_weight, device=X.device)
+            sample_weight = upload(sample_weight, X.device)
         if sample_weight.dim() != 1:
             raise ValueError("Sample weights must be 1D array or scalar")
         if tuple(sample_weight.shape) != (n_samples,):

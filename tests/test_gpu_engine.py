@@ -332,3 +332,34 @@ def test_dlpack_inputs_give_the_same_fit(cuda, dtype):
     else:
         np.testing.assert_allclose(a.cluster_centers_, b.cluster_centers_, rtol=1e-12, atol=1e-13)
     assert a.n_iter_ == b.n_iter_
+
+
+def test_numpy_inputs_are_uploaded_through_pinned_staging(cuda):
+    """Large numpy inputs travel through two pinned staging buffers (several chunks, a ragged
+    last one); the device copy is bit-identical to the host array, for every dtype and for
+    sizes below the staging threshold (plain copy)."""
+    import torch
+
+    from sklearn_numba_dpex_amd.common import _buffers
+
+    rng = np.random.default_rng(5)
+    for shape, dtype in (((3_000_017, 7), np.float32), ((1_100_003, 9), np.float64), ((4_000_001,), np.float32),
+                         ((1000, 3), np.float32), ((9_000_001,), np.int32)):
+        a = rng.standard_normal(shape).astype(dtype) if np.issubdtype(dtype, np.floating) \
+            else rng.integers(-5, 5, shape).astype(dtype)
+        t = _buffers.upload(a, cuda)
+        assert t.device.type == "cuda" and tuple(t.shape) == shape
+        np.testing.assert_array_equal(t.cpu().numpy(), a)
+    assert _buffers._stage is not None and _buffers._stage[0][0].is_pinned()
+    # and the engine takes that route: a fit from numpy equals a fit from a device tensor
+    X = rng.standard_normal((400_000, 6)).astype(np.float32) + rng.integers(0, 4, (400_000, 1)).astype(np.float32) * 5
+    w = rng.uniform(0.5, 1.5, 400_000).astype(np.float32)
+    init = X[:4].copy()
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    a = KMeans(n_clusters=4, init=init, n_init=1, max_iter=5, tol=0).fit(X, sample_weight=w)
+    b = KMeans(n_clusters=4, init=init, n_init=1, max_iter=5, tol=0).fit(torch.as_tensor(X, device=cuda),
+                                                                       sample_weight=torch.as_tensor(w, device=cuda))
+    # (four clusters: the vector-ALU step with floating-point atomics, reproducible to rounding only)
+    # (one blob sits at the origin: its centroid's coordinates are noise around zero, hence the absolute term)
+    np.testing.assert_allclose(_np(a.cluster_centers_), _np(b.cluster_centers_), rtol=1e-5, atol=1e-5)
