@@ -391,7 +391,9 @@ def gpu_components(cfg):
     put("euclidean_distances", t, m * (s * d + s * k),
         f"kmx_euclidean_distances on {m} samples (output {m}x{k}, allocation included)")
     t = timed(lambda: topk_idx(per_sample, 16))
-    put("topk_idx_16", t, 4 * n * s, "radix select of the 16 largest of n values: 4 passes of 8 bits over fp32 keys")
+    put("topk_idx_16", t, 2 * n * s,
+        "radix select of the 16 largest of n values: two reads of the values (first digit, then winners + "
+        "candidates), the remaining digits on the few candidates; six launches whose ends wait on each other")
     t = timed(lambda: sum_reduction(X_t, axis=1))
     put("sum_rows_d_by_n", t, n * d * s, "kmx_sum_rows over X_t (d, n): the feature sums of the centering")
     from sklearn_numba_dpex_amd.common.matmul import matmul

@@ -370,12 +370,30 @@ int32_t kmx_fill_zero(void* data, int64_t n_bytes, void* stream);
 int32_t kmx_centroid_shifts(const void* a_t, const void* b_t, void* out, int32_t d, int32_t k,
                             int32_t dtype, void* stream);
 
+/* Workspace of the top-k entry points for `rows` rows of `n` values: per row a histogram, the
+ * k winners and a side buffer for a quarter of the row.  0 for arguments the entry points
+ * refuse.  kmx_topk_workspace_bytes is the one-row size that serves either dtype. */
+size_t kmx_topk_rows_workspace_bytes(int64_t rows, int64_t n, int32_t k, int32_t dtype);
 size_t kmx_topk_workspace_bytes(int64_t n, int32_t k);
 
-/* Indices of the k largest values of a 1-D array by radix select (8-bit digits, most
- * significant first, on the order-preserving unsigned image of the floats), ordered by
- * descending value then ascending index.  Replaces topk_idx for one row
- * (common/topk.py:194-270, 273-527, 540-1123, 1250-1365). */
+/* out_indices (rows, k) = per row of the C-contiguous matrix `values` (rows, n), the indices
+ * of its k largest values by radix select (digits of 11 or 10 bits, most significant first, on
+ * the order-preserving unsigned image of the floats; -0.0 counts as +0.0, NaNs of positive
+ * sign rank above +inf), ordered by descending value then ascending index; of equal values at
+ * the threshold the lowest indices are taken.  All rows advance in one chain of launches.  The
+ * final ordering compares every pair of winners, k^2 comparisons per row.  Replaces topk_idx
+ * (common/topk.py:194-270, 273-527, 540-1123, 1250-1365), whose output order is undefined. */
+int32_t kmx_topk_idx_rows(const void* values, int64_t* out_indices, int64_t rows, int64_t n,
+                          int32_t k, void* workspace, size_t workspace_bytes, int32_t dtype,
+                          void* stream);
+
+/* out_values (rows, k) = the k largest values of each row, descending (the values at the
+ * indices kmx_topk_idx_rows returns, bit for bit).  Replaces topk (common/topk.py:112-191,
+ * 1127-1247). */
+int32_t kmx_topk_values(const void* values, void* out_values, int64_t rows, int64_t n, int32_t k,
+                        void* workspace, size_t workspace_bytes, int32_t dtype, void* stream);
+
+/* kmx_topk_idx_rows for one row: topk_idx on a 1-D array (common/topk.py:229-235). */
 int32_t kmx_topk_idx(const void* values, int64_t* out_indices, int64_t n, int32_t k,
                      void* workspace, size_t workspace_bytes, int32_t dtype, void* stream);
 

@@ -140,7 +140,10 @@ SIGNATURES = {
     "kmx_fill_zero": (_I32, [_P, _I64, _P]),
     "kmx_centroid_shifts": (_I32, [_P, _P, _P, _I32, _I32, _I32, _P]),
     "kmx_topk_workspace_bytes": (_SZ, [_I64, _I32]),
+    "kmx_topk_rows_workspace_bytes": (_SZ, [_I64, _I64, _I32, _I32]),
     "kmx_topk_idx": (_I32, [_P, _P, _I64, _I32, _P, _SZ, _I32, _P]),
+    "kmx_topk_idx_rows": (_I32, [_P, _P, _I64, _I64, _I32, _P, _SZ, _I32, _P]),
+    "kmx_topk_values": (_I32, [_P, _P, _I64, _I64, _I32, _P, _SZ, _I32, _P]),
     "kmx_is_same_clustering": (_I32, [_P, _P, _P, _P, _I64, _I32, _P]),
     "kmx_count_distinct_clusters": (_I32, [_P, _P, _P, _I64, _I32, _P]),
     "kmx_matmul": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _P]),

@@ -1,39 +1,111 @@
-// Radix-select top-k of a 1-D float array on gfx950 (used to relocate empty clusters onto
-// the samples farthest from their centroid).
+// Radix-select top-k of the rows of a float matrix on gfx950 (a 1-D array is one row; KMeans
+// uses it to relocate empty clusters onto the samples farthest from their centroid).
 //
-// Floats are mapped to unsigned keys whose integer order is the float order.  The key of the
-// k-th largest value is fixed 8 bits at a time, most significant digit first: each pass
-// histograms one digit of the keys that match the prefix found so far (LDS histogram per
-// workgroup, flushed with 64-bit atomics), then a one-workgroup kernel walks the 256 buckets
-// from the top.  4 passes for fp32, 8 for fp64; nothing returns to the host in between.
-// Selection afterwards: every key above the threshold, plus the needed number of keys equal
-// to it, lowest indices first.  The k winners are finally ordered by descending value, then
-// ascending index, so the result is deterministic.
+// Floats are mapped to unsigned keys whose integer order is the float order (-0.0 counts as
+// +0.0).  The key of the k-th largest value of a row is fixed digit by digit, most significant
+// first; digits are 11 or 10 bits wide (3 digits for fp32, 6 for fp64).  All rows advance
+// together: the row is the second grid dimension of every kernel.
+//
+//   pass 0   reads the row once (128-bit loads), histogram of the first digit in LDS, flushed
+//            to the row's global histogram with 64-bit atomics.
+//   pass 1   reads the row a second time: keys whose first digit is above the selected one are
+//            winners and go straight to the result slots; keys that share it are the
+//            candidates: each workgroup appends them to its own segment of a side buffer
+//            (an LDS counter, no global atomics) and histograms their second digit.
+//   pass 2.. walk the candidates only (typically a few thousand keys); when a segment of the
+//            side buffer overflowed (the buffer holds a quarter of the row), they walk the
+//            row itself instead.
+//   gather   candidates above the threshold key are winners; of the keys equal to it, the
+//            lowest indices are taken.
+//   order    the k winners are ranked by descending value, then ascending index, so the result
+//            is deterministic.
+//
+// The workgroup that finishes a pass last (a ticket counter per row) walks the histogram from
+// the top and fixes the digit, so a pass is one launch and nothing returns to the host.  What
+// workgroups exchange inside a launch (histogram, ticket, overflow flag, lowest tie) moves
+// through device-scope atomics only, which are performed at the memory side: waiting for them
+// to complete orders them, and no cache write-back or invalidation is needed (a full fence
+// costs about 60 us per launch here, the L2 of every chiplet being flushed by every workgroup).
 #include "kmx_common.h"
 
 namespace {
 
+constexpr int TOPK_WG = 1024;  // few, large workgroups: what they exchange goes through same-address atomics,
+                               // which the memory side performs one after the other (10-20 ns each)
+constexpr int TOPK_MAX_BUCKETS = 2048;
+constexpr unsigned int TOPK_TIE_LIST = 1024;  // indices of keys equal to the threshold kept aside
+constexpr int TOPK_WIDE = 11;  // bits of the first digits; the last ones may take 10
+
 struct TopkState {
     unsigned long long prefix;      // digits fixed so far (threshold key after the last pass)
     long long k_rem;                // how many keys equal to the threshold belong to the top k
-    unsigned long long n_greater;   // slot counter of the gather
+    unsigned long long n_out;       // winners written so far
     unsigned long long tie_min;     // lowest index holding the threshold key
-    unsigned long long n_ties_taken;
-    unsigned long long pad[3];
+    unsigned int ticket;            // workgroups that finished the running pass
+    unsigned int overflow;          // set by a workgroup whose segment of the side buffer was too small
+    unsigned int cand_ok;           // 1: the side buffer holds every candidate
+    unsigned int n_ties;            // indices appended to the tie list (may exceed its capacity)
+    unsigned int pad[4];
 };
+
+constexpr int TOPK_MAX_SEGMENTS = 256;  // workgroups per row of the passes that read the row
 
 struct TopkLayout {
-    size_t off_state, off_hist, off_keys, off_idx, total;
+    size_t off_state, off_hist, off_counts, off_keys, off_idx, off_cand_keys, off_cand_idx, row_bytes;
+    int64_t n_seg, seg_cap;  // segments of the side buffer (one per workgroup of pass 1) and their capacity
 };
 
-TopkLayout topk_layout(int32_t k) {
+TopkLayout topk_layout(int64_t rows, int64_t n, int32_t k, int32_t dtype) {
     TopkLayout L;
+    const int64_t vec = dtype == KMX_F64 ? 2 : 4;
+    // >= 4 loads of 128 bits per lane, and about TOPK_MAX_SEGMENTS workgroups over all rows
+    L.n_seg = kmx_cdiv(kmx_cdiv(n + vec, vec), TOPK_WG * 4);
+    const int64_t share = kmx_cdiv(TOPK_MAX_SEGMENTS, rows);
+    if (L.n_seg > share) L.n_seg = share;
+    if (L.n_seg < 1) L.n_seg = 1;
+    L.seg_cap = kmx_cdiv(kmx_cdiv(n, 4), L.n_seg);
+    if (L.seg_cap < 64) L.seg_cap = 64;
+    const size_t cap = (size_t)(L.n_seg * L.seg_cap);
     L.off_state = 0;
     L.off_hist = 256;
-    L.off_keys = L.off_hist + 256 * sizeof(unsigned long long);
+    L.off_counts = L.off_hist + TOPK_MAX_BUCKETS * sizeof(unsigned long long);
+    L.off_keys = L.off_counts + kmx_align256((size_t)L.n_seg * sizeof(unsigned int));
     L.off_idx = L.off_keys + kmx_align256((size_t)k * sizeof(unsigned long long));
-    L.total = L.off_idx + kmx_align256((size_t)k * sizeof(long long));
+    L.off_cand_keys = L.off_idx + kmx_align256((size_t)k * sizeof(long long));
+    L.off_cand_idx = L.off_cand_keys + kmx_align256(cap * kmx_dtype_size(dtype));
+    L.row_bytes = L.off_cand_idx + kmx_align256(cap * sizeof(long long));
     return L;
+}
+
+// Per-row pointers into the workspace.
+struct TopkRow {
+    TopkState* st;
+    unsigned long long* hist;
+    unsigned int* counts;
+    unsigned long long* keys;
+    long long* idx;
+    void* cand_keys;
+    long long* cand_idx;
+};
+
+struct TopkArgs {
+    char* ws;
+    size_t row_bytes, off_hist, off_counts, off_keys, off_idx, off_cand_keys, off_cand_idx;
+    int64_t n;
+    int32_t k, n_seg, seg_cap;
+};
+
+__device__ __forceinline__ TopkRow topk_row(const TopkArgs& a, int64_t row) {
+    char* base = a.ws + (size_t)row * a.row_bytes;
+    TopkRow r;
+    r.st = (TopkState*)base;
+    r.hist = (unsigned long long*)(base + a.off_hist);
+    r.counts = (unsigned int*)(base + a.off_counts);
+    r.keys = (unsigned long long*)(base + a.off_keys);
+    r.idx = (long long*)(base + a.off_idx);
+    r.cand_keys = base + a.off_cand_keys;
+    r.cand_idx = (long long*)(base + a.off_cand_idx);
+    return r;
 }
 
 template <typename T>
@@ -42,146 +114,397 @@ template <>
 struct KeyOf<float> {
     using U = uint32_t;
     static constexpr int BITS = 32;
+    static constexpr int VEC = 4;  // elements of one 128-bit load
+    static constexpr int PASSES = 3;
     __device__ static __forceinline__ U key(float v) {
-        const U b = __float_as_uint(v);
+        const U b = __float_as_uint(v + 0.0f);  // -0.0 + 0.0 = +0.0
         return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
     }
+    __device__ static __forceinline__ float from_bits(uint32_t w0, uint32_t) { return __uint_as_float(w0); }
 };
 template <>
 struct KeyOf<double> {
     using U = unsigned long long;
     static constexpr int BITS = 64;
+    static constexpr int VEC = 2;
+    static constexpr int PASSES = 6;
     __device__ static __forceinline__ U key(double v) {
-        const U b = (U)__double_as_longlong(v);
+        const U b = (U)__double_as_longlong(v + 0.0);
         return b ^ ((b >> 63) ? 0xFFFFFFFFFFFFFFFFull : 0x8000000000000000ull);
+    }
+    __device__ static __forceinline__ double from_bits(uint32_t w0, uint32_t w1) {
+        return __longlong_as_double((long long)(((unsigned long long)w1 << 32) | w0));
     }
 };
 
-__global__ void topk_reset_kernel(TopkState* st, unsigned long long* hist, int32_t k) {
-    hist[threadIdx.x] = 0ull;
+// Bits of digit `pass` and the shift that brings it to the bottom of the key.
+template <typename T>
+__host__ __device__ constexpr int topk_width(int pass) {
+    return (KeyOf<T>::BITS == 32) ? (pass < 2 ? TOPK_WIDE : 10) : (pass < 4 ? TOPK_WIDE : 10);
+}
+template <typename T>
+__host__ __device__ constexpr int topk_shift(int pass) {
+    int s = KeyOf<T>::BITS;
+    for (int p = 0; p <= pass; ++p) s -= topk_width<T>(p);
+    return s;
+}
+
+__global__ __launch_bounds__(TOPK_WG) void topk_reset_kernel(TopkArgs a) {
+    const TopkRow r = topk_row(a, blockIdx.x);
+    for (int b = threadIdx.x; b < TOPK_MAX_BUCKETS; b += TOPK_WG) r.hist[b] = 0ull;
     if (threadIdx.x == 0) {
-        st->prefix = 0ull;
-        st->k_rem = k;
-        st->n_greater = 0ull;
-        st->tie_min = ~0ull;
-        st->n_ties_taken = 0ull;
+        r.st->prefix = 0ull;
+        r.st->k_rem = a.k;
+        r.st->n_out = 0ull;
+        r.st->tie_min = ~0ull;
+        r.st->ticket = 0u;
+        r.st->overflow = 0u;
+        r.st->cand_ok = 0u;
+        r.st->n_ties = 0u;
     }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void topk_hist_kernel(const T* __restrict__ values, int64_t n,
-                                                        const TopkState* __restrict__ st,
-                                                        unsigned long long* __restrict__ hist,
-                                                        int pass) {
-    using K = KeyOf<T>;
-    using U = typename K::U;
-    __shared__ unsigned int lh[256];
-    lh[threadIdx.x] = 0u;
-    __syncthreads();
-    const int shift = K::BITS - 8 * (pass + 1);
-    const U prefix = (U)st->prefix;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-        const U key = K::key(values[i]);
-        const bool match = (pass == 0) || ((key >> (shift + 8)) == prefix);
-        if (match) atomicAdd(&lh[(unsigned)((key >> shift) & 0xFF)], 1u);
-    }
-    __syncthreads();
-    const unsigned int c = lh[threadIdx.x];
-    if (c) atomicAdd(&hist[threadIdx.x], (unsigned long long)c);
-}
-
-// One workgroup of 256 threads, thread b = bucket b.
-__global__ __launch_bounds__(256) void topk_select_kernel(TopkState* st, unsigned long long* hist) {
-    __shared__ unsigned long long suffix[257];
-    const int b = threadIdx.x;
-    const unsigned long long h = hist[b];
-    suffix[b] = h;
-    if (b == 0) suffix[256] = 0ull;
-    __syncthreads();
-    // inclusive suffix sums: suffix[b] = sum_{b' >= b} h[b']
-    for (int off = 1; off < 256; off <<= 1) {
-        unsigned long long add = 0ull;
-        if (b + off < 256) add = suffix[b + off];
-        __syncthreads();
-        suffix[b] += add;
-        __syncthreads();
-    }
-    const unsigned long long k_rem = (unsigned long long)st->k_rem;
-    const unsigned long long above = suffix[b + 1];
-    __syncthreads();
-    if (above < k_rem && k_rem <= above + h) {
-        st->prefix = (st->prefix << 8) | (unsigned long long)b;
-        st->k_rem = (long long)(k_rem - above);
-    }
-    hist[b] = 0ull;
-}
-
-// Keys strictly above the threshold go to free slots (order fixed later); the lowest index
-// holding the threshold itself is tracked for the common single-tie case.
-template <typename T>
-__global__ __launch_bounds__(256) void topk_gather_kernel(const T* __restrict__ values, int64_t n,
-                                                          TopkState* __restrict__ st,
-                                                          unsigned long long* __restrict__ keys,
-                                                          long long* __restrict__ idx) {
-    using K = KeyOf<T>;
-    using U = typename K::U;
-    const U thr = (U)st->prefix;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-        const U key = K::key(values[i]);
-        if (key > thr) {
-            const unsigned long long slot = atomicAdd(&st->n_greater, 1ull);
-            keys[slot] = (unsigned long long)key;
-            idx[slot] = i;
-        } else if (key == thr) {
-            atomicMin(&st->tie_min, (unsigned long long)i);
+// Calls f(value, element index, valid) for the VEC elements of every aligned 128-bit vector
+// that overlaps the row, the same number of times in every lane of the workgroup (so f may
+// use wave-wide operations).  A vector that overlaps the row lies in one page with an element
+// of the row, so reading all of it cannot fault; elements outside the row are flagged invalid.
+template <typename T, typename F>
+__device__ __forceinline__ void topk_for_each(const T* __restrict__ row_values, int64_t n, F&& f) {
+    constexpr int VEC = KeyOf<T>::VEC;
+    const int64_t lead = (int64_t)(((uintptr_t)row_values / sizeof(T)) % VEC);  // elements before the row
+    const uint4* __restrict__ vecs = (const uint4*)(row_values - lead);
+    const int64_t n_vec = (n + lead + VEC - 1) / VEC;
+    const int64_t stride = (int64_t)gridDim.x * TOPK_WG;
+    constexpr int FLIGHT = 4;  // 128-bit loads in flight per lane
+    for (int64_t v0 = (int64_t)blockIdx.x * TOPK_WG; v0 < n_vec; v0 += FLIGHT * stride) {
+        uint4 w[FLIGHT];
+#pragma unroll
+        for (int u = 0; u < FLIGHT; ++u) {
+            const int64_t v = v0 + u * stride + threadIdx.x;
+            w[u] = make_uint4(0, 0, 0, 0);
+            if (v < n_vec) w[u] = vecs[v];
+        }
+#pragma unroll
+        for (int u = 0; u < FLIGHT; ++u) {
+            const int64_t v = v0 + u * stride + threadIdx.x;
+            const bool in = v < n_vec;
+            const uint32_t words[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const int64_t e = v * VEC + j - lead;
+                const T val = (VEC == 4) ? KeyOf<T>::from_bits(words[j], 0u)
+                                         : KeyOf<T>::from_bits(words[(2 * j) & 3], words[(2 * j + 1) & 3]);
+                f(val, e, in && e >= 0 && e < n);
+            }
         }
     }
 }
 
-// Takes the k_rem lowest indices holding the threshold key.  One workgroup walks the array in
-// index order and stops as soon as enough ties are found.
+// Appends the flagged lanes' (key, index) pairs behind `*counter` with one atomic for the wave.
+// Every lane of the wave must call it.  Slots at or beyond `cap` are dropped (the counter
+// still counts them).
+template <typename U>
+__device__ __forceinline__ void topk_append(bool flag, U key, long long index, unsigned long long* counter,
+                                            U* keys_out, long long* idx_out, unsigned long long cap) {
+    const unsigned long long mask = __ballot(flag);
+    if (mask == 0ull) return;
+    const int lane = threadIdx.x & 63;
+    unsigned long long base = 0ull;
+    if (lane == 0) base = atomicAdd(counter, (unsigned long long)__popcll(mask));
+    base = ((unsigned long long)__builtin_amdgcn_readfirstlane((int)(base >> 32)) << 32) |
+           (unsigned int)__builtin_amdgcn_readfirstlane((int)(base & 0xFFFFFFFFull));
+    if (flag) {
+        const unsigned long long slot = base + (unsigned long long)__popcll(mask & ((1ull << lane) - 1ull));
+        if (slot < cap) {
+            keys_out[slot] = key;
+            idx_out[slot] = index;
+        }
+    }
+}
+
+// One workgroup: walks the `1 << width` buckets from the top, fixes the digit that holds the
+// k_rem-th largest matching key, and clears the histogram for the next pass.
+__device__ __forceinline__ void topk_select_digit(TopkState* st, unsigned long long* hist, int width) {
+    constexpr int PER = TOPK_MAX_BUCKETS / TOPK_WG;  // consecutive buckets per thread
+    constexpr int WAVES = TOPK_WG / 64;
+    __shared__ unsigned long long bins[TOPK_MAX_BUCKETS];
+    __shared__ unsigned long long wave_sum[WAVES];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int n_buckets = 1 << width;
+    // coalesced, independent loads (issued together), staged through LDS
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int b = t + TOPK_WG * j;
+        bins[b] = b < n_buckets ? __hip_atomic_load(&hist[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) hist[t + TOPK_WG * j] = 0ull;
+    __syncthreads();
+    unsigned long long h[PER];
+    unsigned long long mine = 0ull;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        h[j] = bins[t * PER + j];
+        mine += h[j];
+    }
+    // suffix sums over the threads: inside the wave by shuffles, across waves through LDS
+    unsigned long long incl = mine;  // sum over lanes >= lane of this wave
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long o = __shfl_down(incl, off, 64);
+        if (lane + off < 64) incl += o;
+    }
+    if (lane == 0) wave_sum[wave] = incl;
+    __syncthreads();
+    unsigned long long above = incl - mine;  // buckets of higher threads
+    for (int w2 = wave + 1; w2 < WAVES; ++w2) above += wave_sum[w2];
+    const unsigned long long k_rem = (unsigned long long)st->k_rem;
+    const unsigned long long prefix = st->prefix;
+    __syncthreads();
+#pragma unroll
+    for (int j = PER - 1; j >= 0; --j) {
+        if (above < k_rem && k_rem <= above + h[j]) {
+            st->prefix = (prefix << width) | (unsigned long long)(t * PER + j);
+            st->k_rem = (long long)(k_rem - above);
+        }
+        above += h[j];
+    }
+}
+
+// True in the workgroup of the row that arrives last; every workgroup calls it once per launch,
+// after its own atomics on the row's state.  Waits until those have been performed.
+__device__ __forceinline__ bool topk_last_workgroup(TopkState* st) {
+    __shared__ unsigned int is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = (atomicAdd(&st->ticket, 1u) == gridDim.x - 1) ? 1u : 0u;
+    __syncthreads();
+    return is_last != 0u;
+}
+
+// Flushes the workgroup's LDS histogram, and lets the last workgroup of the row fix the digit.
+// Returns true in that workgroup (after the selection).
+__device__ __forceinline__ bool topk_finish_pass(TopkState* st, unsigned long long* hist, unsigned int* lh,
+                                                 int width) {
+    __syncthreads();
+    for (int b = threadIdx.x; b < (1 << width); b += TOPK_WG) {
+        const unsigned int c = lh[b];
+        if (c) atomicAdd(&hist[b], (unsigned long long)c);
+    }
+    if (!topk_last_workgroup(st)) return false;
+    topk_select_digit(st, hist, width);
+    if (threadIdx.x == 0) st->ticket = 0u;
+    return true;
+}
+
+// Pass 0: first digit of every key of the row.
 template <typename T>
-__global__ __launch_bounds__(1024) void topk_ties_kernel(const T* __restrict__ values, int64_t n,
-                                                         TopkState* __restrict__ st,
-                                                         unsigned long long* __restrict__ keys,
-                                                         long long* __restrict__ idx, int32_t k) {
+__global__ __launch_bounds__(TOPK_WG) void topk_first_kernel(const T* __restrict__ values, TopkArgs a) {
+    using K = KeyOf<T>;
+    __shared__ unsigned int lh[TOPK_MAX_BUCKETS];
+    const TopkRow r = topk_row(a, blockIdx.y);
+    constexpr int W = topk_width<T>(0), S = topk_shift<T>(0);
+    for (int b = threadIdx.x; b < (1 << W); b += TOPK_WG) lh[b] = 0u;
+    __syncthreads();
+    topk_for_each<T>(values + (size_t)blockIdx.y * a.n, a.n, [&](T v, int64_t, bool valid) {
+        if (valid) atomicAdd(&lh[(unsigned)(K::key(v) >> S)], 1u);
+    });
+    topk_finish_pass(r.st, r.hist, lh, W);
+}
+
+// Pass 1: winners above the first digit, candidates inside it, histogram of their second digit.
+template <typename T>
+__global__ __launch_bounds__(TOPK_WG) void topk_second_kernel(const T* __restrict__ values, TopkArgs a) {
     using K = KeyOf<T>;
     using U = typename K::U;
-    const U thr = (U)st->prefix;
-    const long long k_rem = st->k_rem;
-    const long long base_slot = (long long)k - k_rem;
+    __shared__ unsigned int lh[TOPK_MAX_BUCKETS];
+    __shared__ unsigned int seg_count;
+    const TopkRow r = topk_row(a, blockIdx.y);
+    constexpr int W = topk_width<T>(1), S = topk_shift<T>(1), S0 = topk_shift<T>(0);
+    for (int b = threadIdx.x; b < (1 << W); b += TOPK_WG) lh[b] = 0u;
+    if (threadIdx.x == 0) seg_count = 0u;
+    __syncthreads();
+    const U first = (U)r.st->prefix;
+    const int lane = threadIdx.x & 63;
+    U* __restrict__ seg_keys = (U*)r.cand_keys + (size_t)blockIdx.x * a.seg_cap;
+    long long* __restrict__ seg_idx = r.cand_idx + (size_t)blockIdx.x * a.seg_cap;
+    topk_for_each<T>(values + (size_t)blockIdx.y * a.n, a.n, [&](T v, int64_t e, bool valid) {
+        const U key = K::key(v);
+        const U digit = key >> S0;
+        const bool cand = valid && digit == first;
+        topk_append(valid && digit > first, (unsigned long long)key, e, &r.st->n_out, r.keys, r.idx,
+                    (unsigned long long)a.k);
+        const unsigned long long mask = __ballot(cand);
+        if (mask) {  // the wave's candidates go behind the workgroup's LDS counter
+            unsigned int base = 0u;
+            if (lane == 0) base = atomicAdd(&seg_count, (unsigned int)__popcll(mask));
+            base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
+            if (cand) {
+                const unsigned int slot = base + (unsigned int)__popcll(mask & ((1ull << lane) - 1ull));
+                if (slot < (unsigned int)a.seg_cap) {
+                    seg_keys[slot] = key;
+                    seg_idx[slot] = e;
+                }
+                atomicAdd(&lh[(unsigned)((key >> S) & ((1u << W) - 1u))], 1u);
+            }
+        }
+    });
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned int c = seg_count;
+        r.counts[blockIdx.x] = c < (unsigned int)a.seg_cap ? c : (unsigned int)a.seg_cap;
+        if (c > (unsigned int)a.seg_cap) atomicOr(&r.st->overflow, 1u);
+    }
+    if (topk_finish_pass(r.st, r.hist, lh, W) && threadIdx.x == 0)
+        r.st->cand_ok = __hip_atomic_load(&r.st->overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ? 0u : 1u;
+}
+
+// Calls f(key, element index, valid) for every candidate of the row: from the side buffer, or
+// from the row itself when the buffer was too small.  Uniform trip count per workgroup.
+template <typename T, typename F>
+__device__ __forceinline__ void topk_for_each_candidate(const T* __restrict__ row_values, const TopkArgs& a,
+                                                        const TopkRow& r, F&& f) {
+    using K = KeyOf<T>;
+    using U = typename K::U;
+    if (r.st->cand_ok) {
+        const U* __restrict__ ck = (const U*)r.cand_keys;
+        for (int seg = blockIdx.x; seg < a.n_seg; seg += gridDim.x) {
+            const int count = (int)r.counts[seg];
+            const size_t base = (size_t)seg * a.seg_cap;
+            for (int i0 = 0; i0 < count; i0 += TOPK_WG) {
+                const int i = i0 + threadIdx.x;
+                const bool in = i < count;
+                f(in ? ck[base + i] : (U)0, in ? r.cand_idx[base + i] : 0ll, in);
+            }
+        }
+    } else {
+        topk_for_each<T>(row_values, a.n, [&](T v, int64_t e, bool valid) { f(K::key(v), (long long)e, valid); });
+    }
+}
+
+// Passes 2..: one more digit of the candidates that match the digits fixed so far.
+template <typename T>
+__global__ __launch_bounds__(TOPK_WG) void topk_next_kernel(const T* __restrict__ values, TopkArgs a, int width,
+                                                            int shift) {
+    using K = KeyOf<T>;
+    using U = typename K::U;
+    __shared__ unsigned int lh[TOPK_MAX_BUCKETS];
+    const TopkRow r = topk_row(a, blockIdx.y);
+    for (int b = threadIdx.x; b < (1 << width); b += TOPK_WG) lh[b] = 0u;
+    __syncthreads();
+    const U prefix = (U)r.st->prefix;
+    const U digit_mask = (U)((1u << width) - 1u);
+    topk_for_each_candidate<T>(values + (size_t)blockIdx.y * a.n, a, r, [&](U key, long long, bool valid) {
+        if (valid && (key >> (shift + width)) == prefix) atomicAdd(&lh[(unsigned)((key >> shift) & digit_mask)], 1u);
+    });
+    topk_finish_pass(r.st, r.hist, lh, width);
+}
+
+// Candidates above the threshold key are winners; the lowest index holding the threshold key
+// itself is tracked (the common case takes exactly one of them).  The last workgroup of the
+// row then takes the k_rem lowest indices that hold the threshold key, walking the row in
+// index order from the first of them and stopping as soon as it has enough.
+template <typename T>
+__global__ __launch_bounds__(TOPK_WG) void topk_gather_kernel(const T* __restrict__ values, TopkArgs a) {
+    using K = KeyOf<T>;
+    using U = typename K::U;
+    const TopkRow r = topk_row(a, blockIdx.y);
+    const T* __restrict__ row_values = values + (size_t)blockIdx.y * a.n;
+    constexpr int S0 = topk_shift<T>(0);
+    const U thr = (U)r.st->prefix;
+    const U first = thr >> S0;
+    const int lane = threadIdx.x & 63;
+    long long* __restrict__ tie_list = (long long*)r.hist;
+    __shared__ unsigned int ties_full;
+    if (threadIdx.x == 0) ties_full = 0u;
+    __syncthreads();
+    topk_for_each_candidate<T>(row_values, a, r, [&](U key, long long e, bool valid) {
+        const bool mine = valid && (key >> S0) == first;  // keys above the first digit went out in pass 1
+        topk_append<unsigned long long>(mine && key > thr, (unsigned long long)key, e, &r.st->n_out, r.keys, r.idx,
+                                        (unsigned long long)a.k);
+        const bool tie = mine && key == thr;
+        const unsigned long long tie_mask = __ballot(tie);
+        if (tie_mask) {
+            unsigned long long m = tie ? (unsigned long long)e : ~0ull;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const unsigned long long o = __shfl_xor(m, off, 64);
+                m = o < m ? o : m;
+            }
+            if (lane == 0) atomicMin(&r.st->tie_min, m);
+            // the indices that hold the threshold key are listed in the (now unused) histogram
+            // while they fit; a workgroup stops once it has seen the list full
+            if (!ties_full) {
+                unsigned int base = 0u;
+                if (lane == 0) base = atomicAdd(&r.st->n_ties, (unsigned int)__popcll(tie_mask));
+                base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
+                if (tie) {
+                    const unsigned int slot = base + (unsigned int)__popcll(tie_mask & ((1ull << lane) - 1ull));
+                    if (slot < TOPK_TIE_LIST)  // read by another workgroup of this launch: device-scope store
+                        __hip_atomic_store(&tie_list[slot], e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (base + (unsigned int)__popcll(tie_mask) > TOPK_TIE_LIST) ties_full = 1u;  // benign race
+            }
+        }
+    });
+
+    if (!topk_last_workgroup(r.st)) return;
+    const long long k_rem = r.st->k_rem;
+    const long long base_slot = (long long)a.k - k_rem;
+    const unsigned long long tie_min =
+        __hip_atomic_load(&r.st->tie_min, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) r.st->ticket = 0u;
     if (k_rem == 1) {
         if (threadIdx.x == 0) {
-            keys[base_slot] = (unsigned long long)thr;
-            idx[base_slot] = (long long)st->tie_min;
+            r.keys[base_slot] = (unsigned long long)thr;
+            r.idx[base_slot] = (long long)tie_min;
         }
         return;
     }
-    __shared__ int wave_counts[16];
+    const unsigned int n_ties = __hip_atomic_load(&r.st->n_ties, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (n_ties <= TOPK_TIE_LIST) {
+        // the list is complete: its k_rem lowest indices, by rank
+        __shared__ long long ties[TOPK_TIE_LIST];
+        for (unsigned int i = threadIdx.x; i < n_ties; i += TOPK_WG)
+            ties[i] = (long long)__hip_atomic_load((unsigned long long*)&tie_list[i], __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        for (unsigned int i = threadIdx.x; i < n_ties; i += TOPK_WG) {
+            const long long mine = ties[i];
+            long long rank = 0;
+            for (unsigned int j = 0; j < n_ties; ++j) rank += ties[j] < mine ? 1 : 0;
+            if (rank < k_rem) {
+                r.keys[base_slot + rank] = (unsigned long long)thr;
+                r.idx[base_slot + rank] = mine;
+            }
+        }
+        return;
+    }
+    // too many to list: they are dense, and walking the row in index order from the first of
+    // them finds k_rem of them soon
+    __shared__ int wave_counts[TOPK_WG / 64];
     __shared__ long long taken_s;
     if (threadIdx.x == 0) taken_s = 0;
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int64_t i0 = st->tie_min; i0 < n; i0 += 1024) {
+    const int wave = threadIdx.x >> 6;
+    for (int64_t i0 = (int64_t)tie_min; i0 < a.n; i0 += TOPK_WG) {
         const long long taken = taken_s;
         if (taken >= k_rem) break;
         const int64_t i = i0 + threadIdx.x;
-        const bool flag = (i < n) && (K::key(values[i]) == thr);
+        const bool flag = (i < a.n) && (K::key(row_values[i]) == thr);
         const unsigned long long mask = __ballot(flag);
         if (lane == 0) wave_counts[wave] = __popcll(mask);
         __syncthreads();
         long long offset = taken;
         int all = 0;
-        for (int w2 = 0; w2 < 16; ++w2) {
+        for (int w2 = 0; w2 < TOPK_WG / 64; ++w2) {
             if (w2 < wave) offset += wave_counts[w2];
             all += wave_counts[w2];
         }
         const long long rank = offset + __popcll(mask & ((1ull << lane) - 1ull));
         if (flag && rank < k_rem) {
-            keys[base_slot + rank] = (unsigned long long)thr;
-            idx[base_slot + rank] = i;
+            r.keys[base_slot + rank] = (unsigned long long)thr;
+            r.idx[base_slot + rank] = i;
         }
         __syncthreads();
         if (threadIdx.x == 0) taken_s = taken + all;
@@ -189,74 +512,109 @@ __global__ __launch_bounds__(1024) void topk_ties_kernel(const T* __restrict__ v
     }
 }
 
-// Rank sort of the k winners: descending key, ascending index.
-__global__ __launch_bounds__(256) void topk_order_kernel(const unsigned long long* __restrict__ keys,
-                                                         const long long* __restrict__ idx,
-                                                         int64_t* __restrict__ out, int32_t k) {
+// Rank sort of the k winners of a row (descending key, ascending index); writes the indices
+// and/or the values in that order.
+template <typename T>
+__global__ __launch_bounds__(256) void topk_order_kernel(const T* __restrict__ values, TopkArgs a,
+                                                         int64_t* __restrict__ out_idx, T* __restrict__ out_values) {
+    const TopkRow r = topk_row(a, blockIdx.y);
     const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= k) return;
-    const unsigned long long ki = keys[i];
-    const long long ii = idx[i];
+    if (i >= a.k) return;
+    const unsigned long long ki = r.keys[i];
+    const long long ii = r.idx[i];
     int rank = 0;
-    for (int j = 0; j < k; ++j) {
-        const unsigned long long kj = keys[j];
-        const long long ij = idx[j];
+    for (int j = 0; j < a.k; ++j) {
+        const unsigned long long kj = r.keys[j];
+        const long long ij = r.idx[j];
         rank += (kj > ki || (kj == ki && ij < ii)) ? 1 : 0;
     }
-    out[rank] = ii;
+    const size_t o = (size_t)blockIdx.y * a.k + rank;
+    if (out_idx) out_idx[o] = ii;
+    if (out_values) out_values[o] = values[(size_t)blockIdx.y * a.n + ii];
 }
 
 template <typename T>
-int32_t topk_impl(const void* values, int64_t* out, int64_t n, int32_t k, char* ws,
-                  hipStream_t stream) {
-    const TopkLayout L = topk_layout(k);
-    auto* st = (TopkState*)(ws + L.off_state);
-    auto* hist = (unsigned long long*)(ws + L.off_hist);
-    auto* keys = (unsigned long long*)(ws + L.off_keys);
-    auto* idx = (long long*)(ws + L.off_idx);
-    int64_t blocks = kmx_cdiv(n, 256 * 8);
-    const int64_t cap = (int64_t)kmx_num_cus() * 4;
-    if (blocks > cap) blocks = cap;
-    if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL(topk_reset_kernel, dim3(1), dim3(256), 0, stream, st, hist, k);
-    const int passes = KeyOf<T>::BITS / 8;
-    for (int p = 0; p < passes; ++p) {
-        hipLaunchKernelGGL((topk_hist_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                           (const T*)values, n, st, hist, p);
-        hipLaunchKernelGGL(topk_select_kernel, dim3(1), dim3(256), 0, stream, st, hist);
+int32_t topk_impl(const void* values_, int64_t* out_idx, void* out_values, int64_t rows, int64_t n, int32_t k,
+                  char* ws, int32_t dtype, hipStream_t stream) {
+    const TopkLayout L = topk_layout(rows, n, k, dtype);
+    // rows are taken in slices of the grid's second dimension
+    for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
+        const int64_t nr = rows - r0 < 65535 ? rows - r0 : 65535;
+        const T* values = (const T*)values_ + (size_t)r0 * n;
+        TopkArgs a;
+        a.ws = ws + (size_t)r0 * L.row_bytes;
+        a.row_bytes = L.row_bytes;
+        a.off_hist = L.off_hist;
+        a.off_counts = L.off_counts;
+        a.off_keys = L.off_keys;
+        a.off_idx = L.off_idx;
+        a.off_cand_keys = L.off_cand_keys;
+        a.off_cand_idx = L.off_cand_idx;
+        a.n = n;
+        a.k = k;
+        a.n_seg = (int32_t)L.n_seg;
+        a.seg_cap = (int32_t)L.seg_cap;
+        // the passes over the candidates: a quarter of the workgroups (each takes several segments)
+        const int64_t per_row_cand = L.n_seg >= 4 ? L.n_seg / 4 : 1;
+        const dim3 grid_full((unsigned)L.n_seg, (unsigned)nr), grid_cand((unsigned)per_row_cand, (unsigned)nr);
+        hipLaunchKernelGGL(topk_reset_kernel, dim3((unsigned)nr), dim3(TOPK_WG), 0, stream, a);
+        hipLaunchKernelGGL((topk_first_kernel<T>), grid_full, dim3(TOPK_WG), 0, stream, values, a);
+        hipLaunchKernelGGL((topk_second_kernel<T>), grid_full, dim3(TOPK_WG), 0, stream, values, a);
+        for (int p = 2; p < KeyOf<T>::PASSES; ++p)
+            hipLaunchKernelGGL((topk_next_kernel<T>), grid_cand, dim3(TOPK_WG), 0, stream, values, a,
+                               topk_width<T>(p), topk_shift<T>(p));
+        hipLaunchKernelGGL((topk_gather_kernel<T>), grid_cand, dim3(TOPK_WG), 0, stream, values, a);
+        hipLaunchKernelGGL((topk_order_kernel<T>), dim3((unsigned)kmx_cdiv(k, 256), (unsigned)nr), dim3(256), 0,
+                           stream, values, a, out_idx ? out_idx + (size_t)r0 * k : nullptr,
+                           out_values ? (T*)out_values + (size_t)r0 * k : nullptr);
     }
-    hipLaunchKernelGGL((topk_gather_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                       (const T*)values, n, st, keys, idx);
-    hipLaunchKernelGGL((topk_ties_kernel<T>), dim3(1), dim3(1024), 0, stream, (const T*)values, n,
-                       st, keys, idx, k);
-    hipLaunchKernelGGL(topk_order_kernel, dim3((unsigned)kmx_cdiv(k, 256)), dim3(256), 0, stream,
-                       keys, idx, out, k);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
+}
+
+int32_t topk_entry(const void* values, int64_t* out_idx, void* out_values, int64_t rows, int64_t n, int32_t k,
+                   void* workspace, size_t workspace_bytes, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(values);
+    KMX_REQUIRE_PTR(workspace);
+    if (rows <= 0 || n <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    if (k > n) return KMX_ERR_BAD_ARGUMENT;
+    KMX_REQUIRE_DTYPE(dtype);
+    if (workspace_bytes < kmx_topk_rows_workspace_bytes(rows, n, k, dtype)) return KMX_ERR_WORKSPACE;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == KMX_F32)
+        return topk_impl<float>(values, out_idx, out_values, rows, n, k, (char*)workspace, dtype, stream);
+    return topk_impl<double>(values, out_idx, out_values, rows, n, k, (char*)workspace, dtype, stream);
 }
 
 }  // namespace
 
 extern "C" {
 
-size_t kmx_topk_workspace_bytes(int64_t n, int32_t k) {
-    if (n <= 0 || k <= 0 || k > n) return 0;
-    return topk_layout(k).total;
+size_t kmx_topk_rows_workspace_bytes(int64_t rows, int64_t n, int32_t k, int32_t dtype) {
+    if (rows <= 0 || n <= 0 || k <= 0 || k > n) return 0;
+    if (dtype != KMX_F32 && dtype != KMX_F64) return 0;
+    return (size_t)rows * topk_layout(rows, n, k, dtype).row_bytes;
 }
 
-int32_t kmx_topk_idx(const void* values, int64_t* out_indices, int64_t n, int32_t k,
-                     void* workspace, size_t workspace_bytes, int32_t dtype, void* stream_) {
-    KMX_ENTRY();
-    KMX_REQUIRE_PTR(values);
+size_t kmx_topk_workspace_bytes(int64_t n, int32_t k) { return kmx_topk_rows_workspace_bytes(1, n, k, KMX_F64); }
+
+int32_t kmx_topk_idx_rows(const void* values, int64_t* out_indices, int64_t rows, int64_t n, int32_t k,
+                          void* workspace, size_t workspace_bytes, int32_t dtype, void* stream) {
     KMX_REQUIRE_PTR(out_indices);
-    KMX_REQUIRE_PTR(workspace);
-    if (n <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
-    if (k > n) return KMX_ERR_BAD_ARGUMENT;
-    KMX_REQUIRE_DTYPE(dtype);
-    if (workspace_bytes < topk_layout(k).total) return KMX_ERR_WORKSPACE;
-    hipStream_t stream = (hipStream_t)stream_;
-    if (dtype == KMX_F32) return topk_impl<float>(values, out_indices, n, k, (char*)workspace, stream);
-    return topk_impl<double>(values, out_indices, n, k, (char*)workspace, stream);
+    return topk_entry(values, out_indices, nullptr, rows, n, k, workspace, workspace_bytes, dtype, stream);
+}
+
+int32_t kmx_topk_values(const void* values, void* out_values, int64_t rows, int64_t n, int32_t k, void* workspace,
+                        size_t workspace_bytes, int32_t dtype, void* stream) {
+    KMX_REQUIRE_PTR(out_values);
+    return topk_entry(values, nullptr, out_values, rows, n, k, workspace, workspace_bytes, dtype, stream);
+}
+
+int32_t kmx_topk_idx(const void* values, int64_t* out_indices, int64_t n, int32_t k, void* workspace,
+                     size_t workspace_bytes, int32_t dtype, void* stream) {
+    KMX_REQUIRE_PTR(out_indices);
+    return topk_entry(values, out_indices, nullptr, 1, n, k, workspace, workspace_bytes, dtype, stream);
 }
 
 }  // extern "C"

@@ -74,6 +74,10 @@ def test_workspace_queries():
     assert lib.kmx_kpp_workspace_bytes(1000, 4, 8, 17, 0) == 0  # more trials than supported
     assert lib.kmx_topk_workspace_bytes(1000, 10) > 0
     assert lib.kmx_topk_workspace_bytes(5, 10) == 0
+    one_row = lib.kmx_topk_rows_workspace_bytes(1, 1000, 10, 0)
+    assert 0 < one_row <= lib.kmx_topk_workspace_bytes(1000, 10)
+    assert lib.kmx_topk_rows_workspace_bytes(7, 1000, 10, 0) == 7 * one_row
+    assert lib.kmx_topk_rows_workspace_bytes(7, 1000, 10, 5) == 0
     assert lib.kmx_sum_workspace_bytes(7, 1_000_000) >= 7 * 256 * 8
 
 
@@ -180,6 +184,10 @@ def test_bad_arguments_are_rejected_without_a_device():
     assert lib.kmx_euclidean_distances(p, p, p, 10, 2, 2, 5, NULL) == -3
     assert lib.kmx_topk_idx(p, p, 5, 10, p, 4096, 0, NULL) == -5      # k > n
     assert lib.kmx_topk_idx(p, p, 50, 10, p, 8, 0, NULL) == -4
+    assert lib.kmx_topk_idx_rows(p, p, 0, 50, 10, p, 1 << 20, 0, NULL) == -2   # no rows
+    assert lib.kmx_topk_idx_rows(p, NULL, 3, 50, 10, p, 1 << 20, 0, NULL) == -1
+    assert lib.kmx_topk_values(p, p, 3, 50, 10, p, 8, 1, NULL) == -4
+    assert lib.kmx_topk_values(p, p, 3, 50, 10, p, 1 << 20, 7, NULL) == -3     # unknown dtype
     assert lib.kmx_broadcast_rows(p, p, 2, 2, 3, 0, NULL) == -5       # unknown op
     assert lib.kmx_kpp_init(p, p, 20, p, p, p, 1 << 20, 10, 2, 2, 2, 0, NULL) in (-4, -5)
     assert lib.kmx_kpp_run(p, p, p, 0, p, p, p, 16, 10, 2, 2, 2, 0, NULL) == -4

@@ -92,13 +92,46 @@ def test_topk_multirow_and_random(cuda, dtype):
 
     a = np.array(TOPK_CASES, dtype=dtype)
     got = topk(_dev(a, cuda), 3).cpu().numpy()
-    np.testing.assert_array_equal(np.sort(got, axis=1), np.sort(a, axis=1)[:, -3:])
+    np.testing.assert_array_equal(got, -np.sort(-a, axis=1)[:, :3])  # descending
     rng = np.random.default_rng(123)
-    big = rng.normal(size=(8, 1000)).astype(dtype)  # reference uses (1000, 1000); same per-row path
-    for k in (1, 3):
-        idx = topk_idx(_dev(big, cuda), k).cpu().numpy()
-        for r in range(big.shape[0]):
-            np.testing.assert_array_equal(idx[r], ok.top_k_indices(big[r], k))
+    # the reference's random case (common/tests/test_topk.py:62-80): 1000 rows of 1000 values;
+    # 1001 columns here so that most rows start off a 16-byte boundary
+    big = rng.normal(size=(1000, 1001)).astype(dtype)
+    d_big = _dev(big, cuda)
+    for k in (1, 3, 40):
+        idx = topk_idx(d_big, k).cpu().numpy()
+        assert idx.shape == (1000, k) and idx.dtype == np.int64
+        want = np.stack([ok.top_k_indices(big[r], k) for r in range(big.shape[0])])
+        np.testing.assert_array_equal(idx, want)
+        vals = topk(d_big, k).cpu().numpy()
+        np.testing.assert_array_equal(vals, np.take_along_axis(big, want, axis=1))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_topk_dense_threshold_bucket_and_signed_zeros(cuda, dtype):
+    """Rows whose largest values share their leading digits: more candidates than the side
+    buffer holds (all of [1, 1.25) and a constant row), a quarter-full one (uniform [0, 1)),
+    and -0.0 / +0.0, which rank as equal (lowest index first)."""
+    from sklearn_numba_dpex_amd.common.topk import topk, topk_idx
+
+    rng = np.random.default_rng(77)
+    n = 300_001
+    rows = np.stack([
+        rng.uniform(1.0, 1.25, n),
+        np.full(n, 3.0),
+        rng.uniform(0.0, 1.0, n),
+        -rng.uniform(1.0, 1.25, n),
+    ]).astype(dtype)
+    d_rows = _dev(rows, cuda)
+    for k in (1, 7, 2000):
+        idx = topk_idx(d_rows, k).cpu().numpy()
+        want = np.stack([ok.top_k_indices(rows[r], k) for r in range(rows.shape[0])])
+        np.testing.assert_array_equal(idx, want)
+        np.testing.assert_array_equal(topk(d_rows, k).cpu().numpy(), np.take_along_axis(rows, want, axis=1))
+    z = np.array([-1.0, -0.0, 0.0, -0.0, 0.0, -2.0], dtype=dtype)
+    np.testing.assert_array_equal(topk_idx(_dev(z, cuda), 3).cpu().numpy(), [1, 2, 3])
+    got = topk(_dev(z, cuda), 3).cpu().numpy()
+    np.testing.assert_array_equal(np.signbit(got), [True, False, True])  # the stored values, bit for bit
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
