@@ -404,7 +404,12 @@ def gpu_components(cfg):
     put("matmul_4096", t, 3 * 4096 * 4096 * s, "kmx_matmul fp32 4096 x 4096 x 4096 on the matrix cores (contraction bound)")
     out["matmul_4096"]["TFLOPs"] = 2.0 * 4096**3 / t / 1e12
     out["matmul_4096"]["fp32_peak_frac"] = out["matmul_4096"]["TFLOPs"] / FP32_PEAK_TFLOPS
-    del A, B
+    A64, B64 = A.double(), B.double()
+    t = timed(lambda: matmul(A64, B64))
+    put("matmul_4096_f64", t, 3 * 4096 * 4096 * 8, "kmx_matmul fp64 4096 x 4096 x 4096 (v_mfma_f64_16x16x4_f64)")
+    out["matmul_4096_f64"]["TFLOPs"] = 2.0 * 4096**3 / t / 1e12
+    out["matmul_4096_f64"]["fp64_peak_frac"] = out["matmul_4096_f64"]["TFLOPs"] / 78.6
+    del A, B, A64, B64
     Xc = X_t.clone()
     t = timed(lambda: drivers.prepare_data_for_lloyd(Xc, cent_t.clone(), 1e-4, w_d, copy_x=False))
     put("prepare_data_for_lloyd", t, 4 * n * d * s,

@@ -411,6 +411,22 @@ int32_t kmx_count_distinct_clusters(const uint32_t* labels, int32_t* seen, int32
 int32_t kmx_matmul(const void* X, const void* Y_t, void* out, int32_t m, int32_t p, int32_t q,
                    int32_t dtype, void* stream);
 
+/* The scalar combined over K (multiply_fn of make_matmul_2d_kernel, common/matmul.py:64-66) and
+ * the function applied to each finished sum (out_fused_elementwise_fn, :55-62), for the
+ * functions the reference predefines (common/_utils.py:17-33). */
+#define KMX_MATMUL_MULTIPLY 0      /* sum_k x * y: matrix cores */
+#define KMX_MATMUL_MINUS 1         /* sum_k (x - y) */
+#define KMX_MATMUL_PLUS 2          /* sum_k (x + y) */
+#define KMX_MATMUL_OUT_IDENTITY 0
+#define KMX_MATMUL_OUT_SQUARE 1    /* v * v */
+#define KMX_MATMUL_OUT_DIVIDE_BY 2 /* v / out_param */
+
+/* out[i, j] = out_op(sum_k multiply_op(X[i, k], Y_t[j, k])).  make_matmul_2d_kernel with
+ * multiply_fn / out_fused_elementwise_fn, common/matmul.py:13-70,300-567. */
+int32_t kmx_matmul_fused(const void* X, const void* Y_t, void* out, int32_t m, int32_t p,
+                         int32_t q, int32_t multiply_op, int32_t out_op, double out_param,
+                         int32_t dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------ *
  * Machine probes (benchmarks only)                                                      *
  * ------------------------------------------------------------------------------------ */

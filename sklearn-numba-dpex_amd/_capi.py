@@ -147,6 +147,7 @@ SIGNATURES = {
     "kmx_is_same_clustering": (_I32, [_P, _P, _P, _P, _I64, _I32, _P]),
     "kmx_count_distinct_clusters": (_I32, [_P, _P, _P, _I64, _I32, _P]),
     "kmx_matmul": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _P]),
+    "kmx_matmul_fused": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _I32, c_double, _I32, _P]),
     "kmx_probe_copy": (_I32, [_P, _P, _SZ, _P]),
     "kmx_probe_read": (_I32, [_P, _SZ, _P, _P]),
     "kmx_probe_mfma": (_I32, [_I32, _I32, _P, POINTER(c_double), _P]),

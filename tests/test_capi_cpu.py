@@ -195,6 +195,8 @@ def test_bad_arguments_are_rejected_without_a_device():
     assert lib.kmx_relocate_empty_clusters(p, p, p, p, p, 3, NULL, p, p, 10, 2, 2, 0, NULL) == -2
     assert lib.kmx_sum_rows(p, p, 0, 5, 0, p, 4096, 0, NULL) == -2
     assert lib.kmx_matmul(p, p, NULL, 2, 2, 2, 0, NULL) == -1
+    assert lib.kmx_matmul_fused(p, p, p, 2, 2, 2, 3, 0, 0.0, 0, NULL) == -5   # unknown multiply
+    assert lib.kmx_matmul_fused(p, p, p, 2, 2, 2, 0, 3, 0.0, 0, NULL) == -5   # unknown output function
     assert lib.kmx_argmin(p, p, 0, 0, NULL) == -2
 
 

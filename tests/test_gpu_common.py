@@ -193,6 +193,51 @@ def test_matmul(cuda, shape, dtype):
                                rtol=1e-4 if dtype == np.float32 else 1e-11, atol=1e-4 if dtype == np.float32 else 1e-11)
 
 
+# the reference's small shapes with `arange` operands (common/tests/test_matmul.py:13-16,71-104)
+@pytest.mark.parametrize("shapes", [((1, 1), (1, 1)), ((4, 4), (4, 4)), ((5, 5), (5, 5)), ((1, 4), (4, 1)),
+                                    ((1, 5), (5, 1)), ((4, 1), (1, 4)), ((5, 1), (1, 5)), ((4, 5), (5, 4)),
+                                    ((5, 4), (4, 5)), ((5, 4), (4, 8)), ((5, 4), (4, 10)), ((4, 5), (5, 10)),
+                                    ((10, 4), (4, 5)), ((5, 10), (10, 4)), ((1999, 661), (661, 563))])
+def test_matmul_arange(cuda, shapes):
+    from sklearn_numba_dpex_amd.common.matmul import matmul
+
+    (m, p), (_, q) = shapes
+    X = np.arange(m * p, dtype=np.float32).reshape(m, p)
+    Y = np.arange(p * q, dtype=np.float32).reshape(p, q)
+    got = matmul(_dev(X, cuda), _dev(np.ascontiguousarray(Y.T), cuda)).cpu().numpy()
+    np.testing.assert_allclose(got, np.matmul(X, Y), rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(3, 5, 2), (65, 17, 130), (257, 33, 129), (1000, 70, 300)])
+def test_matmul_fused_functions(cuda, shape, dtype):
+    """multiply_fn and out_fused_elementwise_fn of make_matmul_2d_kernel (reference
+    common/matmul.py:55-66) for the functions the reference predefines (common/_utils.py:17-33)."""
+    from sklearn_numba_dpex_amd.common import _utils
+    from sklearn_numba_dpex_amd.common.matmul import matmul
+
+    m, p, q = shape
+    rng = np.random.default_rng(3)
+    X = rng.normal(size=(m, p)).astype(dtype)
+    Y_t = rng.normal(size=(q, p)).astype(dtype)
+    X64, Y64 = X.astype(np.float64), Y_t.astype(np.float64)
+    tol = dict(rtol=1e-4, atol=1e-4) if dtype == np.float32 else dict(rtol=1e-11, atol=1e-11)
+    dX, dY = _dev(X, cuda), _dev(Y_t, cuda)
+    prod = X64 @ Y64.T
+    np.testing.assert_allclose(matmul(dX, dY, out_fused_elementwise_fn=_utils._square).cpu().numpy(), prod**2, **tol)
+    np.testing.assert_allclose(matmul(dX, dY, out_fused_elementwise_fn=_utils._divide_by(4.0)).cpu().numpy(),
+                               prod / 4.0, **tol)
+    minus = X64.sum(axis=1)[:, None] - Y64.sum(axis=1)[None, :]
+    plus = X64.sum(axis=1)[:, None] + Y64.sum(axis=1)[None, :]
+    np.testing.assert_allclose(matmul(dX, dY, multiply_fn=_utils._minus).cpu().numpy(), minus, **tol)
+    np.testing.assert_allclose(matmul(dX, dY, multiply_fn=_utils._plus).cpu().numpy(), plus, **tol)
+    np.testing.assert_allclose(
+        matmul(dX, dY, multiply_fn=_utils._minus, out_fused_elementwise_fn=_utils._square).cpu().numpy(),
+        minus**2, rtol=tol["rtol"] * 10, atol=tol["atol"] * 10)
+    with pytest.raises(NotImplementedError, match="predefined functions"):
+        matmul(dX, dY, multiply_fn=lambda x, y: x * y + 1)
+
+
 def test_label_helpers(cuda):
     from sklearn_numba_dpex_amd.kmeans import drivers
 
