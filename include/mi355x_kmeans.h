@@ -239,6 +239,17 @@ int32_t kmx_per_sample_inertia(const void* X_t, const void* sample_weight, const
                                const uint32_t* labels, void* out, int64_t n, int32_t d,
                                int32_t k, int32_t dtype, void* stream);
 
+/* out_total[0] = sum_i w_i * ||x_i - c_label_i||^2: the per-sample kernel with the sum folded in
+ * (fp64 totals per workgroup in `workspace`, added in order by a second small launch), so the
+ * n per-sample values are neither written nor read back.  Replaces compute_inertia_kernel
+ * followed by the sum reduction at the end of a fit and in get_labels_inertia
+ * (kmeans/drivers.py:379-391, 674-697; kmeans/kernels/compute_inertia.py:9-42). */
+size_t kmx_inertia_workspace_bytes(int64_t n);
+int32_t kmx_inertia(const void* X_t, const void* sample_weight, const void* centroids_t,
+                    const uint32_t* labels, void* out_total, void* workspace,
+                    size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
+                    void* stream);
+
 /* distances_t (k, n): sqrt(sum_f (c_f - x_f)^2).  Replaces
  * make_compute_euclidean_distances_fixed_window_kernel
  * (kmeans/kernels/compute_euclidean_distances.py:15-161). */

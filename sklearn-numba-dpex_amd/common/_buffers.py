@@ -17,8 +17,24 @@ def torch_dtype(dtype):
     return {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64}[np.dtype(dtype)]
 
 
-def workspace(n_bytes, device):
-    return torch.empty(max(int(n_bytes), 1), dtype=torch.uint8, device=device)
+_workspaces = {}
+
+
+def workspace(n_bytes, device, tag=None):
+    """Scratch bytes for one library call.  With a `tag` the buffer is kept and handed out again
+    to the next call with the same tag on the same device and stream (work on one stream is
+    ordered, so the calls cannot overlap); it only ever grows."""
+    n_bytes = max(int(n_bytes), 1)
+    if tag is None:
+        return torch.empty(n_bytes, dtype=torch.uint8, device=device)
+    device = torch.device(device)
+    key = (tag, device.index if device.index is not None else torch.cuda.current_device(),
+           _capi.current_stream())
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < n_bytes:
+        buf = torch.empty(max(n_bytes, 4096), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
 
 
 def dcode(t):

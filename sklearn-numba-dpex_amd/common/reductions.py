@@ -20,7 +20,7 @@ def sum_reduction(array, axis=1, square=False):
         axis = 1
     rows, cols = a.shape
     ws_bytes = lib.kmx_sum_workspace_bytes(rows, cols)
-    ws = workspace(ws_bytes, a.device)
+    ws = workspace(ws_bytes, a.device, tag="sum")
     stream = _capi.current_stream()
     if axis == 1:
         out = torch.empty(rows, dtype=a.dtype, device=a.device)

@@ -20,7 +20,7 @@ def _prepare(array_in, k):
     if a.dtype not in (torch.float32, torch.float64):
         raise ValueError(f"topk currently only supports float32 and float64, got dtype={a.dtype} .")
     ws_bytes = lib.kmx_topk_rows_workspace_bytes(rows, n, k, dcode(a))
-    return a, rows, n, workspace(ws_bytes, a.device), ws_bytes
+    return a, rows, n, workspace(ws_bytes, a.device, tag="topk"), ws_bytes
 
 
 def topk_idx(array_in, k):

@@ -43,11 +43,13 @@ __device__ __forceinline__ void store4(T* __restrict__ row, int64_t i0, int64_t 
 // four consecutive samples (128-bit loads of every feature row); the centroids are staged in
 // LDS when they fit (LDS_CENTROIDS), so that the per-sample gather of the label's centroid
 // does not go through the vector memory pipe.
-template <typename T, bool LDS_CENTROIDS>
+// SUM: nothing is written per sample; the workgroup's total goes to partial[blockIdx.x] in fp64
+// (fixed order inside the workgroup, so the result does not depend on timing).
+template <typename T, bool LDS_CENTROIDS, bool SUM>
 __global__ __launch_bounds__(256) void per_sample_inertia_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight,
     const T* __restrict__ centroids_t, const uint32_t* __restrict__ labels, T* __restrict__ out,
-    int64_t n, int d, int k, int vec_ok) {
+    double* __restrict__ partial, int64_t n, int d, int k, int vec_ok) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* cs = reinterpret_cast<T*>(smem_raw);  // [d * k], same layout as centroids_t
     if (LDS_CENTROIDS) {
@@ -57,6 +59,8 @@ __global__ __launch_bounds__(256) void per_sample_inertia_kernel(
     const T* __restrict__ cent = LDS_CENTROIDS ? cs : centroids_t;
     const int64_t n_groups = (n + 3) >> 2;
     const int64_t stride = (int64_t)gridDim.x * 256;
+    double total = 0.0;
+    (void)total;
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < n_groups; g += stride) {
         const int64_t i0 = g * 4;
         const bool full = vec_ok && (i0 + 4 <= n);
@@ -81,17 +85,61 @@ __global__ __launch_bounds__(256) void per_sample_inertia_kernel(
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[r] *= w[r];
         }
-        store4<T>(out, i0, n, full, acc);
+        if constexpr (SUM) {
+            // samples past n have x = 0 and label 0: their value is dropped here
+#pragma unroll
+            for (int r = 0; r < 4; ++r) total += (i0 + r < n) ? (double)acc[r] : 0.0;
+        } else {
+            store4<T>(out, i0, n, full, acc);
+        }
+    }
+    if constexpr (SUM) {
+        __shared__ double wave_part[4];
+        total = kmx_block_sum<double>(total, wave_part);
+        if (threadIdx.x == 0) partial[blockIdx.x] = total;
     }
 }
 
+// out[0] = sum of the workgroup partials, in order.
+template <typename T>
+__global__ __launch_bounds__(256) void inertia_total_kernel(const double* __restrict__ partial, int count,
+                                                            T* __restrict__ out) {
+    __shared__ double wave_part[4];
+    double v = 0.0;
+    for (int i = threadIdx.x; i < count; i += 256) v += partial[i];
+    v = kmx_block_sum<double>(v, wave_part);
+    if (threadIdx.x == 0) out[0] = (T)v;
+}
+
+// Square root of a non-negative squared distance.  fp32: the hardware approximation (1 ulp)
+// refined by one Newton step on the residual, which is within an ulp of the correctly rounded
+// root at a third of its cost; tiny arguments, where the approximation loses bits, take the
+// library routine.
+__device__ __forceinline__ float dist_sqrt(float a) {
+    if (a < 1e-30f) return sqrtf(a);
+    const float s = __builtin_amdgcn_sqrtf(a);
+    const float half_inv = 0.5f * __builtin_amdgcn_rcpf(s);
+    return fmaf(fmaf(-s, s, a), half_inv, s);
+}
+__device__ __forceinline__ double dist_sqrt(double a) { return sqrt(a); }
+
 // distances_t[c, i] = sqrt(sum_f (c_fc - x_fi)^2).  Output bound (k values written per
-// sample).  A thread keeps the features of four consecutive samples in registers (d <= DREG)
-// and walks the centroids through wave-uniform loads, writing one 128-bit store per centroid.
+// sample).  A thread keeps the features of four consecutive samples in registers (d <= DREG);
+// the workgroup's share of the centroids (blockIdx.y: `c_chunk` of them, a multiple of 4) is
+// staged in LDS, and the thread walks it four centroids at a time: one 128-bit broadcast read
+// per feature, sixteen independent sums, one 128-bit store per centroid row.
 template <typename T, int DREG>
 __global__ __launch_bounds__(256) void euclidean_distances_reg_kernel(
     const T* __restrict__ X_t, const T* __restrict__ centroids_t, T* __restrict__ distances_t,
-    int64_t n, int d, int k, int vec_ok) {
+    int64_t n, int d, int k, int vec_ok, int c_chunk) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* cs = reinterpret_cast<T*>(smem_raw);  // [d][c_chunk]
+    const int c_begin = blockIdx.y * c_chunk;
+    for (int idx = threadIdx.x; idx < d * c_chunk; idx += 256) {
+        const int f = idx / c_chunk, c = c_begin + idx % c_chunk;
+        cs[idx] = c < k ? centroids_t[(size_t)f * k + c] : T(0);
+    }
+    __syncthreads();
     const int64_t n_groups = (n + 3) >> 2;
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < n_groups; g += stride) {
@@ -107,22 +155,35 @@ __global__ __launch_bounds__(256) void euclidean_distances_reg_kernel(
                 for (int r = 0; r < 4; ++r) x[f][r] = T(0);
             }
         }
-        for (int c = 0; c < k; ++c) {
-            T acc[4] = {T(0), T(0), T(0), T(0)};
+        for (int c4 = 0; c4 < c_chunk; c4 += 4) {
+            T acc[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[j][r] = T(0);
 #pragma unroll
             for (int f = 0; f < DREG; ++f) {
                 if (f < d) {
-                    const T cv = centroids_t[(size_t)f * k + c];  // wave-uniform
+                    T cv[4];
+                    load4<T>(cs + f * c_chunk, c4, c_chunk, true, cv);  // same address in every lane
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const T diff = cv - x[f][r];
-                        acc[r] = fma(diff, diff, acc[r]);
-                    }
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const T diff = cv[j] - x[f][r];
+                            acc[j][r] = fma(diff, diff, acc[j][r]);
+                        }
                 }
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] = sqrt(acc[r]);
-            store4<T>(distances_t + (size_t)c * n, i0, n, full, acc);
+            for (int j = 0; j < 4; ++j) {
+                const int c = c_begin + c4 + j;
+                if (c < k) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[j][r] = dist_sqrt(acc[j][r]);
+                    store4<T>(distances_t + (size_t)c * n, i0, n, full, acc[j]);
+                }
+            }
         }
     }
 }
@@ -151,7 +212,7 @@ __global__ __launch_bounds__(256) void euclidean_distances_kernel(
             }
 #pragma unroll
             for (int j = 0; j < KC; ++j)
-                if (c0 + j < k) distances_t[(size_t)(c0 + j) * n + i] = sqrt(acc[j]);
+                if (c0 + j < k) distances_t[(size_t)(c0 + j) * n + i] = dist_sqrt(acc[j]);
         }
     }
 }
@@ -192,6 +253,41 @@ int stream_grid(int64_t n) {
 
 extern "C" {
 
+static int32_t inertia_launch(const void* X_t, const void* sample_weight, const void* centroids_t,
+                              const uint32_t* labels, void* out, double* partial, int64_t n, int32_t d, int32_t k,
+                              int32_t dtype, hipStream_t stream) {
+    const bool sum = partial != nullptr;
+    const int grid = stream_grid(kmx_cdiv(n, 4));
+    const size_t es = kmx_dtype_size(dtype);
+    auto al16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
+    const int vec_ok =
+        (n % 4 == 0) && al16(X_t) && (sum || al16(out)) && (sample_weight == nullptr || al16(sample_weight));
+    const size_t lds = (size_t)d * k * es;
+    const bool in_lds = lds <= 48 * 1024;
+#define KMX_INERTIA(T, L, S)                                                                       \
+    hipLaunchKernelGGL((per_sample_inertia_kernel<T, L, S>), dim3(grid), dim3(256), (L) ? lds : 0,  \
+                       stream, (const T*)X_t, (const T*)sample_weight, (const T*)centroids_t,      \
+                       labels, (S) ? nullptr : (T*)out, partial, n, d, k, vec_ok)
+#define KMX_INERTIA_T(T)                                                        \
+    do {                                                                        \
+        if (in_lds && sum) KMX_INERTIA(T, true, true);                          \
+        else if (in_lds) KMX_INERTIA(T, true, false);                           \
+        else if (sum) KMX_INERTIA(T, false, true);                              \
+        else KMX_INERTIA(T, false, false);                                      \
+    } while (0)
+    if (dtype == KMX_F32) KMX_INERTIA_T(float); else KMX_INERTIA_T(double);
+#undef KMX_INERTIA_T
+#undef KMX_INERTIA
+    if (sum) {
+        if (dtype == KMX_F32)
+            hipLaunchKernelGGL((inertia_total_kernel<float>), dim3(1), dim3(256), 0, stream, partial, grid, (float*)out);
+        else
+            hipLaunchKernelGGL((inertia_total_kernel<double>), dim3(1), dim3(256), 0, stream, partial, grid, (double*)out);
+    }
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
 int32_t kmx_per_sample_inertia(const void* X_t, const void* sample_weight, const void* centroids_t,
                                const uint32_t* labels, void* out, int64_t n, int32_t d, int32_t k,
                                int32_t dtype, void* stream_) {
@@ -202,25 +298,28 @@ int32_t kmx_per_sample_inertia(const void* X_t, const void* sample_weight, const
     KMX_REQUIRE_PTR(out);
     if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
     KMX_REQUIRE_DTYPE(dtype);
-    hipStream_t stream = (hipStream_t)stream_;
-    const int grid = stream_grid(kmx_cdiv(n, 4));
-    const size_t es = kmx_dtype_size(dtype);
-    auto al16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
-    const int vec_ok = (n % 4 == 0) && al16(X_t) && al16(out) && (sample_weight == nullptr || al16(sample_weight));
-    const size_t lds = (size_t)d * k * es;
-    const bool in_lds = lds <= 48 * 1024;
-#define KMX_INERTIA(T, L)                                                                         \
-    hipLaunchKernelGGL((per_sample_inertia_kernel<T, L>), dim3(grid), dim3(256), (L) ? lds : 0,     \
-                       stream, (const T*)X_t, (const T*)sample_weight, (const T*)centroids_t,      \
-                       labels, (T*)out, n, d, k, vec_ok)
-    if (dtype == KMX_F32) {
-        if (in_lds) KMX_INERTIA(float, true); else KMX_INERTIA(float, false);
-    } else {
-        if (in_lds) KMX_INERTIA(double, true); else KMX_INERTIA(double, false);
-    }
-#undef KMX_INERTIA
-    KMX_LAUNCH_CHECK();
-    return KMX_OK;
+    return inertia_launch(X_t, sample_weight, centroids_t, labels, out, nullptr, n, d, k, dtype, (hipStream_t)stream_);
+}
+
+size_t kmx_inertia_workspace_bytes(int64_t n) {
+    if (n <= 0) return 0;
+    return kmx_align256((size_t)stream_grid(kmx_cdiv(n, 4)) * sizeof(double));
+}
+
+int32_t kmx_inertia(const void* X_t, const void* sample_weight, const void* centroids_t, const uint32_t* labels,
+                    void* out_total, void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
+                    int32_t dtype, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(centroids_t);
+    KMX_REQUIRE_PTR(labels);
+    KMX_REQUIRE_PTR(out_total);
+    KMX_REQUIRE_PTR(workspace);
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    if (workspace_bytes < kmx_inertia_workspace_bytes(n)) return KMX_ERR_WORKSPACE;
+    return inertia_launch(X_t, sample_weight, centroids_t, labels, out_total, (double*)workspace, n, d, k, dtype,
+                          (hipStream_t)stream_);
 }
 
 int32_t kmx_euclidean_distances(const void* X_t, const void* centroids_t, void* distances_t,
@@ -234,18 +333,30 @@ int32_t kmx_euclidean_distances(const void* X_t, const void* centroids_t, void* 
     hipStream_t stream = (hipStream_t)stream_;
     auto al16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     const int vec_ok = (n % 4 == 0) && al16(X_t) && al16(distances_t);
-    if (dtype == KMX_F32 && d <= 32) {
-        const int grid = stream_grid(kmx_cdiv(n, 4));
+    // register kernel: the centroid range is split over blockIdx.y until there are about six
+    // workgroups per compute unit (a thread's walk over the centroids is one dependent chain)
+    const int64_t wgx = stream_grid(kmx_cdiv(n, 4));
+    int64_t gy = kmx_cdiv((int64_t)kmx_num_cus() * 6, wgx);
+    if (gy > kmx_cdiv(k, 16)) gy = kmx_cdiv(k, 16);
+    if (gy < 1) gy = 1;
+    const int c_chunk = (int)(4 * kmx_cdiv(kmx_cdiv(k, gy), 4));
+    gy = kmx_cdiv(k, c_chunk);
+    const size_t es = kmx_dtype_size(dtype);
+    const size_t lds = (size_t)d * c_chunk * es;
+    const dim3 rgrid((unsigned)wgx, (unsigned)gy);
+    if (dtype == KMX_F32 && d <= 32 && lds <= 64 * 1024) {
         if (d <= 16)
-            hipLaunchKernelGGL((euclidean_distances_reg_kernel<float, 16>), dim3(grid), dim3(256), 0, stream,
-                               (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d, k, vec_ok);
+            hipLaunchKernelGGL((euclidean_distances_reg_kernel<float, 16>), rgrid, dim3(256), lds, stream,
+                               (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d, k, vec_ok,
+                               c_chunk);
         else
-            hipLaunchKernelGGL((euclidean_distances_reg_kernel<float, 32>), dim3(grid), dim3(256), 0, stream,
-                               (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d, k, vec_ok);
-    } else if (dtype == KMX_F64 && d <= 16) {
-        const int grid = stream_grid(kmx_cdiv(n, 4));
-        hipLaunchKernelGGL((euclidean_distances_reg_kernel<double, 16>), dim3(grid), dim3(256), 0, stream,
-                           (const double*)X_t, (const double*)centroids_t, (double*)distances_t, n, d, k, vec_ok);
+            hipLaunchKernelGGL((euclidean_distances_reg_kernel<float, 32>), rgrid, dim3(256), lds, stream,
+                               (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d, k, vec_ok,
+                               c_chunk);
+    } else if (dtype == KMX_F64 && d <= 16 && lds <= 64 * 1024) {
+        hipLaunchKernelGGL((euclidean_distances_reg_kernel<double, 16>), rgrid, dim3(256), lds, stream,
+                           (const double*)X_t, (const double*)centroids_t, (double*)distances_t, n, d, k, vec_ok,
+                           c_chunk);
     } else if (dtype == KMX_F32) {
         hipLaunchKernelGGL((euclidean_distances_kernel<float, 8>), dim3(stream_grid(n)), dim3(256), 0, stream,
                            (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d,

@@ -133,7 +133,7 @@ def _assign(X_t, centroids_t, labels_out, flags=None):
     dc = dcode(X_t)
     flags = _capi.DEFAULT_FLAGS if flags is None else int(flags)
     ws_bytes = lib.kmx_assign_workspace_bytes_for(n, d, k, dc, flags)
-    ws = workspace(ws_bytes, X_t.device)
+    ws = workspace(ws_bytes, X_t.device, tag="assign")
     check(lib.kmx_assign_labels(ptr(X_t), ptr(centroids_t), ptr(labels_out), ptr(ws), ws_bytes, n, d, k,
                                 dc, flags, _capi.current_stream()), "kmx_assign_labels")
 
@@ -148,9 +148,21 @@ def _per_sample_inertia(X_t, sample_weight, centroids_t, labels, out=None):
     return out
 
 
+def _inertia_array(X_t, sample_weight, centroids_t, labels):
+    """1-element numpy array: the weighted sum of squared distances to the assigned centroids
+    (the per-sample values are summed inside the kernel, not written out)."""
+    d, n = X_t.shape
+    k = centroids_t.shape[1]
+    ws_bytes = lib.kmx_inertia_workspace_bytes(n)
+    ws = workspace(ws_bytes, X_t.device, tag="inertia")
+    out = torch.empty(1, dtype=X_t.dtype, device=X_t.device)
+    check(lib.kmx_inertia(ptr(X_t), ptr(sample_weight), ptr(centroids_t), ptr(labels), ptr(out), ptr(ws), ws_bytes,
+                          n, d, k, dcode(X_t), _capi.current_stream()), "kmx_inertia")
+    return out.cpu().numpy()
+
+
 def _inertia(X_t, sample_weight, centroids_t, labels):
-    per_sample = _per_sample_inertia(X_t, sample_weight, centroids_t, labels)
-    return sum_reduction(per_sample).cpu().numpy()[0]
+    return _inertia_array(X_t, sample_weight, centroids_t, labels)[0]
 
 
 def _relocate_empty_clusters(
@@ -263,8 +275,7 @@ def get_labels_inertia(X_t, centroids_t, sample_weight, with_inertia):
     _assign(X_t, centroids_t, assignments_idx)
     if not with_inertia:
         return assignments_idx, None
-    per_sample = _per_sample_inertia(X_t, contiguous(sample_weight), centroids_t, assignments_idx)
-    return assignments_idx, sum_reduction(per_sample).cpu().numpy()
+    return assignments_idx, _inertia_array(X_t, contiguous(sample_weight), centroids_t, assignments_idx)
 
 
 def get_euclidean_distances(X_t, Y_t):

@@ -289,3 +289,26 @@ def test_distances_and_inertia_kernels(cuda, shape):
     _capi.check(lib.kmx_per_sample_inertia(ptr(X_t), None, ptr(C_t), ptr(lab_d), ptr(out), n, d, k,
                                            _capi.dtype_code(X.dtype), _capi.current_stream()), "inertia")
     np.testing.assert_allclose(out.cpu().numpy(), per_sample, rtol=rtol * 5, atol=rtol)
+    # the same kernel with the sum folded in (no per-sample values written)
+    total = drivers._inertia_array(X_t, _dev(w, cuda), C_t, lab_d)
+    assert total.shape == (1,) and total.dtype == dtype
+    np.testing.assert_allclose(total[0], (per_sample * w.astype(np.float64)).sum(), rtol=rtol)
+    total_unit = drivers._inertia_array(X_t, None, C_t, lab_d)
+    np.testing.assert_allclose(total_unit[0], per_sample.sum(), rtol=rtol)
+
+
+def test_distances_with_few_samples_split_the_centroids(cuda):
+    """With few samples the centroid range is split over the second grid dimension (ragged last
+    share, k not a multiple of 4), and exact zeros / tiny distances go through the square root."""
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    rng = np.random.default_rng(5)
+    n, d, k = 2000, 14, 127
+    X = rng.normal(size=(n, d)).astype(np.float32)
+    C = rng.normal(size=(k, d)).astype(np.float32)
+    C[3] = X[10]            # distance exactly 0
+    C[4] = X[11] + 1e-20    # below the fast path's range
+    exact = np.sqrt(((X.astype(np.float64)[:, None, :] - C.astype(np.float64)[None, :, :]) ** 2).sum(axis=2))
+    got = drivers.get_euclidean_distances(_dev(X.T, cuda), _dev(C.T, cuda)).cpu().numpy()
+    np.testing.assert_allclose(got, exact, rtol=1e-5, atol=1e-6)
+    assert got[10, 3] == 0.0 and np.isfinite(got).all()
