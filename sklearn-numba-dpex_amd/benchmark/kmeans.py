@@ -116,13 +116,41 @@ def main(argv=None):
             if reference is None:
                 reference = got
             else:
-                rtol = 1e-4 if dtype == np.float32 else 1e-9
-                mismatch = int((reference["labels"] != got["labels"]).sum())
-                print(f"consistency: {mismatch} of {n} labels differ, "
-                      f"inertia {reference['inertia']:.8g} vs {got['inertia']:.8g}")
-                np.testing.assert_allclose(reference["inertia"], got["inertia"], rtol=rtol)
-                np.testing.assert_allclose(reference["centers"], got["centers"], rtol=1e-2, atol=1e-2)
+                _check_same_fit(X, reference, got, dtype, args.max_iter)
     return 0
+
+
+def _check_same_fit(X, reference, got, dtype, n_iter):
+    """Two providers ran the same iterations from the same centres: inertia within 1e-5 (fp32) /
+    1e-12 (fp64), centres within that tolerance per iteration run (relative to the coordinate,
+    with the centroid's largest coordinate as floor), and labels equal except where the two
+    nearest centres of the reference fit are tied to within ten times the centre tolerance.
+    (The reference compares labels exactly and everything else with assert_allclose's default,
+    and calls its own check unreliable: benchmark/kmeans.py:172-206, 326-327.)"""
+    rtol = 1e-5 if np.dtype(dtype) == np.float32 else 1e-12
+    centres_rtol = rtol * max(1, n_iter)
+    ref_c = np.asarray(reference["centers"], dtype=np.float64)
+    got_c = np.asarray(got["centers"], dtype=np.float64)
+    n = reference["labels"].shape[0]
+    differ = np.flatnonzero(reference["labels"] != got["labels"])
+    print(f"consistency: {differ.size} of {n} labels differ, "
+          f"inertia {reference['inertia']:.8g} vs {got['inertia']:.8g}")
+    np.testing.assert_allclose(got["inertia"], reference["inertia"], rtol=rtol * max(1, n_iter))
+    scale = np.abs(ref_c).max(axis=1, keepdims=True)
+    bound = centres_rtol * np.maximum(np.abs(ref_c), scale)
+    worst = float(np.max(np.abs(got_c - ref_c) / np.maximum(bound, 1e-300)))
+    if worst > 1.0:
+        raise AssertionError(f"cluster centres differ: largest error is {worst:.2f} x the bound (rtol {centres_rtol:g})")
+    if differ.size:
+        if differ.size > max(1, n // 1000):
+            raise AssertionError(f"{differ.size} of {n} labels differ")
+        rows = np.asarray(X, dtype=np.float64)[differ]
+        dist = ((rows[:, None, :] - ref_c[None, :, :]) ** 2).sum(axis=2)
+        at = np.arange(differ.size)
+        gap = np.abs(dist[at, reference["labels"][differ].astype(np.int64)]
+                     - dist[at, got["labels"][differ].astype(np.int64)])
+        if not np.all(gap <= 10.0 * centres_rtol * dist.max(axis=1)):
+            raise AssertionError(f"{differ.size} labels differ and not all of them are ties between two centres")
 
 
 def _to_numpy(value):

@@ -119,7 +119,7 @@ class KMeansEngine(_EngineBase):
             init = self._check_init(init, X)
 
         X_t, X_mean, self.init, self.tol, self.sample_weight_is_uniform = prepare_data_for_lloyd(
-            X.T, init, estimator.tol, sample_weight, estimator.copy_x
+            X.T, init, estimator.tol, sample_weight, estimator.copy_x and not self._owns_X
         )
         if self._is_in_testing_mode and X_mean is not None:
             X_mean = _to_numpy(X_mean)
@@ -263,9 +263,8 @@ class KMeansEngine(_EngineBase):
             if not X_t.is_contiguous():
                 X_t = X_t.contiguous()
                 owns_copy = True
-            elif estimator.copy_x and reset and not owns_copy:
-                X_t = X_t.clone()
         else:
+            owns_copy = True  # the upload below is this engine's own device copy
             X_np = check_array(
                 X,
                 accept_sparse=False,
@@ -282,6 +281,8 @@ class KMeansEngine(_EngineBase):
             X_t = upload(np.ascontiguousarray(X_np.T) if X_np.flags.f_contiguous else X_np, self.device)
             X_t = X_t if X_np.flags.f_contiguous else X_t.T.contiguous()
 
+        # prepare_fit centres the data in place when this buffer is not the caller's (or copy_x is off)
+        self._owns_X = owns_copy
         if reset:
             estimator.n_features_in_ = n_features
             if self._is_in_testing_mode:

@@ -243,6 +243,10 @@ def test_copy_x_false_restores_a_device_input(cuda):
     X_np = X.copy()
     KMeans(n_clusters=3, init=X[:3].copy(), n_init=1, copy_x=True).fit(X_np)
     assert_array_equal(X_np, X)
+    # copy_x=True on a device tensor that could be centred in place: one copy is made, and the
+    # caller's buffer is never written
+    KMeans(n_clusters=3, init=X[:3].copy(), n_init=1, copy_x=True).fit(X_dev)
+    assert_array_equal(X_dev.cpu().numpy(), before)
 
 
 def test_input_validation_errors(cuda):

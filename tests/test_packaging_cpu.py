@@ -54,3 +54,32 @@ def test_built_package_imports_under_its_installed_name(tmp_path):
     lines = proc.stdout.strip().splitlines()
     assert lines[0].startswith(str(pkg)), lines
     assert lines[1].split() == [str(__import__("sklearn_numba_dpex_amd._capi", fromlist=["x"]).ABI_VERSION), "kmeans"]
+
+
+def test_benchmark_consistency_rule():
+    """The benchmark's check between two providers: centres and inertia at 1e-5 per iteration,
+    labels equal except at ties between two centres."""
+    import numpy as np
+    import pytest
+
+    from sklearn_numba_dpex_amd.benchmark.kmeans import _check_same_fit
+
+    rng = np.random.default_rng(0)
+    centers = np.array([[0.0, 0.0], [4.0, 0.0], [0.0, 4.0]], dtype=np.float32)
+    X = (centers[rng.integers(0, 3, 300)] + 0.3 * rng.standard_normal((300, 2))).astype(np.float32)
+    X[0] = [2.0, 0.0]  # exactly between the first two centres
+    labels = ((X[:, None, :] - centers[None]) ** 2).sum(axis=2).argmin(axis=1).astype(np.int32)
+    ref = dict(labels=labels, centers=centers, inertia=10.0)
+    same = dict(labels=labels.copy(), centers=centers * (1 + 2e-6), inertia=10.0 * (1 + 2e-6))
+    _check_same_fit(X, ref, same, np.float32, 1)
+    tie = dict(same, labels=labels.copy())
+    tie["labels"][0] = 1 - labels[0]
+    _check_same_fit(X, ref, tie, np.float32, 1)
+    wrong = dict(same, labels=labels.copy())
+    wrong["labels"][5] = (labels[5] + 1) % 3
+    with pytest.raises(AssertionError, match="not all of them are ties"):
+        _check_same_fit(X, ref, wrong, np.float32, 1)
+    with pytest.raises(AssertionError, match="cluster centres differ"):
+        _check_same_fit(X, ref, dict(same, centers=centers + np.float32(1e-3)), np.float32, 1)
+    with pytest.raises(AssertionError):
+        _check_same_fit(X, ref, dict(same, inertia=10.01), np.float32, 1)
