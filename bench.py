@@ -224,6 +224,26 @@ def gpu_measured_peaks():
         t = timed(lambda: _capi.check(lib.kmx_probe_mfma(kind, 20000, ptr(scratch), ctypes.byref(flops), stream),
                                       "probe_mfma"), 3)
         out[name] = flops.value / t / 1e12
+    # issue slots: ns per loop round (two MFMAs + 2 V vector-ALU instructions per wave, three waves per SIMD)
+    iters = 20000
+    issue = {}
+    for kind, name in ((2, "valu_only"), (0, "mfma_f16"), (1, "mfma_f32")):
+        for v in (0, 8, 16, 32):
+            if kind == 2 and v == 0:
+                continue
+            t = timed(lambda: _capi.check(lib.kmx_probe_issue(kind, v, iters, ptr(scratch), stream), "probe_issue"), 3)
+            issue[f"{name}_valu{v}"] = t * 1e9 / iters
+    per_valu = issue["valu_only_valu32"] / (3 * 64)   # 3 waves x 64 instructions per round
+    out["issue"] = {
+        "what": "ns per loop round of 3 waves on one SIMD, each issuing two MFMAs and 2 V independent v_max3_f32 "
+                "(valuV); hidden = share of the MFMA-only time that disappears when the vector work is added",
+        "ns_per_round": issue,
+        "ns_per_valu_instruction": per_valu,
+        "ns_per_mfma_f16": issue["mfma_f16_valu0"] / 6, "ns_per_mfma_f32": issue["mfma_f32_valu0"] / 6,
+        "mfma_f16_hidden_at_valu16": 1.0 - (issue["mfma_f16_valu16"] - issue["valu_only_valu16"]) / issue["mfma_f16_valu0"],
+        "mfma_f16_hidden_at_valu8": 1.0 - (issue["mfma_f16_valu8"] - issue["valu_only_valu8"]) / issue["mfma_f16_valu0"],
+        "mfma_f32_hidden_at_valu16": 1.0 - (issue["mfma_f32_valu16"] - issue["valu_only_valu16"]) / issue["mfma_f32_valu0"],
+    }
     del src, dst
     return out
 
@@ -542,7 +562,7 @@ def main():
     log(f"[bench] every product in fp32: {all_fp32['ms_per_step']:.4f} ms/iter, fused step "
         f"{kms32[0]:.4f} ms = {all_fp32['frac_of_fp32_peak']:.3f} of fp32 peak")
     peaks = gpu_measured_peaks()
-    log("[bench] measured peaks: " + ", ".join(f"{k2} {v:.1f}" for k2, v in peaks.items() if k2 != "what"))
+    log("[bench] measured peaks: " + ", ".join(f"{k2} {v:.1f}" for k2, v in peaks.items() if isinstance(v, float)))
     hbm_roof["frac_of_measured_peak"] = hbm_roof["achieved"] / peaks["read_GBps"]
     mfma_roof["frac_of_measured_peak"] = mfma_roof["achieved"] / peaks["mfma_f32_TFLOPs"]
     all_fp32["frac_of_measured_fp32_peak"] = all_fp32["fused_step_TFLOPs"] / peaks["mfma_f32_TFLOPs"]

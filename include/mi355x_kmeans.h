@@ -454,6 +454,13 @@ int32_t kmx_probe_copy(const void* src, void* dst, size_t n_bytes, void* stream)
 int32_t kmx_probe_read(const void* src, size_t n_bytes, void* scratch, void* stream);
 int32_t kmx_probe_mfma(int32_t kind, int32_t iters, void* scratch, double* flops_host, void* stream);
 
+/* How matrix-core and vector-ALU instructions share a SIMD's issue slots: `iters` rounds of two
+ * independent MFMAs (kind 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_f32_32x32x2_f32, 2: none) and
+ * 2 * valu_per_mfma (0, 8, 16 or 32) independent v_max3_f32, three waves per SIMD on every SIMD.
+ * The caller times the launch; scratch: 1 MiB.  It has no counterpart in the reference
+ * (benchmarks only). */
+int32_t kmx_probe_issue(int32_t kind, int32_t valu_per_mfma, int32_t iters, void* scratch, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -153,6 +153,7 @@ SIGNATURES = {
     "kmx_probe_copy": (_I32, [_P, _P, _SZ, _P]),
     "kmx_probe_read": (_I32, [_P, _SZ, _P, _P]),
     "kmx_probe_mfma": (_I32, [_I32, _I32, _P, POINTER(c_double), _P]),
+    "kmx_probe_issue": (_I32, [_I32, _I32, _I32, _P, _P]),
 }
 
 

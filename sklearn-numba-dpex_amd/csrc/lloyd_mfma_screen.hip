@@ -403,6 +403,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
 #pragma unroll
                 for (int s = 0; s < NK; ++s) {
                     unsigned int hw[4], lw[4];
+                    // the spare slot's constant (prefetched rows arrive without it)
+                    float x7 = x[s][7][t];
+                    if (HK && s == NK - 1) x7 = h ? hk_x : x7;
                     // Sixteen instructions in ONE statement: between separate statements the
                     // compiler pads every dependency on an assembly result with a wait state
                     // (it must assume a partial register write).  The real rule - a 16-bit write
@@ -430,7 +433,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                         : "=&v"(hw[0]), "=&v"(hw[1]), "=&v"(hw[2]), "=&v"(hw[3]), "=&v"(lw[0]), "=&v"(lw[1]),
                           "=&v"(lw[2]), "=&v"(lw[3])
                         : "v"(x[s][0][t]), "v"(x[s][1][t]), "v"(x[s][2][t]), "v"(x[s][3][t]), "v"(x[s][4][t]),
-                          "v"(x[s][5][t]), "v"(x[s][6][t]), "v"(x[s][7][t]), "s"(xs_sc));
+                          "v"(x[s][5][t]), "v"(x[s][6][t]), "v"(x7), "s"(xs_sc));
                     if (!UPDATE) {
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
@@ -809,7 +812,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const int f = 16 * s + 2 * i + h;
             row_off[s][i] = (uint32_t)(f < d ? f : d - 1) * (uint32_t)n * 4u + (uint32_t)(MC * j) * 4u;
         }
-    auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
+    // (the spare slot's constant is put in where the rows are consumed: a select here would make
+    // the wave wait for loads it has only just requested)
+    auto load_rows_raw = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
         const char* const tile = xbytes + (size_t)wt * (size_t)(TILE * 4);  // wave-uniform
 #pragma unroll
         for (int s = 0; s < NK; ++s)
@@ -819,6 +824,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 dst[s][i][0] = q.x;
                 dst[s][i][1] = q.y;
             }
+    };
+    auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
+        load_rows_raw(wt, dst);
         if (HK) {
             // the spare slot carries the constant whose scaled value is SCR_HK_X1
 #pragma unroll
@@ -848,7 +856,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         uint32_t pl_next = 0u;
         auto request = [&](const int wt_) __attribute__((always_inline)) {
             if (wt_ < n_main) {  // wave-uniform
-                load_rows(wt_, x);
+                load_rows_raw(wt_, x);
                 if (UPDATE) {
                     const int64_t idx = (int64_t)wt_ * TILE + MC * j + h;
                     norm_next = norms[idx];

@@ -80,9 +80,67 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(float* __restrict__ out
     out[(size_t)blockIdx.x * 512 + threadIdx.x] = total;
 }
 
+// How matrix-core and vector-ALU instructions of one SIMD share its issue slots: every loop
+// round issues two independent MFMAs (KIND 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_f32_32x32x2_f32,
+// 2: none) and 2 * VALU independent v_max3_f32 on private registers; three waves per SIMD.
+template <int KIND, int VALU>
+__global__ __launch_bounds__(768) void probe_issue_kernel(float* __restrict__ out, int iters) {
+    const float seed = (float)(threadIdx.x & 63) * 0.001f;
+    v16f c0 = {0}, c1 = {0};
+    v8h ah, bh;
+    for (int i = 0; i < 8; ++i) {
+        ah[i] = (_Float16)(seed + (float)i);
+        bh[i] = (_Float16)(1.0f - seed);
+    }
+    float r[8];
+    for (int i = 0; i < 8; ++i) r[i] = seed + (float)i;
+    for (int it = 0; it < iters; ++it) {
+        if constexpr (KIND == 0) {
+            c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(bh, ah, c1, 0, 0, 0);
+        } else if constexpr (KIND == 1) {
+            c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(seed, 1.0f - seed, c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(1.0f - seed, seed, c1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int q = 0; q < 2 * VALU; ++q)
+            asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(r[q & 7]) : "v"(r[(q + 1) & 7]), "v"(r[(q + 3) & 7]));
+    }
+    float total = 0.0f;
+    for (int i = 0; i < 8; ++i) total += r[i];
+    for (int i = 0; i < 16; ++i) total += c0[i] + c1[i];
+    out[(size_t)blockIdx.x * 768 + threadIdx.x] = total;
+}
+
+template <int KIND>
+bool launch_issue(int valu, unsigned grid, hipStream_t stream, float* out, int iters) {
+    switch (valu) {
+        case 0: hipLaunchKernelGGL((probe_issue_kernel<KIND, 0>), dim3(grid), dim3(768), 0, stream, out, iters); return true;
+        case 8: hipLaunchKernelGGL((probe_issue_kernel<KIND, 8>), dim3(grid), dim3(768), 0, stream, out, iters); return true;
+        case 16: hipLaunchKernelGGL((probe_issue_kernel<KIND, 16>), dim3(grid), dim3(768), 0, stream, out, iters); return true;
+        case 32: hipLaunchKernelGGL((probe_issue_kernel<KIND, 32>), dim3(grid), dim3(768), 0, stream, out, iters); return true;
+        default: return false;
+    }
+}
+
 }  // namespace
 
 extern "C" {
+
+int32_t kmx_probe_issue(int32_t kind, int32_t valu_per_mfma, int32_t iters, void* scratch, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(scratch);
+    if (iters <= 0) return KMX_ERR_BAD_SHAPE;
+    const unsigned grid = (unsigned)kmx_num_cus();
+    hipStream_t stream = (hipStream_t)stream_;
+    bool ok = false;
+    if (kind == 0) ok = launch_issue<0>(valu_per_mfma, grid, stream, (float*)scratch, iters);
+    else if (kind == 1) ok = launch_issue<1>(valu_per_mfma, grid, stream, (float*)scratch, iters);
+    else if (kind == 2) ok = launch_issue<2>(valu_per_mfma, grid, stream, (float*)scratch, iters);
+    if (!ok) return KMX_ERR_BAD_ARGUMENT;
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
 
 int32_t kmx_probe_copy(const void* src, void* dst, size_t n_bytes, void* stream_) {
     KMX_ENTRY();
