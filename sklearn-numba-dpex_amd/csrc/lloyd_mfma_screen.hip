@@ -2,7 +2,7 @@
 // (v_mfma_f32_32x32x16_f16, 16x the rate of the fp32 MFMA) and CERTIFIED per sample.
 //
 // X and the centroids are scaled by one power of two, 2^-a, that brings max|x| into
-// [2^14, 2^15) (exact, and it leaves the arg-max unchanged).  Every scaled value is split into
+// [2^12, 2^13) (exact, and it leaves the arg-max unchanged).  Every scaled value is split into
 // two fp16 numbers, v = hi + lo + rest, by two round-to-nearest conversions (the subtraction
 // v - hi is exact): |rest| <= 2^-22 |v|, or at most 2^-14 in absolute terms should the
 // hardware flush fp16 subnormals.  The score of sample x against centroid c,
@@ -44,6 +44,7 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef double v8d __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
 // Error bound of one approximate score, in scaled units:
 //   (SCR_ERR_SPLIT + r) ||x|| C + r H + SCR_ERR_ABS sqrt(d) (||x|| + C),
@@ -803,7 +804,15 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     // is the scalar address of the tile in row 0 plus a 32-bit byte offset of the lane that does
     // not change from tile to tile (d * n * 4 < 2^32 is a condition of this path): no vector
     // arithmetic and no branch per tile.
-    const char* const xbytes = reinterpret_cast<const char*>(X_t);
+    // The loads are buffer loads: resource descriptor (the array) and tile offset in scalar
+    // registers, the lane's offset in one vector register, so a load needs no address arithmetic.
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(X_t), 0, (int)(uint32_t)((uint64_t)d * (uint64_t)n * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t norms_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(UPDATE ? norms : X_t), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t pl_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(UPDATE ? labels_prev : labels), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
+    const uint32_t own_off = (uint32_t)(MC * j + h) * 4u;  // the lane's own sample inside a tile
     uint32_t row_off[NK][8];
 #pragma unroll
     for (int s = 0; s < NK; ++s)
@@ -815,14 +824,14 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     // (the spare slot's constant is put in where the rows are consumed: a select here would make
     // the wave wait for loads it has only just requested)
     auto load_rows_raw = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
-        const char* const tile = xbytes + (size_t)wt * (size_t)(TILE * 4);  // wave-uniform
+        const uint32_t tile = (uint32_t)wt * (uint32_t)(TILE * 4);  // wave-uniform byte offset in row 0
 #pragma unroll
         for (int s = 0; s < NK; ++s)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float2 q = *reinterpret_cast<const float2*>(tile + row_off[s][i]);
-                dst[s][i][0] = q.x;
-                dst[s][i][1] = q.y;
+                const v2u q = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, row_off[s][i], tile, 0);
+                dst[s][i][0] = __uint_as_float(q[0]);
+                dst[s][i][1] = __uint_as_float(q[1]);
             }
     };
     auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
@@ -858,9 +867,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             if (wt_ < n_main) {  // wave-uniform
                 load_rows_raw(wt_, x);
                 if (UPDATE) {
-                    const int64_t idx = (int64_t)wt_ * TILE + MC * j + h;
-                    norm_next = norms[idx];
-                    pl_next = labels_prev[idx];
+                    const uint32_t tile = (uint32_t)wt_ * (uint32_t)(TILE * 4);
+                    norm_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(norms_rsrc, own_off, tile, 0));
+                    pl_next = __builtin_amdgcn_raw_buffer_load_b32(pl_rsrc, own_off, tile, 0);
                 }
             }
         };
