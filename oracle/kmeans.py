@@ -34,7 +34,8 @@ defect with no stable output to reproduce):
     reduction, common/reductions.py:440-449, squares partial sums again);
   * relocation distances: `relocation="sklearn"` (default) measures to the centroids the
     labels were computed from, `relocation="literal"` to the un-normalised sums
-    (drivers.py:252-259);
+    (drivers.py:252-259).  PARITY UNPINNED for the `literal` branch: nothing outside this
+    file fixes its output (the reference's own relocation test passes with either);
   * far samples are paired with empty clusters canonically: empty ids ascending, samples
     by descending distance then ascending index (the reference's order comes from atomics);
   * kmeans++ `sampler="exact"` searches an fp64 inclusive scan, `sampler="literal"`
