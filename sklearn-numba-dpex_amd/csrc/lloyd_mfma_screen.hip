@@ -80,6 +80,11 @@ constexpr int SCR_WORD_DELTA = 2;
 #ifndef KMX_SCR_PIPE
 #define KMX_SCR_PIPE 1
 #endif
+// The winning group of a full tile is copied under an execution mask that the compare writes
+// directly (one assembly block); 0 restores the compiler's save / branch / restore.
+#ifndef KMX_SCR_CMPX
+#define KMX_SCR_CMPX 1
+#endif
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
 
 struct ScreenLds {
@@ -480,8 +485,36 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             // states an MFMA result needs before a vector-ALU read, which it does not
             // do for operands of inline assembly.
             float m = __builtin_amdgcn_fmed3f(av[g * G], av[g * G + 1], pos_inf);
-            // (one statement: see the conversion above)
             static_assert(G == 8, "three three-operand maxima after the first pair");
+            const v8d ad = __builtin_bit_cast(v8d, av);
+            if constexpr (FULL && KMX_SCR_CMPX) {
+                // One statement (see the conversion above).  Every lane of a full tile is active
+                // here: the compare writes the execution mask itself, the copies of the winning
+                // group run under it and the mask is set back to all lanes - no scalar save /
+                // branch / restore around six instructions that nearly always run anyway (some
+                // lane of 64 improves in almost every group).  Strict: the earlier group keeps a tie.
+                asm volatile(
+                    "v_max3_f32 %[m], %[m], %[v2], %[v3]\n\t"
+                    "v_max3_f32 %[m], %[m], %[v4], %[v5]\n\t"
+                    "v_max3_f32 %[m], %[m], %[v6], %[v7]\n\t"
+                    "v_med3_f32 %[sec], %[bst], %[sec], %[m]\n\t"
+                    "v_cmpx_gt_f32_e32 %[m], %[bst]\n\t"
+                    "v_mov_b32 %[bst], %[m]\n\t"
+                    "v_mov_b32 %[cde], %[cd]\n\t"
+                    "v_mov_b64 %[sa], %[a0]\n\t"
+                    "v_mov_b64 %[sb], %[a1]\n\t"
+                    "v_mov_b64 %[sc], %[a2]\n\t"
+                    "v_mov_b64 %[sd], %[a3]\n\t"
+                    "s_mov_b64 exec, -1"
+                    : [m] "+v"(m), [sec] "+v"(sec), [bst] "+v"(bst), [cde] "+v"(cde), [sa] "+v"(sa), [sb] "+v"(sb),
+                      [sc] "+v"(sc), [sd] "+v"(sd)
+                    : [v2] "v"(av[g * G + 2]), [v3] "v"(av[g * G + 3]), [v4] "v"(av[g * G + 4]), [v5] "v"(av[g * G + 5]),
+                      [v6] "v"(av[g * G + 6]), [v7] "v"(av[g * G + 7]), [cd] "s"(cd), [a0] "v"(ad[g * 4]),
+                      [a1] "v"(ad[g * 4 + 1]), [a2] "v"(ad[g * 4 + 2]), [a3] "v"(ad[g * 4 + 3])
+                    : "vcc");
+                return;
+            }
+            // (one statement: see the conversion above)
             asm("v_max3_f32 %0, %0, %2, %3\n\t"
                 "v_max3_f32 %0, %0, %4, %5\n\t"
                 "v_max3_f32 %0, %0, %6, %7\n\t"
@@ -493,7 +526,6 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             if (m > bst) {
                 bst = m;
                 cde = cd;
-                const v8d ad = __builtin_bit_cast(v8d, av);
                 asm volatile("v_mov_b64 %0, %1" : "+v"(sa) : "v"(ad[g * 4]));
                 asm volatile("v_mov_b64 %0, %1" : "+v"(sb) : "v"(ad[g * 4 + 1]));
                 asm volatile("v_mov_b64 %0, %1" : "+v"(sc) : "v"(ad[g * 4 + 2]));
