@@ -250,6 +250,19 @@ int32_t kmx_inertia(const void* X_t, const void* sample_weight, const void* cent
                     size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t dtype,
                     void* stream);
 
+/* Labels and the weighted inertia of that labelling in one call: kmx_assign_labels followed by
+ * kmx_inertia, except that where the screened label kernel applies (fp32, d <= 32) X is read
+ * once - the kernel sums w_i ||x_i - c_label_i||^2 of its samples on the way.  sample_weight may
+ * be NULL (unit weights).  out_total: one element of the compute dtype.  Replaces
+ * get_labels_inertia with with_inertia=True and the final E-step of a fit
+ * (kmeans/drivers.py:356-391, 630-699). */
+size_t kmx_assign_inertia_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype,
+                                          uint32_t flags);
+int32_t kmx_assign_labels_inertia(const void* X_t, const void* sample_weight,
+                                  const void* centroids_t, uint32_t* labels, void* out_total,
+                                  void* workspace, size_t workspace_bytes, int64_t n, int32_t d,
+                                  int32_t k, int32_t dtype, uint32_t flags, void* stream);
+
 /* distances_t (k, n): sqrt(sum_f (c_f - x_f)^2).  Replaces
  * make_compute_euclidean_distances_fixed_window_kernel
  * (kmeans/kernels/compute_euclidean_distances.py:15-161). */

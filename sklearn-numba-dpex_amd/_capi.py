@@ -118,6 +118,8 @@ SIGNATURES = {
     "kmx_per_sample_inertia": (_I32, [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_inertia_workspace_bytes": (_SZ, [_I64]),
     "kmx_inertia": (_I32, [_P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _P]),
+    "kmx_assign_inertia_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _U32]),
+    "kmx_assign_labels_inertia": (_I32, [_P, _P, _P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _U32, _P]),
     "kmx_euclidean_distances": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_relocate_empty_clusters": (_I32, [_P, _P, _P, _P, _P, _I32, _P, _P, _P, _I64, _I32, _I32, _I32, _P]),
     "kmx_rng_init_states": (_I32, [ctypes.c_uint64, _I32, _I32, _P]),

@@ -251,6 +251,15 @@ int stream_grid(int64_t n) {
 
 }  // namespace
 
+int32_t kmx_inertia_total_launch(const double* partial, int count, void* out, int32_t dtype, hipStream_t stream) {
+    if (dtype == KMX_F32)
+        hipLaunchKernelGGL((inertia_total_kernel<float>), dim3(1), dim3(256), 0, stream, partial, count, (float*)out);
+    else
+        hipLaunchKernelGGL((inertia_total_kernel<double>), dim3(1), dim3(256), 0, stream, partial, count, (double*)out);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
 extern "C" {
 
 static int32_t inertia_launch(const void* X_t, const void* sample_weight, const void* centroids_t,

@@ -1054,4 +1054,51 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     return KMX_OK;
 }
 
+// Workspace of kmx_assign_labels_inertia: the label kernel's (with room for the wide path's list),
+// then 8 fp64 partial sums per compute unit or what kmx_inertia wants, whichever is more.
+static size_t assign_inertia_partials_bytes(int64_t n) {
+    const size_t a = (size_t)kmx_num_cus() * 8 * sizeof(double);
+    const size_t b = kmx_inertia_workspace_bytes(n);
+    return kmx_align256(a > b ? a : b);
+}
+
+size_t kmx_assign_inertia_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags) {
+    const size_t a = kmx_assign_workspace_bytes_for(n, d, k, dtype, flags);
+    if (a == 0) return 0;
+    return kmx_align256(a) + assign_inertia_partials_bytes(n);
+}
+
+int32_t kmx_assign_labels_inertia(const void* X_t, const void* sample_weight, const void* centroids_t,
+                                  uint32_t* labels, void* out_total, void* workspace, size_t workspace_bytes,
+                                  int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(X_t);
+    KMX_REQUIRE_PTR(centroids_t);
+    KMX_REQUIRE_PTR(labels);
+    KMX_REQUIRE_PTR(out_total);
+    KMX_REQUIRE_PTR(workspace);
+    if (n <= 0 || d <= 0 || k <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    if (!kmx_flags_valid(flags)) return KMX_ERR_BAD_ARGUMENT;
+    const size_t need = kmx_assign_inertia_workspace_bytes(n, d, k, dtype, flags);
+    if (need == 0 || workspace_bytes < need) return KMX_ERR_WORKSPACE;
+    const size_t assign_bytes = kmx_align256(kmx_assign_workspace_bytes_for(n, d, k, dtype, flags));
+    char* ws = (char*)workspace;
+    double* partial = (double*)(ws + assign_bytes);
+    hipStream_t stream = (hipStream_t)stream_;
+    const LloydLayout L = lloyd_layout(n, d, k, dtype, flags);
+    if (dtype == KMX_F32 && L.screen) {
+        // one pass over X: the screened label kernel sums the inertia on the way
+        int n_partials = 0;
+        const int32_t rc = kmx_assign_labels_inertia_mfma_screen(X_t, sample_weight, centroids_t, labels, partial,
+                                                                 &n_partials, n, d, k, L.wgs_per_cu, stream);
+        if (rc != KMX_OK) return rc;
+        return kmx_inertia_total_launch(partial, n_partials, out_total, dtype, stream);
+    }
+    const int32_t rc = kmx_assign_labels(X_t, centroids_t, labels, workspace, assign_bytes, n, d, k, dtype, flags, stream_);
+    if (rc != KMX_OK) return rc;
+    return kmx_inertia(X_t, sample_weight, centroids_t, labels, out_total, partial, assign_inertia_partials_bytes(n), n,
+                       d, k, dtype, stream_);
+}
+
 }  // extern "C"

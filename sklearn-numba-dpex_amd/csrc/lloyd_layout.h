@@ -176,6 +176,11 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
 // labels only, screened the same way (scale from the centroids, norms taken per tile)
 int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);
+int32_t kmx_assign_labels_inertia_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
+                                              uint32_t* labels, double* inertia_partial, int* n_partials,
+                                              int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);
+// out[0] = sum of `count` fp64 partial sums, in order (inertia_distances.hip)
+int32_t kmx_inertia_total_launch(const double* partial, int count, void* out, int32_t dtype, hipStream_t stream);
 int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream);
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,

@@ -173,14 +173,21 @@ __device__ __forceinline__ uint32_t redo_column_fp32(ColumnRows rows, const floa
     return (uint32_t)bc;
 }
 
-template <int NK, bool UPDATE, bool HK>
+// INERTIA (labels only): the kernel also sums w_i ||x_i - c_label_i||^2 over its samples, in fp32
+// per sample (the lane pair of a sample each takes every other feature) and fp64 across samples,
+// into inertia_partial[blockIdx.x].  sample_weight may be null (unit weights).  The rows of a tile
+// are then still needed at its end, so the next tile's are requested there and not while the
+// tile is scored.
+template <int NK, bool UPDATE, bool HK, bool INERTIA = false>
 __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2) void lloyd_screen_kernel(
     const float* __restrict__ X_t, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
     const unsigned int* __restrict__ absmax, const int* __restrict__ q_exp,
     unsigned long long* __restrict__ gsum, uint32_t* __restrict__ uncertain_count,
-    const float* __restrict__ norms, int64_t n, int d, int k, int vec_ok) {
+    const float* __restrict__ norms, int64_t n, int d, int k, int vec_ok,
+    double* __restrict__ inertia_partial = nullptr) {
+    static_assert(!(UPDATE && INERTIA), "the inertia rides with the labels-only kernel");
     if (UPDATE && status->state != KMX_RUNNING) return;
 
     constexpr int WAVES = scr_waves(NK), THREADS = 64 * WAVES;
@@ -345,6 +352,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     const int n_wtiles = (int)((n + TILE - 1) / TILE);  // n < 2^29: tile and sample indices fit 32 bits
     unsigned int changed = 0;
     unsigned int n_uncertain = 0;  // wave-uniform
+    double inertia_lane = 0.0;     // INERTIA: the lane's share of the weighted sum
 
     // uncertain when best - second <= thr_x * ||x|| + thr_0: twice the error bound, with a
     // margin for the rounding of the bound itself and of the hardware square root
@@ -452,7 +460,12 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 }
             }
         }
-        refill();
+        if constexpr (!INERTIA) refill();
+        // (INERTIA: the owner's weight, wanted at the end of the tile)
+        float w_mine = 1.0f;
+        if constexpr (INERTIA) {
+            if (sample_weight != nullptr && in_range && owner) w_mine = sample_weight[my_idx];
+        }
 
         // Running arg-max by groups of G accumulator registers, plus the second largest of
         // the group maxima (the median of best, second and the new maximum).
@@ -753,7 +766,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                         for (int i = 0; i < 8; ++i) entry[16 * s + 2 * i + h] = __float_as_uint(xr[s][i][t]);
                     if (h == 0) {
                         const int64_t idx_t = i0 + t;
-                        entry[Q_WEIGHT] = UPDATE ? __float_as_uint(sample_weight[idx_t]) : 0u;
+                        entry[Q_WEIGHT] = (UPDATE || (INERTIA && sample_weight != nullptr))
+                                              ? __float_as_uint(sample_weight[idx_t])
+                                              : __float_as_uint(1.0f);
                         entry[Q_INDEX] = (uint32_t)idx_t;
                         entry[Q_PREV] = UPDATE ? labels_prev[idx_t] : 0u;
                     }
@@ -763,6 +778,37 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         }
 
         if (in_range && owner) labels[my_idx] = lab_mine;
+
+        if constexpr (INERTIA) {
+            // both columns' labels in every lane: the lane takes its features of both samples,
+            // in feature order from an fp32 copy of the centroids in LDS; a sample's two halves
+            // are added by its owner.  Queued samples are added when the queue is worked off.
+            uint32_t lab[NC];
+            const auto ll = __builtin_amdgcn_permlane32_swap(lab_mine, lab_mine, false, false);
+            lab[0] = ll[0];
+            if (NC == 2) lab[NC - 1] = ll[1];
+            float part[NC];
+#pragma unroll
+            for (int t = 0; t < NC; ++t) {
+                part[t] = 0.0f;
+                const float* ccol = ct + (lab[t] < (uint32_t)kp ? lab[t] : 0u);
+#pragma unroll
+                for (int s = 0; s < NK; ++s)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int f = 16 * s + 2 * i + h;
+                        if (f < d) {
+                            const float diff = x[s][i][t] - ccol[f * kp];
+                            part[t] = fmaf(diff, diff, part[t]);
+                        }
+                    }
+            }
+            const auto qq = __builtin_amdgcn_permlane32_swap(__float_as_uint(part[0]), __float_as_uint(part[NC - 1]),
+                                                             false, false);
+            const float sq_mine = __uint_as_float(qq[0]) + __uint_as_float(qq[1]);
+            if (in_range && owner && !queued_mine) inertia_lane += (double)(sq_mine * w_mine);
+            refill();
+        }
 
         if (UPDATE) {
             const bool counted_mine = in_range && owner && !queued_mine;
@@ -1040,6 +1086,15 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 labels[sample] = (uint32_t)bc;
                 if (UPDATE) changed += entry[Q_PREV] != (uint32_t)bc ? 1u : 0u;
             }
+            if constexpr (INERTIA) {
+                float sq = 0.0f;
+                if (lane < d) {
+                    const float diff = xe[lane] - ct[lane * kp + bc];
+                    sq = diff * diff;
+                }
+                sq = kmx_wave_sum<float>(sq);
+                if (lane == 0) inertia_lane += (double)(sq * __uint_as_float(entry[Q_WEIGHT]));
+            }
             if (UPDATE) {
                 // lane f adds feature f, lane d the weight: the same fixed-point terms as above;
                 // when the sums are only corrected, a sample that stays in its cluster adds
@@ -1059,6 +1114,19 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
 
     if (UPDATE && changed) atomicAdd(&changed_block, changed);
     if (lane == 0 && n_uncertain) atomicAdd(&uncertain_block, n_uncertain);
+    if constexpr (INERTIA) {
+        // wave totals in order, then the waves in order
+        const double wsum = kmx_wave_sum<double>(inertia_lane);
+        double* wave_tot = reinterpret_cast<double*>(wave_key);  // the queue's keys are no longer needed
+        __syncthreads();
+        if (lane == 0) wave_tot[wave] = wsum;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double total = 0.0;
+            for (int w2 = 0; w2 < WAVES; ++w2) total += wave_tot[w2];
+            inertia_partial[blockIdx.x] = total;
+        }
+    }
     __syncthreads();
     if (threadIdx.x == 0 && uncertain_block && uncertain_count != nullptr)
         atomicAdd(uncertain_count, uncertain_block);
@@ -1252,11 +1320,12 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags) {
 }
 
 namespace {
-template <bool UPDATE>
+template <bool UPDATE, bool INERTIA = false>
 int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, const uint32_t* labels_prev,
                       uint32_t* labels, kmx_lloyd_status* status, const unsigned int* absmax,
                       const int* q_exp, unsigned long long* gsum, uint32_t* uncertain_count,
-                      const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
+                      const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream,
+                      double* inertia_partial = nullptr, int* grid_out = nullptr) {
     if (!kmx_mfma_screen_fits(n, d, k)) return KMX_ERR_UNSUPPORTED;
     const int nk = (d + 15) / 16;
     const int waves = scr_waves(nk);
@@ -1278,14 +1347,14 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
     do {                                                                                                    \
         if (lds > 64 * 1024) {                                                                              \
             const hipError_t e = hipFuncSetAttribute(                                                       \
-                reinterpret_cast<const void*>(&lloyd_screen_kernel<NK_, UPDATE, HK_>),                      \
+                reinterpret_cast<const void*>(&lloyd_screen_kernel<NK_, UPDATE, HK_, INERTIA>),             \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                      \
             if (e != hipSuccess) return (int32_t)e;                                                         \
         }                                                                                                   \
-        hipLaunchKernelGGL((lloyd_screen_kernel<NK_, UPDATE, HK_>), dim3((unsigned)grid),                   \
+        hipLaunchKernelGGL((lloyd_screen_kernel<NK_, UPDATE, HK_, INERTIA>), dim3((unsigned)grid),          \
                            dim3(64 * scr_waves(NK_)), lds, stream, (const float*)X_t, (const float*)w,      \
                            (const float*)centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,     \
-                           uncertain_count, norms, n, d, k, vec_ok);                                        \
+                           uncertain_count, norms, n, d, k, vec_ok, inertia_partial);                       \
     } while (0)
     if (nk == 1) {
         if (hk) KMX_SCR_LAUNCH(1, true); else KMX_SCR_LAUNCH(1, false);
@@ -1294,6 +1363,7 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
     }
 #undef KMX_SCR_LAUNCH
     KMX_LAUNCH_CHECK();
+    if (grid_out) *grid_out = (int)grid;
     return KMX_OK;
 }
 }  // namespace
@@ -1318,6 +1388,15 @@ int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, 
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
     return launch_screen<false>(X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr, nullptr,
                                 nullptr, nullptr, nullptr, n, d, k, wgs_per_cu, stream);
+}
+
+// The same with the weighted inertia of the labelling summed on the way: one fp64 partial sum per
+// workgroup in inertia_partial (room for 8 per compute unit), *n_partials receives how many.
+int32_t kmx_assign_labels_inertia_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
+                                              uint32_t* labels, double* inertia_partial, int* n_partials,
+                                              int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
+    return launch_screen<false, true>(X_t, w, centroids_t, nullptr, labels, nullptr, nullptr, nullptr, nullptr,
+                                      nullptr, nullptr, n, d, k, wgs_per_cu, stream, inertia_partial, n_partials);
 }
 
 // Diagnostics of the screen: approximate scores and error bounds as the fused step forms them.

@@ -122,8 +122,7 @@ def lloyd(
     # labels for the final centroids and the exact inertia (kmeans/drivers.py:356-391)
     best = cent[n_iteration % 2]
     assignments_idx = labels[0]
-    _assign(X_t, best, assignments_idx, flags)
-    inertia = _inertia(X_t, sample_weight, best, assignments_idx)
+    inertia = _assign_with_inertia(X_t, sample_weight, best, assignments_idx, flags)[0]
     return assignments_idx, inertia, best, n_iteration
 
 
@@ -136,6 +135,22 @@ def _assign(X_t, centroids_t, labels_out, flags=None):
     ws = workspace(ws_bytes, X_t.device, tag="assign")
     check(lib.kmx_assign_labels(ptr(X_t), ptr(centroids_t), ptr(labels_out), ptr(ws), ws_bytes, n, d, k,
                                 dc, flags, _capi.current_stream()), "kmx_assign_labels")
+
+
+def _assign_with_inertia(X_t, sample_weight, centroids_t, labels_out, flags=None):
+    """Labels into `labels_out` and the weighted inertia of that labelling as a 1-element numpy
+    array, in one library call (one pass over X where the screened label kernel applies)."""
+    d, n = X_t.shape
+    k = centroids_t.shape[1]
+    dc = dcode(X_t)
+    flags = _capi.DEFAULT_FLAGS if flags is None else int(flags)
+    ws_bytes = lib.kmx_assign_inertia_workspace_bytes(n, d, k, dc, flags)
+    ws = workspace(ws_bytes, X_t.device, tag="assign_inertia")
+    out = torch.empty(1, dtype=X_t.dtype, device=X_t.device)
+    check(lib.kmx_assign_labels_inertia(ptr(X_t), ptr(sample_weight), ptr(centroids_t), ptr(labels_out), ptr(out),
+                                        ptr(ws), ws_bytes, n, d, k, dc, flags, _capi.current_stream()),
+          "kmx_assign_labels_inertia")
+    return out.cpu().numpy()
 
 
 def _per_sample_inertia(X_t, sample_weight, centroids_t, labels, out=None):
@@ -272,10 +287,10 @@ def get_labels_inertia(X_t, centroids_t, sample_weight, with_inertia):
     centroids_t = contiguous(centroids_t)
     n = X_t.shape[1]
     assignments_idx = torch.empty(n, dtype=torch.int32, device=X_t.device)
-    _assign(X_t, centroids_t, assignments_idx)
     if not with_inertia:
+        _assign(X_t, centroids_t, assignments_idx)
         return assignments_idx, None
-    return assignments_idx, _inertia_array(X_t, contiguous(sample_weight), centroids_t, assignments_idx)
+    return assignments_idx, _assign_with_inertia(X_t, contiguous(sample_weight), centroids_t, assignments_idx)
 
 
 def get_euclidean_distances(X_t, Y_t):

@@ -608,3 +608,44 @@ def test_many_ties_stay_affordable(cuda):
     assert int(labels.max()) == 0
     print(f"usual {usual:.3f} ms, every sample tied {tied:.3f} ms")
     assert tied < 10 * usual + 0.5
+
+
+@pytest.mark.parametrize("shape", [(60_001, 14, 127, np.float32), (20_000, 16, 64, np.float32), (9_000, 20, 40, np.float32),
+                                   (5_000, 1, 16, np.float32), (70_000, 9, 300, np.float32),
+                                   (4_000, 40, 20, np.float32), (3_000, 7, 5, np.float32), (6_000, 12, 30, np.float64)])
+@pytest.mark.parametrize("weighted", [True, False])
+def test_labels_and_inertia_in_one_call(cuda, shape, weighted):
+    """kmx_assign_labels_inertia: the labels of kmx_assign_labels and the inertia of kmx_inertia on
+    them, on shapes the screened kernel takes in one pass over X (one and two K steps, odd d, d = 1,
+    a ragged last tile, more than 64 KB of LDS) and on shapes that fall back to the two calls (wide,
+    tiny k, fp64); samples the screen cannot certify (duplicate centroids) included."""
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    def _dev(a, device):
+        return torch.as_tensor(np.ascontiguousarray(a), device=device)
+
+    n, d, k, dtype = shape
+    rng = np.random.default_rng(n + d + k)
+    centers = rng.normal(size=(k, d)).astype(dtype) * 3
+    centers[1] = centers[0]  # every sample of these two clusters is tied: the fp32 route
+    X = (centers[rng.integers(0, k, n)] + rng.normal(size=(n, d))).astype(dtype)
+    w = rng.uniform(0.5, 2.0, n).astype(dtype) if weighted else None
+    X_t, C_t = _dev(X.T, cuda), _dev(centers.T, cuda)
+    w_d = _dev(w, cuda) if weighted else None
+
+    labels = torch.empty(n, dtype=torch.int32, device=cuda)
+    total = drivers._assign_with_inertia(X_t, w_d, C_t, labels)
+    assert total.shape == (1,) and total.dtype == dtype
+
+    ref_labels = torch.empty(n, dtype=torch.int32, device=cuda)
+    drivers._assign(X_t, C_t, ref_labels)
+    np.testing.assert_array_equal(labels.cpu().numpy(), ref_labels.cpu().numpy())
+    two_calls = drivers._inertia_array(X_t, w_d, C_t, ref_labels)
+    rtol = 1e-5 if dtype == np.float32 else 1e-12
+    np.testing.assert_allclose(total[0], two_calls[0], rtol=rtol)
+    got = labels.cpu().numpy().astype(np.int64)
+    exact = ((X.astype(np.float64) - centers.astype(np.float64)[got]) ** 2).sum(axis=1)
+    exact = float((exact * (w.astype(np.float64) if weighted else 1.0)).sum())
+    np.testing.assert_allclose(float(total[0]), exact, rtol=rtol)
