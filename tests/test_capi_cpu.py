@@ -181,6 +181,11 @@ def test_bad_arguments_are_rejected_without_a_device():
     assert lib.kmx_assign_labels(p, p, NULL, p, 4096, 10, 2, 2, 0, 0, NULL) == -1
     assert lib.kmx_assign_labels(p, p, p, p, 4096, 10, 2, 2, 0, 0x30, NULL) == -5
     assert lib.kmx_per_sample_inertia(p, NULL, p, p, p, 0, 2, 2, 0, NULL) == -2
+    assert lib.kmx_inertia(p, NULL, p, p, p, p, 8, 0, 2, 2, 0, NULL) == -2
+    assert lib.kmx_inertia(p, NULL, p, p, p, NULL, 1 << 20, 10, 2, 2, 0, NULL) == -1
+    assert lib.kmx_assign_labels_inertia(p, NULL, p, p, p, p, 16, 1000, 14, 127, 0, 0, NULL) == -4
+    assert lib.kmx_assign_labels_inertia(p, NULL, p, p, NULL, p, 1 << 30, 1000, 14, 127, 0, 0, NULL) == -1
+    assert lib.kmx_assign_inertia_workspace_bytes(1000, 14, 127, 0, 0) > lib.kmx_assign_workspace_bytes_for(1000, 14, 127, 0, 0)
     assert lib.kmx_euclidean_distances(p, p, p, 10, 2, 2, 5, NULL) == -3
     assert lib.kmx_topk_idx(p, p, 5, 10, p, 4096, 0, NULL) == -5      # k > n
     assert lib.kmx_topk_idx(p, p, 50, 10, p, 8, 0, NULL) == -4

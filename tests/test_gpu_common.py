@@ -135,6 +135,26 @@ def test_topk_dense_threshold_bucket_and_signed_zeros(cuda, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_topk_edges(cuda, dtype):
+    """k = n, a single value, infinities, and more rows than one grid dimension holds."""
+    from sklearn_numba_dpex_amd.common.topk import topk, topk_idx
+
+    rng = np.random.default_rng(9)
+    v = rng.normal(size=37).astype(dtype)
+    np.testing.assert_array_equal(topk_idx(_dev(v, cuda), 37).cpu().numpy(), ok.top_k_indices(v, 37))
+    np.testing.assert_array_equal(topk_idx(_dev(v[:1], cuda), 1).cpu().numpy(), [0])
+    w = v.copy()
+    w[[3, 20]] = np.inf
+    w[[5, 6]] = -np.inf
+    np.testing.assert_array_equal(topk_idx(_dev(w, cuda), 4).cpu().numpy(), ok.top_k_indices(w, 4))
+    np.testing.assert_array_equal(topk(_dev(w, cuda), 37).cpu().numpy()[-2:], [-np.inf, -np.inf])
+    many = rng.normal(size=(70_000, 5)).astype(dtype)  # 70 000 rows: two slices of the grid
+    got = topk_idx(_dev(many, cuda), 2).cpu().numpy()
+    want = np.argsort(-many, axis=1, kind="stable")[:, :2]
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_topk_large_with_ties_and_negatives(cuda, dtype):
     from sklearn_numba_dpex_amd.common.topk import topk_idx
 
