@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Lloyd throughput of the MI355X KMeans engine on one GPU.
 
-Workload (BASELINE.json configs[1]): fp32 X of shape 5,000,000 x 14 from 127 Gaussian blobs
+Workload (the second of the frozen configurations, configs[1]): fp32 X of shape 5,000,000 x 14 from 127 Gaussian blobs
 (seed 1), k = 127, random-row init, sample weights uniform in [0.5, 1.5], tol = 0.
 A "step" is one Lloyd iteration (fused assignment + partial sums, reduction, finalisation)
 with X, the weights and the centroids already resident in HBM.
