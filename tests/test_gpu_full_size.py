@@ -166,3 +166,39 @@ def test_kmeanspp_first_centres_match_oracle_at_full_n(cuda):
     seed64 = orng.seed_from_random_state(np.random.RandomState(cfg["seed"]))
     _, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact")
     np.testing.assert_array_equal(idx.cpu().numpy(), ref_idx)
+
+
+def test_score_path_and_topk_at_full_size(cuda):
+    """configs[1] at full size: labels and inertia in one pass equal the two-pass results (labels
+    bit for bit, inertia to 1e-5 and to an exact fp64 sum on a slice-free formula), and the
+    top-k of the 5e6 per-sample values - unique values, then heavy ties - equals a host sort."""
+    import torch
+
+    from sklearn_numba_dpex_amd.common.topk import topk, topk_idx
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    cfg = datasets.config2()
+    X, init, w = cfg["X"], cfg["init"], cfg["sample_weight"]
+    n = X.shape[0]
+    X_t = torch.as_tensor(X, device=cuda).T.contiguous()
+    C_t = torch.as_tensor(np.ascontiguousarray(init.T), device=cuda)
+    w_d = torch.as_tensor(w, device=cuda)
+    labels = torch.empty(n, dtype=torch.int32, device=cuda)
+    total = drivers._assign_with_inertia(X_t, w_d, C_t, labels)
+    ref = torch.empty(n, dtype=torch.int32, device=cuda)
+    drivers._assign(X_t, C_t, ref)
+    assert torch.equal(labels, ref)
+    per_sample = drivers._per_sample_inertia(X_t, w_d, C_t, ref)
+    exact = float(per_sample.double().sum())
+    assert abs(float(total[0]) - exact) <= 1e-5 * exact
+    assert abs(float(drivers._inertia_array(X_t, w_d, C_t, ref)[0]) - exact) <= 1e-5 * exact
+
+    host = per_sample.cpu().numpy()
+    for k in (1, 16, 127):
+        want = ok.top_k_indices(host, k)
+        np.testing.assert_array_equal(topk_idx(per_sample, k).cpu().numpy(), want)
+        np.testing.assert_array_equal(topk(per_sample, k).cpu().numpy(), host[want])
+    tied = torch.floor(per_sample)  # a few hundred distinct values: every threshold is a tie
+    host = tied.cpu().numpy()
+    for k in (16, 1000):
+        np.testing.assert_array_equal(topk_idx(tied, k).cpu().numpy(), ok.top_k_indices(host, k))
