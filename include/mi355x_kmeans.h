@@ -142,9 +142,11 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
  * make_centroid_shifts_kernel (kmeans/kernels/utils.py:79-110) and the loop body of
  * lloyd(), kmeans/drivers.py:188-343.
  *   X_rowmajor       IN   (n, d)  optional (may be NULL) row-major copy of the same data; used
- *                                 only by the wide fp32 path (plan.variant == 42),
- *                                 which then sums each cluster's rows instead of issuing one
- *                                 global atomic per (sample, feature)
+ *                                 by the wide fp32 path (plan.variant == 42), which then sums
+ *                                 each cluster's rows instead of issuing one global atomic per
+ *                                 (sample, feature), and by the bucketed sums (plan.variant
+ *                                 3, 13 or 53), which read whole rows from it instead of
+ *                                 gathering the feature-major array
  *   centroids_t      IN   (d, k)  centroids the labels are computed from: the array given to
  *                                 kmx_lloyd_init for the first iteration, then the
  *                                 new_centroids_t of the previous one (the workspace holds a

@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
     const T* __restrict__ half_norms, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, T* __restrict__ partial, kmx_lloyd_status* __restrict__ status,
     int64_t n, int d, int k, int dpad, int n_copies, int vec_ok) {
-    if (ACC != ACC_NONE && status->state != KMX_RUNNING) return;
+    if (status != nullptr && status->state != KMX_RUNNING) return;
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* acc = reinterpret_cast<T*>(smem_raw);
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     T* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k,
     int n_copies) {
-    if (ACC != ACC_NONE && status->state != KMX_RUNNING) return;
+    if (status != nullptr && status->state != KMX_RUNNING) return;
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* acc = reinterpret_cast<T*>(smem_raw);
@@ -547,7 +547,7 @@ __global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words)
 
 // Workgroups of a vector-ALU fused step (also the number of partial slots it fills).
 int lloyd_fused_grid(const LloydLayout& L, int64_t n, int d, int dtype) {
-    if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n, L.wgs_per_cu, L.cols);
+    if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n, d, L.wgs_per_cu, L.cols, L.partial_slots());
     const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype) : 2;
     const int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
     const int cap = L.grid_cap(kmx_num_cus());
@@ -574,7 +574,8 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_MFMA_F64) {
         (void)kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
-                                      status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, stream);
+                                      status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, L.partial_slots(),
+                                      stream);
     } else if (L.variant == KMX_VARIANT_REGISTER) {
 #define KMX_REG_CASE(DR, RR)                                                                    \
     launch_reg<T, DR, RR, ACC>(L, X_t, w, cpack, half_norms, labels_prev, labels, partial, status, \
@@ -630,6 +631,14 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
         }
         gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
         q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
+    } else if (L.acc_mode == KMX_ACC_BUCKET) {
+        launch_fused<T, ACC_NONE>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
+                                  partial, status, n, d, k, stream);
+        KMX_LAUNCH_CHECK();
+        const int32_t rc = kmx_lloyd_bucket_sums(X_t, X_rowmajor, w, labels_prev, labels, partial, status,
+                                                 ws + L.off_bucket, n, d, k,
+                                                 sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
+        if (rc != KMX_OK) return rc;
     } else if (L.acc_mode == ACC_LDS) {
         launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
                                  partial, status, n, d, k, stream);
@@ -647,7 +656,7 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     const bool small_tail = gsum == nullptr && (size_t)items * sizeof(T) <= 48 * 1024;
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)reduce_grid), dim3(256), 0,
                        stream, partial, n_partials_used,
-                       (L.acc_mode == ACC_GLOBAL && gsum == nullptr) ? 1 : 0,
+                       ((L.acc_mode == ACC_GLOBAL || L.acc_mode == KMX_ACC_BUCKET) && gsum == nullptr) ? 1 : 0,
                        (T*)new_centroids_t, (T*)sizes, empty_clusters, status, d, k, gsum, q_exp,
                        small_tail ? 0 : 1);
     KMX_LAUNCH_CHECK();
@@ -825,7 +834,12 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
                            (uint32_t*)(ws + L.off_wscreen), (size_t)64);
         KMX_LAUNCH_CHECK();
     }
-    if (L.acc_mode == ACC_GLOBAL && L.partial_bytes > 0) {
+    if (L.acc_mode == KMX_ACC_BUCKET) {
+        hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(4), dim3(256), 0, stream,
+                           (uint32_t*)(ws + L.off_bucket), (size_t)k);
+        KMX_LAUNCH_CHECK();
+    }
+    if ((L.acc_mode == ACC_GLOBAL || L.acc_mode == KMX_ACC_BUCKET) && L.partial_bytes > 0) {
         const size_t words = L.partial_bytes / 4;
         hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1024), dim3(256), 0, stream,
                            (uint32_t*)(ws + L.off_partial), words);

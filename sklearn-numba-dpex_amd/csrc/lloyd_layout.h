@@ -12,6 +12,7 @@ constexpr int KMX_VARIANT_MFMA_F64 = 5;  // fp64 distances on the matrix cores, 
 
 constexpr int KMX_ACC_LDS = 1;
 constexpr int KMX_ACC_GLOBAL = 2;
+constexpr int KMX_ACC_BUCKET = 3;  // labels-only kernel, then sums per bucket of samples (lloyd_bucket.hip)
 
 constexpr int KMX_MAX_PARTIALS = 1024;          // upper bound on fused-step workgroups
 constexpr size_t KMX_LDS_ACC_LIMIT = 40000;     // bytes of LDS accumulators per workgroup
@@ -49,6 +50,15 @@ static inline bool kmx_flags_valid(uint32_t flags) {
 bool kmx_mfma_supported(int d, int k);
 bool kmx_mfma_wide_supported(int d, int k);
 bool kmx_mfma_f64_supported(int d, int k);
+bool kmx_mfma_f64_labels_supported(int d, int k);  // without the accumulators in LDS
+// bucketed sums (lloyd_bucket.hip)
+size_t kmx_bucket_bytes(int64_t n, int k);
+int32_t kmx_bucket_order(const uint32_t* labels, const int* counts, int* offsets, const int* ranks,
+                         int* order, int64_t n, int k, hipStream_t stream);
+int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const void* w,
+                              const uint32_t* labels_prev, const uint32_t* labels, void* sums,
+                              kmx_lloyd_status* status, char* bucket, int64_t n, int d, int k,
+                              int32_t dtype, hipStream_t stream);
 // fp32 matrix-core step with fp16 screening of the labels (lloyd_mfma_screen.hip): whether the
 // shape fits the kernel at all, and whether the flags (or, left to the library, the measured
 // break-even) select it
@@ -77,8 +87,11 @@ struct LloydLayout {
     // partial slots.
     int grid_cap(int cus) const {
         const int g = (wgs_per_cu > 0 ? wgs_per_cu : 4) * cus;
-        return g < n_partials ? g : n_partials;
+        return g < partial_slots() ? g : partial_slots();
     }
+    // Workgroups that may write partial sums (the labels-only kernel of the bucketed mode
+    // writes none).
+    int partial_slots() const { return acc_mode == KMX_ACC_BUCKET ? KMX_MAX_PARTIALS : n_partials; }
 };
 
 static inline int lloyd_reg_samples_per_thread(int d, int dtype) {
@@ -121,9 +134,24 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
         L.variant = KMX_VARIANT_MFMA_WIDE;
         L.acc_mode = KMX_ACC_GLOBAL;  // always the global fixed-point sums (variant code 42)
     }
-    else if (dtype == KMX_F64 && L.acc_mode == KMX_ACC_LDS && kmx_mfma_f64_supported(d, k) &&
-             (forced < 0 || forced == KMX_VARIANT_MFMA))
+    else if (dtype == KMX_F64 && kmx_mfma_f64_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA)) {
         L.variant = KMX_VARIANT_MFMA_F64;
+        if (L.acc_mode != KMX_ACC_LDS) {
+            // accumulators beyond what the vector-ALU kernels keep in LDS: one workgroup per
+            // compute unit with all of its LDS, and only as many partial slots as that needs
+            L.acc_mode = KMX_ACC_LDS;
+            const int slots = 256 * (L.wgs_per_cu > 0 ? L.wgs_per_cu : 1);
+            L.n_partials = slots < KMX_MAX_PARTIALS ? slots : KMX_MAX_PARTIALS;
+        }
+    }
+    if (L.acc_mode == KMX_ACC_GLOBAL && L.variant != KMX_VARIANT_MFMA_WIDE && n <= INT32_MAX) {
+        // float atomics on a few global copies of the sums are slow on this hardware: labels
+        // only (on the fp64 matrix cores where the centroids alone fit in LDS), then bucketed sums
+        L.acc_mode = KMX_ACC_BUCKET;
+        L.n_partials = 1;
+        if (dtype == KMX_F64 && kmx_mfma_f64_labels_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA))
+            L.variant = KMX_VARIANT_MFMA_F64;
+    }
     L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
@@ -138,8 +166,9 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     // screened path: the counter of samples evaluated in fp32 and its copy for the host (256
     // bytes), then ||x_i|| per sample
     const size_t bucket_bytes =
-        L.variant == KMX_VARIANT_MFMA_WIDE ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int)
-        : L.screen                         ? (size_t)256 + (size_t)n * sizeof(float)
+        (L.variant == KMX_VARIANT_MFMA_WIDE || L.acc_mode == KMX_ACC_BUCKET)
+            ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int)
+        : L.screen ? (size_t)256 + (size_t)n * sizeof(float)
                                            : 0;
     // wide matrix-core path: header, scaled half norms and fp16 parts of the centroids for the
     // screened label step (lloyd_mfma_wide_screen.hip)
@@ -210,9 +239,9 @@ int32_t kmx_assign_labels_mfma_wide_f32(const LloydLayout& L, const void* X_t,
 
 // fp64 matrix-core fused step (lloyd_mfma_f64.hip): fills partial[0 .. grid) like the
 // vector-ALU kernels with LDS accumulators; `update` false = labels only
-int kmx_mfma_f64_grid(int64_t n, int wgs_per_cu, int cols);
+int kmx_mfma_f64_grid(int64_t n, int d, int wgs_per_cu, int cols, int max_slots);
 int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* centroids_t,
                                 const void* half_norms, const uint32_t* labels_prev,
                                 uint32_t* labels, void* partial, kmx_lloyd_status* status,
                                 int64_t n, int d, int k, bool update, int wgs_per_cu, int cols,
-                                hipStream_t stream);
+                                int max_slots, hipStream_t stream);

@@ -1,5 +1,5 @@
-// fp64 fused Lloyd step on the matrix cores (gfx950), for d <= 32 when the (d + 1) * k
-// accumulators fit in LDS.
+// fp64 fused Lloyd step on the matrix cores (gfx950), for d <= 64 when the (d + 1) * k
+// accumulators and the centroids' operand fragments fit in the LDS of a compute unit.
 //
 // Replaces, for these shapes, the kernel pair fused_lloyd_single_step
 // (sklearn_numba_dpex/kmeans/kernels/lloyd_single_step.py:35-424) + the zero-fill / half-norm
@@ -54,11 +54,12 @@ __global__ __launch_bounds__(64 * f64_waves(NC)) void lloyd_mfma_f64_kernel(
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     double* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k,
     int vec_ok) {
-    if (UPDATE && status->state != KMX_RUNNING) return;
+    if (status != nullptr && status->state != KMX_RUNNING) return;
     constexpr int F64_WAVES = f64_waves(NC);
     constexpr int THREADS = 64 * F64_WAVES;
     constexpr int TILE = 16 * NC;
-    constexpr bool PREFETCH = NC == 2;
+    // (beyond 32 features the rows of one tile already take 64 registers)
+    constexpr bool PREFETCH = NC == 2 && NKS <= 8;
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int n_cb = (k + 15) >> 4;  // centroid blocks of 16
@@ -277,24 +278,30 @@ size_t mfma_f64_lds_bytes(int d, int k, bool update) {
 
 }  // namespace
 
+// One workgroup per compute unit may take all of its LDS (160 KB less the static variables).
 bool kmx_mfma_f64_supported(int d, int k) {
-    return d <= 32 && k >= 16 && mfma_f64_lds_bytes(d, k, true) <= 64 * 1024;
+    return d <= 64 && k >= 16 && mfma_f64_lds_bytes(d, k, true) <= 160 * 1024 - 256;
+}
+
+bool kmx_mfma_f64_labels_supported(int d, int k) {
+    return d <= 64 && k >= 16 && mfma_f64_lds_bytes(d, k, false) <= 160 * 1024 - 256;
 }
 
 // Sample columns per lane: two (three waves per SIMD, next tile in flight) once there are
 // several tiles per wave, four for small inputs.  KMX_FLAG_COLS(2 | 4) overrides this for
-// experiments.
-static int f64_cols(int64_t n, int cols) {
+// experiments.  More than 32 features: two (four would need 128 registers for the rows).
+static int f64_cols(int64_t n, int d, int cols) {
+    if (d > 32) return 2;
     if (cols == 2 || cols == 4) return cols;
     return n >= (int64_t)1 << 19 ? 2 : 4;
 }
 
-int kmx_mfma_f64_grid(int64_t n, int wgs_per_cu, int cols_asked) {
-    const int nc = f64_cols(n, cols_asked);
+int kmx_mfma_f64_grid(int64_t n, int d, int wgs_per_cu, int cols_asked, int max_slots) {
+    const int nc = f64_cols(n, d, cols_asked);
     const int64_t tiles = kmx_cdiv(kmx_cdiv(n, 16 * nc), f64_waves(nc));
     const int64_t cap = (int64_t)(wgs_per_cu > 0 ? wgs_per_cu : 1) * kmx_num_cus();
     int64_t grid = tiles < cap ? tiles : cap;
-    if (grid > KMX_MAX_PARTIALS) grid = KMX_MAX_PARTIALS;
+    if (grid > max_slots) grid = max_slots;
     return grid < 1 ? 1 : (int)grid;
 }
 
@@ -302,17 +309,24 @@ int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* cent
                                 const void* half_norms, const uint32_t* labels_prev,
                                 uint32_t* labels, void* partial, kmx_lloyd_status* status,
                                 int64_t n, int d, int k, bool update, int wgs_per_cu, int cols_asked,
-                                hipStream_t stream) {
-    if (!kmx_mfma_f64_supported(d, k)) return KMX_ERR_UNSUPPORTED;
+                                int max_slots, hipStream_t stream) {
+    if (!(update ? kmx_mfma_f64_supported(d, k) : kmx_mfma_f64_labels_supported(d, k)))
+        return KMX_ERR_UNSUPPORTED;
     const size_t lds = mfma_f64_lds_bytes(d, k, update);
-    const int grid = kmx_mfma_f64_grid(n, wgs_per_cu, cols_asked);
+    const int grid = kmx_mfma_f64_grid(n, d, wgs_per_cu, cols_asked, max_slots);
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     // rows start 16-byte aligned when n is even; 4 samples per lane need n % 4 == 0 only for
     // the 128-bit label accesses
     const int vec_ok = (n % 4 == 0) && aligned16(X_t) && aligned16(labels) &&
                        (!update || (aligned16(w) && aligned16(labels_prev)));
-    const int cols = f64_cols(n, cols_asked);
+    const int cols = f64_cols(n, d, cols_asked);
 #define KMX_F64_LAUNCH(NKS, NC, UPD)                                                              \
+    if (lds > 64 * 1024) {                                                                        \
+        const hipError_t e = hipFuncSetAttribute(                                                 \
+            reinterpret_cast<const void*>(&lloyd_mfma_f64_kernel<NKS, NC, UPD>),                   \
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                \
+        if (e != hipSuccess) return (int32_t)e;                                                   \
+    }                                                                                             \
     hipLaunchKernelGGL((lloyd_mfma_f64_kernel<NKS, NC, UPD>), dim3((unsigned)grid),                 \
                        dim3(64 * f64_waves(NC)), lds, stream, (const double*)X_t, (const double*)w, \
                        (const double*)centroids_t, (const double*)half_norms, labels_prev, labels,  \
@@ -320,11 +334,11 @@ int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* cent
 #define KMX_F64_CASE(NKS)                                    \
     do {                                                     \
         if (cols == 2) {                                     \
-            if (update) KMX_F64_LAUNCH(NKS, 2, true);        \
-            else KMX_F64_LAUNCH(NKS, 2, false);              \
+            if (update) { KMX_F64_LAUNCH(NKS, 2, true); }    \
+            else { KMX_F64_LAUNCH(NKS, 2, false); }          \
         } else {                                             \
-            if (update) KMX_F64_LAUNCH(NKS, 4, true);        \
-            else KMX_F64_LAUNCH(NKS, 4, false);              \
+            if (update) { KMX_F64_LAUNCH(NKS, 4, true); }    \
+            else { KMX_F64_LAUNCH(NKS, 4, false); }          \
         }                                                    \
     } while (0)
     switch ((d + 3) / 4) {
@@ -335,7 +349,21 @@ int32_t kmx_lloyd_step_mfma_f64(const void* X_t, const void* w, const void* cent
         case 5: KMX_F64_CASE(5); break;
         case 6: KMX_F64_CASE(6); break;
         case 7: KMX_F64_CASE(7); break;
-        default: KMX_F64_CASE(8); break;
+        case 8: KMX_F64_CASE(8); break;
+#define KMX_F64_CASE2(NKS)                            \
+    do {                                              \
+        if (update) { KMX_F64_LAUNCH(NKS, 2, true); } \
+        else { KMX_F64_LAUNCH(NKS, 2, false); }       \
+    } while (0)
+        case 9: KMX_F64_CASE2(9); break;
+        case 10: KMX_F64_CASE2(10); break;
+        case 11: KMX_F64_CASE2(11); break;
+        case 12: KMX_F64_CASE2(12); break;
+        case 13: KMX_F64_CASE2(13); break;
+        case 14: KMX_F64_CASE2(14); break;
+        case 15: KMX_F64_CASE2(15); break;
+        default: KMX_F64_CASE2(16); break;
+#undef KMX_F64_CASE2
     }
 #undef KMX_F64_LAUNCH
 #undef KMX_F64_CASE

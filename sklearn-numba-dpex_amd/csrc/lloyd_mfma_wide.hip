@@ -242,45 +242,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_mfma_wide_kernel(
 
 // ---- bucketed accumulation ---------------------------------------------------------------
 // counts[c] samples carry label c and ranks[i] is the position of sample i among them (the
-// value its counting atomic returned).  offsets = exclusive scan of counts (one workgroup),
-// order[offsets[c] + rank] = the samples of cluster c (any order: the sums below are integers).
-
-__global__ __launch_bounds__(1024) void bucket_offsets_kernel(const int* __restrict__ counts,
-                                                             int* __restrict__ offsets, int k) {
-    __shared__ int wave_tot[16];
-    __shared__ int carry_s;
-    if (threadIdx.x == 0) carry_s = 0;
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int c0 = 0; c0 < k; c0 += 1024) {
-        const int c = c0 + threadIdx.x;
-        const int v = c < k ? counts[c] : 0;
-        int incl = v;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int o = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += o;
-        }
-        if (lane == 63) wave_tot[wave] = incl;
-        __syncthreads();
-        int base = carry_s;
-        for (int w2 = 0; w2 < wave; ++w2) base += wave_tot[w2];
-        if (c < k) offsets[c] = base + incl - v;
-        __syncthreads();
-        if (threadIdx.x == 1023) carry_s = base + incl;
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) offsets[k] = carry_s;
-}
-
-__global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint32_t* __restrict__ labels,
-                                                             const int* __restrict__ offsets,
-                                                             const int* __restrict__ ranks,
-                                                             int* __restrict__ order, int64_t n) {
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-        order[offsets[labels[i]] + ranks[i]] = (int)i;
-}
+// value its counting atomic returned).  offsets = exclusive scan of counts and
+// order[offsets[c] + rank] = the samples of cluster c come from kmx_bucket_order
+// (lloyd_bucket.hip); any order will do: the sums below are integers.
 
 // One workgroup per ACC_CHUNK consecutive positions of `order` (samples sorted by cluster),
 // whatever the cluster sizes: a workgroup walks the cluster segments inside its range and
@@ -502,11 +466,8 @@ int32_t kmx_lloyd_step_mfma_wide_f32(const LloydLayout& L, const void* X_t, cons
         rc = launch_wide<MODE_COUNT>(L, X_t, w, centroids_t, half_norms, labels_prev, labels, status,
                                      q_exp, gsum, counts, ranks, n, d, k, stream);
     if (rc != KMX_OK) return rc;
-    hipLaunchKernelGGL(bucket_offsets_kernel, dim3(1), dim3(1024), 0, stream, counts, offsets, k);
-    int64_t sg = kmx_cdiv(n, 256 * 4);
-    if (sg > 2048) sg = 2048;
-    hipLaunchKernelGGL(bucket_scatter_kernel, dim3((unsigned)sg), dim3(256), 0, stream, labels, offsets, ranks,
-                       order, n);
+    rc = kmx_bucket_order(labels, counts, offsets, ranks, order, n, k, stream);
+    if (rc != KMX_OK) return rc;
     const unsigned ag = (unsigned)kmx_cdiv(n, ACC_CHUNK);
     if (d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0))
         hipLaunchKernelGGL((bucket_accumulate_kernel<true>), dim3(ag), dim3(256), 0, stream,

@@ -21,6 +21,9 @@ from ..common.topk import topk_idx
 # How many Lloyd iterations may be enqueued before the host next reads the status.
 _MAX_LOOKAHEAD = 16
 
+# Kernel variants (codes of the plan) that read a row-major copy of X besides the feature-major one.
+_ROW_MAJOR_VARIANTS = (42, 3, 13, 53)
+
 
 def lloyd(
     X_t,
@@ -66,9 +69,9 @@ def lloyd(
     empty_list = torch.empty(k, dtype=torch.int32, device=dev)
     verbose = bool(verbose)
 
-    # the wide fp32 path sums each cluster's rows from a row-major copy of X (one transpose per
-    # run, n * d extra elements of HBM) instead of one global atomic per (sample, feature)
-    X_rm = X_t.T.contiguous() if plan.variant == 42 else None
+    # the wide fp32 path and the bucketed sums add up each cluster's rows from a row-major copy
+    # of X (one transpose per run, n * d extra elements of HBM): whole cache lines per sample
+    X_rm = X_t.T.contiguous() if plan.variant in _ROW_MAJOR_VARIANTS else None
 
     check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), int(max_iter),
                              float(tol), stream),

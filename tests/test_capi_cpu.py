@@ -61,7 +61,11 @@ def test_workspace_queries():
     # the screened fp32 step keeps ||x_i|| per sample: 4 bytes per sample
     assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0, 0) - small - 4 * 4_900_000) < 256
     assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0)
-    assert lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) > (32 << 20)  # global copies
+    # sums beyond LDS off the wide path: sample order and ranks (2 n words) + one copy of the sums
+    assert 8_000_000 + 4 * 301 * 1024 < lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) < (16 << 20)
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 3
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0) == 51
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 32, 500, 1, 0) == 53
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0, 0) == 0
     assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7, 0) == 0
     assert lib.kmx_assign_workspace_bytes(14, 127, 0) > 127 * 16 * 4
@@ -90,9 +94,13 @@ def test_kernel_variant_selection():
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 64, 0, 0) == 61
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 32, 0, 0) == 31
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0) == 51    # fp64: matrix cores + LDS
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0) in (12, 2)  # accumulators too big for LDS
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 64, 128, 1, 0) == 51    # with all of a compute unit's LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 500, 1, 0) == 53    # labels on the matrix cores, bucketed sums
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0) == 13   # centroids too big for LDS as well
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 100, 1, 0) == 3
+    assert lib.kmx_lloyd_kernel_variant(1 << 31, 100, 100, 1, 0) == 2      # too many samples for 32-bit buckets
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0, 0) == 42  # wide MFMA + global sums
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 2   # streaming + global copies
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 3   # streaming labels + bucketed sums
     assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0, 0) == 11           # too few clusters for MFMA
     assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0, 0) == -2
     assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4, 0) == -3

@@ -46,8 +46,18 @@ def _small_configs():
         # kernel keeps in LDS: the wide path with one chunk of features (d <= 32)
         "M32e": lambda: dict(_blob_config(20_000, 14, 600, np.float32, 18), flags=0x10, variant=42),
         "M32f": lambda: dict(_blob_config(20_000, 14, 700, np.float32, 20), variant=42),
-        # fp64 whose accumulators do not fit LDS: vector-ALU kernel with global copies
-        "F64d": lambda: _blob_config(20_000, 32, 300, np.float64, 19),
+        # accumulators beyond LDS off the wide fp32 path: a labels-only kernel (fp64 matrix cores
+        # where the centroids fit, else vector ALU) and sums per bucket of samples
+        "F64d": lambda: dict(_blob_config(20_000, 32, 500, np.float64, 19), variant=53),
+        "B64a": lambda: dict(_blob_config(20_001, 100, 100, np.float64, 25), variant=3),
+        "B64b": lambda: dict(_blob_config(30_000, 8, 5000, np.float64, 26), variant=13),
+        "B32a": lambda: dict(_blob_config(9_001, 300, 40, np.float32, 27, skew=True), variant=3),
+        # fp64 on the matrix cores beyond 32 features (no rows in flight for the next tile) and
+        # with accumulators that need most of a compute unit's LDS
+        "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=51),
+        "F64f": lambda: dict(_blob_config(8_000, 64, 100, np.float64, 22), variant=51),
+        "F64g": lambda: dict(_blob_config(20_000, 32, 300, np.float64, 23), variant=51),
+        "F64h": lambda: dict(_blob_config(6_001, 61, 33, np.float64, 24), variant=51),
     }
 
 
@@ -72,7 +82,8 @@ def _odd_config():
 
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
-                                  "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d"])
+                                  "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d", "F64e", "F64f",
+                                  "F64g", "F64h", "B64a", "B64b", "B32a"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -98,8 +109,8 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
     _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), 100, 0.0, stream), "init")
-    if rowmajor and plan.variant != 42:
-        pytest.skip("the row-major copy is only used by the wide fp32 path")
+    if rowmajor and plan.variant not in (42, 3, 13, 53):
+        pytest.skip("the row-major copy is only used by the wide fp32 path and the bucketed sums")
     X_rm = _dev(X, cuda) if rowmajor else None
     _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev),
                                    ptr(labels), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
@@ -131,7 +142,8 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
-@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d",
+                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
