@@ -83,6 +83,7 @@ typedef struct kmx_lloyd_status {
 #define KMX_FLAG_PATH_STREAM 0x1u      /* features re-read per centroid window                */
 #define KMX_FLAG_PATH_REGISTER 0x2u    /* samples in registers, vector ALU                    */
 #define KMX_FLAG_PATH_MFMA 0x3u        /* matrix cores wherever the shape allows              */
+#define KMX_FLAG_PATH_GEMM 0x4u        /* tiled matrix-core labels + bucketed sums (any shape) */
 #define KMX_FLAG_LABELS_MASK 0x00000030u
 #define KMX_FLAG_LABELS_AUTO 0x00u
 #define KMX_FLAG_LABELS_F32 0x10u      /* every product of the fp32 paths taken in fp32       */

@@ -31,6 +31,7 @@ KMX_ERR_BAD_PLAN = -7
 FLAG_PATH_STREAM = 0x1
 FLAG_PATH_REGISTER = 0x2
 FLAG_PATH_MFMA = 0x3
+FLAG_PATH_GEMM = 0x4
 FLAG_LABELS_F32 = 0x10
 FLAG_LABELS_SCREEN = 0x20
 
@@ -201,7 +202,7 @@ def _flags_from_environment():
     flags = 0
     flags |= {"f32": FLAG_LABELS_F32, "screen": FLAG_LABELS_SCREEN}.get(os.environ.get("KMX_LLOYD_ASSIGN", ""), 0)
     flags |= {"stream": FLAG_PATH_STREAM, "register": FLAG_PATH_REGISTER,
-              "mfma": FLAG_PATH_MFMA}.get(os.environ.get("KMX_LLOYD_VARIANT", ""), 0)
+              "mfma": FLAG_PATH_MFMA, "gemm": FLAG_PATH_GEMM}.get(os.environ.get("KMX_LLOYD_VARIANT", ""), 0)
     wgs = os.environ.get("KMX_LLOYD_WGS_PER_CU", "")
     if wgs.isdigit() and 1 <= int(wgs) <= 8:
         flags |= flag_wgs_per_cu(int(wgs))

@@ -64,12 +64,14 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
     int64_t n, int d, int k, int dpad, int n_copies, int vec_ok) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
 
+    // LDS accumulators are fp64 for both types: ds_add_f64 is fast on this hardware, ds_add_f32
+    // is not (about 195 cycles per wave instruction)
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* acc = reinterpret_cast<T*>(smem_raw);
+    double* acc = reinterpret_cast<double*>(smem_raw);
     __shared__ unsigned int changed_block;
     const int items = (d + 1) * k;
     if (ACC == ACC_LDS) {
-        for (int j = threadIdx.x; j < items; j += 256) acc[j] = T(0);
+        for (int j = threadIdx.x; j < items; j += 256) acc[j] = 0.0;
     }
     if (threadIdx.x == 0) changed_block = 0;
     __syncthreads();
@@ -136,11 +138,18 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
                 if (ACC != ACC_NONE) {
                     changed += (labels_prev[i] != bi[r]) ? 1u : 0u;
                     const T wr = sample_weight[i];
-                    T* dst = (ACC == ACC_LDS) ? acc : gacc;
-                    kmx_atomic_add(dst + (size_t)d * k + bi[r], wr);
+                    if (ACC == ACC_LDS) {
+                        kmx_atomic_add(acc + (size_t)d * k + bi[r], (double)wr);
 #pragma unroll
-                    for (int f = 0; f < DREG; ++f) {
-                        if (f < d) kmx_atomic_add(dst + (size_t)f * k + bi[r], x[f][r] * wr);
+                        for (int f = 0; f < DREG; ++f) {
+                            if (f < d) kmx_atomic_add(acc + (size_t)f * k + bi[r], (double)x[f][r] * (double)wr);
+                        }
+                    } else {
+                        kmx_atomic_add(gacc + (size_t)d * k + bi[r], wr);
+#pragma unroll
+                        for (int f = 0; f < DREG; ++f) {
+                            if (f < d) kmx_atomic_add(gacc + (size_t)f * k + bi[r], x[f][r] * wr);
+                        }
                     }
                 }
             }
@@ -152,7 +161,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
         __syncthreads();
         if (ACC == ACC_LDS) {
             T* out = partial + (size_t)blockIdx.x * items;
-            for (int j = threadIdx.x; j < items; j += 256) out[j] = acc[j];
+            for (int j = threadIdx.x; j < items; j += 256) out[j] = (T)acc[j];
         }
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
     }
@@ -170,12 +179,14 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
     int n_copies) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
 
+    // LDS accumulators are fp64 for both types: ds_add_f64 is fast on this hardware, ds_add_f32
+    // is not (about 195 cycles per wave instruction)
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* acc = reinterpret_cast<T*>(smem_raw);
+    double* acc = reinterpret_cast<double*>(smem_raw);
     __shared__ unsigned int changed_block;
     const int items = (d + 1) * k;
     if (ACC == ACC_LDS) {
-        for (int j = threadIdx.x; j < items; j += 256) acc[j] = T(0);
+        for (int j = threadIdx.x; j < items; j += 256) acc[j] = 0.0;
     }
     if (threadIdx.x == 0) changed_block = 0;
     __syncthreads();
@@ -241,10 +252,15 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
                 if (ACC != ACC_NONE) {
                     changed += (labels_prev[i] != bi[r]) ? 1u : 0u;
                     const T wr = sample_weight[i];
-                    T* dst = (ACC == ACC_LDS) ? acc : gacc;
-                    kmx_atomic_add(dst + (size_t)d * k + bi[r], wr);
-                    for (int f = 0; f < d; ++f)
-                        kmx_atomic_add(dst + (size_t)f * k + bi[r], X_t[(size_t)f * n + i] * wr);
+                    if (ACC == ACC_LDS) {
+                        kmx_atomic_add(acc + (size_t)d * k + bi[r], (double)wr);
+                        for (int f = 0; f < d; ++f)
+                            kmx_atomic_add(acc + (size_t)f * k + bi[r], (double)X_t[(size_t)f * n + i] * (double)wr);
+                    } else {
+                        kmx_atomic_add(gacc + (size_t)d * k + bi[r], wr);
+                        for (int f = 0; f < d; ++f)
+                            kmx_atomic_add(gacc + (size_t)f * k + bi[r], X_t[(size_t)f * n + i] * wr);
+                    }
                 }
             }
         }
@@ -255,7 +271,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
         __syncthreads();
         if (ACC == ACC_LDS) {
             T* out = partial + (size_t)blockIdx.x * items;
-            for (int j = threadIdx.x; j < items; j += 256) out[j] = acc[j];
+            for (int j = threadIdx.x; j < items; j += 256) out[j] = (T)acc[j];
         }
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
     }
@@ -282,6 +298,16 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
             const long long iv = (long long)gsum[item];
             gsum[item] = 0ull;
             const T v = (T)ldexp((double)iv, -q_exp[item / k]);
+            if (item < d * k)
+                sums_t[item] = v;
+            else
+                sizes[item - d * k] = v;
+        }
+    } else if (n_partials == 1) {
+        // one copy of the sums (bucketed accumulation): moved and cleared by the same few blocks
+        for (int item = blockIdx.x * 256 + threadIdx.x; item < items; item += gridDim.x * 256) {
+            const T v = partial[item];
+            if (clear_partials) partial[item] = T(0);
             if (item < d * k)
                 sums_t[item] = v;
             else
@@ -559,7 +585,7 @@ template <typename T, int DREG, int R, int ACC>
 void launch_reg(const LloydLayout& L, const void* X_t, const void* w, const T* cpack,
                 const T* half_norms, const uint32_t* labels_prev, uint32_t* labels, T* partial,
                 kmx_lloyd_status* status, int64_t n, int d, int k, int grid, hipStream_t stream) {
-    const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(T) : 0;
+    const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(double) : 0;
     const int vec_ok = (n % R == 0) && (((uintptr_t)X_t) % (R * sizeof(T)) == 0);
     hipLaunchKernelGGL((lloyd_fused_reg_kernel<T, DREG, R, ACC>), dim3(grid), dim3(256), lds, stream,
                        (const T*)X_t, (const T*)w, cpack, half_norms, labels_prev, labels, partial,
@@ -572,7 +598,10 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
                   uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
                   hipStream_t stream) {
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
-    if (L.variant == KMX_VARIANT_MFMA_F64) {
+    if (L.variant == KMX_VARIANT_GEMM) {
+        (void)kmx_lloyd_gemm_labels(X_t, centroids_t, half_norms, labels, status, n, d, k,
+                                    sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
+    } else if (L.variant == KMX_VARIANT_MFMA_F64) {
         (void)kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
                                       status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, L.partial_slots(),
                                       stream);
@@ -600,7 +629,7 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
 #undef KMX_REG_CASE
     } else {
         constexpr int R = 2, KC = 8;
-        const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(T) : 0;
+        const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(double) : 0;
         hipLaunchKernelGGL((lloyd_fused_stream_kernel<T, R, KC, ACC>), dim3(grid), dim3(256), lds,
                            stream, (const T*)X_t, (const T*)w, (const T*)centroids_t, half_norms,
                            labels_prev, labels, partial, status, n, d, k, L.n_partials);
@@ -650,8 +679,9 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[1], stream);
     const int items = (d + 1) * k;
-    const int64_t reduce_grid =
-        gsum != nullptr ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128) : kmx_cdiv(items, RED_ITEMS);
+    const int64_t reduce_grid = (gsum != nullptr || n_partials_used == 1)
+                                    ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128)
+                                    : kmx_cdiv(items, RED_ITEMS);
     // sums that fit in LDS are finished by one workgroup (no device-wide fences or tickets)
     const bool small_tail = gsum == nullptr && (size_t)items * sizeof(T) <= 48 * 1024;
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)reduce_grid), dim3(256), 0,

@@ -1,0 +1,307 @@
+// Labels for any shape on the matrix cores (gfx950): a tiled product of the samples with the
+// centroids whose epilogue keeps, per sample, the best score and its centroid.
+//
+// Replaces, for shapes no specialised kernel takes (fp32 beyond 256 features, fp64 beyond 64
+// features or with centroids beyond LDS, few clusters of wide samples), the label half of
+// fused_lloyd_single_step (sklearn_numba_dpex/kmeans/kernels/lloyd_single_step.py:35-424) and
+// assignment (kmeans/kernels/compute_labels.py:29-288): the reference slides windows of
+// centroids through local memory and multiplies on the vector ALU; here the products run on
+// v_mfma_f32_32x32x2_f32 / v_mfma_f64_16x16x4_f64.  The sums of the update step come from the
+// bucketed accumulation (lloyd_bucket.hip).
+//
+//   * score(i, c) = <x_i, c> - 0.5 ||c||^2, the label is its arg-max with the lowest centroid
+//     winning a tie (the reference minimises 0.5 ||c||^2 - <x, c> with a strict comparison in
+//     increasing centroid order).
+//   * A workgroup of four waves owns 128 samples and walks the centroids in tiles of 128; the
+//     features are staged 16 (fp32) or 8 (fp64) at a time through double-buffered LDS tiles.
+//     Both arrays are feature-major in memory, as the tiles are in LDS: a stage is a copy of
+//     rows (128-bit loads where alignment allows), rows padded so that the operand reads of a
+//     wave fall on distinct banks.  The next stage's loads are in flight during the MFMAs.
+//   * A wave multiplies all 128 centroids of the tile with its own 32 samples: centroids are
+//     the rows of the MFMA result and samples its columns, so a lane holds scores of ONE
+//     sample (fp32) or two (fp64) and the running arg-max needs no exchange until the end,
+//     where the two (fp32) or four (fp64) lanes that share a sample are combined.
+//   * Accumulators start at -0.5 ||c||^2 (-inf past the last centroid).
+#include "lloyd_layout.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef double v4d __attribute__((ext_vector_type(4)));
+
+constexpr int GT = 128;       // samples per workgroup, centroids per tile
+constexpr int GK32 = 16;      // features per stage, fp32
+constexpr int GK64 = 8;       // features per stage, fp64
+constexpr int GLD32 = GT + 32;  // LDS row length in floats: the two K rows of a wave's read 32 banks apart
+constexpr int GLD64 = GT + 16;  // in doubles: the K rows of a half-wave's read 32 banks apart
+
+// One stage of one operand: rows f0 .. f0 + GK32 - 1 of a feature-major array with `len`
+// columns, columns c0 .. c0 + 127, zero outside the array.  Thread t takes the groups of four
+// columns t and t + 256 (row g / 32, columns 4 (g % 32)).
+__device__ __forceinline__ void stage_load_f32(float4 (&r)[2], const float* __restrict__ base, int64_t len,
+                                               int64_t c0, int d, int f0, bool vec_ok) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        const int f = f0 + (g >> 5);
+        const int64_t c = c0 + 4 * (g & 31);
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (f < d) {
+            const float* __restrict__ src = base + (size_t)f * (size_t)len + c;
+            if (vec_ok && c + 4 <= len) {
+                v = *reinterpret_cast<const float4*>(src);
+            } else {
+                if (c + 0 < len) v.x = src[0];
+                if (c + 1 < len) v.y = src[1];
+                if (c + 2 < len) v.z = src[2];
+                if (c + 3 < len) v.w = src[3];
+            }
+        }
+        r[l] = v;
+    }
+}
+
+__device__ __forceinline__ void stage_store_f32(float (*tile)[GLD32], const float4 (&r)[2]) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        *reinterpret_cast<float4*>(&tile[g >> 5][4 * (g & 31)]) = r[l];
+    }
+}
+
+__global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ centroids_t,
+    const float* __restrict__ half_norms, uint32_t* __restrict__ labels,
+    const kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int x_vec, int c_vec) {
+    if (status != nullptr && status->state != KMX_RUNNING) return;
+    __shared__ __align__(16) float xs[2][GK32][GLD32];
+    __shared__ __align__(16) float cs[2][GK32][GLD32];
+    __shared__ float hn[GT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, j = lane & 31;
+    const int n_stages = (d + GK32 - 1) / GK32;
+    const int64_t n_tiles = (n + GT - 1) / GT;
+
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i0 = tile * GT;
+        float best = -kmx_inf<float>();
+        int bidx = 0;
+        for (int c0 = 0; c0 < k; c0 += GT) {
+            __syncthreads();  // the previous tile's reads of hn and of the stage buffers are over
+            if (threadIdx.x < GT)
+                hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<float>();
+            float4 rx[2], rc[2];
+            stage_load_f32(rx, X_t, n, i0, d, 0, x_vec != 0);
+            stage_load_f32(rc, centroids_t, k, c0, d, 0, c_vec != 0);
+            stage_store_f32(xs[0], rx);
+            stage_store_f32(cs[0], rc);
+            __syncthreads();
+
+            // accumulator register r of lane (j, h): centroid 32 a + 8 (r / 4) + 4 h + r % 4
+            v16f acc[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[a][r] = hn[32 * a + 8 * (r >> 2) + 4 * h + (r & 3)];
+
+            for (int st = 0; st < n_stages; ++st) {
+                const int cur = st & 1;
+                if (st + 1 < n_stages) {
+                    stage_load_f32(rx, X_t, n, i0, d, (st + 1) * GK32, x_vec != 0);
+                    stage_load_f32(rc, centroids_t, k, c0, d, (st + 1) * GK32, c_vec != 0);
+                }
+#pragma unroll
+                for (int s = 0; s < GK32 / 2; ++s) {
+                    // lane (j, h) supplies feature 2 s + h of centroid / sample j of the 32
+                    const float bf = xs[cur][2 * s + h][32 * wave + j];
+                    float af[4];
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) af[a] = cs[cur][2 * s + h][32 * a + j];
+#pragma unroll
+                    for (int a = 0; a < 4; ++a)
+                        acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[a], bf, acc[a], 0, 0, 0);
+                }
+                if (st + 1 < n_stages) {
+                    stage_store_f32(xs[cur ^ 1], rx);
+                    stage_store_f32(cs[cur ^ 1], rc);
+                }
+                __syncthreads();
+            }
+
+            // increasing centroid order per lane, strict comparison: the lowest index keeps a tie
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float v = acc[a][r];
+                    const int c = c0 + 32 * a + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (v > best) {
+                        best = v;
+                        bidx = c;
+                    }
+                }
+        }
+        // the two lanes of a sample
+        const float ob = __shfl_xor(best, 32, 64);
+        const int oi = __shfl_xor(bidx, 32, 64);
+        if (ob > best || (ob == best && oi < bidx)) bidx = oi;
+        const int64_t i = i0 + 32 * wave + j;
+        if (h == 0 && i < n) labels[i] = (uint32_t)bidx;
+    }
+}
+
+// fp64: thread t takes the pairs of columns t and t + 256 (row g / 64, columns 2 (g % 64)).
+__device__ __forceinline__ void stage_load_f64(double2 (&r)[2], const double* __restrict__ base, int64_t len,
+                                               int64_t c0, int d, int f0, bool vec_ok) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        const int f = f0 + (g >> 6);
+        const int64_t c = c0 + 2 * (g & 63);
+        double2 v = make_double2(0.0, 0.0);
+        if (f < d) {
+            const double* __restrict__ src = base + (size_t)f * (size_t)len + c;
+            if (vec_ok && c + 2 <= len) {
+                v = *reinterpret_cast<const double2*>(src);
+            } else {
+                if (c + 0 < len) v.x = src[0];
+                if (c + 1 < len) v.y = src[1];
+            }
+        }
+        r[l] = v;
+    }
+}
+
+__device__ __forceinline__ void stage_store_f64(double (*tile)[GLD64], const double2 (&r)[2]) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        *reinterpret_cast<double2*>(&tile[g >> 6][2 * (g & 63)]) = r[l];
+    }
+}
+
+__global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
+    const double* __restrict__ X_t, const double* __restrict__ centroids_t,
+    const double* __restrict__ half_norms, uint32_t* __restrict__ labels,
+    const kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int x_vec, int c_vec) {
+    if (status != nullptr && status->state != KMX_RUNNING) return;
+    __shared__ __align__(16) double xs[2][GK64][GLD64];
+    __shared__ __align__(16) double cs[2][GK64][GLD64];
+    __shared__ double hn[GT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, j = lane & 15;
+    const int n_stages = (d + GK64 - 1) / GK64;
+    const int64_t n_tiles = (n + GT - 1) / GT;
+
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i0 = tile * GT;
+        double best[2] = {-kmx_inf<double>(), -kmx_inf<double>()};
+        int bidx[2] = {0, 0};
+        for (int c0 = 0; c0 < k; c0 += GT) {
+            __syncthreads();
+            if (threadIdx.x < GT)
+                hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<double>();
+            double2 rx[2], rc[2];
+            stage_load_f64(rx, X_t, n, i0, d, 0, x_vec != 0);
+            stage_load_f64(rc, centroids_t, k, c0, d, 0, c_vec != 0);
+            stage_store_f64(xs[0], rx);
+            stage_store_f64(cs[0], rc);
+            __syncthreads();
+
+            // accumulator r of lane (g, j), row tile a, column tile b: centroid 16 a + g + 4 r of
+            // sample 32 wave + 16 b + j
+            v4d acc[8][2];
+#pragma unroll
+            for (int a = 0; a < 8; ++a)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const double v = hn[16 * a + g + 4 * r];
+                    acc[a][0][r] = v;
+                    acc[a][1][r] = v;
+                }
+
+            for (int st = 0; st < n_stages; ++st) {
+                const int cur = st & 1;
+                if (st + 1 < n_stages) {
+                    stage_load_f64(rx, X_t, n, i0, d, (st + 1) * GK64, x_vec != 0);
+                    stage_load_f64(rc, centroids_t, k, c0, d, (st + 1) * GK64, c_vec != 0);
+                }
+#pragma unroll
+                for (int s = 0; s < GK64 / 4; ++s) {
+                    // lane (g, j) supplies feature 4 s + g of centroid / sample j of the 16
+                    double bf[2];
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) bf[b] = xs[cur][4 * s + g][32 * wave + 16 * b + j];
+#pragma unroll
+                    for (int a = 0; a < 8; ++a) {
+                        const double af = cs[cur][4 * s + g][16 * a + j];
+#pragma unroll
+                        for (int b = 0; b < 2; ++b)
+                            acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(af, bf[b], acc[a][b], 0, 0, 0);
+                    }
+                }
+                if (st + 1 < n_stages) {
+                    stage_store_f64(xs[cur ^ 1], rx);
+                    stage_store_f64(cs[cur ^ 1], rc);
+                }
+                __syncthreads();
+            }
+
+#pragma unroll
+            for (int a = 0; a < 8; ++a)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int c = c0 + 16 * a + g + 4 * r;
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        const double v = acc[a][b][r];
+                        if (v > best[b]) {
+                            best[b] = v;
+                            bidx[b] = c;
+                        }
+                    }
+                }
+        }
+        // the four lanes of a sample
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const double ob = __shfl_xor(best[b], off, 64);
+                const int oi = __shfl_xor(bidx[b], off, 64);
+                if (ob > best[b] || (ob == best[b] && oi < bidx[b])) {
+                    best[b] = ob;
+                    bidx[b] = oi;
+                }
+            }
+            const int64_t i = i0 + 32 * wave + 16 * b + j;
+            if (g == 0 && i < n) labels[i] = (uint32_t)bidx[b];
+        }
+    }
+}
+
+}  // namespace
+
+// Labels of all samples; `half_norms` = 0.5 ||c||^2 per centroid; a null `status` or one in the
+// running state lets the kernel work, any other state makes it a no-op.
+int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const void* half_norms,
+                              uint32_t* labels, const kmx_lloyd_status* status, int64_t n, int d, int k,
+                              int32_t dtype, hipStream_t stream) {
+    const size_t s = kmx_dtype_size(dtype);
+    const int per_vec = (int)(16 / s);
+    auto vec_ok = [&](const void* p, int64_t len) { return (len % per_vec == 0) && ((((uintptr_t)p) & 15) == 0); };
+    const int x_vec = vec_ok(X_t, n), c_vec = vec_ok(centroids_t, k);
+    int64_t grid = kmx_cdiv(n, GT);
+    const int64_t cap = (int64_t)2 * kmx_num_cus();
+    if (grid > cap) grid = cap;
+    if (dtype == KMX_F32)
+        hipLaunchKernelGGL(lloyd_gemm_labels_f32_kernel, dim3((unsigned)grid), dim3(256), 0, stream,
+                           (const float*)X_t, (const float*)centroids_t, (const float*)half_norms, labels,
+                           status, n, d, k, x_vec, c_vec);
+    else
+        hipLaunchKernelGGL(lloyd_gemm_labels_f64_kernel, dim3((unsigned)grid), dim3(256), 0, stream,
+                           (const double*)X_t, (const double*)centroids_t, (const double*)half_norms, labels,
+                           status, n, d, k, x_vec, c_vec);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}

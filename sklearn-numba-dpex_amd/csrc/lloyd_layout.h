@@ -9,13 +9,14 @@ constexpr int KMX_VARIANT_REGISTER = 1;  // samples held in registers, centroids
 constexpr int KMX_VARIANT_MFMA = 3;      // fp32 distances on the matrix cores, LDS accumulators
 constexpr int KMX_VARIANT_MFMA_WIDE = 4; // fp32 matrix cores, samples in registers, global sums
 constexpr int KMX_VARIANT_MFMA_F64 = 5;  // fp64 distances on the matrix cores, LDS accumulators
+constexpr int KMX_VARIANT_GEMM = 6;      // labels by a tiled matrix-core product (any shape), bucketed sums
 
 constexpr int KMX_ACC_LDS = 1;
 constexpr int KMX_ACC_GLOBAL = 2;
 constexpr int KMX_ACC_BUCKET = 3;  // labels-only kernel, then sums per bucket of samples (lloyd_bucket.hip)
 
 constexpr int KMX_MAX_PARTIALS = 1024;          // upper bound on fused-step workgroups
-constexpr size_t KMX_LDS_ACC_LIMIT = 40000;     // bytes of LDS accumulators per workgroup
+constexpr size_t KMX_LDS_ACC_LIMIT = 40000;     // bytes of (fp64) LDS accumulators per workgroup
 constexpr size_t KMX_GLOBAL_COPIES_BYTES = 64u << 20;
 
 // Kernel selection comes from the caller's `flags` (KMX_FLAG_* of the public header) and from
@@ -27,6 +28,7 @@ static inline int kmx_flags_forced_variant(uint32_t flags) {
         case KMX_FLAG_PATH_STREAM: return 0;
         case KMX_FLAG_PATH_REGISTER: return 1;
         case KMX_FLAG_PATH_MFMA: return 3;
+        case KMX_FLAG_PATH_GEMM: return 6;
         default: return -1;
     }
 }
@@ -40,7 +42,7 @@ static inline int kmx_flags_cols(uint32_t flags) {
 }
 static inline bool kmx_flags_valid(uint32_t flags) {
     if (flags & ~(uint32_t)0x7f3f) return false;
-    if ((flags & KMX_FLAG_PATH_MASK) > KMX_FLAG_PATH_MFMA) return false;
+    if ((flags & KMX_FLAG_PATH_MASK) > KMX_FLAG_PATH_GEMM) return false;
     if ((flags & KMX_FLAG_LABELS_MASK) == KMX_FLAG_LABELS_MASK) return false;
     const uint32_t w = (flags >> 8) & 0xfu, c = (flags >> 12) & 0x7u;
     return w <= 8 && (c == 0 || c == 2 || c == 4);
@@ -51,6 +53,10 @@ bool kmx_mfma_supported(int d, int k);
 bool kmx_mfma_wide_supported(int d, int k);
 bool kmx_mfma_f64_supported(int d, int k);
 bool kmx_mfma_f64_labels_supported(int d, int k);  // without the accumulators in LDS
+// labels of any shape by a tiled matrix-core product (lloyd_gemm.hip)
+int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const void* half_norms,
+                              uint32_t* labels, const kmx_lloyd_status* status, int64_t n, int d, int k,
+                              int32_t dtype, hipStream_t stream);
 // bucketed sums (lloyd_bucket.hip)
 size_t kmx_bucket_bytes(int64_t n, int k);
 int32_t kmx_bucket_order(const uint32_t* labels, const int* counts, int* offsets, const int* ranks,
@@ -114,7 +120,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     const int forced = kmx_flags_forced_variant(flags);
     if (forced == KMX_VARIANT_STREAM) L.variant = KMX_VARIANT_STREAM;
     if (forced == KMX_VARIANT_REGISTER && reg_ok) L.variant = KMX_VARIANT_REGISTER;
-    if (items * s <= KMX_LDS_ACC_LIMIT) {
+    if (items * sizeof(double) <= KMX_LDS_ACC_LIMIT) {
         L.acc_mode = KMX_ACC_LDS;
         L.n_partials = KMX_MAX_PARTIALS;
     } else {
@@ -126,11 +132,17 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     }
     // (the screened step has the whole LDS of a compute unit and covers shapes the all-fp32
     // step, which stays within 64 KB, does not)
-    if (dtype == KMX_F32 && L.acc_mode == KMX_ACC_LDS &&
+    // (their accumulators are 64-bit fixed point with a bound of their own)
+    if (dtype == KMX_F32 && items * sizeof(float) <= KMX_LDS_ACC_LIMIT &&
         (kmx_mfma_supported(d, k) || kmx_mfma_screen_supported(n, d, k, flags)) &&
-        (forced < 0 || forced == KMX_VARIANT_MFMA))
+        (forced < 0 || forced == KMX_VARIANT_MFMA)) {
         L.variant = KMX_VARIANT_MFMA;
-    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA)) {
+        L.acc_mode = KMX_ACC_LDS;
+        L.n_partials = KMX_MAX_PARTIALS;
+    }
+    // (the wide path is built for many clusters: up to 256 the tiled product below is faster)
+    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) &&
+             ((forced < 0 && k > 256) || forced == KMX_VARIANT_MFMA)) {
         L.variant = KMX_VARIANT_MFMA_WIDE;
         L.acc_mode = KMX_ACC_GLOBAL;  // always the global fixed-point sums (variant code 42)
     }
@@ -144,13 +156,26 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
             L.n_partials = slots < KMX_MAX_PARTIALS ? slots : KMX_MAX_PARTIALS;
         }
     }
-    if (L.acc_mode == KMX_ACC_GLOBAL && L.variant != KMX_VARIANT_MFMA_WIDE && n <= INT32_MAX) {
-        // float atomics on a few global copies of the sums are slow on this hardware: labels
-        // only (on the fp64 matrix cores where the centroids alone fit in LDS), then bucketed sums
-        L.acc_mode = KMX_ACC_BUCKET;
-        L.n_partials = 1;
-        if (dtype == KMX_F64 && kmx_mfma_f64_labels_supported(d, k) && (forced < 0 || forced == KMX_VARIANT_MFMA))
-            L.variant = KMX_VARIANT_MFMA_F64;
+    const bool specialised = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE ||
+                             L.variant == KMX_VARIANT_MFMA_F64;
+    if (n <= INT32_MAX && (!specialised || forced == KMX_VARIANT_GEMM)) {
+        // No specialised fused kernel.  From 16 clusters on, or whenever the accumulators do not
+        // fit in LDS (float atomics on global copies of the sums are slow on this hardware):
+        // labels only, on the matrix cores -- the fp64 kernel when the centroid operands alone
+        // fit in LDS, else the tiled product -- then bucketed sums.  Fewer clusters with
+        // accumulators in LDS: the fused vector-ALU kernels.
+        const bool matrix_ok = forced < 0 || forced == KMX_VARIANT_MFMA || forced == KMX_VARIANT_GEMM;
+        if (forced == KMX_VARIANT_GEMM) {
+            L.variant = KMX_VARIANT_GEMM;
+            L.acc_mode = KMX_ACC_BUCKET;
+        } else if (matrix_ok && (k >= 16 || L.acc_mode == KMX_ACC_GLOBAL)) {
+            L.variant = (dtype == KMX_F64 && kmx_mfma_f64_labels_supported(d, k)) ? KMX_VARIANT_MFMA_F64
+                                                                                 : KMX_VARIANT_GEMM;
+            L.acc_mode = KMX_ACC_BUCKET;
+        } else if (L.acc_mode == KMX_ACC_GLOBAL) {
+            L.acc_mode = KMX_ACC_BUCKET;  // the vector-ALU kernel asked for, labels only
+        }
+        if (L.acc_mode == KMX_ACC_BUCKET) L.n_partials = 1;
     }
     L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
     L.off_status = 0;

@@ -22,7 +22,7 @@ from ..common.topk import topk_idx
 _MAX_LOOKAHEAD = 16
 
 # Kernel variants (codes of the plan) that read a row-major copy of X besides the feature-major one.
-_ROW_MAJOR_VARIANTS = (42, 3, 13, 53)
+_ROW_MAJOR_VARIANTS = (42, 3, 13, 53, 63)
 
 
 def lloyd(

@@ -63,7 +63,7 @@ def test_workspace_queries():
     assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0)
     # sums beyond LDS off the wide path: sample order and ranks (2 n words) + one copy of the sums
     assert 8_000_000 + 4 * 301 * 1024 < lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) < (16 << 20)
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 3
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 63
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0) == 51
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 32, 500, 1, 0) == 53
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0, 0) == 0
@@ -96,12 +96,19 @@ def test_kernel_variant_selection():
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0) == 51    # fp64: matrix cores + LDS
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 64, 128, 1, 0) == 51    # with all of a compute unit's LDS
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 500, 1, 0) == 53    # labels on the matrix cores, bucketed sums
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0) == 13   # centroids too big for LDS as well
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 100, 1, 0) == 3
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0) == 63   # centroids too big for LDS as well: tiled product
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0x2) == 13  # vector-ALU labels when asked for
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 100, 1, 0) == 63     # tiled matrix-core labels, bucketed sums
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 100, 1, 0x1) == 3     # vector-ALU labels when asked for
     assert lib.kmx_lloyd_kernel_variant(1 << 31, 100, 100, 1, 0) == 2      # too many samples for 32-bit buckets
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0, 0) == 42  # wide MFMA + global sums
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 3   # streaming labels + bucketed sums
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 63  # tiled matrix-core labels + bucketed sums
     assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0, 0) == 11           # too few clusters for MFMA
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 64, 0, 0) == 63    # the wide path only beyond 256 clusters
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 300, 0, 0) == 42
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 0, 0) == 1     # few clusters, sums in LDS: fused vector-ALU step
+    assert lib.kmx_lloyd_kernel_variant(100_000, 784, 10, 0, 0) == 63      # sums beyond LDS
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0x4) == 63  # the tiled product on request
     assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0, 0) == -2
     assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4, 0) == -3
     # the caller's flags, and nothing else, move the choice

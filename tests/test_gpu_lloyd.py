@@ -38,7 +38,8 @@ def _small_configs():
         "M32b": lambda: _blob_config(5_000, 40, 20, np.float32, 15),
         "M32c": lambda: _blob_config(33, 14, 16, np.float32, 16),
         # wide fp32 path with very unequal clusters (bucket sizes from 0 to a third of n)
-        "C3k": lambda: _blob_config(40_000, 128, 64, np.float32, 17, skew=True),
+        "C3k": lambda: dict(_blob_config(40_000, 128, 64, np.float32, 17, skew=True), flags=0x3, variant=42),
+        "C3k2": lambda: dict(_blob_config(40_000, 128, 64, np.float32, 17, skew=True), variant=63),
         # few features, many clusters: accumulators and centroid copies need more than 64 KB of
         # LDS, which only the screened step (one workgroup per compute unit) may take
         "M32d": lambda: dict(_blob_config(20_000, 14, 600, np.float32, 18), variant=61),
@@ -49,9 +50,13 @@ def _small_configs():
         # accumulators beyond LDS off the wide fp32 path: a labels-only kernel (fp64 matrix cores
         # where the centroids fit, else vector ALU) and sums per bucket of samples
         "F64d": lambda: dict(_blob_config(20_000, 32, 500, np.float64, 19), variant=53),
-        "B64a": lambda: dict(_blob_config(20_001, 100, 100, np.float64, 25), variant=3),
-        "B64b": lambda: dict(_blob_config(30_000, 8, 5000, np.float64, 26), variant=13),
-        "B32a": lambda: dict(_blob_config(9_001, 300, 40, np.float32, 27, skew=True), variant=3),
+        "B64a": lambda: dict(_blob_config(20_001, 100, 100, np.float64, 25), variant=63),
+        "B64b": lambda: dict(_blob_config(30_000, 8, 5000, np.float64, 26), variant=63),
+        "B64d": lambda: dict(_blob_config(30_000, 8, 5000, np.float64, 26), flags=0x2, variant=13),
+        "B64e": lambda: dict(_blob_config(10_000, 100, 100, np.float64, 30), flags=0x1, variant=3),
+        "B32a": lambda: dict(_blob_config(9_001, 300, 40, np.float32, 27, skew=True), variant=63),
+        "B32b": lambda: dict(_blob_config(3_000, 784, 130, np.float32, 28), variant=63),
+        "B64c": lambda: dict(_blob_config(2_999, 70, 260, np.float64, 29), variant=63),
         # fp64 on the matrix cores beyond 32 features (no rows in flight for the next tile) and
         # with accumulators that need most of a compute unit's LDS
         "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=51),
@@ -83,7 +88,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "B64a", "B64b", "B32a"])
+                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -109,7 +114,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
     _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), 100, 0.0, stream), "init")
-    if rowmajor and plan.variant not in (42, 3, 13, 53):
+    if rowmajor and plan.variant not in (42, 3, 13, 53, 63):
         pytest.skip("the row-major copy is only used by the wide fp32 path and the bucketed sums")
     X_rm = _dev(X, cuda) if rowmajor else None
     _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev),
@@ -143,7 +148,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d",
-                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a"])
+                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is

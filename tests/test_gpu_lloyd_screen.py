@@ -20,6 +20,7 @@ pytestmark = pytest.mark.gpu
 # on); the tests here want the screened kernel on every shape it can run.
 SCREEN = 0x20   # KMX_FLAG_LABELS_SCREEN
 ALL_F32 = 0x10  # KMX_FLAG_LABELS_F32
+WIDE = 0x3      # KMX_FLAG_PATH_MFMA: the wide path also for the few clusters that are left to the tiled product
 
 
 def _one_iteration(X, w, init, cuda, flags=SCREEN):
@@ -45,7 +46,7 @@ def _one_iteration(X, w, init, cuda, flags=SCREEN):
     stream = _capi.current_stream()
     variant = plan.variant
     _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(c_in), 10, 0.0, stream), "init")
-    X_rm = dev(X) if variant == 42 else None  # the wide path sums (and screens) with a row-major copy
+    X_rm = dev(X) if variant in (42, 63) else None  # the wide path sums (and screens) with a row-major copy
     _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev),
                                    ptr(labels), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
     status = _capi.LloydStatus()
@@ -500,7 +501,7 @@ def test_wide_screened_step_matches_oracle(cuda, shape):
     goes through the all-fp32 matrix-core kernel."""
     n, d, k = shape
     X, w, init = _blobs(n, d, k, seed=n + d)
-    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=SCREEN | WIDE)
     assert variant == 42
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
     assert rechecked <= 8 + n // 10
@@ -516,10 +517,10 @@ def test_wide_screened_labels_only_match_oracle(cuda, shape):
 
     n, d, k = shape
     X, _, init = _blobs(n, d, k, seed=n + d + 2)
-    assert lib.kmx_assign_workspace_bytes_for(n, d, k, 0, SCREEN) > lib.kmx_assign_workspace_bytes(d, k, 0)
+    assert lib.kmx_assign_workspace_bytes_for(n, d, k, 0, SCREEN | WIDE) > lib.kmx_assign_workspace_bytes(d, k, 0)
     ref = ok.assign_labels(X, init)
     for roomy in (True, False):
-        labels = _labels_only(X, init, cuda, roomy=roomy)
+        labels = _labels_only(X, init, cuda, roomy=roomy, flags=SCREEN | WIDE)
         assert labels.min() >= 0 and labels.max() < k
         assert_labels_match(labels, ref, X, init)
 
@@ -532,7 +533,7 @@ def test_wide_labels_only_with_samples_far_from_the_centroids(cuda):
     C = rng.standard_normal((k, d)).astype(np.float32)
     C[7] = C[3]
     X = (1000.0 * rng.standard_normal((n, d))).astype(np.float32)
-    labels = _labels_only(X, C, cuda)
+    labels = _labels_only(X, C, cuda, flags=SCREEN | WIDE)
     assert not np.any(labels == 7)
     assert_labels_match(labels, ok.assign_labels(X, C), X, C)
 
@@ -541,7 +542,7 @@ def test_wide_duplicate_centroids_take_the_lowest_index(cuda):
     X, w, init = _blobs(8_000, 128, 96, seed=41)
     init[70] = init[5]
     init[95] = init[64]
-    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=SCREEN | WIDE)
     assert variant == 42
     assert not np.any(labels == 70) and not np.any(labels == 95)
     ref = ok.assign_labels(X, init)
@@ -553,7 +554,7 @@ def test_wide_duplicate_centroids_take_the_lowest_index(cuda):
 def test_wide_all_centroids_identical(cuda):
     X, w, init = _blobs(3_000, 96, 64, seed=42)
     init[:] = init[0]
-    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=SCREEN | WIDE)
     assert variant == 42
     assert np.all(labels == 0)
     assert rechecked == X.shape[0]
@@ -562,7 +563,7 @@ def test_wide_all_centroids_identical(cuda):
 
 def test_wide_screen_switched_off_by_flag(cuda):
     X, w, init = _blobs(5_000, 128, 64, seed=43)
-    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=ALL_F32)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=ALL_F32 | WIDE)
     assert variant == 42 and rechecked == 0
     _check_against_oracle(X, w, init, labels, c_out, sizes, status)
 
