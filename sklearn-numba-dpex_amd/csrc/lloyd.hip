@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cpack,
     const T* __restrict__ half_norms, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, T* __restrict__ partial, kmx_lloyd_status* __restrict__ status,
-    int64_t n, int d, int k, int dpad, int n_copies, int vec_ok) {
+    int64_t n, int d, int k, int dpad, int n_copies, int vec_ok, int lds_copies) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
 
     // LDS accumulators are fp64 for both types: ds_add_f64 is fast on this hardware, ds_add_f32
@@ -71,7 +71,9 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
     __shared__ unsigned int changed_block;
     const int items = (d + 1) * k;
     if (ACC == ACC_LDS) {
-        for (int j = threadIdx.x; j < items; j += 256) acc[j] = 0.0;
+        for (int j = threadIdx.x; j < items * lds_copies; j += 256) acc[j] = 0.0;
+        // few clusters mean many lanes of a wave on one address: lanes spread over copies
+        acc += (size_t)(threadIdx.x & (lds_copies - 1)) * items;
     }
     if (threadIdx.x == 0) changed_block = 0;
     __syncthreads();
@@ -161,14 +163,21 @@ __global__ __launch_bounds__(256) void lloyd_fused_reg_kernel(
         __syncthreads();
         if (ACC == ACC_LDS) {
             T* out = partial + (size_t)blockIdx.x * items;
-            for (int j = threadIdx.x; j < items; j += 256) out[j] = (T)acc[j];
+            const double* all = reinterpret_cast<const double*>(smem_raw);
+            for (int j = threadIdx.x; j < items; j += 256) {
+                double tot = all[j];
+                for (int c = 1; c < lds_copies; ++c) tot += all[(size_t)c * items + j];
+                out[j] = (T)tot;
+            }
         }
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
     }
 }
 
 // ------------------------------------------------------------------------------------------
-// Streaming fused step for wide samples: windows of KC centroids, features re-read per window.
+// Streaming fused step for wide samples and few clusters: windows of KC centroids, features
+// re-read per window (one window up to KC clusters).  A thread owns R consecutive samples and
+// reads them with one 128-bit load per feature row.
 // ------------------------------------------------------------------------------------------
 template <typename T, int R, int KC, int ACC>
 __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
     const T* __restrict__ centroids_t, const T* __restrict__ half_norms,
     const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
     T* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k,
-    int n_copies) {
+    int n_copies, int vec_ok, int lds_copies) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
 
     // LDS accumulators are fp64 for both types: ds_add_f64 is fast on this hardware, ds_add_f32
@@ -186,7 +195,9 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
     __shared__ unsigned int changed_block;
     const int items = (d + 1) * k;
     if (ACC == ACC_LDS) {
-        for (int j = threadIdx.x; j < items; j += 256) acc[j] = 0.0;
+        for (int j = threadIdx.x; j < items * lds_copies; j += 256) acc[j] = 0.0;
+        // few clusters mean many lanes of a wave on one address: lanes spread over copies
+        acc += (size_t)(threadIdx.x & (lds_copies - 1)) * items;
     }
     if (threadIdx.x == 0) changed_block = 0;
     __syncthreads();
@@ -197,9 +208,7 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
     const int64_t n_tiles = (n + tile_samples - 1) / tile_samples;
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        int64_t idx[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) idx[r] = tile * tile_samples + r * 256 + threadIdx.x;
+        const int64_t i0 = tile * tile_samples + (int64_t)threadIdx.x * R;
 
         T best[R];
         uint32_t bi[R];
@@ -215,10 +224,10 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int j = 0; j < KC; ++j) dot[r][j] = T(0);
+#pragma unroll 4
             for (int f = 0; f < d; ++f) {
                 T xv[R];
-#pragma unroll
-                for (int r = 0; r < R; ++r) xv[r] = (idx[r] < n) ? X_t[(size_t)f * n + idx[r]] : T(0);
+                load_row<T, R>(X_t + (size_t)f * n, i0, n, vec_ok != 0, xv);
                 const T* __restrict__ crow = centroids_t + (size_t)f * k;  // wave-uniform
 #pragma unroll
                 for (int j = 0; j < KC; ++j) {
@@ -245,21 +254,32 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
         }
 
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int64_t i = idx[r];
-            if (i < n) {
-                labels[i] = bi[r];
-                if (ACC != ACC_NONE) {
-                    changed += (labels_prev[i] != bi[r]) ? 1u : 0u;
-                    const T wr = sample_weight[i];
-                    if (ACC == ACC_LDS) {
-                        kmx_atomic_add(acc + (size_t)d * k + bi[r], (double)wr);
-                        for (int f = 0; f < d; ++f)
-                            kmx_atomic_add(acc + (size_t)f * k + bi[r], (double)X_t[(size_t)f * n + i] * (double)wr);
-                    } else {
-                        kmx_atomic_add(gacc + (size_t)d * k + bi[r], wr);
-                        for (int f = 0; f < d; ++f)
-                            kmx_atomic_add(gacc + (size_t)f * k + bi[r], X_t[(size_t)f * n + i] * wr);
+        for (int r = 0; r < R; ++r)
+            if (i0 + r < n) labels[i0 + r] = bi[r];
+
+        if (ACC != ACC_NONE) {
+            T wr[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const bool live = i0 + r < n;
+                wr[r] = live ? sample_weight[i0 + r] : T(0);
+                changed += (live && labels_prev[i0 + r] != bi[r]) ? 1u : 0u;
+                if (live) {
+                    if (ACC == ACC_LDS) kmx_atomic_add(acc + (size_t)d * k + bi[r], (double)wr[r]);
+                    else kmx_atomic_add(gacc + (size_t)d * k + bi[r], wr[r]);
+                }
+            }
+#pragma unroll 4
+            for (int f = 0; f < d; ++f) {
+                T xv[R];
+                load_row<T, R>(X_t + (size_t)f * n, i0, n, vec_ok != 0, xv);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    if (i0 + r < n) {
+                        if (ACC == ACC_LDS)
+                            kmx_atomic_add(acc + (size_t)f * k + bi[r], (double)xv[r] * (double)wr[r]);
+                        else
+                            kmx_atomic_add(gacc + (size_t)f * k + bi[r], xv[r] * wr[r]);
                     }
                 }
             }
@@ -271,7 +291,12 @@ __global__ __launch_bounds__(256) void lloyd_fused_stream_kernel(
         __syncthreads();
         if (ACC == ACC_LDS) {
             T* out = partial + (size_t)blockIdx.x * items;
-            for (int j = threadIdx.x; j < items; j += 256) out[j] = (T)acc[j];
+            const double* all = reinterpret_cast<const double*>(smem_raw);
+            for (int j = threadIdx.x; j < items; j += 256) {
+                double tot = all[j];
+                for (int c = 1; c < lds_copies; ++c) tot += all[(size_t)c * items + j];
+                out[j] = (T)tot;
+            }
         }
         if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
     }
@@ -571,25 +596,43 @@ __global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words)
 // Host-side launchers
 // ------------------------------------------------------------------------------------------
 
+// Samples per thread of the streaming kernel: one 128-bit load per feature row, or single
+// samples while that would leave compute units without a workgroup.
+static int lloyd_stream_samples_per_thread(int64_t n, int dtype) {
+    const int rv = dtype == KMX_F32 ? 4 : 2;
+    return n >= (int64_t)256 * rv * 2 * kmx_num_cus() ? rv : 1;
+}
+
 // Workgroups of a vector-ALU fused step (also the number of partial slots it fills).
 int lloyd_fused_grid(const LloydLayout& L, int64_t n, int d, int dtype) {
     if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n, d, L.wgs_per_cu, L.cols, L.partial_slots());
-    const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype) : 2;
+    const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype)
+                                                      : lloyd_stream_samples_per_thread(n, dtype);
     const int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
     const int cap = L.grid_cap(kmx_num_cus());
     int grid = (int)(tiles < cap ? tiles : cap);
     return grid < 1 ? 1 : grid;
 }
 
+// Copies of the LDS accumulators of the vector-ALU kernels (a power of two, at most 8, within
+// KMX_LDS_ACC_LIMIT): with k clusters a wave's atomics of one feature fall on k addresses.
+static int lds_acc_copies(int d, int k) {
+    const size_t one = (size_t)(d + 1) * k * sizeof(double);
+    int copies = 1;
+    while (copies < 8 && copies * 2 * (size_t)k <= 64 && one * copies * 2 <= KMX_LDS_ACC_LIMIT) copies *= 2;
+    return copies;
+}
+
 template <typename T, int DREG, int R, int ACC>
 void launch_reg(const LloydLayout& L, const void* X_t, const void* w, const T* cpack,
                 const T* half_norms, const uint32_t* labels_prev, uint32_t* labels, T* partial,
                 kmx_lloyd_status* status, int64_t n, int d, int k, int grid, hipStream_t stream) {
-    const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(double) : 0;
+    const int copies = lds_acc_copies(d, k);
+    const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(double) * copies : 0;
     const int vec_ok = (n % R == 0) && (((uintptr_t)X_t) % (R * sizeof(T)) == 0);
     hipLaunchKernelGGL((lloyd_fused_reg_kernel<T, DREG, R, ACC>), dim3(grid), dim3(256), lds, stream,
                        (const T*)X_t, (const T*)w, cpack, half_norms, labels_prev, labels, partial,
-                       status, n, d, k, L.dpad, L.n_partials, vec_ok);
+                       status, n, d, k, L.dpad, L.n_partials, vec_ok, copies);
 }
 
 template <typename T, int ACC>
@@ -628,11 +671,19 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
         }
 #undef KMX_REG_CASE
     } else {
-        constexpr int R = 2, KC = 8;
-        const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(double) : 0;
-        hipLaunchKernelGGL((lloyd_fused_stream_kernel<T, R, KC, ACC>), dim3(grid), dim3(256), lds,
-                           stream, (const T*)X_t, (const T*)w, (const T*)centroids_t, half_norms,
-                           labels_prev, labels, partial, status, n, d, k, L.n_partials);
+        constexpr int RV = 16 / (int)sizeof(T), KC = 16;
+        const int copies = lds_acc_copies(d, k);
+        const size_t lds = (ACC == ACC_LDS) ? (size_t)(d + 1) * k * sizeof(double) * copies : 0;
+        if (lloyd_stream_samples_per_thread(n, sizeof(T) == 8 ? KMX_F64 : KMX_F32) == 1) {
+            hipLaunchKernelGGL((lloyd_fused_stream_kernel<T, 1, KC, ACC>), dim3(grid), dim3(256), lds,
+                               stream, (const T*)X_t, (const T*)w, (const T*)centroids_t, half_norms,
+                               labels_prev, labels, partial, status, n, d, k, L.n_partials, 0, copies);
+        } else {
+            const int vec_ok = (n % RV == 0) && (((uintptr_t)X_t) % 16 == 0);
+            hipLaunchKernelGGL((lloyd_fused_stream_kernel<T, RV, KC, ACC>), dim3(grid), dim3(256), lds,
+                               stream, (const T*)X_t, (const T*)w, (const T*)centroids_t, half_norms,
+                               labels_prev, labels, partial, status, n, d, k, L.n_partials, vec_ok, copies);
+        }
     }
 }
 
