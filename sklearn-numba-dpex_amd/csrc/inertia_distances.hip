@@ -3,6 +3,8 @@
 // coalesced loads (consecutive lanes = consecutive samples of one feature row).
 #include "kmx_common.h"
 
+#include <type_traits>
+
 namespace {
 
 // Four consecutive values of a row at i0 (128-bit accesses when `full`), zero past n.
@@ -188,31 +190,119 @@ __global__ __launch_bounds__(256) void euclidean_distances_reg_kernel(
     }
 }
 
-// Any d: the thread keeps KC running sums for a window of centroids (wave-uniform centroid
-// loads) and writes KC coalesced rows; X is re-read per window through the caches.
-template <typename T, int KC>
-__global__ __launch_bounds__(256) void euclidean_distances_kernel(
-    const T* __restrict__ X_t, const T* __restrict__ centroids_t, T* __restrict__ distances_t,
-    int64_t n, int d, int k) {
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-        for (int c0 = 0; c0 < k; c0 += KC) {
-            T acc[KC];
+// Any d: a workgroup owns a tile of DT_S samples x DT_C centroids, a thread a 4 x 8 block of it;
+// the features are staged DT_K at a time through LDS (both arrays are feature-major, as the
+// tiles: a stage is a copy of rows, 128-bit loads where alignment allows), the next stage's
+// loads in flight during the arithmetic.  Per staged feature a thread reads its four samples
+// and eight centroids from LDS (the centroid reads are broadcasts) and updates 32 sums with a
+// difference and a fused multiply-add each, features in order: vector-ALU bound.
+constexpr int DT_S = 128, DT_C = 64, DT_K = 16;
+
+template <typename T, int COLS>
+__device__ __forceinline__ void dt_stage_load(T (*regs)[16 / sizeof(T)], const T* __restrict__ base, int64_t len,
+                                              int64_t c0, int d, int f0, bool vec_ok) {
+    constexpr int V = 16 / sizeof(T);                 // elements per 128-bit vector
+    constexpr int PER_ROW = COLS / V;                 // vectors per staged row
+    constexpr int N = DT_K * PER_ROW / 256;           // vectors per thread
 #pragma unroll
-            for (int j = 0; j < KC; ++j) acc[j] = T(0);
-            for (int f = 0; f < d; ++f) {
-                const T xv = X_t[(size_t)f * n + i];
-                const T* __restrict__ crow = centroids_t + (size_t)f * k;
+    for (int l = 0; l < N; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        const int f = f0 + g / PER_ROW;
+        const int64_t c = c0 + (int64_t)V * (g % PER_ROW);
 #pragma unroll
-                for (int j = 0; j < KC; ++j) {
-                    const int c = (c0 + j < k) ? c0 + j : k - 1;
-                    const T diff = crow[c] - xv;
-                    acc[j] = fma(diff, diff, acc[j]);
-                }
+        for (int e = 0; e < V; ++e) regs[l][e] = T(0);
+        if (f < d) {
+            const T* __restrict__ src = base + (size_t)f * (size_t)len + c;
+            if (vec_ok && c + V <= len) {
+                using Vec = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+                union {
+                    Vec v;
+                    T s[V];
+                } u;
+                u.v = *reinterpret_cast<const Vec*>(src);
+#pragma unroll
+                for (int e = 0; e < V; ++e) regs[l][e] = u.s[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                    if (c + e < len) regs[l][e] = src[e];
             }
+        }
+    }
+}
+
+template <typename T, int COLS>
+__device__ __forceinline__ void dt_stage_store(T (*tile)[COLS], const T (*regs)[16 / sizeof(T)]) {
+    constexpr int V = 16 / sizeof(T);
+    constexpr int PER_ROW = COLS / V;
+    constexpr int N = DT_K * PER_ROW / 256;
 #pragma unroll
-            for (int j = 0; j < KC; ++j)
-                if (c0 + j < k) distances_t[(size_t)(c0 + j) * n + i] = dist_sqrt(acc[j]);
+    for (int l = 0; l < N; ++l) {
+        const int g = threadIdx.x + 256 * l;
+#pragma unroll
+        for (int e = 0; e < V; ++e) tile[g / PER_ROW][V * (g % PER_ROW) + e] = regs[l][e];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void euclidean_distances_tiled_kernel(
+    const T* __restrict__ X_t, const T* __restrict__ centroids_t, T* __restrict__ distances_t,
+    int64_t n, int d, int k, int x_vec, int c_vec, int out_vec) {
+    constexpr int V = 16 / sizeof(T);
+    __shared__ __align__(16) T xs[DT_K][DT_S];
+    __shared__ __align__(16) T cs[DT_K][DT_C];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int64_t i0 = (int64_t)blockIdx.x * DT_S;
+    const int c0 = blockIdx.y * DT_C;
+    T rx[DT_K * DT_S / V / 256][V], rc[DT_K * DT_C / V / 256][V];
+    T acc[8][4];
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[c][i] = T(0);
+
+    dt_stage_load<T, DT_S>(rx, X_t, n, i0, d, 0, x_vec != 0);
+    dt_stage_load<T, DT_C>(rc, centroids_t, k, c0, d, 0, c_vec != 0);
+    const int n_stages = (d + DT_K - 1) / DT_K;
+    for (int st = 0; st < n_stages; ++st) {
+        __syncthreads();  // the previous stage's reads are over
+        dt_stage_store<T, DT_S>(xs, rx);
+        dt_stage_store<T, DT_C>(cs, rc);
+        __syncthreads();
+        if (st + 1 < n_stages) {
+            dt_stage_load<T, DT_S>(rx, X_t, n, i0, d, (st + 1) * DT_K, x_vec != 0);
+            dt_stage_load<T, DT_C>(rc, centroids_t, k, c0, d, (st + 1) * DT_K, c_vec != 0);
+        }
+        // (rows past d hold zeros on both sides: their differences add nothing)
+#pragma unroll
+        for (int kk = 0; kk < DT_K; ++kk) {
+            T xv[4], cv[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xv[i] = xs[kk][4 * tx + i];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) cv[c] = cs[kk][8 * ty + c];
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const T diff = cv[c] - xv[i];
+                    acc[c][i] = fma(diff, diff, acc[c][i]);
+                }
+        }
+    }
+    const int64_t i = i0 + 4 * tx;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int cc = c0 + 8 * ty + c;
+        if (cc >= k) continue;
+        T* __restrict__ dst = distances_t + (size_t)cc * (size_t)n + i;
+        if (sizeof(T) == 4 && out_vec && i + 4 <= n) {
+            *reinterpret_cast<float4*>(dst) = make_float4((float)dist_sqrt(acc[c][0]), (float)dist_sqrt(acc[c][1]),
+                                                          (float)dist_sqrt(acc[c][2]), (float)dist_sqrt(acc[c][3]));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (i + e < n) dst[e] = dist_sqrt(acc[c][e]);
         }
     }
 }
@@ -366,14 +456,18 @@ int32_t kmx_euclidean_distances(const void* X_t, const void* centroids_t, void* 
         hipLaunchKernelGGL((euclidean_distances_reg_kernel<double, 16>), rgrid, dim3(256), lds, stream,
                            (const double*)X_t, (const double*)centroids_t, (double*)distances_t, n, d, k, vec_ok,
                            c_chunk);
-    } else if (dtype == KMX_F32) {
-        hipLaunchKernelGGL((euclidean_distances_kernel<float, 8>), dim3(stream_grid(n)), dim3(256), 0, stream,
-                           (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d,
-                           k);
     } else {
-        hipLaunchKernelGGL((euclidean_distances_kernel<double, 8>), dim3(stream_grid(n)), dim3(256), 0,
-                           stream, (const double*)X_t, (const double*)centroids_t,
-                           (double*)distances_t, n, d, k);
+        const dim3 tgrid((unsigned)kmx_cdiv(n, DT_S), (unsigned)kmx_cdiv(k, DT_C));
+        const int per_vec = (int)(16 / es);
+        const int x_vec = (n % per_vec == 0) && al16(X_t), c_vec = (k % per_vec == 0) && al16(centroids_t);
+        if (dtype == KMX_F32)
+            hipLaunchKernelGGL((euclidean_distances_tiled_kernel<float>), tgrid, dim3(256), 0, stream,
+                               (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d, k, x_vec,
+                               c_vec, vec_ok);
+        else
+            hipLaunchKernelGGL((euclidean_distances_tiled_kernel<double>), tgrid, dim3(256), 0, stream,
+                               (const double*)X_t, (const double*)centroids_t, (double*)distances_t, n, d, k,
+                               x_vec, c_vec, 0);
     }
     KMX_LAUNCH_CHECK();
     return KMX_OK;

@@ -275,11 +275,12 @@ def test_label_helpers(cuda):
     assert int(drivers.get_nb_distinct_clusters(_dev(a, cuda), 50)) == len(np.unique(a))
 
 
-# every instantiation of the distance and inertia kernels (register / windowed distances,
+# every instantiation of the distance and inertia kernels (register / tiled distances,
 # centroids in LDS or not, 128-bit or scalar accesses) against numpy in fp64
 @pytest.mark.parametrize("shape", [(1003, 14, 127, np.float32), (4096, 32, 7, np.float32), (777, 33, 5, np.float32),
                                    (1001, 16, 9, np.float64), (500, 17, 3, np.float64), (1000, 300, 50, np.float32),
-                                   (3, 2, 2, np.float64)])
+                                   (3, 2, 2, np.float64), (1000, 70, 130, np.float64), (1028, 100, 64, np.float32),
+                                   (515, 129, 67, np.float32), (1026, 48, 66, np.float64)])
 def test_distances_and_inertia_kernels(cuda, shape):
     import torch
 
