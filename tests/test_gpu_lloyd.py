@@ -237,3 +237,29 @@ def test_full_lloyd_run_matches_oracle(cuda, name):
 
 def n_samples_differ_cap(X):
     return X.shape[0] // 1000
+
+
+@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "B64a", "B64b", "B32a", "B32b", "B64c", "odd"])
+def test_labels_and_score_paths_on_every_label_kernel(cuda, name):
+    """kmx_assign_labels, labels + inertia in one call and the distances on the shapes of the
+    tiled matrix-core product, of the labels-only fp64 matrix-core kernel and of the vector-ALU
+    kernels, against the oracle."""
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    cfg = _small_configs()[name]()
+    X, init, w = cfg["X"], cfg["init"], cfg["sample_weight"]
+    n = X.shape[0]
+    X_t, C_t, w_d = _dev(X.T, cuda), _dev(init.T, cuda), _dev(w, cuda)
+    ref = ok.assign_labels(X, init)
+    labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
+    drivers._assign(X_t, C_t, labels)
+    got = labels.cpu().numpy().astype(np.int64)
+    assert_labels_match(got, ref, X, init)
+    labels2, inertia = drivers.get_labels_inertia(X_t, C_t, w_d, True)
+    np.testing.assert_array_equal(labels2.cpu().numpy().astype(np.int64), got)
+    assert float(inertia[0]) == pytest.approx(float(ok.inertia(X, w, init, got)), rel=RTOL[X.dtype] * 5)
+    dist = drivers.get_euclidean_distances(X_t[:, :512].contiguous(), C_t).cpu().numpy()
+    exact = np.sqrt(((X[:512].astype(np.float64)[:, None, :] - init.astype(np.float64)[None, :, :]) ** 2).sum(axis=2))
+    np.testing.assert_allclose(dist, exact, rtol=RTOL[X.dtype] * 2, atol=RTOL[X.dtype])
