@@ -269,7 +269,7 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False, flags=0):
     variant = plan.variant
     X_rm = torch.as_tensor(X, device=dev)
     X_t = X_rm.T.contiguous()
-    if variant != 42:
+    if variant not in (42, 3, 13, 53, 63):  # the variants that sum rows of a row-major copy
         X_rm = None
     w_d = torch.as_tensor(w, device=dev)
     cent = [torch.as_tensor(np.ascontiguousarray(init.T), device=dev), None]
@@ -355,6 +355,35 @@ def extra_configs():
         "fused_step_frac_of_hbm_peak": nbytes / (kms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
     log(f"[bench] config 5: {out['config5']['ms_per_iter']:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
+    del c5
+    out["other_shapes"] = other_shapes()
+    return out
+
+
+def other_shapes():
+    """Shapes off the specialised kernels, as users bring them: few clusters of wide samples,
+    fp64 with sums beyond LDS, more than 256 features.  Overlapping blobs (the labels keep
+    changing), wall time per iteration over iterations 6-13 of the driver's loop."""
+    out = []
+    for name, n, d, k, dtype in (("70000 x 784, 10 clusters, fp32", 70_000, 784, 10, np.float32),
+                                 ("2e6 x 100, 10 clusters, fp32", 2_000_000, 100, 10, np.float32),
+                                 ("1e6 x 100, 100 clusters, fp64", 1_000_000, 100, 100, np.float64),
+                                 ("1e6 x 48, 64 clusters, fp64", 1_000_000, 48, 64, np.float64),
+                                 ("1e5 x 300, 300 clusters, fp32", 100_000, 300, 300, np.float32)):
+        t0 = time.time()
+        rng = np.random.default_rng(n + d + k)
+        centers = (rng.uniform(-1.0, 1.0, (k, d)) * (4.0 / np.sqrt(d))).astype(dtype)  # overlapping blobs
+        X = centers[rng.integers(0, k, n)]
+        X += rng.standard_normal((n, d), dtype=dtype)
+        cfg = {"X": X, "init": X[rng.choice(n, k, replace=False)].copy(), "sample_weight": np.ones(n, dtype=dtype), "k": k}
+        kms, variant, wall_ms = gpu_lloyd_step_time(cfg, 8, consecutive=True)
+        s = np.dtype(dtype).itemsize
+        out.append({"shape": name, "kernel_variant": variant, "ms_per_iter": wall_ms,
+                    "label_and_sum_kernels_ms": float(kms[0]),
+                    "TFLOPs": lloyd_flops(n, d, k) / (wall_ms * 1e-3) / 1e12,
+                    "X_bytes_per_iter_TBs": n * d * s / (wall_ms * 1e-3) / 1e12})
+        log(f"[bench] {name}: variant {variant}, {wall_ms:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
+        del X, cfg
     return out
 
 
