@@ -386,6 +386,14 @@ int32_t kmx_broadcast_rows(void* a, const void* v, int64_t rows, int64_t cols, i
 int32_t kmx_broadcast_div_cols(void* a, const void* v, int64_t rows, int64_t cols, int32_t dtype,
                                void* stream);
 
+/* dst (cols, rows) = the transpose of src (rows, cols), both row-major and distinct.  The
+ * reference leaves its transposed copies to the array library (`X.T` through dpctl /
+ * `dpt.asarray(..., order="C")`: sklearn_numba_dpex/kmeans/engine.py:88-98,
+ * kmeans/drivers.py:43-53); here the ingest of a row-major X and the row-major copy that the
+ * bucketed sums read go through this kernel. */
+int32_t kmx_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int32_t dtype,
+                      void* stream);
+
 /* data[i] = data[i] / divisor.  make_apply_elementwise_func with _divide_by,
  * common/kernels.py:11-36, common/_utils.py:17-33. */
 int32_t kmx_divide_by(void* data, int64_t n_items, double divisor, int32_t dtype, void* stream);

@@ -142,6 +142,7 @@ SIGNATURES = {
     "kmx_broadcast_rows": (_I32, [_P, _P, _I64, _I64, _I32, _I32, _P]),
     "kmx_broadcast_div_cols": (_I32, [_P, _P, _I64, _I64, _I32, _P]),
     "kmx_divide_by": (_I32, [_P, _I64, c_double, _I32, _P]),
+    "kmx_transpose": (_I32, [_P, _P, _I64, _I64, _I32, _P]),
     "kmx_fill_zero": (_I32, [_P, _I64, _P]),
     "kmx_centroid_shifts": (_I32, [_P, _P, _P, _I32, _I32, _I32, _P]),
     "kmx_topk_workspace_bytes": (_SZ, [_I64, _I32]),

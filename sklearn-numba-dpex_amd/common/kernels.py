@@ -47,6 +47,17 @@ def divide_by(data, divisor):
           "kmx_divide_by")
 
 
+def transposed_copy(array):
+    """A C-contiguous copy of array.T for a C-contiguous 2-d fp32 / fp64 array (the reference
+    leaves these copies to the array library: kmeans/engine.py:88-98)."""
+    _require_contiguous(array)
+    rows, cols = array.shape
+    out = torch.empty((cols, rows), dtype=array.dtype, device=array.device)
+    check(lib.kmx_transpose(ptr(array), ptr(out), rows, cols, dcode(array), _capi.current_stream()),
+          "kmx_transpose")
+    return out
+
+
 def initialize_to_zeros(data):
     """Zero fill, in place (common/kernels.py:38-57)."""
     _require_contiguous(data)

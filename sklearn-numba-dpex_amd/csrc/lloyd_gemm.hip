@@ -12,7 +12,8 @@
 //   * score(i, c) = <x_i, c> - 0.5 ||c||^2, the label is its arg-max with the lowest centroid
 //     winning a tie (the reference minimises 0.5 ||c||^2 - <x, c> with a strict comparison in
 //     increasing centroid order).
-//   * A workgroup of four waves owns 128 samples and walks the centroids in tiles of 128; the
+//   * A workgroup of four waves owns 128 samples and walks the centroids in tiles of 128 (one
+//     tile of 32 or 64 for that few clusters); the
 //     features are staged 16 (fp32) or 8 (fp64) at a time through double-buffered LDS tiles.
 //     Both arrays are feature-major in memory, as the tiles are in LDS: a stage is a copy of
 //     rows (128-bit loads where alignment allows), rows padded so that the operand reads of a
@@ -69,6 +70,10 @@ __device__ __forceinline__ void stage_store_f32(float (*tile)[GLD32], const floa
     }
 }
 
+// NA: 32-centroid row tiles per pass over the features (4: tiles of 128 centroids; 1 or 2 for
+// up to 32 / 64 clusters, where wider tiles would multiply padding).  A stage always copies 128
+// centroid columns; only the first 32 NA are used.
+template <int NA>
 __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
     const float* __restrict__ X_t, const float* __restrict__ centroids_t,
     const float* __restrict__ half_norms, uint32_t* __restrict__ labels,
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
         const int64_t i0 = tile * GT;
         float best = -kmx_inf<float>();
         int bidx = 0;
-        for (int c0 = 0; c0 < k; c0 += GT) {
+        for (int c0 = 0; c0 < k; c0 += 32 * NA) {
             __syncthreads();  // the previous tile's reads of hn and of the stage buffers are over
             if (threadIdx.x < GT)
                 hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<float>();
@@ -98,9 +103,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
             __syncthreads();
 
             // accumulator register r of lane (j, h): centroid 32 a + 8 (r / 4) + 4 h + r % 4
-            v16f acc[4];
+            v16f acc[NA];
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
+            for (int a = 0; a < NA; ++a)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[a][r] = hn[32 * a + 8 * (r >> 2) + 4 * h + (r & 3)];
 
@@ -114,11 +119,11 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
                 for (int s = 0; s < GK32 / 2; ++s) {
                     // lane (j, h) supplies feature 2 s + h of centroid / sample j of the 32
                     const float bf = xs[cur][2 * s + h][32 * wave + j];
-                    float af[4];
+                    float af[NA];
 #pragma unroll
-                    for (int a = 0; a < 4; ++a) af[a] = cs[cur][2 * s + h][32 * a + j];
+                    for (int a = 0; a < NA; ++a) af[a] = cs[cur][2 * s + h][32 * a + j];
 #pragma unroll
-                    for (int a = 0; a < 4; ++a)
+                    for (int a = 0; a < NA; ++a)
                         acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[a], bf, acc[a], 0, 0, 0);
                 }
                 if (st + 1 < n_stages) {
@@ -130,7 +135,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
 
             // increasing centroid order per lane, strict comparison: the lowest index keeps a tie
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
+            for (int a = 0; a < NA; ++a)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float v = acc[a][r];
@@ -180,6 +185,8 @@ __device__ __forceinline__ void stage_store_f64(double (*tile)[GLD64], const dou
     }
 }
 
+// NA: 16-centroid row tiles per pass (8: tiles of 128 centroids; 2 or 4 for up to 32 / 64 clusters).
+template <int NA>
 __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
     const double* __restrict__ X_t, const double* __restrict__ centroids_t,
     const double* __restrict__ half_norms, uint32_t* __restrict__ labels,
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
         const int64_t i0 = tile * GT;
         double best[2] = {-kmx_inf<double>(), -kmx_inf<double>()};
         int bidx[2] = {0, 0};
-        for (int c0 = 0; c0 < k; c0 += GT) {
+        for (int c0 = 0; c0 < k; c0 += 16 * NA) {
             __syncthreads();
             if (threadIdx.x < GT)
                 hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<double>();
@@ -210,9 +217,9 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
 
             // accumulator r of lane (g, j), row tile a, column tile b: centroid 16 a + g + 4 r of
             // sample 32 wave + 16 b + j
-            v4d acc[8][2];
+            v4d acc[NA][2];
 #pragma unroll
-            for (int a = 0; a < 8; ++a)
+            for (int a = 0; a < NA; ++a)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const double v = hn[16 * a + g + 4 * r];
@@ -233,7 +240,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
 #pragma unroll
                     for (int b = 0; b < 2; ++b) bf[b] = xs[cur][4 * s + g][32 * wave + 16 * b + j];
 #pragma unroll
-                    for (int a = 0; a < 8; ++a) {
+                    for (int a = 0; a < NA; ++a) {
                         const double af = cs[cur][4 * s + g][16 * a + j];
 #pragma unroll
                         for (int b = 0; b < 2; ++b)
@@ -248,7 +255,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
             }
 
 #pragma unroll
-            for (int a = 0; a < 8; ++a)
+            for (int a = 0; a < NA; ++a)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int c = c0 + 16 * a + g + 4 * r;
@@ -294,14 +301,20 @@ int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const vo
     int64_t grid = kmx_cdiv(n, GT);
     const int64_t cap = (int64_t)2 * kmx_num_cus();
     if (grid > cap) grid = cap;
-    if (dtype == KMX_F32)
-        hipLaunchKernelGGL(lloyd_gemm_labels_f32_kernel, dim3((unsigned)grid), dim3(256), 0, stream,
-                           (const float*)X_t, (const float*)centroids_t, (const float*)half_norms, labels,
-                           status, n, d, k, x_vec, c_vec);
-    else
-        hipLaunchKernelGGL(lloyd_gemm_labels_f64_kernel, dim3((unsigned)grid), dim3(256), 0, stream,
-                           (const double*)X_t, (const double*)centroids_t, (const double*)half_norms, labels,
-                           status, n, d, k, x_vec, c_vec);
+#define KMX_GEMM_LAUNCH(KERNEL, T)                                                                    \
+    hipLaunchKernelGGL(KERNEL, dim3((unsigned)grid), dim3(256), 0, stream, (const T*)X_t,             \
+                       (const T*)centroids_t, (const T*)half_norms, labels, status, n, d, k, x_vec, c_vec)
+    // centroid tile: 32 / 64 for that few clusters, else 128
+    if (dtype == KMX_F32) {
+        if (k <= 32) KMX_GEMM_LAUNCH(lloyd_gemm_labels_f32_kernel<1>, float);
+        else if (k <= 64) KMX_GEMM_LAUNCH(lloyd_gemm_labels_f32_kernel<2>, float);
+        else KMX_GEMM_LAUNCH(lloyd_gemm_labels_f32_kernel<4>, float);
+    } else {
+        if (k <= 32) KMX_GEMM_LAUNCH(lloyd_gemm_labels_f64_kernel<2>, double);
+        else if (k <= 64) KMX_GEMM_LAUNCH(lloyd_gemm_labels_f64_kernel<4>, double);
+        else KMX_GEMM_LAUNCH(lloyd_gemm_labels_f64_kernel<8>, double);
+    }
+#undef KMX_GEMM_LAUNCH
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

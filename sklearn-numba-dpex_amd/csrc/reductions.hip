@@ -263,6 +263,38 @@ int sum_blocks_per_row(int64_t cols) {
     return (int)(b < 1 ? 1 : b);
 }
 
+
+// dst (cols x rows) = transpose of src (rows x cols), 64 x 64 tiles through LDS (rows padded
+// by one word: the transposed reads fall on distinct banks); both sides move whole segments.
+// One workgroup per tile, tiles numbered along the columns first.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst,
+                                                        int64_t rows, int64_t cols, int64_t tiles_c) {
+    __shared__ T tile[64][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t r0 = ((int64_t)blockIdx.x / tiles_c) * 64, c0 = ((int64_t)blockIdx.x % tiles_c) * 64;
+    const int nr = rows - r0 < 64 ? (int)(rows - r0) : 64, nc = cols - c0 < 64 ? (int)(cols - c0) : 64;
+    if (cols <= 64) {
+        // narrow source: the tile's rows are one contiguous run of nr * cols elements
+        const T* __restrict__ run = src + (size_t)r0 * cols;
+        for (int e = threadIdx.x; e < nr * (int)cols; e += 256) tile[e / (int)cols][e % (int)cols] = run[e];
+    } else {
+#pragma unroll 4
+        for (int i = ty; i < 64; i += 4)
+            if (i < nr && tx < nc) tile[i][tx] = src[(size_t)(r0 + i) * cols + c0 + tx];
+    }
+    __syncthreads();
+    if (rows <= 64) {
+        // narrow result: the tile's columns are one contiguous run of nc * rows elements
+        T* __restrict__ run = dst + (size_t)c0 * rows;
+        for (int e = threadIdx.x; e < nc * (int)rows; e += 256) run[e] = tile[e % (int)rows][e / (int)rows];
+    } else {
+#pragma unroll 4
+        for (int i = ty; i < 64; i += 4)
+            if (i < nc && tx < nr) dst[(size_t)(c0 + i) * rows + r0 + tx] = tile[tx][i];
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -419,6 +451,26 @@ int32_t kmx_half_sq_norms(const void* a_t, void* out, int32_t rows, int32_t cols
     else
         hipLaunchKernelGGL((half_sq_norms_kernel<double>), dim3(grid), dim3(256), 0, stream,
                            (const double*)a_t, (double*)out, rows, cols);
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+int32_t kmx_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int32_t dtype, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(src);
+    KMX_REQUIRE_PTR(dst);
+    if (rows <= 0 || cols <= 0) return KMX_ERR_BAD_SHAPE;
+    KMX_REQUIRE_DTYPE(dtype);
+    if (src == dst) return KMX_ERR_BAD_ARGUMENT;
+    const int64_t tiles_c = kmx_cdiv(cols, 64), tiles = tiles_c * kmx_cdiv(rows, 64);
+    if (tiles > INT32_MAX) return KMX_ERR_BAD_SHAPE;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (dtype == KMX_F32)
+        hipLaunchKernelGGL((transpose_kernel<float>), dim3((unsigned)tiles), dim3(256), 0, stream,
+                           (const float*)src, (float*)dst, rows, cols, tiles_c);
+    else
+        hipLaunchKernelGGL((transpose_kernel<double>), dim3((unsigned)tiles), dim3(256), 0, stream,
+                           (const double*)src, (double*)dst, rows, cols, tiles_c);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

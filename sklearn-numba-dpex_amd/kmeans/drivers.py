@@ -13,7 +13,7 @@ import torch
 from .. import _capi
 from .._capi import LloydStatus, check, lib, ptr
 from ..common._buffers import contiguous, dcode, require_cuda, workspace
-from ..common.kernels import broadcast_rows, divide_by
+from ..common.kernels import broadcast_rows, divide_by, transposed_copy
 from ..common.random import create_xoroshiro128pp_states, get_random_raw, raw_to_uniform
 from ..common.reductions import sum_reduction
 from ..common.topk import topk_idx
@@ -71,7 +71,7 @@ def lloyd(
 
     # the wide fp32 path and the bucketed sums add up each cluster's rows from a row-major copy
     # of X (one transpose per run, n * d extra elements of HBM): whole cache lines per sample
-    X_rm = X_t.T.contiguous() if plan.variant in _ROW_MAJOR_VARIANTS else None
+    X_rm = transposed_copy(X_t) if plan.variant in _ROW_MAJOR_VARIANTS else None
 
     check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), int(max_iter),
                              float(tol), stream),

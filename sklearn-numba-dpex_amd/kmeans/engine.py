@@ -37,6 +37,7 @@ except ImportError:  # stock scikit-learn
 
 
 from ..common._buffers import require_cuda, upload
+from ..common.kernels import transposed_copy
 from .drivers import (
     get_euclidean_distances,
     get_labels_inertia,
@@ -261,7 +262,7 @@ class KMeansEngine(_EngineBase):
             X_t = X_dev.T
             owns_copy = X_dev.data_ptr() != X.data_ptr()
             if not X_t.is_contiguous():
-                X_t = X_t.contiguous()
+                X_t = transposed_copy(X_dev) if X_dev.is_contiguous() else X_t.contiguous()
                 owns_copy = True
         else:
             owns_copy = True  # the upload below is this engine's own device copy
@@ -279,7 +280,7 @@ class KMeansEngine(_EngineBase):
             # upload, then transpose on the device: (d, n) contiguous
             # (through pinned staging buffers when the array is large)
             X_t = upload(np.ascontiguousarray(X_np.T) if X_np.flags.f_contiguous else X_np, self.device)
-            X_t = X_t if X_np.flags.f_contiguous else X_t.T.contiguous()
+            X_t = X_t if X_np.flags.f_contiguous else transposed_copy(X_t)
 
         # prepare_fit centres the data in place when this buffer is not the caller's (or copy_x is off)
         self._owns_X = owns_copy

@@ -333,3 +333,16 @@ def test_distances_with_few_samples_split_the_centroids(cuda):
     got = drivers.get_euclidean_distances(_dev(X.T, cuda), _dev(C.T, cuda)).cpu().numpy()
     np.testing.assert_allclose(got, exact, rtol=1e-5, atol=1e-6)
     assert got[10, 3] == 0.0 and np.isfinite(got).all()
+
+
+@pytest.mark.parametrize("shape", [(5_000, 14), (14, 5_000), (1, 1), (64, 64), (65, 129), (300, 1), (1, 300), (1_000, 784)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_transposed_copy(cuda, shape, dtype):
+    import torch
+
+    from sklearn_numba_dpex_amd.common.kernels import transposed_copy
+
+    a = np.arange(shape[0] * shape[1], dtype=dtype).reshape(shape)
+    got = transposed_copy(_dev(a, cuda))
+    assert got.is_contiguous() and tuple(got.shape) == (shape[1], shape[0])
+    np.testing.assert_array_equal(got.cpu().numpy(), a.T)
