@@ -159,16 +159,17 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     const bool specialised = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE ||
                              L.variant == KMX_VARIANT_MFMA_F64;
     if (n <= INT32_MAX && (!specialised || forced == KMX_VARIANT_GEMM)) {
-        // No specialised fused kernel.  From 16 clusters on, or whenever the accumulators do not
+        // No specialised fused kernel.  Beyond 16 clusters (one window of the streaming kernel; the
+        // measured break-even lies between 16 and 32), or whenever the accumulators do not
         // fit in LDS (float atomics on global copies of the sums are slow on this hardware):
         // labels only, on the matrix cores -- the fp64 kernel when the centroid operands alone
-        // fit in LDS, else the tiled product -- then bucketed sums.  Fewer clusters with
+        // fit in LDS, else the tiled product -- then bucketed sums.  Up to 16 clusters with
         // accumulators in LDS: the fused vector-ALU kernels.
         const bool matrix_ok = forced < 0 || forced == KMX_VARIANT_MFMA || forced == KMX_VARIANT_GEMM;
         if (forced == KMX_VARIANT_GEMM) {
             L.variant = KMX_VARIANT_GEMM;
             L.acc_mode = KMX_ACC_BUCKET;
-        } else if (matrix_ok && (k >= 16 || L.acc_mode == KMX_ACC_GLOBAL)) {
+        } else if (matrix_ok && (k > 16 || L.acc_mode == KMX_ACC_GLOBAL)) {
             L.variant = (dtype == KMX_F64 && kmx_mfma_f64_labels_supported(d, k)) ? KMX_VARIANT_MFMA_F64
                                                                                  : KMX_VARIANT_GEMM;
             L.acc_mode = KMX_ACC_BUCKET;
