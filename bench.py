@@ -364,27 +364,29 @@ def other_shapes():
     """Shapes off the specialised kernels, as users bring them: few clusters of wide samples,
     fp64 with sums beyond LDS, more than 256 features.  Overlapping blobs (the labels keep
     changing), wall time per iteration over iterations 6-13 of the driver's loop."""
-    out = []
-    for name, n, d, k, dtype in (("70000 x 784, 10 clusters, fp32", 70_000, 784, 10, np.float32),
-                                 ("2e6 x 100, 10 clusters, fp32", 2_000_000, 100, 10, np.float32),
-                                 ("1e6 x 100, 100 clusters, fp64", 1_000_000, 100, 100, np.float64),
-                                 ("1e6 x 48, 64 clusters, fp64", 1_000_000, 48, 64, np.float64),
-                                 ("1e5 x 300, 300 clusters, fp32", 100_000, 300, 300, np.float32)):
-        t0 = time.time()
-        rng = np.random.default_rng(n + d + k)
-        centers = (rng.uniform(-1.0, 1.0, (k, d)) * (4.0 / np.sqrt(d))).astype(dtype)  # overlapping blobs
-        X = centers[rng.integers(0, k, n)]
-        X += rng.standard_normal((n, d), dtype=dtype)
-        cfg = {"X": X, "init": X[rng.choice(n, k, replace=False)].copy(), "sample_weight": np.ones(n, dtype=dtype), "k": k}
-        kms, variant, wall_ms = gpu_lloyd_step_time(cfg, 8, consecutive=True)
-        s = np.dtype(dtype).itemsize
-        out.append({"shape": name, "kernel_variant": variant, "ms_per_iter": wall_ms,
-                    "label_and_sum_kernels_ms": float(kms[0]),
-                    "TFLOPs": lloyd_flops(n, d, k) / (wall_ms * 1e-3) / 1e12,
-                    "X_bytes_per_iter_TBs": n * d * s / (wall_ms * 1e-3) / 1e12})
-        log(f"[bench] {name}: variant {variant}, {wall_ms:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
-        del X, cfg
-    return out
+    return [one_shape(*spec) for spec in (("70000 x 784, 10 clusters, fp32", 70_000, 784, 10, np.float32),
+                                          ("2e6 x 100, 10 clusters, fp32", 2_000_000, 100, 10, np.float32),
+                                          ("1e6 x 100, 100 clusters, fp64", 1_000_000, 100, 100, np.float64),
+                                          ("1e6 x 48, 64 clusters, fp64", 1_000_000, 48, 64, np.float64),
+                                          ("1e5 x 300, 300 clusters, fp32", 100_000, 300, 300, np.float32))]
+
+
+def one_shape(name, n, d, k, dtype, reps=8):
+    """Overlapping Gaussian blobs of the given shape: wall time per iteration over iterations
+    6 .. 5 + reps of the driver's loop and the kernel times of a first iteration."""
+    t0 = time.time()
+    rng = np.random.default_rng(n + d + k)
+    centers = (rng.uniform(-1.0, 1.0, (k, d)) * (4.0 / np.sqrt(d))).astype(dtype)  # overlapping blobs
+    X = centers[rng.integers(0, k, n)]
+    X += rng.standard_normal((n, d), dtype=dtype)
+    cfg = {"X": X, "init": X[rng.choice(n, k, replace=False)].copy(), "sample_weight": np.ones(n, dtype=dtype), "k": k}
+    kms, variant, wall_ms = gpu_lloyd_step_time(cfg, reps, consecutive=True)
+    s = np.dtype(dtype).itemsize
+    log(f"[bench] {name}: variant {variant}, {wall_ms:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
+    return {"shape": name, "kernel_variant": variant, "ms_per_iter": wall_ms,
+            "label_and_sum_kernels_ms": float(kms[0]),
+            "TFLOPs": lloyd_flops(n, d, k) / (wall_ms * 1e-3) / 1e12,
+            "X_bytes_per_iter_TBs": n * d * s / (wall_ms * 1e-3) / 1e12}
 
 
 def gpu_components(cfg):
@@ -511,11 +513,19 @@ def main():
     ap.add_argument("--no-kpp", action="store_true", help="skip the kmeans++ leg")
     ap.add_argument("--cpu-iters", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="skip the config 3 / config 5 legs")
+    ap.add_argument("--shape", default=None, metavar="N,D,K,f32|f64",
+                    help="only time Lloyd iterations on synthetic blobs of this shape (one JSON line) and exit")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run five 1 GiB device-to-device copies (calibration of HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    if args.shape:
+        n_s, d_s, k_s, t_s = args.shape.split(",")
+        print(json.dumps(one_shape(f"{n_s} x {d_s}, {k_s} clusters, {t_s}", int(n_s), int(d_s), int(k_s),
+                                   np.float64 if t_s == "f64" else np.float32, reps=max(1, args.steps))), flush=True)
+        return
 
     from sklearn_numba_dpex_amd import datasets
 
