@@ -299,7 +299,9 @@ int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const vo
     auto vec_ok = [&](const void* p, int64_t len) { return (len % per_vec == 0) && ((((uintptr_t)p) & 15) == 0); };
     const int x_vec = vec_ok(X_t, n), c_vec = vec_ok(centroids_t, k);
     int64_t grid = kmx_cdiv(n, GT);
-    const int64_t cap = (int64_t)2 * kmx_num_cus();  // (one workgroup per tile instead measured 4 % slower)
+    // workgroups per compute unit: what registers and LDS allow (one workgroup per tile instead
+    // measured 4 % slower)
+    const int64_t cap = (int64_t)(dtype == KMX_F32 ? 3 : 2) * kmx_num_cus();
     if (grid > cap) grid = cap;
 #define KMX_GEMM_LAUNCH(KERNEL, T)                                                                    \
     hipLaunchKernelGGL(KERNEL, dim3((unsigned)grid), dim3(256), 0, stream, (const T*)X_t,             \

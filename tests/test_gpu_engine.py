@@ -367,3 +367,38 @@ def test_numpy_inputs_are_uploaded_through_pinned_staging(cuda):
     # (four clusters: the vector-ALU step with floating-point atomics, reproducible to rounding only)
     # (one blob sits at the origin: its centroid's coordinates are noise around zero, hence the absolute term)
     np.testing.assert_allclose(_np(a.cluster_centers_), _np(b.cluster_centers_), rtol=1e-5, atol=1e-5)
+
+
+# The same estimator-level comparison (reference test_kmeans.py:28-110) on shapes that take every
+# family of label kernels: screened / all-fp32 / fp64 matrix-core steps, the wide path, the tiled
+# product with bucketed sums, the fp64 matrix-core labels with bucketed sums and the vector-ALU
+# steps.  A fit from the same explicit centres must follow scikit-learn's iterations: same number
+# of iterations, the same labels up to samples on a boundary, inertia and centres to rounding.
+@pytest.mark.parametrize("shape", [(20_000, 14, 127, np.float32, 61), (20_000, 40, 30, np.float32, 31),
+                                   (20_000, 32, 64, np.float64, 51), (6_000, 70, 300, np.float32, 42),
+                                   (6_000, 300, 40, np.float32, 63), (6_000, 100, 100, np.float64, 63),
+                                   (20_000, 32, 400, np.float64, 53), (20_000, 100, 10, np.float32, 1),
+                                   (20_000, 20, 8, np.float64, 11), (1_500, 784, 10, np.float32, 63)])
+def test_fit_follows_scikit_learn_on_every_kernel_family(cuda, shape):
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    n, d, k, dtype, variant = shape
+    assert _capi.lloyd_plan(n, d, k, _capi.dtype_code(dtype), None).variant == variant
+    rng = np.random.default_rng(n + d + k)
+    centers = (rng.uniform(-1.0, 1.0, (k, d)) * (6.0 / np.sqrt(d))).astype(dtype)
+    X = centers[rng.integers(0, k, n)] + rng.standard_normal((n, d)).astype(dtype)
+    init = X[rng.choice(n, k, replace=False)].copy()
+    truth = SkKMeans(n_clusters=k, init=init, n_init=1, max_iter=8, tol=0.0, algorithm="lloyd").fit(X)
+    engine = KMeans(n_clusters=k, init=init, n_init=1, max_iter=8, tol=0.0).fit(X)
+    assert engine.n_iter_ == truth.n_iter_
+    differ = int(np.count_nonzero(_np(engine.labels_) != truth.labels_))
+    assert differ <= n // 1000, f"{differ} labels differ"
+    rtol = 1e-4 if dtype == np.float32 else 1e-9
+    assert_allclose(engine.inertia_, truth.inertia_, rtol=rtol)
+    if differ == 0:
+        assert_allclose(_np(engine.cluster_centers_), truth.cluster_centers_, rtol=rtol, atol=rtol)
+    assert_array_equal(_np(engine.predict(X)), _np(engine.labels_))
+    assert_allclose(_np(engine.transform(X[:256])), truth.transform(X[:256]) if differ == 0 else
+                    np.sqrt(((X[:256, None, :].astype(np.float64) - _np(engine.cluster_centers_)[None]) ** 2).sum(2)),
+                    rtol=rtol * 10, atol=rtol * 10)
