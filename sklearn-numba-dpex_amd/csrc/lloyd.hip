@@ -666,8 +666,10 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
                 KMX_REG_CASE(8, 2);
             else if (d <= 16)
                 KMX_REG_CASE(16, 2);
-            else
+            else if (d <= 32)
                 KMX_REG_CASE(32, 1);
+            else
+                KMX_REG_CASE(64, 1);
         }
 #undef KMX_REG_CASE
     } else {
