@@ -61,6 +61,14 @@ def _small_configs():
         "B32c": lambda: dict(_blob_config(5_001, 300, 20, np.float32, 31), variant=63),
         "B64f": lambda: dict(_blob_config(4_000, 100, 24, np.float64, 32), variant=63),
         "B64g": lambda: dict(_blob_config(4_003, 90, 50, np.float64, 33), variant=63),
+        # few clusters: the register-resident and the streaming vector-ALU steps
+        "R64a": lambda: dict(_blob_config(5_003, 50, 7, np.float64, 34), variant=11),
+        "R32a": lambda: dict(_blob_config(5_003, 40, 8, np.float32, 35), variant=11),
+        "S64a": lambda: dict(_blob_config(5_002, 90, 16, np.float64, 36), variant=1),
+        "S32a": lambda: dict(_blob_config(300_000, 70, 5, np.float32, 37), variant=1),
+        # enough samples for four (fp32) / two (fp64) consecutive samples per thread
+        "S32b": lambda: dict(_blob_config(600_000, 70, 5, np.float32, 38), variant=1),
+        "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
         # fp64 on the matrix cores beyond 32 features (no rows in flight for the next tile) and
         # with accumulators that need most of a compute unit's LDS
         "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=51),
@@ -92,7 +100,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g"])
+                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -152,7 +160,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d",
-                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g"])
+                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
@@ -243,7 +251,7 @@ def n_samples_differ_cap(X):
     return X.shape[0] // 1000
 
 
-@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g"])
+@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a"])
 def test_labels_and_score_paths_on_every_label_kernel(cuda, name):
     """kmx_assign_labels, labels + inertia in one call and the distances on the shapes of the
     tiled matrix-core product, of the labels-only fp64 matrix-core kernel and of the vector-ALU
