@@ -69,6 +69,11 @@ def _small_configs():
         # enough samples for four (fp32) / two (fp64) consecutive samples per thread
         "S32b": lambda: dict(_blob_config(600_000, 70, 5, np.float32, 38), variant=1),
         "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
+        # extremes of the tiled product: thousands of features (many passes of the bucketed sums),
+        # more clusters than the bucket counts hold in LDS and than the wide path takes
+        "X32a": lambda: dict(_blob_config(1_500, 3_000, 20, np.float32, 40), variant=63),
+        "X32b": lambda: dict(_blob_config(30_000, 8, 9_000, np.float32, 41), variant=63),
+        "X64a": lambda: dict(_blob_config(12_000, 3, 5_000, np.float64, 42), variant=63),
         # fp64 on the matrix cores beyond 32 features (no rows in flight for the next tile) and
         # with accumulators that need most of a compute unit's LDS
         "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=51),
@@ -100,7 +105,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b"])
+                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
