@@ -146,8 +146,8 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
  *                                 by the wide fp32 path (plan.variant == 42), which then sums
  *                                 each cluster's rows instead of issuing one global atomic per
  *                                 (sample, feature), and by the bucketed sums (plan.variant
- *                                 3, 13 or 53), which read whole rows from it instead of
- *                                 gathering the feature-major array
+ *                                 63, 53, 13 or 3), which read whole rows from it instead
+ *                                 of gathering the feature-major array
  *   centroids_t      IN   (d, k)  centroids the labels are computed from: the array given to
  *                                 kmx_lloyd_init for the first iteration, then the
  *                                 new_centroids_t of the previous one (the workspace holds a
@@ -210,10 +210,13 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
                           int32_t k, void* stream);
 
 /* Which fused-step kernel kmx_lloyd_iter uses for a shape and flags, as 10 * path + accumulation:
- * path 0 = streaming (wide samples), 1 = register-resident samples, 3 = MFMA (fp32) with the
- * centroids resident in LDS, 4 = MFMA (fp32) with samples in registers and centroids streamed,
- * 5 = MFMA (fp64), 6 = path 3 with the labels screened on the fp16 matrix cores;
- * accumulation 1 = workgroup-private LDS accumulators, 2 = global sums. */
+ * path 0 = streaming vector-ALU step (wide samples, up to 16 clusters), 1 = register-resident
+ * samples (vector ALU), 3 = MFMA (fp32) with the centroids resident in LDS, 4 = MFMA (fp32)
+ * with samples in registers and centroids streamed (more than 256 clusters), 5 = MFMA (fp64)
+ * with the centroids resident in LDS, 6 = labels by a tiled matrix-core product (any shape,
+ * fp32 and fp64); accumulation 1 = workgroup-private LDS accumulators, 2 = global sums,
+ * 3 = labels only, then sums per bucket of samples sorted by label.  61 is path 3 with the
+ * labels screened on the fp16 matrix cores. */
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* ------------------------------------------------------------------------------------ *
