@@ -257,7 +257,7 @@ int32_t kmx_inertia(const void* X_t, const void* sample_weight, const void* cent
                     void* stream);
 
 /* Labels and the weighted inertia of that labelling in one call: kmx_assign_labels followed by
- * kmx_inertia, except that where the screened label kernel applies (fp32, d <= 32) X is read
+ * kmx_inertia, except that where the screened label kernel applies (fp32, d <= 64) X is read
  * once - the kernel sums w_i ||x_i - c_label_i||^2 of its samples on the way.  sample_weight may
  * be NULL (unit weights).  out_total: one element of the compute dtype.  Replaces
  * get_labels_inertia with with_inertia=True and the final E-step of a fit

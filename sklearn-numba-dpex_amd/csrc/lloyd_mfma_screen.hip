@@ -85,7 +85,7 @@ constexpr int SCR_WORD_DELTA = 2;
 #ifndef KMX_SCR_CMPX
 #define KMX_SCR_CMPX 1
 #endif
-constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : 4; }
+constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : (nk == 2 ? 4 : 8); }
 
 struct ScreenLds {
     size_t off_afh, off_afl, off_hneg, off_ct, off_hx, off_queue, total;
@@ -95,9 +95,10 @@ struct ScreenLds {
 };
 constexpr int SCR_QUEUE_MAX = 256;
 // LDS a workgroup may take: the compute unit has 160 KB; one workgroup of twelve waves per
-// compute unit (one K step) can have nearly all of it, two workgroups of four waves (two K
-// steps) half each.  Above 64 KB the kernel needs hipFuncAttributeMaxDynamicSharedMemorySize.
-__host__ __device__ constexpr size_t scr_lds_max(int nk) { return nk == 1 ? 156 * 1024 : 78 * 1024; }
+// compute unit (one K step) or one of eight (three or four K steps: 256 registers per lane
+// leave room for two waves per SIMD) can have nearly all of it, two workgroups of four waves
+// (two K steps) half each.  Above 64 KB the kernel needs hipFuncAttributeMaxDynamicSharedMemorySize.
+__host__ __device__ constexpr size_t scr_lds_max(int nk) { return nk == 2 ? 78 * 1024 : 156 * 1024; }
 __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
     ScreenLds s;
     // (an even number of centroid blocks: the scoring loop takes them in pairs; a block past
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
 
     __shared__ unsigned int xmax_bits;
     __shared__ unsigned int tile_ticket;
-    __shared__ int q_lds[36];  // binary points of the fixed-point sums: features, then the weights
+    __shared__ int q_lds[68];  // binary points of the fixed-point sums: features (d <= 64), then the weights
     if (UPDATE && threadIdx.x <= d) q_lds[threadIdx.x] = q_exp[threadIdx.x];
     if (threadIdx.x == 0) {
         tile_ticket = 0;
@@ -951,7 +952,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 }
             }
         };
-        // (two K steps: the registers do not allow it, the tile's data are requested when it starts)
+        // (more than one K step: the registers do not allow it, the tile's data are requested when it starts)
         constexpr bool AHEAD = NK == 1;
         int wt = tile_of(draw());
         if (AHEAD) request(wt);
@@ -1019,7 +1020,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     {
         const int n_queued = (int)min(queue_count, (unsigned int)q_cap);
         double magic_lane = 0.0;  // lane f: of feature f; lane d: of the weights
-        if (UPDATE && n_queued > 0) magic_lane = fix_magic(q_exp[lane < d ? lane : d]);
+        double magic_w64 = 0.0;   // d = 64 leaves no lane for the weights: lane 0 adds them as well
+        if (UPDATE && n_queued > 0) {
+            magic_lane = fix_magic(q_exp[lane < d ? lane : d]);
+            if (d == 64) magic_w64 = fix_magic(q_exp[64]);
+        }
         for (int e = wave; e < n_queued; e += WAVES) {
             const uint32_t* entry = queue + e * QW;
             const uint32_t sample = entry[Q_INDEX];
@@ -1107,6 +1112,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     const int word = lane < d ? lane : d_even;
                     atomicAdd(acc + bc * acc_stride + word, fixed);
                     if (!full_mode) atomicSub(acc + prev * (uint32_t)acc_stride + word, fixed);
+                }
+                if (d == 64 && lane == 0 && (full_mode || prev != (uint32_t)bc)) {
+                    const unsigned long long fixed = to_fixed_q(wq + magic_w64, magic_w64);
+                    atomicAdd(acc + bc * acc_stride + d_even, fixed);
+                    if (!full_mode) atomicSub(acc + prev * (uint32_t)acc_stride + d_even, fixed);
                 }
             }
         }
@@ -1299,10 +1309,10 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 
 }  // namespace
 
-// Shapes the screened step covers: d <= 32, everything within the workgroup's LDS, byte offsets
+// Shapes the screened step covers: d <= 64 (one to four K steps of 16 features), everything within the workgroup's LDS, byte offsets
 // inside two rows of X_t within 32 bits.
 bool kmx_mfma_screen_fits(int64_t n, int d, int k) {
-    if (d < 1 || d > 32 || k < 16 || n >= ((int64_t)1 << 29)) return false;
+    if (d < 1 || d > 64 || k < 16 || n >= ((int64_t)1 << 29)) return false;
     return screen_lds(d, k, (d + 15) / 16, true).off_queue <= scr_lds_max((d + 15) / 16);
 }
 
@@ -1358,8 +1368,12 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
     } while (0)
     if (nk == 1) {
         if (hk) KMX_SCR_LAUNCH(1, true); else KMX_SCR_LAUNCH(1, false);
-    } else {
+    } else if (nk == 2) {
         if (hk) KMX_SCR_LAUNCH(2, true); else KMX_SCR_LAUNCH(2, false);
+    } else if (nk == 3) {
+        if (hk) KMX_SCR_LAUNCH(3, true); else KMX_SCR_LAUNCH(3, false);
+    } else {
+        if (hk) KMX_SCR_LAUNCH(4, true); else KMX_SCR_LAUNCH(4, false);
     }
 #undef KMX_SCR_LAUNCH
     KMX_LAUNCH_CHECK();

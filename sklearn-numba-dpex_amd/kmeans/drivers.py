@@ -71,7 +71,12 @@ def lloyd(
 
     # the wide fp32 path and the bucketed sums add up each cluster's rows from a row-major copy
     # of X (one transpose per run, n * d extra elements of HBM): whole cache lines per sample
-    X_rm = transposed_copy(X_t) if plan.variant in _ROW_MAJOR_VARIANTS else None
+    X_rm = None
+    if plan.variant in _ROW_MAJOR_VARIANTS:
+        try:
+            X_rm = transposed_copy(X_t)
+        except torch.cuda.OutOfMemoryError:
+            X_rm = None  # the kernels then gather the feature-major array (slower, same results)
 
     check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(sample_weight), ptr(cent[0]), int(max_iter),
                              float(tol), stream),

@@ -89,7 +89,9 @@ def test_kernel_variant_selection():
     from sklearn_numba_dpex_amd._capi import lib
 
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0) == 61   # fp16-screened MFMA + LDS accumulators
-    assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0, 0) == 31   # fp32 MFMA + LDS accumulators
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0, 0) == 61   # three K steps of the screen
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 64, 120, 0, 0) == 61   # four, all of a compute unit's LDS
+    assert lib.kmx_lloyd_kernel_variant(5_000_000, 40, 127, 0, 0x10) == 31  # fp32 MFMA + LDS accumulators
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 4, 127, 0, 0) == 31    # too few features for the screen to pay
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 64, 0, 0) == 61
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 32, 0, 0) == 31

@@ -82,7 +82,10 @@ def _blobs(n, d, k, seed, offset=0.0, scale=1.0):
 @pytest.mark.parametrize("shape", [(20_000, 14, 127), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40),
                                    (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16),
                                    # more than 64 KB of LDS per workgroup
-                                   (20_000, 16, 512), (9_000, 14, 600), (6_000, 8, 512), (5_000, 32, 128)])
+                                   (20_000, 16, 512), (9_000, 14, 600), (6_000, 8, 512), (5_000, 32, 128),
+                                   # three and four K steps (eight waves, the whole LDS of a compute unit)
+                                   (6_000, 33, 16), (6_000, 48, 64), (5_003, 64, 64), (6_000, 40, 127),
+                                   (6_000, 64, 120), (7_001, 63, 20), (6_000, 33, 200)])
 def test_screened_step_matches_oracle(cuda, shape):
     n, d, k = shape
     X, w, init = _blobs(n, d, k, seed=n + d)
@@ -116,7 +119,9 @@ def _labels_only(X, C, cuda, roomy=True, flags=SCREEN):
 
 @pytest.mark.parametrize("shape", [(20_000, 14, 127), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40),
                                    (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16),
-                                   (20_000, 16, 512), (9_000, 14, 600), (5_000, 32, 128)])
+                                   (20_000, 16, 512), (9_000, 14, 600), (5_000, 32, 128),
+                                   (6_000, 33, 16), (6_000, 48, 64), (5_003, 64, 64), (6_000, 40, 127),
+                                   (6_000, 64, 120), (7_001, 63, 20)])
 def test_screened_labels_only_match_oracle(cuda, shape):
     n, d, k = shape
     X, _, init = _blobs(n, d, k, seed=n + d + 1)
@@ -397,6 +402,11 @@ def _screen_cases():
     cases["d=200 random"] = (rng.standard_normal((1_024, 200)).astype(np.float32) * 7,
                              rng.standard_normal((32, 200)).astype(np.float32) * 7)
     cases["d=70"] = (rng.standard_normal((1_024, 70)).astype(np.float32), rng.standard_normal((64, 70)).astype(np.float32))
+    # three and four K steps of the narrow kernel
+    X, _, C = _blobs(3_000, 48, 64, seed=34)
+    cases["blobs d=48 k=64"] = (X, C)
+    X = (rng.standard_normal((2_048, 64)) * 2 + rng.standard_normal(64) * 5).astype(np.float32)
+    cases["d=64, centroids = samples"] = (X, X[:48].copy())
     return cases
 
 
@@ -425,7 +435,8 @@ def test_error_bound_of_the_screen_holds_on_the_hardware(cuda, name):
     assert np.median(bounds) <= 1e-3 * max(typical, np.abs(exact).max() * 1e-3)
 
 
-@pytest.mark.parametrize("shape", [(60_000, 14, 127), (30_001, 9, 45), (40_000, 16, 64), (60_000, 20, 60)])
+@pytest.mark.parametrize("shape", [(60_000, 14, 127), (30_001, 9, 45), (40_000, 16, 64), (60_000, 20, 60),
+                                   (40_000, 48, 40), (40_000, 64, 30)])
 def test_sums_corrected_for_label_changes_equal_rebuilt_sums(cuda, shape):
     """Once few labels change per iteration the screened step no longer rebuilds the fixed-point
     sums but takes every sample that changes cluster off its old cluster and adds it to the new
@@ -613,7 +624,8 @@ def test_many_ties_stay_affordable(cuda):
 
 @pytest.mark.parametrize("shape", [(60_001, 14, 127, np.float32), (20_000, 16, 64, np.float32), (9_000, 20, 40, np.float32),
                                    (5_000, 1, 16, np.float32), (70_000, 9, 300, np.float32),
-                                   (4_000, 40, 20, np.float32), (3_000, 7, 5, np.float32), (6_000, 12, 30, np.float64)])
+                                   (4_000, 40, 20, np.float32), (3_000, 7, 5, np.float32), (6_000, 12, 30, np.float64),
+                                   (9_001, 48, 64, np.float32), (9_000, 64, 100, np.float32)])
 @pytest.mark.parametrize("weighted", [True, False])
 def test_labels_and_inertia_in_one_call(cuda, shape, weighted):
     """kmx_assign_labels_inertia: the labels of kmx_assign_labels and the inertia of kmx_inertia on
