@@ -27,7 +27,7 @@ def _run_iterations(cuda, cfg, n_iter):
     X_rm = torch.as_tensor(X, device=cuda)
     X_t = X_rm.T.contiguous()
     plan = _capi.lloyd_plan(n, d, k, dc, 0)
-    if plan.variant != 42:
+    if plan.variant not in (42, 63, 53, 13, 3):  # the variants that sum rows of a row-major copy
         X_rm = None
     w_d = torch.as_tensor(w, device=cuda)
     cent = [torch.as_tensor(np.ascontiguousarray(init.T), device=cuda), None]
@@ -202,3 +202,29 @@ def test_score_path_and_topk_at_full_size(cuda):
     host = tied.cpu().numpy()
     for k in (16, 1000):
         np.testing.assert_array_equal(topk_idx(tied, k).cpu().numpy(), ok.top_k_indices(host, k))
+
+
+@pytest.mark.parametrize("shape", [(2_000_000, 100, 100, np.float64, 63), (1_000_000, 32, 500, np.float64, 53),
+                                   (500_000, 300, 300, np.float32, 63), (2_000_000, 100, 10, np.float32, 1),
+                                   (2_000_000, 48, 64, np.float32, 61), (1_000_000, 64, 128, np.float64, 51)])
+def test_large_shapes_off_the_benchmark_configurations(cuda, shape):
+    """The same properties on large inputs of the other kernel families: the tiled matrix-core
+    product and the fp64 matrix-core labels with bucketed sums, the streaming vector-ALU step,
+    the screened step with three K steps, the fp64 step with a compute unit's whole LDS."""
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    n, d, k, dtype, variant = shape
+    assert _capi.lloyd_plan(n, d, k, _capi.dtype_code(dtype), 0).variant == variant
+    rng = np.random.default_rng(n + d + k)
+    centers = (rng.uniform(-1.0, 1.0, (k, d)) * (6.0 / np.sqrt(d))).astype(dtype)
+    X = centers[rng.integers(0, k, n)]
+    X += rng.standard_normal((n, d), dtype=dtype)
+    cfg = dict(X=X, init=X[rng.choice(n, k, replace=False)].copy(), sample_weight=rng.uniform(0.5, 1.5, n).astype(dtype), k=k)
+    rtol = 1e-5 if dtype == np.float32 else 1e-12
+    X_t, w_d, recs = _run_iterations(cuda, cfg, 3)
+    ties = sum(_check_iteration(X, X_t, w_d, rec, k, rtol, rng) for rec in recs)
+    print(f"{shape}: {len(recs)} iterations, near-tie label differences on the slices: {ties}")
+    assert len(recs) == 3 and all(r["state"] == 0 for r in recs)
+    inertias = [float(drivers._inertia(X_t, w_d, r["inp"], r["labels"])) for r in recs]
+    assert all(b <= a * (1 + 1e-6) for a, b in zip(inertias, inertias[1:])), inertias
