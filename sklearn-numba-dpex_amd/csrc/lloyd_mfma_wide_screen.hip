@@ -107,18 +107,31 @@ __global__ __launch_bounds__(256) void wide_split_kernel(const float* __restrict
         dst[0] = __builtin_bit_cast(uint4, hi);
         dst[64] = __builtin_bit_cast(uint4, lo);
     }
-    for (int c = blockIdx.x * 256 + threadIdx.x; c < n_cg * CG; c += gridDim.x * 256) {
-        float v = -kmx_inf<float>();
+    // -0.5||c||^2 of the scaled centroids: 64 centroids per workgroup and pass, the features in
+    // four interleaved slices (one per wave) whose partial sums are added in a fixed order
+    __shared__ float part_s[4][64];
+    const int cl = threadIdx.x & 63, fs = threadIdx.x >> 6;
+    for (int c0 = blockIdx.x * 64; c0 < n_cg * CG; c0 += gridDim.x * 64) {
+        const int c = c0 + cl;
+        float sq = 0.0f;
         if (c < k) {
-            float sq = 0.0f;
-            for (int f = 0; f < d; ++f) {
+            for (int f = fs; f < d; f += 4) {
                 const float cv = centroids_t[(size_t)f * k + c] * xs;
                 sq += cv * cv;
             }
-            v = -(sq / 2.0f);
-            atomicMax(header + HDR_HMAX, __float_as_uint(sq / 2.0f));
         }
-        hneg[c] = v;
+        part_s[fs][cl] = sq;
+        __syncthreads();
+        if (fs == 0) {
+            float v = -kmx_inf<float>();
+            if (c < k) {
+                const float tot = (part_s[0][cl] + part_s[1][cl]) + (part_s[2][cl] + part_s[3][cl]);
+                v = -(tot / 2.0f);
+                atomicMax(header + HDR_HMAX, __float_as_uint(tot / 2.0f));
+            }
+            hneg[c] = v;
+        }
+        __syncthreads();
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) header[HDR_SCALE] = __float_as_uint(xs);
 }
