@@ -236,6 +236,18 @@ class KMeansEngine(_EngineBase):
             return array.to(device=self.device, dtype=dtype)
         return torch.as_tensor(np.asarray(array), device=self.device).to(dtype)
 
+    def _assert_all_finite(self, X_t, X_host):
+        """scikit-learn's check of the input (check_array(ensure_all_finite=True), as the
+        reference's engine runs it: kmeans/engine.py:293-302), taken on the device: one pass at
+        memory speed instead of a single-threaded host pass that costs more than the upload.
+        Non-finite data then get scikit-learn's own error from the host copy."""
+        if bool(torch.isfinite(X_t).all()):
+            return
+        from sklearn.utils.validation import _assert_all_finite
+
+        host = X_host if X_host is not None else X_t.T.cpu().numpy()
+        _assert_all_finite(host, input_name="X", estimator_name=type(self.estimator).__name__)
+
     def _validate_data(self, X, reset=True):
         """Returns X on the device as the transposed view of a contiguous (d, n) buffer, dtype
         float64 or float32 (other dtypes are converted to float64, as scikit-learn does)."""
@@ -264,6 +276,7 @@ class KMeansEngine(_EngineBase):
             if not X_t.is_contiguous():
                 X_t = transposed_copy(X_dev) if X_dev.is_contiguous() else X_t.contiguous()
                 owns_copy = True
+            self._assert_all_finite(X_t, None)
         else:
             owns_copy = True  # the upload below is this engine's own device copy
             X_np = check_array(
@@ -272,7 +285,7 @@ class KMeansEngine(_EngineBase):
                 dtype=list(_ACCEPTED_DTYPES),
                 order=None,
                 copy=False,
-                ensure_all_finite=True,
+                ensure_all_finite=False,  # checked on the device below: the host pass costs more than the upload
                 estimator=estimator,
                 input_name="X",
             )
@@ -281,6 +294,7 @@ class KMeansEngine(_EngineBase):
             # (through pinned staging buffers when the array is large)
             X_t = upload(np.ascontiguousarray(X_np.T) if X_np.flags.f_contiguous else X_np, self.device)
             X_t = X_t if X_np.flags.f_contiguous else transposed_copy(X_t)
+            self._assert_all_finite(X_t, X_np)
 
         # prepare_fit centres the data in place when this buffer is not the caller's (or copy_x is off)
         self._owns_X = owns_copy

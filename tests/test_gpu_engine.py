@@ -402,3 +402,28 @@ def test_fit_follows_scikit_learn_on_every_kernel_family(cuda, shape):
     assert_allclose(_np(engine.transform(X[:256])), truth.transform(X[:256]) if differ == 0 else
                     np.sqrt(((X[:256, None, :].astype(np.float64) - _np(engine.cluster_centers_)[None]) ** 2).sum(2)),
                     rtol=rtol * 10, atol=rtol * 10)
+
+
+@pytest.mark.parametrize("bad", [np.nan, np.inf, -np.inf])
+@pytest.mark.parametrize("kind", ["numpy", "torch_cuda"])
+def test_non_finite_input_is_refused_like_scikit_learn(cuda, kind, bad):
+    """The finiteness check runs on the device; the error is scikit-learn's."""
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, _ = make_blobs(n_samples=300, random_state=1)
+    X = X.astype(np.float32)
+    km = KMeans(n_clusters=3, n_init=1, random_state=0).fit(X)
+    X_bad = X.copy()
+    X_bad[17, 1] = bad
+    expected = None
+    try:
+        SkKMeans(n_clusters=3, n_init=1).fit(X_bad)
+    except ValueError as e:
+        expected = str(e)
+    assert expected is not None
+    arg = X_bad if kind == "numpy" else _as_cuda(X_bad, np.float32)
+    for call in (lambda: KMeans(n_clusters=3, n_init=1).fit(arg), lambda: km.predict(arg), lambda: km.transform(arg),
+                 lambda: km.score(arg)):
+        with pytest.raises(ValueError) as err:
+            call()
+        assert str(err.value) == expected
