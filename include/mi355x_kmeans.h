@@ -87,7 +87,7 @@ typedef struct kmx_lloyd_status {
 #define KMX_FLAG_LABELS_MASK 0x00000030u
 #define KMX_FLAG_LABELS_AUTO 0x00u
 #define KMX_FLAG_LABELS_F32 0x10u      /* every product of the fp32 paths taken in fp32       */
-#define KMX_FLAG_LABELS_SCREEN 0x20u   /* fp16 screen + fp32 certificate wherever it fits     */
+#define KMX_FLAG_LABELS_SCREEN 0x20u   /* fp16 screen + fp32 certificate wherever it fits (also the tiled product) */
 #define KMX_FLAG_WGS_PER_CU(x) (((uint32_t)(x) & 0xfu) << 8)  /* 1..8 workgroups per CU; 0: default */
 #define KMX_FLAG_COLS(x) (((uint32_t)(x) & 0x7u) << 12)       /* 2 | 4 sample columns per lane; 0: default */
 

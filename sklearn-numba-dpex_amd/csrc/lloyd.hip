@@ -639,11 +639,15 @@ template <typename T, int ACC>
 void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
                   const T* cpack, const T* half_norms, const uint32_t* labels_prev,
                   uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
-                  hipStream_t stream) {
+                  hipStream_t stream, const unsigned int* screen_absmax = nullptr, char* screen_area = nullptr) {
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_GEMM) {
-        (void)kmx_lloyd_gemm_labels(X_t, centroids_t, half_norms, labels, status, n, d, k,
-                                    sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
+        if (sizeof(T) == 4 && L.gemm_screen && screen_area != nullptr)
+            (void)kmx_lloyd_gemm_screen_labels(X_t, centroids_t, half_norms, screen_absmax, screen_area, labels,
+                                               status, n, d, k, stream);
+        else
+            (void)kmx_lloyd_gemm_labels(X_t, centroids_t, half_norms, labels, status, n, d, k,
+                                        sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
     } else if (L.variant == KMX_VARIANT_MFMA_F64) {
         (void)kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
                                       status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, L.partial_slots(),
@@ -715,7 +719,8 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
         q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
     } else if (L.acc_mode == KMX_ACC_BUCKET) {
         launch_fused<T, ACC_NONE>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
-                                  partial, status, n, d, k, stream);
+                                  partial, status, n, d, k, stream,
+                                  reinterpret_cast<const unsigned int*>(ws + L.off_scales), ws + L.off_wscreen);
         KMX_LAUNCH_CHECK();
         const int32_t rc = kmx_lloyd_bucket_sums(X_t, X_rowmajor, w, labels_prev, labels, partial, status,
                                                  ws + L.off_bucket, n, d, k,
@@ -901,7 +906,8 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),
                            (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
     KMX_LAUNCH_CHECK();
-    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE) {
+    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen) {
+        // (for the screened tiled product: max|x| per feature, from which its scale is taken)
         const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, stream);
         if (rc != KMX_OK) return rc;
     }
@@ -1061,6 +1067,8 @@ int32_t kmx_lloyd_recheck_count(const kmx_lloyd_plan* plan, const void* workspac
         src = (const char*)workspace + L.off_bucket + sizeof(uint32_t);
     else if (L.variant == KMX_VARIANT_MFMA_WIDE && kmx_wide_screen_enabled(n, d, k, L.flags))
         src = kmx_wide_screen_counter((const char*)workspace + L.off_wscreen);
+    else if (L.gemm_screen)
+        src = kmx_gemm_screen_counter((const char*)workspace + L.off_wscreen);
     if (src == nullptr) return KMX_OK;
     hipStream_t stream = (hipStream_t)stream_;
     hipError_t e = hipMemcpyAsync(count_host, src, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
@@ -1090,10 +1098,18 @@ size_t kmx_assign_workspace_bytes(int32_t d, int32_t k, int32_t dtype) {
     return lloyd_layout(1, d, k, dtype, 0).off_bucket;
 }
 
+// Room for the screened tiled product behind the minimal workspace: max|c| per feature (the
+// stand-in for max|x|), then the screen's header and list.
+static size_t assign_gemm_screen_bytes(int64_t n, int d) {
+    return kmx_align256((size_t)d * sizeof(unsigned int)) + kmx_gemm_screen_bytes(n);
+}
+
 size_t kmx_assign_workspace_bytes_for(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags) {
     const size_t base = kmx_assign_workspace_bytes(d, k, dtype);
     if (base == 0 || n <= 0 || dtype != KMX_F32 || !kmx_flags_valid(flags)) return base;
-    if (lloyd_layout(n, d, k, dtype, flags).variant != KMX_VARIANT_MFMA_WIDE) return base;
+    const LloydLayout L = lloyd_layout(n, d, k, dtype, flags);
+    if (L.gemm_screen) return kmx_align256(base) + assign_gemm_screen_bytes(n, d);
+    if (L.variant != KMX_VARIANT_MFMA_WIDE) return base;
     const size_t extra = kmx_assign_wide_screen_bytes(n, d, k, flags);
     return extra ? kmx_align256(base) + extra : base;
 }
@@ -1133,9 +1149,20 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
                                                          k, stream);
             return kmx_assign_labels_mfma_wide_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
         }
+        // the tiled product screened in fp16 when the caller's workspace has room for its list
+        // (kmx_assign_workspace_bytes_for); the scale then comes from the centroids
+        const size_t extra_off = kmx_align256(L.off_bucket);
+        unsigned int* absmax = nullptr;
+        char* area = nullptr;
+        if (L.gemm_screen && workspace_bytes >= extra_off + assign_gemm_screen_bytes(n, d)) {
+            absmax = reinterpret_cast<unsigned int*>(ws + extra_off);
+            area = ws + extra_off + kmx_align256((size_t)d * sizeof(unsigned int));
+            const int32_t rc = kmx_wide_screen_scale_from_centroids(centroids_t, absmax, d, k, stream);
+            if (rc != KMX_OK) return rc;
+        }
         launch_fused<float, ACC_NONE>(L, X_t, nullptr, centroids_t, (const float*)(ws + L.off_cpack),
                                       (const float*)(ws + L.off_half), nullptr, labels, nullptr,
-                                      nullptr, n, d, k, stream);
+                                      nullptr, n, d, k, stream, absmax, area);
     } else {
         hipLaunchKernelGGL((lloyd_pack_kernel<double>), dim3(grid), dim3(256), 0, stream,
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),

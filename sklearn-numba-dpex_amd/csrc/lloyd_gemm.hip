@@ -70,33 +70,72 @@ __device__ __forceinline__ void stage_store_f32(float (*tile)[GLD32], const floa
     }
 }
 
+// The same stage for LISTED samples: column c of the tile is sample cols[.] of X_t (gathered,
+// one load per value); a negative index is a column past the end of the list.
+__device__ __forceinline__ void stage_load_listed_f32(float4 (&r)[2], const float* __restrict__ X_t, int64_t n,
+                                                      const int (&cols)[2][4], int d, int f0) {
+#pragma unroll
+    for (int l = 0; l < 2; ++l) {
+        const int g = threadIdx.x + 256 * l;
+        const int f = f0 + (g >> 5);
+        const bool row_ok = f < d;
+        const float* __restrict__ row = X_t + (size_t)(row_ok ? f : 0) * (size_t)n;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const bool ok = row_ok && cols[l][e] >= 0;
+            const float x = row[ok ? cols[l][e] : 0];
+            v[e] = ok ? x : 0.0f;
+        }
+        r[l] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+}
+
 // NA: 32-centroid row tiles per pass over the features (4: tiles of 128 centroids; 1 or 2 for
 // up to 32 / 64 clusters, where wider tiles would multiply padding).  A stage always copies 128
 // centroid columns; only the first 32 NA are used.
-template <int NA>
+// LISTED: the samples are list[0 .. *list_count) instead of 0 .. n (what a screened label
+// kernel could not certify); a workgroup without a tile of the list leaves at once.
+template <int NA, bool LISTED = false>
 __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
     const float* __restrict__ X_t, const float* __restrict__ centroids_t,
     const float* __restrict__ half_norms, uint32_t* __restrict__ labels,
-    const kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int x_vec, int c_vec) {
+    const kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int x_vec, int c_vec,
+    const int* __restrict__ list = nullptr, const unsigned int* __restrict__ list_count = nullptr) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
+    const int64_t n_work = LISTED ? (int64_t)*list_count : n;
     __shared__ __align__(16) float xs[2][GK32][GLD32];
     __shared__ __align__(16) float cs[2][GK32][GLD32];
     __shared__ float hn[GT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, j = lane & 31;
     const int n_stages = (d + GK32 - 1) / GK32;
-    const int64_t n_tiles = (n + GT - 1) / GT;
+    const int64_t n_tiles = (n_work + GT - 1) / GT;
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t i0 = tile * GT;
         float best = -kmx_inf<float>();
         int bidx = 0;
+        int cols[2][4];  // LISTED: the samples behind the thread's columns of a stage
+        if constexpr (LISTED) {
+#pragma unroll
+            for (int l = 0; l < 2; ++l)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int64_t slot = i0 + 4 * ((threadIdx.x + 256 * l) & 31) + e;
+                    cols[l][e] = slot < n_work ? list[slot] : -1;
+                }
+        }
+        auto load_x = [&](float4(&r)[2], const int f0) {
+            if constexpr (LISTED) stage_load_listed_f32(r, X_t, n, cols, d, f0);
+            else stage_load_f32(r, X_t, n, i0, d, f0, x_vec != 0);
+        };
         for (int c0 = 0; c0 < k; c0 += 32 * NA) {
             __syncthreads();  // the previous tile's reads of hn and of the stage buffers are over
             if (threadIdx.x < GT)
                 hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<float>();
             float4 rx[2], rc[2];
-            stage_load_f32(rx, X_t, n, i0, d, 0, x_vec != 0);
+            load_x(rx, 0);
             stage_load_f32(rc, centroids_t, k, c0, d, 0, c_vec != 0);
             stage_store_f32(xs[0], rx);
             stage_store_f32(cs[0], rc);
@@ -112,7 +151,7 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
             for (int st = 0; st < n_stages; ++st) {
                 const int cur = st & 1;
                 if (st + 1 < n_stages) {
-                    stage_load_f32(rx, X_t, n, i0, d, (st + 1) * GK32, x_vec != 0);
+                    load_x(rx, (st + 1) * GK32);
                     stage_load_f32(rc, centroids_t, k, c0, d, (st + 1) * GK32, c_vec != 0);
                 }
 #pragma unroll
@@ -150,8 +189,8 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
         const float ob = __shfl_xor(best, 32, 64);
         const int oi = __shfl_xor(bidx, 32, 64);
         if (ob > best || (ob == best && oi < bidx)) bidx = oi;
-        const int64_t i = i0 + 32 * wave + j;
-        if (h == 0 && i < n) labels[i] = (uint32_t)bidx;
+        const int64_t slot = i0 + 32 * wave + j;
+        if (h == 0 && slot < n_work) labels[LISTED ? (int64_t)list[slot] : slot] = (uint32_t)bidx;
     }
 }
 
@@ -317,6 +356,29 @@ int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const vo
         else KMX_GEMM_LAUNCH(lloyd_gemm_labels_f64_kernel<8>, double);
     }
 #undef KMX_GEMM_LAUNCH
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+// The fp32 kernel on the samples list[0 .. *list_count) (both on the device): what a screened
+// label kernel could not certify.  The grid covers the worst case; workgroups without a tile
+// of the list leave at once.
+int32_t kmx_lloyd_gemm_labels_listed(const void* X_t, const void* centroids_t, const void* half_norms,
+                                     uint32_t* labels, const kmx_lloyd_status* status, const int* list,
+                                     const unsigned int* list_count, int64_t n, int d, int k,
+                                     hipStream_t stream) {
+    const int c_vec = (k % 4 == 0) && ((((uintptr_t)centroids_t) & 15) == 0);
+    int64_t grid = kmx_cdiv(n, GT);
+    const int64_t cap = (int64_t)3 * kmx_num_cus();
+    if (grid > cap) grid = cap;
+#define KMX_GEMM_LISTED(NA_)                                                                                   \
+    hipLaunchKernelGGL((lloyd_gemm_labels_f32_kernel<NA_, true>), dim3((unsigned)grid), dim3(256), 0, stream,   \
+                       (const float*)X_t, (const float*)centroids_t, (const float*)half_norms, labels, status, \
+                       n, d, k, 0, c_vec, list, list_count)
+    if (k <= 32) KMX_GEMM_LISTED(1);
+    else if (k <= 64) KMX_GEMM_LISTED(2);
+    else KMX_GEMM_LISTED(4);
+#undef KMX_GEMM_LISTED
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

@@ -57,6 +57,18 @@ bool kmx_mfma_f64_labels_supported(int d, int k);  // without the accumulators i
 int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const void* half_norms,
                               uint32_t* labels, const kmx_lloyd_status* status, int64_t n, int d, int k,
                               int32_t dtype, hipStream_t stream);
+int32_t kmx_lloyd_gemm_labels_listed(const void* X_t, const void* centroids_t, const void* half_norms,
+                                     uint32_t* labels, const kmx_lloyd_status* status, const int* list,
+                                     const unsigned int* list_count, int64_t n, int d, int k,
+                                     hipStream_t stream);
+// the same product screened on the fp16 matrix cores (lloyd_gemm_screen.hip), fp32 only
+size_t kmx_gemm_screen_bytes(int64_t n);
+bool kmx_gemm_screen_enabled(int64_t n, int d, int k, uint32_t flags);
+const uint32_t* kmx_gemm_screen_counter(const char* area);
+int32_t kmx_lloyd_gemm_screen_labels(const void* X_t, const void* centroids_t, const void* half_norms,
+                                     const unsigned int* absmax, char* area, uint32_t* labels,
+                                     const kmx_lloyd_status* status, int64_t n, int d, int k,
+                                     hipStream_t stream);
 // bucketed sums (lloyd_bucket.hip)
 size_t kmx_bucket_bytes(int64_t n, int k);
 int32_t kmx_bucket_order(const uint32_t* labels, const int* counts, int* offsets, const int* ranks,
@@ -83,6 +95,7 @@ struct LloydLayout {
     int n_partials;      // slots in `partial` (workgroups for LDS mode, copies for global mode)
     int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
     bool screen;         // KMX_VARIANT_MFMA with fp16-screened labels (variant code 61)
+    bool gemm_screen;    // KMX_VARIANT_GEMM (fp32) with fp16-screened labels
     uint32_t flags;      // the caller's KMX_FLAG_* selection
     int wgs_per_cu;      // workgroups per compute unit asked for (0: the kernel's default)
     int cols;            // sample columns per lane asked for (0: the kernel's default)
@@ -180,6 +193,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
         if (L.acc_mode == KMX_ACC_BUCKET) L.n_partials = 1;
     }
     L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
+    L.gemm_screen = L.variant == KMX_VARIANT_GEMM && dtype == KMX_F32 && kmx_gemm_screen_enabled(n, d, k, flags);
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
     L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));
@@ -200,7 +214,11 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     // wide matrix-core path: header, scaled half norms and fp16 parts of the centroids for the
     // screened label step (lloyd_mfma_wide_screen.hip)
     L.off_wscreen = L.off_bucket + kmx_align256(bucket_bytes);
-    const size_t wscreen_bytes = L.variant == KMX_VARIANT_MFMA_WIDE ? kmx_wide_screen_bytes(n, d, k) : 0;  // (reserved whatever the flags say: the layout does not move with them)
+    // (reserved whatever the flags say: the layout does not move with them); the screened tiled
+    // product (fp32, on request) keeps its header and its list of uncertified samples there
+    const size_t wscreen_bytes = L.variant == KMX_VARIANT_MFMA_WIDE ? kmx_wide_screen_bytes(n, d, k)
+                                 : L.gemm_screen                    ? kmx_gemm_screen_bytes(n)
+                                                                    : 0;
     L.off_partial = L.off_wscreen + kmx_align256(wscreen_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
     const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE;

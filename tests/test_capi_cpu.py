@@ -61,8 +61,11 @@ def test_workspace_queries():
     # the screened fp32 step keeps ||x_i|| per sample: 4 bytes per sample
     assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0, 0) - small - 4 * 4_900_000) < 256
     assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0)
-    # sums beyond LDS off the wide path: sample order and ranks (2 n words) + one copy of the sums
+    # sums beyond LDS off the wide path: sample order and ranks (2 n words) + one copy of the sums;
+    # the screened tiled product (on request) adds its list (n words)
     assert 8_000_000 + 4 * 301 * 1024 < lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) < (16 << 20)
+    assert (lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0x20)
+            >= lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) + 4_000_000)
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 63
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0) == 51
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 32, 500, 1, 0) == 53

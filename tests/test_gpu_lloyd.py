@@ -74,6 +74,11 @@ def _small_configs():
         "X32a": lambda: dict(_blob_config(1_500, 3_000, 20, np.float32, 40), variant=63),
         "X32b": lambda: dict(_blob_config(30_000, 8, 9_000, np.float32, 41), variant=63),
         "X64a": lambda: dict(_blob_config(12_000, 3, 5_000, np.float64, 42), variant=63),
+        # the tiled product screened on the fp16 matrix cores (on request), the uncertified
+        # samples through the listed fp32 pass
+        "G32s": lambda: dict(_blob_config(6_001, 100, 100, np.float32, 43), flags=0x20, variant=63),
+        "G32t": lambda: dict(_blob_config(3_000, 784, 40, np.float32, 44, skew=True), flags=0x20, variant=63),
+        "G32u": lambda: dict(_blob_config(5_000, 70, 20, np.float32, 45), flags=0x20, variant=63),
         # fp64 on the matrix cores beyond 32 features (no rows in flight for the next tile) and
         # with accumulators that need most of a compute unit's LDS
         "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=51),
@@ -105,7 +110,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a"])
+                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -165,7 +170,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d",
-                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a"])
+                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "G32s", "G32t"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is

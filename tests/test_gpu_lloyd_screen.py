@@ -662,3 +662,24 @@ def test_labels_and_inertia_in_one_call(cuda, shape, weighted):
     exact = ((X.astype(np.float64) - centers.astype(np.float64)[got]) ** 2).sum(axis=1)
     exact = float((exact * (w.astype(np.float64) if weighted else 1.0)).sum())
     np.testing.assert_allclose(float(total[0]), exact, rtol=rtol)
+
+
+@pytest.mark.parametrize("shape", [(4_000, 100, 100), (3_001, 300, 40), (2_000, 784, 130), (5_000, 70, 20)])
+def test_tiled_product_screened_on_request(cuda, shape):
+    """KMX_FLAG_LABELS_SCREEN on shapes of the tiled matrix-core product: its fp16-screened version
+    (the uncertified samples through the listed all-fp32 pass) gives the oracle's labels, through
+    kmx_assign_labels with both workspace sizes and through one Lloyd iteration; samples far
+    larger than the centroids (labels only: the scale comes from the centroids) overflow fp16
+    and are all listed."""
+    n, d, k = shape
+    X, w, init = _blobs(n, d, k, seed=n + d + 3)
+    ref = ok.assign_labels(X, init)
+    for roomy in (True, False):
+        labels = _labels_only(X, init, cuda, roomy=roomy, flags=SCREEN)
+        assert_labels_match(labels, ref, X, init)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=SCREEN)
+    assert variant == 63 and 0 < rechecked < n // 2
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+    big = (X * 1000.0).astype(np.float32)
+    labels = _labels_only(big, init, cuda, roomy=True, flags=SCREEN)
+    assert_labels_match(labels, ok.assign_labels(big, init), big, init)
