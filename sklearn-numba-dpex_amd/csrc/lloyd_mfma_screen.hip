@@ -392,7 +392,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     // `x`, `norm_in`, `pl_in`: the lane's rows, the owner's norm and previous label, loaded by the
     // caller (for full tiles: while the previous tile was being scored); `refill` is called once
     // they have been consumed and may load the next tile's into the same variables.
-    auto process = [&](auto nc_tag, auto full_tag, auto&& load, auto&& refill,
+    // `put_label(label, whether the lane owns a sample in range, its index)` writes the label, at
+    // once or (full tiles) together with the next tile's requests.
+    auto process = [&](auto nc_tag, auto full_tag, auto&& load, auto&& refill, auto&& put_label,
                        float(&x)[NK][8][decltype(nc_tag)::value], float& norm_in, uint32_t& pl_in,
                        const int64_t i0) __attribute__((always_inline)) {
         constexpr int NC = decltype(nc_tag)::value;
@@ -402,8 +404,18 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         const bool in_range = FULL || my_idx < n;
 
         // the owner's norm and previous label
+        // (taken here, with the rows: a wait for them further down would also wait for the label
+        // store and the requests issued in between)
         float norm_mine = norm_in;
-        const uint32_t pl_mine = pl_in;
+        uint32_t pl_mine = pl_in;
+        asm volatile("" : "+v"(norm_mine), "+v"(pl_mine));
+        // the A operands of the first centroid block, asked for ahead of the conversion below
+        constexpr bool PIPELINED = KMX_SCR_PIPE && NK == 1 && decltype(nc_tag)::value == 2;
+        v8h ah_first, al_first;
+        if constexpr (PIPELINED) {
+            ah_first = afh[lane];
+            al_first = afl[lane];
+        }
 
         // scaled fp16 split of the B operand: hi = fp16(x * 2^-a), lo = fp16(x * 2^-a - hi), each
         // one mixed-precision fused multiply-add with a single rounding (the product with a power
@@ -568,7 +580,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             }
         };
 
-        if constexpr (KMX_SCR_PIPE && NK == 1 && NC == 2) {
+        if constexpr (PIPELINED) {
             // Software pipeline over the stages (block cb, column t), t fastest: while the vector
             // ALU works through the scores of one stage, the matrix core already forms those of
             // the next (the other column's accumulator), one MFMA of its chain of three issued
@@ -578,8 +590,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             // units take turns.
             v16f a0, a1, hv;  // hv: the accumulators' start, -0.5||c||^2 of the block or (HK) zero
             v8h ahA, alA, ahB, alB;  // A operands of the block at hand and of the next one
-            ahA = afh[lane];
-            alA = afl[lane];
+            ahA = ah_first;
+            alA = al_first;
             if constexpr (HK) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) hv[r] = 0.0f;
@@ -778,7 +790,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             }
         }
 
-        if (in_range && owner) labels[my_idx] = lab_mine;
+        put_label(lab_mine, in_range && owner, my_idx);
 
         if constexpr (INERTIA) {
             // both columns' labels in every lane: the lane takes its features of both samples,
@@ -954,6 +966,16 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         };
         // (more than one K step: the registers do not allow it, the tile's data are requested when it starts)
         constexpr bool AHEAD = NK == 1;
+        // The labels of a tile are written when the NEXT tile has started, just ahead of the
+        // requests for the tile after it: the wave waits for everything it has in flight when it
+        // starts a tile (stores count like loads), and a store issued at the end of a tile would
+        // make it wait for that store's acknowledgement every time.
+        uint32_t lab_pending = 0u;
+        int wt_pending = -1;  // wave-uniform; -1: nothing to write
+        uint32_t* const labels_lane = labels + own_off / 4u;
+        auto write_pending = [&]() __attribute__((always_inline)) {
+            if (wt_pending >= 0) labels_lane[(int64_t)wt_pending * TILE] = lab_pending;
+        };
         int wt = tile_of(draw());
         if (AHEAD) request(wt);
         while (wt < n_main) {  // every wave gets out: the counter only grows
@@ -961,16 +983,25 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const int64_t i0 = (int64_t)wt * TILE + MC * j;
             const int wt_now = wt;
             if (!AHEAD) request(wt_now);
+            uint32_t lab_now = 0u;
             process(
                 Cols2{}, std::true_type{},
                 [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_rows(wt_now, xr); },
                 [&]() __attribute__((always_inline)) {
+                    write_pending();
                     if (AHEAD) request(wt_next);
                 },
+                [&](const uint32_t lab, bool, int64_t) __attribute__((always_inline)) { lab_now = lab; },
                 x, norm_next, pl_next, i0);
+            lab_pending = lab_now;
+            wt_pending = wt_now;
             wt = wt_next;
         }
+        write_pending();
     }
+    auto put_now = [&](const uint32_t lab, const bool mine, const int64_t idx) __attribute__((always_inline)) {
+        if (mine) labels[idx] = lab;
+    };
     // scalar loads of the lane's rows (row d - 1 where the feature does not exist)
     auto load_scalar = [&](auto nc_tag, const int64_t i0, float(&dst)[NK][8][decltype(nc_tag)::value])
                            __attribute__((always_inline)) {
@@ -996,8 +1027,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             uint32_t pl_now = UPDATE ? labels_prev[i0] : 0u;
             process(
                 Cols1{}, std::true_type{},
-                [&](float(&xr)[NK][8][1]) __attribute__((always_inline)) { load_scalar(Cols1{}, i0, xr); }, [] {}, x,
-                norm_now, pl_now, i0);
+                [&](float(&xr)[NK][8][1]) __attribute__((always_inline)) { load_scalar(Cols1{}, i0, xr); }, [] {},
+                put_now, x, norm_now, pl_now, i0);
         }
     }
     // The rest: a partial last tile, or every tile when vector accesses are not legal
@@ -1010,8 +1041,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         uint32_t pl_now = (UPDATE && mine_exists) ? labels_prev[i0 + h] : 0u;
         process(
             Cols2{}, std::false_type{},
-            [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_scalar(Cols2{}, i0, xr); }, [] {}, x,
-            norm_now, pl_now, i0);
+            [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_scalar(Cols2{}, i0, xr); }, [] {},
+            put_now, x, norm_now, pl_now, i0);
     }
 
     // The queue: one wave per entry, lane l on the centroids l, l + 64, ... (fused multiply-adds
