@@ -33,12 +33,20 @@ HIPCC_FLAGS = [
 ]
 
 
+# Per source file.  lloyd_mfma_screen.hip: atomics stay as written - the rewrite of an atomic on a
+# uniform address into a wave-wide reduction reads the returned value at once, and the kernel
+# wants the answer of its chunk counter a tile later, not on the spot.
+EXTRA_FLAGS = {
+    "lloyd_mfma_screen.hip": ["-mllvm", "-amdgpu-atomic-optimizer-strategy=None"],
+}
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
 def _compile(src, obj):
-    cmd = ["hipcc", *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = ["hipcc", *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)

@@ -70,7 +70,6 @@ constexpr int SCR_REDO_COLUMN = 3;  // uncertain samples from which a 32-sample 
 // fp32 by the running iteration, the same of the last finished one, and whether the next step
 // may correct the sums for the label changes only (written by the finalisation).
 constexpr int SCR_WORD_DELTA = 2;
-
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
 #ifndef KMX_SCR_WAVES
 #define KMX_SCR_WAVES 12
@@ -88,12 +87,18 @@ constexpr int SCR_WORD_DELTA = 2;
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : (nk == 2 ? 4 : 8); }
 
 struct ScreenLds {
-    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, off_queue, total;
+    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, off_queue, off_moved, total;
     int kp;       // centroids rounded up to a multiple of 64
     int q_cap;    // entries of the queue of samples the screen could not certify
     int q_words;  // 32-bit words per entry: 16 nk feature values, weight, sample index, old label
+    int m_cap;    // entries of the list of samples that change cluster (fused step)
 };
 constexpr int SCR_QUEUE_MAX = 256;
+// The list serves the iterations that correct the sums (at most one label in 64 changed in the
+// iteration before: about n / 64 / workgroups entries); a tile that finds it full adds its
+// changes on the spot.
+constexpr int SCR_MOVED_MAX = 512;
+constexpr int SCR_MOVED_WORDS = 3;  // sample index, old label, new label
 // LDS a workgroup may take: the compute unit has 160 KB; one workgroup of twelve waves per
 // compute unit (one K step) or one of eight (three or four K steps: 256 registers per lane
 // leave room for two waves per SIMD) can have nearly all of it, two workgroups of four waves
@@ -119,7 +124,10 @@ __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool updat
     const size_t cap = scr_lds_max(nk);
     const size_t room = s.off_queue < cap ? (cap - s.off_queue) / ((size_t)s.q_words * 4) : 0;
     s.q_cap = (int)(room < (size_t)SCR_QUEUE_MAX ? room : (size_t)SCR_QUEUE_MAX);
-    s.total = s.off_queue + (size_t)s.q_cap * s.q_words * 4;
+    s.off_moved = s.off_queue + (size_t)s.q_cap * s.q_words * 4;
+    const size_t room_m = (update && s.off_moved < cap) ? (cap - s.off_moved) / ((size_t)SCR_MOVED_WORDS * 4) : 0;
+    s.m_cap = (int)(room_m < (size_t)SCR_MOVED_MAX ? room_m : (size_t)SCR_MOVED_MAX);
+    s.total = s.off_moved + (size_t)s.m_cap * SCR_MOVED_WORDS * 4;
     return s;
 }
 
@@ -133,6 +141,46 @@ __device__ __forceinline__ unsigned long long to_fixed_q(double v_plus_magic, do
     unsigned int hi;
     asm("v_sub_u32 %0, %1, %2" : "=v"(hi) : "v"(__double2hiint(v_plus_magic)), "v"(__double2hiint(magic)));
     return ((unsigned long long)hi << 32) | (unsigned int)__double2loint(v_plus_magic);
+}
+
+// 2^-a with max|x| * 2^-a in [2^(SCR_SCALE_EXP - 1), 2^SCR_SCALE_EXP) (1 for all-zero or non-finite data)
+__device__ __forceinline__ float screen_scale(const float xmax) {
+    return (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, SCR_SCALE_EXP - 1 - ilogbf(xmax)) : 1.0f;
+}
+
+// The fp16 pair of eight scaled values, as operand registers: hi = fp16(x * 2^-a) and
+// lo = fp16(x * 2^-a - hi), each one mixed-precision fused multiply-add with a single rounding
+// (the product with a power of two and the difference are exact); value i goes to half i % 2 of
+// register i / 2.  `scale` is a scalar operand.
+// Sixteen instructions in ONE statement: between separate statements the compiler pads every
+// dependency on an assembly result with a wait state (it must assume a partial register
+// write).  The real rule - a 16-bit write needs one instruction between it and a read of that
+// register - is kept by the order: the four registers are written in rotation.  The closing
+// s_nop gives a vector-ALU result the two wait states it needs before a matrix instruction may
+// read it.
+__device__ __forceinline__ void split_eight(const float v0, const float v1, const float v2, const float v3,
+                                            const float v4, const float v5, const float v6, const float v7,
+                                            const float scale, unsigned int (&hw)[4], unsigned int (&lw)[4]) {
+    asm("v_fma_mixlo_f16 %0, %8, %16, 0\n\t"
+        "v_fma_mixlo_f16 %1, %10, %16, 0\n\t"
+        "v_fma_mixlo_f16 %2, %12, %16, 0\n\t"
+        "v_fma_mixlo_f16 %3, %14, %16, 0\n\t"
+        "v_fma_mixhi_f16 %0, %9, %16, 0\n\t"
+        "v_fma_mixhi_f16 %1, %11, %16, 0\n\t"
+        "v_fma_mixhi_f16 %2, %13, %16, 0\n\t"
+        "v_fma_mixhi_f16 %3, %15, %16, 0\n\t"
+        "v_fma_mixlo_f16 %4, %8, %16, -%0 op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixlo_f16 %5, %10, %16, -%1 op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixlo_f16 %6, %12, %16, -%2 op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixlo_f16 %7, %14, %16, -%3 op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %4, %9, %16, -%0 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %5, %11, %16, -%1 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %6, %13, %16, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %7, %15, %16, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+        "s_nop 1"
+        : "=&v"(hw[0]), "=&v"(hw[1]), "=&v"(hw[2]), "=&v"(hw[3]), "=&v"(lw[0]), "=&v"(lw[1]), "=&v"(lw[2]),
+          "=&v"(lw[3])
+        : "v"(v0), "v"(v1), "v"(v2), "v"(v3), "v"(v4), "v"(v5), "v"(v6), "v"(v7), "s"(scale));
 }
 
 // One column of 32 samples against all centroids in plain fp32 on the matrix cores
@@ -227,6 +275,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     constexpr int QW = 16 * NK + 4, Q_WEIGHT = 16 * NK, Q_INDEX = 16 * NK + 1, Q_PREV = 16 * NK + 2;
     constexpr uint32_t QUEUE_FREE = 0xffffffffu;
     __shared__ unsigned int queue_count;
+    // Samples that change cluster while the sums are only corrected: (index, old label, new
+    // label), their terms moved from the old to the new cluster after the last tile.
+    uint32_t* moved = reinterpret_cast<uint32_t*>(smem_raw + lay.off_moved);    // [m_cap][3]
+    const int m_cap = lay.m_cap;
+    __shared__ unsigned int moved_count;
     __shared__ unsigned int changed_block;
     __shared__ unsigned int hmax_bits;
     __shared__ unsigned int uncertain_block;
@@ -237,13 +290,82 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     __shared__ int q_lds[68];  // binary points of the fixed-point sums: features (d <= 64), then the weights
     if (UPDATE && threadIdx.x <= d) q_lds[threadIdx.x] = q_exp[threadIdx.x];
     if (threadIdx.x == 0) {
-        tile_ticket = 0;
+        tile_ticket = WAVES;  // (the first WAVES tickets are the waves' own indices)
         changed_block = 0;
         queue_count = 0;
+        moved_count = 0;
         hmax_bits = 0;
         uncertain_block = 0;
         xmax_bits = 0;
     }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, j = lane & 31;
+    const int wt_step = (int)gridDim.x * WAVES;
+    const int wt_first = (int)blockIdx.x * WAVES + wave;
+    const int n_fast = vec_ok ? (int)(n / TILE) : 0;
+    // a last round of full tiles that is at most three quarters full is cut into
+    // single-column tiles of 32 samples, spread over all the waves
+    const int n_rounds = n_fast / wt_step;
+    const int n_left = n_fast - n_rounds * wt_step;
+    const bool halves = n_left > 0 && 4 * (int64_t)n_left <= 3 * (int64_t)wt_step;
+    const int n_main = halves ? n_rounds * wt_step : n_fast;
+
+    // Rows of the lane: feature 2 p + h for the pairs p = 8 s + i, row d - 1 where that feature
+    // does not exist (the centroid operand is zero there, so any finite value will do).  A load
+    // is the scalar address of the tile in row 0 plus a 32-bit byte offset of the lane that does
+    // not change from tile to tile (d * n * 4 < 2^32 is a condition of this path): no vector
+    // arithmetic and no branch per tile.
+    // The loads are buffer loads: resource descriptor (the array) and tile offset in scalar
+    // registers, the lane's offset in one vector register, so a load needs no address arithmetic.
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(X_t), 0, (int)(uint32_t)((uint64_t)d * (uint64_t)n * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t norms_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(UPDATE ? norms : X_t), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t pl_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(UPDATE ? labels_prev : labels), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
+    const uint32_t own_off = (uint32_t)(MC * j + h) * 4u;  // the lane's own sample inside a tile
+    uint32_t row_off[NK][8];
+#pragma unroll
+    for (int s = 0; s < NK; ++s)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int f = 16 * s + 2 * i + h;
+            row_off[s][i] = (uint32_t)(f < d ? f : d - 1) * (uint32_t)n * 4u + (uint32_t)(MC * j) * 4u;
+        }
+    // (the spare slot's constant is put in where the rows are consumed: a select here would make
+    // the wave wait for loads it has only just requested)
+    auto load_rows_raw = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
+        const uint32_t tile = (uint32_t)wt * (uint32_t)(TILE * 4);  // wave-uniform byte offset in row 0
+#pragma unroll
+        for (int s = 0; s < NK; ++s)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const v2u q = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, row_off[s][i], tile, 0);
+                dst[s][i][0] = __uint_as_float(q[0]);
+                dst[s][i][1] = __uint_as_float(q[1]);
+            }
+    };
+    // The rows, norm and previous label of a tile are requested while the tile before it
+    // is scored (they are consumed at the very start of a tile, and nothing else of a tile
+    // can start before them): a wave's own loads then cost it no waiting.
+    float x[NK][8][MC];
+    float norm_next = 0.0f;
+    uint32_t pl_next = 0u;
+    auto request = [&](const int wt_) __attribute__((always_inline)) {
+        if (wt_ < n_main) {  // wave-uniform
+            load_rows_raw(wt_, x);
+            if (UPDATE) {
+                const uint32_t tile = (uint32_t)wt_ * (uint32_t)(TILE * 4);
+                norm_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(norms_rsrc, own_off, tile, 0));
+                pl_next = __builtin_amdgcn_raw_buffer_load_b32(pl_rsrc, own_off, tile, 0);
+            }
+        }
+    };
+    // (more than one K step: the registers do not allow it, the tile's data are requested when it starts)
+    constexpr bool AHEAD = NK == 1;
+    // the wave's first tile: ticket = its index in the workgroup (in a scalar register: tile offsets are scalar operands)
+    const int wt_start = __builtin_amdgcn_readfirstlane((int)blockIdx.x * WAVES + wave);
+
     // Everything below is derived from one pass over the centroids in memory: row f goes to
     // wave f % WAVES, all its loads are in flight together, and the fragments and norms are
     // then computed from the copy in LDS.
@@ -259,14 +381,16 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 ct[f * kp + c] = v;
                 if (!UPDATE) my_absmax = max(my_absmax, __float_as_uint(fabsf(v) * 4.0f));
             }
+        // The wave's first tile is requested here, behind the loads of the centroids (loads
+        // return in order): its rows travel while the operands are prepared.
+        if (AHEAD) request(wt_start);
         __syncthreads();  // the shared words above are zero
         // (non-negative floats order like their bits)
         if (UPDATE ? threadIdx.x < d : my_absmax != 0u) atomicMax(&xmax_bits, my_absmax);
     }
     __syncthreads();
     // 2^-a with max|x| * 2^-a in [2^(SCR_SCALE_EXP - 1), 2^SCR_SCALE_EXP) (1 for all-zero or non-finite data)
-    const float xmax = __uint_as_float(xmax_bits);
-    const float xs = (xmax > 0.0f && xmax < kmx_inf<float>()) ? ldexpf(1.0f, SCR_SCALE_EXP - 1 - ilogbf(xmax)) : 1.0f;
+    const float xs = screen_scale(__uint_as_float(xmax_bits));
     // The four pieces of work below start at different waves (thread index rotated by a third,
     // a half, two thirds of the workgroup): each is a chain of LDS round trips too short to
     // fill the workgroup, and one after the other on the same threads they took 3.7 us.
@@ -345,10 +469,9 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     if (UPDATE)
         for (int jx = rotated(ROT_ZERO); jx < items; jx += THREADS) acc[jx] = 0ull;
     for (int e = rotated(ROT_ZERO); e < q_cap; e += THREADS) queue[e * QW + Q_INDEX] = QUEUE_FREE;
+    for (int e = rotated(ROT_ZERO); e < m_cap; e += THREADS) moved[e * SCR_MOVED_WORDS] = QUEUE_FREE;
     __syncthreads();
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int h = lane >> 5, j = lane & 31;
     const unsigned int h4 = 4u * (unsigned int)h;
     const int n_wtiles = (int)((n + TILE - 1) / TILE);  // n < 2^29: tile and sample indices fit 32 bits
     unsigned int changed = 0;
@@ -417,9 +540,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             al_first = afl[lane];
         }
 
-        // scaled fp16 split of the B operand: hi = fp16(x * 2^-a), lo = fp16(x * 2^-a - hi), each
-        // one mixed-precision fused multiply-add with a single rounding (the product with a power
-        // of two and the difference are exact)
+        // scaled fp16 split of the B operand (split_eight)
         v8h xh[NK][NC], xl[NK][NC];
         float own_sq[NC];  // labels only: the lane's part of ||x||^2, scaled
         {
@@ -433,34 +554,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     // the spare slot's constant (prefetched rows arrive without it)
                     float x7 = x[s][7][t];
                     if (HK && s == NK - 1) x7 = h ? hk_x : x7;
-                    // Sixteen instructions in ONE statement: between separate statements the
-                    // compiler pads every dependency on an assembly result with a wait state
-                    // (it must assume a partial register write).  The real rule - a 16-bit write
-                    // needs one instruction between it and a read of that register - is kept
-                    // by the order: the four registers are written in rotation.  The closing
-                    // s_nop gives a vector-ALU result the two wait states it needs before a
-                    // matrix instruction may read it.
-                    asm("v_fma_mixlo_f16 %0, %8, %16, 0\n\t"
-                        "v_fma_mixlo_f16 %1, %10, %16, 0\n\t"
-                        "v_fma_mixlo_f16 %2, %12, %16, 0\n\t"
-                        "v_fma_mixlo_f16 %3, %14, %16, 0\n\t"
-                        "v_fma_mixhi_f16 %0, %9, %16, 0\n\t"
-                        "v_fma_mixhi_f16 %1, %11, %16, 0\n\t"
-                        "v_fma_mixhi_f16 %2, %13, %16, 0\n\t"
-                        "v_fma_mixhi_f16 %3, %15, %16, 0\n\t"
-                        "v_fma_mixlo_f16 %4, %8, %16, -%0 op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixlo_f16 %5, %10, %16, -%1 op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixlo_f16 %6, %12, %16, -%2 op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixlo_f16 %7, %14, %16, -%3 op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixhi_f16 %4, %9, %16, -%0 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixhi_f16 %5, %11, %16, -%1 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixhi_f16 %6, %13, %16, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
-                        "v_fma_mixhi_f16 %7, %15, %16, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
-                        "s_nop 1"
-                        : "=&v"(hw[0]), "=&v"(hw[1]), "=&v"(hw[2]), "=&v"(hw[3]), "=&v"(lw[0]), "=&v"(lw[1]),
-                          "=&v"(lw[2]), "=&v"(lw[3])
-                        : "v"(x[s][0][t]), "v"(x[s][1][t]), "v"(x[s][2][t]), "v"(x[s][3][t]), "v"(x[s][4][t]),
-                          "v"(x[s][5][t]), "v"(x[s][6][t]), "v"(x7), "s"(xs_sc));
+                    split_eight(x[s][0][t], x[s][1][t], x[s][2][t], x[s][3][t], x[s][4][t], x[s][5][t], x[s][6][t],
+                                x7, xs_sc, hw, lw);
                     if (!UPDATE) {
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
@@ -746,8 +841,6 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         bool queued_mine = false;
         const unsigned long long todo_all = __ballot(unsure_mine);  // bit 32 t + j: sample j of column t
         if (__builtin_expect(todo_all != 0ull, 0)) {                // cold: spills belong in here
-            float xr[NK][8][NC];
-            load(xr);
 #pragma unroll
             for (int t = 0; t < NC; ++t) {
                 const unsigned int todo = (unsigned int)(todo_all >> (32 * t));  // wave-uniform
@@ -763,6 +856,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 }
                 const bool col_mine = NC == 2 ? h == t : true;  // whether the lane's own sample is in column t
                 if (redo) {
+                    float xr[NK][8][NC];
+                    load(xr);
                     ColumnRows rows;
 #pragma unroll
                     for (int s = 0; s < NK; ++s)
@@ -771,20 +866,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     const uint32_t r = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
                     if (col_mine) lab_mine = r;
                 } else if ((todo >> j) & 1u) {  // both lanes of the sample
+                    // (the index alone: the entry's features, weight and previous label are
+                    // fetched after the last tile, all entries of the workgroup at once, so
+                    // that the tile does not wait for a second read of its rows)
                     const unsigned int slot = base + (unsigned int)__popc(todo & ((1u << j) - 1u));
-                    uint32_t* entry = queue + slot * QW;
-#pragma unroll
-                    for (int s = 0; s < NK; ++s)
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) entry[16 * s + 2 * i + h] = __float_as_uint(xr[s][i][t]);
-                    if (h == 0) {
-                        const int64_t idx_t = i0 + t;
-                        entry[Q_WEIGHT] = (UPDATE || (INERTIA && sample_weight != nullptr))
-                                              ? __float_as_uint(sample_weight[idx_t])
-                                              : __float_as_uint(1.0f);
-                        entry[Q_INDEX] = (uint32_t)idx_t;
-                        entry[Q_PREV] = UPDATE ? labels_prev[idx_t] : 0u;
-                    }
+                    if (h == 0) queue[slot * QW + Q_INDEX] = (uint32_t)(i0 + t);
                     if (col_mine) queued_mine = true;
                 }
             }
@@ -830,7 +916,25 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             // which samples the sums have to hear of: all of them when the sums are rebuilt,
             // those that change cluster otherwise (bit 32 t + j: sample j of column t)
             const unsigned long long act_all = __ballot(full_mode ? counted_mine : chg_mine);
-            if (act_all != 0ull) {
+            // Sums only corrected: the few samples that move go on the workgroup's list and are
+            // dealt with after the last tile (one thread per sample and feature, all reads in
+            // flight together); a tile does not read its rows a second time for them.
+            bool listed = false;  // wave-uniform
+            if (act_all != 0ull && !full_mode && m_cap > 0) {
+                const unsigned int n_act = (unsigned int)__popcll(act_all);
+                unsigned int base = 0;
+                if (lane == 0) base = atomicAdd(&moved_count, n_act);
+                base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
+                listed = base + n_act <= (unsigned int)m_cap;
+                if (listed && chg_mine) {
+                    uint32_t* entry =
+                        moved + (base + (unsigned int)__popcll(act_all & ((1ull << lane) - 1ull))) * SCR_MOVED_WORDS;
+                    entry[1] = pl_mine;
+                    entry[2] = lab_mine;
+                    entry[0] = (uint32_t)my_idx;
+                }
+            }
+            if (act_all != 0ull && !listed) {
                 float xr[NK][8][NC];
                 load(xr);
                 // both columns' labels in every lane (the lane adds its features of both samples)
@@ -880,51 +984,6 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         }
     };
 
-    const int wt_step = (int)gridDim.x * WAVES;
-    const int wt_first = (int)blockIdx.x * WAVES + wave;
-    const int n_fast = vec_ok ? (int)(n / TILE) : 0;
-    // a last round of full tiles that is at most three quarters full is cut into
-    // single-column tiles of 32 samples, spread over all the waves
-    const int n_rounds = n_fast / wt_step;
-    const int n_left = n_fast - n_rounds * wt_step;
-    const bool halves = n_left > 0 && 4 * (int64_t)n_left <= 3 * (int64_t)wt_step;
-    const int n_main = halves ? n_rounds * wt_step : n_fast;
-
-    // Rows of the lane: feature 2 p + h for the pairs p = 8 s + i, row d - 1 where that feature
-    // does not exist (the centroid operand is zero there, so any finite value will do).  A load
-    // is the scalar address of the tile in row 0 plus a 32-bit byte offset of the lane that does
-    // not change from tile to tile (d * n * 4 < 2^32 is a condition of this path): no vector
-    // arithmetic and no branch per tile.
-    // The loads are buffer loads: resource descriptor (the array) and tile offset in scalar
-    // registers, the lane's offset in one vector register, so a load needs no address arithmetic.
-    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float*>(X_t), 0, (int)(uint32_t)((uint64_t)d * (uint64_t)n * 4u), 0x00020000);
-    const __amdgpu_buffer_rsrc_t norms_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float*>(UPDATE ? norms : X_t), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
-    const __amdgpu_buffer_rsrc_t pl_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint32_t*>(UPDATE ? labels_prev : labels), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
-    const uint32_t own_off = (uint32_t)(MC * j + h) * 4u;  // the lane's own sample inside a tile
-    uint32_t row_off[NK][8];
-#pragma unroll
-    for (int s = 0; s < NK; ++s)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int f = 16 * s + 2 * i + h;
-            row_off[s][i] = (uint32_t)(f < d ? f : d - 1) * (uint32_t)n * 4u + (uint32_t)(MC * j) * 4u;
-        }
-    // (the spare slot's constant is put in where the rows are consumed: a select here would make
-    // the wave wait for loads it has only just requested)
-    auto load_rows_raw = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
-        const uint32_t tile = (uint32_t)wt * (uint32_t)(TILE * 4);  // wave-uniform byte offset in row 0
-#pragma unroll
-        for (int s = 0; s < NK; ++s)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const v2u q = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, row_off[s][i], tile, 0);
-                dst[s][i][0] = __uint_as_float(q[0]);
-                dst[s][i][1] = __uint_as_float(q[1]);
-            }
-    };
     auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
         load_rows_raw(wt, dst);
         if (HK) {
@@ -948,24 +1007,6 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const int q = __builtin_amdgcn_readfirstlane((int)ticket_);
             return (int)blockIdx.x * WAVES + q % WAVES + (q / WAVES) * wt_step;
         };
-        // The rows, norm and previous label of a tile are requested while the tile before it
-        // is scored (they are consumed at the very start of a tile, and nothing else of a tile
-        // can start before them): a wave's own loads then cost it no waiting.
-        float x[NK][8][MC];
-        float norm_next = 0.0f;
-        uint32_t pl_next = 0u;
-        auto request = [&](const int wt_) __attribute__((always_inline)) {
-            if (wt_ < n_main) {  // wave-uniform
-                load_rows_raw(wt_, x);
-                if (UPDATE) {
-                    const uint32_t tile = (uint32_t)wt_ * (uint32_t)(TILE * 4);
-                    norm_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(norms_rsrc, own_off, tile, 0));
-                    pl_next = __builtin_amdgcn_raw_buffer_load_b32(pl_rsrc, own_off, tile, 0);
-                }
-            }
-        };
-        // (more than one K step: the registers do not allow it, the tile's data are requested when it starts)
-        constexpr bool AHEAD = NK == 1;
         // The labels of a tile are written when the NEXT tile has started, just ahead of the
         // requests for the tile after it: the wave waits for everything it has in flight when it
         // starts a tile (stores count like loads), and a store issued at the end of a tile would
@@ -976,8 +1017,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         auto write_pending = [&]() __attribute__((always_inline)) {
             if (wt_pending >= 0) labels_lane[(int64_t)wt_pending * TILE] = lab_pending;
         };
-        int wt = tile_of(draw());
-        if (AHEAD) request(wt);
+        int wt = wt_start;
         while (wt < n_main) {  // every wave gets out: the counter only grows
             const int wt_next = tile_of(draw());
             const int64_t i0 = (int64_t)wt * TILE + MC * j;
@@ -1047,7 +1087,70 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
 
     // The queue: one wave per entry, lane l on the centroids l, l + 64, ... (fused multiply-adds
     // in feature order from -0.5||c||^2, strict '>' in increasing order), then the wave combines.
-    __syncthreads();  // entries complete; provisional labels have reached memory
+    __syncthreads();  // lists complete; provisional labels have reached memory
+    {
+        // The queue's entries: features in feature order (zero past d), weight, previous label.
+        const int n_queued = (int)min(queue_count, (unsigned int)q_cap);
+        for (int item = threadIdx.x; item < n_queued * QW; item += THREADS) {
+            const int e = item / QW, wq = item - e * QW;
+            const uint32_t sample = queue[e * QW + Q_INDEX];
+            if (sample == QUEUE_FREE || wq == Q_INDEX || wq > Q_PREV) continue;
+            uint32_t v;
+            if (wq < 16 * NK)
+                v = wq < d ? __float_as_uint(X_t[(size_t)wq * n + sample]) : 0u;
+            else if (wq == Q_WEIGHT)
+                v = (UPDATE || (INERTIA && sample_weight != nullptr)) ? __float_as_uint(sample_weight[sample])
+                                                                      : __float_as_uint(1.0f);
+            else
+                v = UPDATE ? labels_prev[sample] : 0u;
+            queue[item] = v;
+        }
+    }
+    if (UPDATE) {
+        // The moved samples: thread (entry, word) takes the term of feature `word` (word d: of the
+        // weight) off the old cluster and adds it to the new one - the same fixed-point terms
+        // a tile would have added.  Four items per thread and pass, their reads issued together.
+        const int n_moved = (int)min(moved_count, (unsigned int)m_cap);
+        const int wpe = d + 1, total = n_moved * wpe;
+        constexpr int U = 4;
+        for (int first = 0; first < total; first += U * THREADS) {
+            float xv[U], wv[U];
+            uint32_t from_c[U], to_c[U];
+            int word[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int item = first + u * THREADS + (int)threadIdx.x;
+                word[u] = -1;
+                xv[u] = 1.0f;
+                wv[u] = 0.0f;
+                from_c[u] = to_c[u] = 0u;
+                if (item < total) {
+                    const int e = item / wpe;
+                    const uint32_t* entry = moved + e * SCR_MOVED_WORDS;
+                    const uint32_t sample = entry[0];
+                    if (sample != QUEUE_FREE) {
+                        word[u] = item - e * wpe;
+                        from_c[u] = entry[1];
+                        to_c[u] = entry[2];
+                        wv[u] = sample_weight[sample];
+                        if (word[u] < d) xv[u] = X_t[(size_t)word[u] * n + sample];
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (word[u] < 0) continue;
+                const double magic = fix_magic(q_lds[word[u]]);
+                // x * w is exact in fp64; one rounding, to a multiple of 2^-q (the weight's word: w itself)
+                const double v = word[u] < d ? fma((double)xv[u], (double)wv[u], magic) : (double)wv[u] + magic;
+                const unsigned long long term = to_fixed_q(v, magic);
+                const int slot = word[u] < d ? word[u] : d_even;
+                atomicAdd(acc + to_c[u] * (uint32_t)acc_stride + slot, term);
+                atomicSub(acc + from_c[u] * (uint32_t)acc_stride + slot, term);
+            }
+        }
+    }
+    __syncthreads();  // entries complete
     {
         const int n_queued = (int)min(queue_count, (unsigned int)q_cap);
         double magic_lane = 0.0;  // lane f: of feature f; lane d: of the weights
