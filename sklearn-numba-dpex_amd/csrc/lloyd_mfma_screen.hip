@@ -183,6 +183,21 @@ __device__ __forceinline__ void split_eight(const float v0, const float v1, cons
         : "v"(v0), "v"(v1), "v"(v2), "v"(v3), "v"(v4), "v"(v5), "v"(v6), "v"(v7), "s"(scale));
 }
 
+// Largest value over the 64 lanes of a wave (all of them active), the same in every lane: within
+// rows of 16 lanes by four data-parallel steps (neighbour, other pair, other quad, other half of
+// the row), then the four rows through scalar registers.
+__device__ __forceinline__ unsigned int wave_umax(unsigned int v) {
+    v = max(v, (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, true));   // quad_perm [1, 0, 3, 2]
+    v = max(v, (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true));   // quad_perm [2, 3, 0, 1]
+    v = max(v, (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, true));  // row_half_mirror
+    v = max(v, (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, true));  // row_mirror
+    const unsigned int r0 = (unsigned int)__builtin_amdgcn_readlane((int)v, 0);
+    const unsigned int r1 = (unsigned int)__builtin_amdgcn_readlane((int)v, 16);
+    const unsigned int r2 = (unsigned int)__builtin_amdgcn_readlane((int)v, 32);
+    const unsigned int r3 = (unsigned int)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(r0, r1), max(r2, r3));
+}
+
 // One column of 32 samples against all centroids in plain fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32 from -0.5||c||^2, lowest index wins a tie): the route for columns with
 // several samples the screen cannot certify.  rows.v[8 s + i] = feature 16 s + 2 i + h of the
@@ -283,7 +298,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     __shared__ unsigned int changed_block;
     __shared__ unsigned int hmax_bits;
     __shared__ unsigned int uncertain_block;
-    __shared__ unsigned long long wave_key[WAVES];
+    __shared__ unsigned long long wave_key[WAVES];  // INERTIA: one fp64 total per wave
 
     __shared__ unsigned int xmax_bits;
     __shared__ unsigned int tile_ticket;
@@ -1166,40 +1181,31 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const float* xe = reinterpret_cast<const float*>(entry);
             float bs = neg_inf;
             int bc = 0x7fffffff;
-            // Two centroids per lane and pass, the features in batches of 8, 4, 2, 1 whose LDS
-            // reads are in flight together; the additions stay in feature order.
+            // Two centroids per lane and pass, sixteen features at a time whose LDS reads are in
+            // flight together (past d the last row is read again and the sum left alone); the
+            // additions stay in feature order.
             for (int c = lane; c < kp; c += 128) {
                 const bool two = c + 64 < kp;  // wave-uniform: kp is a multiple of 64
                 const int c1 = two ? c + 64 : c;
                 const float* col0 = ct + c;
                 const float* col1 = ct + c1;
                 float s0 = -hx[c], s1 = -hx[c1];
-                auto batch = [&](auto nb_tag, const int f0) {
-                    constexpr int NB = decltype(nb_tag)::value;
-                    float xv[NB], a0[NB], a1[NB];
+                for (int f0 = 0; f0 < d; f0 += 16) {
+                    float xv[16], a0[16], a1[16];
 #pragma unroll
-                    for (int i = 0; i < NB; ++i) {
-                        xv[i] = xe[f0 + i];
-                        a0[i] = col0[(f0 + i) * kp];
-                        a1[i] = col1[(f0 + i) * kp];
+                    for (int i = 0; i < 16; ++i) {
+                        const int f = f0 + i < d ? f0 + i : d - 1;  // wave-uniform
+                        xv[i] = xe[f];
+                        a0[i] = col0[f * kp];
+                        a1[i] = col1[f * kp];
                     }
 #pragma unroll
-                    for (int i = 0; i < NB; ++i) {
-                        s0 = fmaf(xv[i], a0[i], s0);
-                        s1 = fmaf(xv[i], a1[i], s1);
+                    for (int i = 0; i < 16; ++i) {
+                        const float t0 = fmaf(xv[i], a0[i], s0), t1 = fmaf(xv[i], a1[i], s1);
+                        s0 = f0 + i < d ? t0 : s0;
+                        s1 = f0 + i < d ? t1 : s1;
                     }
-                };
-                int f = 0;
-                for (; f + 8 <= d; f += 8) batch(std::integral_constant<int, 8>{}, f);
-                if (f + 4 <= d) {
-                    batch(std::integral_constant<int, 4>{}, f);
-                    f += 4;
                 }
-                if (f + 2 <= d) {
-                    batch(std::integral_constant<int, 2>{}, f);
-                    f += 2;
-                }
-                if (f < d) batch(std::integral_constant<int, 1>{}, f);
                 if (s0 > bs) {
                     bs = s0;
                     bc = c;
@@ -1209,17 +1215,12 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     bc = c1;
                 }
             }
-            // one 64-bit key per lane, (score in an order-preserving integer form, ~index):
-            // the largest key is the best score, the lowest index among equal scores; the
-            // wave's LDS word takes the maximum (LDS operations of a wave execute in order)
+            // The wave's best: the largest score (in an order-preserving integer form), then the
+            // lowest index among the lanes that hold it.
             const unsigned int sb = __float_as_uint(bs);
             const unsigned int ordered = sb ^ ((sb >> 31) ? 0xffffffffu : 0x80000000u);
-            const unsigned long long key = ((unsigned long long)ordered << 32) | (unsigned int)~bc;
-            if (lane == 0) wave_key[wave] = 0ull;
-            __builtin_amdgcn_wave_barrier();  // keeps the three accesses in this order
-            atomicMax(&wave_key[wave], key);
-            __builtin_amdgcn_wave_barrier();
-            bc = (int)~(unsigned int)*(volatile unsigned long long*)&wave_key[wave];
+            const unsigned int top = wave_umax(ordered);
+            bc = (int)~wave_umax(ordered == top ? (unsigned int)~bc : 0u);
             if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
             if (lane == 0) {
                 labels[sample] = (uint32_t)bc;
@@ -1261,7 +1262,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     if constexpr (INERTIA) {
         // wave totals in order, then the waves in order
         const double wsum = kmx_wave_sum<double>(inertia_lane);
-        double* wave_tot = reinterpret_cast<double*>(wave_key);  // the queue's keys are no longer needed
+        double* wave_tot = reinterpret_cast<double*>(wave_key);
         __syncthreads();
         if (lane == 0) wave_tot[wave] = wsum;
         __syncthreads();
