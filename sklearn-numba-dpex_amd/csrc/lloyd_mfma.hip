@@ -604,10 +604,16 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         // labels screened on the fp16 matrix cores (lloyd_mfma_screen.hip)
         uint32_t* uncertain = reinterpret_cast<uint32_t*>(ws + L.off_bucket);
         tail.clear_word = uncertain;
-        // sums corrected instead of rebuilt once an iteration changes at most one label in 64
-        // (above that nearly every 64-sample tile holds a change and rebuilding is cheaper)
+        // Sums corrected instead of rebuilt once an iteration changes at most one label in 3
+        // (a sample that moves costs two sets of LDS atomics, one that is rebuilt one).  Up to one
+        // change in 24 the step collects the moving samples and fetches them after its last
+        // tile; above that the fetch (a 64-byte sector per value) would cost more than a second
+        // read of the rows by the tiles.  Measured at 5e6 x 14: a step that rebuilds takes
+        // 130 us, one that corrects from the list 91 us plus about 11 us per percent of labels
+        // that change.
         tail.n_samples = n;
-        tail.delta_divisor = 64;
+        tail.delta_divisor = 3;
+        tail.list_divisor = 24;
         const int32_t rc = kmx_lloyd_step_mfma_screen(
             X_t, w, centroids_t, labels_prev, labels, tail.status,
             reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain,

@@ -67,8 +67,9 @@ constexpr float SCR_ERR_HNEG = 3.0e-7f;  // 2^-22 for the two-part value, 2^-24 
 constexpr int SCR_GROUP = 8;  // accumulator registers per arg-max group
 constexpr int SCR_REDO_COLUMN = 3;  // uncertain samples from which a 32-sample column is redone in fp32
 // Words of the step's counter block in the workspace (`uncertain_count`): samples evaluated in
-// fp32 by the running iteration, the same of the last finished one, and whether the next step
-// may correct the sums for the label changes only (written by the finalisation).
+// fp32 by the running iteration, the same of the last finished one, and how the next step is
+// to bring the sums up to date (written by the finalisation): 0 rebuild them, 1 correct them for
+// the samples that change cluster, collected in the workgroup's list, 2 correct them tile by tile.
 constexpr int SCR_WORD_DELTA = 2;
 // Waves per workgroup (one workgroup per compute unit, or two of four waves).
 #ifndef KMX_SCR_WAVES
@@ -94,10 +95,10 @@ struct ScreenLds {
     int m_cap;    // entries of the list of samples that change cluster (fused step)
 };
 constexpr int SCR_QUEUE_MAX = 256;
-// The list serves the iterations that correct the sums (at most one label in 64 changed in the
-// iteration before: about n / 64 / workgroups entries); a tile that finds it full adds its
+// The list serves the iterations that correct the sums (at most one label in 24 changed in the
+// iteration before: about n / 24 / workgroups entries); a tile that finds it full adds its
 // changes on the spot.
-constexpr int SCR_MOVED_MAX = 512;
+constexpr int SCR_MOVED_MAX = 1024;
 constexpr int SCR_MOVED_WORDS = 3;  // sample index, old label, new label
 // LDS a workgroup may take: the compute unit has 160 KB; one workgroup of twelve waves per
 // compute unit (one K step) or one of eight (three or four K steps: 256 registers per lane
@@ -518,6 +519,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     // fixed-point sums are integers, so taking a sample's terms off its old cluster and adding
     // them to the new one leaves exactly the sums a full pass would produce.
     const bool full_mode = UPDATE ? (uncertain_count[SCR_WORD_DELTA] == 0u) : false;  // wave-uniform
+    // (corrected sums: whether the samples that move are few enough for the workgroup's list)
+    const bool use_list = UPDATE ? (uncertain_count[SCR_WORD_DELTA] == 1u) : false;
 
     // One tile of NC sample columns per lane.  NC = 2: 64 samples, lane (j, h) scores samples
     // i0 and i0 + 1 (i0 = first + 2 j) against its half of every centroid block and, once the
@@ -935,7 +938,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             // dealt with after the last tile (one thread per sample and feature, all reads in
             // flight together); a tile does not read its rows a second time for them.
             bool listed = false;  // wave-uniform
-            if (act_all != 0ull && !full_mode && m_cap > 0) {
+            if (act_all != 0ull && use_list && m_cap > 0) {
                 const unsigned int n_act = (unsigned int)__popcll(act_all);
                 unsigned int base = 0;
                 if (lane == 0) base = atomicAdd(&moved_count, n_act);

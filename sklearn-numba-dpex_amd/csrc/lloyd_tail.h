@@ -20,9 +20,12 @@ struct LloydTail {
     // Screened fused step only: word clear_word[2] tells the next step whether it may correct the
     // fixed-point sums for the samples that change cluster instead of rebuilding them; the sums
     // then stay in `gsum` instead of being cleared.  Chosen when the iteration just finished
-    // changed at most n_samples / delta_divisor labels (0: always rebuild).
+    // changed at most n_samples / delta_divisor labels (0: always rebuild): the word is then 2,
+    // or 1 when it changed at most n_samples / list_divisor labels (few enough for the step to
+    // collect them in a list and deal with them after its last tile).
     int64_t n_samples = 0;
     int delta_divisor = 0;
+    int list_divisor = 0;
 };
 
 // Empty-cluster list (ascending) and heaviest cluster; one workgroup of 256 threads.
@@ -223,7 +226,10 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
         }
         return;
     }
-    if (a.clear_word != nullptr && threadIdx.x == 0) a.clear_word[2] = keep_sums ? 1u : 0u;
+    if (a.clear_word != nullptr && threadIdx.x == 0)
+        a.clear_word[2] = !keep_sums ? 0u
+                          : (a.list_divisor > 0 && (int64_t)a.status->n_changed * a.list_divisor <= a.n_samples) ? 1u
+                                                                                                              : 2u;
     double shift = 0.0;
 #pragma unroll 4
     for (int jx = threadIdx.x; jx < dk; jx += 256) {
