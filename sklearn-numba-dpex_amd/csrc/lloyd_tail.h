@@ -177,6 +177,18 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
     unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<T> a) {
     extern __shared__ __align__(16) unsigned char fin_raw[];
     __shared__ double scratch[4];
+    // The old centroids are asked for before anything else (up to eight values per thread: what
+    // (d + 1) k <= 2048 needs): the kernel is a chain of memory round trips, and this one then
+    // runs beside those of the state and of the sums.
+    constexpr int OLD_AHEAD = 8;
+    const int dk_ahead = a.d * a.k;
+    const bool old_ahead = dk_ahead <= 256 * OLD_AHEAD;
+    T old_v[OLD_AHEAD];
+#pragma unroll
+    for (int i = 0; i < OLD_AHEAD; ++i) {
+        const int jx = (int)threadIdx.x + 256 * i;
+        old_v[i] = (old_ahead && jx < dk_ahead) ? a.old_centroids_t[jx] : T(0);
+    }
     if (a.status->state != KMX_RUNNING) return;
     if (a.clear_word != nullptr && threadIdx.x == 0) {
         a.clear_word[1] = a.clear_word[0];  // kept for kmx_lloyd_recheck_count
@@ -197,7 +209,8 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
             const long long iv = (long long)gsum[jx];
             if (!keep_sums) gsum[jx] = 0ull;
             const int f = jx / k;
-            const T val = (T)ldexp((double)iv, -q_exp[f]);
+            // (times 2^-q, built from its exponent field: exact, like ldexp)
+            const T val = (T)((double)iv * __hiloint2double((1023 - q_exp[f]) << 20, 0));
             vals[jx] = val;
             if (f < d)
                 out_t[jx] = val;
@@ -231,15 +244,24 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
                           : (a.list_divisor > 0 && (int64_t)a.status->n_changed * a.list_divisor <= a.n_samples) ? 1u
                                                                                                               : 2u;
     double shift = 0.0;
-#pragma unroll 4
-    for (int jx = threadIdx.x; jx < dk; jx += 256) {
+    auto divide = [&](const int jx, const T old_value) __attribute__((always_inline)) {
         const int f = jx / k, c = jx - f * k;
         const T nv = vals[jx] / sizes_s[c];
-        const T df = old_t[jx] - nv;
+        const T df = old_value - nv;
         shift += (double)(df * df);
         vals[jx] = nv;
         out_t[jx] = nv;
         a.cpack[(size_t)c * dpad + f] = nv;
+    };
+    if (old_ahead) {  // (the same elements in the same order as the loop below)
+#pragma unroll
+        for (int i = 0; i < OLD_AHEAD; ++i) {
+            const int jx = (int)threadIdx.x + 256 * i;
+            if (jx < dk) divide(jx, old_v[i]);
+        }
+    } else {
+#pragma unroll 4
+        for (int jx = threadIdx.x; jx < dk; jx += 256) divide(jx, old_t[jx]);
     }
     __syncthreads();
     for (int c = threadIdx.x; c < k; c += 256) {
