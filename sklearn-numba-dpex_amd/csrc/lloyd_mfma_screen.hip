@@ -202,12 +202,15 @@ __device__ __forceinline__ unsigned int wave_umax(unsigned int v) {
 // One column of 32 samples against all centroids in plain fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32 from -0.5||c||^2, lowest index wins a tie): the route for columns with
 // several samples the screen cannot certify.  rows.v[8 s + i] = feature 16 s + 2 i + h of the
-// lane's sample; ct (d, kp) and hx (kp) are the fp32 centroids and half norms in LDS.
+// lane's sample (NK K steps of 16 features); ct (d, kp) and hx (kp) are the fp32 centroids and
+// half norms in LDS.
+template <int NK>
 struct ColumnRows {
-    float v[16];
+    float v[8 * NK];
 };
-__device__ __forceinline__ uint32_t redo_column_fp32(ColumnRows rows, const float* ct, const float* hx,
-                                                  int nk, int n_cb, int d, int kp, int h, int j) {
+template <int NK>
+__device__ __forceinline__ uint32_t redo_column_fp32(const ColumnRows<NK>& rows, const float* ct, const float* hx,
+                                                  int n_cb, int d, int kp, int h, int j) {
     float bv = -kmx_inf<float>();
     int bc = 0x7fffffff;
     for (int cb = 0; cb < n_cb; ++cb) {
@@ -215,9 +218,9 @@ __device__ __forceinline__ uint32_t redo_column_fp32(ColumnRows rows, const floa
 #pragma unroll
         for (int r = 0; r < 16; ++r) a[r] = -hx[32 * cb + 8 * (r >> 2) + 4 * h + (r & 3)];
 #pragma unroll
-        for (int p = 0; p < 16; ++p) {
-            const int p0 = 2 * p;  // features p0 + h; wave-uniform guards
-            if (p < 8 * nk && p0 < d) {
+        for (int p = 0; p < 8 * NK; ++p) {
+            const int p0 = 2 * p;  // features p0 + h; wave-uniform guard
+            if (p0 < d) {
                 const bool ok = p0 + h < d;
                 const float af = ok ? ct[(p0 + h) * kp + 32 * cb + j] : 0.0f;
                 const float xv = ok ? rows.v[p] : 0.0f;
@@ -876,12 +879,12 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 if (redo) {
                     float xr[NK][8][NC];
                     load(xr);
-                    ColumnRows rows;
+                    ColumnRows<NK> rows;
 #pragma unroll
                     for (int s = 0; s < NK; ++s)
 #pragma unroll
                         for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = xr[s][i][t];
-                    const uint32_t r = redo_column_fp32(rows, ct, hx, NK, n_cb, d, kp, h, j);
+                    const uint32_t r = redo_column_fp32<NK>(rows, ct, hx, n_cb, d, kp, h, j);
                     if (col_mine) lab_mine = r;
                 } else if ((todo >> j) & 1u) {  // both lanes of the sample
                     // (the index alone: the entry's features, weight and previous label are

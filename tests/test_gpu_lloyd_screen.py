@@ -186,10 +186,12 @@ def test_fp32_matrix_core_step_selected_by_flag(cuda):
     assert_labels_match(got["screen"], got["f32"], X, init)
 
 
-def test_duplicate_centroids_take_the_lowest_index(cuda):
+@pytest.mark.parametrize("d", [14, 24, 40, 64])
+def test_duplicate_centroids_take_the_lowest_index(cuda, d):
     """Two pairs of identical centroids: exact ties, none of them certifiable; the reference's
-    strict '<' in increasing centroid order keeps the lower index."""
-    X, w, init = _blobs(20_000, 14, 64, seed=21)
+    strict '<' in increasing centroid order keeps the lower index.  Whole 32-sample columns are
+    redone in fp32 here, with one to four K steps of 16 features."""
+    X, w, init = _blobs(20_000, d, 64, seed=21)
     init[40] = init[3]
     init[63] = init[17]
     labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
@@ -202,9 +204,10 @@ def test_duplicate_centroids_take_the_lowest_index(cuda):
     assert status.n_empty == 2 and status.state == 4
 
 
-def test_all_centroids_identical(cuda):
+@pytest.mark.parametrize("d", [14, 30, 48, 57])
+def test_all_centroids_identical(cuda, d):
     """No sample can be certified: every label comes from the fp32 evaluation and is 0."""
-    X, w, init = _blobs(5_000, 14, 16, seed=22)
+    X, w, init = _blobs(5_000, d, 16, seed=22)
     init[:] = init[0]
     labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda)
     assert variant == 61
@@ -311,15 +314,30 @@ def test_all_zero_data(cuda):
     assert sizes[0] == 4_096 and status.n_empty == 15
 
 
-def test_ten_iterations_stay_in_lockstep_with_the_oracle(cuda):
-    """Ten iterations through the driver-level loop of the C ABI; every iteration is compared
-    from the centroids the GPU started it with, and the count of fp32 evaluations stays small."""
+@pytest.mark.parametrize("shape,iterations", [((50_000, 14, 127), 10), ((60_000, 9, 45), 25),
+                                              # accumulators and operands fill the LDS: no room for the list of
+                                              # samples that change cluster, little for the queue
+                                              ((20_000, 16, 512), 15), ((30_000, 14, 600), 15),
+                                              # three and four K steps
+                                              ((30_000, 40, 127), 15), ((30_000, 64, 100), 15)])
+def test_iterations_stay_in_lockstep_with_the_oracle(cuda, shape, iterations):
+    """Iterations through the driver-level loop of the C ABI; every iteration is compared from
+    the centroids the GPU started it with - labels against the oracle's, centroids against the
+    weighted means of the labels the GPU wrote, whichever way the step brought its sums up to
+    date (rebuilt, corrected tile by tile, corrected from the list) - and the count of fp32
+    evaluations stays small."""
     import torch
 
     from sklearn_numba_dpex_amd import _capi
     from sklearn_numba_dpex_amd._capi import lib, ptr
 
-    X, w, init = _blobs(50_000, 14, 127, seed=26)
+    X, w, init = _blobs(*shape, seed=26)
+    if shape[1] > 16:
+        # overlapping blobs: no cluster runs empty and the labels keep moving for many iterations
+        rng = np.random.default_rng(26)
+        n_, d_, k_ = shape
+        X = (rng.uniform(-1.5, 1.5, (k_, d_))[rng.integers(0, k_, n_)] + rng.standard_normal((n_, d_))).astype(np.float32)
+        init = X[rng.choice(n_, k_, replace=False)].copy()
     n, d = X.shape
     k = init.shape[0]
     dev = lambda a: torch.as_tensor(np.ascontiguousarray(a), device=cuda)
@@ -336,7 +354,7 @@ def test_ten_iterations_stay_in_lockstep_with_the_oracle(cuda):
     _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 100, 0.0, stream), "init")
     status = _capi.LloydStatus()
     rechecked = ctypes.c_uint32(0)
-    for it in range(10):
+    for it in range(iterations):
         a, b = it % 2, (it + 1) % 2
         c_in = cent[a].cpu().numpy().T.copy()
         _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
@@ -346,7 +364,7 @@ def test_ten_iterations_stay_in_lockstep_with_the_oracle(cuda):
         got = labels[b].cpu().numpy().astype(np.int64)
         assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
         assert rechecked.value <= n // 50
-        if status.n_empty:
+        if status.n_empty or status.state != _capi.KMX_RUNNING:
             break
         sums, ref_sizes = ok.weighted_sums(X, w, got, k)
         assert_centers_close(cent[b].cpu().numpy().T, sums / ref_sizes[:, None], np.float32)
