@@ -169,6 +169,51 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
+@pytest.mark.parametrize("name", ["C2", "M32a", "M32b", "C3", "C3s", "C5", "F64d", "B64a", "B64d", "B64e", "odd", "S64a"])
+def test_duplicate_and_identical_centroids_on_every_kernel_family(cuda, name):
+    """Exact ties: with two centroids duplicated no sample may take the copy with the higher
+    index, with all centroids identical every label is 0 (the reference's strict '<' in
+    increasing centroid order), whichever label kernel the shape selects."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    cfg = _small_configs()[name]()
+    X, w, k = cfg["X"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    dc = _capi.dtype_code(X.dtype)
+    X_t, w_d = _dev(X.T, cuda), _dev(w, cuda)
+    labels_prev = torch.zeros(n, dtype=torch.int32, device=cuda)
+    labels = torch.empty(n, dtype=torch.int32, device=cuda)
+    sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    plan = _capi.lloyd_plan(n, d, k, dc, cfg.get("flags", 0))
+    ws = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+
+    def one_iteration(init):
+        c_in = _dev(init.T, cuda)
+        c_out = torch.empty_like(c_in)
+        _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), plan.workspace_bytes, ptr(X_t), ptr(w_d), ptr(c_in), 100, 0.0,
+                                       stream), "init")
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w_d), ptr(c_in), ptr(c_out), ptr(labels_prev),
+                                       ptr(labels), ptr(sizes), ptr(empty), ptr(ws), plan.workspace_bytes, stream),
+                    "iter")
+        return labels.cpu().numpy().astype(np.int64)
+
+    init = cfg["init"].copy()
+    init[k - 1] = init[0]
+    init[k // 2] = init[1]
+    got = one_iteration(init)
+    assert not np.any(got == k - 1) and not np.any(got == k // 2)
+    assert_labels_match(got, ok.assign_labels(X, init), X, init)
+
+    init = cfg["init"].copy()
+    init[:] = init[0]
+    assert np.all(one_iteration(init) == 0)
+
+
 @pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d",
                                   "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "G32s", "G32t"])
 def test_lockstep_iterations_match_oracle(cuda, name):
