@@ -1450,11 +1450,24 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 
 }  // namespace
 
+// K steps the kernel runs with: as many as the features need - or three for 17 to 32 features
+// whose accumulators and operands do not fit the half of a compute unit's LDS that a workgroup
+// of the two-step kernel gets: the three-step kernel is one workgroup with all of it (its third
+// step then holds no feature: zero operands, exact), which keeps such shapes off the wide path.
+static int screen_k_steps(int d, int k, bool update) {
+    const int nk = (d + 15) / 16;
+    if (nk == 2 && screen_lds(d, k, 2, update).off_queue > scr_lds_max(2) &&
+        screen_lds(d, k, 3, update).off_queue <= scr_lds_max(3))
+        return 3;
+    return nk;
+}
+
 // Shapes the screened step covers: d <= 64 (one to four K steps of 16 features), everything within the workgroup's LDS, byte offsets
 // inside two rows of X_t within 32 bits.
 bool kmx_mfma_screen_fits(int64_t n, int d, int k) {
     if (d < 1 || d > 64 || k < 16 || n >= ((int64_t)1 << 29)) return false;
-    return screen_lds(d, k, (d + 15) / 16, true).off_queue <= scr_lds_max((d + 15) / 16);
+    const int nk = screen_k_steps(d, k, true);
+    return screen_lds(d, k, nk, true).off_queue <= scr_lds_max(nk);
 }
 
 // Left to the library it is chosen where it is the faster one: the all-fp32 step pays d / 2 fp32
@@ -1478,7 +1491,7 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
                       const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream,
                       double* inertia_partial = nullptr, int* grid_out = nullptr) {
     if (!kmx_mfma_screen_fits(n, d, k)) return KMX_ERR_UNSUPPORTED;
-    const int nk = (d + 15) / 16;
+    const int nk = screen_k_steps(d, k, UPDATE);
     const int waves = scr_waves(nk);
     const int64_t n_wtiles = kmx_cdiv(n, 64);
     int64_t grid = kmx_cdiv(n_wtiles, waves);

@@ -85,7 +85,10 @@ def _blobs(n, d, k, seed, offset=0.0, scale=1.0):
                                    (20_000, 16, 512), (9_000, 14, 600), (6_000, 8, 512), (5_000, 32, 128),
                                    # three and four K steps (eight waves, the whole LDS of a compute unit)
                                    (6_000, 33, 16), (6_000, 48, 64), (5_003, 64, 64), (6_000, 40, 127),
-                                   (6_000, 64, 120), (7_001, 63, 20), (6_000, 33, 200)])
+                                   (6_000, 64, 120), (7_001, 63, 20), (6_000, 33, 200),
+                                   # 17 to 32 features that need more than half the LDS of a compute unit: the
+                                   # three-step kernel (one workgroup, all of the LDS) with an empty third step
+                                   (9_000, 20, 300), (8_000, 32, 256), (6_001, 17, 280)])
 def test_screened_step_matches_oracle(cuda, shape):
     n, d, k = shape
     X, w, init = _blobs(n, d, k, seed=n + d)
@@ -121,7 +124,8 @@ def _labels_only(X, C, cuda, roomy=True, flags=SCREEN):
                                    (5_000, 32, 64), (777, 1, 20), (2_000, 2, 33), (64, 31, 16),
                                    (20_000, 16, 512), (9_000, 14, 600), (5_000, 32, 128),
                                    (6_000, 33, 16), (6_000, 48, 64), (5_003, 64, 64), (6_000, 40, 127),
-                                   (6_000, 64, 120), (7_001, 63, 20)])
+                                   (6_000, 64, 120), (7_001, 63, 20),
+                                   (9_000, 20, 300), (8_000, 32, 256), (9_000, 24, 440)])
 def test_screened_labels_only_match_oracle(cuda, shape):
     n, d, k = shape
     X, _, init = _blobs(n, d, k, seed=n + d + 1)
@@ -319,7 +323,9 @@ def test_all_zero_data(cuda):
                                               # samples that change cluster, little for the queue
                                               ((20_000, 16, 512), 15), ((30_000, 14, 600), 15),
                                               # three and four K steps
-                                              ((30_000, 40, 127), 15), ((30_000, 64, 100), 15)])
+                                              ((30_000, 40, 127), 15), ((30_000, 64, 100), 15),
+                                              # two K steps' worth of features on the three-step kernel
+                                              ((30_000, 20, 300), 15), ((30_000, 32, 256), 12)])
 def test_iterations_stay_in_lockstep_with_the_oracle(cuda, shape, iterations):
     """Iterations through the driver-level loop of the C ABI; every iteration is compared from
     the centroids the GPU started it with - labels against the oracle's, centroids against the
