@@ -642,7 +642,9 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
                   hipStream_t stream, const unsigned int* screen_absmax = nullptr, char* screen_area = nullptr) {
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_GEMM) {
-        if (sizeof(T) == 4 && L.gemm_screen && screen_area != nullptr)
+        if (sizeof(T) == 4 && L.screen_labels)
+            (void)kmx_lloyd_labels_mfma_screen(X_t, centroids_t, labels, status, n, d, k, L.wgs_per_cu, stream);
+        else if (sizeof(T) == 4 && L.gemm_screen && screen_area != nullptr)
             (void)kmx_lloyd_gemm_screen_labels(X_t, centroids_t, half_norms, screen_absmax, screen_area, labels,
                                                status, n, d, k, stream);
         else
@@ -1132,7 +1134,8 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32) {
         // labels screened on the fp16 matrix cores: one kernel, straight from the centroids
-        if (L.screen) return kmx_assign_labels_mfma_screen(X_t, centroids_t, labels, n, d, k, L.wgs_per_cu, stream);
+        if (L.screen || L.screen_labels)
+            return kmx_assign_labels_mfma_screen(X_t, centroids_t, labels, n, d, k, L.wgs_per_cu, stream);
         hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
                            (const float*)centroids_t, (float*)(ws + L.off_cpack),
                            (float*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
@@ -1211,7 +1214,7 @@ int32_t kmx_assign_labels_inertia(const void* X_t, const void* sample_weight, co
     double* partial = (double*)(ws + assign_bytes);
     hipStream_t stream = (hipStream_t)stream_;
     const LloydLayout L = lloyd_layout(n, d, k, dtype, flags);
-    if (dtype == KMX_F32 && L.screen) {
+    if (dtype == KMX_F32 && (L.screen || L.screen_labels)) {
         // one pass over X: the screened label kernel sums the inertia on the way
         int n_partials = 0;
         const int32_t rc = kmx_assign_labels_inertia_mfma_screen(X_t, sample_weight, centroids_t, labels, partial,

@@ -82,6 +82,11 @@ int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const voi
 // break-even) select it
 bool kmx_mfma_screen_fits(int64_t n, int d, int k);
 bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags);
+// the same kernel without the sums (labels only): needs less LDS
+bool kmx_mfma_screen_labels_fits(int64_t n, int d, int k);
+int32_t kmx_lloyd_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
+                                     kmx_lloyd_status* status, int64_t n, int d, int k, int wgs_per_cu,
+                                     hipStream_t stream);
 // screened label step of the wide path (lloyd_mfma_wide_screen.hip)
 size_t kmx_wide_screen_bytes(int64_t n, int d, int k);
 const int* kmx_wide_screen_list(const char* area, int d, int k);
@@ -96,6 +101,7 @@ struct LloydLayout {
     int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
     bool screen;         // KMX_VARIANT_MFMA with fp16-screened labels (variant code 61)
     bool gemm_screen;    // KMX_VARIANT_GEMM (fp32) with fp16-screened labels
+    bool screen_labels;  // KMX_VARIANT_GEMM (fp32, d <= 64): labels by the screened kernel of variant 61 without its sums
     uint32_t flags;      // the caller's KMX_FLAG_* selection
     int wgs_per_cu;      // workgroups per compute unit asked for (0: the kernel's default)
     int cols;            // sample columns per lane asked for (0: the kernel's default)
@@ -132,6 +138,9 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     const bool reg_ok = d <= 64;
     L.variant = reg_ok ? KMX_VARIANT_REGISTER : KMX_VARIANT_STREAM;
     const int forced = kmx_flags_forced_variant(flags);
+    const bool screen_labels_ok = dtype == KMX_F32 && n <= INT32_MAX &&
+                                  (flags & KMX_FLAG_LABELS_MASK) != KMX_FLAG_LABELS_F32 &&
+                                  kmx_mfma_screen_labels_fits(n, d, k);
     if (forced == KMX_VARIANT_STREAM) L.variant = KMX_VARIANT_STREAM;
     if (forced == KMX_VARIANT_REGISTER && reg_ok) L.variant = KMX_VARIANT_REGISTER;
     if (items * sizeof(double) <= KMX_LDS_ACC_LIMIT) {
@@ -154,9 +163,11 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
         L.acc_mode = KMX_ACC_LDS;
         L.n_partials = KMX_MAX_PARTIALS;
     }
-    // (the wide path is built for many clusters: up to 256 the tiled product below is faster)
+    // (the wide path is built for many clusters: up to 256 the tiled product below is faster; and
+    // up to 64 features the labels-only form of the screened kernel above, where its operands fit
+    // the LDS, with sums per bucket of samples, is faster than either)
     else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) &&
-             ((forced < 0 && k > 256) || forced == KMX_VARIANT_MFMA)) {
+             ((forced < 0 && k > 256 && !screen_labels_ok) || forced == KMX_VARIANT_MFMA)) {
         L.variant = KMX_VARIANT_MFMA_WIDE;
         L.acc_mode = KMX_ACC_GLOBAL;  // always the global fixed-point sums (variant code 42)
     }
@@ -194,6 +205,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     }
     L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
     L.gemm_screen = L.variant == KMX_VARIANT_GEMM && dtype == KMX_F32 && kmx_gemm_screen_enabled(n, d, k, flags);
+    L.screen_labels = L.variant == KMX_VARIANT_GEMM && screen_labels_ok && !L.gemm_screen && forced != KMX_VARIANT_GEMM;
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
     L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));

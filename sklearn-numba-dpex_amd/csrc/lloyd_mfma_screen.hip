@@ -256,7 +256,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     const float* __restrict__ norms, int64_t n, int d, int k, int vec_ok,
     double* __restrict__ inertia_partial = nullptr) {
     static_assert(!(UPDATE && INERTIA), "the inertia rides with the labels-only kernel");
-    if (UPDATE && status->state != KMX_RUNNING) return;
+    // (labels only: `status` is null outside the iteration loop)
+    if ((UPDATE || status != nullptr) && status->state != KMX_RUNNING) return;
 
     constexpr int WAVES = scr_waves(NK), THREADS = 64 * WAVES;
     constexpr int MC = 2, TILE = 64;
@@ -1470,6 +1471,14 @@ bool kmx_mfma_screen_fits(int64_t n, int d, int k) {
     return screen_lds(d, k, nk, true).off_queue <= scr_lds_max(nk);
 }
 
+// The labels-only kernel needs no accumulators: shapes whose fused step does not fit the LDS
+// can still have their labels screened (the sums are then taken per bucket of samples).
+bool kmx_mfma_screen_labels_fits(int64_t n, int d, int k) {
+    if (d < 1 || d > 64 || k < 16 || n >= ((int64_t)1 << 29)) return false;
+    const int nk = screen_k_steps(d, k, false);
+    return screen_lds(d, k, nk, false).off_queue <= scr_lds_max(nk);
+}
+
 // Left to the library it is chosen where it is the faster one: the all-fp32 step pays d / 2 fp32
 // MFMAs per block of 32 centroids, the screen three fp16 ones plus the split and the certificate
 // whatever d is; measured on 2e6 samples the screen wins from d = 10 on, from d = 8 for k >= 64
@@ -1490,7 +1499,7 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
                       const int* q_exp, unsigned long long* gsum, uint32_t* uncertain_count,
                       const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream,
                       double* inertia_partial = nullptr, int* grid_out = nullptr) {
-    if (!kmx_mfma_screen_fits(n, d, k)) return KMX_ERR_UNSUPPORTED;
+    if (!(UPDATE ? kmx_mfma_screen_fits(n, d, k) : kmx_mfma_screen_labels_fits(n, d, k))) return KMX_ERR_UNSUPPORTED;
     const int nk = screen_k_steps(d, k, UPDATE);
     const int waves = scr_waves(nk);
     const int64_t n_wtiles = kmx_cdiv(n, 64);
@@ -1556,6 +1565,14 @@ int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, 
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
     return launch_screen<false>(X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr, nullptr,
                                 nullptr, nullptr, nullptr, n, d, k, wgs_per_cu, stream);
+}
+
+// The same inside the iteration loop (no work once the run's state is terminal).
+int32_t kmx_lloyd_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
+                                     kmx_lloyd_status* status, int64_t n, int d, int k, int wgs_per_cu,
+                                     hipStream_t stream) {
+    return launch_screen<false>(X_t, nullptr, centroids_t, nullptr, labels, status, nullptr, nullptr, nullptr,
+                                nullptr, nullptr, n, d, k, wgs_per_cu, stream);
 }
 
 // The same with the weighted inertia of the labelling summed on the way: one fp64 partial sum per

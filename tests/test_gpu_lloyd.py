@@ -46,7 +46,10 @@ def _small_configs():
         # the same with the screen switched off, and a shape whose accumulators exceed what any
         # kernel keeps in LDS: the wide path with one chunk of features (d <= 32)
         "M32e": lambda: dict(_blob_config(20_000, 14, 600, np.float32, 18), flags=0x10, variant=42),
-        "M32f": lambda: dict(_blob_config(20_000, 14, 700, np.float32, 20), variant=42),
+        # beyond the LDS of the fused screened step: its labels-only form with sums per bucket of
+        # samples; the wide path on request
+        "M32f": lambda: dict(_blob_config(20_000, 14, 700, np.float32, 20), variant=63),
+        "M32g": lambda: dict(_blob_config(20_000, 14, 700, np.float32, 20), flags=0x3, variant=42),
         # accumulators beyond LDS off the wide fp32 path: a labels-only kernel (fp64 matrix cores
         # where the centroids fit, else vector ALU) and sums per bucket of samples
         "F64d": lambda: dict(_blob_config(20_000, 32, 500, np.float64, 19), variant=53),
@@ -109,7 +112,7 @@ def _odd_config():
 
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
-                                  "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "F64d", "F64e", "F64f",
+                                  "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
                                   "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
