@@ -123,14 +123,16 @@ __device__ __forceinline__ double read_lane(double v, int src) {
 // ROW_MAJOR: X is the n x d copy (a sample's features are contiguous), else the d x n array.
 // Sums are taken in fp64 whatever T is; the workgroup adds one total per feature and per
 // cluster segment of its chunk to `sums` ((d + 1) x k, feature-major, the weights last).
-// Clears counts for the next iteration.
-template <typename T, bool ROW_MAJOR>
+// Clears counts for the next iteration.  NJ: features per lane and pass (64 NJ features per
+// pass; one for arrays of up to 64 features, which then pay for one load and one product per
+// lane and sample and not for four).
+template <typename T, bool ROW_MAJOR, int NJ>
 __global__ __launch_bounds__(256) void bucket_sum_kernel(
     const T* __restrict__ X, const T* __restrict__ sample_weight, const int* __restrict__ order,
     const int* __restrict__ offsets, int* __restrict__ counts, T* __restrict__ sums,
     const kmx_lloyd_status* __restrict__ status, int n, int d, int k) {
     if (status->state != KMX_RUNNING) return;
-    constexpr int FB = 256;  // features per pass: four per lane
+    constexpr int FB = 64 * NJ;  // features per pass
     __shared__ double red[4][FB + 1];
     __shared__ int c_first;
     const int P0 = blockIdx.x * BUCKET_CHUNK;
@@ -147,10 +149,10 @@ __global__ __launch_bounds__(256) void bucket_sum_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
     for (int fb = 0; fb < d; fb += FB) {
-        size_t col[4];   // the lane's features of this pass (clamped: past d the value is dropped)
-        bool live[4];
+        size_t col[NJ];   // the lane's features of this pass (clamped: past d the value is dropped)
+        bool live[NJ];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
             const int f = fb + lane + 64 * j;
             live[j] = f < d;
             const int fc = live[j] ? f : d - 1;
@@ -162,7 +164,9 @@ __global__ __launch_bounds__(256) void bucket_sum_kernel(
             const int c_end = offsets[c + 1];  // wave-uniform
             const int p0 = pos, p1 = c_end < P1 ? c_end : P1;
             if (p1 > p0) {
-                double acc[4] = {0.0, 0.0, 0.0, 0.0};
+                double acc[NJ];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[j] = 0.0;
                 double wsum = 0.0;
                 // each lane fetches one sample index and its weight (a coalesced load and a
                 // gather per 64 samples); lanes past the end hold the last sample, weight 0
@@ -172,7 +176,7 @@ __global__ __launch_bounds__(256) void bucket_sum_kernel(
                     const double my_w = pl < p1 ? (double)sample_weight[my_idx] : 0.0;
                     const int n_here = p1 - base < 64 ? p1 - base : 64;
                     for (int u0 = wave; u0 < n_here; u0 += 4 * U) {
-                        T xv[U][4];
+                        T xv[U][NJ];
                         double wv[U];
 #pragma unroll
                         for (int u = 0; u < U; ++u) {
@@ -181,19 +185,19 @@ __global__ __launch_bounds__(256) void bucket_sum_kernel(
                             wv[u] = src < n_here ? read_lane(my_w, src & 63) : 0.0;
                             const T* __restrict__ row = ROW_MAJOR ? X + (size_t)idx * (size_t)d : X + idx;
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) xv[u][j] = row[col[j]];
+                            for (int j = 0; j < NJ; ++j) xv[u][j] = row[col[j]];
                         }
 #pragma unroll
                         for (int u = 0; u < U; ++u) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) acc[j] = fma((double)xv[u][j], wv[u], acc[j]);
+                            for (int j = 0; j < NJ; ++j) acc[j] = fma((double)xv[u][j], wv[u], acc[j]);
                             wsum += wv[u];
                         }
                     }
                 }
                 // the four waves' totals meet in LDS; one global atomic per feature and segment
 #pragma unroll
-                for (int j = 0; j < 4; ++j) red[wave][lane + 64 * j] = live[j] ? acc[j] : 0.0;
+                for (int j = 0; j < NJ; ++j) red[wave][lane + 64 * j] = live[j] ? acc[j] : 0.0;
                 if (lane == 0) red[wave][FB] = wsum;
                 __syncthreads();
                 {
@@ -253,9 +257,15 @@ int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const voi
     const int32_t rc = kmx_bucket_order(labels, counts, offsets, ranks, order, n, k, stream);
     if (rc != KMX_OK) return rc;
     const unsigned ag = (unsigned)kmx_cdiv(n, BUCKET_CHUNK);
-#define KMX_BUCKET_SUM(T, RM, XP)                                                                  \
-    hipLaunchKernelGGL((bucket_sum_kernel<T, RM>), dim3(ag), dim3(256), 0, stream, (const T*)(XP), \
+#define KMX_BUCKET_SUM_NJ(T, RM, XP, NJ_)                                                                \
+    hipLaunchKernelGGL((bucket_sum_kernel<T, RM, NJ_>), dim3(ag), dim3(256), 0, stream, (const T*)(XP), \
                        (const T*)w, order, offsets, counts, (T*)sums, status, (int)n, d, k)
+#define KMX_BUCKET_SUM(T, RM, XP)                      \
+    do {                                               \
+        if (d <= 64) KMX_BUCKET_SUM_NJ(T, RM, XP, 1);  \
+        else if (d <= 128) KMX_BUCKET_SUM_NJ(T, RM, XP, 2); \
+        else KMX_BUCKET_SUM_NJ(T, RM, XP, 4);          \
+    } while (0)
     if (dtype == KMX_F32) {
         if (X_rowmajor != nullptr) KMX_BUCKET_SUM(float, true, X_rowmajor);
         else KMX_BUCKET_SUM(float, false, X_t);
@@ -264,6 +274,7 @@ int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const voi
         else KMX_BUCKET_SUM(double, false, X_t);
     }
 #undef KMX_BUCKET_SUM
+#undef KMX_BUCKET_SUM_NJ
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
