@@ -724,10 +724,18 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
                                   partial, status, n, d, k, stream,
                                   reinterpret_cast<const unsigned int*>(ws + L.off_scales), ws + L.off_wscreen);
         KMX_LAUNCH_CHECK();
-        const int32_t rc = kmx_lloyd_bucket_sums(X_t, X_rowmajor, w, labels_prev, labels, partial, status,
-                                                 ws + L.off_bucket, n, d, k,
-                                                 sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
-        if (rc != KMX_OK) return rc;
+        if (sizeof(T) == 4 && L.direct_sums) {
+            gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
+            q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
+            const int32_t rc = kmx_lloyd_direct_sums(X_t, w, labels_prev, labels, q_exp, gsum, status, n, d, k,
+                                                     stream);
+            if (rc != KMX_OK) return rc;
+        } else {
+            const int32_t rc = kmx_lloyd_bucket_sums(X_t, X_rowmajor, w, labels_prev, labels, partial, status,
+                                                     ws + L.off_bucket, n, d, k,
+                                                     sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
+            if (rc != KMX_OK) return rc;
+        }
     } else if (L.acc_mode == ACC_LDS) {
         launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
                                  partial, status, n, d, k, stream);
@@ -739,6 +747,28 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[1], stream);
     const int items = (d + 1) * k;
+    if constexpr (sizeof(T) == 4) {
+        if (L.direct_sums && (size_t)items * sizeof(float) <= 48 * 1024) {
+            // fixed-point sums that fit in LDS as fp32: converted, cleared and finished by one workgroup
+            if (events) (void)hipEventRecord(events[2], stream);
+            LloydTail<float> tail;
+            tail.sums_t = (float*)new_centroids_t;
+            tail.sizes = (float*)sizes;
+            tail.empty_clusters = empty_clusters;
+            tail.old_centroids_t = (const float*)centroids_t;
+            tail.cpack = cpack;
+            tail.half_norms = half_norms;
+            tail.status = status;
+            tail.d = d;
+            tail.k = k;
+            tail.dpad = L.dpad;
+            hipLaunchKernelGGL((lloyd_small_finalize_kernel<float, true>), dim3(1), dim3(256),
+                               (size_t)items * sizeof(float), stream, gsum, q_exp, tail);
+            KMX_LAUNCH_CHECK();
+            if (events) (void)hipEventRecord(events[3], stream);
+            return KMX_OK;
+        }
+    }
     const int64_t reduce_grid = (gsum != nullptr || n_partials_used == 1)
                                     ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128)
                                     : kmx_cdiv(items, RED_ITEMS);
@@ -908,7 +938,7 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),
                            (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
     KMX_LAUNCH_CHECK();
-    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen) {
+    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen || L.direct_sums) {
         // (for the screened tiled product: max|x| per feature, from which its scale is taken)
         const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, stream);
         if (rc != KMX_OK) return rc;

@@ -220,6 +220,81 @@ __global__ __launch_bounds__(256) void bucket_sum_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------- sums without buckets
+// fp32, every cluster's sums within one workgroup's LDS as 64-bit fixed point (the scales are
+// those of the fused matrix-core steps: term = round(x * w * 2^q_f), so that the sums do not
+// depend on the order of the additions): a thread takes a sample, reads its label, and adds its
+// features with LDS atomics; the workgroup then adds its accumulators to the global ones.  One
+// pass over X_t in its own order, no sorting of the samples, one launch instead of four.
+constexpr int DS_THREADS = 1024;
+constexpr int DS_AHEAD = 8;  // features of a sample in flight together
+
+// 1.5 * 2^(52 - q): adding it to |v| < 2^(51 - q) leaves round-to-nearest(v * 2^q) in the low
+// mantissa bits (the low word of the constant is zero).
+__device__ __forceinline__ double ds_magic(int q) {
+    return __hiloint2double((int)(0x43380000u - ((unsigned int)q << 20)), 0);
+}
+__device__ __forceinline__ unsigned long long ds_fixed(double v_plus_magic, double magic) {
+    return (unsigned long long)(__double_as_longlong(v_plus_magic) - __double_as_longlong(magic));
+}
+
+__global__ __launch_bounds__(DS_THREADS) void direct_sums_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ w, const uint32_t* __restrict__ labels_prev,
+    const uint32_t* __restrict__ labels, const int* __restrict__ q_exp,
+    unsigned long long* __restrict__ gsum, kmx_lloyd_status* __restrict__ status, int n, int d, int k) {
+    if (status->state != KMX_RUNNING) return;
+    extern __shared__ unsigned long long ds_acc[];  // (d + 1, k), feature-major like gsum
+    __shared__ int q_s[65];
+    __shared__ unsigned int changed_block;
+    const int items = (d + 1) * k;
+    for (int j = threadIdx.x; j < items; j += DS_THREADS) ds_acc[j] = 0ull;
+    if (threadIdx.x <= d) q_s[threadIdx.x] = q_exp[threadIdx.x];
+    if (threadIdx.x == 0) changed_block = 0u;
+    __syncthreads();
+    unsigned int changed = 0u;
+    for (int64_t base = (int64_t)blockIdx.x * DS_THREADS; base < n; base += (int64_t)gridDim.x * DS_THREADS) {
+        const int64_t i = base + threadIdx.x;
+        const bool live = i < n;
+        const int64_t ic = live ? i : n - 1;
+        const uint32_t lab = labels[ic];
+        changed += (live && labels_prev[ic] != lab) ? 1u : 0u;
+        const double wd = live ? (double)w[ic] : 0.0;
+        unsigned long long* mine = ds_acc + lab;
+        for (int f0 = 0; f0 < d; f0 += DS_AHEAD) {
+            float xv[DS_AHEAD];
+#pragma unroll
+            for (int u = 0; u < DS_AHEAD; ++u) {
+                const int f = f0 + u < d ? f0 + u : d - 1;  // (uniform; the repeats are not added)
+                xv[u] = X_t[(size_t)f * n + ic];
+            }
+#pragma unroll
+            for (int u = 0; u < DS_AHEAD; ++u)
+                if (f0 + u < d) {
+                    const double magic = ds_magic(q_s[f0 + u]);
+                    // x * w is exact in fp64; one rounding, to a multiple of 2^-q
+                    const unsigned long long term = ds_fixed(fma((double)xv[u], wd, magic), magic);
+                    if (live) atomicAdd(mine + (size_t)(f0 + u) * k, term);
+                }
+        }
+        if (live) {
+            const double magic_w = ds_magic(q_s[d]);
+            atomicAdd(mine + (size_t)d * k, ds_fixed(wd + magic_w, magic_w));
+        }
+    }
+    if (changed) atomicAdd(&changed_block, changed);
+    __syncthreads();
+    if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+    // every workgroup starts at another word: they finish together and would otherwise queue up
+    // on the same addresses
+    const int rot = (int)(((int64_t)blockIdx.x * items) / gridDim.x);
+    for (int jy = threadIdx.x; jy < items; jy += DS_THREADS) {
+        const int jx = jy + rot < items ? jy + rot : jy + rot - items;
+        const unsigned long long v = ds_acc[jx];
+        if (v) atomicAdd(gsum + jx, v);
+    }
+}
+
 }  // namespace
 
 size_t kmx_bucket_bytes(int64_t n, int k) { return ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int); }
@@ -275,6 +350,35 @@ int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const voi
     }
 #undef KMX_BUCKET_SUM
 #undef KMX_BUCKET_SUM_NJ
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+// The sums of kmx_lloyd_direct_sums fit one workgroup's LDS (160 KB on this hardware, some of it
+// left to the kernel's own words).
+bool kmx_direct_sums_fits(int d, int k) {
+    return d <= 64 && (size_t)(d + 1) * k * sizeof(unsigned long long) <= (size_t)150 * 1024;
+}
+
+// Adds sum w x per cluster (and sum w in row d) to the fixed-point sums `gsum` ((d + 1, k), scales
+// `q_exp` as prepared for the fused matrix-core steps) and the number of changed labels to the
+// status; fp32 only.
+int32_t kmx_lloyd_direct_sums(const void* X_t, const void* w, const uint32_t* labels_prev,
+                              const uint32_t* labels, const int* q_exp, unsigned long long* gsum,
+                              kmx_lloyd_status* status, int64_t n, int d, int k, hipStream_t stream) {
+    if (!kmx_direct_sums_fits(d, k) || n > INT32_MAX || n < 1) return KMX_ERR_UNSUPPORTED;
+    const size_t lds = (size_t)(d + 1) * k * sizeof(unsigned long long);
+    if (lds > 64 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&direct_sums_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int32_t)e;
+    }
+    int64_t grid = kmx_cdiv(n, DS_THREADS);
+    const int cus = kmx_num_cus();
+    if (grid > cus) grid = cus;
+    hipLaunchKernelGGL(direct_sums_kernel, dim3((unsigned)grid), dim3(DS_THREADS), lds, stream,
+                       (const float*)X_t, (const float*)w, labels_prev, labels, q_exp, gsum, status, (int)n,
+                       d, k);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

@@ -77,6 +77,11 @@ int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const voi
                               const uint32_t* labels_prev, const uint32_t* labels, void* sums,
                               kmx_lloyd_status* status, char* bucket, int64_t n, int d, int k,
                               int32_t dtype, hipStream_t stream);
+// fp32 sums straight from the labels, accumulators of every cluster in LDS (lloyd_bucket.hip)
+bool kmx_direct_sums_fits(int d, int k);
+int32_t kmx_lloyd_direct_sums(const void* X_t, const void* w, const uint32_t* labels_prev,
+                              const uint32_t* labels, const int* q_exp, unsigned long long* gsum,
+                              kmx_lloyd_status* status, int64_t n, int d, int k, hipStream_t stream);
 // fp32 matrix-core step with fp16 screening of the labels (lloyd_mfma_screen.hip): whether the
 // shape fits the kernel at all, and whether the flags (or, left to the library, the measured
 // break-even) select it
@@ -102,6 +107,7 @@ struct LloydLayout {
     bool screen;         // KMX_VARIANT_MFMA with fp16-screened labels (variant code 61)
     bool gemm_screen;    // KMX_VARIANT_GEMM (fp32) with fp16-screened labels
     bool screen_labels;  // KMX_VARIANT_GEMM (fp32, d <= 64): labels by the screened kernel of variant 61 without its sums
+    bool direct_sums;    // with screen_labels: sums straight from the labels (fixed point in LDS) instead of per bucket
     uint32_t flags;      // the caller's KMX_FLAG_* selection
     int wgs_per_cu;      // workgroups per compute unit asked for (0: the kernel's default)
     int cols;            // sample columns per lane asked for (0: the kernel's default)
@@ -206,6 +212,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
     L.gemm_screen = L.variant == KMX_VARIANT_GEMM && dtype == KMX_F32 && kmx_gemm_screen_enabled(n, d, k, flags);
     L.screen_labels = L.variant == KMX_VARIANT_GEMM && screen_labels_ok && !L.gemm_screen && forced != KMX_VARIANT_GEMM;
+    L.direct_sums = L.screen_labels && kmx_direct_sums_fits(d, k);
     L.off_status = 0;
     // fixed-point scales of the matrix-core path: LloydScales, then (d + 1) * k int64 sums
     L.off_scales = kmx_align256(sizeof(kmx_lloyd_status));

@@ -377,6 +377,69 @@ def test_iterations_stay_in_lockstep_with_the_oracle(cuda, shape, iterations):
         assert status.n_iter == it + 1
 
 
+@pytest.mark.parametrize("shape,direct", [((30_000, 14, 700), True),     # sums finished by one workgroup
+                                          ((9_001, 8, 1_024), True),
+                                          ((20_000, 64, 256), True),     # sums beyond what one workgroup finishes
+                                          ((12_345, 48, 300), True),
+                                          ((40_000, 16, 1_140), False)])  # accumulators beyond the LDS: sums per bucket
+def test_screened_labels_with_separate_sums_run_to_convergence(cuda, shape, direct):
+    """Shapes whose operands fit the screened kernel but whose accumulators do not fit beside them:
+    labels by the screened kernel, sums by a kernel of their own (every cluster's fixed-point
+    accumulators in LDS where they fit, else per bucket of samples).  Uneven weights with zeros
+    among them; every iteration is compared with the oracle from the centroids it started with,
+    and the run must stop exactly when an iteration changes no label (60 iterations at most)."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+
+    n, d, k = shape
+    rng = np.random.default_rng(n + d + k)
+    # (wide samples: blobs that overlap, or the second iteration already changes nothing)
+    noise = 0.3 if d <= 16 else 1.0
+    X = (rng.uniform(-2, 2, (k, d))[rng.integers(0, k, n)] + noise * rng.standard_normal((n, d))).astype(np.float32)
+    w = rng.uniform(0.5, 2.0, n).astype(np.float32)
+    w[rng.integers(0, n, n // 50)] = 0.0
+    chosen = rng.choice(n, k, replace=False)
+    w[chosen] = 1.0  # (a cluster of one sample of weight zero would be empty at once)
+    init = X[chosen].copy()
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a), device=cuda)
+    X_t, w_d = dev(X.T), dev(w)
+    cent = [dev(init.T), torch.empty(d, k, dtype=torch.float32, device=cuda)]
+    labels = [torch.full((n,), k, dtype=torch.int32, device=cuda) for _ in range(2)]
+    sizes = torch.empty(k, dtype=torch.float32, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    plan = _capi.lloyd_plan(n, d, k, 0, 0)
+    assert plan.variant == 63
+    ws_bytes = plan.workspace_bytes
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 200, 0.0, stream), "init")
+    status = _capi.LloydStatus()
+    previous = None
+    for it in range(60):
+        a, b = it % 2, (it + 1) % 2
+        c_in = cent[a].cpu().numpy().T.copy()
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
+        _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+        got = labels[b].cpu().numpy().astype(np.int64)
+        assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
+        sums, ref_sizes = ok.weighted_sums(X, w, got, k)
+        np.testing.assert_allclose(sizes.cpu().numpy(), ref_sizes, rtol=1e-5)
+        if status.n_empty:
+            assert status.state == _capi.KMX_NEED_RELOCATION
+            break
+        assert_centers_close(cent[b].cpu().numpy().T, sums / ref_sizes[:, None], np.float32)
+        assert status.n_iter == it + 1
+        if previous is not None and np.array_equal(got, previous):
+            assert status.state == _capi.KMX_CONVERGED_STRICT
+            break
+        assert status.state == _capi.KMX_RUNNING, (it, status.state)
+        previous = got
+    assert it >= 1, (it, status.state, status.n_empty)
+
+
 def _screen_scores(X, C, cuda):
     import torch
 
