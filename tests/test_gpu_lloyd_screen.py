@@ -377,9 +377,10 @@ def test_iterations_stay_in_lockstep_with_the_oracle(cuda, shape, iterations):
         assert status.n_iter == it + 1
 
 
-@pytest.mark.parametrize("shape,direct", [((30_000, 14, 700), True),     # sums finished by one workgroup
+@pytest.mark.parametrize("shape,direct", [((20_000, 4, 1_100), True),     # few sums: finished by one workgroup
+                                          ((30_000, 14, 700), True),
                                           ((9_001, 8, 1_024), True),
-                                          ((20_000, 64, 256), True),     # sums beyond what one workgroup finishes
+                                          ((20_000, 64, 256), True),
                                           ((12_345, 48, 300), True),
                                           ((40_000, 16, 1_140), False)])  # accumulators beyond the LDS: sums per bucket
 def test_screened_labels_with_separate_sums_run_to_convergence(cuda, shape, direct):
