@@ -775,7 +775,7 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
                                     ? (kmx_cdiv(items, 256) < 128 ? kmx_cdiv(items, 256) : 128)
                                     : kmx_cdiv(items, RED_ITEMS);
     // sums that fit in LDS are finished by one workgroup (no device-wide fences or tickets)
-    const bool small_tail = gsum == nullptr && (size_t)items * sizeof(T) <= 48 * 1024;
+    const bool small_tail = gsum == nullptr && items <= 6 * 1024;
     hipLaunchKernelGGL((lloyd_reduce_kernel<T>), dim3((unsigned)reduce_grid), dim3(256), 0,
                        stream, partial, n_partials_used,
                        ((L.acc_mode == ACC_GLOBAL || L.acc_mode == KMX_ACC_BUCKET) && gsum == nullptr) ? 1 : 0,
