@@ -269,7 +269,7 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False, flags=0):
     variant = plan.variant
     X_rm = torch.as_tensor(X, device=dev)
     X_t = X_rm.T.contiguous()
-    if variant not in (42, 3, 13, 53, 63):  # the variants that sum rows of a row-major copy
+    if lib.kmx_lloyd_plan_reads_rowmajor(plan) != 1:  # (only some kernels sum rows of a row-major copy)
         X_rm = None
     w_d = torch.as_tensor(w, device=dev)
     cent = [torch.as_tensor(np.ascontiguousarray(init.T), device=dev), None]

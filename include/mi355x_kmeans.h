@@ -219,6 +219,13 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
  * labels screened on the fp16 matrix cores. */
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
+/* 1 when the plan's kernels read the row-major copy of X that kmx_lloyd_iter takes as
+ * `X_rowmajor` (the wide fp32 step always; the sums per bucket of samples optionally, NULL makes
+ * them gather the feature-major array), 0 when they ignore it, negative: error.  Host only.
+ * Has no counterpart in the reference, whose kernels read one layout (the transposed copy made
+ * in sklearn_numba_dpex/kmeans/engine.py:88-98): it lets a caller skip the second copy of X. */
+int32_t kmx_lloyd_plan_reads_rowmajor(const kmx_lloyd_plan* plan);
+
 /* ------------------------------------------------------------------------------------ *
  * Labels, inertia, distances                                                            *
  * ------------------------------------------------------------------------------------ */

@@ -113,6 +113,7 @@ SIGNATURES = {
     "kmx_lloyd_recheck_count": (_I32, [_PLAN, _P, POINTER(ctypes.c_uint32), _P]),
     "kmx_screen_scores": (_I32, [_P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _P]),
     "kmx_lloyd_kernel_variant": (_I32, [_I64, _I32, _I32, _I32, _U32]),
+    "kmx_lloyd_plan_reads_rowmajor": (_I32, [_PLAN]),
     "kmx_assign_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "kmx_assign_workspace_bytes_for": (_SZ, [_I64, _I32, _I32, _I32, _U32]),
     "kmx_assign_labels": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _U32, _P]),

@@ -913,6 +913,13 @@ int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype,
     return rc == KMX_OK ? plan.variant : rc;
 }
 
+int32_t kmx_lloyd_plan_reads_rowmajor(const kmx_lloyd_plan* plan) {
+    KMX_REQUIRE_PLAN(plan);
+    const LloydLayout L = lloyd_layout(plan->n, plan->d, plan->k, plan->dtype, plan->flags);
+    if (L.variant == KMX_VARIANT_MFMA_WIDE) return 1;
+    return (L.acc_mode == KMX_ACC_BUCKET && !L.direct_sums) ? 1 : 0;
+}
+
 int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t workspace_bytes,
                        const void* X_t, const void* sample_weight, const void* centroids_t,
                        int32_t max_iter, double tol, void* stream_) {

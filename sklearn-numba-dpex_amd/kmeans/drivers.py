@@ -21,8 +21,6 @@ from ..common.topk import topk_idx
 # How many Lloyd iterations may be enqueued before the host next reads the status.
 _MAX_LOOKAHEAD = 16
 
-# Kernel variants (codes of the plan) that read a row-major copy of X besides the feature-major one.
-_ROW_MAJOR_VARIANTS = (42, 3, 13, 53, 63)
 
 
 def lloyd(
@@ -72,7 +70,10 @@ def lloyd(
     # the wide fp32 path and the bucketed sums add up each cluster's rows from a row-major copy
     # of X (one transpose per run, n * d extra elements of HBM): whole cache lines per sample
     X_rm = None
-    if plan.variant in _ROW_MAJOR_VARIANTS:
+    reads_rowmajor = lib.kmx_lloyd_plan_reads_rowmajor(plan)
+    if reads_rowmajor < 0:
+        check(reads_rowmajor, "kmx_lloyd_plan_reads_rowmajor")
+    if reads_rowmajor == 1:
         try:
             X_rm = transposed_copy(X_t)
         except torch.cuda.OutOfMemoryError:

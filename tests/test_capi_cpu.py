@@ -54,6 +54,7 @@ def test_error_strings_and_codes():
 
 
 def test_workspace_queries():
+    from sklearn_numba_dpex_amd import _capi
     from sklearn_numba_dpex_amd._capi import lib
 
     small = lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 0, 0)
@@ -67,6 +68,12 @@ def test_workspace_queries():
     assert (lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0x20)
             >= lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) + 4_000_000)
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 63
+    # the second (row-major) copy of X: read by the wide step and by the sums per bucket, not by the
+    # fused steps nor by the sums taken straight from the labels
+    for (n_, d_, k_, dt_), reads in {(1_000_000, 256, 1024, 0): 1, (1_000_000, 300, 1024, 0): 1,
+                                     (1_000_000, 100, 100, 1): 1, (5_000_000, 14, 127, 0): 0,
+                                     (1_000_000, 14, 700, 0): 0, (2_000_000, 32, 64, 1): 0}.items():
+        assert lib.kmx_lloyd_plan_reads_rowmajor(_capi.lloyd_plan(n_, d_, k_, dt_, 0)) == reads, (n_, d_, k_, dt_)
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0) == 51
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 32, 500, 1, 0) == 53
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0, 0) == 0
