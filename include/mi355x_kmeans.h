@@ -215,8 +215,9 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
  * with samples in registers and centroids streamed (more than 256 clusters), 5 = MFMA (fp64)
  * with the centroids resident in LDS, 6 = labels by a tiled matrix-core product (any shape,
  * fp32 and fp64); accumulation 1 = workgroup-private LDS accumulators, 2 = global sums,
- * 3 = labels only, then sums per bucket of samples sorted by label.  61 is path 3 with the
- * labels screened on the fp16 matrix cores. */
+ * 3 = labels only, then sums by a kernel of their own (per bucket of samples sorted by label,
+ * or, fp32, straight from the labels into fixed-point accumulators in LDS where those of every
+ * cluster fit).  61 is path 3 with the labels screened on the fp16 matrix cores. */
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* 1 when the plan's kernels read the row-major copy of X that kmx_lloyd_iter takes as
