@@ -1,5 +1,7 @@
 """Device-buffer helpers: torch tensors serve only as HIP allocations."""
 
+import threading
+
 import numpy as np
 import torch
 
@@ -18,23 +20,38 @@ def torch_dtype(dtype):
 
 
 _workspaces = {}
+_workspaces_lock = threading.Lock()
+# a kept buffer larger than this is not kept (the list of uncertified samples of a wide label
+# call is 4 bytes per sample)
+_WORKSPACE_KEEP_BYTES = 64 << 20
 
 
 def workspace(n_bytes, device, tag=None):
     """Scratch bytes for one library call.  With a `tag` the buffer is kept and handed out again
-    to the next call with the same tag on the same device and stream (work on one stream is
-    ordered, so the calls cannot overlap); it only ever grows."""
+    to the next call with the same tag by the same host thread on the same device and stream
+    (one thread's work on one stream is ordered, so those calls cannot overlap; two threads
+    that share a stream each get a buffer of their own).  A kept buffer only grows, up to
+    64 MiB: a larger one is made for the call and released with it.  `release_workspaces()`
+    drops them all."""
     n_bytes = max(int(n_bytes), 1)
-    if tag is None:
+    if tag is None or n_bytes > _WORKSPACE_KEEP_BYTES:
         return torch.empty(n_bytes, dtype=torch.uint8, device=device)
     device = torch.device(device)
     key = (tag, device.index if device.index is not None else torch.cuda.current_device(),
-           _capi.current_stream())
-    buf = _workspaces.get(key)
-    if buf is None or buf.numel() < n_bytes:
-        buf = torch.empty(max(n_bytes, 4096), dtype=torch.uint8, device=device)
-        _workspaces[key] = buf
+           _capi.current_stream(), threading.get_ident())
+    with _workspaces_lock:
+        buf = _workspaces.get(key)
+        if buf is None or buf.numel() < n_bytes:
+            buf = torch.empty(max(n_bytes, 4096), dtype=torch.uint8, device=device)
+            _workspaces[key] = buf
     return buf
+
+
+def release_workspaces():
+    """Forgets every kept scratch buffer (their memory goes back to the allocator once the
+    calls that use them have run)."""
+    with _workspaces_lock:
+        _workspaces.clear()
 
 
 def dcode(t):
@@ -55,6 +72,7 @@ def contiguous(t):
 _STAGE_BYTES = 32 << 20
 _STAGE_MIN_BYTES = 4 << 20   # below this a plain copy is as fast
 _stage = None
+_stage_lock = threading.Lock()   # one upload at a time: the two buffers and their events are shared
 
 
 def _staging():
@@ -74,8 +92,8 @@ def upload(array, device):
     out = torch.empty(array.shape, dtype=torch.from_numpy(array[:0].reshape(-1)).dtype, device=dev)
     src = torch.from_numpy(array.reshape(-1).view(np.uint8))
     dst = out.view(-1).view(torch.uint8)
-    stage = _staging()
-    with torch.cuda.device(dev):
+    with _stage_lock, torch.cuda.device(dev):
+        stage = _staging()
         for turn, lo in enumerate(range(0, src.numel(), _STAGE_BYTES)):
             hi = min(lo + _STAGE_BYTES, src.numel())
             buf, busy = stage[turn % 2]

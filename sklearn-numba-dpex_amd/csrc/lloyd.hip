@@ -635,25 +635,27 @@ void launch_reg(const LloydLayout& L, const void* X_t, const void* w, const T* c
                        status, n, d, k, L.dpad, L.n_partials, vec_ok, copies);
 }
 
+// Returns the status of the entry point it hands over to (a refusal there would leave `labels`
+// unwritten, and the sums kernels that follow index LDS and memory with them).
 template <typename T, int ACC>
-void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
+int32_t launch_fused(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
                   const T* cpack, const T* half_norms, const uint32_t* labels_prev,
                   uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
                   hipStream_t stream, const unsigned int* screen_absmax = nullptr, char* screen_area = nullptr) {
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_GEMM) {
         if (sizeof(T) == 4 && L.screen_labels)
-            (void)kmx_lloyd_labels_mfma_screen(X_t, centroids_t, labels, status, n, d, k, L.wgs_per_cu, stream);
+            return kmx_lloyd_labels_mfma_screen(X_t, centroids_t, labels, status, n, d, k, L.wgs_per_cu, stream);
         else if (sizeof(T) == 4 && L.gemm_screen && screen_area != nullptr)
-            (void)kmx_lloyd_gemm_screen_labels(X_t, centroids_t, half_norms, screen_absmax, screen_area, labels,
-                                               status, n, d, k, stream);
+            return kmx_lloyd_gemm_screen_labels(X_t, centroids_t, half_norms, screen_absmax, screen_area, labels,
+                                                status, n, d, k, stream);
         else
-            (void)kmx_lloyd_gemm_labels(X_t, centroids_t, half_norms, labels, status, n, d, k,
-                                        sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
+            return kmx_lloyd_gemm_labels(X_t, centroids_t, half_norms, labels, status, n, d, k,
+                                         sizeof(T) == 8 ? KMX_F64 : KMX_F32, stream);
     } else if (L.variant == KMX_VARIANT_MFMA_F64) {
-        (void)kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
-                                      status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, L.partial_slots(),
-                                      stream);
+        return kmx_lloyd_step_mfma_f64(X_t, w, centroids_t, half_norms, labels_prev, labels, partial,
+                                       status, n, d, k, ACC != ACC_NONE, L.wgs_per_cu, L.cols, L.partial_slots(),
+                                       stream);
     } else if (L.variant == KMX_VARIANT_REGISTER) {
 #define KMX_REG_CASE(DR, RR)                                                                    \
     launch_reg<T, DR, RR, ACC>(L, X_t, w, cpack, half_norms, labels_prev, labels, partial, status, \
@@ -693,6 +695,8 @@ void launch_fused(const LloydLayout& L, const void* X_t, const void* w, const vo
                                labels_prev, labels, partial, status, n, d, k, L.n_partials, vec_ok, copies);
         }
     }
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
 }
 
 template <typename T>
@@ -720,10 +724,11 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
         gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
         q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
     } else if (L.acc_mode == KMX_ACC_BUCKET) {
-        launch_fused<T, ACC_NONE>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
-                                  partial, status, n, d, k, stream,
-                                  reinterpret_cast<const unsigned int*>(ws + L.off_scales), ws + L.off_wscreen);
-        KMX_LAUNCH_CHECK();
+        const int32_t rc_labels =
+            launch_fused<T, ACC_NONE>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
+                                      partial, status, n, d, k, stream,
+                                      reinterpret_cast<const unsigned int*>(ws + L.off_scales), ws + L.off_wscreen);
+        if (rc_labels != KMX_OK) return rc_labels;
         if (sizeof(T) == 4 && L.direct_sums) {
             gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
             q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
@@ -737,12 +742,16 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
             if (rc != KMX_OK) return rc;
         }
     } else if (L.acc_mode == ACC_LDS) {
-        launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
-                                 partial, status, n, d, k, stream);
+        const int32_t rc_step =
+            launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
+                                     partial, status, n, d, k, stream);
+        if (rc_step != KMX_OK) return rc_step;
         n_partials_used = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     } else {
-        launch_fused<T, ACC_GLOBAL>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
-                                    partial, status, n, d, k, stream);
+        const int32_t rc_step =
+            launch_fused<T, ACC_GLOBAL>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
+                                        partial, status, n, d, k, stream);
+        if (rc_step != KMX_OK) return rc_step;
     }
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[1], stream);
@@ -1202,19 +1211,22 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
             const int32_t rc = kmx_wide_screen_scale_from_centroids(centroids_t, absmax, d, k, stream);
             if (rc != KMX_OK) return rc;
         }
-        launch_fused<float, ACC_NONE>(L, X_t, nullptr, centroids_t, (const float*)(ws + L.off_cpack),
-                                      (const float*)(ws + L.off_half), nullptr, labels, nullptr,
-                                      nullptr, n, d, k, stream, absmax, area);
+        const int32_t rc = launch_fused<float, ACC_NONE>(L, X_t, nullptr, centroids_t,
+                                                         (const float*)(ws + L.off_cpack),
+                                                         (const float*)(ws + L.off_half), nullptr, labels, nullptr,
+                                                         nullptr, n, d, k, stream, absmax, area);
+        if (rc != KMX_OK) return rc;
     } else {
         hipLaunchKernelGGL((lloyd_pack_kernel<double>), dim3(grid), dim3(256), 0, stream,
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),
                            (double*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
                            0.0);
         KMX_LAUNCH_CHECK();
-        launch_fused<double, ACC_NONE>(L, X_t, nullptr, centroids_t,
-                                       (const double*)(ws + L.off_cpack),
-                                       (const double*)(ws + L.off_half), nullptr, labels, nullptr,
-                                       nullptr, n, d, k, stream);
+        const int32_t rc = launch_fused<double, ACC_NONE>(L, X_t, nullptr, centroids_t,
+                                                          (const double*)(ws + L.off_cpack),
+                                                          (const double*)(ws + L.off_half), nullptr, labels, nullptr,
+                                                          nullptr, n, d, k, stream);
+        if (rc != KMX_OK) return rc;
     }
     KMX_LAUNCH_CHECK();
     return KMX_OK;

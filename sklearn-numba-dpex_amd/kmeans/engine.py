@@ -387,7 +387,9 @@ class KMeansEngine(_EngineBase):
                 estimator=self.estimator,
                 input_name="init",
             )
-            init_dev = torch.as_tensor(init_np, device=X.device)
+            # check_array hands back the caller's own array when nothing had to change, and that
+            # one may be read-only: wrap a private copy
+            init_dev = torch.as_tensor(np.array(init_np, copy=True), device=X.device)
         self._validate_center_shape(X, init_dev)
         init_t = init_dev.T.contiguous()
         if init_t.data_ptr() == getattr(init, "data_ptr", lambda: None)():

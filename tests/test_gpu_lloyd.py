@@ -305,6 +305,142 @@ def test_full_lloyd_run_matches_oracle(cuda, name):
         assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-4)
 
 
+def _converging_configs():
+    """Cases whose Lloyd run at tol = 0 reaches strict convergence (an iteration that changes no
+    label) well below max_iter = 100.  Per case: the data, the kernel variant the plan must
+    choose, and the iteration count of the oracle (found on the CPU; scikit-learn's Cython loop
+    takes the same number when run on 8 threads, but its own count moves with its thread count
+    - 43 instead of 39 on C1 with 4 threads - because its per-thread partial sums round
+    differently and a Lloyd trajectory at tol = 0 amplifies every flipped near-tie)."""
+    return {
+        # BASELINE configs[0] at full size (fused screened step, sums corrected per moved sample)
+        "C1": (lambda: datasets.config1(), 61, 39),
+        # configs[1] (weighted, unequal blobs, one cluster empties and is relocated) and
+        # configs[4] (fp64, sixteen clusters that empty on the first iteration) on fewer samples
+        "C2_30k": (lambda: datasets.config2(n=30_000), 61, 38),
+        "C5_100k": (lambda: datasets.config5(n=100_000), 51, 67),
+        # screened labels with the sums taken straight from the labels, and with sums per bucket
+        "direct": (lambda: _blob_config(20_000, 14, 700, np.float32, 20), 63, 8),
+        "bucket": (lambda: _blob_config(20_000, 32, 500, np.float64, 19), 53, 8),
+    }
+
+
+@pytest.mark.parametrize("name", ["C1", "C2_30k", "C5_100k", "direct", "bucket"])
+def test_n_iter_at_real_strict_convergence(cuda, name):
+    """n_iter must be identical at tol = 0: whole runs with max_iter = 100 that stop because an
+    iteration changed no label, not because of the cap, against the oracle, and against
+    scikit-learn's own Lloyd loop wherever that one stayed on the oracle's trajectory."""
+    from sklearn.cluster._kmeans import _kmeans_single_lloyd
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    make, variant, expected_n_iter = _converging_configs()[name]
+    cfg = make()
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    assert _capi.lloyd_plan(n, d, k, _capi.dtype_code(X.dtype), 0).variant == variant
+    mean = X.mean(axis=0).astype(X.dtype)
+    Xc, initc = X - mean, init - mean
+    max_iter = 100
+    labels, inertia, centers_t, n_iter = drivers.lloyd(
+        _dev(Xc.T, cuda), _dev(w, cuda), _dev(initc.T, cuda), False, max_iter=max_iter, tol=0.0
+    )
+    ref_labels, ref_inertia, ref_centers, ref_n_iter = ok.lloyd(Xc, w, initc, max_iter=max_iter, tol=0.0)
+    # the case is not decided by the cap
+    assert ref_n_iter == expected_n_iter < max_iter
+    assert n_iter == ref_n_iter
+    centers = centers_t.cpu().numpy().T
+    got = labels.cpu().numpy().astype(np.int64)
+    # strict convergence: the returned labels are those of the last iteration and the argmin for
+    # the returned centroids
+    assert_labels_match(got, ok.assign_labels(Xc, centers), Xc, centers)
+    assert float(inertia) == pytest.approx(float(ok.inertia(Xc, w, centers, got)), rel=RTOL[X.dtype] * 10)
+    n_diff = np.count_nonzero(got != ref_labels.astype(np.int64))
+    if n_diff == 0:
+        # same final partition: the centroids are the same weighted means, 1e-5 / 1e-12
+        assert_centers_close(centers, ref_centers, X.dtype)
+        assert float(inertia) == pytest.approx(float(ref_inertia), rel=RTOL[X.dtype] * 10)
+    else:
+        # a near-tie went the other way in some iteration and the run ended in a neighbouring
+        # fixed point after the same number of iterations: a few boundary samples (iteration by
+        # iteration parity from identical inputs is what the lockstep tests assert)
+        assert n_diff <= n_samples_differ_cap(X)
+        assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-4)
+    sk_labels, sk_inertia, sk_centers, sk_n_iter = _kmeans_single_lloyd(
+        Xc, w, initc.copy(), max_iter=max_iter, tol=0.0, n_threads=8
+    )
+    if np.array_equal(sk_labels, ref_labels):
+        # scikit-learn ended in the oracle's partition: it took the oracle's path
+        assert n_iter == sk_n_iter
+    assert float(inertia) == pytest.approx(float(sk_inertia), rel=1e-3)
+
+
+def test_lockstep_to_strict_convergence_where_free_runs_part_ways(cuda):
+    """configs[1] on 100 000 samples: at iteration 3 one sample lies within 4e-9 (relative) of a
+    bisector, the kernel and the oracle label it differently, and from there the two free runs
+    (and scikit-learn's) follow different trajectories: 69, 84 and 84 iterations.  What can be
+    pinned there is every single iteration up to the end: the oracle repeats each iteration from
+    the centroids the GPU started it with, through the relocation of the cluster that empties, and
+    the run must stop at the first iteration whose labels equal the previous ones."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    cfg = datasets.config2(n=100_000)
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    mean = X.mean(axis=0).astype(X.dtype)
+    X, init = X - mean, init - mean
+    n, d = X.shape
+    dc = _capi.dtype_code(X.dtype)
+    X_t, w_d = _dev(X.T, cuda), _dev(w, cuda)
+    cent = [_dev(init.T, cuda), None]
+    cent[1] = torch.empty_like(cent[0])
+    labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
+    sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    plan = _capi.lloyd_plan(n, d, k, dc, 0)
+    assert plan.variant == 61
+    ws_bytes = plan.workspace_bytes
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
+    stream = _capi.current_stream()
+    status = _capi.LloydStatus()
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), ws_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 100, 0.0, stream), "init")
+    prev = None
+    n_relocations = 0
+    for it in range(100):
+        a, b = it % 2, (it + 1) % 2
+        c_in = cent[a].cpu().numpy().T.copy()
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), ws_bytes, stream), "iter")
+        _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+        got = labels[b].cpu().numpy().astype(np.int64)
+        assert_labels_match(got, ok.assign_labels(X, c_in), X, c_in)
+        sums, ref_sizes = ok.weighted_sums(X, w, got, k)
+        if status.state == _capi.KMX_NEED_RELOCATION:
+            n_relocations += 1
+            assert status.n_empty == int(np.count_nonzero(ref_sizes == 0)) and status.n_iter == it
+            drivers._relocate_empty_clusters(status.n_empty, X_t, w_d, cent[b], sizes, labels[b], empty, cent[a])
+            _capi.check(lib.kmx_lloyd_finalize(plan, ptr(cent[a]), ptr(cent[b]), ptr(sizes), ptr(ws), ws_bytes, stream),
+                        "finalize")
+            _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+            ok.relocate_empty_clusters(X, w, sums, ref_sizes, got, ok.sq_dist_to_assigned(X, c_in, got))
+        assert status.n_iter == it + 1
+        assert_centers_close(cent[b].cpu().numpy().T, sums / ref_sizes[:, None], X.dtype)
+        strict = prev is not None and np.array_equal(got, prev)
+        assert (status.state == _capi.KMX_CONVERGED_STRICT) == strict
+        if strict:
+            break
+        assert status.state == _capi.KMX_RUNNING
+        prev = got
+    assert status.state == _capi.KMX_CONVERGED_STRICT and n_relocations >= 1
+    # the driver's own loop (iterations enqueued ahead) stops at the same iteration
+    n_iter = drivers.lloyd(X_t, w_d, _dev(init.T, cuda), False, max_iter=100, tol=0.0)[3]
+    assert n_iter == status.n_iter
+
+
 def n_samples_differ_cap(X):
     return X.shape[0] // 1000
 
