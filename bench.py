@@ -11,9 +11,12 @@ Prints ONE JSON line: iterations/s, plus
                 recorded around that kernel on its stream (kmx_lloyd_iter_timed): HBM for the
                 kernel that screens the labels on the fp16 matrix cores (variant 61), the fp32
                 MFMA peak for the all-fp32 kernel (variant 31, KMX_FLAG_LABELS_F32);
-  roofline_other_bound  the same kernel against the other of the two;
-  cpu_baseline  scikit-learn's OpenMP/Cython Lloyd on the same data on this host's cores;
-  kmeanspp_ms   kmeans++ seeding time on configs[3] (1,000,000 x 64, k = 256).
+  roofline_other_bound  the same kernel's fp32-equivalent rate (variant 61) or HBM fraction (31);
+  cpu_baseline  scikit-learn's OpenMP/Cython Lloyd on the same data on this host's cores (the
+                inner routine, and the estimator-level fit of the reference's benchmark protocol);
+  kmeanspp_ms   kmeans++ seeding time on configs[3] (1,000,000 x 64, k = 256), with
+                cpu_baseline_kmeanspp (scikit-learn's seeding on the same data) and the default
+                sampler's picks against the reference's own sampler beside it.
 """
 
 import argparse
@@ -32,6 +35,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3    # MI355X fp32, vector and matrix
 RAMP_MS = 60.0              # untimed iterations before every timed region, for the GPU clocks
 FLAG_LABELS_F32 = 0x10      # KMX_FLAG_LABELS_F32: every product of the fp32 paths in fp32
+REGIONS = 3                 # timed regions of --steps iterations; the median one is reported
 
 
 def log(*a):
@@ -142,12 +146,17 @@ def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
     restart()
     for _ in range(warmup):
         enqueue()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        enqueue()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    # REGIONS timed regions of `steps` iterations each, one after the other in the same fit; the
+    # median region is the one reported
+    regions = []
+    for _ in range(REGIONS):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            enqueue()
+        torch.cuda.synchronize()
+        regions.append(time.perf_counter() - t0)
+    elapsed = float(np.median(regions))
 
     # per-kernel durations from HIP events on the launch stream; three untimed iterations are
     # enqueued before every timed one, so that the clocks do not sag in the gaps the
@@ -169,7 +178,7 @@ def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
     rechecked = ctypes.c_uint32(0)
     _capi.check(lib.kmx_lloyd_recheck_count(plan, ptr(ws), ctypes.byref(rechecked), stream), "recheck_count")
     if not gates:
-        return elapsed, kernel_ms, 0, plan.variant, int(rechecked.value), ramp_iters
+        return elapsed, kernel_ms, 0, plan.variant, int(rechecked.value), ramp_iters, regions
 
     # parity gate 1: the labels the last Lloyd iteration wrote, against exact fp64 distances to
     # the centroids it started from, on a slice
@@ -184,7 +193,7 @@ def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
     _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(X_t.new_tensor(cur.T.copy())), ptr(lab), ptr(aws_t), aws,
                                       n, d, k, dc, flags, stream), "assign")
     ties = ties_iter + check_labels(lab[:m].cpu().numpy(), X[:m], cur)
-    return elapsed, kernel_ms, ties, plan.variant, int(rechecked.value), ramp_iters
+    return elapsed, kernel_ms, ties, plan.variant, int(rechecked.value), ramp_iters, regions
 
 
 def gpu_measured_peaks():
@@ -486,6 +495,89 @@ def gpu_kmeanspp(cfg):
     return float(np.median(times)), idx.cpu().numpy()
 
 
+def kpp_sampler_report(cfg):
+    """The default sampler (search of the fp64 inclusive scan) against the reference's own
+    (running sum in the compute dtype, KMX_KPP_SAMPLER_LITERAL) on the same seeding: for every
+    centre both samplers draw their candidates from the same closest-distance array with the
+    same uniforms, then the seeding goes on with the default sampler's.  Reports how many draws
+    pick another sample and how far apart the picks are in cumulative probability."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    dev = torch.device("cuda:0")
+    X_t = torch.as_tensor(cfg["X"], device=dev).T.contiguous()
+    w = torch.as_tensor(cfg["sample_weight"], device=dev)
+    d, n = X_t.shape
+    k, tn = cfg["k"], cfg["n_local_trials"]
+    dc = _capi.dtype_code(X_t.dtype)
+    start_raw, table = drivers.kpp_uniforms(k, tn, np.random.RandomState(cfg["seed"]), np.float32)
+    uniforms = torch.from_numpy(table).to(dev)
+    centers_t = torch.empty((d, k), dtype=X_t.dtype, device=dev)
+    indices = torch.full((k,), -1, dtype=torch.int32, device=dev)
+    ws_bytes = lib.kmx_kpp_workspace_bytes(n, d, k, tn, dc)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    st = _capi.current_stream()
+    _capi.check(lib.kmx_kpp_init(ptr(X_t), ptr(w), int(start_raw % n), ptr(centers_t), ptr(indices), ptr(ws), ws_bytes,
+                                 n, d, k, tn, dc, 0, st), "kpp_init")
+    rows_off = lib.kmx_kpp_closest_ptr(ptr(ws), n, d, k, tn, dc) - ws.data_ptr()
+    cand_lit = torch.empty(tn, dtype=torch.int32, device=dev)
+    cand_scan = torch.empty(tn, dtype=torch.int32, device=dev)
+    draws = differ = 0
+    shift_samples = []
+    gap_prob = []
+    lit_ms = 0.0
+    for c in range(1, k):
+        u = uniforms[c - 1]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _capi.check(lib.kmx_kpp_sample_candidates(ptr(X_t), ptr(u), ptr(cand_lit), ptr(ws), ws_bytes, n, d, k, tn, dc,
+                                                  _capi.KMX_KPP_SAMPLER_LITERAL, st), "kpp_sample literal")
+        torch.cuda.synchronize()
+        lit_ms += (time.perf_counter() - t0) * 1e3
+        _capi.check(lib.kmx_kpp_sample_candidates(ptr(X_t), ptr(u), ptr(cand_scan), ptr(ws), ws_bytes, n, d, k, tn, dc,
+                                                  _capi.KMX_KPP_SAMPLER_SCAN, st), "kpp_sample")
+        a, b = cand_lit.cpu().numpy().astype(np.int64), cand_scan.cpu().numpy().astype(np.int64)
+        draws += tn
+        if np.any(a != b):
+            best_row = int(ws[:4].view(torch.int32).item())
+            lo = rows_off + best_row * n * 4
+            closest = ws[lo:lo + n * 4].view(torch.float32).cpu().numpy()
+            cum = np.cumsum(closest.astype(np.float64))
+            rv = table[c - 1] * cum[-1]
+            for t in np.flatnonzero(a != b):
+                differ += 1
+                shift_samples.append(abs(int(a[t]) - int(b[t])))
+                gap_prob.append(abs(rv[t] - cum[a[t]]) / cum[-1])
+        _capi.check(lib.kmx_kpp_step(ptr(X_t), ptr(w), c, ptr(centers_t), ptr(indices), ptr(ws), ws_bytes, n, d, k, tn,
+                                     dc, 0, st), "kpp_step")
+    return {
+        "what": "default sampler (fp64 inclusive scan) against the reference's running sum in fp32 "
+                "(KMX_KPP_SAMPLER_LITERAL), same closest-distance array and uniforms for every draw of one seeding",
+        "draws": draws, "draws_with_another_pick": differ,
+        "index_shift_samples_median": float(np.median(shift_samples)) if shift_samples else 0.0,
+        "index_shift_samples_max": int(max(shift_samples)) if shift_samples else 0,
+        "max_gap_rv_minus_cum_at_literal_pick_over_total": float(max(gap_prob)) if gap_prob else 0.0,
+        "literal_sampler_ms_per_centre": lit_ms / (k - 1),
+    }
+
+
+def cpu_kmeanspp_baseline(cfg):
+    """scikit-learn's own seeding on the same data: wall clock of
+    sklearn.cluster.kmeans_plusplus(X, k, random_state=seed), after a small warm-up call."""
+    from sklearn.cluster import kmeans_plusplus
+    from sklearn.utils._openmp_helpers import _openmp_effective_n_threads
+
+    X = cfg["X"]
+    kmeans_plusplus(X[:10_000], 8, random_state=0)
+    t0 = time.perf_counter()
+    kmeans_plusplus(X, cfg["k"], random_state=cfg["seed"])
+    elapsed = time.perf_counter() - t0
+    return elapsed * 1e3, _openmp_effective_n_threads()
+
+
 def cpu_lloyd_baseline(cfg, max_iter):
     """scikit-learn's Lloyd (OpenMP Cython) on the same data, inner routine only."""
     from sklearn.cluster._kmeans import _kmeans_single_lloyd
@@ -499,6 +591,27 @@ def cpu_lloyd_baseline(cfg, max_iter):
     elapsed = time.perf_counter() - t0
     # the routine ends with one extra labelling pass; count it as the work it is
     return n_iter / elapsed, threads, n_iter, elapsed
+
+
+def cpu_fit_baseline(cfg, max_iter):
+    """The reference benchmark's own protocol (benchmark/kmeans.py:137-170) on stock
+    scikit-learn: KMeans(init=<array>, n_init=1, tol=0, algorithm="lloyd", copy_x=True).fit
+    timed with perf_counter after a max_iter=1 dry run; iterations per second = n_iter_ / elapsed."""
+    from sklearn.cluster import KMeans
+
+    X, init, w = cfg["X"], cfg["init"], cfg["sample_weight"]
+    kwargs = dict(n_clusters=cfg["k"], init=init.copy(), n_init=1, max_iter=max_iter, tol=0, random_state=0,
+                  copy_x=True, algorithm="lloyd")
+    import warnings
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")   # ConvergenceWarning: max_iter is the point
+        KMeans(**kwargs).set_params(max_iter=1).fit(X, sample_weight=w)
+        est = KMeans(**kwargs)
+        t0 = time.perf_counter()
+        est.fit(X, sample_weight=w)
+        elapsed = time.perf_counter() - t0
+    return est.n_iter_ / elapsed, int(est.n_iter_), elapsed
 
 
 def main():
@@ -545,7 +658,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    elapsed, kernel_ms, ties, variant, rechecked, ramp_iters = gpu_lloyd(cfg, args.steps, args.warmup)
+    elapsed, kernel_ms, ties, variant, rechecked, ramp_iters, regions = gpu_lloyd(cfg, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     iters_per_s = args.steps / elapsed
     fused_s = kernel_ms[0] * 1e-3
@@ -556,10 +669,14 @@ def main():
         f"samples evaluated in fp32 by the last iteration: {rechecked} ({rechecked / n:.2e} of n)")
 
     traffic = None
+    traffic_source = None
     traffic_file = os.path.join(ROOT, "profiles", "lloyd_fused_step_c2_traffic.json")
     if os.path.exists(traffic_file) and n == 5_000_000:
         with open(traffic_file) as f:
             traffic = json.load(f).get("hbm_bytes_per_launch")
+        traffic_source = ("profiles/lloyd_fused_step_c2_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
+                          "kernel on this workload, calibrated against a 1 GiB copy; a committed counter reading, "
+                          "not taken in this run")
 
     mfma_roof = {
         "bound": "mfma",
@@ -568,6 +685,7 @@ def main():
         "unit": "TFLOP/s",
         "frac": flops / fused_s / 1e12 / FP32_PEAK_TFLOPS,
         "traffic": traffic,
+        "traffic_source": traffic_source,
         "kernel": "fused Lloyd step",
         "flops_per_launch": flops,
     }
@@ -578,6 +696,7 @@ def main():
         "unit": "GB/s",
         "frac": nbytes / fused_s / 1e9 / HBM_PEAK_GBS,
         "traffic": traffic,
+        "traffic_source": traffic_source,
         "kernel": "fused Lloyd step",
         "bytes_per_launch": nbytes,
     }
@@ -586,11 +705,19 @@ def main():
     # Variant 31 (KMX_FLAG_LABELS_F32) multiplies in fp32 and is priced against the fp32 MFMA peak.
     roofline, roofline_other = (hbm_roof, mfma_roof) if int(variant) == 61 else (mfma_roof, hbm_roof)
     if int(variant) == 61:
-        mfma_roof["note"] = ("2 n d k flops of the exact contraction over the fp32 MFMA peak, for comparison "
-                             "with the all-fp32 kernel; this kernel runs 3 fp16 products per fp32 one instead")
+        # this kernel multiplies on the fp16 matrix cores: the fp32 peak does not bound it, so the
+        # rate of the exact contraction it replaces is reported as a rate, not as a fraction
+        roofline_other = {
+            "fp32_equivalent_TFLOPs": mfma_roof["achieved"],
+            "flops_per_launch": flops,
+            "kernel": "fused Lloyd step",
+            "note": "2 n d k + 2 n d flops of the exact fp32 contraction over the kernel time, for comparison "
+                    "with the all-fp32 kernel (all_fp32); this kernel runs 3 fp16 products per fp32 one "
+                    "instead, so the fp32 MFMA peak (157.3 TFLOP/s) is no bound for it",
+        }
 
     # the same fit with every product taken in fp32 (variant 31), timed the same way
-    e32, kms32, _, variant32, _, _ = gpu_lloyd(cfg, args.steps, args.warmup, flags=FLAG_LABELS_F32, gates=False)
+    e32, kms32, _, variant32, _, _, _ = gpu_lloyd(cfg, args.steps, args.warmup, flags=FLAG_LABELS_F32, gates=False)
     all_fp32 = {
         "switch": "KMX_FLAG_LABELS_F32", "kernel_variant": int(variant32),
         "ms_per_step": e32 / args.steps * 1e3, "iters_per_sec": args.steps / e32,
@@ -603,7 +730,8 @@ def main():
     peaks = gpu_measured_peaks()
     log("[bench] measured peaks: " + ", ".join(f"{k2} {v:.1f}" for k2, v in peaks.items() if isinstance(v, float)))
     hbm_roof["frac_of_measured_peak"] = hbm_roof["achieved"] / peaks["read_GBps"]
-    mfma_roof["frac_of_measured_peak"] = mfma_roof["achieved"] / peaks["mfma_f32_TFLOPs"]
+    if int(variant) != 61:
+        mfma_roof["frac_of_measured_peak"] = mfma_roof["achieved"] / peaks["mfma_f32_TFLOPs"]
     all_fp32["frac_of_measured_fp32_peak"] = all_fp32["fused_step_TFLOPs"] / peaks["mfma_f32_TFLOPs"]
 
     out = {
@@ -614,7 +742,10 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "clock_ramp_iters": int(ramp_iters),
-        "timed_iterations": f"{args.warmup + 1}..{args.warmup + args.steps} of a fit from the initial centroids",
+        "timed_iterations": f"{REGIONS} regions of {args.steps} iterations, one after the other from iteration "
+                            f"{args.warmup + 1} of a fit from the initial centroids; value and ms_per_step are the "
+                            "median region's",
+        "ms_per_step_regions": [r / args.steps * 1e3 for r in regions],
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -649,6 +780,19 @@ def main():
                            "ms": kpp_ms, "hbm_GBs": kpp_bytes / (kpp_ms * 1e-3) / 1e9,
                            "hbm_frac": kpp_bytes / (kpp_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
         log(f"[bench] kmeans++ {kpp_ms:.1f} ms ({time.time() - t0:.1f}s incl. data)")
+        t0 = time.time()
+        out["kmeanspp"]["sampler_vs_reference"] = kpp_sampler_report(c4)
+        log(f"[bench] kmeans++ samplers: {out['kmeanspp']['sampler_vs_reference']} ({time.time() - t0:.1f}s)")
+        if not args.no_cpu:
+            cpu_kpp_ms, cpu_kpp_threads = cpu_kmeanspp_baseline(c4)
+            out["cpu_baseline_kmeanspp"] = {
+                "value": cpu_kpp_ms, "unit": "ms", "cores": int(cpu_kpp_threads), "kind": "reference",
+                "impl": "sklearn.cluster.kmeans_plusplus(X, %d, random_state=%d), scikit-learn %s (numpy/BLAS "
+                        "distances, one candidate batch per centre)" % (c4["k"], c4["seed"],
+                                                                         __import__("sklearn").__version__),
+                "sample": f"the whole seeding at full n={n4}, d={d4}",
+            }
+            log(f"[bench] sklearn CPU kmeans++: {cpu_kpp_ms:.0f} ms")
         del c4
 
     if not args.no_extra:
@@ -662,6 +806,14 @@ def main():
         if cfg is None:
             cfg = datasets.config2(n=args.n)
         cpu_ips, threads, cpu_iters, cpu_elapsed = cpu_lloyd_baseline(cfg, args.cpu_iters)
+        fit_ips, fit_iters, fit_elapsed = cpu_fit_baseline(cfg, args.cpu_iters)
+        try:
+            from threadpoolctl import threadpool_info
+
+            pools = [{key: p.get(key) for key in ("user_api", "internal_api", "prefix", "num_threads", "version")}
+                     for p in threadpool_info()]
+        except Exception as exc:  # the baseline does not depend on it
+            pools = repr(exc)
         out["cpu_baseline"] = {
             "value": cpu_ips,
             "unit": "iter/s",
@@ -671,6 +823,11 @@ def main():
                     "plugin subclasses and falls back to" % __import__("sklearn").__version__,
             "sample": f"same data and init, {cpu_iters} iterations at full n={n} in {cpu_elapsed:.1f}s "
                       f"(os.cpu_count()={os.cpu_count()})",
+            "estimator_fit": {"iters_per_sec": fit_ips, "n_iter": fit_iters, "seconds": fit_elapsed,
+                              "what": "KMeans(init=array, n_init=1, tol=0, algorithm='lloyd', copy_x=True).fit(X, "
+                                      "sample_weight) after a max_iter=1 dry run: input validation, centering "
+                                      "and the final labelling included"},
+            "threadpool_info": pools,
         }
         log(f"[bench] sklearn CPU Lloyd: {cpu_ips:.3f} iter/s on {threads} threads")
 

@@ -46,7 +46,7 @@ extern "C" {
 
 #define KMX_ERR_BAD_PLAN (-7)       /* kmx_lloyd_plan not made by kmx_lloyd_plan_init, or edited */
 
-#define KMX_ABI_VERSION 2
+#define KMX_ABI_VERSION 3
 int32_t kmx_abi_version(void);
 const char* kmx_error_string(int32_t code);
 
@@ -316,18 +316,34 @@ size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials
 int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_index,
                      void* centers_t, int32_t* center_indices, void* workspace,
                      size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
-                     int32_t dtype, void* stream);
+                     int32_t dtype, uint32_t flags, void* stream);
 
-/* Candidate t = first j with (inclusive fp64 scan of closest)_j >= uniforms[t] * total,
- * clipped to [0, n-1].  Replaces make_sample_center_candidates_kernel
- * (kmeans/kernels/kmeans_plusplus.py:61-103), whose serial scan becomes a two-level search
- * over the block potentials already held in the workspace.
+/* Which sampler kmx_kpp_sample_candidates and kmx_kpp_run use (`flags`).
+ * KMX_KPP_SAMPLER_SCAN (default): candidate t = first j with (inclusive fp64 scan of closest)_j
+ * >= uniforms[t] * total, clipped to [0, n-1]: a two-level search over the block potentials
+ * already held in the workspace.
+ * KMX_KPP_SAMPLER_LITERAL: the reference's sampler statement by statement
+ * (kmeans/kernels/kmeans_plusplus.py:79-100): running sum of closest in the compute dtype from
+ * sample 0, first j whose running sum reaches T(uniforms[t]) * T(total), clipped to n-1; a
+ * trial with uniforms[t] * total <= 0 gets n-1 (the reference leaves -1 there, which its next
+ * kernel reads as an index from the end).  With the same flag kmx_kpp_init and kmx_kpp_step
+ * round the product and the sum of every squared difference separately, as the reference's two
+ * statements do (the default is one fused multiply-add: the running sum in the compute dtype
+ * turns a last-bit difference in one distance into another candidate), and kmx_kpp_step
+ * compares the trial potentials after rounding them to the compute dtype.  One wave walks the
+ * array: about 8 ns per sample and centre, for parity checks against the reference, not for
+ * speed. */
+#define KMX_KPP_SAMPLER_SCAN 0x0u
+#define KMX_KPP_SAMPLER_LITERAL 0x1u
+
+/* Replaces make_sample_center_candidates_kernel (kmeans/kernels/kmeans_plusplus.py:61-103).
  *   uniforms_for_step  IN  (n_trials) doubles in [0, 1)
- *   candidates         OUT (n_trials) int32, may be NULL (they stay in the workspace) */
+ *   candidates         OUT (n_trials) int32, may be NULL (they stay in the workspace)
+ *   flags              KMX_KPP_SAMPLER_*; anything else: KMX_ERR_BAD_ARGUMENT */
 int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_step,
                                   int32_t* candidates, void* workspace, size_t workspace_bytes,
                                   int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype,
-                                  void* stream);
+                                  uint32_t flags, void* stream);
 
 /* For every candidate t and sample i: min(w_i ||x_i - x_cand_t||^2, closest_i), row sums,
  * argmin over t (lowest t wins ties), closest <- best row, centers_t[:, c] <- x_best,
@@ -337,15 +353,16 @@ int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_st
 int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_slot,
                      void* centers_t, int32_t* center_indices, void* workspace,
                      size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
-                     int32_t dtype, void* stream);
+                     int32_t dtype, uint32_t flags, void* stream);
 
 /* The whole seeding (init, then k-1 x [sample, step]) with no host round trip.
  *   uniforms  IN (k-1, n_trials) doubles: row c-1 holds what trial t draws for centre c.
+ *   flags     KMX_KPP_SAMPLER_*
  * Replaces kmeans_plusplus(), kmeans/drivers.py:735-910. */
 int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* uniforms,
                     int32_t start_index, void* centers_t, int32_t* center_indices,
                     void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
-                    int32_t n_trials, int32_t dtype, void* stream);
+                    int32_t n_trials, int32_t dtype, uint32_t flags, void* stream);
 
 /* Views into the kmeans++ workspace, for tests: closest (n) in `dtype`, potentials
  * (n_trials) doubles of the last step, candidates (n_trials) int32. */

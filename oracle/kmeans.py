@@ -336,7 +336,8 @@ def kmeans_plusplus(X, sample_weight, n_clusters, seed, sampler="exact", return_
         cands = np.empty(n_trials, dtype=np.int64)
         for t in range(n_trials):
             if sampler == "literal":
-                cands[t] = _sample_literal(closest, total, table[c - 1, t])
+                # -1 (rv <= 0) is used by the reference's next kernel as an index from the end
+                cands[t] = _sample_literal(closest, total, table[c - 1, t]) % n
             else:
                 cands[t] = _sample_exact(closest, table[c - 1, t])
         rows = np.stack([np.minimum(wdist(int(i)), closest) for i in cands])

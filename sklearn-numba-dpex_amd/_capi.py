@@ -25,6 +25,10 @@ KMX_CONVERGED_TOL = 2
 KMX_MAX_ITER = 3
 KMX_NEED_RELOCATION = 4
 
+# kmeans++ samplers (KMX_KPP_SAMPLER_* of the header)
+KMX_KPP_SAMPLER_SCAN = 0
+KMX_KPP_SAMPLER_LITERAL = 1
+
 KMX_ERR_BAD_PLAN = -7
 
 # kernel selection flags (KMX_FLAG_* of the header)
@@ -44,7 +48,7 @@ def flag_cols(x):
     return (int(x) & 0x7) << 12
 
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 LIB_NAME = "libmi355x_kmeans.so"
 # (KMX_LIBRARY_PATH: another build of the same library, for experiments; read when this module is imported)
@@ -127,10 +131,10 @@ SIGNATURES = {
     "kmx_rng_init_states": (_I32, [ctypes.c_uint64, _I32, _I32, _P]),
     "kmx_rng_next_raw": (_I32, [_P, _I32, _I32, _P]),
     "kmx_kpp_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
-    "kmx_kpp_init": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
-    "kmx_kpp_sample_candidates": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
-    "kmx_kpp_step": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
-    "kmx_kpp_run": (_I32, [_P, _P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _P]),
+    "kmx_kpp_init": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _U32, _P]),
+    "kmx_kpp_sample_candidates": (_I32, [_P, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _U32, _P]),
+    "kmx_kpp_step": (_I32, [_P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _U32, _P]),
+    "kmx_kpp_run": (_I32, [_P, _P, _P, _I32, _P, _P, _P, _SZ, _I64, _I32, _I32, _I32, _I32, _U32, _P]),
     "kmx_kpp_closest_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),
     "kmx_kpp_potentials_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),
     "kmx_kpp_candidates_ptr": (_P, [_P, _I64, _I32, _I32, _I32, _I32]),

@@ -50,8 +50,24 @@ KppLayout kpp_layout(int64_t n, int d, int n_trials, int dtype) {
     return L;
 }
 
+// acc + diff^2.  FUSED: one rounding (fused multiply-add), the default.  Not FUSED: product and
+// sum rounded separately, the two statements of the reference's kernels taken literally
+// (kmeans/kernels/kmeans_plusplus.py:44-48, 226-230); the literal sampler's running sum in the
+// compute dtype amplifies a last-bit difference in one distance into another candidate, so
+// the literal mode has to reproduce the distances bit for bit as well.
+template <bool FUSED, typename T>
+__device__ __forceinline__ T kpp_sq_acc(T diff, T acc) {
+    if constexpr (FUSED) {
+        return fma(diff, diff, acc);
+    } else {
+#pragma clang fp contract(off)
+        const T p = diff * diff;
+        return acc + p;
+    }
+}
+
 // closest = w * ||x - x_start||^2 into row 0; per-block potential; slot 0 of the outputs.
-template <typename T>
+template <typename T, bool FUSED>
 __global__ __launch_bounds__(256) void kpp_init_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight, int32_t start,
     T* __restrict__ centers_t, int32_t* __restrict__ center_indices, T* __restrict__ rows,
@@ -65,7 +81,7 @@ __global__ __launch_bounds__(256) void kpp_init_kernel(
         for (int r = 0; r < 4; ++r) {
             if (i0 + r < n) {
                 const T diff = row[i0 + r] - sv;
-                acc[r] = fma(diff, diff, acc[r]);
+                acc[r] = kpp_sq_acc<FUSED>(diff, acc[r]);
             }
         }
     }
@@ -129,7 +145,7 @@ __device__ __forceinline__ void store4(T* __restrict__ row, int64_t i0, int64_t 
 // Candidate rows come from a small (TN, d) buffer through wave-uniform loads (the values sit
 // in SGPRs, no LDS, no barriers in the feature loop); every thread streams 4 consecutive
 // samples of 8 features at a time with 128-bit loads.
-template <typename T, int TN>
+template <typename T, int TN, bool FUSED>
 __global__ __launch_bounds__(256) void kpp_step_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cand_rows,
     T* __restrict__ rows, double* __restrict__ block_pot, const KppHeader* __restrict__ header,
@@ -179,7 +195,7 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
                             const T diff = xv[j][r] - cv;
-                            acc[t][r] = fma(diff, diff, acc[t][r]);
+                            acc[t][r] = kpp_sq_acc<FUSED>(diff, acc[t][r]);
                         }
                     }
                 }
@@ -324,10 +340,15 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
             }
         }
         __syncthreads();
+        // do_select == 2: the potentials are compared after rounding to T, as the reference's
+        // argmin over its T-typed row sums does (kmeans/drivers.py:895-901)
+        const bool in_T = do_select == 2;
         double best_pot = (wave_pot[0][0] + wave_pot[1][0]) + (wave_pot[2][0] + wave_pot[3][0]);
+        if (in_T) best_pot = (double)(T)best_pot;
         best = 0;
         for (int t = 1; t < n_trials; ++t) {
-            const double pt = (wave_pot[0][t] + wave_pot[1][t]) + (wave_pot[2][t] + wave_pot[3][t]);
+            double pt = (wave_pot[0][t] + wave_pot[1][t]) + (wave_pot[2][t] + wave_pot[3][t]);
+            if (in_T) pt = (double)(T)pt;
             if (pt < best_pot) {
                 best_pot = pt;
                 best = t;
@@ -435,6 +456,135 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     for (int f = threadIdx.x; f < d; f += 256) cand_rows[(size_t)trial * d + f] = X_t[(size_t)f * n + cand];
 }
 
+// The reference's sampler taken literally (kmeans/kernels/kmeans_plusplus.py:79-100): a
+// running sum of `closest` in T, element by element from sample 0, and per trial the first j
+// whose running sum reaches rv_t = T(u_t) * T(total), clipped to n - 1.  A floating-point
+// running sum cannot be split over threads without changing its roundings, so one wave walks the
+// array once for all trials (sorted by rv: the sum of non-negative terms never decreases, so
+// the trials are met in that order) while the workgroup's 256 threads keep the next 1 024
+// values on their way into LDS.  A trial with rv <= 0 leaves the reference's loop at once with
+// candidate -1, which its next kernel uses as an index from the end: sample n - 1.
+// About 8 ns per sample (8 ms per centre on 10^6 samples): a parity mode, not the default.
+template <typename T>
+__global__ __launch_bounds__(256) void kpp_sample_literal_kernel(
+    const T* __restrict__ X_t, const double* __restrict__ uniforms, int32_t* __restrict__ cand_next,
+    int32_t* __restrict__ cand_out, const T* __restrict__ rows, const double* __restrict__ block_pot,
+    const KppHeader* __restrict__ header, T* __restrict__ cand_rows, int64_t n, int64_t n_blocks, int d,
+    int n_trials) {
+    __shared__ T buf[2][CHUNK];
+    __shared__ double wave_tot[4];
+    __shared__ T rv_sorted[TN_MAX + 1];
+    __shared__ int trial_sorted[TN_MAX];
+    __shared__ int cand_s[TN_MAX];
+    __shared__ int done_s;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int best = header->best_row;
+    const T* __restrict__ closest = rows + (size_t)best * n;
+
+    // total potential: the block sums of the best row in fp64, rounded to T once
+    double local = 0.0;
+    for (int64_t b = threadIdx.x; b < n_blocks; b += 256) local += block_pot[(size_t)b * TN_MAX + best];
+    const double ws = kmx_wave_sum<double>(local);
+    if (lane == 0) wave_tot[wave] = ws;
+    __syncthreads();
+    const T total = (T)((wave_tot[0] + wave_tot[1]) + (wave_tot[2] + wave_tot[3]));
+
+    if (threadIdx.x == 0) {
+        // insertion sort of the trials by rv; rv <= 0 (or NaN) first
+        int m = 0;
+        for (int t = 0; t < n_trials; ++t) {
+            const T rv = (T)uniforms[t] * total;
+            const bool low = !(rv > T(0));
+            int pos = m;
+            while (pos > 0) {
+                const T prev = rv_sorted[pos - 1];
+                const bool prev_low = !(prev > T(0));
+                if (prev_low || (!low && !(rv < prev))) break;
+                rv_sorted[pos] = prev;
+                trial_sorted[pos] = trial_sorted[pos - 1];
+                --pos;
+            }
+            rv_sorted[pos] = rv;
+            trial_sorted[pos] = t;
+            ++m;
+        }
+        rv_sorted[n_trials] = T(0);
+        done_s = 0;
+    }
+    const int64_t n_chunks = n_blocks;
+    // first chunk
+    {
+        const int64_t j0 = (int64_t)threadIdx.x * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) buf[0][threadIdx.x * 4 + r] = (j0 + r < n) ? closest[j0 + r] : T(0);
+    }
+    __syncthreads();
+
+    int cur = 0;
+    T cum = T(0);
+    if (wave == 0) {
+        // trials that never enter the loop
+        while (cur < n_trials && !(rv_sorted[cur] > T(0))) {
+            if (lane == 0) cand_s[trial_sorted[cur]] = (int)(n - 1);
+            ++cur;
+        }
+    }
+    for (int64_t c = 0; c < n_chunks; ++c) {
+        T nxt[4] = {T(0), T(0), T(0), T(0)};
+        if (c + 1 < n_chunks) {
+            const int64_t j0 = (c + 1) * CHUNK + (int64_t)threadIdx.x * 4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) nxt[r] = (j0 + r < n) ? closest[j0 + r] : T(0);
+        }
+        if (wave == 0) {
+            const T* __restrict__ b = buf[c & 1];
+            const int64_t base = c * CHUNK;
+            const int lim = (int)((n - base) < CHUNK ? (n - base) : CHUNK);
+            T rv_cur = rv_sorted[cur];
+            for (int i = 0; i < lim && cur < n_trials; i += 16) {
+                if (i + 16 <= lim) {
+                    T v[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) v[r] = b[i + r];
+                    T cc = cum;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) cc = cc + v[r];
+                    if (rv_cur > cc) {
+                        cum = cc;
+                        continue;
+                    }
+                }
+                for (int r = 0; r < 16 && i + r < lim; ++r) {
+                    cum = cum + b[i + r];
+                    while (cur < n_trials && !(rv_cur > cum)) {
+                        if (lane == 0) cand_s[trial_sorted[cur]] = (int)(base + i + r);
+                        ++cur;
+                        rv_cur = rv_sorted[cur];
+                    }
+                }
+            }
+            if (lane == 0 && cur >= n_trials) done_s = 1;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) buf[(c + 1) & 1][threadIdx.x * 4 + r] = nxt[r];
+        __syncthreads();
+        if (done_s) break;
+    }
+    if (wave == 0 && lane == 0) {
+        // the running sum never reached these: the reference's loop stops at the last sample
+        for (; cur < n_trials; ++cur) cand_s[trial_sorted[cur]] = (int)(n - 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < n_trials) {
+        cand_next[threadIdx.x] = cand_s[threadIdx.x];
+        if (cand_out) cand_out[threadIdx.x] = cand_s[threadIdx.x];
+    }
+    for (int t = 0; t < n_trials; ++t) {
+        const int64_t cand = cand_s[t];
+        for (int f = threadIdx.x; f < d; f += 256) cand_rows[(size_t)t * d + f] = X_t[(size_t)f * n + cand];
+    }
+}
+
 struct KppPtrs {
     KppHeader* header;
     void* cand_rows;
@@ -469,33 +619,52 @@ int32_t kpp_check(const void* X_t, const void* w, void* ws, size_t ws_bytes, int
 
 template <typename T>
 void launch_init(const void* X_t, const void* w, int32_t start, void* centers_t, int32_t* idx,
-                 const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k, hipStream_t s) {
-    hipLaunchKernelGGL((kpp_init_kernel<T>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
-                       (const T*)X_t, (const T*)w, start, (T*)centers_t, idx, (T*)p.rows,
-                       p.block_pot, p.header, n, d, k);
+                 const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k, hipStream_t s, bool literal) {
+    if (literal)
+        hipLaunchKernelGGL((kpp_init_kernel<T, false>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
+                           (const T*)X_t, (const T*)w, start, (T*)centers_t, idx, (T*)p.rows,
+                           p.block_pot, p.header, n, d, k);
+    else
+        hipLaunchKernelGGL((kpp_init_kernel<T, true>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
+                           (const T*)X_t, (const T*)w, start, (T*)centers_t, idx, (T*)p.rows,
+                           p.block_pot, p.header, n, d, k);
 }
 
 template <typename T>
 void launch_step(const void* X_t, const void* w, const int32_t* cand, const KppPtrs& p,
-                 const KppLayout& L, int64_t n, int d, int n_trials, hipStream_t s) {
+                 const KppLayout& L, int64_t n, int d, int n_trials, hipStream_t s, bool literal) {
     (void)cand;  // the candidates' rows were copied to p.cand_rows when they were sampled
     const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0) && (((uintptr_t)w) % 16 == 0) &&
                        (((uintptr_t)p.rows) % 16 == 0);
-    if (n_trials <= 8)
-        hipLaunchKernelGGL((kpp_step_kernel<T, 8>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
-                           (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,
-                           p.header, n, d, n_trials, vec_ok);
-    else
-        hipLaunchKernelGGL((kpp_step_kernel<T, TN_MAX>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
-                           (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,
-                           p.header, n, d, n_trials, vec_ok);
+#define KMX_KPP_STEP(TN, FUSED)                                                                      \
+    hipLaunchKernelGGL((kpp_step_kernel<T, TN, FUSED>), dim3((unsigned)L.n_blocks), dim3(256), 0, s, \
+                       (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,   \
+                       p.header, n, d, n_trials, vec_ok)
+    if (n_trials <= 8) {
+        if (literal) KMX_KPP_STEP(8, false); else KMX_KPP_STEP(8, true);
+    } else {
+        if (literal) KMX_KPP_STEP(TN_MAX, false); else KMX_KPP_STEP(TN_MAX, true);
+    }
+#undef KMX_KPP_STEP
 }
 
 template <typename T>
 void launch_select_sample(const void* X_t, const double* uniforms, const int32_t* cand_prev,
                           int32_t* cand_next, int32_t* cand_out, void* centers_t, int32_t* idx,
                           const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k,
-                          int n_trials, int slot, int do_select, int do_sample, hipStream_t s) {
+                          int n_trials, int slot, int do_select, int do_sample, hipStream_t s,
+                          bool literal = false) {
+    if (literal) {
+        // the selection alone (potentials compared in T), then the serial walk of one workgroup
+        if (do_select)
+            launch_select_sample<T>(X_t, uniforms, cand_prev, cand_next, cand_out, centers_t, idx, p, L, n, d, k,
+                                    n_trials, slot, 2, 0, s);
+        if (do_sample)
+            hipLaunchKernelGGL((kpp_sample_literal_kernel<T>), dim3(1), dim3(256), 0, s, (const T*)X_t, uniforms,
+                               cand_next, cand_out, (const T*)p.rows, p.block_pot, p.header, (T*)p.cand_rows, n,
+                               L.n_blocks, d, n_trials);
+        return;
+    }
     // one workgroup per trial when sampling, one more when a selection is recorded
     const unsigned grid = (do_sample ? (unsigned)n_trials : 0u) + (do_select ? 1u : 0u);
     if (grid == 0) return;
@@ -526,20 +695,22 @@ size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials
 int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_index,
                      void* centers_t, int32_t* center_indices, void* workspace,
                      size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
-                     int32_t dtype, void* stream_) {
+                     int32_t dtype, uint32_t flags, void* stream_) {
     KMX_ENTRY();
     const int32_t rc = kpp_check(X_t, sample_weight, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
     KMX_REQUIRE_PTR(centers_t);
     KMX_REQUIRE_PTR(center_indices);
+    if (flags & ~(uint32_t)KMX_KPP_SAMPLER_LITERAL) return KMX_ERR_BAD_ARGUMENT;
+    const bool literal = (flags & KMX_KPP_SAMPLER_LITERAL) != 0;
     if (start_index < 0 || start_index >= n) return KMX_ERR_BAD_ARGUMENT;
     const KppLayout L = kpp_layout(n, d, n_trials, dtype);
     const KppPtrs p = kpp_ptrs((char*)workspace, L);
     hipStream_t s = (hipStream_t)stream_;
     if (dtype == KMX_F32)
-        launch_init<float>(X_t, sample_weight, start_index, centers_t, center_indices, p, L, n, d, k, s);
+        launch_init<float>(X_t, sample_weight, start_index, centers_t, center_indices, p, L, n, d, k, s, literal);
     else
-        launch_init<double>(X_t, sample_weight, start_index, centers_t, center_indices, p, L, n, d, k, s);
+        launch_init<double>(X_t, sample_weight, start_index, centers_t, center_indices, p, L, n, d, k, s, literal);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
@@ -547,9 +718,11 @@ int32_t kmx_kpp_init(const void* X_t, const void* sample_weight, int32_t start_i
 int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_step,
                                   int32_t* candidates, void* workspace, size_t workspace_bytes,
                                   int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype,
-                                  void* stream_) {
+                                  uint32_t flags, void* stream_) {
     KMX_ENTRY();
     KMX_REQUIRE_PTR(uniforms_for_step);
+    if (flags & ~(uint32_t)KMX_KPP_SAMPLER_LITERAL) return KMX_ERR_BAD_ARGUMENT;
+    const bool literal = (flags & KMX_KPP_SAMPLER_LITERAL) != 0;
     const int32_t rc = kpp_check(X_t, uniforms_for_step, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
     const KppLayout L = kpp_layout(n, d, n_trials, dtype);
@@ -557,10 +730,10 @@ int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_st
     hipStream_t s = (hipStream_t)stream_;
     if (dtype == KMX_F32)
         launch_select_sample<float>(X_t, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
-                                    nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s);
+                                    nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s, literal);
     else
         launch_select_sample<double>(X_t, uniforms_for_step, p.cand, p.cand, candidates, nullptr,
-                                     nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s);
+                                     nullptr, p, L, n, d, k, n_trials, 0, 0, 1, s, literal);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }
@@ -568,24 +741,26 @@ int32_t kmx_kpp_sample_candidates(const void* X_t, const double* uniforms_for_st
 int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_slot,
                      void* centers_t, int32_t* center_indices, void* workspace,
                      size_t workspace_bytes, int64_t n, int32_t d, int32_t k, int32_t n_trials,
-                     int32_t dtype, void* stream_) {
+                     int32_t dtype, uint32_t flags, void* stream_) {
     KMX_ENTRY();
     const int32_t rc = kpp_check(X_t, sample_weight, workspace, workspace_bytes, n, d, k, n_trials, dtype);
     if (rc != KMX_OK) return rc;
     KMX_REQUIRE_PTR(centers_t);
     KMX_REQUIRE_PTR(center_indices);
+    if (flags & ~(uint32_t)KMX_KPP_SAMPLER_LITERAL) return KMX_ERR_BAD_ARGUMENT;
+    const bool literal = (flags & KMX_KPP_SAMPLER_LITERAL) != 0;
     if (center_slot < 1 || center_slot >= k) return KMX_ERR_BAD_ARGUMENT;
     const KppLayout L = kpp_layout(n, d, n_trials, dtype);
     const KppPtrs p = kpp_ptrs((char*)workspace, L);
     hipStream_t s = (hipStream_t)stream_;
     if (dtype == KMX_F32) {
-        launch_step<float>(X_t, sample_weight, p.cand, p, L, n, d, n_trials, s);
+        launch_step<float>(X_t, sample_weight, p.cand, p, L, n, d, n_trials, s, literal);
         launch_select_sample<float>(X_t, nullptr, p.cand, nullptr, nullptr, centers_t, center_indices,
-                                    p, L, n, d, k, n_trials, center_slot, 1, 0, s);
+                                    p, L, n, d, k, n_trials, center_slot, 1, 0, s, literal);
     } else {
-        launch_step<double>(X_t, sample_weight, p.cand, p, L, n, d, n_trials, s);
+        launch_step<double>(X_t, sample_weight, p.cand, p, L, n, d, n_trials, s, literal);
         launch_select_sample<double>(X_t, nullptr, p.cand, nullptr, nullptr, centers_t,
-                                     center_indices, p, L, n, d, k, n_trials, center_slot, 1, 0, s);
+                                     center_indices, p, L, n, d, k, n_trials, center_slot, 1, 0, s, literal);
     }
     KMX_LAUNCH_CHECK();
     return KMX_OK;
@@ -594,10 +769,12 @@ int32_t kmx_kpp_step(const void* X_t, const void* sample_weight, int32_t center_
 int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* uniforms,
                     int32_t start_index, void* centers_t, int32_t* center_indices,
                     void* workspace, size_t workspace_bytes, int64_t n, int32_t d, int32_t k,
-                    int32_t n_trials, int32_t dtype, void* stream_) {
+                    int32_t n_trials, int32_t dtype, uint32_t flags, void* stream_) {
     KMX_ENTRY();
+    if (flags & ~(uint32_t)KMX_KPP_SAMPLER_LITERAL) return KMX_ERR_BAD_ARGUMENT;
+    const bool literal = (flags & KMX_KPP_SAMPLER_LITERAL) != 0;
     int32_t rc = kmx_kpp_init(X_t, sample_weight, start_index, centers_t, center_indices, workspace,
-                              workspace_bytes, n, d, k, n_trials, dtype, stream_);
+                              workspace_bytes, n, d, k, n_trials, dtype, flags, stream_);
     if (rc != KMX_OK) return rc;
     if (k == 1) return KMX_OK;
     KMX_REQUIRE_PTR(uniforms);
@@ -613,22 +790,22 @@ int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* un
         const int do_select = c > 1 ? 1 : 0;
         if (dtype == KMX_F32) {
             launch_select_sample<float>(X_t, u, cand_prev, cand_next, nullptr, centers_t,
-                                        center_indices, p, L, n, d, k, n_trials, c - 1, do_select, 1, s);
-            launch_step<float>(X_t, sample_weight, cand_next, p, L, n, d, n_trials, s);
+                                        center_indices, p, L, n, d, k, n_trials, c - 1, do_select, 1, s, literal);
+            launch_step<float>(X_t, sample_weight, cand_next, p, L, n, d, n_trials, s, literal);
         } else {
             launch_select_sample<double>(X_t, u, cand_prev, cand_next, nullptr, centers_t,
-                                         center_indices, p, L, n, d, k, n_trials, c - 1, do_select, 1, s);
-            launch_step<double>(X_t, sample_weight, cand_next, p, L, n, d, n_trials, s);
+                                         center_indices, p, L, n, d, k, n_trials, c - 1, do_select, 1, s, literal);
+            launch_step<double>(X_t, sample_weight, cand_next, p, L, n, d, n_trials, s, literal);
         }
         KMX_LAUNCH_CHECK();
     }
     int32_t* cand_last = p.cand + ((k - 1) & 1) * TN_MAX;
     if (dtype == KMX_F32)
         launch_select_sample<float>(X_t, nullptr, cand_last, nullptr, nullptr, centers_t,
-                                    center_indices, p, L, n, d, k, n_trials, k - 1, 1, 0, s);
+                                    center_indices, p, L, n, d, k, n_trials, k - 1, 1, 0, s, literal);
     else
         launch_select_sample<double>(X_t, nullptr, cand_last, nullptr, nullptr, centers_t,
-                                     center_indices, p, L, n, d, k, n_trials, k - 1, 1, 0, s);
+                                     center_indices, p, L, n, d, k, n_trials, k - 1, 1, 0, s, literal);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

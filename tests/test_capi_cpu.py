@@ -27,7 +27,7 @@ def test_library_exports_every_declared_function():
     for name in declared:
         assert hasattr(raw, name), f"{name} is declared in the header but not exported"
     assert sorted(_capi.SIGNATURES) == declared, "ctypes signatures and header disagree"
-    assert _capi.lib.kmx_abi_version() == 2
+    assert _capi.lib.kmx_abi_version() == 3
 
 
 def test_header_cites_the_reference_for_every_entry_point():
@@ -221,9 +221,9 @@ def test_bad_arguments_are_rejected_without_a_device():
     assert lib.kmx_topk_values(p, p, 3, 50, 10, p, 8, 1, NULL) == -4
     assert lib.kmx_topk_values(p, p, 3, 50, 10, p, 1 << 20, 7, NULL) == -3     # unknown dtype
     assert lib.kmx_broadcast_rows(p, p, 2, 2, 3, 0, NULL) == -5       # unknown op
-    assert lib.kmx_kpp_init(p, p, 20, p, p, p, 1 << 20, 10, 2, 2, 2, 0, NULL) in (-4, -5)
-    assert lib.kmx_kpp_run(p, p, p, 0, p, p, p, 16, 10, 2, 2, 2, 0, NULL) == -4
-    assert lib.kmx_kpp_step(p, p, 1, p, p, p, 16, 10, 2, 2, 99, 0, NULL) == -6  # too many trials
+    assert lib.kmx_kpp_init(p, p, 20, p, p, p, 1 << 20, 10, 2, 2, 2, 0, 0, NULL) in (-4, -5)
+    assert lib.kmx_kpp_run(p, p, p, 0, p, p, p, 16, 10, 2, 2, 2, 0, 0, NULL) == -4
+    assert lib.kmx_kpp_step(p, p, 1, p, p, p, 16, 10, 2, 2, 99, 0, 0, NULL) == -6  # too many trials
     assert lib.kmx_relocate_empty_clusters(p, p, p, p, p, 3, NULL, p, p, 10, 2, 2, 0, NULL) == -2
     assert lib.kmx_sum_rows(p, p, 0, 5, 0, p, 4096, 0, NULL) == -2
     assert lib.kmx_matmul(p, p, NULL, 2, 2, 2, 0, NULL) == -1

@@ -150,9 +150,13 @@ def test_kmeanspp_contract_at_full_size(cuda):
     assert float(dist.min(dim=1).values.max()) < 30.0
 
 
-def test_kmeanspp_first_centres_match_oracle_at_full_n(cuda):
+@pytest.mark.parametrize("sampler", ["scan", "literal"])
+def test_kmeanspp_first_centres_match_oracle_at_full_n(cuda, sampler):
     """The first 12 centres on the full 1,000,000 x 64 data against the oracle's sampler fed
-    with the same uniform draws (the whole 256-centre seeding would take the oracle minutes)."""
+    with the same uniform draws (the whole 256-centre seeding would take the oracle minutes):
+    the default fp64 scan against the oracle's exact sampler, and the reference's own running
+    sum in fp32 (`KMX_KPP_SAMPLER_LITERAL`, kmeans/kernels/kmeans_plusplus.py:79-100) against the
+    oracle's literal one - at this size the two samplers pick different samples for most draws."""
     import torch
 
     from oracle import rng as orng
@@ -162,9 +166,10 @@ def test_kmeanspp_first_centres_match_oracle_at_full_n(cuda):
     X, k = cfg["X"], 12
     w = cfg["sample_weight"]
     X_t = torch.as_tensor(X, device=cuda).T.contiguous()
-    _, idx = drivers.kmeans_plusplus(X_t, torch.as_tensor(w, device=cuda), k, np.random.RandomState(cfg["seed"]))
+    _, idx = drivers.kmeans_plusplus(X_t, torch.as_tensor(w, device=cuda), k, np.random.RandomState(cfg["seed"]),
+                                     sampler=sampler)
     seed64 = orng.seed_from_random_state(np.random.RandomState(cfg["seed"]))
-    _, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact")
+    _, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact" if sampler == "scan" else "literal")
     np.testing.assert_array_equal(idx.cpu().numpy(), ref_idx)
 
 

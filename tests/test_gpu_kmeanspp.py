@@ -35,15 +35,19 @@ def _cases():
     }
 
 
+@pytest.mark.parametrize("sampler", ["scan", "literal"])
 @pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32", "many_trials_f32", "many_blocks_f64", "weighted_f32"])
-def test_whole_seeding_matches_oracle(cuda, name):
+def test_whole_seeding_matches_oracle(cuda, name, sampler):
+    """Both samplers of the library against their counterparts in the oracle: the fp64 scan
+    (default) and the reference's running sum in the compute dtype (`KMX_KPP_SAMPLER_LITERAL`)."""
     from sklearn_numba_dpex_amd.kmeans import drivers
 
     X, w, k, seed = _cases()[name]
     w = np.ones(len(X), X.dtype) if w is None else w.astype(X.dtype)
-    centers_t, idx = drivers.kmeans_plusplus(_dev(X.T, cuda), _dev(w, cuda), k, np.random.RandomState(seed))
+    centers_t, idx = drivers.kmeans_plusplus(_dev(X.T, cuda), _dev(w, cuda), k, np.random.RandomState(seed),
+                                             sampler=sampler)
     seed64 = orng.seed_from_random_state(np.random.RandomState(seed))
-    ref_centers, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact")
+    ref_centers, ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact" if sampler == "scan" else "literal")
     idx = idx.cpu().numpy()
     np.testing.assert_array_equal(idx, ref_idx)
     np.testing.assert_array_equal(centers_t.cpu().numpy().T, X[idx])
@@ -72,7 +76,7 @@ def test_step_kernels_through_c_abi(cuda, dtype):
     st = _capi.current_stream()
     start = 4242
     _capi.check(lib.kmx_kpp_init(ptr(X_t), ptr(w_d), start, ptr(centers_t), ptr(indices), ptr(ws), ws_bytes,
-                                 n, d, k, tn, dc, st), "kpp_init")
+                                 n, d, k, tn, dc, 0, st), "kpp_init")
     closest = (((X - X[start]) ** 2).sum(axis=1, dtype=dtype) * w).astype(dtype)
     rows_ptr = lib.kmx_kpp_closest_ptr(ptr(ws), n, d, k, tn, dc)
     off = rows_ptr - ws.data_ptr()
@@ -92,12 +96,22 @@ def test_step_kernels_through_c_abi(cuda, dtype):
         u[0] = 0.0 if c == 1 else u[0]            # rv == 0 -> first sample (reference would give -1)
         u[1] = 1.0 - 2.0**-53 if c == 2 else u[1]  # top of the range -> last crossing, clipped to n - 1
         cand = torch.empty(tn, dtype=torch.int32, device=cuda)
+        # the reference's own sampler first (its candidates are overwritten by the default one):
+        # running sum in T; rv <= 0 leaves -1 there, read as an index from the end
+        u_T = u.astype(dtype).astype(np.float64)
+        _capi.check(lib.kmx_kpp_sample_candidates(ptr(X_t), ptr(_dev(u_T, cuda)), ptr(cand), ptr(ws), ws_bytes, n, d, k,
+                                                  tn, dc, _capi.KMX_KPP_SAMPLER_LITERAL, st), "kpp_sample literal")
+        total_T = dtype(closest.sum(dtype=np.float64))
+        literal = np.array([ok._sample_literal(closest, total_T, dtype(uu)) % n for uu in u_T])
+        np.testing.assert_array_equal(cand.cpu().numpy(), literal)
+        assert lib.kmx_kpp_sample_candidates(ptr(X_t), ptr(_dev(u, cuda)), ptr(cand), ptr(ws), ws_bytes, n, d, k, tn,
+                                             dc, 2, st) == -5
         _capi.check(lib.kmx_kpp_sample_candidates(ptr(X_t), ptr(_dev(u, cuda)), ptr(cand), ptr(ws), ws_bytes, n, d, k, tn,
-                                                  dc, st), "kpp_sample")
+                                                  dc, _capi.KMX_KPP_SAMPLER_SCAN, st), "kpp_sample")
         expected = np.array([ok._sample_exact(closest, uu) for uu in u])
         np.testing.assert_array_equal(cand.cpu().numpy(), expected)
         _capi.check(lib.kmx_kpp_step(ptr(X_t), ptr(w_d), c, ptr(centers_t), ptr(indices), ptr(ws), ws_bytes,
-                                     n, d, k, tn, dc, st), "kpp_step")
+                                     n, d, k, tn, dc, 0, st), "kpp_step")
         rows = np.stack([np.minimum((((X - X[i]) ** 2).sum(axis=1, dtype=dtype) * w).astype(dtype), closest)
                          for i in expected])
         pots_ptr = lib.kmx_kpp_potentials_ptr(ptr(ws), n, d, k, tn, dc)
