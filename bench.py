@@ -149,27 +149,51 @@ def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
     # REGIONS timed regions of `steps` iterations each, one after the other in the same fit; the
     # median region is the one reported
     regions = []
+    region_event_ms = []
     for _ in range(REGIONS):
+        # (HIP events on the launch stream - torch's current stream is the one the library is
+        # given - around the whole region: two event records per region, not per launch)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
+        ev0.record()
         for _ in range(steps):
             enqueue()
+        ev1.record()
         torch.cuda.synchronize()
         regions.append(time.perf_counter() - t0)
+        region_event_ms.append(ev0.elapsed_time(ev1))
     elapsed = float(np.median(regions))
+    launch_period_ms = float(np.median(region_event_ms)) / steps
 
-    # per-kernel durations from HIP events on the launch stream; three untimed iterations are
-    # enqueued before every timed one, so that the clocks do not sag in the gaps the
-    # synchronising timed call leaves
+    # per-kernel durations from HIP events on the launch stream: a stream of back-to-back
+    # iterations, every one with events around its kernels (kmx_lloyd_iter_traced enqueues and
+    # does not wait), read after the last one.  Iterations that each wait for the host, as
+    # kmx_lloyd_iter_timed does, leave the GPU idle in between, and on some machines the kernels
+    # that follow such a gap run for 20 us longer than in a fit.
+    def enqueue_traced():
+        nonlocal it, done
+        if it >= RESTART:
+            restart()
+        a, b = it % 2, (it + 1) % 2
+        _capi.check(lib.kmx_lloyd_iter_traced(plan, ptr(X_t), None, ptr(w_d), ptr(cent[a]), ptr(cent[b]),
+                                              ptr(labels[a]), ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws),
+                                              ws_bytes, stream), "iter_traced")
+        it += 1
+        done += 1
+
     ms = (ctypes.c_float * 3)()
-    acc = np.zeros(3)
-    timed = 25
+    ms_min = (ctypes.c_float * 3)()
+    n_traced = ctypes.c_int32(0)
+    for _ in range(10):
+        enqueue()
+    timed = 100
     for _ in range(timed):
-        for _ in range(3):
-            enqueue()
-        enqueue(ms)
-        acc += np.array(list(ms))
-    kernel_ms = acc / timed
+        enqueue_traced()
+    _capi.check(lib.kmx_lloyd_trace_collect(ms, ms_min, ctypes.byref(n_traced)), "trace_collect")
+    if n_traced.value != timed:
+        raise RuntimeError(f"{n_traced.value} traced launches, expected {timed}")
+    kernel_ms = np.array(list(ms), dtype=np.float64)
     _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
     if status.n_iter != it or checked + it != done:
         raise RuntimeError(f"only {status.n_iter} of {it} iterations did work (state {status.state})")
@@ -178,7 +202,7 @@ def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
     rechecked = ctypes.c_uint32(0)
     _capi.check(lib.kmx_lloyd_recheck_count(plan, ptr(ws), ctypes.byref(rechecked), stream), "recheck_count")
     if not gates:
-        return elapsed, kernel_ms, 0, plan.variant, int(rechecked.value), ramp_iters, regions
+        return elapsed, kernel_ms, 0, plan.variant, int(rechecked.value), ramp_iters, regions, launch_period_ms
 
     # parity gate 1: the labels the last Lloyd iteration wrote, against exact fp64 distances to
     # the centroids it started from, on a slice
@@ -193,7 +217,7 @@ def gpu_lloyd(cfg, steps, warmup, flags=0, gates=True):
     _capi.check(lib.kmx_assign_labels(ptr(X_t), ptr(X_t.new_tensor(cur.T.copy())), ptr(lab), ptr(aws_t), aws,
                                       n, d, k, dc, flags, stream), "assign")
     ties = ties_iter + check_labels(lab[:m].cpu().numpy(), X[:m], cur)
-    return elapsed, kernel_ms, ties, plan.variant, int(rechecked.value), ramp_iters, regions
+    return elapsed, kernel_ms, ties, plan.variant, int(rechecked.value), ramp_iters, regions, launch_period_ms
 
 
 def gpu_measured_peaks():
@@ -658,10 +682,16 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    elapsed, kernel_ms, ties, variant, rechecked, ramp_iters, regions = gpu_lloyd(cfg, args.steps, args.warmup)
+    elapsed, kernel_ms, ties, variant, rechecked, ramp_iters, regions, period_ms = gpu_lloyd(cfg, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     iters_per_s = args.steps / elapsed
-    fused_s = kernel_ms[0] * 1e-3
+    # Variant 61 is ONE kernel per iteration (its last workgroup finishes the iteration), so the
+    # launch period of the back-to-back launches of a timed region - two HIP events around the
+    # region on the launch stream, divided by the launches - is that kernel's duration plus the
+    # gap to the next launch.  Event pairs around every single launch (kernel_ms) add the cost of
+    # their own records to what they bracket, several microseconds per record on these machines.
+    one_kernel = int(variant) == 61 and kernel_ms[1] + kernel_ms[2] < 0.5 * kernel_ms[0]
+    fused_s = (period_ms if one_kernel else kernel_ms[0]) * 1e-3
     flops = lloyd_flops(n, d, k)
     nbytes = lloyd_bytes(n, d, 4)
     log(f"[bench] {ms_per_step:.4f} ms/iter; kernels (ms): fused {kernel_ms[0]:.4f} reduce "
@@ -699,6 +729,10 @@ def main():
         "traffic_source": traffic_source,
         "kernel": "fused Lloyd step",
         "bytes_per_launch": nbytes,
+        "launch_duration_ms": fused_s * 1e3,
+        "launch_duration_from": ("HIP events around each timed region of back-to-back launches (one kernel per "
+                                 "iteration) / launches: kernel plus the gap to the next launch"
+                                 if one_kernel else "HIP events around every launch of the kernel"),
     }
     # Variant 61 screens the labels on the fp16 matrix cores: the fp32 contraction that bounded
     # variant 31 is gone, and what is left to approach is the HBM time of the algorithmic bytes.
@@ -717,7 +751,7 @@ def main():
         }
 
     # the same fit with every product taken in fp32 (variant 31), timed the same way
-    e32, kms32, _, variant32, _, _, _ = gpu_lloyd(cfg, args.steps, args.warmup, flags=FLAG_LABELS_F32, gates=False)
+    e32, kms32, _, variant32, _, _, _, _ = gpu_lloyd(cfg, args.steps, args.warmup, flags=FLAG_LABELS_F32, gates=False)
     all_fp32 = {
         "switch": "KMX_FLAG_LABELS_F32", "kernel_variant": int(variant32),
         "ms_per_step": e32 / args.steps * 1e3, "iters_per_sec": args.steps / e32,
@@ -759,7 +793,10 @@ def main():
                    "sums": "fp32 inputs, 64-bit fixed point"},
         "samples_clusters_per_sec": iters_per_s * n * k,
         "kernel_ms": {"fused_step": float(kernel_ms[0]), "reduce": float(kernel_ms[1]),
-                      "finalize": float(kernel_ms[2])},
+                      "finalize": float(kernel_ms[2]),
+                      "what": "HIP event pairs around every kernel of 100 back-to-back traced iterations "
+                              "(kmx_lloyd_iter_traced); each interval includes the cost of an event record"},
+        "launch_period_ms": period_ms,
         "roofline": roofline,
         "roofline_other_bound": roofline_other,
         "all_fp32": all_fp32,

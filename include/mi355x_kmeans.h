@@ -179,6 +179,21 @@ int32_t kmx_lloyd_iter_timed(const kmx_lloyd_plan* plan, const void* X_t, const 
                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
                              size_t workspace_bytes, void* stream, float* kernel_ms_host);
 
+/* kmx_lloyd_iter with the same events, without waiting: the launch is enqueued like any other and
+ * its four events are kept by the library (up to 1 024 launches: KMX_ERR_UNSUPPORTED beyond), so
+ * that a benchmark can time every launch of a stream of back-to-back iterations instead of
+ * iterations that each wait for the host.  kmx_lloyd_trace_collect waits for the launches
+ * enqueued so far, writes the mean (and, if kernel_ms_min is not NULL, the minimum) duration in
+ * milliseconds of each of the three kernel groups over them, their number, and forgets them.
+ * Not for concurrent fits: the list is one per process.  No counterpart in the reference
+ * (benchmark/kmeans.py:163-165 times whole fits). */
+int32_t kmx_lloyd_iter_traced(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
+                              const void* sample_weight, const void* centroids_t,
+                              void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                              size_t workspace_bytes, void* stream);
+int32_t kmx_lloyd_trace_collect(float* kernel_ms_mean, float* kernel_ms_min, int32_t* n_launches);
+
 /* Second half of (2) alone, for the iteration that stopped with KMX_NEED_RELOCATION after
  * the host has relocated the empty clusters: sums / sizes, shift, convergence test, state
  * back to KMX_RUNNING (or a terminal state).  kmeans/drivers.py:275,326-343. */

@@ -110,6 +110,8 @@ SIGNATURES = {
     "kmx_lloyd_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _U32]),
     "kmx_lloyd_init": (_I32, [_PLAN, _P, _SZ, _P, _P, _P, _I32, c_double, _P]),
     "kmx_lloyd_iter": (_I32, [_PLAN, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "kmx_lloyd_iter_traced": (_I32, [_PLAN, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "kmx_lloyd_trace_collect": (_I32, [_P, _P, _P]),
     "kmx_lloyd_iter_timed": (_I32, [_PLAN, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P,
                                     POINTER(ctypes.c_float)]),
     "kmx_lloyd_finalize": (_I32, [_PLAN, _P, _P, _P, _P, _SZ, _P]),

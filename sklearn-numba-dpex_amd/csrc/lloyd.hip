@@ -13,6 +13,9 @@
 // float atomics.  The MFMA variant for fp32 lives in lloyd_mfma.hip.
 #include "kmx_common.h"
 #include "lloyd_layout.h"
+
+#include <mutex>
+#include <vector>
 #include "lloyd_tail.h"
 
 namespace {
@@ -1056,6 +1059,69 @@ int32_t kmx_lloyd_iter_timed(const kmx_lloyd_plan* plan, const void* X_t, const 
         if (e != hipSuccess) rc = (int32_t)e;
     }
     for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
+    return rc;
+}
+
+// Events of the launches that kmx_lloyd_iter_traced has enqueued and kmx_lloyd_trace_collect has
+// not yet read: four per launch.
+static std::mutex trace_mutex;
+static std::vector<hipEvent_t> trace_events;
+constexpr size_t KMX_TRACE_MAX_LAUNCHES = 1024;
+
+int32_t kmx_lloyd_iter_traced(const kmx_lloyd_plan* plan, const void* X_t, const void* X_rowmajor,
+                              const void* sample_weight, const void* centroids_t,
+                              void* new_centroids_t, const uint32_t* labels_prev, uint32_t* labels,
+                              void* cluster_sizes, uint32_t* empty_clusters, void* workspace,
+                              size_t workspace_bytes, void* stream_) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PLAN(plan);
+    std::lock_guard<std::mutex> guard(trace_mutex);
+    if (trace_events.size() >= 4 * KMX_TRACE_MAX_LAUNCHES) return KMX_ERR_UNSUPPORTED;
+    hipEvent_t ev[4];
+    for (int i = 0; i < 4; ++i) {
+        const hipError_t e = hipEventCreate(&ev[i]);
+        if (e != hipSuccess) {
+            for (int j = 0; j < i; ++j) (void)hipEventDestroy(ev[j]);
+            return (int32_t)e;
+        }
+    }
+    const int32_t rc = lloyd_iter_dispatch(plan, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t,
+                                           labels_prev, labels, cluster_sizes, empty_clusters, workspace,
+                                           workspace_bytes, stream_, ev);
+    if (rc != KMX_OK) {
+        for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
+        return rc;
+    }
+    trace_events.insert(trace_events.end(), ev, ev + 4);
+    return KMX_OK;
+}
+
+int32_t kmx_lloyd_trace_collect(float* kernel_ms_mean, float* kernel_ms_min, int32_t* n_launches) {
+    KMX_ENTRY();
+    KMX_REQUIRE_PTR(kernel_ms_mean);
+    KMX_REQUIRE_PTR(n_launches);
+    std::lock_guard<std::mutex> guard(trace_mutex);
+    const size_t launches = trace_events.size() / 4;
+    *n_launches = (int32_t)launches;
+    double sum[3] = {0.0, 0.0, 0.0};
+    float low[3] = {0.0f, 0.0f, 0.0f};
+    int32_t rc = KMX_OK;
+    for (size_t l = 0; l < launches && rc == KMX_OK; ++l) {
+        hipError_t e = hipEventSynchronize(trace_events[4 * l + 3]);
+        for (int i = 0; i < 3 && e == hipSuccess; ++i) {
+            float ms = 0.0f;
+            e = hipEventElapsedTime(&ms, trace_events[4 * l + i], trace_events[4 * l + i + 1]);
+            sum[i] += ms;
+            if (l == 0 || ms < low[i]) low[i] = ms;
+        }
+        if (e != hipSuccess) rc = (int32_t)e;
+    }
+    for (hipEvent_t ev : trace_events) (void)hipEventDestroy(ev);
+    trace_events.clear();
+    for (int i = 0; i < 3; ++i) {
+        kernel_ms_mean[i] = launches ? (float)(sum[i] / (double)launches) : 0.0f;
+        if (kernel_ms_min) kernel_ms_min[i] = low[i];
+    }
     return rc;
 }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "kmx_common.h"
+#include "lloyd_tail.h"
 
 constexpr int KMX_VARIANT_STREAM = 0;    // wide samples: features re-read per centroid window
 constexpr int KMX_VARIANT_REGISTER = 1;  // samples held in registers, centroids in SGPRs
@@ -258,6 +259,11 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
 int32_t kmx_assign_labels_mfma_f32(const LloydLayout& L, const void* X_t, const void* centroids_t,
                                    uint32_t* labels, char* ws, int64_t n, int d, int k,
                                    hipStream_t stream);
+// Whether the screened fused step finishes the iteration itself (its last workgroup) instead of
+// a finalisation launch; 0 restores the separate launch for comparison.
+#ifndef KMX_SCR_FUSE_TAIL
+#define KMX_SCR_FUSE_TAIL 1
+#endif
 // screened fused step (lloyd_mfma_screen.hip); `uncertain_count`: one word for the number of
 // samples evaluated in fp32
 int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
@@ -265,7 +271,7 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    kmx_lloyd_status* status, const unsigned int* absmax,
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, const float* norms, int64_t n, int d,
-                                   int k, int wgs_per_cu, hipStream_t stream);
+                                   int k, int wgs_per_cu, hipStream_t stream, const LloydTail<float>* tail);
 // labels only, screened the same way (scale from the centroids, norms taken per tile)
 int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);

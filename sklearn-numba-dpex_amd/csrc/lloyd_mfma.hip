@@ -617,11 +617,17 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
         const int32_t rc = kmx_lloyd_step_mfma_screen(
             X_t, w, centroids_t, labels_prev, labels, tail.status,
             reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain,
-            reinterpret_cast<const float*>(ws + L.off_bucket + 256), n, d, k, L.wgs_per_cu, stream);
+            reinterpret_cast<const float*>(ws + L.off_bucket + 256), n, d, k, L.wgs_per_cu, stream,
+            KMX_SCR_FUSE_TAIL ? &tail : nullptr);
         if (rc != KMX_OK) return rc;
         if (events) {
             (void)hipEventRecord(events[1], stream);
             (void)hipEventRecord(events[2], stream);
+        }
+        if (KMX_SCR_FUSE_TAIL) {
+            // (the step's last workgroup has finished the iteration)
+            if (events) (void)hipEventRecord(events[3], stream);
+            return KMX_OK;
         }
     } else {
         const int32_t rc = launch_mfma<true>(L, X_t, w, centroids_t, labels_prev, labels,

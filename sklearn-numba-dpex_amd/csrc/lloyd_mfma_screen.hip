@@ -254,7 +254,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     const unsigned int* __restrict__ absmax, const int* __restrict__ q_exp,
     unsigned long long* __restrict__ gsum, uint32_t* __restrict__ uncertain_count,
     const float* __restrict__ norms, int64_t n, int d, int k, int vec_ok,
-    double* __restrict__ inertia_partial = nullptr) {
+    double* __restrict__ inertia_partial, const LloydTail<float> tail, const int fuse_tail) {
     static_assert(!(UPDATE && INERTIA), "the inertia rides with the labels-only kernel");
     // (labels only: `status` is null outside the iteration loop)
     if ((UPDATE || status != nullptr) && status->state != KMX_RUNNING) return;
@@ -1294,6 +1294,25 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const unsigned long long v = acc[c * acc_stride + (f < d ? f : d_even)];
             if (v) atomicAdd(gsum + jx, v);
         }
+        // The workgroup that gets done last finishes the iteration (empty-cluster list, division,
+        // shift, convergence test, what the next step needs) instead of a launch of its own, which
+        // would cost its launch, its first round trips to memory and the gap between two dependent
+        // launches.  What the workgroups hand over - sums, changed-label count, the counter of
+        // samples evaluated in fp32 - went through device-scope atomics, performed at the memory
+        // side; each workgroup waits for its own before it draws its ticket, and the last one
+        // reads them with device-scope loads.  No device-wide fence.
+        if (fuse_tail) {
+            __shared__ unsigned int is_last;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (threadIdx.x == 0) is_last = (atomicAdd(&status->ticket, 1u) == gridDim.x - 1) ? 1u : 0u;
+            __syncthreads();
+            if (is_last != 0u) {
+                // (the accumulators are flushed: their LDS holds the (d + 1) k sums as floats)
+                lloyd_small_finalize_body<float, true, true>(gsum, q_exp, tail, reinterpret_cast<float*>(smem_raw));
+                if (threadIdx.x == 0) status->ticket = 0u;
+            }
+        }
     }
 }
 
@@ -1498,7 +1517,8 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
                       uint32_t* labels, kmx_lloyd_status* status, const unsigned int* absmax,
                       const int* q_exp, unsigned long long* gsum, uint32_t* uncertain_count,
                       const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream,
-                      double* inertia_partial = nullptr, int* grid_out = nullptr) {
+                      double* inertia_partial = nullptr, int* grid_out = nullptr,
+                      const LloydTail<float>* tail = nullptr) {
     if (!(UPDATE ? kmx_mfma_screen_fits(n, d, k) : kmx_mfma_screen_labels_fits(n, d, k))) return KMX_ERR_UNSUPPORTED;
     const int nk = screen_k_steps(d, k, UPDATE);
     const int waves = scr_waves(nk);
@@ -1527,7 +1547,8 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
         hipLaunchKernelGGL((lloyd_screen_kernel<NK_, UPDATE, HK_, INERTIA>), dim3((unsigned)grid),          \
                            dim3(64 * scr_waves(NK_)), lds, stream, (const float*)X_t, (const float*)w,      \
                            (const float*)centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,     \
-                           uncertain_count, norms, n, d, k, vec_ok, inertia_partial);                       \
+                           uncertain_count, norms, n, d, k, vec_ok, inertia_partial,                        \
+                           tail ? *tail : LloydTail<float>(), tail ? 1 : 0);                                \
     } while (0)
     if (nk == 1) {
         if (hk) KMX_SCR_LAUNCH(1, true); else KMX_SCR_LAUNCH(1, false);
@@ -1549,14 +1570,16 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
 // evaluated in fp32 to (zero on entry; the finalisation that follows moves it to the next word
 // and clears it).  `absmax`: bits of max|X_t row| per feature, as kmx_lloyd_mfma_prepare leaves
 // them; `norms`: ||x_i|| per sample (kmx_sample_norms).
+// `tail` (may be null): what the finalisation of the iteration needs; the workgroup of the step
+// that gets done last then runs it, and no finalisation launch must follow.
 int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* centroids_t,
                                    const uint32_t* labels_prev, uint32_t* labels,
                                    kmx_lloyd_status* status, const unsigned int* absmax,
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, const float* norms, int64_t n, int d,
-                                   int k, int wgs_per_cu, hipStream_t stream) {
+                                   int k, int wgs_per_cu, hipStream_t stream, const LloydTail<float>* tail) {
     return launch_screen<true>(X_t, w, centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,
-                               uncertain_count, norms, n, d, k, wgs_per_cu, stream);
+                               uncertain_count, norms, n, d, k, wgs_per_cu, stream, nullptr, nullptr, tail);
 }
 
 // Labels only, screened the same way: nothing but X and the centroids is needed (the scale comes

@@ -28,20 +28,21 @@ struct LloydTail {
     int list_divisor = 0;
 };
 
-// Empty-cluster list (ascending) and heaviest cluster; one workgroup of 256 threads.
-// Returns the number of empty clusters (same value in every thread).
+// Empty-cluster list (ascending) and heaviest cluster; one workgroup of up to 1024 threads, all
+// of which call it.  Returns the number of empty clusters (same value in every thread).
 template <typename T>
 __device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters, int k,
                                        int* heaviest_out) {
-    __shared__ int wave_counts[4];
-    __shared__ T hv_val[4];
-    __shared__ int hv_idx[4];
+    __shared__ int wave_counts[16];
+    __shared__ T hv_val[16];
+    __shared__ int hv_idx[16];
     __shared__ int result_s[2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_threads = (int)blockDim.x, n_waves = (n_threads + 63) >> 6;
     int base = 0;
     T my_max = -kmx_inf<T>();
     int my_arg = 0x7fffffff;
-    for (int c0 = 0; c0 < k; c0 += 256) {
+    for (int c0 = 0; c0 < k; c0 += n_threads) {
         const int c = c0 + threadIdx.x;
         T sz = T(1);
         if (c < k) {
@@ -60,7 +61,7 @@ __device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters,
         int offset = base;
         for (int w2 = 0; w2 < wave; ++w2) offset += wave_counts[w2];
         if (flag) empty_clusters[offset + prefix] = (uint32_t)c;
-        base += wave_counts[0] + wave_counts[1] + wave_counts[2] + wave_counts[3];
+        for (int w2 = 0; w2 < n_waves; ++w2) base += wave_counts[w2];
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -80,7 +81,7 @@ __device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters,
     if (threadIdx.x == 0) {
         T bv = hv_val[0];
         int bidx = hv_idx[0];
-        for (int w2 = 1; w2 < 4; ++w2) {
+        for (int w2 = 1; w2 < n_waves; ++w2) {
             if (hv_val[w2] > bv || (hv_val[w2] == bv && hv_idx[w2] < bidx)) {
                 bv = hv_val[w2];
                 bidx = hv_idx[w2];
@@ -95,9 +96,8 @@ __device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters,
 
 // End of an iteration, by one thread: iteration count, shift, and the next state (strict
 // convergence from the second iteration on, then the tolerance, then the iteration limit).
-__device__ inline void lloyd_update_status(kmx_lloyd_status* st, double total_shift) {
+__device__ inline void lloyd_update_status(kmx_lloyd_status* st, double total_shift, unsigned int changed) {
     const int n_iter = st->n_iter + 1;
-    const unsigned int changed = st->n_changed;
     st->n_iter = n_iter;
     st->shift_sum = total_shift;
     st->n_changed = 0;
@@ -158,55 +158,80 @@ __device__ inline void lloyd_finalize_block(const LloydTail<T>& a, int n_empty, 
         }
     }
     const double total = kmx_block_sum<double>(shift, scratch);
-    if (threadIdx.x == 0) lloyd_update_status(a.status, total);
+    if (threadIdx.x == 0) lloyd_update_status(a.status, total, a.status->n_changed);
 }
 
 
-// One workgroup finishes an iteration whose (d + 1) * k sums fit in LDS: empty-cluster list
-// and, if no cluster is empty, division by the sizes, packed copy and half norms for the next
-// iteration, centroid shift, convergence test.  The sums stay in LDS between the phases;
-// global memory is read once and written once per output, and no device-wide fence is needed
-// (the kernel boundary orders it after the producers).
+// One workgroup (every thread of it, up to 1024) finishes an iteration whose (d + 1) * k sums fit
+// in LDS: empty-cluster list and, if no cluster is empty, division by the sizes, packed copy and
+// half norms for the next iteration, centroid shift, convergence test.  The sums stay in LDS
+// (`vals`, (d + 1) * k elements) between the phases; global memory is read once and written once
+// per output.
 //   FROM_GSUM: the sums arrive as 64-bit fixed point (`gsum`, binary point q_exp[f]) and are
 //              converted, stored to sums_t / sizes and cleared here;
 //   otherwise: sums_t / sizes already hold the reduced sums.
 // With an empty cluster the raw sums and sizes stay in global memory for the relocation and
 // the state becomes KMX_NEED_RELOCATION.
-template <typename T, bool FROM_GSUM>
-__global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
-    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<T> a) {
-    extern __shared__ __align__(16) unsigned char fin_raw[];
-    __shared__ double scratch[4];
+//   COHERENT: called by the last workgroup of the launch whose workgroups produced the sums, the
+//             changed-label count and the counter word with device-scope atomics (and waited for
+//             them before they drew their ticket): those words are read with device-scope loads,
+//             which do not stop at a cache of the own chiplet that may hold an older copy.
+template <typename T, bool FROM_GSUM, bool COHERENT>
+__device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict__ gsum,
+                                                 const int* __restrict__ q_exp, const LloydTail<T>& a,
+                                                 T* __restrict__ vals) {
+    __shared__ double scratch[16];
+    const int n_threads = (int)blockDim.x;
     // The old centroids are asked for before anything else (up to eight values per thread: what
-    // (d + 1) k <= 2048 needs): the kernel is a chain of memory round trips, and this one then
-    // runs beside those of the state and of the sums.
+    // (d + 1) k <= 2048 needs with 256 threads): the routine is a chain of memory round trips, and
+    // this one then runs beside those of the state and of the sums ...
     constexpr int OLD_AHEAD = 8;
     const int dk_ahead = a.d * a.k;
-    const bool old_ahead = dk_ahead <= 256 * OLD_AHEAD;
+    const bool old_ahead = dk_ahead <= n_threads * OLD_AHEAD;
     T old_v[OLD_AHEAD];
 #pragma unroll
     for (int i = 0; i < OLD_AHEAD; ++i) {
-        const int jx = (int)threadIdx.x + 256 * i;
+        const int jx = (int)threadIdx.x + n_threads * i;
         old_v[i] = (old_ahead && jx < dk_ahead) ? a.old_centroids_t[jx] : T(0);
-    }
-    if (a.status->state != KMX_RUNNING) return;
-    if (a.clear_word != nullptr && threadIdx.x == 0) {
-        a.clear_word[1] = a.clear_word[0];  // kept for kmx_lloyd_recheck_count
-        a.clear_word[0] = 0u;
     }
     const int d = a.d, k = a.k, dpad = a.dpad;
     const int items = (d + 1) * k, dk = d * k;
-    T* vals = reinterpret_cast<T*>(fin_raw);  // [(d + 1) * k]: sums, then sizes
-    const T* sizes_s = vals + dk;
+    // ... and so are the sums themselves (up to eight per thread), the changed-label count and
+    // the counter word: one round trip for all of them instead of one after the other
+    auto load_sum = [&](const int jx) __attribute__((always_inline)) {
+        return (long long)(COHERENT ? __hip_atomic_load(&gsum[jx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                    : gsum[jx]);
+    };
+    constexpr int SUMS_AHEAD = 8;
+    const bool sums_ahead = FROM_GSUM && items <= n_threads * SUMS_AHEAD;
+    long long sum_v[SUMS_AHEAD];
+    if constexpr (FROM_GSUM) {
+#pragma unroll
+        for (int i = 0; i < SUMS_AHEAD; ++i) {
+            const int jx = (int)threadIdx.x + n_threads * i;
+            sum_v[i] = (sums_ahead && jx < items) ? load_sum(jx) : 0ll;
+        }
+    }
+    unsigned int counter_word = 0u;
+    if (a.clear_word != nullptr && threadIdx.x == 0)
+        counter_word = COHERENT ? __hip_atomic_load(&a.clear_word[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                : a.clear_word[0];
+    const unsigned int n_changed =
+        COHERENT ? __hip_atomic_load(&a.status->n_changed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                 : a.status->n_changed;
+    if (a.clear_word != nullptr && threadIdx.x == 0) {
+        a.clear_word[1] = counter_word;  // kept for kmx_lloyd_recheck_count
+        a.clear_word[0] = 0u;
+    }
+    const T* sizes_s = vals + dk;  // vals: [(d + 1) * k], sums, then sizes
     T* __restrict__ out_t = a.sums_t;
     const T* __restrict__ old_t = a.old_centroids_t;
     // (the label changes of the iteration at hand; every thread reads the same word before
     // thread 0 resets it at the end of the kernel)
     const bool keep_sums = FROM_GSUM && a.clear_word != nullptr && a.delta_divisor > 0 &&
-                           (int64_t)a.status->n_changed * a.delta_divisor <= a.n_samples;
-    for (int jx = threadIdx.x; jx < items; jx += 256) {
-        if constexpr (FROM_GSUM) {
-            const long long iv = (long long)gsum[jx];
+                           (int64_t)n_changed * a.delta_divisor <= a.n_samples;
+    if constexpr (FROM_GSUM) {
+        auto convert = [&](const int jx, const long long iv) __attribute__((always_inline)) {
             if (!keep_sums) gsum[jx] = 0ull;
             const int f = jx / k;
             // (times 2^-q, built from its exponent field: exact, like ldexp)
@@ -216,9 +241,18 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
                 out_t[jx] = val;
             else
                 a.sizes[jx - dk] = val;
+        };
+        if (sums_ahead) {
+#pragma unroll
+            for (int i = 0; i < SUMS_AHEAD; ++i) {
+                const int jx = (int)threadIdx.x + n_threads * i;
+                if (jx < items) convert(jx, sum_v[i]);
+            }
         } else {
-            vals[jx] = jx < dk ? out_t[jx] : a.sizes[jx - dk];
+            for (int jx = threadIdx.x; jx < items; jx += n_threads) convert(jx, load_sum(jx));
         }
+    } else {
+        for (int jx = threadIdx.x; jx < items; jx += n_threads) vals[jx] = jx < dk ? out_t[jx] : a.sizes[jx - dk];
     }
     __syncthreads();
     int heaviest = 0;
@@ -231,7 +265,7 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
         // the host relocates and finishes the iteration; the next step rebuilds the sums
         if constexpr (FROM_GSUM) {
             if (keep_sums)
-                for (int jx = threadIdx.x; jx < items; jx += 256) gsum[jx] = 0ull;
+                for (int jx = threadIdx.x; jx < items; jx += n_threads) gsum[jx] = 0ull;
         }
         if (threadIdx.x == 0) {
             a.status->state = KMX_NEED_RELOCATION;
@@ -241,8 +275,8 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
     }
     if (a.clear_word != nullptr && threadIdx.x == 0)
         a.clear_word[2] = !keep_sums ? 0u
-                          : (a.list_divisor > 0 && (int64_t)a.status->n_changed * a.list_divisor <= a.n_samples) ? 1u
-                                                                                                              : 2u;
+                          : (a.list_divisor > 0 && (int64_t)n_changed * a.list_divisor <= a.n_samples) ? 1u
+                                                                                                    : 2u;
     double shift = 0.0;
     auto divide = [&](const int jx, const T old_value) __attribute__((always_inline)) {
         const int f = jx / k, c = jx - f * k;
@@ -256,20 +290,29 @@ __global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
     if (old_ahead) {  // (the same elements in the same order as the loop below)
 #pragma unroll
         for (int i = 0; i < OLD_AHEAD; ++i) {
-            const int jx = (int)threadIdx.x + 256 * i;
+            const int jx = (int)threadIdx.x + n_threads * i;
             if (jx < dk) divide(jx, old_v[i]);
         }
     } else {
 #pragma unroll 4
-        for (int jx = threadIdx.x; jx < dk; jx += 256) divide(jx, old_t[jx]);
+        for (int jx = threadIdx.x; jx < dk; jx += n_threads) divide(jx, old_t[jx]);
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < k; c += 256) {
+    for (int c = threadIdx.x; c < k; c += n_threads) {
         T sq = T(0);
         for (int f = 0; f < d; ++f) sq += vals[f * k + c] * vals[f * k + c];
         a.half_norms[c] = sq / T(2);
         for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = T(0);
     }
     const double total = kmx_block_sum<double>(shift, scratch);
-    if (threadIdx.x == 0) lloyd_update_status(a.status, total);
+    if (threadIdx.x == 0) lloyd_update_status(a.status, total, n_changed);
+}
+
+// The same as a launch of its own: ordered after the producers of the sums by the kernel boundary.
+template <typename T, bool FROM_GSUM>
+__global__ __launch_bounds__(256) void lloyd_small_finalize_kernel(
+    unsigned long long* __restrict__ gsum, const int* __restrict__ q_exp, LloydTail<T> a) {
+    extern __shared__ __align__(16) unsigned char fin_raw[];
+    if (a.status->state != KMX_RUNNING) return;
+    lloyd_small_finalize_body<T, FROM_GSUM, false>(gsum, q_exp, a, reinterpret_cast<T*>(fin_raw));
 }
