@@ -4,6 +4,7 @@
 // block order), so results do not change from run to run.
 #include "kmx_common.h"
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -64,6 +65,74 @@ __global__ __launch_bounds__(256) void sum_rows_stage2(const double* __restrict_
     __shared__ double scratch[4];
     const double tot = kmx_block_sum<double>(acc, scratch);
     if (threadIdx.x == 0) out[row] = (T)tot;
+}
+
+// Row sums in ONE launch (up to SUM_TICKET_ROWS rows): stage 1 as above, then the workgroup of a
+// row that gets done last adds the row's partial sums in the order of stage 2 - the same value,
+// bit for bit, without the second launch and the gap before it.  The partial sums are handed
+// over through device-scope stores, each workgroup waits for its own before it draws its ticket,
+// and the last one reads them with device-scope loads (no device-wide fence).
+// The tickets live in a device array of the library, zero when the library is loaded and left
+// zero by every launch; concurrent launches take different slots of it (handed out in turn).
+constexpr int SUM_TICKET_SLOTS = 256;
+constexpr int SUM_TICKET_ROWS = 64;
+__device__ unsigned int sum_tickets[SUM_TICKET_SLOTS][SUM_TICKET_ROWS];
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void sum_rows_fused(const T* __restrict__ in, double* __restrict__ partial,
+                                                      T* __restrict__ out, int64_t cols, int square, int slot) {
+    const int64_t row = blockIdx.y;
+    const T* __restrict__ p = in + (size_t)row * cols;
+    double acc = 0.0;
+    if constexpr (VEC) {
+        constexpr int W = 16 / sizeof(T);
+        using V = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
+        const V* __restrict__ pv = reinterpret_cast<const V*>(p);
+        const int64_t groups = cols / W;
+        const int64_t stride = (int64_t)gridDim.x * 256;
+        int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        auto add = [&](const V& v) {
+            const T* e = reinterpret_cast<const T*>(&v);
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                const double x = (double)e[j];
+                acc += square ? x * x : x;
+            }
+        };
+        for (; g + stride < groups; g += 2 * stride) {
+            const V a = pv[g];
+            const V b = pv[g + stride];
+            add(a);
+            add(b);
+        }
+        if (g < groups) add(pv[g]);
+    } else {
+        const int64_t stride = (int64_t)gridDim.x * 256;
+        for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += stride) {
+            const double v = (double)p[c];
+            acc += square ? v * v : v;
+        }
+    }
+    __shared__ double scratch[4];
+    __shared__ unsigned int is_last;
+    const int n_partials = (int)gridDim.x;
+    const double tot = kmx_block_sum<double>(acc, scratch);
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&partial[(size_t)row * n_partials + blockIdx.x], tot, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned int* ticket = &sum_tickets[slot][row];
+        const unsigned int arrived = atomicAdd(ticket, 1u);
+        is_last = arrived == (unsigned int)n_partials - 1u ? 1u : 0u;
+        if (is_last) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (is_last == 0u) return;
+    double acc2 = 0.0;
+    for (int j = threadIdx.x; j < n_partials; j += 256)
+        acc2 += __hip_atomic_load(&partial[(size_t)row * n_partials + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const double tot2 = kmx_block_sum<double>(acc2, scratch);
+    if (threadIdx.x == 0) out[row] = (T)tot2;
 }
 
 template <typename T>
@@ -320,12 +389,24 @@ int32_t kmx_sum_rows(const void* in, void* out, int64_t rows, int64_t cols, int3
     double* partial = (double*)workspace;
     const size_t es = kmx_dtype_size(dtype);
     const bool vec = (((uintptr_t)in) % 16 == 0) && ((cols * es) % 16 == 0);
+    // Few workgroups (one round of them on the chip): one launch, the last workgroup of a row
+    // finishes it (same sums, same order).  The hand-over costs every workgroup two round trips
+    // to memory at its end, which a launch of many short workgroups pays for more dearly than
+    // for the second launch: 14 rows of 5e6 values took 69 us that way against 45 us.
+    static std::atomic<unsigned int> next_slot{0};
+    const bool fused = rows <= SUM_TICKET_ROWS && rows * (int64_t)b <= 2 * (int64_t)kmx_num_cus();
+    const int slot = fused ? (int)(next_slot.fetch_add(1u) % (unsigned int)SUM_TICKET_SLOTS) : 0;
 #define KMX_SUM_ROWS(T, VEC)                                                                       \
     do {                                                                                           \
-        hipLaunchKernelGGL((sum_rows_stage1<T, VEC>), dim3(b, (unsigned)rows), dim3(256), 0, stream, \
-                           (const T*)in, partial, cols, square);                                   \
-        hipLaunchKernelGGL((sum_rows_stage2<T>), dim3((unsigned)rows), dim3(256), 0, stream,        \
-                           partial, (T*)out, b);                                                   \
+        if (fused) {                                                                               \
+            hipLaunchKernelGGL((sum_rows_fused<T, VEC>), dim3(b, (unsigned)rows), dim3(256), 0, stream, \
+                               (const T*)in, partial, (T*)out, cols, square, slot);                \
+        } else {                                                                                   \
+            hipLaunchKernelGGL((sum_rows_stage1<T, VEC>), dim3(b, (unsigned)rows), dim3(256), 0, stream, \
+                               (const T*)in, partial, cols, square);                               \
+            hipLaunchKernelGGL((sum_rows_stage2<T>), dim3((unsigned)rows), dim3(256), 0, stream,    \
+                               partial, (T*)out, b);                                               \
+        }                                                                                          \
     } while (0)
     if (dtype == KMX_F32) {
         if (vec) KMX_SUM_ROWS(float, true); else KMX_SUM_ROWS(float, false);
