@@ -173,7 +173,8 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     // (the wide path is built for many clusters: up to 256 the tiled product below is faster; and
     // up to 64 features the labels-only form of the screened kernel above, where its operands fit
     // the LDS, with sums per bucket of samples, is faster than either)
-    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) &&
+    // (its sample order, ranks and counts are 32-bit: kmx_lloyd_step_mfma_wide_f32 refuses more samples)
+    else if (dtype == KMX_F32 && kmx_mfma_wide_supported(d, k) && n <= INT32_MAX &&
              ((forced < 0 && k > 256 && !screen_labels_ok) || forced == KMX_VARIANT_MFMA)) {
         L.variant = KMX_VARIANT_MFMA_WIDE;
         L.acc_mode = KMX_ACC_GLOBAL;  // always the global fixed-point sums (variant code 42)

@@ -276,3 +276,35 @@ def test_missing_gpu_fails_loudly():
 
     with pytest.raises(RuntimeError, match="needs a ROCm GPU"):
         drivers.get_labels_inertia(torch.zeros(2, 3), torch.zeros(2, 2), torch.ones(3), False)
+
+
+def test_plans_for_arrays_past_32_bit_limits():
+    """Which kernel a plan chooses follows from what the kernel can address: the screened fused
+    step numbers tiles and samples with 32 bits (n < 2^29) and takes its fast path only while
+    d * n * 4 < 2^32 (decided per launch); the bucketed sums and the wide path keep 32-bit sample
+    orders (n <= INT32_MAX); past that only the fused vector-ALU kernels and the all-fp32 / fp64
+    matrix-core steps, whose index arithmetic is 64-bit throughout, are planned.  The other entry
+    points refuse what they cannot address."""
+    from sklearn_numba_dpex_amd._capi import lib
+
+    big = 1 << 31
+    assert lib.kmx_lloyd_kernel_variant((1 << 29) - 1, 14, 127, 0, 0) == 61
+    assert lib.kmx_lloyd_kernel_variant(1 << 29, 14, 127, 0, 0) == 31          # all-fp32 step, 64-bit tiles
+    assert lib.kmx_lloyd_kernel_variant(big, 14, 127, 0, 0) == 31
+    assert lib.kmx_lloyd_kernel_variant(1 << 29, 256, 512, 0, 0) == 42         # wide, screen off (n >= 2^29)
+    assert lib.kmx_lloyd_kernel_variant(big, 14, 1270, 0, 0) in (2, 12)        # no 32-bit sample order past 2^31
+    assert lib.kmx_lloyd_kernel_variant(big, 300, 3000, 0, 0) == 2
+    assert lib.kmx_lloyd_kernel_variant(big, 32, 64, 1, 0) == 51
+    assert lib.kmx_lloyd_kernel_variant(3_000_000_000, 8, 5000, 1, 0) == 12
+    # forcing the tiled product or the wide path on such an input does not produce a plan that uses them
+    assert lib.kmx_lloyd_kernel_variant(big, 300, 3000, 0, 0x4) == 2
+    assert lib.kmx_lloyd_kernel_variant(big, 14, 1270, 0, 0x3) in (2, 12)
+    # arrays past 2^31 ELEMENTS with fewer samples keep the fast kernels
+    assert lib.kmx_lloyd_kernel_variant(4_300_000, 512, 300, 0, 0) == 63
+    assert lib.kmx_lloyd_kernel_variant(8_500_000, 256, 512, 0, 0) == 42
+    assert lib.kmx_lloyd_kernel_variant(34_000_000, 64, 64, 0, 0) == 61
+    # kmeans++ and top-k address samples with 32 bits
+    assert lib.kmx_kpp_workspace_bytes(big, 8, 4, 3, 0) > 0
+    p = ctypes.c_void_p(4096)
+    assert lib.kmx_kpp_init(p, p, 0, p, p, p, 1 << 62, big, 8, 4, 3, 0, 0, None) == -2
+    assert lib.kmx_argmin(p, p, big, 0, None) == -2

@@ -233,3 +233,96 @@ def test_large_shapes_off_the_benchmark_configurations(cuda, shape):
     assert len(recs) == 3 and all(r["state"] == 0 for r in recs)
     inertias = [float(drivers._inertia(X_t, w_d, r["inp"], r["labels"])) for r in recs]
     assert all(b <= a * (1 + 1e-6) for a, b in zip(inertias, inertias[1:])), inertias
+
+
+@pytest.mark.parametrize("n,d,k,variant", [(4_300_000, 512, 300, 63), (8_500_000, 256, 512, 42)])
+def test_array_past_two_to_the_31_elements(cuda, n, d, k, variant):
+    """4 300 000 x 512 (tiled product + sums per bucket) and 8 500 000 x 256 with 512 clusters (the
+    wide path: labels screened in fp16, fp32 pass over the uncertified samples, bucketed
+    accumulation) in fp32: 2.2e9 elements, 8.8 GB, generated on the device.  Feature rows from
+    125 on start more than 2^31 bytes into the array and the last samples of the last row lie
+    past element 2^31: three Lloyd iterations through the C ABI (tiled matrix-core labels, sums
+    per bucket of samples from the row-major copy), checked through size-independent properties
+    - conservation of the weighted sums, labels against exact fp64 distances on slices at the
+    start, in the middle and at the very end, inertia that does not rise - then labels + inertia
+    as the end of a fit takes them."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    assert n * d > 2**31
+    g = torch.Generator(device=cuda)
+    g.manual_seed(5)
+    centers = torch.randn(k, d, device=cuda, generator=g) * 2.0
+    X_t = torch.empty((d, n), dtype=torch.float32, device=cuda)
+    chunk = 100_000
+    for lo in range(0, n, chunk):
+        hi = min(lo + chunk, n)
+        y = torch.randint(0, k, (hi - lo,), device=cuda, generator=g)
+        X_t[:, lo:hi] = (centers[y] + torch.randn(hi - lo, d, device=cuda, generator=g)).T
+    w = torch.rand(n, device=cuda, generator=g) + 0.5
+    # (one initial centroid near every blob: random rows leave some blobs without one, and a
+    # cluster then empties in the second iteration, which is the host's relocation path)
+    init = centers + 0.5 * torch.randn(k, d, device=cuda, generator=g)
+    cent = [init.T.contiguous(), torch.empty((d, k), dtype=torch.float32, device=cuda)]
+    dc = 0
+    plan = _capi.lloyd_plan(n, d, k, dc, 0)
+    assert plan.variant == variant and lib.kmx_lloyd_plan_reads_rowmajor(plan) == 1
+    X_rm = X_t.T.contiguous()
+    ws = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=cuda)
+    labels = [torch.zeros(n, dtype=torch.int32, device=cuda) for _ in range(2)]
+    sizes = torch.empty(k, dtype=torch.float32, device=cuda)
+    empty = torch.empty(k, dtype=torch.int32, device=cuda)
+    stream = _capi.current_stream()
+    status = _capi.LloydStatus()
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), plan.workspace_bytes, ptr(X_t), ptr(w), ptr(cent[0]), 10, 0.0, stream), "init")
+
+    slices = [slice(0, 3000), slice(n // 2 + 1, n // 2 + 3001), slice(n - 3000, n)]
+
+    def exact_labels(c_t, sl):
+        Xs = X_t[:, sl].double()
+        dist = (Xs * Xs).sum(0)[:, None] - 2.0 * Xs.T @ c_t.double() + (c_t.double() ** 2).sum(0)[None, :]
+        return dist
+
+    w64_total = float(w.double().sum())
+    wx = torch.stack([(X_t[f].double() * w.double()).sum() for f in range(0, d, 37)])   # every 37th feature
+    inertias = []
+    for it in range(3):
+        a, b = it % 2, (it + 1) % 2
+        print(f"large array: iteration {it}", flush=True)
+        _capi.check(lib.kmx_lloyd_iter(plan, ptr(X_t), ptr(X_rm), ptr(w), ptr(cent[a]), ptr(cent[b]), ptr(labels[a]),
+                                       ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws), plan.workspace_bytes, stream),
+                    "iter")
+        _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+        assert status.n_empty == 0 and status.n_iter == it + 1, (status.n_empty, status.n_iter, status.state)
+        for sl in slices:
+            dist = exact_labels(cent[a], sl)
+            got = labels[b][sl].long()
+            best = dist.argmin(dim=1)
+            bad = torch.nonzero(got != best).flatten()
+            if bad.numel():
+                gap = dist[bad, got[bad]] - dist[bad, best[bad]]
+                assert bool(torch.all(gap <= 1e-6 * dist[bad].max(dim=1).values)), (sl, int(bad.numel()))
+        assert float(sizes.double().sum()) == pytest.approx(w64_total, rel=1e-5)
+        got_wx = (cent[b][::37].double() * sizes.double()[None, :]).sum(dim=1)
+        assert torch.allclose(got_wx, wx, rtol=1e-4, atol=1e-4 * float(wx.abs().max()))
+        inertias.append(float(drivers._inertia(X_t, w, cent[b], labels[b])))
+        last = b
+        if status.state != _capi.KMX_RUNNING:
+            # well separated blobs: the second iteration changes no label
+            assert status.state == _capi.KMX_CONVERGED_STRICT and it >= 1
+            break
+    assert all(later <= earlier * (1 + 1e-6) for earlier, later in zip(inertias, inertias[1:]))
+    # the end of a fit: labels for the final centroids and their inertia, in one library call
+    final = torch.empty(n, dtype=torch.int32, device=cuda)
+    inertia = drivers._assign_with_inertia(X_t, w, cent[last], final)[0]
+    for sl in slices:
+        dist = exact_labels(cent[last], sl)
+        got = final[sl].long()
+        bad = torch.nonzero(got != dist.argmin(dim=1)).flatten()
+        if bad.numel():
+            gap = dist[bad, got[bad]] - dist[bad].min(dim=1).values
+            assert bool(torch.all(gap <= 1e-6 * dist[bad].max(dim=1).values))
+    assert float(inertia) <= inertias[-1] * (1 + 1e-5)
