@@ -891,7 +891,9 @@ static int32_t plan_validate(const kmx_lloyd_plan* p) {
         if (rc_ != KMX_OK) return rc_;          \
     } while (0)
 
-static int32_t layout_variant_code(const LloydLayout& L) { return L.screen ? 61 : L.variant * 10 + L.acc_mode; }
+static int32_t layout_variant_code(const LloydLayout& L) {
+    return L.screen ? 61 : L.screen64 ? 71 : L.variant * 10 + L.acc_mode;
+}
 
 int32_t kmx_lloyd_plan_init(kmx_lloyd_plan* plan, int64_t n, int32_t d, int32_t k, int32_t dtype,
                             uint32_t flags) {
@@ -959,16 +961,17 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
                            (const double*)centroids_t, (double*)(ws + L.off_cpack),
                            (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
     KMX_LAUNCH_CHECK();
-    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen || L.direct_sums) {
+    if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen || L.direct_sums ||
+        L.screen64) {
         // (for the screened tiled product: max|x| per feature, from which its scale is taken)
-        const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, stream);
+        const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, dtype, stream);
         if (rc != KMX_OK) return rc;
     }
-    if (L.variant == KMX_VARIANT_MFMA_WIDE || L.screen) {
+    if (L.variant == KMX_VARIANT_MFMA_WIDE || L.screen || L.screen64) {
         // cluster counts of the wide path / the counter of uncertain samples of the screened one
         hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(4), dim3(256), 0, stream,
                            (uint32_t*)(ws + L.off_bucket),
-                           L.screen ? (size_t)64 : (size_t)k);
+                           (L.screen || L.screen64) ? (size_t)64 : (size_t)k);
         KMX_LAUNCH_CHECK();
     }
     if (L.variant == KMX_VARIANT_MFMA_WIDE) {
@@ -1020,6 +1023,10 @@ static int32_t lloyd_iter_dispatch(const kmx_lloyd_plan* plan, const void* X_t, 
                                       labels_prev, labels, cluster_sizes, empty_clusters,
                                       (char*)workspace, n, d, k, stream, events);
     }
+    if (L.screen64)
+        return kmx_lloyd_iter_mfma_screen_f64(L, X_t, sample_weight, centroids_t, new_centroids_t, labels_prev,
+                                              labels, cluster_sizes, empty_clusters, (char*)workspace, n, d, k,
+                                              stream, events);
     return lloyd_iter_impl<double>(L, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev,
                                    labels, cluster_sizes, empty_clusters, (char*)workspace, n, d, k,
                                    stream, events);
@@ -1179,7 +1186,7 @@ int32_t kmx_lloyd_recheck_count(const kmx_lloyd_plan* plan, const void* workspac
     const LloydLayout L = lloyd_layout(n, d, k, plan->dtype, plan->flags);
     *count_host = 0;
     const void* src = nullptr;
-    if (L.screen)
+    if (L.screen || L.screen64)
         src = (const char*)workspace + L.off_bucket + sizeof(uint32_t);
     else if (L.variant == KMX_VARIANT_MFMA_WIDE && kmx_wide_screen_enabled(n, d, k, L.flags))
         src = kmx_wide_screen_counter((const char*)workspace + L.off_wscreen);

@@ -88,6 +88,7 @@ int32_t kmx_lloyd_direct_sums(const void* X_t, const void* w, const uint32_t* la
 // break-even) select it
 bool kmx_mfma_screen_fits(int64_t n, int d, int k);
 bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags);
+bool kmx_mfma_screen_f64_supported(int64_t n, int d, int k, uint32_t flags);  // fp64 inputs
 // the same kernel without the sums (labels only): needs less LDS
 bool kmx_mfma_screen_labels_fits(int64_t n, int d, int k);
 int32_t kmx_lloyd_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
@@ -106,6 +107,7 @@ struct LloydLayout {
     int n_partials;      // slots in `partial` (workgroups for LDS mode, copies for global mode)
     int k_for_gsum;      // n_clusters (size of the fixed-point sum array is (d + 1) * k)
     bool screen;         // KMX_VARIANT_MFMA with fp16-screened labels (variant code 61)
+    bool screen64;       // fp64 inputs: the same screened fused step (variant code 71)
     bool gemm_screen;    // KMX_VARIANT_GEMM (fp32) with fp16-screened labels
     bool screen_labels;  // KMX_VARIANT_GEMM (fp32, d <= 64): labels by the screened kernel of variant 61 without its sums
     bool direct_sums;    // with screen_labels: sums straight from the labels (fixed point in LDS) instead of per bucket
@@ -212,6 +214,9 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
         if (L.acc_mode == KMX_ACC_BUCKET) L.n_partials = 1;
     }
     L.screen = L.variant == KMX_VARIANT_MFMA && kmx_mfma_screen_supported(n, d, k, flags);
+    // (where the fp64 matrix-core step would run with its accumulators in LDS)
+    L.screen64 = dtype == KMX_F64 && L.variant == KMX_VARIANT_MFMA_F64 && L.acc_mode == KMX_ACC_LDS &&
+                 kmx_mfma_screen_f64_supported(n, d, k, flags);
     L.gemm_screen = L.variant == KMX_VARIANT_GEMM && dtype == KMX_F32 && kmx_gemm_screen_enabled(n, d, k, flags);
     L.screen_labels = L.variant == KMX_VARIANT_GEMM && screen_labels_ok && !L.gemm_screen && forced != KMX_VARIANT_GEMM;
     L.direct_sums = L.screen_labels && kmx_direct_sums_fits(d, k);
@@ -230,7 +235,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     const size_t bucket_bytes =
         (L.variant == KMX_VARIANT_MFMA_WIDE || L.acc_mode == KMX_ACC_BUCKET)
             ? ((size_t)2 * k + 1 + 2 * (size_t)n) * sizeof(int)
-        : L.screen ? (size_t)256 + (size_t)n * sizeof(float)
+        : (L.screen || L.screen64) ? (size_t)256 + (size_t)n * sizeof(float)
                                            : 0;
     // wide matrix-core path: header, scaled half norms and fp16 parts of the centroids for the
     // screened label step (lloyd_mfma_wide_screen.hip)
@@ -242,7 +247,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
                                                                     : 0;
     L.off_partial = L.off_wscreen + kmx_align256(wscreen_bytes);
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
-    const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE;
+    const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.screen64;
     L.partial_bytes = fixed_point ? 0 : (size_t)L.n_partials * items * s;
     L.total = L.off_partial + kmx_align256(L.partial_bytes);
     return L;
@@ -251,7 +256,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
 // fp32 matrix-core implementations (lloyd_mfma.hip)
 // Fixed-point exponents from max|X_t row|, max|w| and n; clears the fixed-point sums.
 int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void* w, char* ws,
-                               int64_t n, int d, hipStream_t stream);
+                               int64_t n, int d, int dtype, hipStream_t stream);
 int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const void* w,
                                 const void* centroids_t, void* new_centroids_t,
                                 const uint32_t* labels_prev, uint32_t* labels, void* sizes,
@@ -273,6 +278,19 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    const int* q_exp, unsigned long long* gsum,
                                    uint32_t* uncertain_count, const float* norms, int64_t n, int d,
                                    int k, int wgs_per_cu, hipStream_t stream, const LloydTail<float>* tail);
+// the same on fp64 inputs: labels screened on the fp16 matrix cores from the inputs rounded to
+// fp32, uncertified samples and sums in fp64
+int32_t kmx_lloyd_step_mfma_screen_f64(const void* X_t, const void* w, const void* centroids_t,
+                                       const uint32_t* labels_prev, uint32_t* labels,
+                                       kmx_lloyd_status* status, const unsigned int* absmax,
+                                       const int* q_exp, unsigned long long* gsum,
+                                       uint32_t* uncertain_count, const float* norms, int64_t n, int d,
+                                       int k, int wgs_per_cu, hipStream_t stream, const LloydTail<double>* tail);
+int32_t kmx_lloyd_iter_mfma_screen_f64(const LloydLayout& L, const void* X_t, const void* w,
+                                       const void* centroids_t, void* new_centroids_t,
+                                       const uint32_t* labels_prev, uint32_t* labels, void* sizes,
+                                       uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
+                                       hipStream_t stream, hipEvent_t* events);
 // labels only, screened the same way (scale from the centroids, norms taken per tile)
 int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);
@@ -281,7 +299,7 @@ int32_t kmx_assign_labels_inertia_mfma_screen(const void* X_t, const void* w, co
                                               int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);
 // out[0] = sum of `count` fp64 partial sums, in order (inertia_distances.hip)
 int32_t kmx_inertia_total_launch(const double* partial, int count, void* out, int32_t dtype, hipStream_t stream);
-int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream);
+int32_t kmx_sample_norms(const void* X_t, float* norms, int64_t n, int d, int dtype, hipStream_t stream);
 int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float* scores,
                                float* bounds, float* half_norms, float* scale, unsigned int* scratch,
                                int64_t n, int d, int k, hipStream_t stream);

@@ -50,31 +50,37 @@ __global__ void absmax_zero_kernel(unsigned int* absmax, int count) {
 }
 
 // Row r < d: max |X_t[r, :]|; row d: max |w|.  Non-negative floats order like their bits.
-__global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ X_t,
-                                                          const float* __restrict__ w,
+// (fp64 inputs: the maximum of the values rounded to fp32, which is what the screened step works
+// with; its fixed-point exponents leave a factor of two of room above it)
+__device__ __forceinline__ float amax_vec(float a, const float4& v) {
+    return fmaxf(fmaxf(a, fabsf(v.x)), fmaxf(fabsf(v.y), fmaxf(fabsf(v.z), fabsf(v.w))));
+}
+__device__ __forceinline__ float amax_vec(float a, const double2& v) {
+    return fmaxf(a, fmaxf(fabsf((float)v.x), fabsf((float)v.y)));
+}
+template <typename T>
+__global__ __launch_bounds__(256) void absmax_rows_kernel(const T* __restrict__ X_t,
+                                                          const T* __restrict__ w,
                                                           unsigned int* __restrict__ absmax,
                                                           int64_t n, int d, int vec_ok) {
     const int row = blockIdx.y;
-    const float* __restrict__ p = row < d ? X_t + (size_t)row * n : w;
+    const T* __restrict__ p = row < d ? X_t + (size_t)row * n : w;
     float m = 0.0f;
     const int64_t stride = (int64_t)gridDim.x * 256;
     if (vec_ok) {
         // rows start 16-byte aligned and n is a multiple of 4: 128-bit loads
-        const float4* __restrict__ p4 = reinterpret_cast<const float4*>(p);
-        auto amax4 = [](float a, const float4& v) {
-            return fmaxf(fmaxf(a, fabsf(v.x)), fmaxf(fabsf(v.y), fmaxf(fabsf(v.z), fabsf(v.w))));
-        };
-        const int64_t n4 = n >> 2;
+        using V = std::conditional_t<sizeof(T) == 8, double2, float4>;
+        const V* __restrict__ p4 = reinterpret_cast<const V*>(p);
+        const int64_t n4 = n / (int64_t)(16 / sizeof(T));
         int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
         for (; g + 3 * stride < n4; g += 4 * stride) {  // four loads in flight per lane
-            const float4 v0 = p4[g], v1 = p4[g + stride], v2 = p4[g + 2 * stride],
-                         v3 = p4[g + 3 * stride];
-            m = amax4(amax4(amax4(amax4(m, v0), v1), v2), v3);
+            const V v0 = p4[g], v1 = p4[g + stride], v2 = p4[g + 2 * stride], v3 = p4[g + 3 * stride];
+            m = amax_vec(amax_vec(amax_vec(amax_vec(m, v0), v1), v2), v3);
         }
-        for (; g < n4; g += stride) m = amax4(m, p4[g]);
+        for (; g < n4; g += stride) m = amax_vec(m, p4[g]);
     } else {
         for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-            m = fmaxf(m, fabsf(p[i]));
+            m = fmaxf(m, fabsf((float)p[i]));
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
@@ -557,7 +563,7 @@ bool kmx_mfma_supported(int d, int k) {
 }
 
 int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void* w, char* ws,
-                               int64_t n, int d, hipStream_t stream) {
+                               int64_t n, int d, int dtype, hipStream_t stream) {
     unsigned int* absmax = reinterpret_cast<unsigned int*>(ws + L.off_scales);
     int* q_exp = reinterpret_cast<int*>(absmax + (d + 1));
     hipLaunchKernelGGL(absmax_zero_kernel, dim3(1), dim3(256), 0, stream, absmax, d + 1);
@@ -565,8 +571,12 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
     if (gx > 64) gx = 64;
     if (gx * (d + 1) < 1024) gx = kmx_cdiv(1024, d + 1) < kmx_cdiv(n, 1024) ? kmx_cdiv(1024, d + 1) : kmx_cdiv(n, 1024);
     const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0) && ((((uintptr_t)w) & 15) == 0);
-    hipLaunchKernelGGL(absmax_rows_kernel, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
-                       stream, (const float*)X_t, (const float*)w, absmax, n, d, vec_ok);
+    if (dtype == KMX_F64)
+        hipLaunchKernelGGL(absmax_rows_kernel<double>, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
+                           stream, (const double*)X_t, (const double*)w, absmax, n, d, vec_ok);
+    else
+        hipLaunchKernelGGL(absmax_rows_kernel<float>, dim3((unsigned)gx, (unsigned)(d + 1)), dim3(256), 0,
+                           stream, (const float*)X_t, (const float*)w, absmax, n, d, vec_ok);
     hipLaunchKernelGGL(fixed_point_exponents_kernel, dim3((unsigned)kmx_cdiv(d + 1, 128)), dim3(128), 0,
                        stream, absmax, q_exp, n, d);
     const size_t words = (size_t)(d + 1) * L.k_for_gsum * 2;
@@ -574,9 +584,8 @@ int32_t kmx_lloyd_mfma_prepare(const LloydLayout& L, const void* X_t, const void
                        reinterpret_cast<unsigned int*>(ws + L.off_gsum), (int)words);
     KMX_LAUNCH_CHECK();
     // the screened step compares score gaps with a bound proportional to ||x_i||
-    if (L.screen)
-        return kmx_sample_norms((const float*)X_t, reinterpret_cast<float*>(ws + L.off_bucket + 256), n, d,
-                                stream);
+    if (L.screen || L.screen64)
+        return kmx_sample_norms(X_t, reinterpret_cast<float*>(ws + L.off_bucket + 256), n, d, dtype, stream);
     return KMX_OK;
 }
 
@@ -642,6 +651,43 @@ int32_t kmx_lloyd_iter_mfma_f32(const LloydLayout& L, const void* X_t, const voi
                        (size_t)(d + 1) * k * sizeof(float), stream, gsum, q_exp, tail);
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[3], stream);
+    return KMX_OK;
+}
+
+// fp64 inputs: the screened fused step (lloyd_mfma_screen.hip), whose last workgroup finishes
+// the iteration.
+int32_t kmx_lloyd_iter_mfma_screen_f64(const LloydLayout& L, const void* X_t, const void* w,
+                                       const void* centroids_t, void* new_centroids_t,
+                                       const uint32_t* labels_prev, uint32_t* labels, void* sizes,
+                                       uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
+                                       hipStream_t stream, hipEvent_t* events) {
+    if (!L.screen64) return KMX_ERR_UNSUPPORTED;
+    LloydTail<double> tail;
+    tail.sums_t = (double*)new_centroids_t;
+    tail.sizes = (double*)sizes;
+    tail.empty_clusters = empty_clusters;
+    tail.old_centroids_t = (const double*)centroids_t;
+    tail.cpack = reinterpret_cast<double*>(ws + L.off_cpack);
+    tail.half_norms = reinterpret_cast<double*>(ws + L.off_half);
+    tail.status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
+    tail.d = d;
+    tail.k = k;
+    tail.dpad = L.dpad;
+    const int* q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
+    unsigned long long* gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
+    uint32_t* uncertain = reinterpret_cast<uint32_t*>(ws + L.off_bucket);
+    tail.clear_word = uncertain;
+    tail.n_samples = n;
+    tail.delta_divisor = 3;  // (as for fp32 inputs)
+    tail.list_divisor = 24;
+    if (events) (void)hipEventRecord(events[0], stream);
+    const int32_t rc = kmx_lloyd_step_mfma_screen_f64(
+        X_t, w, centroids_t, labels_prev, labels, tail.status,
+        reinterpret_cast<const unsigned int*>(ws + L.off_scales), q_exp, gsum, uncertain,
+        reinterpret_cast<const float*>(ws + L.off_bucket + 256), n, d, k, L.wgs_per_cu, stream, &tail);
+    if (rc != KMX_OK) return rc;
+    if (events)
+        for (int i = 1; i < 4; ++i) (void)hipEventRecord(events[i], stream);
     return KMX_OK;
 }
 

@@ -1,4 +1,4 @@
-// fp32 fused Lloyd step whose label assignment is SCREENED on the fp16 matrix cores of gfx950
+// Fused Lloyd step (fp32 or fp64 inputs) whose label assignment is SCREENED on the fp16 matrix cores of gfx950
 // (v_mfma_f32_32x32x16_f16, 16x the rate of the fp32 MFMA) and CERTIFIED per sample.
 //
 // X and the centroids are scaled by one power of two, 2^-a, that brings max|x| into
@@ -25,6 +25,14 @@
 // decides), and the sums are taken from the fp32 inputs in 64-bit fixed point exactly as in
 // lloyd_mfma.hip.  Non-finite scores make a sample uncertain.
 //
+// fp64 inputs (TX = double) go through the same screen: the rows are rounded to fp32 as they
+// arrive (one more 2^-24 per value, counted in the bound), the part of the bound that belongs to a
+// centroid is kept per centroid (see PER_CENTROID in the kernel), and the samples the screen cannot
+// certify - a few percent where two centroids share a blob, since the bound is relative to fp32
+// roundings - are noted in a list of the workgroup and evaluated sixteen at a time on the fp64
+// matrix cores after the last tile.  The sums are taken from the fp64 inputs, one rounding to the
+// 64-bit fixed point per term.
+//
 // The same kernel without the update assigns labels only (kmx_assign_labels): there the scale
 // comes from the centroids (any scale is correct, a sample that overflows fp16 merely fails the
 // test) and each tile takes the norms of its samples itself.
@@ -45,11 +53,17 @@ typedef double v8d __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 // Error bound of one approximate score, in scaled units:
 //   (SCR_ERR_SPLIT + r) ||x|| C + r H + SCR_ERR_ABS sqrt(d) (||x|| + C),
 // r = SCR_ERR_ROUND * 51 * (K steps of 16 features): one ulp per addition of the accumulation
 constexpr float SCR_ERR_SPLIT = 7.2e-7f;  // 3.01 * 2^-22, rounded up
+// fp64 inputs reach the split through one rounding to fp32 (2^-24 relative, for x and for c): what
+// the two fp16 parts leave out is then at most 1.25 * 2^-22 of a value instead of 2^-22, and the
+// half norms in the scores are those of the rounded centroids (2^-23 relative)
+constexpr float SCR_ERR_SPLIT_F64 = 9.6e-7f;  // 4.01 * 2^-22, rounded up
+constexpr float SCR_ERR_HNEG_F64 = 1.2e-7f;   // 2^-23, rounded up
 constexpr float SCR_ERR_ROUND = 1.2e-7f;  // 2^-23, rounded up
 constexpr float SCR_ERR_ABS = 6.2e-5f;    // 2^-14, rounded up
 // Scaled data lie in [2^(SCR_SCALE_EXP - 1), 2^SCR_SCALE_EXP): low enough for -0.5||c||^2 / SCR_HK_X1
@@ -88,13 +102,18 @@ constexpr int SCR_WORD_DELTA = 2;
 constexpr int scr_waves(int nk) { return nk == 1 ? KMX_SCR_WAVES : (nk == 2 ? 4 : 8); }
 
 struct ScreenLds {
-    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, off_queue, off_moved, total;
+    size_t off_afh, off_afl, off_hneg, off_ct, off_hx, off_ctx, off_hxx, off_qlist, off_queue, off_moved, total;
     int kp;       // centroids rounded up to a multiple of 64
+    int ql_cap;   // fp64 inputs: samples the workgroup can note for evaluation (there is no queue then)
     int q_cap;    // entries of the queue of samples the screen could not certify
-    int q_words;  // 32-bit words per entry: 16 nk feature values, weight, sample index, old label
+    int q_words;  // 32-bit words per entry: 16 nk feature values and the weight (in the input type), sample index, old label
     int m_cap;    // entries of the list of samples that change cluster (fused step)
 };
 constexpr int SCR_QUEUE_MAX = 256;
+// fp64 inputs: a few percent of the samples of a blob that two centroids share fail a screen whose
+// bound is relative to fp32 roundings, so the workgroup notes their indices (this many at most)
+// and works them off sixteen at a time on the fp64 matrix cores, their rows gathered from memory
+constexpr int SCR_QLIST_F64 = 4096;
 // The list serves the iterations that correct the sums (at most one label in 24 changed in the
 // iteration before: about n / 24 / workgroups entries); a tile that finds it full adds its
 // changes on the spot.
@@ -105,7 +124,9 @@ constexpr int SCR_MOVED_WORDS = 3;  // sample index, old label, new label
 // leave room for two waves per SIMD) can have nearly all of it, two workgroups of four waves
 // (two K steps) half each.  Above 64 KB the kernel needs hipFuncAttributeMaxDynamicSharedMemorySize.
 __host__ __device__ constexpr size_t scr_lds_max(int nk) { return nk == 2 ? 78 * 1024 : 156 * 1024; }
-__host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update) {
+// esize: bytes of an input element (4, or 8: fp64 inputs keep an fp64 copy of the centroids and
+// of their half norms for the samples the screen cannot certify)
+__host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool update, int esize = 4) {
     ScreenLds s;
     // (an even number of centroid blocks: the scoring loop takes them in pairs; a block past
     // the last one holds padding only, whose scores are -inf)
@@ -116,15 +137,19 @@ __host__ __device__ inline ScreenLds screen_lds(int d, int k, int nk, bool updat
     s.off_afl = s.off_afh + n_cb * nk * 64 * 16;
     s.off_hneg = s.off_afl + n_cb * nk * 64 * 16;
     s.kp = (k + 63) & ~63;
-    s.off_ct = s.off_hneg + n_cb * 32 * 4;             // fp32 centroids, (d, kp)
-    s.off_hx = s.off_ct + (size_t)d * s.kp * 4;        // fp32 0.5||c||^2, (kp), +inf past k
-    s.off_queue = s.off_hx + (size_t)s.kp * 4;
+    s.off_ct = s.off_hneg + n_cb * 32 * 4;             // fp32 centroids, (d, kp) (fp32 inputs only)
+    s.off_hx = s.off_ct + (esize == 8 ? 0 : (size_t)d * s.kp * 4);  // fp32 (kp): 0.5||c||^2, +inf past k; fp64 inputs: the centroid's term of the bound
+    s.off_ctx = (s.off_hx + (size_t)s.kp * 4 + 7) & ~(size_t)7;                   // fp64 inputs: centroids and half norms in fp64
+    s.off_hxx = s.off_ctx + (esize == 8 ? (size_t)d * s.kp * 8 : 0);
+    s.off_qlist = s.off_hxx + (esize == 8 ? (size_t)s.kp * 8 : 0);
+    s.ql_cap = esize == 8 ? SCR_QLIST_F64 : 0;
+    s.off_queue = s.off_qlist + (size_t)s.ql_cap * 4;
     // the queue takes what is left of the workgroup's LDS, up to SCR_QUEUE_MAX entries (none:
     // every uncertain sample is then handled where it turns up)
-    s.q_words = 16 * nk + 4;
+    s.q_words = (esize / 4) * (16 * nk + 1) + (esize == 8 ? 2 : 3);
     const size_t cap = scr_lds_max(nk);
     const size_t room = s.off_queue < cap ? (cap - s.off_queue) / ((size_t)s.q_words * 4) : 0;
-    s.q_cap = (int)(room < (size_t)SCR_QUEUE_MAX ? room : (size_t)SCR_QUEUE_MAX);
+    s.q_cap = esize == 8 ? 0 : (int)(room < (size_t)SCR_QUEUE_MAX ? room : (size_t)SCR_QUEUE_MAX);
     s.off_moved = s.off_queue + (size_t)s.q_cap * s.q_words * 4;
     const size_t room_m = (update && s.off_moved < cap) ? (cap - s.off_moved) / ((size_t)SCR_MOVED_WORDS * 4) : 0;
     s.m_cap = (int)(room_m < (size_t)SCR_MOVED_MAX ? room_m : (size_t)SCR_MOVED_MAX);
@@ -199,6 +224,9 @@ __device__ __forceinline__ unsigned int wave_umax(unsigned int v) {
     return max(max(r0, r1), max(r2, r3));
 }
 
+__device__ __forceinline__ float scr_fma(float a, float b, float c) { return fmaf(a, b, c); }
+__device__ __forceinline__ double scr_fma(double a, double b, double c) { return fma(a, b, c); }
+
 // One column of 32 samples against all centroids in plain fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32 from -0.5||c||^2, lowest index wins a tie): the route for columns with
 // several samples the screen cannot certify.  rows.v[8 s + i] = feature 16 s + 2 i + h of the
@@ -246,16 +274,22 @@ __device__ __forceinline__ uint32_t redo_column_fp32(const ColumnRows<NK>& rows,
 // into inertia_partial[blockIdx.x].  sample_weight may be null (unit weights).  The rows of a tile
 // are then still needed at its end, so the next tile's are requested there and not while the
 // tile is scored.
-template <int NK, bool UPDATE, bool HK, bool INERTIA = false>
+// TX: the type of X, the weights and the centroids.  fp64 inputs are rounded to fp32 where the rows
+// arrive and are screened like fp32 ones (the bound counts that rounding); the samples the screen
+// cannot certify are evaluated in fp64, and the sums are taken from the fp64 inputs.
+template <typename TX, int NK, bool UPDATE, bool HK, bool INERTIA = false>
 __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2) void lloyd_screen_kernel(
-    const float* __restrict__ X_t, const float* __restrict__ sample_weight,
-    const float* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
+    const TX* __restrict__ X_t, const TX* __restrict__ sample_weight,
+    const TX* __restrict__ centroids_t, const uint32_t* __restrict__ labels_prev,
     uint32_t* __restrict__ labels, kmx_lloyd_status* __restrict__ status,
     const unsigned int* __restrict__ absmax, const int* __restrict__ q_exp,
     unsigned long long* __restrict__ gsum, uint32_t* __restrict__ uncertain_count,
     const float* __restrict__ norms, int64_t n, int d, int k, int vec_ok,
-    double* __restrict__ inertia_partial, const LloydTail<float> tail, const int fuse_tail) {
+    double* __restrict__ inertia_partial, const LloydTail<TX> tail, const int fuse_tail) {
     static_assert(!(UPDATE && INERTIA), "the inertia rides with the labels-only kernel");
+    constexpr bool F64 = sizeof(TX) == 8;
+    static_assert(!(F64 && INERTIA), "fp64 inputs: labels and inertia are two calls");
+    constexpr int ES = (int)sizeof(TX), FW = ES / 4;  // bytes and 32-bit words of an input element
     // (labels only: `status` is null outside the iteration loop)
     if ((UPDATE || status != nullptr) && status->state != KMX_RUNNING) return;
 
@@ -279,21 +313,40 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     const int d_even = (d + 1) & ~1;
     const int acc_stride = d_even + 1;
     const int items = acc_stride * k;
-    const ScreenLds lay = screen_lds(d, k, NK, UPDATE);
+    const ScreenLds lay = screen_lds(d, k, NK, UPDATE, ES);
     unsigned long long* acc = reinterpret_cast<unsigned long long*>(smem_raw);  // [k][d_even + 1]
     v8h* afh = reinterpret_cast<v8h*>(smem_raw + lay.off_afh);                  // [n_cb][NK][64]
     v8h* afl = reinterpret_cast<v8h*>(smem_raw + lay.off_afl);
     float* hneg = reinterpret_cast<float*>(smem_raw + lay.off_hneg);            // [n_cb][2][16]
     float* ct = reinterpret_cast<float*>(smem_raw + lay.off_ct);                // [d][kp]
     float* hx = reinterpret_cast<float*>(smem_raw + lay.off_hx);                // [kp]
+    // what the samples the screen cannot certify are evaluated with: the centroids and half norms
+    // in the input type (fp32 inputs: the two arrays above)
+    TX* ctx = F64 ? reinterpret_cast<TX*>(smem_raw + lay.off_ctx) : reinterpret_cast<TX*>(ct);   // [d][kp]
+    TX* hxx = F64 ? reinterpret_cast<TX*>(smem_raw + lay.off_hxx) : reinterpret_cast<TX*>(hx);   // [kp]
     const int kp = lay.kp;
+    // centroid value (f, c) as the screen takes it
+    auto cval = [&](const int f, const int c) __attribute__((always_inline)) {
+        if constexpr (F64) return (float)ctx[f * kp + c];
+        else return ct[f * kp + c];
+    };
     // Queue of the samples the screen could not certify, evaluated in fp32 by the whole
     // workgroup after the last tile: per entry the 16 NK feature values in feature order, the
     // weight, the sample index (QUEUE_FREE: never written) and the previous label.
     uint32_t* queue = reinterpret_cast<uint32_t*>(smem_raw + lay.off_queue);    // [q_cap][q_words]
     const int q_cap = lay.q_cap;
-    constexpr int QW = 16 * NK + 4, Q_WEIGHT = 16 * NK, Q_INDEX = 16 * NK + 1, Q_PREV = 16 * NK + 2;
+    // (features and weight in the input type, then two 32-bit words)
+    constexpr int NKF = 16 * NK;
+    constexpr int QW = FW * (NKF + 1) + (F64 ? 2 : 3), Q_WEIGHT = FW * NKF, Q_INDEX = FW * (NKF + 1),
+                  Q_PREV = FW * (NKF + 1) + 1;
     constexpr uint32_t QUEUE_FREE = 0xffffffffu;
+    // where a tile notes the index of an uncertain sample: the entry's index word, or (fp64
+    // inputs) a list of indices
+    uint32_t* qlist = reinterpret_cast<uint32_t*>(smem_raw + lay.off_qlist);
+    const int note_cap = F64 ? lay.ql_cap : q_cap;
+    auto noted = [&](const int slot) __attribute__((always_inline)) -> uint32_t& {
+        return F64 ? qlist[slot] : queue[slot * QW + Q_INDEX];
+    };
     __shared__ unsigned int queue_count;
     // Samples that change cluster while the sums are only corrected: (index, old label, new
     // label), their terms moved from the old to the new cluster after the last tile.
@@ -338,9 +391,10 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     // The loads are buffer loads: resource descriptor (the array) and tile offset in scalar
     // registers, the lane's offset in one vector register, so a load needs no address arithmetic.
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float*>(X_t), 0, (int)(uint32_t)((uint64_t)d * (uint64_t)n * 4u), 0x00020000);
+        const_cast<TX*>(X_t), 0, (int)(uint32_t)((uint64_t)d * (uint64_t)n * (uint64_t)ES), 0x00020000);
     const __amdgpu_buffer_rsrc_t norms_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float*>(UPDATE ? norms : X_t), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
+        const_cast<float*>(UPDATE ? norms : reinterpret_cast<const float*>(X_t)), 0,
+        (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
     const __amdgpu_buffer_rsrc_t pl_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint32_t*>(UPDATE ? labels_prev : labels), 0, (int)(uint32_t)((uint64_t)n * 4u), 0x00020000);
     const uint32_t own_off = (uint32_t)(MC * j + h) * 4u;  // the lane's own sample inside a tile
@@ -350,19 +404,27 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int f = 16 * s + 2 * i + h;
-            row_off[s][i] = (uint32_t)(f < d ? f : d - 1) * (uint32_t)n * 4u + (uint32_t)(MC * j) * 4u;
+            row_off[s][i] = (uint32_t)(f < d ? f : d - 1) * (uint32_t)n * (uint32_t)ES + (uint32_t)(MC * j * ES);
         }
     // (the spare slot's constant is put in where the rows are consumed: a select here would make
     // the wave wait for loads it has only just requested)
-    auto load_rows_raw = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
-        const uint32_t tile = (uint32_t)wt * (uint32_t)(TILE * 4);  // wave-uniform byte offset in row 0
+    auto load_rows_raw = [&](const int wt, auto& dst) __attribute__((always_inline)) {
+        using TD = std::remove_reference_t<decltype(dst[0][0][0])>;  // float: for the screen; TX: for the sums
+        const uint32_t tile = (uint32_t)wt * (uint32_t)(TILE * ES);  // wave-uniform byte offset in row 0
 #pragma unroll
         for (int s = 0; s < NK; ++s)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const v2u q = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, row_off[s][i], tile, 0);
-                dst[s][i][0] = __uint_as_float(q[0]);
-                dst[s][i][1] = __uint_as_float(q[1]);
+                if constexpr (F64) {
+                    // two fp64 samples per load (rounded to fp32 for the screen)
+                    const v4u q = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, row_off[s][i], tile, 0);
+                    dst[s][i][0] = (TD)__hiloint2double((int)q[1], (int)q[0]);
+                    dst[s][i][1] = (TD)__hiloint2double((int)q[3], (int)q[2]);
+                } else {
+                    const v2u q = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, row_off[s][i], tile, 0);
+                    dst[s][i][0] = __uint_as_float(q[0]);
+                    dst[s][i][1] = __uint_as_float(q[1]);
+                }
             }
     };
     // The rows, norm and previous label of a tile are requested while the tile before it
@@ -371,18 +433,42 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     float x[NK][8][MC];
     float norm_next = 0.0f;
     uint32_t pl_next = 0u;
+    // fp64 inputs: the rows arrive as they are in memory (two samples per register quad) and are
+    // rounded to fp32 when their tile starts - a conversion at the request would wait for the data
+    v4u x_raw[F64 ? NK : 1][8];
+    auto arrive = [&]() __attribute__((always_inline)) {
+        if constexpr (F64) {
+#pragma unroll
+            for (int s = 0; s < NK; ++s)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    x[s][i][0] = (float)__hiloint2double((int)x_raw[s][i][1], (int)x_raw[s][i][0]);
+                    x[s][i][1] = (float)__hiloint2double((int)x_raw[s][i][3], (int)x_raw[s][i][2]);
+                }
+        }
+    };
     auto request = [&](const int wt_) __attribute__((always_inline)) {
         if (wt_ < n_main) {  // wave-uniform
-            load_rows_raw(wt_, x);
+            if constexpr (F64) {
+                const uint32_t tile = (uint32_t)wt_ * (uint32_t)(TILE * ES);
+#pragma unroll
+                for (int s = 0; s < NK; ++s)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        x_raw[s][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, row_off[s][i], tile, 0);
+            } else {
+                load_rows_raw(wt_, x);
+            }
             if (UPDATE) {
-                const uint32_t tile = (uint32_t)wt_ * (uint32_t)(TILE * 4);
+                const uint32_t tile = (uint32_t)wt_ * (uint32_t)(TILE * 4);  // (4-byte arrays whatever the input type)
                 norm_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(norms_rsrc, own_off, tile, 0));
                 pl_next = __builtin_amdgcn_raw_buffer_load_b32(pl_rsrc, own_off, tile, 0);
             }
         }
     };
-    // (more than one K step: the registers do not allow it, the tile's data are requested when it starts)
-    constexpr bool AHEAD = NK == 1;
+    // (more than one K step: the registers do not allow it, the tile's data are requested when it
+    // starts; fp64 inputs of up to 32 features leave room for the raw rows of the next tile)
+    constexpr bool AHEAD = NK == 1 || (F64 && NK == 2);
     // the wave's first tile: ticket = its index in the workgroup (in a scalar register: tile offsets are scalar operands)
     const int wt_start = __builtin_amdgcn_readfirstlane((int)blockIdx.x * WAVES + wave);
 
@@ -394,19 +480,24 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         // Labels only: max|x| is not known and any scale is a correct one (a sample that overflows
         // fp16 gives infinite or NaN scores, fails the test and is evaluated in fp32), so four
         // times max|c| stands in for it: samples lie around the centroids they are assigned to.
+        // Fused step: the larger of max|x| and max|c|.  Centroids that are means of samples never
+        // exceed max|x|; initial centroids from elsewhere can, and would overflow fp16 and leave
+        // every sample uncertified.
         unsigned int my_absmax = (UPDATE && threadIdx.x < d) ? absmax[threadIdx.x] : 0u;
         for (int f = wave_; f < d; f += WAVES)
             for (int c = lane_; c < kp; c += 64) {
-                const float v = c < k ? centroids_t[(size_t)f * k + c] : 0.0f;
-                ct[f * kp + c] = v;
-                if (!UPDATE) my_absmax = max(my_absmax, __float_as_uint(fabsf(v) * 4.0f));
+                const TX vx = c < k ? centroids_t[(size_t)f * k + c] : TX(0);
+                const float v = (float)vx;
+                if constexpr (F64) ctx[f * kp + c] = vx;
+                else ct[f * kp + c] = v;
+                my_absmax = max(my_absmax, __float_as_uint(fabsf(v) * (UPDATE ? 1.0f : 4.0f)));
             }
         // The wave's first tile is requested here, behind the loads of the centroids (loads
         // return in order): its rows travel while the operands are prepared.
         if (AHEAD) request(wt_start);
         __syncthreads();  // the shared words above are zero
         // (non-negative floats order like their bits)
-        if (UPDATE ? threadIdx.x < d : my_absmax != 0u) atomicMax(&xmax_bits, my_absmax);
+        if (my_absmax != 0u) atomicMax(&xmax_bits, my_absmax);
     }
     __syncthreads();
     // 2^-a with max|x| * 2^-a in [2^(SCR_SCALE_EXP - 1), 2^SCR_SCALE_EXP) (1 for all-zero or non-finite data)
@@ -415,6 +506,19 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     // a half, two thirds of the workgroup): each is a chain of LDS round trips too short to
     // fill the workgroup, and one after the other on the same threads they took 3.7 us.
     auto rotated = [&](const int by) { return (int)((threadIdx.x + THREADS - by) % THREADS); };
+    // PER_CENTROID (fp64 inputs): the error bound of the score of centroid c,
+    //   r (H_c + ||x|| ||c||) + split ||x|| ||c|| + (rounding of H_c) + absolute part,  H_c = 0.5||c||^2,
+    // is kept per centroid instead of through max ||c|| and max H.  With ||x|| ||c|| <= 0.5||x||^2 + H_c
+    // it is at most rho H_c + X, rho = 2 r + split + (rounding of H_c), X = (r + split) 0.5||x||^2 +
+    // absolute part.  The scores start from -(1 - rho) H_c, which makes every computed score an
+    // upper bound of the exact one up to X, and the winner b is certain when it leads by
+    // 2 X + 2 rho H_b.  One far-away centroid (an initial centroid outside the data) then no longer
+    // costs every sample its certificate.
+    constexpr bool PER_CENTROID = F64;
+    const float sigma = SCR_ERR_ROUND * 51.0f * (float)NK + SCR_ERR_SPLIT_F64;
+    const float rho = sigma + SCR_ERR_ROUND * 51.0f * (float)NK + SCR_ERR_HNEG_F64 + (HK ? SCR_ERR_HNEG : 0.0f) +
+                      SCR_ERR_ROUND;
+    const float h_keep = PER_CENTROID ? 1.0f - rho : 1.0f;
     constexpr int ROT_HNEG = (THREADS / 3) & ~63, ROT_HX = THREADS / 2, ROT_ZERO = (2 * THREADS / 3) & ~63;
     // A operand: hi and lo parts of 32 centroids x 16 features per block and K step
     for (int idx = threadIdx.x; idx < n_cbe * NK * 64; idx += THREADS) {
@@ -426,7 +530,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int f = 16 * s + 2 * i + (l >> 5);
-            float v = f < d ? ct[f * kp + c] * xs : 0.0f;
+            float v = f < d ? cval(f, c) * xs : 0.0f;
             if (HK && f == SPARE) {
                 // the spare slot: -0.5||c||^2 / SCR_HK_X1, summed exactly as for hneg below;
                 // -inf for the padding past k, whose scores then never win
@@ -435,10 +539,10 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     float sq = 0.0f;
 #pragma unroll 8
                     for (int g = 0; g < d; ++g) {
-                        const float cv = ct[g * kp + c] * xs;
+                        const float cv = cval(g, c) * xs;
                         sq += cv * cv;
                     }
-                    v = -(sq / 2.0f) * (1.0f / SCR_HK_X1);
+                    v = -(sq / 2.0f) * (1.0f / SCR_HK_X1) * h_keep;
                 }
             }
             const _Float16 hb = (_Float16)v;
@@ -462,33 +566,36 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             float sq = 0.0f;
 #pragma unroll 8
             for (int f = 0; f < d; ++f) {
-                const float cv = ct[f * kp + c] * xs;
+                const float cv = cval(f, c) * xs;
                 sq += cv * cv;
             }
-            v = -(sq / 2.0f);
+            v = -(sq / 2.0f) * h_keep;
             // non-negative floats order like their bits; a NaN norm ends up as the maximum
             // and makes every sample uncertain
             atomicMax(&hmax_bits, __float_as_uint(sq / 2.0f));
+            if constexpr (PER_CENTROID) hx[c] = 2.01f * rho * (sq / 2.0f);
+        } else if (PER_CENTROID && c < kp) {
+            hx[c] = 0.0f;
         }
         hneg[idx] = v;
     }
     // unscaled half norms for the samples the screen cannot certify
     for (int c = rotated(ROT_HX); c < kp; c += THREADS) {
-        float v = kmx_inf<float>();
+        TX v = kmx_inf<TX>();
         if (c < k) {
-            float sq = 0.0f;
+            TX sq = TX(0);
 #pragma unroll 8
             for (int f = 0; f < d; ++f) {
-                const float cv = ct[f * kp + c];
+                const TX cv = ctx[f * kp + c];
                 sq += cv * cv;
             }
-            v = sq / 2.0f;
+            v = sq / TX(2);
         }
-        hx[c] = v;
+        hxx[c] = v;
     }
     if (UPDATE)
         for (int jx = rotated(ROT_ZERO); jx < items; jx += THREADS) acc[jx] = 0ull;
-    for (int e = rotated(ROT_ZERO); e < q_cap; e += THREADS) queue[e * QW + Q_INDEX] = QUEUE_FREE;
+    for (int e = rotated(ROT_ZERO); e < note_cap; e += THREADS) noted(e) = QUEUE_FREE;
     for (int e = rotated(ROT_ZERO); e < m_cap; e += THREADS) moved[e * SCR_MOVED_WORDS] = QUEUE_FREE;
     __syncthreads();
 
@@ -505,9 +612,14 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     const float round_term = SCR_ERR_ROUND * 51.0f * (float)NK;
     // (||x|| comes unscaled from kmx_lloyd_init, hence the factor xs)
     // (and a norm the kernel takes itself, from the scaled values: no factor)
-    const float thr_x = 2.01f * ((SCR_ERR_SPLIT + round_term) * cmax + abs_term) * (UPDATE ? xs : 1.0f);
-    const float thr_0 = 2.01f * (round_term * hmax + abs_term * cmax +
-                                 (HK ? SCR_ERR_HNEG * hmax + SCR_ERR_ABS * SCR_HK_X1 : 0.0f));
+    const float thr_x = 2.01f * (PER_CENTROID ? abs_term : (SCR_ERR_SPLIT + round_term) * cmax + abs_term) *
+                        (UPDATE ? xs : 1.0f);
+    // (per centroid: the term in ||x||^2)
+    const float thr_xx = PER_CENTROID ? 2.01f * 0.5f * sigma * (UPDATE ? xs * xs : 1.0f) : 0.0f;
+    const float thr_0 =
+        PER_CENTROID ? 2.01f * (abs_term * cmax + (HK ? SCR_ERR_ABS * SCR_HK_X1 : 0.0f))
+                     : 2.01f * (round_term * hmax + abs_term * cmax +
+                                (HK ? SCR_ERR_HNEG * hmax + SCR_ERR_ABS * SCR_HK_X1 : 0.0f));
     // what a sample carries in the spare slot: its scaled value is SCR_HK_X1
     const float hk_x = SCR_HK_X1 / xs;
     // +inf the optimiser cannot see through (it would turn the median below into a maximum
@@ -525,6 +637,87 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
     const bool full_mode = UPDATE ? (uncertain_count[SCR_WORD_DELTA] == 0u) : false;  // wave-uniform
     // (corrected sums: whether the samples that move are few enough for the workgroup's list)
     const bool use_list = UPDATE ? (uncertain_count[SCR_WORD_DELTA] == 1u) : false;
+
+    // One sample against every centroid in the input type, by the whole wave: lane l takes the
+    // centroids l, l + 64, ... (fused multiply-adds in feature order from -0.5||c||^2, strict '>'
+    // in increasing order), then the wave combines: the largest score, the lowest index among
+    // the lanes that hold it.  `xat(f)`: feature f of the sample (wave-uniform).
+    auto evaluate_sample = [&](auto&& xat) __attribute__((always_inline)) {
+        TX bs = -kmx_inf<TX>();
+        int bc = 0x7fffffff;
+        // Two centroids per lane and pass, FB features at a time whose reads are in flight
+        // together (past d the last row is read again and the sum left alone); the additions
+        // stay in feature order.
+        constexpr int FB = F64 ? 8 : 16;
+        for (int c = lane; c < kp; c += 128) {
+            const bool two = c + 64 < kp;  // wave-uniform: kp is a multiple of 64
+            const int c1 = two ? c + 64 : c;
+            const TX* col0 = ctx + c;
+            const TX* col1 = ctx + c1;
+            TX s0 = -hxx[c], s1 = -hxx[c1];
+            if (F64 && !two) {
+                // (a last odd pass: one chain; fp64 multiply-adds are not free)
+                for (int f0 = 0; f0 < d; f0 += FB) {
+                    TX xv[FB], a0[FB];
+#pragma unroll
+                    for (int i = 0; i < FB; ++i) {
+                        const int f = f0 + i < d ? f0 + i : d - 1;  // wave-uniform
+                        xv[i] = xat(f);
+                        a0[i] = col0[f * kp];
+                    }
+#pragma unroll
+                    for (int i = 0; i < FB; ++i) {
+                        const TX t0 = scr_fma(xv[i], a0[i], s0);
+                        s0 = f0 + i < d ? t0 : s0;
+                    }
+                }
+            } else {
+                for (int f0 = 0; f0 < d; f0 += FB) {
+                    TX xv[FB], a0[FB], a1[FB];
+#pragma unroll
+                    for (int i = 0; i < FB; ++i) {
+                        const int f = f0 + i < d ? f0 + i : d - 1;  // wave-uniform
+                        xv[i] = xat(f);
+                        a0[i] = col0[f * kp];
+                        a1[i] = col1[f * kp];
+                    }
+#pragma unroll
+                    for (int i = 0; i < FB; ++i) {
+                        const TX t0 = scr_fma(xv[i], a0[i], s0), t1 = scr_fma(xv[i], a1[i], s1);
+                        s0 = f0 + i < d ? t0 : s0;
+                        s1 = f0 + i < d ? t1 : s1;
+                    }
+                }
+            }
+            if (s0 > bs) {
+                bs = s0;
+                bc = c;
+            }
+            if (two && s1 > bs) {
+                bs = s1;
+                bc = c1;
+            }
+        }
+        if constexpr (F64) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const TX ov = __shfl_xor(bs, off, 64);
+                const int oc = __shfl_xor(bc, off, 64);
+                if (ov > bs || (ov == bs && oc < bc)) {
+                    bs = ov;
+                    bc = oc;
+                }
+            }
+        } else {
+            // (the score in an order-preserving integer form)
+            const unsigned int sb = __float_as_uint((float)bs);
+            const unsigned int ordered = sb ^ ((sb >> 31) ? 0xffffffffu : 0x80000000u);
+            const unsigned int top = wave_umax(ordered);
+            bc = (int)~wave_umax(ordered == top ? (unsigned int)~bc : 0u);
+        }
+        if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
+        return bc;
+    };
 
     // One tile of NC sample columns per lane.  NC = 2: 64 samples, lane (j, h) scores samples
     // i0 and i0 + 1 (i0 = first + 2 j) against its half of every centroid block and, once the
@@ -850,8 +1043,14 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             norm_mine = sqrtf(__uint_as_float(qq[0]) + __uint_as_float(qq[1]));
         }
         // written so that a NaN anywhere makes the sample uncertain
-        const float thr = fmaf(thr_x, norm_mine, thr_0);
+        float thr = fmaf(thr_x, norm_mine, thr_0);
+        if constexpr (PER_CENTROID)  // (an index below kp whatever the scores)
+            thr = fmaf(fmaf(thr_xx, norm_mine, thr_x), norm_mine, thr_0) + hx[lab_mine];
+#ifdef KMX_SCR_NO_UNSURE
+        const bool unsure_mine = false;
+#else
         const bool unsure_mine = !(b - s2 > thr) && in_range && owner;
+#endif
 
         // Samples the screen cannot certify go to the workgroup's queue (their label below is
         // provisional and they take no part in the sums here); the queue is worked off in plain
@@ -869,30 +1068,43 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 if (todo == 0u) continue;
                 const int n_todo = __popc(todo);
                 n_uncertain += (unsigned int)n_todo;
-                bool redo = n_todo >= SCR_REDO_COLUMN;
+                // (fp64 inputs have no matrix-core route for a whole column: everything goes to the queue)
+                bool redo = !F64 && n_todo >= SCR_REDO_COLUMN;
                 unsigned int base = 0;
                 if (!redo) {
                     if (lane == 0) base = atomicAdd(&queue_count, (unsigned int)n_todo);
                     base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
-                    redo = base + (unsigned int)n_todo > (unsigned int)q_cap;
+                    redo = base + (unsigned int)n_todo > (unsigned int)note_cap;
                 }
                 const bool col_mine = NC == 2 ? h == t : true;  // whether the lane's own sample is in column t
-                if (redo) {
-                    float xr[NK][8][NC];
-                    load(xr);
-                    ColumnRows<NK> rows;
+                if (redo && F64) {
+                    // queue full: the wave evaluates the column's uncertain samples at once, one
+                    // after the other, its features straight from memory
+                    for (unsigned int rest = todo; rest != 0u; rest &= rest - 1u) {
+                        const int jj = __builtin_ctz(rest);  // wave-uniform
+                        const int64_t smp = i0 - (NC == 2 ? MC * j : j) + (NC == 2 ? MC * jj + t : jj);
+                        const uint32_t r = (uint32_t)evaluate_sample(
+                            [&](const int f) __attribute__((always_inline)) { return X_t[(size_t)f * n + smp]; });
+                        if (col_mine && j == jj) lab_mine = r;
+                    }
+                } else if (redo) {
+                    if constexpr (!F64) {
+                        float xr[NK][8][NC];
+                        load(xr);
+                        ColumnRows<NK> rows;
 #pragma unroll
-                    for (int s = 0; s < NK; ++s)
+                        for (int s = 0; s < NK; ++s)
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = xr[s][i][t];
-                    const uint32_t r = redo_column_fp32<NK>(rows, ct, hx, n_cb, d, kp, h, j);
-                    if (col_mine) lab_mine = r;
+                            for (int i = 0; i < 8; ++i) rows.v[8 * s + i] = xr[s][i][t];
+                        const uint32_t r = redo_column_fp32<NK>(rows, ct, hx, n_cb, d, kp, h, j);
+                        if (col_mine) lab_mine = r;
+                    }
                 } else if ((todo >> j) & 1u) {  // both lanes of the sample
                     // (the index alone: the entry's features, weight and previous label are
                     // fetched after the last tile, all entries of the workgroup at once, so
                     // that the tile does not wait for a second read of its rows)
                     const unsigned int slot = base + (unsigned int)__popc(todo & ((1u << j) - 1u));
-                    if (h == 0) queue[slot * QW + Q_INDEX] = (uint32_t)(i0 + t);
+                    if (h == 0) noted((int)slot) = (uint32_t)(i0 + t);
                     if (col_mine) queued_mine = true;
                 }
             }
@@ -957,7 +1169,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                 }
             }
             if (act_all != 0ull && !listed) {
-                float xr[NK][8][NC];
+                TX xr[NK][8][NC];
                 load(xr);
                 // both columns' labels in every lane (the lane adds its features of both samples)
                 uint32_t lab[NC], pl[NC];
@@ -975,7 +1187,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     if (act_col == 0u) continue;
                     const bool act = (act_col >> j) & 1u;
                     // samples past the end and samples that stay put are not in the mask
-                    const double wd = act ? (double)sample_weight[i0 + t] : 0.0;
+                    const double wd = act ? (double)sample_weight[i0 + t] : 0.0;  // (fp64 inputs: exact)
                     unsigned long long* to = acc + lab[t] * (uint32_t)acc_stride + h;    // word h of the new cluster
                     unsigned long long* from = acc + pl[t] * (uint32_t)acc_stride + h;   // and of the old one
 #pragma unroll
@@ -1006,12 +1218,13 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         }
     };
 
-    auto load_rows = [&](const int wt, float(&dst)[NK][8][MC]) __attribute__((always_inline)) {
+    auto load_rows = [&](const int wt, auto& dst) __attribute__((always_inline)) {
+        using TD = std::remove_reference_t<decltype(dst[0][0][0])>;
         load_rows_raw(wt, dst);
         if (HK) {
             // the spare slot carries the constant whose scaled value is SCR_HK_X1
 #pragma unroll
-            for (int t = 0; t < MC; ++t) dst[NK - 1][7][t] = h ? hk_x : dst[NK - 1][7][t];
+            for (int t = 0; t < MC; ++t) dst[NK - 1][7][t] = h ? (TD)hk_x : dst[NK - 1][7][t];
         }
     };
 
@@ -1045,10 +1258,11 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const int64_t i0 = (int64_t)wt * TILE + MC * j;
             const int wt_now = wt;
             if (!AHEAD) request(wt_now);
+            arrive();
             uint32_t lab_now = 0u;
             process(
                 Cols2{}, std::true_type{},
-                [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_rows(wt_now, xr); },
+                [&](auto& xr) __attribute__((always_inline)) { load_rows(wt_now, xr); },
                 [&]() __attribute__((always_inline)) {
                     write_pending();
                     if (AHEAD) request(wt_next);
@@ -1065,18 +1279,18 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         if (mine) labels[idx] = lab;
     };
     // scalar loads of the lane's rows (row d - 1 where the feature does not exist)
-    auto load_scalar = [&](auto nc_tag, const int64_t i0, float(&dst)[NK][8][decltype(nc_tag)::value])
-                           __attribute__((always_inline)) {
+    auto load_scalar = [&](auto nc_tag, const int64_t i0, auto& dst) __attribute__((always_inline)) {
+        using TD = std::remove_reference_t<decltype(dst[0][0][0])>;
         constexpr int NC = decltype(nc_tag)::value;
 #pragma unroll
         for (int s = 0; s < NK; ++s)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int f = 16 * s + 2 * i + h;
-                const float* row = X_t + (size_t)(f < d ? f : d - 1) * n;
-                const float absent = (HK && f == SPARE) ? hk_x : 0.0f;  // the spare slot, or no feature at all
+                const TX* row = X_t + (size_t)(f < d ? f : d - 1) * n;
+                const TD absent = (HK && f == SPARE) ? (TD)hk_x : TD(0);  // the spare slot, or no feature at all
 #pragma unroll
-                for (int t = 0; t < NC; ++t) dst[s][i][t] = f < d ? (i0 + t < n ? row[i0 + t] : 0.0f) : absent;
+                for (int t = 0; t < NC; ++t) dst[s][i][t] = f < d ? (i0 + t < n ? (TD)row[i0 + t] : TD(0)) : absent;
             }
     };
     if (halves) {
@@ -1089,7 +1303,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             uint32_t pl_now = UPDATE ? labels_prev[i0] : 0u;
             process(
                 Cols1{}, std::true_type{},
-                [&](float(&xr)[NK][8][1]) __attribute__((always_inline)) { load_scalar(Cols1{}, i0, xr); }, [] {},
+                [&](auto& xr) __attribute__((always_inline)) { load_scalar(Cols1{}, i0, xr); }, [] {},
                 put_now, x, norm_now, pl_now, i0);
         }
     }
@@ -1103,29 +1317,66 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         uint32_t pl_now = (UPDATE && mine_exists) ? labels_prev[i0 + h] : 0u;
         process(
             Cols2{}, std::false_type{},
-            [&](float(&xr)[NK][8][MC]) __attribute__((always_inline)) { load_scalar(Cols2{}, i0, xr); }, [] {},
+            [&](auto& xr) __attribute__((always_inline)) { load_scalar(Cols2{}, i0, xr); }, [] {},
             put_now, x, norm_now, pl_now, i0);
     }
 
-    // The queue: one wave per entry, lane l on the centroids l, l + 64, ... (fused multiply-adds
-    // in feature order from -0.5||c||^2, strict '>' in increasing order), then the wave combines.
+    // The samples noted by the tiles.
     __syncthreads();  // lists complete; provisional labels have reached memory
-    {
-        // The queue's entries: features in feature order (zero past d), weight, previous label.
-        const int n_queued = (int)min(queue_count, (unsigned int)q_cap);
-        for (int item = threadIdx.x; item < n_queued * QW; item += THREADS) {
-            const int e = item / QW, wq = item - e * QW;
-            const uint32_t sample = queue[e * QW + Q_INDEX];
-            if (sample == QUEUE_FREE || wq == Q_INDEX || wq > Q_PREV) continue;
-            uint32_t v;
-            if (wq < 16 * NK)
-                v = wq < d ? __float_as_uint(X_t[(size_t)wq * n + sample]) : 0u;
-            else if (wq == Q_WEIGHT)
-                v = (UPDATE || (INERTIA && sample_weight != nullptr)) ? __float_as_uint(sample_weight[sample])
-                                                                      : __float_as_uint(1.0f);
-            else
-                v = UPDATE ? labels_prev[sample] : 0u;
-            queue[item] = v;
+    const int n_noted = (int)min(queue_count, (unsigned int)note_cap);
+    if constexpr (!F64) {
+        // one wave per entry of the queue (evaluate_sample), once the entries are filled in
+        const int n_queued = n_noted;
+        // The queue's entries: features in feature order (zero past d) and the weight in the input
+        // type, then the index and the previous label.  Thread (entry, slot) fetches one value,
+        // eight per thread and pass with all their reads in flight together (a loop of one load and
+        // one store per pass would take a trip to memory per pass).
+        {
+            constexpr int SLOTS = NKF + 2;  // features, weight, (index, previous label)
+            constexpr int U = 8;
+            const int total = n_queued * SLOTS;
+            for (int first = 0; first < total; first += U * THREADS) {
+                TX val[U];
+                uint32_t idx[U], prv[U];
+                int at[U];  // first word of the value in the queue; -1: nothing to store
+                bool pair[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int item = first + u * THREADS + (int)threadIdx.x;
+                    at[u] = -1;
+                    pair[u] = false;
+                    val[u] = TX(0);
+                    idx[u] = prv[u] = 0u;
+                    if (item < total) {
+                        const int e = item / SLOTS, sl = item - e * SLOTS;
+                        const uint32_t sample = noted(e);
+                        if (sl == NKF + 1) {
+                            // (QUEUE_FREE: a slot reserved and never written; the index word says so)
+                            at[u] = e * QW + Q_INDEX;
+                            pair[u] = true;
+                            idx[u] = sample;
+                            if (UPDATE && sample != QUEUE_FREE) prv[u] = labels_prev[sample];
+                        } else if (sample != QUEUE_FREE) {
+                            at[u] = e * QW + FW * sl;
+                            if (sl < NKF) {
+                                if (sl < d) val[u] = X_t[(size_t)sl * n + sample];
+                            } else {
+                                val[u] = (UPDATE || (INERTIA && sample_weight != nullptr)) ? sample_weight[sample] : TX(1);
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (at[u] < 0) continue;
+                    if (pair[u]) {
+                        queue[at[u]] = idx[u];
+                        queue[at[u] + 1] = prv[u];
+                    } else {
+                        *reinterpret_cast<TX*>(queue + at[u]) = val[u];
+                    }
+                }
+            }
         }
     }
     if (UPDATE) {
@@ -1136,15 +1387,15 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         const int wpe = d + 1, total = n_moved * wpe;
         constexpr int U = 4;
         for (int first = 0; first < total; first += U * THREADS) {
-            float xv[U], wv[U];
+            TX xv[U], wv[U];
             uint32_t from_c[U], to_c[U];
             int word[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int item = first + u * THREADS + (int)threadIdx.x;
                 word[u] = -1;
-                xv[u] = 1.0f;
-                wv[u] = 0.0f;
+                xv[u] = TX(1);
+                wv[u] = TX(0);
                 from_c[u] = to_c[u] = 0u;
                 if (item < total) {
                     const int e = item / wpe;
@@ -1163,7 +1414,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             for (int u = 0; u < U; ++u) {
                 if (word[u] < 0) continue;
                 const double magic = fix_magic(q_lds[word[u]]);
-                // x * w is exact in fp64; one rounding, to a multiple of 2^-q (the weight's word: w itself)
+                // x * w is exact in fp64 (fp32 inputs); one rounding, to a multiple of 2^-q (the weight's word: w itself)
                 const double v = word[u] < d ? fma((double)xv[u], (double)wv[u], magic) : (double)wv[u] + magic;
                 const unsigned long long term = to_fixed_q(v, magic);
                 const int slot = word[u] < d ? word[u] : d_even;
@@ -1173,8 +1424,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
         }
     }
     __syncthreads();  // entries complete
-    {
-        const int n_queued = (int)min(queue_count, (unsigned int)q_cap);
+    if constexpr (!F64) {
+        const int n_queued = n_noted;
         double magic_lane = 0.0;  // lane f: of feature f; lane d: of the weights
         double magic_w64 = 0.0;   // d = 64 leaves no lane for the weights: lane 0 adds them as well
         if (UPDATE && n_queued > 0) {
@@ -1185,50 +1436,8 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             const uint32_t* entry = queue + e * QW;
             const uint32_t sample = entry[Q_INDEX];
             if (sample == QUEUE_FREE) continue;  // reserved by a column that was redone instead
-            const float* xe = reinterpret_cast<const float*>(entry);
-            float bs = neg_inf;
-            int bc = 0x7fffffff;
-            // Two centroids per lane and pass, sixteen features at a time whose LDS reads are in
-            // flight together (past d the last row is read again and the sum left alone); the
-            // additions stay in feature order.
-            for (int c = lane; c < kp; c += 128) {
-                const bool two = c + 64 < kp;  // wave-uniform: kp is a multiple of 64
-                const int c1 = two ? c + 64 : c;
-                const float* col0 = ct + c;
-                const float* col1 = ct + c1;
-                float s0 = -hx[c], s1 = -hx[c1];
-                for (int f0 = 0; f0 < d; f0 += 16) {
-                    float xv[16], a0[16], a1[16];
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int f = f0 + i < d ? f0 + i : d - 1;  // wave-uniform
-                        xv[i] = xe[f];
-                        a0[i] = col0[f * kp];
-                        a1[i] = col1[f * kp];
-                    }
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const float t0 = fmaf(xv[i], a0[i], s0), t1 = fmaf(xv[i], a1[i], s1);
-                        s0 = f0 + i < d ? t0 : s0;
-                        s1 = f0 + i < d ? t1 : s1;
-                    }
-                }
-                if (s0 > bs) {
-                    bs = s0;
-                    bc = c;
-                }
-                if (two && s1 > bs) {
-                    bs = s1;
-                    bc = c1;
-                }
-            }
-            // The wave's best: the largest score (in an order-preserving integer form), then the
-            // lowest index among the lanes that hold it.
-            const unsigned int sb = __float_as_uint(bs);
-            const unsigned int ordered = sb ^ ((sb >> 31) ? 0xffffffffu : 0x80000000u);
-            const unsigned int top = wave_umax(ordered);
-            bc = (int)~wave_umax(ordered == top ? (unsigned int)~bc : 0u);
-            if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
+            const TX* xe = reinterpret_cast<const TX*>(entry);
+            const int bc = evaluate_sample([&](const int f) __attribute__((always_inline)) { return xe[f]; });
             if (lane == 0) {
                 labels[sample] = (uint32_t)bc;
                 if (UPDATE) changed += entry[Q_PREV] != (uint32_t)bc ? 1u : 0u;
@@ -1236,18 +1445,18 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             if constexpr (INERTIA) {
                 float sq = 0.0f;
                 if (lane < d) {
-                    const float diff = xe[lane] - ct[lane * kp + bc];
+                    const float diff = (float)xe[lane] - ct[lane * kp + bc];
                     sq = diff * diff;
                 }
                 sq = kmx_wave_sum<float>(sq);
-                if (lane == 0) inertia_lane += (double)(sq * __uint_as_float(entry[Q_WEIGHT]));
+                if (lane == 0) inertia_lane += (double)(sq * (float)xe[NKF]);
             }
             if (UPDATE) {
                 // lane f adds feature f, lane d the weight: the same fixed-point terms as above;
                 // when the sums are only corrected, a sample that stays in its cluster adds
                 // nothing and one that moves is taken off the old cluster
                 const uint32_t prev = entry[Q_PREV];
-                const double wq = (double)__uint_as_float(entry[Q_WEIGHT]);
+                const double wq = (double)xe[NKF];  // (the weight follows the features)
                 if (lane <= d && (full_mode || prev != (uint32_t)bc)) {
                     const double term = lane < d ? fma((double)xe[lane], wq, magic_lane) : wq + magic_lane;
                     const unsigned long long fixed = to_fixed_q(term, magic_lane);
@@ -1259,6 +1468,83 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
                     const unsigned long long fixed = to_fixed_q(wq + magic_w64, magic_w64);
                     atomicAdd(acc + bc * acc_stride + d_even, fixed);
                     if (!full_mode) atomicSub(acc + prev * (uint32_t)acc_stride + d_even, fixed);
+                }
+            }
+        }
+    } else {
+        // fp64 inputs: sixteen noted samples at a time on the fp64 matrix cores
+        // (v_mfma_f64_16x16x4_f64: A = 16 centroids x 4 features, lane l: centroid l % 16, feature
+        // l / 16; B = 4 features x 16 samples, lane l: feature l / 16, sample l % 16; D: lane l holds
+        // rows l / 16 + 4 r, r = 0..3, of column l % 16).  Lane (g, m) = (l / 16, l % 16) gathers
+        // features 4 s + g of sample m straight from memory, all of them in flight together, and
+        // afterwards adds the same values to the sums of the sample's cluster.
+        typedef double v4d __attribute__((ext_vector_type(4)));
+        constexpr int NS = 4 * NK;  // K steps of four features
+        const int g4 = lane >> 4, m16 = lane & 15;
+        const int n_groups = (n_noted + 15) >> 4;
+        for (int gq = wave; gq < n_groups; gq += WAVES) {
+            const int slot = 16 * gq + m16;
+            const uint32_t sample = slot < n_noted ? qlist[slot] : QUEUE_FREE;
+            const bool valid = sample != QUEUE_FREE;  // (free: reserved and never written)
+            const size_t at = valid ? (size_t)sample : 0;
+            double xk[NS];
+#pragma unroll
+            for (int s4 = 0; s4 < NS; ++s4) {
+                const int f = 4 * s4 + g4;
+                xk[s4] = f < d ? (double)X_t[(size_t)f * n + at] : 0.0;
+            }
+            const double wv = UPDATE ? (double)sample_weight[at] : 1.0;
+            const uint32_t prev = UPDATE ? labels_prev[at] : 0u;
+            double bs = -kmx_inf<double>();
+            int bc = 0x7fffffff;
+            for (int cb = 0; cb < (kp >> 4); ++cb) {
+                const TX* hp = hxx + 16 * cb + g4;
+                v4d a = {-(double)hp[0], -(double)hp[4], -(double)hp[8], -(double)hp[12]};
+#pragma unroll
+                for (int s4 = 0; s4 < NS; ++s4) {
+                    const int f = 4 * s4 + g4;
+                    const double af = f < d ? (double)ctx[f * kp + 16 * cb + m16] : 0.0;
+                    a = __builtin_amdgcn_mfma_f64_16x16x4f64(af, xk[s4], a, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)  // increasing centroid index inside the lane; strict
+                    if (a[r] > bs) {
+                        bs = a[r];
+                        bc = 16 * cb + g4 + 4 * r;
+                    }
+            }
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const double ob = __shfl_xor(bs, off, 64);
+                const int oc = __shfl_xor(bc, off, 64);
+                if (ob > bs || (ob == bs && oc < bc)) {
+                    bs = ob;
+                    bc = oc;
+                }
+            }
+            if (bc == 0x7fffffff) bc = 0;  // no score compares: the reference's running arg-min keeps 0
+            if (valid && g4 == 0) {
+                labels[sample] = (uint32_t)bc;
+                if (UPDATE) changed += prev != (uint32_t)bc ? 1u : 0u;
+            }
+            if (UPDATE && valid && (full_mode || prev != (uint32_t)bc)) {
+                // the same fixed-point terms as a tile adds; when the sums are only corrected, a
+                // sample that moves is taken off the old cluster
+#pragma unroll
+                for (int s4 = 0; s4 < NS; ++s4) {
+                    const int f = 4 * s4 + g4;
+                    if (f < d) {
+                        const double magic = fix_magic(q_lds[f]);
+                        const unsigned long long term = to_fixed_q(fma(xk[s4], wv, magic), magic);
+                        atomicAdd(acc + bc * acc_stride + f, term);
+                        if (!full_mode) atomicSub(acc + prev * (uint32_t)acc_stride + f, term);
+                    }
+                }
+                if (g4 == 0) {
+                    const double magic_w = fix_magic(q_lds[d]);
+                    const unsigned long long term = to_fixed_q(wv + magic_w, magic_w);
+                    atomicAdd(acc + bc * acc_stride + d_even, term);
+                    if (!full_mode) atomicSub(acc + prev * (uint32_t)acc_stride + d_even, term);
                 }
             }
         }
@@ -1309,7 +1595,7 @@ __global__ __launch_bounds__(64 * scr_waves(NK), NK == 1 ? scr_waves(1) / 4 : 2)
             __syncthreads();
             if (is_last != 0u) {
                 // (the accumulators are flushed: their LDS holds the (d + 1) k sums as floats)
-                lloyd_small_finalize_body<float, true, true>(gsum, q_exp, tail, reinterpret_cast<float*>(smem_raw));
+                lloyd_small_finalize_body<TX, true, true>(gsum, q_exp, tail, reinterpret_cast<TX*>(smem_raw));
                 if (threadIdx.x == 0) status->ticket = 0u;
             }
         }
@@ -1474,10 +1760,10 @@ __global__ __launch_bounds__(64) void screen_scores_kernel(
 // whose accumulators and operands do not fit the half of a compute unit's LDS that a workgroup
 // of the two-step kernel gets: the three-step kernel is one workgroup with all of it (its third
 // step then holds no feature: zero operands, exact), which keeps such shapes off the wide path.
-static int screen_k_steps(int d, int k, bool update) {
+static int screen_k_steps(int d, int k, bool update, int esize = 4) {
     const int nk = (d + 15) / 16;
-    if (nk == 2 && screen_lds(d, k, 2, update).off_queue > scr_lds_max(2) &&
-        screen_lds(d, k, 3, update).off_queue <= scr_lds_max(3))
+    if (nk == 2 && screen_lds(d, k, 2, update, esize).off_queue > scr_lds_max(2) &&
+        screen_lds(d, k, 3, update, esize).off_queue <= scr_lds_max(3))
         return 3;
     return nk;
 }
@@ -1488,6 +1774,21 @@ bool kmx_mfma_screen_fits(int64_t n, int d, int k) {
     if (d < 1 || d > 64 || k < 16 || n >= ((int64_t)1 << 29)) return false;
     const int nk = screen_k_steps(d, k, true);
     return screen_lds(d, k, nk, true).off_queue <= scr_lds_max(nk);
+}
+
+// The same step on fp64 inputs: the centroids in LDS are fp64, and the list of noted samples
+// takes the place of the queue.
+static bool screen_fits_f64(int64_t n, int d, int k) {
+    if (d < 1 || d > 64 || k < 16 || n >= ((int64_t)1 << 29)) return false;
+    const int nk = screen_k_steps(d, k, true, 8);
+    return screen_lds(d, k, nk, true, 8).off_queue <= scr_lds_max(nk);
+}
+
+// Left to the library it is used wherever it fits (measured at 2e6 x 32, 64 clusters: 2.0x the
+// fp64 matrix-core step); KMX_FLAG_LABELS_F32 - "no fp16 screen" - switches it off.
+bool kmx_mfma_screen_f64_supported(int64_t n, int d, int k, uint32_t flags) {
+    if ((flags & KMX_FLAG_LABELS_MASK) == KMX_FLAG_LABELS_F32) return false;
+    return screen_fits_f64(n, d, k);
 }
 
 // The labels-only kernel needs no accumulators: shapes whose fused step does not fit the LDS
@@ -1512,15 +1813,19 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags) {
 }
 
 namespace {
-template <bool UPDATE, bool INERTIA = false>
+template <bool UPDATE, bool INERTIA = false, typename TX = float>
 int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, const uint32_t* labels_prev,
                       uint32_t* labels, kmx_lloyd_status* status, const unsigned int* absmax,
                       const int* q_exp, unsigned long long* gsum, uint32_t* uncertain_count,
                       const float* norms, int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream,
                       double* inertia_partial = nullptr, int* grid_out = nullptr,
-                      const LloydTail<float>* tail = nullptr) {
-    if (!(UPDATE ? kmx_mfma_screen_fits(n, d, k) : kmx_mfma_screen_labels_fits(n, d, k))) return KMX_ERR_UNSUPPORTED;
-    const int nk = screen_k_steps(d, k, UPDATE);
+                      const LloydTail<TX>* tail = nullptr) {
+    constexpr int ES = (int)sizeof(TX);
+    static_assert(ES == 4 || (UPDATE && !INERTIA), "fp64 inputs: the fused step only");
+    if (!(ES == 8 ? screen_fits_f64(n, d, k)
+                  : (UPDATE ? kmx_mfma_screen_fits(n, d, k) : kmx_mfma_screen_labels_fits(n, d, k))))
+        return KMX_ERR_UNSUPPORTED;
+    const int nk = screen_k_steps(d, k, UPDATE, ES);
     const int waves = scr_waves(nk);
     const int64_t n_wtiles = kmx_cdiv(n, 64);
     int64_t grid = kmx_cdiv(n_wtiles, waves);
@@ -1530,25 +1835,25 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
     if (grid < 1) grid = 1;
     auto aligned16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     // (the fast path addresses a lane's rows with 32-bit byte offsets from the tile's address in row 0)
-    const int vec_ok = ((uint64_t)d * (uint64_t)n * 4u < ((uint64_t)1 << 32)) && (n % 4 == 0) && aligned16(X_t) &&
+    const int vec_ok = ((uint64_t)d * (uint64_t)n * (uint64_t)ES < ((uint64_t)1 << 32)) && (n % 4 == 0) && aligned16(X_t) &&
                        aligned16(labels) && aligned16(w) &&
                        aligned16(labels_prev);
-    const size_t lds = screen_lds(d, k, nk, UPDATE).total;
+    const size_t lds = screen_lds(d, k, nk, UPDATE, ES).total;
     // -0.5||c||^2 in a spare feature slot of the last K step whenever there is one
     const bool hk = d % 16 != 0;
 #define KMX_SCR_LAUNCH(NK_, HK_)                                                                            \
     do {                                                                                                    \
         if (lds > 64 * 1024) {                                                                              \
             const hipError_t e = hipFuncSetAttribute(                                                       \
-                reinterpret_cast<const void*>(&lloyd_screen_kernel<NK_, UPDATE, HK_, INERTIA>),             \
+                reinterpret_cast<const void*>(&lloyd_screen_kernel<TX, NK_, UPDATE, HK_, INERTIA>),         \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                      \
             if (e != hipSuccess) return (int32_t)e;                                                         \
         }                                                                                                   \
-        hipLaunchKernelGGL((lloyd_screen_kernel<NK_, UPDATE, HK_, INERTIA>), dim3((unsigned)grid),          \
-                           dim3(64 * scr_waves(NK_)), lds, stream, (const float*)X_t, (const float*)w,      \
-                           (const float*)centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,     \
+        hipLaunchKernelGGL((lloyd_screen_kernel<TX, NK_, UPDATE, HK_, INERTIA>), dim3((unsigned)grid),      \
+                           dim3(64 * scr_waves(NK_)), lds, stream, (const TX*)X_t, (const TX*)w,            \
+                           (const TX*)centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,        \
                            uncertain_count, norms, n, d, k, vec_ok, inertia_partial,                        \
-                           tail ? *tail : LloydTail<float>(), tail ? 1 : 0);                                \
+                           tail ? *tail : LloydTail<TX>(), tail ? 1 : 0);                                   \
     } while (0)
     if (nk == 1) {
         if (hk) KMX_SCR_LAUNCH(1, true); else KMX_SCR_LAUNCH(1, false);
@@ -1580,6 +1885,18 @@ int32_t kmx_lloyd_step_mfma_screen(const void* X_t, const void* w, const void* c
                                    int k, int wgs_per_cu, hipStream_t stream, const LloydTail<float>* tail) {
     return launch_screen<true>(X_t, w, centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,
                                uncertain_count, norms, n, d, k, wgs_per_cu, stream, nullptr, nullptr, tail);
+}
+
+// The same on fp64 inputs (X_t, w, centroids_t and the tail's arrays are fp64; norms stay fp32).
+int32_t kmx_lloyd_step_mfma_screen_f64(const void* X_t, const void* w, const void* centroids_t,
+                                       const uint32_t* labels_prev, uint32_t* labels,
+                                       kmx_lloyd_status* status, const unsigned int* absmax,
+                                       const int* q_exp, unsigned long long* gsum,
+                                       uint32_t* uncertain_count, const float* norms, int64_t n, int d,
+                                       int k, int wgs_per_cu, hipStream_t stream, const LloydTail<double>* tail) {
+    return launch_screen<true, false, double>(X_t, w, centroids_t, labels_prev, labels, status, absmax, q_exp, gsum,
+                                              uncertain_count, norms, n, d, k, wgs_per_cu, stream, nullptr, nullptr,
+                                              tail);
 }
 
 // Labels only, screened the same way: nothing but X and the centroids is needed (the scale comes
@@ -1638,22 +1955,28 @@ int32_t kmx_screen_scores_impl(const float* X_t, const float* centroids_t, float
 namespace {
 // ||x_i|| in fp32, features in order; one thread per sample (consecutive threads, consecutive
 // addresses in every feature row).
-__global__ __launch_bounds__(256) void sample_norms_kernel(const float* __restrict__ X_t,
+// (fp64 inputs: rounded to fp32 first, as the screen sees them)
+template <typename TX>
+__global__ __launch_bounds__(256) void sample_norms_kernel(const TX* __restrict__ X_t,
                                                            float* __restrict__ norms, int64_t n, int d) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     float sq = 0.0f;
 #pragma unroll 8
     for (int f = 0; f < d; ++f) {
-        const float v = X_t[(size_t)f * n + i];
+        const float v = (float)X_t[(size_t)f * n + i];
         sq = fmaf(v, v, sq);
     }
     norms[i] = sqrtf(sq);
 }
 }  // namespace
 
-int32_t kmx_sample_norms(const float* X_t, float* norms, int64_t n, int d, hipStream_t stream) {
-    hipLaunchKernelGGL(sample_norms_kernel, dim3((unsigned)kmx_cdiv(n, 256)), dim3(256), 0, stream, X_t, norms, n, d);
+int32_t kmx_sample_norms(const void* X_t, float* norms, int64_t n, int d, int dtype, hipStream_t stream) {
+    const dim3 grid((unsigned)kmx_cdiv(n, 256));
+    if (dtype == KMX_F64)
+        hipLaunchKernelGGL(sample_norms_kernel<double>, grid, dim3(256), 0, stream, (const double*)X_t, norms, n, d);
+    else
+        hipLaunchKernelGGL(sample_norms_kernel<float>, grid, dim3(256), 0, stream, (const float*)X_t, norms, n, d);
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

@@ -61,7 +61,13 @@ def test_workspace_queries():
     assert 0 < small < 64 << 20
     # the screened fp32 step keeps ||x_i|| per sample: 4 bytes per sample
     assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 0, 0) - small - 4 * 4_900_000) < 256
-    assert lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0) == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0)
+    # and so does the screened fp64 step; the all-fp64 matrix-core step (screen switched off) keeps nothing per sample
+    assert abs(lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0)
+               - lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0) - 4 * 4_900_000) < 256
+    assert (lib.kmx_lloyd_workspace_bytes(5_000_000, 14, 127, 1, 0x10)
+            == lib.kmx_lloyd_workspace_bytes(100_000, 14, 127, 1, 0x10))
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0) == 71
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0x10) == 51
     # sums beyond LDS off the wide path: sample order and ranks (2 n words) + one copy of the sums;
     # the screened tiled product (on request) adds its list (n words)
     assert 8_000_000 + 4 * 301 * 1024 < lib.kmx_lloyd_workspace_bytes(1_000_000, 300, 1024, 0, 0) < (16 << 20)
@@ -74,7 +80,9 @@ def test_workspace_queries():
                                      (1_000_000, 100, 100, 1): 1, (5_000_000, 14, 127, 0): 0,
                                      (1_000_000, 14, 700, 0): 0, (2_000_000, 32, 64, 1): 0}.items():
         assert lib.kmx_lloyd_plan_reads_rowmajor(_capi.lloyd_plan(n_, d_, k_, dt_, 0)) == reads, (n_, d_, k_, dt_)
-    assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0) == 51
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0) == 71
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 48, 64, 1, 0x10) == 51
+    assert lib.kmx_lloyd_kernel_variant(1_000_000, 64, 100, 1, 0) == 51  # (both copies of the centroids: beyond the LDS)
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 32, 500, 1, 0) == 53
     assert lib.kmx_lloyd_workspace_bytes(0, 14, 127, 0, 0) == 0
     assert lib.kmx_lloyd_workspace_bytes(10, 14, 127, 7, 0) == 0
@@ -105,7 +113,8 @@ def test_kernel_variant_selection():
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 4, 127, 0, 0) == 31    # too few features for the screen to pay
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 64, 0, 0) == 61
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 8, 32, 0, 0) == 31
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0) == 51    # fp64: matrix cores + LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0) == 71    # fp64: fp16-screened labels, fp64 sums in LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 64, 1, 0x10) == 51  # screen off: fp64 matrix cores + LDS
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 64, 128, 1, 0) == 51    # with all of a compute unit's LDS
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 500, 1, 0) == 53    # labels on the matrix cores, bucketed sums
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 32, 1024, 1, 0) == 63   # centroids too big for LDS as well: tiled product

@@ -84,10 +84,19 @@ def _small_configs():
         "G32u": lambda: dict(_blob_config(5_000, 70, 20, np.float32, 45), flags=0x20, variant=63),
         # fp64 on the matrix cores beyond 32 features (no rows in flight for the next tile) and
         # with accumulators that need most of a compute unit's LDS
-        "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=51),
+        # (fp64 inputs up to 64 features: labels screened on the fp16 matrix cores, the rest in
+        # fp64 - variant 71; with the screen switched off the all-fp64 matrix-core step, 51)
+        "F64e": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), variant=71),
+        # (64 features x 100 clusters: the fp64 and fp32 copies of the centroids do not both fit the LDS)
         "F64f": lambda: dict(_blob_config(8_000, 64, 100, np.float64, 22), variant=51),
         "F64g": lambda: dict(_blob_config(20_000, 32, 300, np.float64, 23), variant=51),
-        "F64h": lambda: dict(_blob_config(6_001, 61, 33, np.float64, 24), variant=51),
+        "F64h": lambda: dict(_blob_config(6_001, 61, 33, np.float64, 24), variant=71),
+        "F64e1": lambda: dict(_blob_config(20_003, 48, 64, np.float64, 21), flags=0x10, variant=51),
+        "F64h1": lambda: dict(_blob_config(6_001, 61, 33, np.float64, 24), flags=0x10, variant=51),
+        "C5f": lambda: dict(datasets.config5(n=100_000), flags=0x10, variant=51),
+        # fp64 screened step, one K step of 16 features with and without a spare slot
+        "F64i": lambda: dict(_blob_config(30_000, 16, 127, np.float64, 46), variant=71),
+        "F64j": lambda: dict(_blob_config(30_004, 14, 127, np.float64, 47), variant=71),
     }
 
 
@@ -113,7 +122,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u"])
+                                  "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -172,7 +181,7 @@ def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     print(f"{name}: near-tie label differences: {n_ties}")
 
 
-@pytest.mark.parametrize("name", ["C2", "M32a", "M32b", "C3", "C3s", "C5", "F64d", "B64a", "B64d", "B64e", "odd", "S64a"])
+@pytest.mark.parametrize("name", ["C2", "M32a", "M32b", "C3", "C3s", "C5", "C5f", "F64j", "F64d", "B64a", "B64d", "B64e", "odd", "S64a"])
 def test_duplicate_and_identical_centroids_on_every_kernel_family(cuda, name):
     """Exact ties: with two centroids duplicated no sample may take the copy with the higher
     index, with all centroids identical every label is 0 (the reference's strict '<' in
@@ -218,7 +227,7 @@ def test_duplicate_and_identical_centroids_on_every_kernel_family(cuda, name):
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3s", "C3w", "odd", "F64a", "F64b", "M32a", "M32b", "C3k", "M32d", "M32e", "F64d",
-                                  "F64e", "F64f", "F64g", "F64h", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "G32s", "G32t"])
+                                  "F64e", "F64f", "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "G32s", "G32t"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
@@ -318,7 +327,7 @@ def _converging_configs():
         # configs[1] (weighted, unequal blobs, one cluster empties and is relocated) and
         # configs[4] (fp64, sixteen clusters that empty on the first iteration) on fewer samples
         "C2_30k": (lambda: datasets.config2(n=30_000), 61, 38),
-        "C5_100k": (lambda: datasets.config5(n=100_000), 51, 67),
+        "C5_100k": (lambda: datasets.config5(n=100_000), 71, 67),
         # screened labels with the sums taken straight from the labels, and with sums per bucket
         "direct": (lambda: _blob_config(20_000, 14, 700, np.float32, 20), 63, 8),
         "bucket": (lambda: _blob_config(20_000, 32, 500, np.float64, 19), 53, 8),

@@ -40,7 +40,7 @@ def _one_iteration(X, w, init, cuda, flags=SCREEN):
     labels = torch.full((n,), -1, dtype=torch.int32, device=cuda)
     sizes = torch.empty(k, dtype=X_t.dtype, device=cuda)
     empty = torch.empty(k, dtype=torch.int32, device=cuda)
-    plan = _capi.lloyd_plan(n, d, k, 0, flags)
+    plan = _capi.lloyd_plan(n, d, k, _capi.dtype_code(X.dtype), flags)
     ws_bytes = plan.workspace_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
     stream = _capi.current_stream()
@@ -62,12 +62,12 @@ def _check_against_oracle(X, w, init, labels, c_out, sizes, status):
     assert labels.min() >= 0 and labels.max() < k
     assert_labels_match(labels, ok.assign_labels(X, init), X, init)
     sums, ref_sizes = ok.weighted_sums(X, w, labels, k)
-    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-5)
+    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-5 if X.dtype == np.float32 else 1e-12)
     assert status.n_empty == int(np.count_nonzero(ref_sizes == 0))
     if status.n_empty == 0:
-        assert_centers_close(c_out, sums / ref_sizes[:, None], np.float32)
+        assert_centers_close(c_out, sums / ref_sizes[:, None], X.dtype)
     else:
-        assert_centers_close(c_out, sums, np.float32)
+        assert_centers_close(c_out, sums, X.dtype)
 
 
 def _blobs(n, d, k, seed, offset=0.0, scale=1.0):
@@ -771,3 +771,117 @@ def test_tiled_product_screened_on_request(cuda, shape):
     big = (X * 1000.0).astype(np.float32)
     labels = _labels_only(big, init, cuda, roomy=True, flags=SCREEN)
     assert_labels_match(labels, ok.assign_labels(big, init), big, init)
+
+
+# ------------------------------------------------------------------------------------------
+# fp64 inputs: the same screen on the inputs rounded to fp32 (kernel variant 71); the samples it
+# cannot certify are evaluated on the fp64 matrix cores, the sums are taken from the fp64 inputs
+
+
+def _blobs64(n, d, k, seed, spread=1.0):
+    rng = np.random.default_rng(seed)
+    centers = rng.uniform(-10, 10, (k, d))
+    X = centers[rng.integers(0, k, n)] + spread * rng.standard_normal((n, d))
+    init = X[rng.choice(n, k, replace=False)].copy()
+    w = rng.uniform(0.5, 1.5, n)
+    return X, w, init
+
+
+@pytest.mark.parametrize("shape", [(20_000, 32, 64), (10_003, 9, 45), (4_096, 16, 16), (3_001, 17, 40), (777, 1, 20),
+                                   (64, 31, 16), (6_000, 33, 16), (6_000, 48, 64), (5_003, 64, 64), (7_001, 63, 20),
+                                   (20_000, 16, 256), (9_000, 14, 300)])
+def test_fp64_screened_step_matches_oracle(cuda, shape):
+    n, d, k = shape
+    X, w, init = _blobs64(n, d, k, seed=n + d)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=0)
+    assert variant == 71
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+    assert rechecked <= 8 + n // 10
+
+
+def test_fp64_screen_switched_off_by_flag(cuda):
+    X, w, init = _blobs64(20_000, 32, 64, seed=3)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=ALL_F32)
+    assert variant == 51 and rechecked == 0
+    _check_against_oracle(X, w, init, labels, c_out, sizes, status)
+
+
+@pytest.mark.parametrize("d", [14, 32, 40, 64])
+def test_fp64_duplicate_and_identical_centroids(cuda, d):
+    X, w, init = _blobs64(20_000, d, 64, seed=41)
+    dup = init.copy()
+    dup[40] = dup[3]
+    dup[63] = dup[17]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, dup, cuda, flags=0)
+    assert variant == 71
+    assert not np.any(labels == 40) and not np.any(labels == 63)
+    ref = ok.assign_labels(X, dup)
+    assert_labels_match(labels, ref, X, dup)
+    assert rechecked >= int(np.count_nonzero((ref == 3) | (ref == 17)))
+    same = init.copy()
+    same[:] = same[0]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, same, cuda, flags=0)
+    assert np.all(labels == 0) and rechecked == X.shape[0] and status.n_empty == 63
+
+
+def test_fp64_more_uncertain_samples_than_the_list_holds(cuda):
+    """One workgroup per compute unit and identical centroids: every sample is uncertain, 8192 per
+    workgroup, twice what its list of noted samples holds; the rest is evaluated where it turns
+    up.  Labels, sums and sizes must not depend on the route."""
+    rng = np.random.default_rng(43)
+    n, d, k = 1 << 21, 4, 16
+    # (off the origin: the 64-bit fixed-point sums resolve 2^-61 of n max|w| max|x|, which is 1e-12 of
+    # a cluster's sum unless that sum all but cancels)
+    X = 3.0 + rng.standard_normal((n, d))
+    w = rng.uniform(0.5, 1.5, n)
+    init = np.tile(X[5], (k, 1))
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=1 << 8)
+    assert variant == 71
+    assert np.all(labels == 0) and rechecked == n
+    assert status.n_empty == k - 1
+    sums, ref_sizes = ok.weighted_sums(X, w, labels, k)
+    np.testing.assert_allclose(sizes, ref_sizes, rtol=1e-12)
+    assert_centers_close(c_out, sums, np.float64)
+
+
+def test_fp64_initial_centroids_far_outside_the_data(cuda):
+    """A quarter of the initial centroids at +1e3 in every coordinate (as in the configuration with
+    forced empty clusters): they set the fp16 scale and have huge norms, and must cost neither the
+    other centroids' scores their precision nor the samples their certificate."""
+    X, w, init = _blobs64(60_000, 32, 64, seed=47, spread=0.5)
+    init[48:] = 1e3 + np.arange(16)[:, None]
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, init, cuda, flags=0)
+    assert variant == 71
+    assert labels.max() < 48 and status.n_empty >= 16
+    assert_labels_match(labels, ok.assign_labels(X, init), X, init)
+    assert rechecked <= X.shape[0] // 2
+
+
+@pytest.mark.parametrize("d,k", [(32, 64), (14, 20), (48, 33)])
+def test_fp64_certificate_passes_no_label_that_fp64_would_not_give(cuda, d, k):
+    """Samples at distances from a bisector spread over twelve decades (gaps between the two best
+    squared distances from 1e-14 to 1e-2 of their size): whatever the screen certifies must be
+    the fp64 arg-min - labels may differ from an extended-precision evaluation only where fp64
+    itself cannot tell, far below anything fp32 or fp16 resolves."""
+    rng = np.random.default_rng(53 + d)
+    n = 40_000
+    C = rng.uniform(-10, 10, (k, d))
+    a = rng.integers(0, k, n)
+    b = (a + 1 + rng.integers(0, k - 1, n)) % k
+    mid = 0.5 * (C[a] + C[b])
+    axis = C[b] - C[a]
+    axis /= np.linalg.norm(axis, axis=1, keepdims=True)
+    ortho = 0.01 * rng.standard_normal((n, d))
+    ortho -= (ortho * axis).sum(axis=1, keepdims=True) * axis
+    offset = 10.0 ** rng.uniform(-14, -2, n) * rng.choice([-1.0, 1.0], n)
+    X = mid + ortho + offset[:, None] * axis * np.linalg.norm(C[b] - C[a], axis=1, keepdims=True)
+    w = np.ones(n)
+    labels, c_out, sizes, status, variant, rechecked = _one_iteration(X, w, C, cuda, flags=0)
+    assert variant == 71
+    XL, CL = X.astype(np.longdouble), C.astype(np.longdouble)
+    dist = ((XL[:, None, :] - CL[None, :, :]) ** 2).sum(axis=2)
+    ref = dist.argmin(axis=1)
+    bad = np.flatnonzero(labels != ref)
+    gap = (dist[bad, labels[bad]] - dist[bad, ref[bad]]) / dist[bad].max(axis=1)
+    assert np.all(gap <= 1e-14), f"{bad.size} labels differ, worst relative gap {gap.max():.3e}"
+    assert rechecked > n // 4  # (most of these samples cannot be certified)
