@@ -346,6 +346,58 @@ def gpu_lloyd_step_time(cfg, reps, consecutive=False, flags=0):
     return acc / reps, int(variant)
 
 
+def gpu_lloyd_later_step_time(cfg, start_iter, reps, flags=0):
+    """Mean ms of the fused step over iterations start_iter + 3 .. start_iter + 2 + reps of a run:
+    the driver's loop (relocation of empty clusters included) runs start_iter iterations from the
+    configuration's initial centroids, then the iterations are timed one by one through the C ABI
+    (the first two rebuild the sums, as after every re-initialisation, and are left out).  Also
+    returns the samples per iteration that the label screen could not certify."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd._capi import lib, ptr
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    dev = torch.device("cuda:0")
+    X, init, w, k = cfg["X"], cfg["init"], cfg["sample_weight"], cfg["k"]
+    n, d = X.shape
+    plan = _capi.lloyd_plan(n, d, k, _capi.dtype_code(X.dtype), flags)
+    X_rm = torch.as_tensor(X, device=dev)
+    X_t = X_rm.T.contiguous()
+    if lib.kmx_lloyd_plan_reads_rowmajor(plan) != 1:
+        X_rm = None
+    w_d = torch.as_tensor(w, device=dev)
+    c0 = torch.as_tensor(np.ascontiguousarray(init.T), device=dev)
+    cent = [drivers.lloyd(X_t, w_d, c0, max_iter=start_iter, tol=0.0, flags=flags)[2].clone(), None]
+    cent[1] = torch.empty_like(cent[0])
+    labels = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(2)]
+    sizes = torch.empty(k, dtype=X_t.dtype, device=dev)
+    empty = torch.empty(k, dtype=torch.int32, device=dev)
+    ws = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=dev)
+    stream = _capi.current_stream()
+    ms = (ctypes.c_float * 3)()
+    status = _capi.LloydStatus()
+    count = ctypes.c_uint32(0)
+    _capi.check(lib.kmx_lloyd_init(plan, ptr(ws), plan.workspace_bytes, ptr(X_t), ptr(w_d), ptr(cent[0]), 1000, 0.0,
+                                   stream), "init")
+    fused, uncertain = [], []
+    for it in range(reps + 2):
+        a, b = it % 2, (it + 1) % 2
+        _capi.check(lib.kmx_lloyd_iter_timed(plan, ptr(X_t), ptr(X_rm), ptr(w_d), ptr(cent[a]), ptr(cent[b]),
+                                             ptr(labels[a]), ptr(labels[b]), ptr(sizes), ptr(empty), ptr(ws),
+                                             plan.workspace_bytes, stream, ms), "iter_timed")
+        _capi.check(lib.kmx_lloyd_status_read(ptr(ws), status, stream), "status")
+        _capi.check(lib.kmx_lloyd_recheck_count(plan, ptr(ws), ctypes.byref(count), stream), "recheck")
+        if status.state != _capi.KMX_RUNNING:
+            break
+        if it >= 2:
+            fused.append(float(ms[0]))
+            uncertain.append(int(count.value))
+    if not fused:
+        raise RuntimeError("the run ended before an iteration could be timed")
+    return float(np.mean(fused)), int(np.mean(uncertain)), len(fused)
+
+
 def extra_configs():
     """Configs 3 (fp32, d=256, k=1024: matrix-core bound) and 5 (fp64, forced empty clusters)."""
     from sklearn_numba_dpex_amd import datasets
@@ -377,17 +429,31 @@ def extra_configs():
     t0 = time.time()
     c5 = datasets.config5()
     n, d = c5["X"].shape
-    kms, variant = gpu_lloyd_step_time(c5, 5)
+    kms, variant, wall_ms = gpu_lloyd_step_time(c5, 10, consecutive=True)
+    later_ms, later_uncertain, later_n = gpu_lloyd_later_step_time(c5, 4, 8)
+    # the same with the fp16 screen switched off: every product on the fp64 matrix cores
+    kms64, variant64, wall64_ms = gpu_lloyd_step_time(c5, 10, consecutive=True, flags=FLAG_LABELS_F32)
     flops = lloyd_flops(n, d, c5["k"])
     nbytes = lloyd_bytes(n, d, 8)
     out["config5"] = {
-        "workload": f"configs[4]: Lloyd n={n} d={d} k={c5['k']} fp64, first iteration (16 empty clusters)",
-        "kernel_variant": variant, "ms_per_iter": float(kms.sum()),
+        "workload": f"configs[4]: Lloyd n={n} d={d} k={c5['k']} fp64 (16 clusters that empty on the first iteration); "
+                    "ms_per_iter over iterations 6-15 of the driver's loop, kernel_ms of the first iteration "
+                    "(sums rebuilt from every sample), later_iterations: iterations 7-14 (sums corrected)",
+        "kernel_variant": variant, "ms_per_iter": wall_ms, "iters_per_sec": 1e3 / wall_ms,
+        "labels": "fp16 matrix-core screen on the rows rounded to fp32, certified per sample, fp64 matrix cores "
+                  "where not certified; sums from the fp64 rows",
         "kernel_ms": {"fused_step": float(kms[0]), "reduce": float(kms[1]), "finalize": float(kms[2])},
-        "fused_step_frac_of_fp64_peak": flops / (kms[0] * 1e-3) / 1e12 / 78.6,
+        "later_iterations": {"fused_step_ms": later_ms, "iterations": later_n,
+                             "samples_not_certified": later_uncertain,
+                             "fused_step_frac_of_hbm_peak": nbytes / (later_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "fused_step_frac_of_hbm_peak": nbytes / (kms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "all_fp64": {"switch": "KMX_FLAG_LABELS_F32", "kernel_variant": variant64, "ms_per_iter": wall64_ms,
+                     "fused_step_ms": float(kms64[0]),
+                     "fused_step_frac_of_fp64_peak": flops / (kms64[0] * 1e-3) / 1e12 / 78.6},
     }
-    log(f"[bench] config 5: {out['config5']['ms_per_iter']:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
+    log(f"[bench] config 5: {wall_ms:.3f} ms/iter (fused step: first iteration {kms[0]:.3f} ms, later {later_ms:.3f} ms, "
+        f"{later_uncertain} samples not certified); all fp64: {wall64_ms:.3f} ms/iter, fused step {kms64[0]:.3f} ms "
+        f"({time.time() - t0:.1f}s incl. data)")
     del c5
     out["other_shapes"] = other_shapes()
     return out

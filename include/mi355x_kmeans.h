@@ -86,7 +86,7 @@ typedef struct kmx_lloyd_status {
 #define KMX_FLAG_PATH_GEMM 0x4u        /* tiled matrix-core labels + bucketed sums (any shape) */
 #define KMX_FLAG_LABELS_MASK 0x00000030u
 #define KMX_FLAG_LABELS_AUTO 0x00u
-#define KMX_FLAG_LABELS_F32 0x10u      /* every product of the fp32 paths taken in fp32       */
+#define KMX_FLAG_LABELS_F32 0x10u      /* no fp16 screen: every product in the input type     */
 #define KMX_FLAG_LABELS_SCREEN 0x20u   /* fp16 screen + fp32 certificate wherever it fits (also the tiled product) */
 #define KMX_FLAG_WGS_PER_CU(x) (((uint32_t)(x) & 0xfu) << 8)  /* 1..8 workgroups per CU; 0: default */
 #define KMX_FLAG_COLS(x) (((uint32_t)(x) & 0x7u) << 12)       /* 2 | 4 sample columns per lane; 0: default */
@@ -156,7 +156,7 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
  *   labels_prev      IN   (n)     labels of the previous iteration: from the second iteration on
  *                                 exactly the array the previous kmx_lloyd_iter of this workspace
  *                                 wrote as `labels` (the callers ping-pong two arrays).  Besides
- *                                 the count of changed labels, variant 61 builds on it: once few
+ *                                 the count of changed labels, variants 61 and 71 build on it: once few
  *                                 labels change it no longer rebuilds its integer sums but moves
  *                                 every sample that changes cluster from the old sum to the new one
  *   labels           OUT  (n)
@@ -204,9 +204,9 @@ int32_t kmx_lloyd_finalize(const kmx_lloyd_plan* plan, const void* centroids_t,
 /* Copies the status to host memory and waits for it (the only synchronising call). */
 int32_t kmx_lloyd_status_read(const void* workspace, kmx_lloyd_status* status_host, void* stream);
 
-/* Kernel variant 61 only (fp32 labels screened on the fp16 matrix cores): number of samples
+/* Kernel variants 61 and 71 only (labels screened on the fp16 matrix cores): number of samples
  * whose label the screen of the last completed iteration could not certify and that were
- * evaluated in plain fp32 instead; 0 for the other variants.  Synchronises the stream.
+ * evaluated in the input type instead; 0 for the other variants.  Synchronises the stream.
  * It has no counterpart in the reference (diagnostics). */
 int32_t kmx_lloyd_recheck_count(const kmx_lloyd_plan* plan, const void* workspace,
                                 uint32_t* count_host, void* stream);
@@ -232,7 +232,9 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
  * fp32 and fp64); accumulation 1 = workgroup-private LDS accumulators, 2 = global sums,
  * 3 = labels only, then sums by a kernel of their own (per bucket of samples sorted by label,
  * or, fp32, straight from the labels into fixed-point accumulators in LDS where those of every
- * cluster fit).  61 is path 3 with the labels screened on the fp16 matrix cores. */
+ * cluster fit).  61 is path 3 with the labels screened on the fp16 matrix cores; 71 is the same
+ * step on fp64 inputs (rows rounded to fp32 for the screen, the samples it cannot certify on the
+ * fp64 matrix cores, sums from the fp64 rows), chosen over 51 wherever its operands fit the LDS. */
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* 1 when the plan's kernels read the row-major copy of X that kmx_lloyd_iter takes as

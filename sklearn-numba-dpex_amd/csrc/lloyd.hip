@@ -609,6 +609,7 @@ static int lloyd_stream_samples_per_thread(int64_t n, int dtype) {
 // Workgroups of a vector-ALU fused step (also the number of partial slots it fills).
 int lloyd_fused_grid(const LloydLayout& L, int64_t n, int d, int dtype) {
     if (L.variant == KMX_VARIANT_MFMA_F64) return kmx_mfma_f64_grid(n, d, L.wgs_per_cu, L.cols, L.partial_slots());
+    if (L.variant == KMX_VARIANT_FEWK) return kmx_fewk_grid(n, d, L.k_for_gsum, L.wgs_per_cu);
     const int r = (L.variant == KMX_VARIANT_REGISTER) ? lloyd_reg_samples_per_thread(d, dtype)
                                                       : lloyd_stream_samples_per_thread(n, dtype);
     const int64_t tiles = kmx_cdiv(n, 256 * (int64_t)r);
@@ -644,7 +645,8 @@ template <typename T, int ACC>
 int32_t launch_fused(const LloydLayout& L, const void* X_t, const void* w, const void* centroids_t,
                   const T* cpack, const T* half_norms, const uint32_t* labels_prev,
                   uint32_t* labels, T* partial, kmx_lloyd_status* status, int64_t n, int d, int k,
-                  hipStream_t stream, const unsigned int* screen_absmax = nullptr, char* screen_area = nullptr) {
+                  hipStream_t stream, const unsigned int* screen_absmax = nullptr, char* screen_area = nullptr,
+                  const void* X_rowmajor = nullptr) {
     const int grid = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     if (L.variant == KMX_VARIANT_GEMM) {
         if (sizeof(T) == 4 && L.screen_labels)
@@ -747,7 +749,7 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
     } else if (L.acc_mode == ACC_LDS) {
         const int32_t rc_step =
             launch_fused<T, ACC_LDS>(L, X_t, w, centroids_t, cpack, half_norms, labels_prev, labels,
-                                     partial, status, n, d, k, stream);
+                                     partial, status, n, d, k, stream, nullptr, nullptr, X_rowmajor);
         if (rc_step != KMX_OK) return rc_step;
         n_partials_used = lloyd_fused_grid(L, n, d, sizeof(T) == 8 ? KMX_F64 : KMX_F32);
     } else {
@@ -930,7 +932,7 @@ int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype,
 int32_t kmx_lloyd_plan_reads_rowmajor(const kmx_lloyd_plan* plan) {
     KMX_REQUIRE_PLAN(plan);
     const LloydLayout L = lloyd_layout(plan->n, plan->d, plan->k, plan->dtype, plan->flags);
-    if (L.variant == KMX_VARIANT_MFMA_WIDE) return 1;
+    if (L.variant == KMX_VARIANT_MFMA_WIDE || L.variant == KMX_VARIANT_FEWK) return 1;
     return (L.acc_mode == KMX_ACC_BUCKET && !L.direct_sums) ? 1 : 0;
 }
 
@@ -962,7 +964,7 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
                            (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
     KMX_LAUNCH_CHECK();
     if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen || L.direct_sums ||
-        L.screen64) {
+        L.screen64 || L.variant == KMX_VARIANT_FEWK) {
         // (for the screened tiled product: max|x| per feature, from which its scale is taken)
         const int32_t rc = kmx_lloyd_mfma_prepare(L, X_t, sample_weight, ws, n, d, dtype, stream);
         if (rc != KMX_OK) return rc;
@@ -1019,6 +1021,10 @@ static int32_t lloyd_iter_dispatch(const kmx_lloyd_plan* plan, const void* X_t, 
             return kmx_lloyd_iter_mfma_f32(L, X_t, sample_weight, centroids_t, new_centroids_t,
                                            labels_prev, labels, cluster_sizes, empty_clusters,
                                            (char*)workspace, n, d, k, stream, events);
+        if (L.variant == KMX_VARIANT_FEWK)
+            return kmx_lloyd_iter_fewk(L, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t, labels_prev,
+                                       labels, cluster_sizes, empty_clusters, (char*)workspace, n, d, k, stream,
+                                       events);
         return lloyd_iter_impl<float>(L, X_t, X_rowmajor, sample_weight, centroids_t, new_centroids_t,
                                       labels_prev, labels, cluster_sizes, empty_clusters,
                                       (char*)workspace, n, d, k, stream, events);

@@ -1,0 +1,576 @@
+// fp32 fused Lloyd step for FEW clusters (k <= 16) on WIDE samples (64 < d <= 1216), reading X
+// once per iteration.
+//
+// Replaces, for these shapes, the kernel pair fused_lloyd_single_step
+// (sklearn_numba_dpex/kmeans/kernels/lloyd_single_step.py:35-424) + the reduction of the
+// privatised sums (kmeans/drivers.py:301-312); the reduction over the workgroups' partial sums
+// and the finalisation stay with lloyd.hip.
+//
+// With few clusters neither the labels nor the sums cost much arithmetic; what costs is reading
+// X twice (once for the labels, once more for the sums once the labels are known), which the
+// streaming vector-ALU step does, or sorting the samples by label first, which the bucketed sums
+// do.  Here a workgroup keeps a tile of S samples x all features in LDS and uses it twice:
+//
+//   * labels: scores(16 clusters x 16 samples) = C (16 x d) X_tile (d x 16) - 0.5||c||^2 with
+//     v_mfma_f32_16x16x4_f32 (A: lane l = cluster l % 16, feature l / 16; B: lane l = feature
+//     l / 16, sample l % 16; D: lane l holds clusters 4 (l / 16) + r of sample l % 16).  Each of
+//     the four waves takes a quarter of the features, whose centroid values it holds in
+//     registers for the whole kernel, and the four partial score tiles are added in wave order
+//     by one thread per sample (strict '>' in increasing cluster order: the lowest index wins).
+//   * sums: sums(16 clusters x 16 features) += M (16 clusters x 4 samples) X_tile^T (4 samples x
+//     16 features), M = w_i where sample i carries the row's label and 0 elsewhere; the feature
+//     row d of the tile holds ones, so column d collects the cluster sizes.  A wave owns every
+//     fourth block of 16 features and keeps their accumulators in registers until the end.
+//
+// The rows of the next tile travel from memory into registers while the tile in LDS is worked
+// on.  fp32 accumulation per workgroup (a few thousand samples), the workgroups' partial sums
+// are added by lloyd_reduce_kernel.
+#include "lloyd_layout.h"
+#include "lloyd_tail.h"
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct FewkLds {
+    size_t off_part, off_lab, off_w, total;
+    int rows;    // features of the tile: d, the ones, and padding up to what the unrolled loops address
+    int stride;  // feature-major tile: words per feature row, S + 4
+    int ds;      // sample-major tile: words per sample, >= rows and = 20 mod 64
+                 // (either way the lanes of a matrix operand fall on different banks, nearly)
+};
+
+// K steps of four features per wave for d features
+__host__ __device__ constexpr int fewk_kw(int d) { return (((d + 3) / 4) + 3) / 4; }
+
+__host__ __device__ inline FewkLds fewk_lds(int d, int S) {
+    FewkLds s;
+    const int kw = fewk_kw(d);
+    // the label pass of the last wave reads K steps 3 kw .. 3 kw + 8 ceil(kw / 8) - 1 (with zero
+    // centroid values past its share), the sums pass blocks of 16 rows up to row d
+    const int rows_k = 4 * (3 * kw + 8 * ((kw + 7) / 8));
+    const int rows_f = 16 * ((d + 1 + 15) / 16);
+    s.rows = rows_k > rows_f ? rows_k : rows_f;
+    s.stride = S + 4;
+    s.ds = s.rows + ((20 - s.rows % 64) + 64) % 64;
+    // (room for the larger of the two layouts: the launch does not depend on which one runs)
+    const size_t fm = (size_t)s.rows * s.stride * 4, sm = (size_t)S * s.ds * 4;
+    s.off_part = fm > sm ? fm : sm;                          // [4 waves][S / 16][16 clusters][16 samples]
+    s.off_lab = s.off_part + (size_t)4 * (S / 16) * 256 * 4;
+    s.off_w = s.off_lab + (size_t)S * 4;
+    s.total = s.off_w + (size_t)S * 4;
+    return s;
+}
+
+// 128-bit pieces of the next tile a thread holds in registers (d * S / 4 values over 256 threads)
+constexpr int fewk_prefetch(int kw, int s_log) {
+    return (kw <= 8 && s_log == 5) ? 4 : kw <= 16 ? 8 : kw <= 32 ? 10 : kw <= 52 ? 13 : 19;
+}
+
+// KW: K steps of four features per wave the kernel is unrolled for (d <= 16 KW); S_LOG: log2 of
+// the samples per tile.  Row offsets inside the tile are compile-time multiples of the row stride,
+// so that the reads of the unrolled loops differ by immediate offsets only.
+// RM: the tile is read from the row-major copy of X, (n, d) with d a multiple of 4 - S whole
+// samples are one contiguous stretch of memory, where the feature-major array gives d separate
+// pieces of 4 S bytes - and kept sample-major in LDS.
+// (two waves per SIMD - two workgroups per compute unit - up to 832 features: 256 registers; four
+// with tiles of 32 samples of up to 128 features)
+constexpr int fewk_waves_per_simd(int kw, int s_log) { return (kw <= 8 && s_log == 5) ? 4 : kw <= 52 ? 2 : 1; }
+template <int KW, int S_LOG, bool RM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(fewk_waves_per_simd(KW, S_LOG))))
+void lloyd_fewk_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ X_rm, const float* __restrict__ sample_weight,
+    const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
+    const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
+    float* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int vec_ok) {
+    if (status->state != KMX_RUNNING) return;
+    constexpr int FBW = KW / 4 + 1;  // blocks of 16 features per wave
+    constexpr int PF = fewk_prefetch(KW, S_LOG);
+    constexpr int S = 1 << S_LOG, NB = S >> 4, STRIDE = S + 4;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const FewkLds lay = fewk_lds(d, S);
+    float* tile = reinterpret_cast<float*>(smem_raw);                     // [rows][STRIDE]
+    float* part = reinterpret_cast<float*>(smem_raw + lay.off_part);
+    uint32_t* lab = reinterpret_cast<uint32_t*>(smem_raw + lay.off_lab);  // [S]
+    float* wts = reinterpret_cast<float*>(smem_raw + lay.off_w);          // [S]
+    const int rows = lay.rows;
+    const int DS = lay.ds;
+    __shared__ unsigned int changed_block;
+
+    // (the wave index in a scalar register: conditions on it are then branches of the wave, not
+    // masks over its lanes)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int g4 = lane >> 4, m16 = lane & 15;
+    const int kw = fewk_kw(d);  // K steps per wave (<= KW)
+    const int ks0 = wave * kw;
+    const int n_fb = (d + 1 + 15) >> 4;  // blocks of 16 features, the row of ones included
+    // wave w takes the blocks w, w + 4, ...: FBW of them whatever d is, a block past the last one
+    // standing for the last (its sums are not written) - no branch inside the loop over the
+    // samples, around which the compiler would copy all the accumulators
+
+    // the wave's centroid values: cluster m16, feature 4 (ks0 + s) + g4
+    float ca[KW];
+#pragma unroll
+    for (int s = 0; s < KW; ++s) {
+        const int f = 4 * (ks0 + s) + g4;
+        ca[s] = (s < kw && f < d && m16 < k) ? centroids_t[(size_t)f * k + m16] : 0.0f;
+    }
+    // -0.5||c||^2 of the clusters 4 g4 + r: the start of wave 0's scores
+    v4f start = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) start[r] = (4 * g4 + r < k) ? -half_norms[4 * g4 + r] : 0.0f;
+    }
+    // past the features: ones (feature d, the cluster sizes), then zeros; never overwritten
+    if (RM) {
+        for (int idx = threadIdx.x; idx < S * (DS - d); idx += 256) {
+            const int sm = idx / (DS - d), c = idx - sm * (DS - d);
+            tile[sm * DS + d + c] = c == 0 ? 1.0f : 0.0f;
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < (rows - d) * STRIDE; idx += 256)
+            tile[d * STRIDE + idx] = idx < STRIDE ? 1.0f : 0.0f;
+    }
+    if (threadIdx.x == 0) changed_block = 0;
+
+    v4f acc[FBW];
+#pragma unroll
+    for (int i = 0; i < FBW; ++i) acc[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    unsigned int changed = 0;
+
+    // The tile as 128-bit pieces, PF per thread.
+    // Feature-major: the thread's piece u is four samples (its quarter q_t of the row... of S / 4)
+    // of feature f_t + u * RSTEP.
+    // Row-major: the S / 4 samples of a wave are one contiguous stretch of (S / 4) d floats; lane l
+    // takes its pieces l, l + 64, ...; piece i holds features 4 (i % P) .. + 3 of sample i / P,
+    // P = d / 4.
+    constexpr int Q_LOG = S_LOG - 2, RSTEP = 256 >> Q_LOG;
+    const int f_t = threadIdx.x >> Q_LOG, q_t = threadIdx.x & ((1 << Q_LOG) - 1);
+    const size_t x_mine = (size_t)f_t * n + 4 * q_t;  // (the rest of an address is the same for all threads)
+    float* const tile_mine = tile + f_t * STRIDE + 4 * q_t;
+    const int P = d >> 2, wave_pieces = (S >> 2) * P;
+    float4 pf[PF];
+    // (and, every fourth thread, the weight and the previous label of one sample)
+    float w_next = 0.0f;
+    uint32_t pl_next = 0u;
+    auto fetch = [&](const int64_t s0) __attribute__((always_inline)) {
+        const bool whole = vec_ok && s0 + S <= n;  // workgroup-uniform
+        if ((int)threadIdx.x < 4 * S && (threadIdx.x & 3) == 0 && s0 + (threadIdx.x >> 2) < n) {
+            w_next = sample_weight[s0 + (threadIdx.x >> 2)];
+            pl_next = labels_prev[s0 + (threadIdx.x >> 2)];
+        }
+        if constexpr (RM) {
+            // (pieces of samples past the end are not read)
+            const int64_t left = n - (s0 + (int64_t)wave * (S >> 2));  // samples of the wave's stretch that exist
+            const int64_t live_pieces = left <= 0 ? 0 : (left >= (S >> 2) ? wave_pieces : left * P);
+            const float4* src = reinterpret_cast<const float4*>(X_rm + (size_t)(s0 + wave * (S >> 2)) * d);
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                const int i = lane + 64 * u;
+                pf[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (i < live_pieces) pf[u] = src[i];
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                pf[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (f_t + u * RSTEP < d) {
+                    const float* p = X_t + ((size_t)(u * RSTEP) * n + s0) + x_mine;
+                    if (whole) {
+                        pf[u] = *reinterpret_cast<const float4*>(p);
+                    } else {
+                        const int64_t i = s0 + 4 * q_t;
+                        if (i < n) pf[u].x = p[0];
+                        if (i + 1 < n) pf[u].y = p[1];
+                        if (i + 2 < n) pf[u].z = p[2];
+                        if (i + 3 < n) pf[u].w = p[3];
+                    }
+                }
+            }
+        }
+    };
+    auto deposit = [&]() __attribute__((always_inline)) {
+        if constexpr (RM) {
+            // (sample, piece inside the sample) of the lane's pieces, stepped from one to the next;
+            // the start is made opaque so that the chain is recomputed per tile instead of
+            // occupying a register per piece for the whole kernel
+            int sm = lane / P, r = lane - sm * P;
+            asm volatile("" : "+v"(sm), "+v"(r));
+            const int step_s = 64 / P, step_r = 64 - step_s * P;
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                if (lane + 64 * u < wave_pieces)
+                    *reinterpret_cast<float4*>(tile + (wave * (S >> 2) + sm) * DS + 4 * r) = pf[u];
+                sm += step_s;
+                r += step_r;
+                if (r >= P) {
+                    r -= P;
+                    sm += 1;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < PF; ++u)
+                if (f_t + u * RSTEP < d) *reinterpret_cast<float4*>(tile_mine + u * RSTEP * STRIDE) = pf[u];
+        }
+    };
+
+    const int64_t n_tiles = (n + S - 1) >> S_LOG;
+    int64_t t = blockIdx.x;
+    if (t < n_tiles) fetch(t << S_LOG);
+    // the wave's first row of the label pass (lane: feature g4 of a K step, sample m16 of a block)
+    // and of the sums pass (lane: feature m16 of a block of 16, sample g4 of a group of four)
+    const float* const col_labels = RM ? tile + m16 * DS + 4 * ks0 + g4 : tile + (4 * ks0 + g4) * STRIDE + m16;
+    const float* col_sums[FBW];
+#pragma unroll
+    for (int i = 0; i < FBW; ++i) {
+        const int fb = wave + 4 * i < n_fb ? wave + 4 * i : n_fb - 1;
+        col_sums[i] = RM ? tile + g4 * DS + 16 * fb + m16 : tile + (16 * fb + m16) * STRIDE + g4;
+    }
+    for (; t < n_tiles; t += gridDim.x) {
+        const int64_t s0 = t << S_LOG;
+        __syncthreads();  // the tile before this one is no longer read
+        deposit();
+        const float w_mine = w_next;
+        const uint32_t pl_mine = pl_next;
+#ifndef KMX_FEWK_DBG
+#define KMX_FEWK_DBG 0
+#endif
+        if (KMX_FEWK_DBG != 3 && t + gridDim.x < n_tiles) fetch((t + gridDim.x) << S_LOG);
+        __syncthreads();
+
+        // labels: partial scores of the wave's quarter of the features, eight K steps at a time
+        // (their reads of the tile, for all sample blocks, in flight together), two chains of
+        // accumulation per sample block
+        {
+            v4f sc0[NB], sc1[NB];
+#pragma unroll
+            for (int sb = 0; sb < NB; ++sb) {
+                sc0[sb] = start;
+                sc1[sb] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+#pragma unroll
+            for (int c0 = 0; c0 < KW; c0 += 8) {
+                if (KMX_FEWK_DBG != 2 && c0 < kw) {  // wave-uniform
+                    float b[NB][8];
+                    // (past the wave's share the centroid value is zero and the rows exist)
+#pragma unroll
+                    for (int sb = 0; sb < NB; ++sb)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            b[sb][j] = RM ? col_labels[16 * sb * DS + 4 * (c0 + j)]
+                                          : col_labels[4 * (c0 + j) * STRIDE + 16 * sb];
+#pragma unroll
+                    for (int j = 0; j < 8; j += 2)
+#pragma unroll
+                        for (int sb = 0; sb < NB; ++sb) {
+                            if (c0 + j < KW)
+                                sc0[sb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j < KW ? c0 + j : 0], b[sb][j],
+                                                                               sc0[sb], 0, 0, 0);
+                            if (c0 + j + 1 < KW)
+                                sc1[sb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j + 1 < KW ? c0 + j + 1 : 0],
+                                                                               b[sb][j + 1], sc1[sb], 0, 0, 0);
+                        }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int sb = 0; sb < NB; ++sb) {
+                float* out = part + ((wave * NB + sb) << 8) + m16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) out[(4 * g4 + r) << 4] = sc0[sb][r] + sc1[sb][r];
+            }
+        }
+        __syncthreads();
+        // arg-max: four threads per sample, thread q on the clusters q, q + 4, ... (the four partial
+        // tiles added in wave order, strict '>' in increasing cluster order), then the four combine:
+        // the largest score, the lowest index among equals
+        if ((int)threadIdx.x < 4 * S) {
+            const int s = threadIdx.x >> 2, q = threadIdx.x & 3, sb = s >> 4, m = s & 15;
+            float best = -kmx_inf<float>();
+            uint32_t bi = 0xffffffffu;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = q + 4 * j;
+                if (c < k) {
+                    float v = part[((0 * NB + sb) << 8) + (c << 4) + m];
+#pragma unroll
+                    for (int wv = 1; wv < 4; ++wv) v += part[((wv * NB + sb) << 8) + (c << 4) + m];
+                    if (v > best) {
+                        best = v;
+                        bi = (uint32_t)c;
+                    }
+                }
+            }
+#pragma unroll
+            for (int off = 1; off <= 2; off <<= 1) {
+                const float ov = __shfl_xor(best, off, 64);
+                const uint32_t oi = __shfl_xor(bi, off, 64);
+                if (ov > best || (ov == best && oi < bi)) {
+                    best = ov;
+                    bi = oi;
+                }
+            }
+            if (bi == 0xffffffffu) bi = 0u;  // no score compares: the reference's running arg-min keeps 0
+            const int64_t gi = s0 + s;
+            const bool live = gi < n;
+            if (q == 0) {
+                lab[s] = bi;
+                wts[s] = live ? w_mine : 0.0f;
+                if (live) {
+                    labels[gi] = bi;
+                    changed += pl_mine != bi ? 1u : 0u;
+                }
+            }
+        }
+        __syncthreads();
+
+        // sums: the wave's feature blocks, four samples per matrix instruction
+        // (U groups of four samples at a time, their reads in flight together; the loop is kept a
+        // loop: unrolled, its S / 4 addresses would each take a register for the whole kernel)
+        constexpr int U = FBW <= 5 ? 4 : FBW <= 9 ? 2 : 1;
+        int at = 0;  // offset of the group of samples inside a column of the tile
+        const int at_step = RM ? 4 * U * DS : 4 * U;
+#pragma unroll 1
+        for (int sc4 = 0; sc4 < (KMX_FEWK_DBG == 1 ? 0 : (S >> 2)); sc4 += U) {
+            float aw[U], b[U][FBW];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int s = 4 * (sc4 + u) + g4;
+                const uint32_t lb = lab[s];
+                const float wv = wts[s];
+                aw[u] = lb == (uint32_t)m16 ? wv : 0.0f;
+#pragma unroll
+                for (int i = 0; i < FBW; ++i) b[u][i] = col_sums[i][at + (RM ? 4 * u * DS : 4 * u)];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < FBW; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[u], b[u][i], acc[i], 0, 0, 0);
+            at += at_step;
+        }
+    }
+
+    // The workgroup's sums as they lie in the registers: slot ((wave FBW + i) 4 + r) 64 + lane of
+    // the workgroup's stretch of `partial` (whole cache lines per store; fewk_reduce_kernel knows
+    // which cluster and feature a slot stands for).
+    float* out = partial + (size_t)blockIdx.x * (4 * FBW * 256) + (size_t)wave * (FBW * 256) + lane;
+#pragma unroll
+    for (int i = 0; i < FBW; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) out[(i * 4 + r) * 64] = acc[i][r];
+    if (changed) atomicAdd(&changed_block, changed);
+    __syncthreads();
+    if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+}
+
+// Sum of the workgroups' partial sums, slot by slot and always in the same order, then the end of
+// the iteration.  A workgroup takes 32 slots; its 256 threads are 8 groups that each add every
+// eighth partial (sixteen loads in flight), and the groups are added in order.  The totals go
+// into the 64-bit fixed-point sums of the run, (d + 1, k) feature-major with the sizes in row d,
+// by device-scope stores, and the workgroup that gets done last finishes the iteration - empty
+// clusters, division, shift, convergence test, what the next step needs - reading them with
+// device-scope loads: one launch instead of two.
+template <int FBW>
+__global__ __launch_bounds__(256) void fewk_reduce_kernel(const float* __restrict__ partial, int n_partials,
+                                                          unsigned long long* __restrict__ gsum,
+                                                          const int* __restrict__ q_exp, int d, int k,
+                                                          const LloydTail<float> tail) {
+    extern __shared__ __align__(16) unsigned char red_raw[];
+    kmx_lloyd_status* status = tail.status;
+    if (status->state != KMX_RUNNING) return;
+    constexpr int NSLOT = 4 * FBW * 256;
+    __shared__ float group_sum[8][32];
+    const int sl = threadIdx.x & 31, pg = threadIdx.x >> 5;
+    const int slot = blockIdx.x * 32 + sl;
+    float total = 0.0f;
+    if (slot < NSLOT) {
+        const float* src = partial + slot;
+        int p = pg;
+        for (; p + 8 * 15 < n_partials; p += 8 * 16) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = src[(size_t)(p + 8 * u) * NSLOT];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) total += v[u];
+        }
+        for (; p < n_partials; p += 8) total += src[(size_t)p * NSLOT];
+    }
+    group_sum[pg][sl] = total;
+    __syncthreads();
+    if (threadIdx.x < 32 && slot < NSLOT) {
+        float v = group_sum[0][sl];
+#pragma unroll
+        for (int g = 1; g < 8; ++g) v += group_sum[g][sl];
+        // slot -> (feature, cluster): wave-of-the-step, block, register, lane
+        const int lane = slot & 63, r = (slot >> 6) & 3, wi = slot >> 8;  // wi = wave FBW + i
+        const int wave = wi / FBW, i = wi - wave * FBW;
+        const int f = 16 * (wave + 4 * i) + (lane & 15), c = 4 * (lane >> 4) + r;
+        if (f <= d && c < k && wave + 4 * i < ((d + 1 + 15) >> 4))
+            __hip_atomic_store(gsum + (size_t)f * k + c, (unsigned long long)__double2ll_rn(ldexp((double)v, q_exp[f])),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __shared__ unsigned int is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = (atomicAdd(&status->ticket, 1u) == gridDim.x - 1) ? 1u : 0u;
+    __syncthreads();
+    if (is_last != 0u) {
+        lloyd_small_finalize_body<float, true, true>(gsum, q_exp, tail, reinterpret_cast<float*>(red_raw));
+        if (threadIdx.x == 0) status->ticket = 0u;
+    }
+}
+
+// Samples per tile (a power of two, 16 .. 64) and workgroups per compute unit.
+struct FewkShape {
+    int s_log, kw, per_cu;
+    size_t lds;
+};
+
+bool fewk_shape(int d, int k, FewkShape* out) {
+    if (d <= 64 || d > 1216 || k < 1 || k > 16) return false;
+    const int kw = fewk_kw(d);
+    const int kw_t = kw <= 8 ? 8 : kw <= 16 ? 16 : kw <= 32 ? 32 : kw <= 52 ? 52 : 76;
+    // (tiles of 32 samples up to 512 features while two workgroups fit a compute unit, of 16 beyond:
+    // the instantiated kernels; measured at 2e6 x 100: tiles of 64 samples, which leave room for two
+    // workgroups per compute unit instead of four, take 1.6x as long)
+    for (int s_log = kw_t <= 32 ? 5 : 4; s_log >= (kw_t <= 16 ? 5 : 4); --s_log) {
+        const int S = 1 << s_log;
+        const size_t lds = fewk_lds(d, S).total;
+        const int pieces = (d * (S / 4) + 255) / 256;
+        // (a larger tile only while two workgroups still fit a compute unit)
+        const size_t cap = s_log > 4 ? (size_t)78 * 1024 : (size_t)156 * 1024;
+        if (lds <= cap && pieces <= fewk_prefetch(kw_t, s_log)) {
+            const int by_lds = (int)((size_t)160 * 1024 / (lds + 512));
+            const int by_regs = fewk_waves_per_simd(kw_t, s_log);  // waves per SIMD the kernel is built for
+            const int per_cu = by_lds < by_regs ? by_lds : by_regs;
+            out->s_log = s_log;
+            out->kw = kw_t;
+            out->per_cu = per_cu < 1 ? 1 : per_cu;  // (at most four: 1024 partial slots)
+            out->lds = lds;
+            return true;
+        }
+    }
+    return false;
+}
+
+}  // namespace
+
+bool kmx_fewk_supported(int d, int k) {
+    FewkShape sh;
+    return fewk_shape(d, k, &sh);
+}
+
+// room for the partial sums of the largest grid (four workgroups per compute unit)
+size_t kmx_fewk_partial_bytes(int d, int k) {
+    FewkShape sh;
+    if (!fewk_shape(d, k, &sh)) return 0;
+    // (a fixed number of compute units: the layout of the workspace is a function of the shape alone;
+    // on a larger device the grid stops at what fits)
+    return (size_t)sh.per_cu * 256 * 4 * (sh.kw / 4 + 1) * 256 * sizeof(float);
+}
+
+int kmx_fewk_grid(int64_t n, int d, int k, int wgs_per_cu) {
+    FewkShape sh;
+    if (!fewk_shape(d, k, &sh)) return 1;
+    const int64_t tiles = (n + (1 << sh.s_log) - 1) >> sh.s_log;
+    int64_t grid = (int64_t)(wgs_per_cu > 0 && wgs_per_cu < sh.per_cu ? wgs_per_cu : sh.per_cu) * kmx_num_cus();
+    if (grid > tiles) grid = tiles;
+    return grid < 1 ? 1 : (int)grid;
+}
+
+// One iteration: the fused step, whose last workgroup also finishes the iteration.  The
+// workspace holds the fixed-point exponents and the cleared sums of kmx_lloyd_mfma_prepare.
+int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X_rowmajor, const void* w,
+                            const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev,
+                            uint32_t* labels, void* sizes, uint32_t* empty_clusters, char* ws, int64_t n, int d,
+                            int k, hipStream_t stream, hipEvent_t* events) {
+    FewkShape sh;
+    if (!fewk_shape(d, k, &sh)) return KMX_ERR_UNSUPPORTED;
+    LloydTail<float> tail;
+    tail.sums_t = (float*)new_centroids_t;
+    tail.sizes = (float*)sizes;
+    tail.empty_clusters = empty_clusters;
+    tail.old_centroids_t = (const float*)centroids_t;
+    tail.cpack = reinterpret_cast<float*>(ws + L.off_cpack);
+    tail.half_norms = reinterpret_cast<float*>(ws + L.off_half);
+    tail.status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
+    tail.d = d;
+    tail.k = k;
+    tail.dpad = L.dpad;
+    const int* q_exp = reinterpret_cast<const int*>(ws + L.off_scales) + (d + 1);
+    unsigned long long* gsum = reinterpret_cast<unsigned long long*>(ws + L.off_gsum);
+    kmx_lloyd_status* status = tail.status;
+    const float* half_norms = tail.half_norms;
+    float* partial = reinterpret_cast<float*>(ws + L.off_partial);
+    int grid = kmx_fewk_grid(n, d, k, L.wgs_per_cu);
+    const int fbw_t = sh.kw / 4 + 1;  // blocks of 16 features per wave of the instantiated kernel
+    const size_t slots = (size_t)4 * fbw_t * 256;
+    if ((size_t)grid * slots * sizeof(float) > L.partial_bytes) grid = (int)(L.partial_bytes / (slots * sizeof(float)));
+    if (grid < 1) return KMX_ERR_WORKSPACE;
+    const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0);
+#ifndef KMX_FEWK_RM
+#define KMX_FEWK_RM 1
+#endif
+    // whole samples from the row-major copy when there is one whose rows are multiples of 16 bytes
+    const bool rm = KMX_FEWK_RM && X_rowmajor != nullptr && d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0);
+    if (events) (void)hipEventRecord(events[0], stream);
+#define KMX_FEWK_LAUNCH_RM(KW_, SL_, RM_)                                                                  \
+    do {                                                                                                  \
+        if (sh.lds > 64 * 1024) {                                                                         \
+            const hipError_t e = hipFuncSetAttribute(                                                     \
+                reinterpret_cast<const void*>(&lloyd_fewk_kernel<KW_, SL_, RM_>),                         \
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh.lds);                                 \
+            if (e != hipSuccess) return (int32_t)e;                                                       \
+        }                                                                                                 \
+        hipLaunchKernelGGL((lloyd_fewk_kernel<KW_, SL_, RM_>), dim3((unsigned)grid), dim3(256), sh.lds,   \
+                           stream, (const float*)X_t, (const float*)X_rowmajor, (const float*)w,          \
+                           (const float*)centroids_t, half_norms, labels_prev, labels, partial, status,   \
+                           n, d, k, vec_ok);                                                              \
+    } while (0)
+#define KMX_FEWK_LAUNCH(KW_, SL_)                \
+    do {                                         \
+        if (rm)                                  \
+            KMX_FEWK_LAUNCH_RM(KW_, SL_, true);  \
+        else                                     \
+            KMX_FEWK_LAUNCH_RM(KW_, SL_, false); \
+    } while (0)
+    if (sh.kw == 8 && sh.s_log == 5) KMX_FEWK_LAUNCH(8, 5);
+    else if (sh.kw == 16 && sh.s_log == 5) KMX_FEWK_LAUNCH(16, 5);
+    else if (sh.kw == 32 && sh.s_log == 5) KMX_FEWK_LAUNCH(32, 5);
+    else if (sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4);
+    else if (sh.kw == 52 && sh.s_log == 4) KMX_FEWK_LAUNCH(52, 4);
+    else if (sh.kw == 76 && sh.s_log == 4) KMX_FEWK_LAUNCH(76, 4);
+    else return KMX_ERR_UNSUPPORTED;
+#undef KMX_FEWK_LAUNCH_RM
+#undef KMX_FEWK_LAUNCH
+    KMX_LAUNCH_CHECK();
+    if (events) (void)hipEventRecord(events[1], stream);
+    const size_t tail_lds = (size_t)(d + 1) * k * sizeof(float);
+    const unsigned red_grid = (unsigned)((slots + 31) / 32);
+#define KMX_FEWK_REDUCE(FBW_)                                                                              \
+    do {                                                                                                  \
+        if (tail_lds > 64 * 1024) {                                                                       \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fewk_reduce_kernel<FBW_>), \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds); \
+            if (e != hipSuccess) return (int32_t)e;                                                       \
+        }                                                                                                 \
+        hipLaunchKernelGGL((fewk_reduce_kernel<FBW_>), dim3(red_grid), dim3(256), tail_lds, stream, partial, grid, \
+                           gsum, q_exp, d, k, tail);                                                      \
+    } while (0)
+    switch (fbw_t) {
+        case 3: KMX_FEWK_REDUCE(3); break;
+        case 5: KMX_FEWK_REDUCE(5); break;
+        case 9: KMX_FEWK_REDUCE(9); break;
+        case 14: KMX_FEWK_REDUCE(14); break;
+        default: KMX_FEWK_REDUCE(20); break;
+    }
+#undef KMX_FEWK_REDUCE
+    KMX_LAUNCH_CHECK();
+    if (events) {
+        (void)hipEventRecord(events[2], stream);
+        (void)hipEventRecord(events[3], stream);
+    }
+    return KMX_OK;
+}

@@ -11,6 +11,7 @@ constexpr int KMX_VARIANT_MFMA = 3;      // fp32 distances on the matrix cores, 
 constexpr int KMX_VARIANT_MFMA_WIDE = 4; // fp32 matrix cores, samples in registers, global sums
 constexpr int KMX_VARIANT_MFMA_F64 = 5;  // fp64 distances on the matrix cores, LDS accumulators
 constexpr int KMX_VARIANT_GEMM = 6;      // labels by a tiled matrix-core product (any shape), bucketed sums
+constexpr int KMX_VARIANT_FEWK = 8;      // fp32, up to 16 clusters, 65 .. 1216 features: a tile of samples in LDS serves labels and sums
 
 constexpr int KMX_ACC_LDS = 1;
 constexpr int KMX_ACC_GLOBAL = 2;
@@ -91,6 +92,10 @@ bool kmx_mfma_screen_supported(int64_t n, int d, int k, uint32_t flags);
 bool kmx_mfma_screen_f64_supported(int64_t n, int d, int k, uint32_t flags);  // fp64 inputs
 // the same kernel without the sums (labels only): needs less LDS
 bool kmx_mfma_screen_labels_fits(int64_t n, int d, int k);
+// few clusters on wide samples, X read once (lloyd_fewk.hip)
+bool kmx_fewk_supported(int d, int k);
+int kmx_fewk_grid(int64_t n, int d, int k, int wgs_per_cu);
+size_t kmx_fewk_partial_bytes(int d, int k);
 int32_t kmx_lloyd_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
                                      kmx_lloyd_status* status, int64_t n, int d, int k, int wgs_per_cu,
                                      hipStream_t stream);
@@ -191,8 +196,14 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
             L.n_partials = slots < KMX_MAX_PARTIALS ? slots : KMX_MAX_PARTIALS;
         }
     }
+    // (few clusters on wide samples: one read of X instead of two, or of a sort by label)
+    else if (dtype == KMX_F32 && forced < 0 && kmx_fewk_supported(d, k)) {
+        L.variant = KMX_VARIANT_FEWK;
+        L.acc_mode = KMX_ACC_LDS;  // (per-workgroup sums, here kept in registers, then the fixed-point sums of the run)
+        L.n_partials = 1;
+    }
     const bool specialised = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE ||
-                             L.variant == KMX_VARIANT_MFMA_F64;
+                             L.variant == KMX_VARIANT_MFMA_F64 || L.variant == KMX_VARIANT_FEWK;
     if (n <= INT32_MAX && (!specialised || forced == KMX_VARIANT_GEMM)) {
         // No specialised fused kernel.  Beyond 16 clusters (one window of the streaming kernel; the
         // measured break-even lies between 16 and 32), or whenever the accumulators do not
@@ -249,6 +260,8 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     // the matrix-core path accumulates into gsum and needs no per-workgroup partials
     const bool fixed_point = L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.screen64;
     L.partial_bytes = fixed_point ? 0 : (size_t)L.n_partials * items * s;
+    // (the few-cluster step: per workgroup the accumulators as they lie in its registers)
+    if (L.variant == KMX_VARIANT_FEWK) L.partial_bytes = kmx_fewk_partial_bytes(d, k);
     L.total = L.off_partial + kmx_align256(L.partial_bytes);
     return L;
 }
@@ -291,6 +304,10 @@ int32_t kmx_lloyd_iter_mfma_screen_f64(const LloydLayout& L, const void* X_t, co
                                        const uint32_t* labels_prev, uint32_t* labels, void* sizes,
                                        uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
                                        hipStream_t stream, hipEvent_t* events);
+int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X_rowmajor, const void* w,
+                            const void* centroids_t, void* new_centroids_t, const uint32_t* labels_prev,
+                            uint32_t* labels, void* sizes, uint32_t* empty_clusters, char* ws, int64_t n, int d,
+                            int k, hipStream_t stream, hipEvent_t* events);
 // labels only, screened the same way (scale from the centroids, norms taken per tile)
 int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, uint32_t* labels,
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream);

@@ -249,7 +249,20 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
                 if (jx < items) convert(jx, sum_v[i]);
             }
         } else {
-            for (int jx = threadIdx.x; jx < items; jx += n_threads) convert(jx, load_sum(jx));
+            // (SUMS_AHEAD loads in flight per thread and pass: a loop of one load and one store per
+            // pass would take a trip to memory per element)
+            for (int base = 0; base < items; base += n_threads * SUMS_AHEAD) {
+#pragma unroll
+                for (int i = 0; i < SUMS_AHEAD; ++i) {
+                    const int jx = base + (int)threadIdx.x + n_threads * i;
+                    sum_v[i] = jx < items ? load_sum(jx) : 0ll;
+                }
+#pragma unroll
+                for (int i = 0; i < SUMS_AHEAD; ++i) {
+                    const int jx = base + (int)threadIdx.x + n_threads * i;
+                    if (jx < items) convert(jx, sum_v[i]);
+                }
+            }
         }
     } else {
         for (int jx = threadIdx.x; jx < items; jx += n_threads) vals[jx] = jx < dk ? out_t[jx] : a.sizes[jx - dk];
@@ -294,8 +307,18 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
             if (jx < dk) divide(jx, old_v[i]);
         }
     } else {
-#pragma unroll 4
-        for (int jx = threadIdx.x; jx < dk; jx += n_threads) divide(jx, old_t[jx]);
+        for (int base = 0; base < dk; base += n_threads * OLD_AHEAD) {
+#pragma unroll
+            for (int i = 0; i < OLD_AHEAD; ++i) {
+                const int jx = base + (int)threadIdx.x + n_threads * i;
+                old_v[i] = jx < dk ? old_t[jx] : T(0);
+            }
+#pragma unroll
+            for (int i = 0; i < OLD_AHEAD; ++i) {
+                const int jx = base + (int)threadIdx.x + n_threads * i;
+                if (jx < dk) divide(jx, old_v[i]);
+            }
+        }
     }
     __syncthreads();
     for (int c = threadIdx.x; c < k; c += n_threads) {

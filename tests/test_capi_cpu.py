@@ -127,8 +127,12 @@ def test_kernel_variant_selection():
     assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0, 0) == 11           # too few clusters for MFMA
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 64, 0, 0) == 63    # the wide path only beyond 256 clusters
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 300, 0, 0) == 42
-    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 0, 0) == 1     # few clusters, sums in LDS: fused vector-ALU step
-    assert lib.kmx_lloyd_kernel_variant(100_000, 784, 10, 0, 0) == 63      # sums beyond LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 0, 0) == 81    # few clusters, wide samples: one read of X
+    assert lib.kmx_lloyd_kernel_variant(100_000, 784, 10, 0, 0) == 81
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 0, 0x1) == 1   # on request: the fused vector-ALU step
+    assert lib.kmx_lloyd_kernel_variant(100_000, 784, 10, 0, 0x4) == 63    # or the tiled product with sums per bucket
+    assert lib.kmx_lloyd_kernel_variant(100_000, 1300, 10, 0, 0) == 63     # a tile of such samples does not fit the LDS
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 1, 0) == 1     # fp64: as before
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0x4) == 63  # the tiled product on request
     assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0, 0) == -2
     assert lib.kmx_lloyd_kernel_variant(10, 3, 5, 4, 0) == -3
