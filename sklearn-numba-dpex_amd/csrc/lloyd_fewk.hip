@@ -64,7 +64,7 @@ __host__ __device__ inline FewkLds fewk_lds(int d, int S) {
 
 // 128-bit pieces of the next tile a thread holds in registers (d * S / 4 values over 256 threads)
 constexpr int fewk_prefetch(int kw, int s_log) {
-    return (kw <= 8 && s_log == 5) ? 4 : kw <= 16 ? 8 : kw <= 32 ? 10 : kw <= 52 ? 13 : 19;
+    return (kw <= 8 && s_log == 5) ? 4 : kw <= 16 ? 8 : kw <= 32 ? 10 : kw <= 52 ? 13 : 19;  // ((8, 6): 8)
 }
 
 // KW: K steps of four features per wave the kernel is unrolled for (d <= 16 KW); S_LOG: log2 of
@@ -76,6 +76,7 @@ constexpr int fewk_prefetch(int kw, int s_log) {
 // (two waves per SIMD - two workgroups per compute unit - up to 832 features: 256 registers; four
 // with tiles of 32 samples of up to 128 features)
 constexpr int fewk_waves_per_simd(int kw, int s_log) { return (kw <= 8 && s_log == 5) ? 4 : kw <= 52 ? 2 : 1; }
+
 template <int KW, int S_LOG, bool RM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(fewk_waves_per_simd(KW, S_LOG))))
 void lloyd_fewk_kernel(
@@ -233,10 +234,7 @@ void lloyd_fewk_kernel(
         deposit();
         const float w_mine = w_next;
         const uint32_t pl_mine = pl_next;
-#ifndef KMX_FEWK_DBG
-#define KMX_FEWK_DBG 0
-#endif
-        if (KMX_FEWK_DBG != 3 && t + gridDim.x < n_tiles) fetch((t + gridDim.x) << S_LOG);
+        if (t + gridDim.x < n_tiles) fetch((t + gridDim.x) << S_LOG);
         __syncthreads();
 
         // labels: partial scores of the wave's quarter of the features, eight K steps at a time
@@ -251,7 +249,7 @@ void lloyd_fewk_kernel(
             }
 #pragma unroll
             for (int c0 = 0; c0 < KW; c0 += 8) {
-                if (KMX_FEWK_DBG != 2 && c0 < kw) {  // wave-uniform
+                if (c0 < kw) {  // wave-uniform
                     float b[NB][8];
                     // (past the wave's share the centroid value is zero and the rows exist)
 #pragma unroll
@@ -332,7 +330,7 @@ void lloyd_fewk_kernel(
         int at = 0;  // offset of the group of samples inside a column of the tile
         const int at_step = RM ? 4 * U * DS : 4 * U;
 #pragma unroll 1
-        for (int sc4 = 0; sc4 < (KMX_FEWK_DBG == 1 ? 0 : (S >> 2)); sc4 += U) {
+        for (int sc4 = 0; sc4 < (S >> 2); sc4 += U) {
             float aw[U], b[U][FBW];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -365,6 +363,185 @@ void lloyd_fewk_kernel(
     if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
 }
 
+// Up to 128 features with a row-major copy of X: every WAVE works on tiles of 16 samples of its
+// own, with no barrier and no exchange between waves - at this width a workgroup's tile is so small
+// that the barriers and the bookkeeping around it (some 400 instructions per wave and tile for 40
+// matrix instructions) cost more than the arithmetic.  The wave holds the centroid values of all
+// features in registers (KS K steps of four), its scores are complete in its own registers (the
+// arg-max is three compares and two exchanges between the lane groups), and it keeps the sums of
+// all NFB feature blocks.  At the end the four waves of a workgroup add their sums in wave order.
+constexpr int fewk_wave_ds(int cols) { return cols + ((20 - cols % 64) + 64) % 64; }
+__host__ __device__ constexpr int fewk_wave_cols(int d, int nfb) {
+    return 4 * ((d + 3) / 4) > 16 * nfb ? 4 * ((d + 3) / 4) : 16 * nfb;
+}
+template <int KS, int NFB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void lloyd_fewk_wave_kernel(
+    const float* __restrict__ X_rm, const float* __restrict__ sample_weight,
+    const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
+    const uint32_t* __restrict__ labels_prev, uint32_t* __restrict__ labels,
+    float* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k) {
+    if (status->state != KMX_RUNNING) return;
+    constexpr int PF = (16 * 16 * NFB / 4 + 63) / 64;  // 128-bit pieces per lane of a tile of 16 samples
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int g4 = lane >> 4, m16 = lane & 15;
+    const int DS = fewk_wave_ds(fewk_wave_cols(d, NFB));
+    float* tile = reinterpret_cast<float*>(smem_raw) + wave * 16 * DS;  // [16 samples][DS], the wave's own
+    const int ksteps = (d + 3) >> 2;
+    const int n_fb = (d + 1 + 15) >> 4;
+    __shared__ unsigned int changed_block;
+
+    float ca[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int f = 4 * s + g4;
+        ca[s] = (f < d && m16 < k) ? centroids_t[(size_t)f * k + m16] : 0.0f;
+    }
+    v4f start;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) start[r] = (4 * g4 + r < k) ? -half_norms[4 * g4 + r] : 0.0f;
+    // past the features: ones (feature d, the cluster sizes), then zeros; never overwritten
+    for (int idx = lane; idx < 16 * (DS - d); idx += 64) {
+        const int sm = idx / (DS - d), c = idx - sm * (DS - d);
+        tile[sm * DS + d + c] = c == 0 ? 1.0f : 0.0f;
+    }
+    if (threadIdx.x == 0) changed_block = 0;
+    __syncthreads();
+
+    v4f acc[NFB];
+#pragma unroll
+    for (int i = 0; i < NFB; ++i) acc[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    unsigned int changed = 0;
+
+    // a tile is one contiguous stretch of 16 d floats; lane l takes its 128-bit pieces l, l + 64, ...;
+    // piece i holds features 4 (i % P) .. + 3 of sample i / P, P = d / 4
+    const int P = d >> 2, tile_pieces = 16 * P;
+    float4 pf[PF];
+    float w_next = 0.0f;
+    uint32_t pl_next = 0u;
+    auto fetch = [&](const int64_t s0) __attribute__((always_inline)) {
+        if (g4 == 0 && s0 + m16 < n) {
+            w_next = sample_weight[s0 + m16];
+            pl_next = labels_prev[s0 + m16];
+        }
+        const int64_t left = n - s0;
+        const int live_pieces = left >= 16 ? tile_pieces : (int)left * P;
+        const float4* src = reinterpret_cast<const float4*>(X_rm + (size_t)s0 * d);
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int i = lane + 64 * u;
+            pf[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (i < live_pieces) pf[u] = src[i];
+        }
+    };
+    auto deposit = [&]() __attribute__((always_inline)) {
+        int sm = lane / P, r = lane - sm * P;
+        asm volatile("" : "+v"(sm), "+v"(r));  // (recomputed per tile instead of a register per piece)
+        const int step_s = 64 / P, step_r = 64 - step_s * P;
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            if (lane + 64 * u < tile_pieces) *reinterpret_cast<float4*>(tile + sm * DS + 4 * r) = pf[u];
+            sm += step_s;
+            r += step_r;
+            if (r >= P) {
+                r -= P;
+                sm += 1;
+            }
+        }
+    };
+
+    const int64_t n_tiles = (n + 15) >> 4;
+    const int64_t t_step = (int64_t)gridDim.x * 4;
+    int64_t t = (int64_t)blockIdx.x * 4 + wave;
+    if (t < n_tiles) fetch(t << 4);
+    const float* const col_labels = tile + m16 * DS + g4;       // feature g4 of a K step, sample m16
+    const float* const col_sums = tile + g4 * DS + m16;         // sample g4 of a group of four, feature m16 of a block
+    for (; t < n_tiles; t += t_step) {
+        const int64_t s0 = t << 4;
+        deposit();
+        const float w_mine = w_next;
+        const uint32_t pl_mine = pl_next;
+        if (t + t_step < n_tiles) fetch((t + t_step) << 4);
+
+        // labels: all K steps, two chains of accumulation
+        v4f sc0 = start, sc1 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c0 = 0; c0 < KS; c0 += 8) {
+            if (c0 < ksteps) {  // wave-uniform (past d the centroid values are zero and the columns exist)
+                float b[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) b[j] = col_labels[4 * (c0 + j < KS ? c0 + j : KS - 1)];
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) {
+                    if (c0 + j < KS) sc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j < KS ? c0 + j : 0], b[j], sc0, 0, 0, 0);
+                    if (c0 + j + 1 < KS)
+                        sc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j + 1 < KS ? c0 + j + 1 : 0], b[j + 1], sc1, 0,
+                                                                   0, 0);
+                }
+            }
+        }
+        // arg-max of sample m16: the lane's clusters 4 g4 + r in increasing order (strict '>'), then
+        // the four lane groups: the largest score, the lowest index among equals
+        float best = -kmx_inf<float>();
+        uint32_t bi = 0xffffffffu;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = sc0[r] + sc1[r];
+            if (4 * g4 + r < k && v > best) {
+                best = v;
+                bi = (uint32_t)(4 * g4 + r);
+            }
+        }
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+            const float ov = __shfl_xor(best, off, 64);
+            const uint32_t oi = __shfl_xor(bi, off, 64);
+            const bool take = ov > best || (ov == best && oi < bi);
+            best = take ? ov : best;
+            bi = take ? oi : bi;
+        }
+        if (bi == 0xffffffffu) bi = 0u;  // no score compares: the reference's running arg-min keeps 0
+        const bool live = s0 + m16 < n;
+        if (g4 == 0 && live) {
+            labels[s0 + m16] = bi;
+            changed += pl_mine != bi ? 1u : 0u;
+        }
+        // (lanes 0 .. 15 hold label and weight of sample m16)
+        const float w_lane = live ? w_mine : 0.0f;
+
+        // sums: four samples per matrix instruction; the row of sample 4 c + g4 carries its weight
+        // in the column of its cluster
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t lb = __shfl(bi, 4 * c + g4, 64);
+            const float wv = __shfl(w_lane, 4 * c + g4, 64);
+            const float aw = lb == (uint32_t)m16 ? wv : 0.0f;
+            float b[NFB];
+#pragma unroll
+            for (int i = 0; i < NFB; ++i) b[i] = col_sums[4 * c * DS + 16 * i];
+#pragma unroll
+            for (int i = 0; i < NFB; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw, b[i], acc[i], 0, 0, 0);
+        }
+    }
+
+    // the four waves' sums are added in wave order (through the LDS of the tiles, now free): one
+    // partial per workgroup, slot (fb 4 + r) 64 + lane
+    if (changed) atomicAdd(&changed_block, changed);
+    __syncthreads();
+    float* mine = reinterpret_cast<float*>(smem_raw) + wave * (NFB * 256) + lane;  // (NFB * 256 <= 16 DS)
+#pragma unroll
+    for (int i = 0; i < NFB; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mine[(i * 4 + r) * 64] = acc[i][r];
+    __syncthreads();
+    const float* all = reinterpret_cast<const float*>(smem_raw);
+    float* out = partial + (size_t)blockIdx.x * (NFB * 256);
+    for (int slot = threadIdx.x; slot < NFB * 256; slot += 256)
+        out[slot] = ((all[slot] + all[NFB * 256 + slot]) + all[2 * NFB * 256 + slot]) + all[3 * NFB * 256 + slot];
+    (void)n_fb;
+    if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
+}
+
 // Sum of the workgroups' partial sums, slot by slot and always in the same order, then the end of
 // the iteration.  A workgroup takes 32 slots; its 256 threads are 8 groups that each add every
 // eighth partial (sixteen loads in flight), and the groups are added in order.  The totals go
@@ -372,7 +549,9 @@ void lloyd_fewk_kernel(
 // by device-scope stores, and the workgroup that gets done last finishes the iteration - empty
 // clusters, division, shift, convergence test, what the next step needs - reading them with
 // device-scope loads: one launch instead of two.
-template <int FBW>
+// PER_WAVE: the partials are those of lloyd_fewk_wave_kernel - FBW blocks of 16 features each,
+// block fb in slots 256 fb .. 256 fb + 255.
+template <int FBW, bool PER_WAVE>
 __global__ __launch_bounds__(256) void fewk_reduce_kernel(const float* __restrict__ partial, int n_partials,
                                                           unsigned long long* __restrict__ gsum,
                                                           const int* __restrict__ q_exp, int d, int k,
@@ -380,7 +559,7 @@ __global__ __launch_bounds__(256) void fewk_reduce_kernel(const float* __restric
     extern __shared__ __align__(16) unsigned char red_raw[];
     kmx_lloyd_status* status = tail.status;
     if (status->state != KMX_RUNNING) return;
-    constexpr int NSLOT = 4 * FBW * 256;
+    constexpr int NSLOT = (PER_WAVE ? 1 : 4) * FBW * 256;
     __shared__ float group_sum[8][32];
     const int sl = threadIdx.x & 31, pg = threadIdx.x >> 5;
     const int slot = blockIdx.x * 32 + sl;
@@ -406,8 +585,9 @@ __global__ __launch_bounds__(256) void fewk_reduce_kernel(const float* __restric
         // slot -> (feature, cluster): wave-of-the-step, block, register, lane
         const int lane = slot & 63, r = (slot >> 6) & 3, wi = slot >> 8;  // wi = wave FBW + i
         const int wave = wi / FBW, i = wi - wave * FBW;
-        const int f = 16 * (wave + 4 * i) + (lane & 15), c = 4 * (lane >> 4) + r;
-        if (f <= d && c < k && wave + 4 * i < ((d + 1 + 15) >> 4))
+        const int fb = PER_WAVE ? wi : wave + 4 * i;
+        const int f = 16 * fb + (lane & 15), c = 4 * (lane >> 4) + r;
+        if (f <= d && c < k && fb < ((d + 1 + 15) >> 4))
             __hip_atomic_store(gsum + (size_t)f * k + c, (unsigned long long)__double2ll_rn(ldexp((double)v, q_exp[f])),
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -434,7 +614,7 @@ bool fewk_shape(int d, int k, FewkShape* out) {
     const int kw_t = kw <= 8 ? 8 : kw <= 16 ? 16 : kw <= 32 ? 32 : kw <= 52 ? 52 : 76;
     // (tiles of 32 samples up to 512 features while two workgroups fit a compute unit, of 16 beyond:
     // the instantiated kernels; measured at 2e6 x 100: tiles of 64 samples, which leave room for two
-    // workgroups per compute unit instead of four, take 1.6x as long)
+    // workgroups per compute unit instead of four, are no faster)
     for (int s_log = kw_t <= 32 ? 5 : 4; s_log >= (kw_t <= 16 ? 5 : 4); --s_log) {
         const int S = 1 << s_log;
         const size_t lds = fewk_lds(d, S).total;
@@ -447,7 +627,7 @@ bool fewk_shape(int d, int k, FewkShape* out) {
             const int per_cu = by_lds < by_regs ? by_lds : by_regs;
             out->s_log = s_log;
             out->kw = kw_t;
-            out->per_cu = per_cu < 1 ? 1 : per_cu;  // (at most four: 1024 partial slots)
+            out->per_cu = per_cu < 1 ? 1 : per_cu;
             out->lds = lds;
             return true;
         }
@@ -468,7 +648,11 @@ size_t kmx_fewk_partial_bytes(int d, int k) {
     if (!fewk_shape(d, k, &sh)) return 0;
     // (a fixed number of compute units: the layout of the workspace is a function of the shape alone;
     // on a larger device the grid stops at what fits)
-    return (size_t)sh.per_cu * 256 * 4 * (sh.kw / 4 + 1) * 256 * sizeof(float);
+    const size_t by_workgroup = (size_t)sh.per_cu * 256 * 4 * (sh.kw / 4 + 1) * 256 * sizeof(float);
+    // (up to 128 features the per-wave kernel may run instead: three workgroups per compute unit, a
+    // partial each of up to nine feature blocks)
+    const size_t by_wave = d <= 128 ? (size_t)3 * 256 * 9 * 256 * sizeof(float) : 0;
+    return by_workgroup > by_wave ? by_workgroup : by_wave;
 }
 
 int kmx_fewk_grid(int64_t n, int d, int k, int wgs_per_cu) {
@@ -505,17 +689,51 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
     const float* half_norms = tail.half_norms;
     float* partial = reinterpret_cast<float*>(ws + L.off_partial);
     int grid = kmx_fewk_grid(n, d, k, L.wgs_per_cu);
-    const int fbw_t = sh.kw / 4 + 1;  // blocks of 16 features per wave of the instantiated kernel
-    const size_t slots = (size_t)4 * fbw_t * 256;
+    const size_t slots = (size_t)4 * (sh.kw / 4 + 1) * 256;  // partial sums of a workgroup of the instantiated kernel
     if ((size_t)grid * slots * sizeof(float) > L.partial_bytes) grid = (int)(L.partial_bytes / (slots * sizeof(float)));
     if (grid < 1) return KMX_ERR_WORKSPACE;
     const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0);
-#ifndef KMX_FEWK_RM
-#define KMX_FEWK_RM 1
-#endif
     // whole samples from the row-major copy when there is one whose rows are multiples of 16 bytes
-    const bool rm = KMX_FEWK_RM && X_rowmajor != nullptr && d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0);
+    const bool rm = X_rowmajor != nullptr && d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0);
     if (events) (void)hipEventRecord(events[0], stream);
+    const size_t tail_lds = (size_t)(d + 1) * k * sizeof(float);
+#define KMX_FEWK_REDUCE(FBW_, PW_, N_PARTIALS)                                                             \
+    do {                                                                                                  \
+        if (tail_lds > 64 * 1024) {                                                                       \
+            const hipError_t e =                                                                          \
+                hipFuncSetAttribute(reinterpret_cast<const void*>(&fewk_reduce_kernel<FBW_, PW_>),        \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds);           \
+            if (e != hipSuccess) return (int32_t)e;                                                       \
+        }                                                                                                 \
+        hipLaunchKernelGGL((fewk_reduce_kernel<FBW_, PW_>),                                               \
+                           dim3((unsigned)(((PW_ ? 1 : 4) * FBW_ * 256 + 31) / 32)), dim3(256), tail_lds, \
+                           stream, partial, N_PARTIALS, gsum, q_exp, d, k, tail);                         \
+    } while (0)
+    if (rm && d <= 128) {
+        // every wave on tiles of its own (no barriers): three workgroups per compute unit
+        const int nfb = (d + 1 + 15) / 16;
+        const int nfb_t = nfb <= 5 ? 5 : nfb <= 7 ? 7 : 9;
+        const size_t wave_lds = (size_t)4 * 16 * fewk_wave_ds(fewk_wave_cols(d, nfb_t)) * sizeof(float);
+        int64_t wgrid = (int64_t)(L.wgs_per_cu > 0 && L.wgs_per_cu < 3 ? L.wgs_per_cu : 3) * kmx_num_cus();
+        const int64_t by_room = (int64_t)(L.partial_bytes / ((size_t)nfb_t * 256 * sizeof(float)));
+        const int64_t by_tiles = kmx_cdiv(kmx_cdiv(n, 16), 4);
+        if (wgrid > by_room) wgrid = by_room;
+        if (wgrid > by_tiles) wgrid = by_tiles;
+        if (wgrid < 1) return KMX_ERR_WORKSPACE;
+#define KMX_FEWK_WAVE(KS_, NFB_)                                                                           \
+    do {                                                                                                  \
+        hipLaunchKernelGGL((lloyd_fewk_wave_kernel<KS_, NFB_>), dim3((unsigned)wgrid), dim3(256), wave_lds, \
+                           stream, (const float*)X_rowmajor, (const float*)w, (const float*)centroids_t,  \
+                           half_norms, labels_prev, labels, partial, status, n, d, k);                    \
+        KMX_LAUNCH_CHECK();                                                                               \
+        if (events) (void)hipEventRecord(events[1], stream);                                              \
+        KMX_FEWK_REDUCE(NFB_, true, (int)wgrid);                                                          \
+    } while (0)
+        if (nfb_t == 5) KMX_FEWK_WAVE(20, 5);
+        else if (nfb_t == 7) KMX_FEWK_WAVE(28, 7);
+        else KMX_FEWK_WAVE(32, 9);
+#undef KMX_FEWK_WAVE
+    } else {
 #define KMX_FEWK_LAUNCH_RM(KW_, SL_, RM_)                                                                  \
     do {                                                                                                  \
         if (sh.lds > 64 * 1024) {                                                                         \
@@ -529,42 +747,25 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
                            (const float*)centroids_t, half_norms, labels_prev, labels, partial, status,   \
                            n, d, k, vec_ok);                                                              \
     } while (0)
-#define KMX_FEWK_LAUNCH(KW_, SL_)                \
-    do {                                         \
-        if (rm)                                  \
-            KMX_FEWK_LAUNCH_RM(KW_, SL_, true);  \
-        else                                     \
-            KMX_FEWK_LAUNCH_RM(KW_, SL_, false); \
+#define KMX_FEWK_LAUNCH(KW_, SL_, FBW_)                                     \
+    do {                                                                   \
+        if (rm)                                                            \
+            KMX_FEWK_LAUNCH_RM(KW_, SL_, true);                            \
+        else                                                               \
+            KMX_FEWK_LAUNCH_RM(KW_, SL_, false);                           \
+        KMX_LAUNCH_CHECK();                                                \
+        if (events) (void)hipEventRecord(events[1], stream);               \
+        KMX_FEWK_REDUCE(FBW_, false, grid);                                \
     } while (0)
-    if (sh.kw == 8 && sh.s_log == 5) KMX_FEWK_LAUNCH(8, 5);
-    else if (sh.kw == 16 && sh.s_log == 5) KMX_FEWK_LAUNCH(16, 5);
-    else if (sh.kw == 32 && sh.s_log == 5) KMX_FEWK_LAUNCH(32, 5);
-    else if (sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4);
-    else if (sh.kw == 52 && sh.s_log == 4) KMX_FEWK_LAUNCH(52, 4);
-    else if (sh.kw == 76 && sh.s_log == 4) KMX_FEWK_LAUNCH(76, 4);
-    else return KMX_ERR_UNSUPPORTED;
+        if (sh.kw == 8 && sh.s_log == 5) KMX_FEWK_LAUNCH(8, 5, 3);
+        else if (sh.kw == 16 && sh.s_log == 5) KMX_FEWK_LAUNCH(16, 5, 5);
+        else if (sh.kw == 32 && sh.s_log == 5) KMX_FEWK_LAUNCH(32, 5, 9);
+        else if (sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4, 9);
+        else if (sh.kw == 52 && sh.s_log == 4) KMX_FEWK_LAUNCH(52, 4, 14);
+        else if (sh.kw == 76 && sh.s_log == 4) KMX_FEWK_LAUNCH(76, 4, 20);
+        else return KMX_ERR_UNSUPPORTED;
 #undef KMX_FEWK_LAUNCH_RM
 #undef KMX_FEWK_LAUNCH
-    KMX_LAUNCH_CHECK();
-    if (events) (void)hipEventRecord(events[1], stream);
-    const size_t tail_lds = (size_t)(d + 1) * k * sizeof(float);
-    const unsigned red_grid = (unsigned)((slots + 31) / 32);
-#define KMX_FEWK_REDUCE(FBW_)                                                                              \
-    do {                                                                                                  \
-        if (tail_lds > 64 * 1024) {                                                                       \
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fewk_reduce_kernel<FBW_>), \
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds); \
-            if (e != hipSuccess) return (int32_t)e;                                                       \
-        }                                                                                                 \
-        hipLaunchKernelGGL((fewk_reduce_kernel<FBW_>), dim3(red_grid), dim3(256), tail_lds, stream, partial, grid, \
-                           gsum, q_exp, d, k, tail);                                                      \
-    } while (0)
-    switch (fbw_t) {
-        case 3: KMX_FEWK_REDUCE(3); break;
-        case 5: KMX_FEWK_REDUCE(5); break;
-        case 9: KMX_FEWK_REDUCE(9); break;
-        case 14: KMX_FEWK_REDUCE(14); break;
-        default: KMX_FEWK_REDUCE(20); break;
     }
 #undef KMX_FEWK_REDUCE
     KMX_LAUNCH_CHECK();

@@ -375,10 +375,13 @@ def test_numpy_inputs_are_uploaded_through_pinned_staging(cuda):
 # steps.  A fit from the same explicit centres must follow scikit-learn's iterations: same number
 # of iterations, the same labels up to samples on a boundary, inertia and centres to rounding.
 @pytest.mark.parametrize("shape", [(20_000, 14, 127, np.float32, 61), (20_000, 4, 30, np.float32, 31), (20_000, 40, 30, np.float32, 61),
-                                   (20_000, 32, 64, np.float64, 51), (6_000, 70, 300, np.float32, 42),
+                                   (20_000, 32, 64, np.float64, 71), (20_000, 64, 100, np.float64, 51),
+                                   (6_000, 70, 300, np.float32, 42),
                                    (6_000, 300, 40, np.float32, 63), (6_000, 100, 100, np.float64, 63),
-                                   (20_000, 32, 400, np.float64, 53), (20_000, 100, 10, np.float32, 1),
-                                   (20_000, 20, 8, np.float64, 11), (1_500, 784, 10, np.float32, 63)])
+                                   (20_000, 32, 400, np.float64, 53), (20_000, 100, 10, np.float32, 81),
+                                   (20_000, 100, 10, np.float64, 1),
+                                   (20_000, 20, 8, np.float64, 11), (1_500, 784, 10, np.float32, 81),
+                                   (6_000, 300, 20, np.float32, 63)])
 def test_fit_follows_scikit_learn_on_every_kernel_family(cuda, shape):
     from sklearn_numba_dpex_amd import _capi
     from sklearn_numba_dpex_amd.kmeans.estimator import KMeans

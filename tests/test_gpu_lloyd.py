@@ -83,6 +83,10 @@ def _small_configs():
         "K32g": lambda: dict(_blob_config(300_000, 70, 5, np.float32, 37), variant=81),
         "K32h": lambda: dict(_blob_config(6_000, 513, 1, np.float32, 54), variant=81),
         "K32i": lambda: dict(_blob_config(8_000, 200, 12, np.float32, 55, skew=True), variant=81),
+        # up to 128 features (a multiple of 4) with the row-major copy: every wave on tiles of its own
+        "K32j": lambda: dict(_blob_config(50_001, 128, 16, np.float32, 56), variant=81),
+        "K32k": lambda: dict(_blob_config(10_000, 68, 3, np.float32, 57), variant=81),
+        "K32l": lambda: dict(_blob_config(30_003, 112, 9, np.float32, 58, skew=True), variant=81),
         "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
         # extremes of the tiled product: thousands of features (many passes of the bucketed sums),
         # more clusters than the bucket counts hold in LDS and than the wide path takes
@@ -135,7 +139,8 @@ def _odd_config():
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
                                   "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
-                                  "K32a", "K32b", "K32c", "K32d", "K32e", "K32f", "K32g", "K32h", "K32i"])
+                                  "K32a", "K32b", "K32c", "K32d", "K32e", "K32f", "K32g", "K32h", "K32i",
+                                  "K32j", "K32k", "K32l"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
