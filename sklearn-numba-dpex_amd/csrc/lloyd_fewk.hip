@@ -543,8 +543,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void l
 }
 
 // Sum of the workgroups' partial sums, slot by slot and always in the same order, then the end of
-// the iteration.  A workgroup takes 32 slots; its 256 threads are 8 groups that each add every
-// eighth partial (sixteen loads in flight), and the groups are added in order.  The totals go
+// the iteration.  A workgroup takes 32 slots; its 1024 threads are 32 groups that each add every
+// 32nd partial (sixteen loads in flight), and the groups are added in order.  The totals go
 // into the 64-bit fixed-point sums of the run, (d + 1, k) feature-major with the sizes in row d,
 // by device-scope stores, and the workgroup that gets done last finishes the iteration - empty
 // clusters, division, shift, convergence test, what the next step needs - reading them with
@@ -552,7 +552,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void l
 // PER_WAVE: the partials are those of lloyd_fewk_wave_kernel - FBW blocks of 16 features each,
 // block fb in slots 256 fb .. 256 fb + 255.
 template <int FBW, bool PER_WAVE>
-__global__ __launch_bounds__(256) void fewk_reduce_kernel(const float* __restrict__ partial, int n_partials,
+__global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restrict__ partial, int n_partials,
                                                           unsigned long long* __restrict__ gsum,
                                                           const int* __restrict__ q_exp, int d, int k,
                                                           const LloydTail<float> tail) {
@@ -560,28 +560,36 @@ __global__ __launch_bounds__(256) void fewk_reduce_kernel(const float* __restric
     kmx_lloyd_status* status = tail.status;
     if (status->state != KMX_RUNNING) return;
     constexpr int NSLOT = (PER_WAVE ? 1 : 4) * FBW * 256;
-    __shared__ float group_sum[8][32];
+    constexpr int GROUPS = 32;
+    __shared__ float group_sum[GROUPS][32];
     const int sl = threadIdx.x & 31, pg = threadIdx.x >> 5;
     const int slot = blockIdx.x * 32 + sl;
     float total = 0.0f;
     if (slot < NSLOT) {
         const float* src = partial + slot;
         int p = pg;
-        for (; p + 8 * 15 < n_partials; p += 8 * 16) {
+        for (; p + GROUPS * 15 < n_partials; p += GROUPS * 16) {
             float v[16];
 #pragma unroll
-            for (int u = 0; u < 16; ++u) v[u] = src[(size_t)(p + 8 * u) * NSLOT];
+            for (int u = 0; u < 16; ++u) v[u] = src[(size_t)(p + GROUPS * u) * NSLOT];
 #pragma unroll
             for (int u = 0; u < 16; ++u) total += v[u];
         }
-        for (; p < n_partials; p += 8) total += src[(size_t)p * NSLOT];
+        {
+            // (the rest, its loads issued together as well)
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = p + GROUPS * u < n_partials ? src[(size_t)(p + GROUPS * u) * NSLOT] : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 16; ++u) total += v[u];
+        }
     }
     group_sum[pg][sl] = total;
     __syncthreads();
     if (threadIdx.x < 32 && slot < NSLOT) {
         float v = group_sum[0][sl];
 #pragma unroll
-        for (int g = 1; g < 8; ++g) v += group_sum[g][sl];
+        for (int g = 1; g < GROUPS; ++g) v += group_sum[g][sl];
         // slot -> (feature, cluster): wave-of-the-step, block, register, lane
         const int lane = slot & 63, r = (slot >> 6) & 3, wi = slot >> 8;  // wi = wave FBW + i
         const int wave = wi / FBW, i = wi - wave * FBW;
@@ -706,7 +714,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
             if (e != hipSuccess) return (int32_t)e;                                                       \
         }                                                                                                 \
         hipLaunchKernelGGL((fewk_reduce_kernel<FBW_, PW_>),                                               \
-                           dim3((unsigned)(((PW_ ? 1 : 4) * FBW_ * 256 + 31) / 32)), dim3(256), tail_lds, \
+                           dim3((unsigned)(((PW_ ? 1 : 4) * FBW_ * 256 + 31) / 32)), dim3(1024), tail_lds, \
                            stream, partial, N_PARTIALS, gsum, q_exp, d, k, tail);                         \
     } while (0)
     if (rm && d <= 128) {
