@@ -483,9 +483,10 @@ def one_shape(name, n, d, k, dtype, reps=8):
     s = np.dtype(dtype).itemsize
     log(f"[bench] {name}: variant {variant}, {wall_ms:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
     return {"shape": name, "kernel_variant": variant, "ms_per_iter": wall_ms,
-            "label_and_sum_kernels_ms": float(kms[0]),
+            "label_and_sum_kernels_ms": float(kms[0]), "reduce_and_finalize_ms": float(kms[1] + kms[2]),
             "TFLOPs": lloyd_flops(n, d, k) / (wall_ms * 1e-3) / 1e12,
-            "X_bytes_per_iter_TBs": n * d * s / (wall_ms * 1e-3) / 1e12}
+            "X_bytes_per_iter_TBs": n * d * s / (wall_ms * 1e-3) / 1e12,
+            "frac_of_hbm_peak": n * d * s / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
 def gpu_components(cfg):

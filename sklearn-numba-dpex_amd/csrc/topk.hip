@@ -51,9 +51,11 @@ struct TopkState {
 constexpr int TOPK_MAX_SEGMENTS = 256;  // workgroups per row of the passes that read the row
 
 struct TopkLayout {
-    size_t off_state, off_hist, off_counts, off_keys, off_idx, off_cand_keys, off_cand_idx, row_bytes;
+    size_t off_state, off_hist, off_counts, off_keys, off_idx, off_cand_keys, off_cand_idx, off_small, row_bytes;
     int64_t n_seg, seg_cap;  // segments of the side buffer (one per workgroup of pass 1) and their capacity
 };
+
+size_t topk_small_bytes(int64_t n, int32_t k);  // (the one-read path for small k, further down)
 
 TopkLayout topk_layout(int64_t rows, int64_t n, int32_t k, int32_t dtype) {
     TopkLayout L;
@@ -73,7 +75,8 @@ TopkLayout topk_layout(int64_t rows, int64_t n, int32_t k, int32_t dtype) {
     L.off_idx = L.off_keys + kmx_align256((size_t)k * sizeof(unsigned long long));
     L.off_cand_keys = L.off_idx + kmx_align256((size_t)k * sizeof(long long));
     L.off_cand_idx = L.off_cand_keys + kmx_align256(cap * kmx_dtype_size(dtype));
-    L.row_bytes = L.off_cand_idx + kmx_align256(cap * sizeof(long long));
+    L.off_small = L.off_cand_idx + kmx_align256(cap * sizeof(long long));
+    L.row_bytes = L.off_small + topk_small_bytes(n, k);
     return L;
 }
 
@@ -533,10 +536,272 @@ __global__ __launch_bounds__(256) void topk_order_kernel(const T* __restrict__ v
     if (out_values) out_values[o] = values[(size_t)blockIdx.y * a.n + ii];
 }
 
+// ------------------------------------------------------------------------------------------
+// Small k on one row of moderate length: ONE read of the row and two launches.
+//
+// Every element is an item (key, index), ordered by descending key, then ascending index: no two
+// items are equal, so "the k largest" needs no rule for ties.  A workgroup of 1024 threads takes
+// VPT elements per thread into registers.  The k-th largest of the 1024 THREAD MAXIMA (a radix
+// select over their bytes, a histogram of 256 bins in LDS per byte) is a threshold that at least
+// k items reach and that at most k threads have an item above: the items that reach it - at most
+// k VPT - are collected in LDS and ranked against each other, and those of rank below k are the
+// workgroup's k largest, in order.  A second launch of one workgroup does the same with the
+// workgroups' results and writes the answer.
+constexpr int TOPK_SMALL_K = 64;       // largest k of this path
+constexpr int TOPK_SMALL_CAND = 2048;  // items the ranking step holds (k * items per thread at most)
+constexpr int TOPK_SMALL_WGS = 1024;   // workgroups of the first launch at most
+
+template <typename T>
+struct SmallItem {
+    typename KeyOf<T>::U key;  // 0: no item (every real key is above it)
+    uint32_t idx;
+};
+template <typename T>
+__device__ __forceinline__ bool item_gt(const SmallItem<T>& a, const SmallItem<T>& b) {
+    return a.key > b.key || (a.key == b.key && a.idx < b.idx);
+}
+
+// The k largest of the workgroup's items (NV per thread, in registers), written in order to
+// top_key / top_idx (k entries, no-item fillers at the end when there are fewer).  Every thread
+// of the 1024 calls it.
+template <typename T, int NV>
+__device__ inline void small_topk_of_workgroup(const SmallItem<T> (&items)[NV], int k,
+                                               typename KeyOf<T>::U* __restrict__ top_key,
+                                               uint32_t* __restrict__ top_idx) {
+    using U = typename KeyOf<T>::U;
+    constexpr int KEY_BYTES = (int)sizeof(U), PASSES = KEY_BYTES + 4;
+    __shared__ unsigned int hist[256];
+    __shared__ unsigned int sel_digit, sel_rem, n_cand, n_valid;
+    __shared__ U cand_key[TOPK_SMALL_CAND];
+    __shared__ uint32_t cand_idx[TOPK_SMALL_CAND];
+    SmallItem<T> best = items[0];
+#pragma unroll
+    for (int v = 1; v < NV; ++v)
+        if (item_gt<T>(items[v], best)) best = items[v];
+    if (threadIdx.x < 256) hist[threadIdx.x] = 0u;
+    if (threadIdx.x == 0) {
+        n_cand = 0u;
+        n_valid = 0u;
+        sel_rem = 0u;
+    }
+    __syncthreads();
+    const unsigned long long has = __ballot(best.key != 0);
+    if ((threadIdx.x & 63) == 0 && has) atomicAdd(&n_valid, (unsigned int)__popcll(has));
+    __syncthreads();
+    // threshold: the k-th largest thread maximum, byte by byte from the top (key, then inverted
+    // index); with at most k maxima every item passes
+    SmallItem<T> thr;
+    thr.key = 0;
+    thr.idx = 0xffffffffu;
+    if (n_valid > (unsigned int)k) {
+        bool alive = best.key != 0;
+        unsigned int rem = (unsigned int)k;  // the threshold is the rem-th largest of the maxima still alive
+        U pk = 0;
+        uint32_t pi = 0;  // (of the inverted index)
+        for (int p = 0; p < PASSES; ++p) {
+            const unsigned int digit = p < KEY_BYTES ? (unsigned int)(best.key >> (8 * (KEY_BYTES - 1 - p))) & 255u
+                                                     : ((~best.idx) >> (8 * (PASSES - 1 - p))) & 255u;
+            if (alive) atomicAdd(&hist[digit], 1u);
+            __syncthreads();
+            if (threadIdx.x < 64) {
+                // lane l: the bins 4 l .. 4 l + 3; the bin in which the count from the top reaches rem
+                const unsigned int b0 = hist[4 * threadIdx.x], b1 = hist[4 * threadIdx.x + 1],
+                                   b2 = hist[4 * threadIdx.x + 2], b3 = hist[4 * threadIdx.x + 3];
+                const unsigned int mine = b0 + b1 + b2 + b3;
+                // count in the bins of the higher lanes: an inclusive suffix sum over the lanes, by doubling
+                unsigned int suffix = mine;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const unsigned int o = __shfl_down(suffix, off, 64);
+                    if ((int)threadIdx.x + off < 64) suffix += o;
+                }
+                const unsigned int above = suffix - mine;
+                if (above < rem && rem <= above + mine) {
+                    unsigned int acc = above, d = 4 * threadIdx.x + 3, left = rem;
+                    const unsigned int bins[4] = {b3, b2, b1, b0};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (acc < rem && rem <= acc + bins[j]) {
+                            d = 4 * threadIdx.x + 3 - j;
+                            left = rem - acc;
+                        }
+                        acc += bins[j];
+                    }
+                    sel_digit = d;
+                    sel_rem = left;
+                }
+            }
+            __syncthreads();
+            const unsigned int sd = sel_digit;
+            rem = sel_rem;
+            alive = alive && digit == sd;
+            if (p < KEY_BYTES)
+                pk |= (U)sd << (8 * (KEY_BYTES - 1 - p));
+            else
+                pi |= sd << (8 * (PASSES - 1 - p));
+            if (threadIdx.x < 256) hist[threadIdx.x] = 0u;
+            __syncthreads();
+        }
+        thr.key = pk;
+        thr.idx = ~pi;
+    }
+    // the items that reach the threshold
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        if (items[v].key != 0 && !item_gt<T>(thr, items[v])) {
+            const unsigned int at = atomicAdd(&n_cand, 1u);
+            if (at < (unsigned int)TOPK_SMALL_CAND) {
+                cand_key[at] = items[v].key;
+                cand_idx[at] = items[v].idx;
+            }
+        }
+    }
+    __syncthreads();
+    const int nc = (int)min(n_cand, (unsigned int)TOPK_SMALL_CAND);
+    for (int j = nc + (int)threadIdx.x; j < k; j += blockDim.x) {  // (fewer items than k: fillers at the end)
+        top_key[j] = 0;
+        top_idx[j] = 0xffffffffu;
+    }
+    for (int c = threadIdx.x; c < nc; c += blockDim.x) {
+        SmallItem<T> me;
+        me.key = cand_key[c];
+        me.idx = cand_idx[c];
+        int rank = 0;
+        for (int j = 0; j < nc; ++j) {
+            SmallItem<T> o;
+            o.key = cand_key[j];
+            o.idx = cand_idx[j];
+            rank += item_gt<T>(o, me) ? 1 : 0;
+        }
+        if (rank < k) {
+            top_key[rank] = me.key;
+            top_idx[rank] = me.idx;
+        }
+    }
+}
+
+template <typename T, int VPT>
+__global__ __launch_bounds__(TOPK_WG) void topk_small_partial_kernel(const T* __restrict__ values, int64_t n, int k,
+                                                                     typename KeyOf<T>::U* __restrict__ part_key,
+                                                                     uint32_t* __restrict__ part_idx, int vec_ok) {
+    constexpr int VEC = KeyOf<T>::VEC, NL = VPT / VEC;  // 128-bit loads per thread
+    SmallItem<T> items[VPT];
+    const int64_t base = (int64_t)blockIdx.x * (TOPK_WG * VPT);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const int64_t i0 = base + ((int64_t)j * TOPK_WG + threadIdx.x) * VEC;
+        T v[VEC];
+        if (vec_ok && i0 + VEC <= n) {
+            const uint4 q = *reinterpret_cast<const uint4*>(values + i0);
+            if (VEC == 4) {
+                v[0] = KeyOf<T>::from_bits(q.x, 0);
+                v[1] = KeyOf<T>::from_bits(q.y, 0);
+                v[VEC - 2] = KeyOf<T>::from_bits(q.z, 0);
+                v[VEC - 1] = KeyOf<T>::from_bits(q.w, 0);
+            } else {
+                v[0] = KeyOf<T>::from_bits(q.x, q.y);
+                v[VEC - 1] = KeyOf<T>::from_bits(q.z, q.w);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = i0 + e < n ? values[i0 + e] : T(0);
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            items[j * VEC + e].key = i0 + e < n ? KeyOf<T>::key(v[e]) : 0;
+            items[j * VEC + e].idx = (uint32_t)(i0 + e);
+        }
+    }
+    small_topk_of_workgroup<T, VPT>(items, k, part_key + (size_t)blockIdx.x * k, part_idx + (size_t)blockIdx.x * k);
+}
+
+template <typename T, int IPT>
+__global__ __launch_bounds__(TOPK_WG) void topk_small_merge_kernel(const T* __restrict__ values, int n_items, int k,
+                                                                   const typename KeyOf<T>::U* __restrict__ part_key,
+                                                                   const uint32_t* __restrict__ part_idx,
+                                                                   int64_t* __restrict__ out_idx,
+                                                                   T* __restrict__ out_values) {
+    using U = typename KeyOf<T>::U;
+    __shared__ U top_key[TOPK_SMALL_K];
+    __shared__ uint32_t top_idx[TOPK_SMALL_K];
+    SmallItem<T> items[IPT];
+#pragma unroll
+    for (int v = 0; v < IPT; ++v) {
+        const int i = v * TOPK_WG + (int)threadIdx.x;
+        items[v].key = i < n_items ? part_key[i] : 0;
+        items[v].idx = i < n_items ? part_idx[i] : 0xffffffffu;
+    }
+    small_topk_of_workgroup<T, IPT>(items, k, top_key, top_idx);
+    __syncthreads();
+    for (int j = threadIdx.x; j < k; j += TOPK_WG) {
+        if (top_key[j] != 0) {  // (k <= n: every slot is filled)
+            if (out_idx) out_idx[j] = (int64_t)top_idx[j];
+            if (out_values) out_values[j] = values[top_idx[j]];
+        }
+    }
+}
+
+// Elements per thread of the first launch (0: the row is not for this path).
+template <typename T>
+int topk_small_vpt(int64_t rows, int64_t n, int32_t k) {
+    if (rows != 1 || k > TOPK_SMALL_K || n >= ((int64_t)1 << 32) - 1) return 0;
+    constexpr int VEC = KeyOf<T>::VEC;
+    for (int vpt = VEC; vpt <= 16; vpt *= 2) {
+        const int64_t g = kmx_cdiv(n, (int64_t)TOPK_WG * vpt);
+        // (few workgroups while the row is short, never more than the second launch can take)
+        if ((g <= 256 || vpt == 16) && g <= TOPK_SMALL_WGS && g * k <= 32 * TOPK_WG && (int64_t)k * vpt <= TOPK_SMALL_CAND)
+            return vpt;
+    }
+    return 0;
+}
+
+template <typename T>
+int32_t topk_small_impl(const T* values, int64_t* out_idx, T* out_values, int64_t n, int32_t k, char* area, int vpt,
+                        hipStream_t stream) {
+    using U = typename KeyOf<T>::U;
+    const int g = (int)kmx_cdiv(n, (int64_t)TOPK_WG * vpt);
+    U* part_key = reinterpret_cast<U*>(area);
+    uint32_t* part_idx = reinterpret_cast<uint32_t*>(area + kmx_align256((size_t)g * k * sizeof(U)));
+    const int vec_ok = (((uintptr_t)values) & 15) == 0;
+#define KMX_TOPK_PART(VPT_)                                                                                     \
+    hipLaunchKernelGGL((topk_small_partial_kernel<T, VPT_>), dim3((unsigned)g), dim3(TOPK_WG), 0, stream, values, n, \
+                       (int)k, part_key, part_idx, vec_ok)
+    if constexpr (KeyOf<T>::VEC == 2) {
+        if (vpt == 2) KMX_TOPK_PART(2);
+    }
+    if (vpt == 4) KMX_TOPK_PART(4);
+    else if (vpt == 8) KMX_TOPK_PART(8);
+    else if (vpt == 16) KMX_TOPK_PART(16);
+#undef KMX_TOPK_PART
+    const int n_items = g * k;
+    const int ipt = (int)kmx_cdiv(n_items, TOPK_WG);
+#define KMX_TOPK_MERGE(IPT_)                                                                                  \
+    hipLaunchKernelGGL((topk_small_merge_kernel<T, IPT_>), dim3(1), dim3(TOPK_WG), 0, stream, values, n_items, \
+                       (int)k, part_key, part_idx, out_idx, out_values)
+    if (ipt <= 1) KMX_TOPK_MERGE(1);
+    else if (ipt <= 2) KMX_TOPK_MERGE(2);
+    else if (ipt <= 4) KMX_TOPK_MERGE(4);
+    else if (ipt <= 8) KMX_TOPK_MERGE(8);
+    else if (ipt <= 16) KMX_TOPK_MERGE(16);
+    else KMX_TOPK_MERGE(32);
+#undef KMX_TOPK_MERGE
+    KMX_LAUNCH_CHECK();
+    return KMX_OK;
+}
+
+// bytes of the first launch's results (the largest grid, the wider key)
+size_t topk_small_bytes(int64_t n, int32_t k) {
+    if (k > TOPK_SMALL_K) return 0;
+    const int64_t g = kmx_cdiv(n, (int64_t)TOPK_WG * 2) < TOPK_SMALL_WGS ? kmx_cdiv(n, (int64_t)TOPK_WG * 2) : TOPK_SMALL_WGS;
+    return kmx_align256((size_t)g * k * 8) + kmx_align256((size_t)g * k * 4);
+}
+
 template <typename T>
 int32_t topk_impl(const void* values_, int64_t* out_idx, void* out_values, int64_t rows, int64_t n, int32_t k,
                   char* ws, int32_t dtype, hipStream_t stream) {
     const TopkLayout L = topk_layout(rows, n, k, dtype);
+    if (const int vpt = topk_small_vpt<T>(rows, n, k); vpt != 0)
+        return topk_small_impl<T>((const T*)values_, out_idx, (T*)out_values, n, k, ws + L.off_small, vpt, stream);
     // rows are taken in slices of the grid's second dimension
     for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
         const int64_t nr = rows - r0 < 65535 ? rows - r0 : 65535;

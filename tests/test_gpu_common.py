@@ -170,6 +170,35 @@ def test_topk_large_with_ties_and_negatives(cuda, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [1, 63, 1_024, 4_097, 65_537, 262_145, 1_048_577, 4_200_003, 16_000_001])
+def test_topk_of_one_row_for_small_k(cuda, dtype, n):
+    """One row and k <= 64 take the path that reads the row once (per workgroup the k largest via
+    the thread maxima, then one workgroup over the workgroups' results): every tier of elements
+    per thread, rows that are sorted either way (all the large values in one thread or one in
+    each), constant rows and rows of few distinct values (ties everywhere: lowest index first)."""
+    from sklearn_numba_dpex_amd.common.topk import topk, topk_idx
+
+    rng = np.random.default_rng(n)
+    rows = {
+        "random": rng.normal(size=n),
+        "ascending": np.arange(n, dtype=np.float64),
+        "descending": -np.arange(n, dtype=np.float64),
+        "constant": np.full(n, -1.5),
+        "few values": rng.integers(0, 3, n).astype(np.float64),
+    }
+    for name, v in rows.items():
+        v = v.astype(dtype)
+        d_v = _dev(v, cuda)
+        for k in (1, 16, 64):
+            if k > n:
+                continue
+            want = ok.top_k_indices(v, k)
+            np.testing.assert_array_equal(topk_idx(d_v, k).cpu().numpy(), want, err_msg=f"{name}, k={k}")
+        k = min(5, n)
+        np.testing.assert_array_equal(topk(d_v, k).cpu().numpy(), v[ok.top_k_indices(v, k)], err_msg=name)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_elementwise_kernels(cuda, dtype):
     from sklearn_numba_dpex_amd.common import kernels
 
