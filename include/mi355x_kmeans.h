@@ -229,7 +229,8 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
  * samples (vector ALU), 3 = MFMA (fp32) with the centroids resident in LDS, 4 = MFMA (fp32)
  * with samples in registers and centroids streamed (more than 256 clusters), 5 = MFMA (fp64)
  * with the centroids resident in LDS, 6 = labels by a tiled matrix-core product (any shape,
- * fp32 and fp64); accumulation 1 = workgroup-private LDS accumulators, 2 = global sums,
+ * fp32 and fp64), 8 = fp32 with up to 16 clusters and 65 .. 1216 features: a tile of samples on chip
+ * serves labels and sums on the matrix cores, X read once; accumulation 1 = workgroup-private LDS accumulators, 2 = global sums,
  * 3 = labels only, then sums by a kernel of their own (per bucket of samples sorted by label,
  * or, fp32, straight from the labels into fixed-point accumulators in LDS where those of every
  * cluster fit).  61 is path 3 with the labels screened on the fp16 matrix cores; 71 is the same
@@ -238,8 +239,8 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
 int32_t kmx_lloyd_kernel_variant(int64_t n, int32_t d, int32_t k, int32_t dtype, uint32_t flags);
 
 /* 1 when the plan's kernels read the row-major copy of X that kmx_lloyd_iter takes as
- * `X_rowmajor` (the wide fp32 step always; the sums per bucket of samples optionally, NULL makes
- * them gather the feature-major array), 0 when they ignore it, negative: error.  Host only.
+ * `X_rowmajor` (the wide fp32 step always; the sums per bucket of samples and the few-cluster step
+ * optionally, NULL makes them read the feature-major array), 0 when they ignore it, negative: error.  Host only.
  * Has no counterpart in the reference, whose kernels read one layout (the transposed copy made
  * in sklearn_numba_dpex/kmeans/engine.py:88-98): it lets a caller skip the second copy of X. */
 int32_t kmx_lloyd_plan_reads_rowmajor(const kmx_lloyd_plan* plan);
