@@ -210,12 +210,15 @@ def test_score_path_and_topk_at_full_size(cuda):
 
 
 @pytest.mark.parametrize("shape", [(2_000_000, 100, 100, np.float64, 63), (1_000_000, 32, 500, np.float64, 53),
-                                   (500_000, 300, 300, np.float32, 63), (2_000_000, 100, 10, np.float32, 1),
-                                   (2_000_000, 48, 64, np.float32, 61), (1_000_000, 64, 128, np.float64, 51)])
+                                   (500_000, 300, 300, np.float32, 63), (2_000_000, 100, 10, np.float32, 81),
+                                   (2_000_000, 100, 10, np.float64, 1), (300_000, 784, 10, np.float32, 81),
+                                   (2_000_000, 48, 64, np.float32, 61), (1_000_000, 64, 128, np.float64, 51),
+                                   (2_000_000, 48, 64, np.float64, 71)])
 def test_large_shapes_off_the_benchmark_configurations(cuda, shape):
     """The same properties on large inputs of the other kernel families: the tiled matrix-core
-    product and the fp64 matrix-core labels with bucketed sums, the streaming vector-ALU step,
-    the screened step with three K steps, the fp64 step with a compute unit's whole LDS."""
+    product and the fp64 matrix-core labels with bucketed sums, the few-cluster step (per-wave and
+    per-workgroup tiles), the streaming vector-ALU step, the screened step with three K steps on
+    fp32 and fp64 inputs, the fp64 step with a compute unit's whole LDS."""
     from sklearn_numba_dpex_amd import _capi
     from sklearn_numba_dpex_amd.kmeans import drivers
 
