@@ -605,7 +605,7 @@ __global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restri
     if (threadIdx.x == 0) is_last = (atomicAdd(&status->ticket, 1u) == gridDim.x - 1) ? 1u : 0u;
     __syncthreads();
     if (is_last != 0u) {
-        lloyd_small_finalize_body<float, true, true>(gsum, q_exp, tail, reinterpret_cast<float*>(red_raw));
+        lloyd_small_finalize_body<float, true, true, true>(gsum, q_exp, tail, reinterpret_cast<float*>(red_raw));
         if (threadIdx.x == 0) status->ticket = 0u;
     }
 }

@@ -176,7 +176,9 @@ __device__ inline void lloyd_finalize_block(const LloydTail<T>& a, int n_empty, 
 //             changed-label count and the counter word with device-scope atomics (and waited for
 //             them before they drew their ticket): those words are read with device-scope loads,
 //             which do not stop at a cache of the own chiplet that may hold an older copy.
-template <typename T, bool FROM_GSUM, bool COHERENT>
+//   WIDE: hundreds of features and few clusters, at most as many as threads (takes 4 KB of LDS
+//         more: a cluster's norm by a group of threads).
+template <typename T, bool FROM_GSUM, bool COHERENT, bool WIDE = false>
 __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict__ gsum,
                                                  const int* __restrict__ q_exp, const LloydTail<T>& a,
                                                  T* __restrict__ vals) {
@@ -321,11 +323,31 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
         }
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < k; c += n_threads) {
+    if constexpr (WIDE) {
+        // wide samples, few clusters: a cluster's norm by a group of threads (thread (g, c) takes
+        // every n_g-th feature, the groups are then added in order) - one thread per cluster
+        // would walk hundreds of features alone while the others wait
+        __shared__ T norm_part[1024];
+        const int n_g = n_threads / k;
+        const int c = (int)threadIdx.x % k, g = (int)threadIdx.x / k;
         T sq = T(0);
-        for (int f = 0; f < d; ++f) sq += vals[f * k + c] * vals[f * k + c];
-        a.half_norms[c] = sq / T(2);
-        for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = T(0);
+        if (g < n_g)
+            for (int f = g; f < d; f += n_g) sq += vals[f * k + c] * vals[f * k + c];
+        norm_part[threadIdx.x] = sq;
+        __syncthreads();
+        if ((int)threadIdx.x < k) {
+            T tot = norm_part[threadIdx.x];
+            for (int g2 = 1; g2 < n_g; ++g2) tot += norm_part[g2 * k + threadIdx.x];
+            a.half_norms[threadIdx.x] = tot / T(2);
+            for (int f = d; f < dpad; ++f) a.cpack[(size_t)threadIdx.x * dpad + f] = T(0);
+        }
+    } else {
+        for (int c = threadIdx.x; c < k; c += n_threads) {
+            T sq = T(0);
+            for (int f = 0; f < d; ++f) sq += vals[f * k + c] * vals[f * k + c];
+            a.half_norms[c] = sq / T(2);
+            for (int f = d; f < dpad; ++f) a.cpack[(size_t)c * dpad + f] = T(0);
+        }
     }
     const double total = kmx_block_sum<double>(shift, scratch);
     if (threadIdx.x == 0) lloyd_update_status(a.status, total, n_changed);
