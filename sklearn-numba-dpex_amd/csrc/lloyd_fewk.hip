@@ -14,23 +14,29 @@
 //   * labels: scores(16 clusters x 16 samples) = C (16 x d) X_tile (d x 16) - 0.5||c||^2 with
 //     v_mfma_f32_16x16x4_f32 (A: lane l = cluster l % 16, feature l / 16; B: lane l = feature
 //     l / 16, sample l % 16; D: lane l holds clusters 4 (l / 16) + r of sample l % 16).  Each of
-//     the four waves takes a quarter of the features, whose centroid values it holds in
-//     registers for the whole kernel, and the four partial score tiles are added in wave order
-//     by one thread per sample (strict '>' in increasing cluster order: the lowest index wins).
+//     the NW waves (four; eight beyond 512 features) takes its share of the features, whose
+//     centroid values it holds in registers for the whole kernel, and the partial score tiles
+//     are added in wave order (strict '>' in increasing cluster order: the lowest index wins).
 //   * sums: sums(16 clusters x 16 features) += M (16 clusters x 4 samples) X_tile^T (4 samples x
 //     16 features), M = w_i where sample i carries the row's label and 0 elsewhere; the feature
 //     row d of the tile holds ones, so column d collects the cluster sizes.  A wave owns every
-//     fourth block of 16 features and keeps their accumulators in registers until the end.
+//     NW-th block of 16 features and keeps their accumulators in registers until the end.
 //
 // The rows of the next tile travel from memory into registers while the tile in LDS is worked
-// on.  fp32 accumulation per workgroup (a few thousand samples), the workgroups' partial sums
-// are added by lloyd_reduce_kernel.
+// on - or, beyond 512 features with a row-major copy of X, straight into LDS, two workgroups per
+// compute unit taking turns at waiting and working.  fp32 accumulation per workgroup (a few
+// thousand samples); fewk_reduce_kernel adds the workgroups' partial sums and finishes the iteration.
 #include "lloyd_layout.h"
 #include "lloyd_tail.h"
 
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Barrier between two passes over the LDS of a workgroup: the wave's own LDS accesses are done, then
+// the barrier.  (__syncthreads() is a fence as well, and a fence waits for every load from memory
+// into LDS that is in flight - the next tile, which is wanted only a whole tile later.)
+__device__ __forceinline__ void fewk_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 struct FewkLds {
     size_t off_part, off_lab, off_w, total;
@@ -40,30 +46,32 @@ struct FewkLds {
                  // (either way the lanes of a matrix operand fall on different banks, nearly)
 };
 
-// K steps of four features per wave for d features
-__host__ __device__ constexpr int fewk_kw(int d) { return (((d + 3) / 4) + 3) / 4; }
+// K steps of four features per wave for d features shared by nw waves
+__host__ __device__ constexpr int fewk_kw(int d, int nw) { return (((d + 3) / 4) + nw - 1) / nw; }
 
-__host__ __device__ inline FewkLds fewk_lds(int d, int S) {
+__host__ __device__ inline FewkLds fewk_lds(int d, int S, int nw, bool two_tiles = false) {
     FewkLds s;
-    const int kw = fewk_kw(d);
-    // the label pass of the last wave reads K steps 3 kw .. 3 kw + 8 ceil(kw / 8) - 1 (with zero
-    // centroid values past its share), the sums pass blocks of 16 rows up to row d
-    const int rows_k = 4 * (3 * kw + 8 * ((kw + 7) / 8));
+    const int kw = fewk_kw(d, nw);
+    // the label pass of the last wave reads K steps (nw - 1) kw .. (nw - 1) kw + 8 ceil(kw / 8) - 1
+    // (with zero centroid values past its share), the sums pass blocks of 16 rows up to row d
+    const int rows_k = 4 * ((nw - 1) * kw + 8 * ((kw + 7) / 8));
     const int rows_f = 16 * ((d + 1 + 15) / 16);
     s.rows = rows_k > rows_f ? rows_k : rows_f;
     s.stride = S + 4;
     s.ds = s.rows + ((20 - s.rows % 64) + 64) % 64;
     // (room for the larger of the two layouts: the launch does not depend on which one runs)
-    const size_t fm = (size_t)s.rows * s.stride * 4, sm = (size_t)S * s.ds * 4;
-    s.off_part = fm > sm ? fm : sm;                          // [4 waves][S / 16][16 clusters][16 samples]
-    s.off_lab = s.off_part + (size_t)4 * (S / 16) * 256 * 4;
+    // (two_tiles: the sample-major tile twice - one is worked on while the next one arrives)
+    const size_t fm = (size_t)s.rows * s.stride * 4, sm = (size_t)S * s.ds * 4 * (two_tiles ? 2 : 1);
+    s.off_part = fm > sm ? fm : sm;                          // [nw waves][S / 16][16 clusters][16 samples]
+    s.off_lab = s.off_part + (size_t)nw * (S / 16) * 256 * 4;
     s.off_w = s.off_lab + (size_t)S * 4;
     s.total = s.off_w + (size_t)S * 4;
     return s;
 }
 
-// 128-bit pieces of the next tile a thread holds in registers (d * S / 4 values over 256 threads)
-constexpr int fewk_prefetch(int kw, int s_log) {
+// 128-bit pieces of the next tile a thread holds in registers (d * S / 4 values over the threads)
+constexpr int fewk_prefetch(int kw, int s_log, int nw) {
+    if (nw == 8) return kw <= 26 ? 7 : 10;
     return (kw <= 8 && s_log == 5) ? 4 : kw <= 16 ? 8 : kw <= 32 ? 10 : kw <= 52 ? 13 : 19;  // ((8, 6): 8)
 }
 
@@ -73,12 +81,28 @@ constexpr int fewk_prefetch(int kw, int s_log) {
 // RM: the tile is read from the row-major copy of X, (n, d) with d a multiple of 4 - S whole
 // samples are one contiguous stretch of memory, where the feature-major array gives d separate
 // pieces of 4 S bytes - and kept sample-major in LDS.
-// (two waves per SIMD - two workgroups per compute unit - up to 832 features: 256 registers; four
-// with tiles of 32 samples of up to 128 features)
-constexpr int fewk_waves_per_simd(int kw, int s_log) { return (kw <= 8 && s_log == 5) ? 4 : kw <= 52 ? 2 : 1; }
+// NW: waves per workgroup.  Beyond 512 features eight waves share the tile: a wave then holds half as
+// many centroid values, sums and pieces of the next tile, twice as many waves fit a SIMD, and the waits
+// of one wave (the tile's reads before its matrix instructions, the barriers between the passes) are
+// filled by another.
+// (two waves per SIMD - two workgroups of four waves per compute unit - up to 832 features: 256
+// registers; four with tiles of 32 samples of up to 128 features and with eight waves up to 832)
+constexpr int fewk_waves_per_simd(int kw, int s_log, int nw, int direct = 0) {
+    if (nw == 8) return direct == 1 ? 4 : 2;
+    return (kw <= 8 && s_log == 5) ? 4 : kw <= 52 ? 2 : 1;
+}
 
-template <int KW, int S_LOG, bool RM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(fewk_waves_per_simd(KW, S_LOG))))
+// DIRECT (with RM): a tile travels from memory straight into LDS (global_load_lds_dwordx4: the 64
+// lanes of a wave fill 1024 consecutive bytes of a sample's row) instead of into registers, from
+// where the waves had to store it once the tile in LDS was free: no registers are held for it, the
+// reads of a pass can be in flight together, and no wave spends instructions on the copy.
+//   1: one tile per workgroup; the workgroup waits for it, and the other workgroup of the compute
+//      unit works meanwhile (two workgroups of eight waves, 128 registers);
+//   2: two tiles, the next one arrives while this one is worked on (one workgroup per compute unit).
+template <int KW, int S_LOG, bool RM, int NW, int DIRECT = 0>
+__global__ __launch_bounds__(64 * NW)
+__attribute__((amdgpu_waves_per_eu(fewk_waves_per_simd(KW, S_LOG, NW, DIRECT),
+                                   fewk_waves_per_simd(KW, S_LOG, NW, DIRECT))))
 void lloyd_fewk_kernel(
     const float* __restrict__ X_t, const float* __restrict__ X_rm, const float* __restrict__ sample_weight,
     const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
@@ -86,10 +110,13 @@ void lloyd_fewk_kernel(
     float* __restrict__ partial, kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int vec_ok) {
     if (status->state != KMX_RUNNING) return;
     constexpr int FBW = KW / 4 + 1;  // blocks of 16 features per wave
-    constexpr int PF = fewk_prefetch(KW, S_LOG);
+    constexpr int PF = fewk_prefetch(KW, S_LOG, NW);
     constexpr int S = 1 << S_LOG, NB = S >> 4, STRIDE = S + 4;
+    constexpr int NT = 64 * NW;    // threads
+    constexpr int SPW = S / NW;    // samples of the tile a wave fetches
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const FewkLds lay = fewk_lds(d, S);
+    static_assert(!DIRECT || RM, "tiles arrive in LDS directly only from the row-major copy");
+    const FewkLds lay = fewk_lds(d, S, NW, DIRECT == 2);
     float* tile = reinterpret_cast<float*>(smem_raw);                     // [rows][STRIDE]
     float* part = reinterpret_cast<float*>(smem_raw + lay.off_part);
     uint32_t* lab = reinterpret_cast<uint32_t*>(smem_raw + lay.off_lab);  // [S]
@@ -102,34 +129,48 @@ void lloyd_fewk_kernel(
     // masks over its lanes)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int g4 = lane >> 4, m16 = lane & 15;
-    const int kw = fewk_kw(d);  // K steps per wave (<= KW)
+    const int kw = fewk_kw(d, NW);  // K steps per wave (<= KW)
     const int ks0 = wave * kw;
     const int n_fb = (d + 1 + 15) >> 4;  // blocks of 16 features, the row of ones included
-    // wave w takes the blocks w, w + 4, ...: FBW of them whatever d is, a block past the last one
+    // wave w takes the blocks w, w + NW, ...: FBW of them whatever d is, a block past the last one
     // standing for the last (its sums are not written) - no branch inside the loop over the
     // samples, around which the compiler would copy all the accumulators
 
     // the wave's centroid values: cluster m16, feature 4 (ks0 + s) + g4
     float ca[KW];
-#pragma unroll
-    for (int s = 0; s < KW; ++s) {
-        const int f = 4 * (ks0 + s) + g4;
-        ca[s] = (s < kw && f < d && m16 < k) ? centroids_t[(size_t)f * k + m16] : 0.0f;
-    }
     // -0.5||c||^2 of the clusters 4 g4 + r: the start of wave 0's scores
-    v4f start = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (wave == 0) {
+    v4f start;
+    // (every lane loads - a clamped address where it has no value - so that the loads are issued
+    // together: under a condition each one became a block of its own that waited for its value)
+    auto load_centroids = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) start[r] = (4 * g4 + r < k) ? -half_norms[4 * g4 + r] : 0.0f;
-    }
+        for (int s = 0; s < KW; ++s) {
+            const int f = 4 * (ks0 + s) + g4;
+            const bool has = s < kw && f < d && m16 < k;
+            const float v = centroids_t[has ? (size_t)f * k + m16 : (size_t)0];
+            ca[s] = has ? v : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float hn = half_norms[4 * g4 + r < k ? 4 * g4 + r : 0];
+            start[r] = (wave == 0 && 4 * g4 + r < k) ? -hn : 0.0f;
+        }
+    };
+    // (DIRECT: after the first tile has been asked for)
+    if constexpr (!DIRECT) load_centroids();
     // past the features: ones (feature d, the cluster sizes), then zeros; never overwritten
-    if (RM) {
-        for (int idx = threadIdx.x; idx < S * (DS - d); idx += 256) {
+    if (DIRECT) {
+        // (both tiles, and zeros in the rows as well: the rows past the last sample are never loaded)
+        for (int r = wave; r < (DIRECT == 2 ? 2 : 1) * S; r += NW)
+            for (int c = lane; c < DS; c += 64) tile[r * DS + c] = c == d ? 1.0f : 0.0f;
+        fewk_lds_barrier();
+    } else if (RM) {
+        for (int idx = threadIdx.x; idx < S * (DS - d); idx += NT) {
             const int sm = idx / (DS - d), c = idx - sm * (DS - d);
             tile[sm * DS + d + c] = c == 0 ? 1.0f : 0.0f;
         }
     } else {
-        for (int idx = threadIdx.x; idx < (rows - d) * STRIDE; idx += 256)
+        for (int idx = threadIdx.x; idx < (rows - d) * STRIDE; idx += NT)
             tile[d * STRIDE + idx] = idx < STRIDE ? 1.0f : 0.0f;
     }
     if (threadIdx.x == 0) changed_block = 0;
@@ -142,14 +183,14 @@ void lloyd_fewk_kernel(
     // The tile as 128-bit pieces, PF per thread.
     // Feature-major: the thread's piece u is four samples (its quarter q_t of the row... of S / 4)
     // of feature f_t + u * RSTEP.
-    // Row-major: the S / 4 samples of a wave are one contiguous stretch of (S / 4) d floats; lane l
+    // Row-major: the S / NW samples of a wave are one contiguous stretch of (S / NW) d floats; lane l
     // takes its pieces l, l + 64, ...; piece i holds features 4 (i % P) .. + 3 of sample i / P,
     // P = d / 4.
-    constexpr int Q_LOG = S_LOG - 2, RSTEP = 256 >> Q_LOG;
+    constexpr int Q_LOG = S_LOG - 2, RSTEP = NT >> Q_LOG;
     const int f_t = threadIdx.x >> Q_LOG, q_t = threadIdx.x & ((1 << Q_LOG) - 1);
     const size_t x_mine = (size_t)f_t * n + 4 * q_t;  // (the rest of an address is the same for all threads)
     float* const tile_mine = tile + f_t * STRIDE + 4 * q_t;
-    const int P = d >> 2, wave_pieces = (S >> 2) * P;
+    const int P = d >> 2, wave_pieces = SPW * P;
     float4 pf[PF];
     // (and, every fourth thread, the weight and the previous label of one sample)
     float w_next = 0.0f;
@@ -162,9 +203,9 @@ void lloyd_fewk_kernel(
         }
         if constexpr (RM) {
             // (pieces of samples past the end are not read)
-            const int64_t left = n - (s0 + (int64_t)wave * (S >> 2));  // samples of the wave's stretch that exist
-            const int64_t live_pieces = left <= 0 ? 0 : (left >= (S >> 2) ? wave_pieces : left * P);
-            const float4* src = reinterpret_cast<const float4*>(X_rm + (size_t)(s0 + wave * (S >> 2)) * d);
+            const int64_t left = n - (s0 + (int64_t)wave * SPW);  // samples of the wave's stretch that exist
+            const int64_t live_pieces = left <= 0 ? 0 : (left >= SPW ? wave_pieces : left * P);
+            const float4* src = reinterpret_cast<const float4*>(X_rm + (size_t)(s0 + wave * SPW) * d);
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
                 const int i = lane + 64 * u;
@@ -201,7 +242,7 @@ void lloyd_fewk_kernel(
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
                 if (lane + 64 * u < wave_pieces)
-                    *reinterpret_cast<float4*>(tile + (wave * (S >> 2) + sm) * DS + 4 * r) = pf[u];
+                    *reinterpret_cast<float4*>(tile + (wave * SPW + sm) * DS + 4 * r) = pf[u];
                 sm += step_s;
                 r += step_r;
                 if (r >= P) {
@@ -216,26 +257,85 @@ void lloyd_fewk_kernel(
         }
     };
 
+    // DIRECT: the wave's SPW rows of the tile at s0, 64 pieces per instruction, into the tile at word
+    // offset buf of the LDS (weight and previous label travel in registers as above)
+    constexpr int PC = (KW * NW + 63) / 64;  // instructions per row for the widest sample of this kernel
+    const int full_chunks = P >> 6, last_chunk = P & 63;  // instructions of 64 pieces per row, pieces of one more
+    auto issue = [&](const int64_t s0, const int buf) __attribute__((always_inline)) {
+        // (the thread that will write the sample's label holds its weight and previous label)
+        if ((int)threadIdx.x < 16 * S && (threadIdx.x & 15) == 0 && s0 + (threadIdx.x >> 4) < n) {
+            w_next = sample_weight[s0 + (threadIdx.x >> 4)];
+            pl_next = labels_prev[s0 + (threadIdx.x >> 4)];
+        }
+#pragma unroll
+        for (int rr = 0; rr < SPW; ++rr) {
+            const int row = wave * SPW + rr;
+            if (s0 + row < n) {  // wave-uniform
+                const float* src = X_rm + (size_t)(s0 + row) * d + 4 * lane;
+                float* dst = tile + buf + row * DS;
+#pragma unroll
+                for (int c = 0; c < PC; ++c) {
+                    if (c < full_chunks) {  // wave-uniform
+                        __builtin_amdgcn_global_load_lds(
+                            (const __attribute__((address_space(1))) void*)(src + 256 * c),
+                            (__attribute__((address_space(3))) void*)(dst + 256 * c), 16, 0, 0);
+                    } else if (c == full_chunks && lane < last_chunk) {
+                        __builtin_amdgcn_global_load_lds(
+                            (const __attribute__((address_space(1))) void*)(src + 256 * c),
+                            (__attribute__((address_space(3))) void*)(dst + 256 * c), 16, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+
     const int64_t n_tiles = (n + S - 1) >> S_LOG;
     int64_t t = blockIdx.x;
-    if (t < n_tiles) fetch(t << S_LOG);
+    const int tile_words = S * DS;
+    int cur = 0;  // DIRECT: word offset of the tile that is worked on
+    if (t < n_tiles) {
+        if constexpr (DIRECT)
+            issue(t << S_LOG, 0);
+        else
+            fetch(t << S_LOG);
+    }
+    if constexpr (DIRECT) load_centroids();
     // the wave's first row of the label pass (lane: feature g4 of a K step, sample m16 of a block)
     // and of the sums pass (lane: feature m16 of a block of 16, sample g4 of a group of four)
-    const float* const col_labels = RM ? tile + m16 * DS + 4 * ks0 + g4 : tile + (4 * ks0 + g4) * STRIDE + m16;
-    const float* col_sums[FBW];
-#pragma unroll
-    for (int i = 0; i < FBW; ++i) {
-        const int fb = wave + 4 * i < n_fb ? wave + 4 * i : n_fb - 1;
-        col_sums[i] = RM ? tile + g4 * DS + 16 * fb + m16 : tile + (16 * fb + m16) * STRIDE + g4;
-    }
+    const float* const col_labels0 = RM ? tile + m16 * DS + 4 * ks0 + g4 : tile + (4 * ks0 + g4) * STRIDE + m16;
+    // (the wave's blocks w, w + NW, ... lie FB_STEP words apart: one address register per SUMS_G blocks,
+    // the rest of an address is an immediate offset - a register per block, each stepped through the
+    // tile, left the compiler no registers to keep the reads of a group in flight together, and every
+    // matrix instruction waited for a read of its own.  A block past the last one reads whatever lies
+    // there, inside the tile or behind it; its sums are not used.)
+    constexpr int FB_STEP = RM ? 16 * NW : 16 * NW * STRIDE;
+    constexpr int SUMS_G = (15000 / FB_STEP) < FBW ? (15000 / FB_STEP) : FBW;
+    constexpr int SUMS_NBASE = (FBW + SUMS_G - 1) / SUMS_G;
+    const float* const col_sums00 = RM ? tile + g4 * DS + 16 * wave + m16 : tile + (16 * wave + m16) * STRIDE + g4;
+    (void)n_fb;
     for (; t < n_tiles; t += gridDim.x) {
         const int64_t s0 = t << S_LOG;
-        __syncthreads();  // the tile before this one is no longer read
-        deposit();
-        const float w_mine = w_next;
-        const uint32_t pl_mine = pl_next;
-        if (t + gridDim.x < n_tiles) fetch((t + gridDim.x) << S_LOG);
-        __syncthreads();
+        float w_mine;
+        uint32_t pl_mine;
+        if constexpr (DIRECT) {
+            // the tile has arrived (every wave waits for its own rows, then for the others), and the
+            // other tile is no longer read
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            w_mine = w_next;
+            pl_mine = pl_next;
+            if constexpr (DIRECT == 2)
+                if (t + gridDim.x < n_tiles) issue((t + gridDim.x) << S_LOG, tile_words - cur);
+        } else {
+            __syncthreads();  // the tile before this one is no longer read
+            deposit();
+            w_mine = w_next;
+            pl_mine = pl_next;
+            if (t + gridDim.x < n_tiles) fetch((t + gridDim.x) << S_LOG);
+            __syncthreads();
+        }
+        const float* const col_labels = col_labels0 + cur;
+        const float* const col_sums0 = col_sums00 + cur;
 
         // labels: partial scores of the wave's quarter of the features, eight K steps at a time
         // (their reads of the tile, for all sample blocks, in flight together), two chains of
@@ -258,6 +358,9 @@ void lloyd_fewk_kernel(
                         for (int j = 0; j < 8; ++j)
                             b[sb][j] = RM ? col_labels[16 * sb * DS + 4 * (c0 + j)]
                                           : col_labels[4 * (c0 + j) * STRIDE + 16 * sb];
+                    // (the reads stay above this line: left alone, the compiler moves each one down to
+                    // the matrix instruction that uses it, which then waits a full trip to the LDS)
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int j = 0; j < 8; j += 2)
 #pragma unroll
@@ -272,18 +375,61 @@ void lloyd_fewk_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (DIRECT) {
+                // [wave][sample][cluster]: the lane's four clusters are one 128-bit store
+                static_assert(!DIRECT || NB == 1, "one block of 16 samples per tile");
+                *reinterpret_cast<v4f*>(part + (wave << 8) + (m16 << 4) + 4 * g4) = sc0[0] + sc1[0];
+            } else {
 #pragma unroll
-            for (int sb = 0; sb < NB; ++sb) {
-                float* out = part + ((wave * NB + sb) << 8) + m16;
+                for (int sb = 0; sb < NB; ++sb) {
+                    float* out = part + ((wave * NB + sb) << 8) + m16;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) out[(4 * g4 + r) << 4] = sc0[sb][r] + sc1[sb][r];
+                    for (int r = 0; r < 4; ++r) out[(4 * g4 + r) << 4] = sc0[sb][r] + sc1[sb][r];
+                }
             }
         }
-        __syncthreads();
+        if constexpr (DIRECT)
+            fewk_lds_barrier();
+        else
+            __syncthreads();
         // arg-max: four threads per sample, thread q on the clusters q, q + 4, ... (the four partial
         // tiles added in wave order, strict '>' in increasing cluster order), then the four combine:
         // the largest score, the lowest index among equals
-        if ((int)threadIdx.x < 4 * S) {
+        if constexpr (DIRECT) {
+            // sixteen threads per sample, one per cluster: the partial scores of the waves added in
+            // wave order, then the largest score, the lowest index among equals (a score that does not
+            // compare, or a cluster past the last, never wins)
+            if ((int)threadIdx.x < 16 * S) {
+                const int m = threadIdx.x >> 4, c = threadIdx.x & 15;
+                float best = part[threadIdx.x];
+#pragma unroll
+                for (int wv = 1; wv < NW; ++wv) best += part[(wv << 8) + threadIdx.x];
+                uint32_t bi = (uint32_t)c;
+                if (!(c < k && best > -kmx_inf<float>())) {
+                    best = -kmx_inf<float>();
+                    bi = 0xffffffffu;
+                }
+#pragma unroll
+                for (int off = 1; off <= 8; off <<= 1) {
+                    const float ov = __shfl_xor(best, off, 64);
+                    const uint32_t oi = __shfl_xor(bi, off, 64);
+                    const bool take = ov > best || (ov == best && oi < bi);
+                    best = take ? ov : best;
+                    bi = take ? oi : bi;
+                }
+                if (bi == 0xffffffffu) bi = 0u;  // no score compares: the reference's running arg-min keeps 0
+                const int64_t gi = s0 + m;
+                const bool live = gi < n;
+                if (c == 0) {
+                    lab[m] = bi;
+                    wts[m] = live ? w_mine : 0.0f;
+                    if (live) {
+                        labels[gi] = bi;
+                        changed += pl_mine != bi ? 1u : 0u;
+                    }
+                }
+            }
+        } else if ((int)threadIdx.x < 4 * S) {
             const int s = threadIdx.x >> 2, q = threadIdx.x & 3, sb = s >> 4, m = s & 15;
             float best = -kmx_inf<float>();
             uint32_t bi = 0xffffffffu;
@@ -293,7 +439,7 @@ void lloyd_fewk_kernel(
                 if (c < k) {
                     float v = part[((0 * NB + sb) << 8) + (c << 4) + m];
 #pragma unroll
-                    for (int wv = 1; wv < 4; ++wv) v += part[((wv * NB + sb) << 8) + (c << 4) + m];
+                    for (int wv = 1; wv < NW; ++wv) v += part[((wv * NB + sb) << 8) + (c << 4) + m];
                     if (v > best) {
                         best = v;
                         bi = (uint32_t)c;
@@ -321,12 +467,15 @@ void lloyd_fewk_kernel(
                 }
             }
         }
-        __syncthreads();
+        if constexpr (DIRECT)
+            fewk_lds_barrier();
+        else
+            __syncthreads();
 
         // sums: the wave's feature blocks, four samples per matrix instruction
         // (U groups of four samples at a time, their reads in flight together; the loop is kept a
         // loop: unrolled, its S / 4 addresses would each take a register for the whole kernel)
-        constexpr int U = FBW <= 5 ? 4 : FBW <= 9 ? 2 : 1;
+        constexpr int U = DIRECT ? 4 : FBW <= 5 ? 4 : FBW <= 9 ? 2 : 1;
         int at = 0;  // offset of the group of samples inside a column of the tile
         const int at_step = RM ? 4 * U * DS : 4 * U;
 #pragma unroll 1
@@ -339,8 +488,13 @@ void lloyd_fewk_kernel(
                 const float wv = wts[s];
                 aw[u] = lb == (uint32_t)m16 ? wv : 0.0f;
 #pragma unroll
-                for (int i = 0; i < FBW; ++i) b[u][i] = col_sums[i][at + (RM ? 4 * u * DS : 4 * u)];
+                for (int g = 0; g < SUMS_NBASE; ++g) {
+                    const float* base = col_sums0 + g * SUMS_G * FB_STEP + at + (RM ? 4 * u * DS : 4 * u);
+#pragma unroll
+                    for (int i = g * SUMS_G; i < (g + 1) * SUMS_G && i < FBW; ++i) b[u][i] = base[(i - g * SUMS_G) * FB_STEP];
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);  // (all reads of the groups, then their matrix instructions)
 #pragma unroll
             for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -348,16 +502,26 @@ void lloyd_fewk_kernel(
                     acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[u], b[u][i], acc[i], 0, 0, 0);
             at += at_step;
         }
+        if constexpr (DIRECT == 2) cur = tile_words - cur;
+        if constexpr (DIRECT == 1) {
+            // (the tile is no longer read: the next one may arrive)
+            if (t + gridDim.x < n_tiles) {
+                fewk_lds_barrier();
+                issue((t + gridDim.x) << S_LOG, 0);
+            }
+        }
     }
 
     // The workgroup's sums as they lie in the registers: slot ((wave FBW + i) 4 + r) 64 + lane of
     // the workgroup's stretch of `partial` (whole cache lines per store; fewk_reduce_kernel knows
     // which cluster and feature a slot stands for).
-    float* out = partial + (size_t)blockIdx.x * (4 * FBW * 256) + (size_t)wave * (FBW * 256) + lane;
+    float* out = partial + (size_t)blockIdx.x * (NW * FBW * 256) + (size_t)wave * (FBW * 256) + lane;
+    // (the rows of clusters past the last one are neither written nor read)
 #pragma unroll
     for (int i = 0; i < FBW; ++i)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) out[(i * 4 + r) * 64] = acc[i][r];
+        for (int r = 0; r < 4; ++r)
+            if (4 * g4 + r < k) out[(i * 4 + r) * 64] = acc[i][r];
     if (changed) atomicAdd(&changed_block, changed);
     __syncthreads();
     if (threadIdx.x == 0 && changed_block) atomicAdd(&status->n_changed, changed_block);
@@ -551,7 +715,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void l
 // device-scope loads: one launch instead of two.
 // PER_WAVE: the partials are those of lloyd_fewk_wave_kernel - FBW blocks of 16 features each,
 // block fb in slots 256 fb .. 256 fb + 255.
-template <int FBW, bool PER_WAVE>
+template <int FBW, bool PER_WAVE, int NW>
 __global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restrict__ partial, int n_partials,
                                                           unsigned long long* __restrict__ gsum,
                                                           const int* __restrict__ q_exp, int d, int k,
@@ -559,13 +723,16 @@ __global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restri
     extern __shared__ __align__(16) unsigned char red_raw[];
     kmx_lloyd_status* status = tail.status;
     if (status->state != KMX_RUNNING) return;
-    constexpr int NSLOT = (PER_WAVE ? 1 : 4) * FBW * 256;
+    constexpr int NSLOT = (PER_WAVE ? 1 : NW) * FBW * 256;
     constexpr int GROUPS = 32;
     __shared__ float group_sum[GROUPS][32];
     const int sl = threadIdx.x & 31, pg = threadIdx.x >> 5;
     const int slot = blockIdx.x * 32 + sl;
     float total = 0.0f;
-    if (slot < NSLOT) {
+    // (slot -> cluster: lane group and register of the step's accumulators; clusters past the last
+    // one were not written)
+    const bool used = slot < NSLOT && 4 * ((slot & 63) >> 4) + ((slot >> 6) & 3) < k;
+    if (used) {
         const float* src = partial + slot;
         int p = pg;
         for (; p + GROUPS * 15 < n_partials; p += GROUPS * 16) {
@@ -586,14 +753,14 @@ __global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restri
     }
     group_sum[pg][sl] = total;
     __syncthreads();
-    if (threadIdx.x < 32 && slot < NSLOT) {
+    if (threadIdx.x < 32 && used) {
         float v = group_sum[0][sl];
 #pragma unroll
         for (int g = 1; g < GROUPS; ++g) v += group_sum[g][sl];
         // slot -> (feature, cluster): wave-of-the-step, block, register, lane
         const int lane = slot & 63, r = (slot >> 6) & 3, wi = slot >> 8;  // wi = wave FBW + i
         const int wave = wi / FBW, i = wi - wave * FBW;
-        const int fb = PER_WAVE ? wi : wave + 4 * i;
+        const int fb = PER_WAVE ? wi : wave + NW * i;
         const int f = 16 * fb + (lane & 15), c = 4 * (lane >> 4) + r;
         if (f <= d && c < k && fb < ((d + 1 + 15) >> 4))
             __hip_atomic_store(gsum + (size_t)f * k + c, (unsigned long long)__double2ll_rn(ldexp((double)v, q_exp[f])),
@@ -612,29 +779,33 @@ __global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restri
 
 // Samples per tile (a power of two, 16 .. 64) and workgroups per compute unit.
 struct FewkShape {
-    int s_log, kw, per_cu;
+    int s_log, kw, nw, per_cu;
     size_t lds;
 };
 
 bool fewk_shape(int d, int k, FewkShape* out) {
     if (d <= 64 || d > 1216 || k < 1 || k > 16) return false;
-    const int kw = fewk_kw(d);
-    const int kw_t = kw <= 8 ? 8 : kw <= 16 ? 16 : kw <= 32 ? 32 : kw <= 52 ? 52 : 76;
+    // (eight waves per workgroup beyond 512 features)
+    const int nw = d > 512 ? 8 : 4;
+    const int kw = fewk_kw(d, nw);
+    const int kw_t = nw == 8 ? (kw <= 26 ? 26 : 38) : kw <= 8 ? 8 : kw <= 16 ? 16 : 32;
     // (tiles of 32 samples up to 512 features while two workgroups fit a compute unit, of 16 beyond:
     // the instantiated kernels; measured at 2e6 x 100: tiles of 64 samples, which leave room for two
     // workgroups per compute unit instead of four, are no faster)
-    for (int s_log = kw_t <= 32 ? 5 : 4; s_log >= (kw_t <= 16 ? 5 : 4); --s_log) {
+    for (int s_log = nw == 4 ? 5 : 4; s_log >= (kw_t <= 16 ? 5 : 4); --s_log) {
         const int S = 1 << s_log;
-        const size_t lds = fewk_lds(d, S).total;
-        const int pieces = (d * (S / 4) + 255) / 256;
+        const size_t lds = fewk_lds(d, S, nw).total;
+        const int pieces = (d * (S / 4) + 64 * nw - 1) / (64 * nw);
         // (a larger tile only while two workgroups still fit a compute unit)
         const size_t cap = s_log > 4 ? (size_t)78 * 1024 : (size_t)156 * 1024;
-        if (lds <= cap && pieces <= fewk_prefetch(kw_t, s_log)) {
+        if (lds <= cap && pieces <= fewk_prefetch(kw_t, s_log, nw)) {
             const int by_lds = (int)((size_t)160 * 1024 / (lds + 512));
-            const int by_regs = fewk_waves_per_simd(kw_t, s_log);  // waves per SIMD the kernel is built for
+            // workgroups per compute unit the kernel's registers allow (waves per SIMD it is built for)
+            const int by_regs = fewk_waves_per_simd(kw_t, s_log, nw, nw == 8 && kw_t == 26 ? 1 : 0) * 4 / nw;
             const int per_cu = by_lds < by_regs ? by_lds : by_regs;
             out->s_log = s_log;
             out->kw = kw_t;
+            out->nw = nw;
             out->per_cu = per_cu < 1 ? 1 : per_cu;
             out->lds = lds;
             return true;
@@ -656,7 +827,7 @@ size_t kmx_fewk_partial_bytes(int d, int k) {
     if (!fewk_shape(d, k, &sh)) return 0;
     // (a fixed number of compute units: the layout of the workspace is a function of the shape alone;
     // on a larger device the grid stops at what fits)
-    const size_t by_workgroup = (size_t)sh.per_cu * 256 * 4 * (sh.kw / 4 + 1) * 256 * sizeof(float);
+    const size_t by_workgroup = (size_t)sh.per_cu * 256 * sh.nw * (sh.kw / 4 + 1) * 256 * sizeof(float);
     // (up to 128 features the per-wave kernel may run instead: three workgroups per compute unit, a
     // partial each of up to nine feature blocks)
     const size_t by_wave = d <= 128 ? (size_t)3 * 256 * 9 * 256 * sizeof(float) : 0;
@@ -685,7 +856,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
     tail.sizes = (float*)sizes;
     tail.empty_clusters = empty_clusters;
     tail.old_centroids_t = (const float*)centroids_t;
-    tail.cpack = reinterpret_cast<float*>(ws + L.off_cpack);
+    tail.cpack = nullptr;  // (the packed copy of the centroids is not read by this step's kernels)
     tail.half_norms = reinterpret_cast<float*>(ws + L.off_half);
     tail.status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
     tail.d = d;
@@ -697,7 +868,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
     const float* half_norms = tail.half_norms;
     float* partial = reinterpret_cast<float*>(ws + L.off_partial);
     int grid = kmx_fewk_grid(n, d, k, L.wgs_per_cu);
-    const size_t slots = (size_t)4 * (sh.kw / 4 + 1) * 256;  // partial sums of a workgroup of the instantiated kernel
+    const size_t slots = (size_t)sh.nw * (sh.kw / 4 + 1) * 256;  // partial sums of a workgroup of the instantiated kernel
     if ((size_t)grid * slots * sizeof(float) > L.partial_bytes) grid = (int)(L.partial_bytes / (slots * sizeof(float)));
     if (grid < 1) return KMX_ERR_WORKSPACE;
     const int vec_ok = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0);
@@ -705,16 +876,16 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
     const bool rm = X_rowmajor != nullptr && d % 4 == 0 && ((((uintptr_t)X_rowmajor) & 15) == 0);
     if (events) (void)hipEventRecord(events[0], stream);
     const size_t tail_lds = (size_t)(d + 1) * k * sizeof(float);
-#define KMX_FEWK_REDUCE(FBW_, PW_, N_PARTIALS)                                                             \
+#define KMX_FEWK_REDUCE(FBW_, PW_, NW_, N_PARTIALS)                                                        \
     do {                                                                                                  \
         if (tail_lds > 64 * 1024) {                                                                       \
             const hipError_t e =                                                                          \
-                hipFuncSetAttribute(reinterpret_cast<const void*>(&fewk_reduce_kernel<FBW_, PW_>),        \
+                hipFuncSetAttribute(reinterpret_cast<const void*>(&fewk_reduce_kernel<FBW_, PW_, NW_>),   \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds);           \
             if (e != hipSuccess) return (int32_t)e;                                                       \
         }                                                                                                 \
-        hipLaunchKernelGGL((fewk_reduce_kernel<FBW_, PW_>),                                               \
-                           dim3((unsigned)(((PW_ ? 1 : 4) * FBW_ * 256 + 31) / 32)), dim3(1024), tail_lds, \
+        hipLaunchKernelGGL((fewk_reduce_kernel<FBW_, PW_, NW_>),                                          \
+                           dim3((unsigned)(((PW_ ? 1 : NW_) * FBW_ * 256 + 31) / 32)), dim3(1024), tail_lds, \
                            stream, partial, N_PARTIALS, gsum, q_exp, d, k, tail);                         \
     } while (0)
     if (rm && d <= 128) {
@@ -735,42 +906,44 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
                            half_norms, labels_prev, labels, partial, status, n, d, k);                    \
         KMX_LAUNCH_CHECK();                                                                               \
         if (events) (void)hipEventRecord(events[1], stream);                                              \
-        KMX_FEWK_REDUCE(NFB_, true, (int)wgrid);                                                          \
+        KMX_FEWK_REDUCE(NFB_, true, 4, (int)wgrid);                                                       \
     } while (0)
         if (nfb_t == 5) KMX_FEWK_WAVE(20, 5);
         else if (nfb_t == 7) KMX_FEWK_WAVE(28, 7);
         else KMX_FEWK_WAVE(32, 9);
 #undef KMX_FEWK_WAVE
     } else {
-#define KMX_FEWK_LAUNCH_RM(KW_, SL_, RM_)                                                                  \
+#define KMX_FEWK_LAUNCH_RM(KW_, SL_, RM_, NW_)                                                             \
     do {                                                                                                  \
+        constexpr int direct_ = (RM_ && NW_ == 8 && KW_ == 26) ? 1 : 0;                                   \
         if (sh.lds > 64 * 1024) {                                                                         \
             const hipError_t e = hipFuncSetAttribute(                                                     \
-                reinterpret_cast<const void*>(&lloyd_fewk_kernel<KW_, SL_, RM_>),                         \
+                reinterpret_cast<const void*>(&lloyd_fewk_kernel<KW_, SL_, RM_, NW_, direct_>),           \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh.lds);                                 \
             if (e != hipSuccess) return (int32_t)e;                                                       \
         }                                                                                                 \
-        hipLaunchKernelGGL((lloyd_fewk_kernel<KW_, SL_, RM_>), dim3((unsigned)grid), dim3(256), sh.lds,   \
-                           stream, (const float*)X_t, (const float*)X_rowmajor, (const float*)w,          \
+        hipLaunchKernelGGL((lloyd_fewk_kernel<KW_, SL_, RM_, NW_, direct_>), dim3((unsigned)grid),        \
+                           dim3(64 * NW_),                                                                \
+                           sh.lds, stream, (const float*)X_t, (const float*)X_rowmajor, (const float*)w,  \
                            (const float*)centroids_t, half_norms, labels_prev, labels, partial, status,   \
                            n, d, k, vec_ok);                                                              \
     } while (0)
-#define KMX_FEWK_LAUNCH(KW_, SL_, FBW_)                                     \
+#define KMX_FEWK_LAUNCH(KW_, SL_, FBW_, NW_)                                \
     do {                                                                   \
         if (rm)                                                            \
-            KMX_FEWK_LAUNCH_RM(KW_, SL_, true);                            \
+            KMX_FEWK_LAUNCH_RM(KW_, SL_, true, NW_);                       \
         else                                                               \
-            KMX_FEWK_LAUNCH_RM(KW_, SL_, false);                           \
+            KMX_FEWK_LAUNCH_RM(KW_, SL_, false, NW_);                      \
         KMX_LAUNCH_CHECK();                                                \
         if (events) (void)hipEventRecord(events[1], stream);               \
-        KMX_FEWK_REDUCE(FBW_, false, grid);                                \
+        KMX_FEWK_REDUCE(FBW_, false, NW_, grid);                           \
     } while (0)
-        if (sh.kw == 8 && sh.s_log == 5) KMX_FEWK_LAUNCH(8, 5, 3);
-        else if (sh.kw == 16 && sh.s_log == 5) KMX_FEWK_LAUNCH(16, 5, 5);
-        else if (sh.kw == 32 && sh.s_log == 5) KMX_FEWK_LAUNCH(32, 5, 9);
-        else if (sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4, 9);
-        else if (sh.kw == 52 && sh.s_log == 4) KMX_FEWK_LAUNCH(52, 4, 14);
-        else if (sh.kw == 76 && sh.s_log == 4) KMX_FEWK_LAUNCH(76, 4, 20);
+        if (sh.nw == 4 && sh.kw == 8 && sh.s_log == 5) KMX_FEWK_LAUNCH(8, 5, 3, 4);
+        else if (sh.nw == 4 && sh.kw == 16 && sh.s_log == 5) KMX_FEWK_LAUNCH(16, 5, 5, 4);
+        else if (sh.nw == 4 && sh.kw == 32 && sh.s_log == 5) KMX_FEWK_LAUNCH(32, 5, 9, 4);
+        else if (sh.nw == 4 && sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4, 9, 4);
+        else if (sh.nw == 8 && sh.kw == 26 && sh.s_log == 4) KMX_FEWK_LAUNCH(26, 4, 7, 8);
+        else if (sh.nw == 8 && sh.kw == 38 && sh.s_log == 4) KMX_FEWK_LAUNCH(38, 4, 10, 8);
         else return KMX_ERR_UNSUPPORTED;
 #undef KMX_FEWK_LAUNCH_RM
 #undef KMX_FEWK_LAUNCH

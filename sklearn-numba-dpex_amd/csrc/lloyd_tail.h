@@ -94,6 +94,40 @@ __device__ inline int lloyd_list_empty(const T* sizes, uint32_t* empty_clusters,
     return base;
 }
 
+// The same for at most 64 clusters, by the first wave alone and with one barrier (the general
+// routine above passes five, each a wait for all the waves of the workgroup).
+template <typename T>
+__device__ inline int lloyd_list_empty_one_wave(const T* sizes, uint32_t* empty_clusters, int k,
+                                                int* heaviest_out) {
+    __shared__ int one_wave_result[2];
+    if (threadIdx.x < 64) {
+        const int c = (int)threadIdx.x;
+        const bool in = c < k;
+        const T sz = in ? sizes[c] : T(1);
+        const bool flag = in && sz == T(0);
+        const unsigned long long mask = __ballot(flag);
+        if (flag) empty_clusters[__popcll(mask & ((1ull << c) - 1ull))] = (uint32_t)c;
+        T my_max = in ? sz : -kmx_inf<T>();
+        int my_arg = in ? c : 0x7fffffff;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const T ov = __shfl_xor(my_max, off, 64);
+            const int oi = __shfl_xor(my_arg, off, 64);
+            if (ov > my_max || (ov == my_max && oi < my_arg)) {
+                my_max = ov;
+                my_arg = oi;
+            }
+        }
+        if (c == 0) {
+            one_wave_result[0] = my_arg;
+            one_wave_result[1] = __popcll(mask);
+        }
+    }
+    __syncthreads();
+    *heaviest_out = one_wave_result[0];
+    return one_wave_result[1];
+}
+
 // End of an iteration, by one thread: iteration count, shift, and the next state (strict
 // convergence from the second iteration on, then the tolerance, then the iteration limit).
 __device__ inline void lloyd_update_status(kmx_lloyd_status* st, double total_shift, unsigned int changed) {
@@ -184,17 +218,31 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
                                                  T* __restrict__ vals) {
     __shared__ double scratch[16];
     const int n_threads = (int)blockDim.x;
+    // Element jx = f k + c of the (d + 1, k) arrays is taken by thread jx % stride in its pass
+    // jx / stride.  WIDE: stride is the largest multiple of k within the workgroup, so that a thread
+    // keeps its cluster and moves on by stride / k features per pass - with thousands of elements
+    // the division of every index by k, three times per element, was most of what this workgroup,
+    // alone on its compute unit, had to issue.
+    const int rows_per_pass = WIDE ? n_threads / a.k : 0;
+    const int stride = WIDE ? rows_per_pass * a.k : n_threads;
+    const bool lane_on = (int)threadIdx.x < stride;
+    const int f_first = WIDE ? (int)threadIdx.x / a.k : 0;
+    const int c_mine = WIDE ? (int)threadIdx.x - f_first * a.k : 0;
+    // feature of the element jx that the thread takes in pass `pass`
+    auto feature_of = [&](const int jx, const int pass) __attribute__((always_inline)) {
+        return WIDE ? f_first + pass * rows_per_pass : jx / a.k;
+    };
     // The old centroids are asked for before anything else (up to eight values per thread: what
     // (d + 1) k <= 2048 needs with 256 threads): the routine is a chain of memory round trips, and
     // this one then runs beside those of the state and of the sums ...
     constexpr int OLD_AHEAD = 8;
     const int dk_ahead = a.d * a.k;
-    const bool old_ahead = dk_ahead <= n_threads * OLD_AHEAD;
+    const bool old_ahead = dk_ahead <= stride * OLD_AHEAD;
     T old_v[OLD_AHEAD];
 #pragma unroll
     for (int i = 0; i < OLD_AHEAD; ++i) {
-        const int jx = (int)threadIdx.x + n_threads * i;
-        old_v[i] = (old_ahead && jx < dk_ahead) ? a.old_centroids_t[jx] : T(0);
+        const int jx = (int)threadIdx.x + stride * i;
+        old_v[i] = (old_ahead && lane_on && jx < dk_ahead) ? a.old_centroids_t[jx] : T(0);
     }
     const int d = a.d, k = a.k, dpad = a.dpad;
     const int items = (d + 1) * k, dk = d * k;
@@ -205,13 +253,16 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
                                     : gsum[jx]);
     };
     constexpr int SUMS_AHEAD = 8;
-    const bool sums_ahead = FROM_GSUM && items <= n_threads * SUMS_AHEAD;
+    const bool sums_ahead = FROM_GSUM && items <= stride * SUMS_AHEAD;
     long long sum_v[SUMS_AHEAD];
+    int q_v[SUMS_AHEAD];  // (their binary points, asked for in the same round trip)
     if constexpr (FROM_GSUM) {
 #pragma unroll
         for (int i = 0; i < SUMS_AHEAD; ++i) {
-            const int jx = (int)threadIdx.x + n_threads * i;
-            sum_v[i] = (sums_ahead && jx < items) ? load_sum(jx) : 0ll;
+            const int jx = (int)threadIdx.x + stride * i;
+            const bool mine = sums_ahead && lane_on && jx < items;
+            sum_v[i] = mine ? load_sum(jx) : 0ll;
+            q_v[i] = mine ? q_exp[feature_of(jx, i)] : 0;
         }
     }
     unsigned int counter_word = 0u;
@@ -232,12 +283,18 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
     // thread 0 resets it at the end of the kernel)
     const bool keep_sums = FROM_GSUM && a.clear_word != nullptr && a.delta_divisor > 0 &&
                            (int64_t)n_changed * a.delta_divisor <= a.n_samples;
+    // WIDE, with every element already in a register of its thread: the sizes are converted
+    // first, and each sum is converted, divided and stored in one go once no cluster is known to be
+    // empty
+    const bool fused = WIDE && FROM_GSUM && sums_ahead && old_ahead;
+    T raw_v[SUMS_AHEAD];
+#pragma unroll
+    for (int i = 0; i < SUMS_AHEAD; ++i) raw_v[i] = T(0);
     if constexpr (FROM_GSUM) {
-        auto convert = [&](const int jx, const long long iv) __attribute__((always_inline)) {
+        auto convert = [&](const int jx, const int f, const long long iv, const int q) __attribute__((always_inline)) {
             if (!keep_sums) gsum[jx] = 0ull;
-            const int f = jx / k;
             // (times 2^-q, built from its exponent field: exact, like ldexp)
-            const T val = (T)((double)iv * __hiloint2double((1023 - q_exp[f]) << 20, 0));
+            const T val = (T)((double)iv * __hiloint2double((1023 - q) << 20, 0));
             vals[jx] = val;
             if (f < d)
                 out_t[jx] = val;
@@ -247,22 +304,34 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
         if (sums_ahead) {
 #pragma unroll
             for (int i = 0; i < SUMS_AHEAD; ++i) {
-                const int jx = (int)threadIdx.x + n_threads * i;
-                if (jx < items) convert(jx, sum_v[i]);
+                const int jx = (int)threadIdx.x + stride * i;
+                if (lane_on && jx < items) {
+                    const int f = feature_of(jx, i);
+                    if (fused && f < d) {
+                        // (kept in its register until the sizes are known: no store of the raw sum,
+                        // no trip through the LDS)
+                        if (!keep_sums) gsum[jx] = 0ull;
+                        raw_v[i] = (T)((double)sum_v[i] * __hiloint2double((1023 - q_v[i]) << 20, 0));
+                    } else {
+                        convert(jx, f, sum_v[i], q_v[i]);
+                    }
+                }
             }
         } else {
             // (SUMS_AHEAD loads in flight per thread and pass: a loop of one load and one store per
             // pass would take a trip to memory per element)
-            for (int base = 0; base < items; base += n_threads * SUMS_AHEAD) {
+            for (int base = 0, pass0 = 0; base < items; base += stride * SUMS_AHEAD, pass0 += SUMS_AHEAD) {
 #pragma unroll
                 for (int i = 0; i < SUMS_AHEAD; ++i) {
-                    const int jx = base + (int)threadIdx.x + n_threads * i;
-                    sum_v[i] = jx < items ? load_sum(jx) : 0ll;
+                    const int jx = base + (int)threadIdx.x + stride * i;
+                    const bool mine = lane_on && jx < items;
+                    sum_v[i] = mine ? load_sum(jx) : 0ll;
+                    q_v[i] = mine ? q_exp[feature_of(jx, pass0 + i)] : 0;
                 }
 #pragma unroll
                 for (int i = 0; i < SUMS_AHEAD; ++i) {
-                    const int jx = base + (int)threadIdx.x + n_threads * i;
-                    if (jx < items) convert(jx, sum_v[i]);
+                    const int jx = base + (int)threadIdx.x + stride * i;
+                    if (lane_on && jx < items) convert(jx, feature_of(jx, pass0 + i), sum_v[i], q_v[i]);
                 }
             }
         }
@@ -271,7 +340,8 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
     }
     __syncthreads();
     int heaviest = 0;
-    const int n_empty = lloyd_list_empty<T>(sizes_s, a.empty_clusters, k, &heaviest);
+    const int n_empty = (WIDE && k <= 64) ? lloyd_list_empty_one_wave<T>(sizes_s, a.empty_clusters, k, &heaviest)
+                                          : lloyd_list_empty<T>(sizes_s, a.empty_clusters, k, &heaviest);
     if (threadIdx.x == 0) {
         a.status->n_empty = n_empty;
         a.status->reserved[0] = heaviest;
@@ -281,6 +351,13 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
         if constexpr (FROM_GSUM) {
             if (keep_sums)
                 for (int jx = threadIdx.x; jx < items; jx += n_threads) gsum[jx] = 0ull;
+            if (fused) {  // (the raw sums, as the relocation reads them)
+#pragma unroll
+                for (int i = 0; i < SUMS_AHEAD; ++i) {
+                    const int jx = (int)threadIdx.x + stride * i;
+                    if (lane_on && jx < dk) out_t[jx] = raw_v[i];
+                }
+            }
         }
         if (threadIdx.x == 0) {
             a.status->state = KMX_NEED_RELOCATION;
@@ -293,32 +370,34 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
                           : (a.list_divisor > 0 && (int64_t)n_changed * a.list_divisor <= a.n_samples) ? 1u
                                                                                                     : 2u;
     double shift = 0.0;
-    auto divide = [&](const int jx, const T old_value) __attribute__((always_inline)) {
-        const int f = jx / k, c = jx - f * k;
-        const T nv = vals[jx] / sizes_s[c];
+    // (a.cpack may be null: the caller's kernels read the (d, k) array only)
+    const T size_mine = WIDE ? sizes_s[c_mine] : T(1);
+    auto divide = [&](const int jx, const int f, const T old_value, const T raw) __attribute__((always_inline)) {
+        const int c = WIDE ? c_mine : jx - f * k;
+        const T nv = (fused ? raw : vals[jx]) / (WIDE ? size_mine : sizes_s[c]);
         const T df = old_value - nv;
         shift += (double)(df * df);
         vals[jx] = nv;
         out_t[jx] = nv;
-        a.cpack[(size_t)c * dpad + f] = nv;
+        if (a.cpack != nullptr) a.cpack[(size_t)c * dpad + f] = nv;
     };
     if (old_ahead) {  // (the same elements in the same order as the loop below)
 #pragma unroll
         for (int i = 0; i < OLD_AHEAD; ++i) {
-            const int jx = (int)threadIdx.x + n_threads * i;
-            if (jx < dk) divide(jx, old_v[i]);
+            const int jx = (int)threadIdx.x + stride * i;
+            if (lane_on && jx < dk) divide(jx, feature_of(jx, i), old_v[i], raw_v[i]);
         }
     } else {
-        for (int base = 0; base < dk; base += n_threads * OLD_AHEAD) {
+        for (int base = 0, pass0 = 0; base < dk; base += stride * OLD_AHEAD, pass0 += OLD_AHEAD) {
 #pragma unroll
             for (int i = 0; i < OLD_AHEAD; ++i) {
-                const int jx = base + (int)threadIdx.x + n_threads * i;
-                old_v[i] = jx < dk ? old_t[jx] : T(0);
+                const int jx = base + (int)threadIdx.x + stride * i;
+                old_v[i] = (lane_on && jx < dk) ? old_t[jx] : T(0);
             }
 #pragma unroll
             for (int i = 0; i < OLD_AHEAD; ++i) {
-                const int jx = base + (int)threadIdx.x + n_threads * i;
-                if (jx < dk) divide(jx, old_v[i]);
+                const int jx = base + (int)threadIdx.x + stride * i;
+                if (lane_on && jx < dk) divide(jx, feature_of(jx, pass0 + i), old_v[i], T(0));
             }
         }
     }
@@ -327,7 +406,11 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
         // wide samples, few clusters: a cluster's norm by a group of threads (thread (g, c) takes
         // every n_g-th feature, the groups are then added in order) - one thread per cluster
         // would walk hundreds of features alone while the others wait
+        // (the groups are added in two steps - eight threads per cluster take every eighth group,
+        // then one adds the eight - where one thread alone would walk a hundred values, a trip to
+        // the LDS each)
         __shared__ T norm_part[1024];
+        __shared__ T norm_part8[8 * 64];
         const int n_g = n_threads / k;
         const int c = (int)threadIdx.x % k, g = (int)threadIdx.x / k;
         T sq = T(0);
@@ -335,11 +418,27 @@ __device__ inline void lloyd_small_finalize_body(unsigned long long* __restrict_
             for (int f = g; f < d; f += n_g) sq += vals[f * k + c] * vals[f * k + c];
         norm_part[threadIdx.x] = sq;
         __syncthreads();
+        const bool two_steps = k <= 64 && n_g >= 16;
+        if (two_steps) {
+            if (g < 8) {
+                T tot = norm_part[g * k + c];
+                for (int g2 = g + 8; g2 < n_g; g2 += 8) tot += norm_part[g2 * k + c];
+                norm_part8[g * k + c] = tot;
+            }
+            __syncthreads();
+        }
         if ((int)threadIdx.x < k) {
-            T tot = norm_part[threadIdx.x];
-            for (int g2 = 1; g2 < n_g; ++g2) tot += norm_part[g2 * k + threadIdx.x];
+            T tot;
+            if (two_steps) {
+                tot = norm_part8[threadIdx.x];
+                for (int g2 = 1; g2 < 8; ++g2) tot += norm_part8[g2 * k + threadIdx.x];
+            } else {
+                tot = norm_part[threadIdx.x];
+                for (int g2 = 1; g2 < n_g; ++g2) tot += norm_part[g2 * k + threadIdx.x];
+            }
             a.half_norms[threadIdx.x] = tot / T(2);
-            for (int f = d; f < dpad; ++f) a.cpack[(size_t)threadIdx.x * dpad + f] = T(0);
+            if (a.cpack != nullptr)
+                for (int f = d; f < dpad; ++f) a.cpack[(size_t)threadIdx.x * dpad + f] = T(0);
         }
     } else {
         for (int c = threadIdx.x; c < k; c += n_threads) {

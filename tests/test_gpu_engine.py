@@ -185,6 +185,42 @@ def test_forced_empty_clusters_config5(cuda):
     assert len(np.unique(labels.cpu().numpy())) == 64
 
 
+@pytest.mark.parametrize("d", [100, 784])
+def test_forced_empty_clusters_few_clusters_on_wide_samples(cuda, d):
+    """fp32, 10 clusters on wide samples (the step that keeps a tile of samples on chip): two of
+    the initial centroids lie far away, empty on iteration 1 and are relocated; compared with the
+    oracle after that iteration and on the final result."""
+    import torch
+
+    from sklearn_numba_dpex_amd import _capi
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    rng = np.random.default_rng(d)
+    n, k = 6_000, 10
+    centers = rng.uniform(-1.0, 1.0, (k, d)) * (8.0 / np.sqrt(d))
+    X = (centers[rng.integers(0, k, n)] + rng.standard_normal((n, d))).astype(np.float32)
+    X -= X.mean(axis=0)
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    init = X[rng.choice(n, k, replace=False)].copy()
+    init[3] += 100.0
+    init[7] -= 100.0
+    assert _capi.lloyd_plan(n, d, k, _capi.dtype_code(np.float32), 0).variant == 81
+    X_t = torch.as_tensor(np.ascontiguousarray(X.T), device=cuda)
+    w_d = torch.as_tensor(w, device=cuda)
+    init_t = torch.as_tensor(np.ascontiguousarray(init.T), device=cuda)
+    labels, inertia, centers_t, n_iter = drivers.lloyd(X_t, w_d, init_t, True, max_iter=1, tol=0.0)
+    it = next(ok.lloyd_iterations(X, w, init, max_iter=1, tol=0.0))
+    assert it["n_empty"] == 2 and n_iter == 1
+    assert_centers_close(centers_t.cpu().numpy().T, it["centers"], np.float32)
+    labels, inertia, centers_t, n_iter = drivers.lloyd(X_t, w_d, init_t, True, max_iter=30, tol=0.0)
+    ref_labels, ref_inertia, ref_centers, ref_n_iter = ok.lloyd(X, w, init, max_iter=30, tol=0.0)
+    assert n_iter == ref_n_iter
+    assert_labels_match(labels.cpu().numpy(), ref_labels, X, ref_centers)
+    assert_centers_close(centers_t.cpu().numpy().T, ref_centers, np.float32)
+    assert float(inertia) == pytest.approx(float(ref_inertia), rel=1e-5)
+    assert len(np.unique(labels.cpu().numpy())) == k
+
+
 def test_more_clusters_than_distinct_points(cuda):
     from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
 
