@@ -89,6 +89,7 @@ constexpr int fewk_prefetch(int kw, int s_log, int nw) {
 // registers; four with tiles of 32 samples of up to 128 features and with eight waves up to 832)
 constexpr int fewk_waves_per_simd(int kw, int s_log, int nw, int direct = 0) {
     if (nw == 8) return direct == 1 ? 4 : 2;
+    if (direct == 1) return 4;
     return (kw <= 8 && s_log == 5) ? 4 : kw <= 52 ? 2 : 1;
 }
 
@@ -475,7 +476,7 @@ void lloyd_fewk_kernel(
         // sums: the wave's feature blocks, four samples per matrix instruction
         // (U groups of four samples at a time, their reads in flight together; the loop is kept a
         // loop: unrolled, its S / 4 addresses would each take a register for the whole kernel)
-        constexpr int U = DIRECT ? 4 : FBW <= 5 ? 4 : FBW <= 9 ? 2 : 1;
+        constexpr int U = DIRECT ? (FBW <= 7 ? 4 : 2) : FBW <= 5 ? 4 : FBW <= 9 ? 2 : 1;
         int at = 0;  // offset of the group of samples inside a column of the tile
         const int at_step = RM ? 4 * U * DS : 4 * U;
 #pragma unroll 1
@@ -555,15 +556,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void l
     const int n_fb = (d + 1 + 15) >> 4;
     __shared__ unsigned int changed_block;
 
+    // (every lane loads, from a clamped address where it has no value: the loads are issued together)
     float ca[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
         const int f = 4 * s + g4;
-        ca[s] = (f < d && m16 < k) ? centroids_t[(size_t)f * k + m16] : 0.0f;
+        const bool has = f < d && m16 < k;
+        const float v = centroids_t[has ? (size_t)f * k + m16 : (size_t)0];
+        ca[s] = has ? v : 0.0f;
     }
     v4f start;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) start[r] = (4 * g4 + r < k) ? -half_norms[4 * g4 + r] : 0.0f;
+    for (int r = 0; r < 4; ++r) {
+        const float hn = half_norms[4 * g4 + r < k ? 4 * g4 + r : 0];
+        start[r] = (4 * g4 + r < k) ? -hn : 0.0f;
+    }
     // past the features: ones (feature d, the cluster sizes), then zeros; never overwritten
     for (int idx = lane; idx < 16 * (DS - d); idx += 64) {
         const int sm = idx / (DS - d), c = idx - sm * (DS - d);
@@ -635,6 +642,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void l
                 float b[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) b[j] = col_labels[4 * (c0 + j < KS ? c0 + j : KS - 1)];
+                // (the reads stay above this line: left alone, the compiler moves each one down to the
+                // matrix instruction that uses it, which then waits a full trip to the LDS)
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int j = 0; j < 8; j += 2) {
                     if (c0 + j < KS) sc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j < KS ? c0 + j : 0], b[j], sc0, 0, 0, 0);
@@ -674,17 +684,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void l
         const float w_lane = live ? w_mine : 0.0f;
 
         // sums: four samples per matrix instruction; the row of sample 4 c + g4 carries its weight
-        // in the column of its cluster
+        // in the column of its cluster (two groups of four samples at a time: their reads, then
+        // their matrix instructions)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t lb = __shfl(bi, 4 * c + g4, 64);
-            const float wv = __shfl(w_lane, 4 * c + g4, 64);
-            const float aw = lb == (uint32_t)m16 ? wv : 0.0f;
-            float b[NFB];
+        for (int c0 = 0; c0 < 4; c0 += 2) {
+            float aw[2], b[2][NFB];
 #pragma unroll
-            for (int i = 0; i < NFB; ++i) b[i] = col_sums[4 * c * DS + 16 * i];
+            for (int u = 0; u < 2; ++u) {
+                const int c = c0 + u;
+                const uint32_t lb = __shfl(bi, 4 * c + g4, 64);
+                const float wv = __shfl(w_lane, 4 * c + g4, 64);
+                aw[u] = lb == (uint32_t)m16 ? wv : 0.0f;
 #pragma unroll
-            for (int i = 0; i < NFB; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw, b[i], acc[i], 0, 0, 0);
+                for (int i = 0; i < NFB; ++i) b[u][i] = col_sums[4 * c * DS + 16 * i];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < NFB; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[u], b[u][i], acc[i], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -792,7 +812,9 @@ bool fewk_shape(int d, int k, FewkShape* out) {
     // (tiles of 32 samples up to 512 features while two workgroups fit a compute unit, of 16 beyond:
     // the instantiated kernels; measured at 2e6 x 100: tiles of 64 samples, which leave room for two
     // workgroups per compute unit instead of four, are no faster)
-    for (int s_log = nw == 4 ? 5 : 4; s_log >= (kw_t <= 16 ? 5 : 4); --s_log) {
+    // (beyond 128 features tiles of 16 samples, which arrive in LDS directly where there is a row-major
+    // copy: four workgroups of four waves per compute unit up to 512 features, two of eight beyond)
+    for (int s_log = (nw == 4 && kw_t <= 8) ? 5 : 4; s_log >= (kw_t <= 8 ? 5 : 4); --s_log) {
         const int S = 1 << s_log;
         const size_t lds = fewk_lds(d, S, nw).total;
         const int pieces = (d * (S / 4) + 64 * nw - 1) / (64 * nw);
@@ -801,7 +823,8 @@ bool fewk_shape(int d, int k, FewkShape* out) {
         if (lds <= cap && pieces <= fewk_prefetch(kw_t, s_log, nw)) {
             const int by_lds = (int)((size_t)160 * 1024 / (lds + 512));
             // workgroups per compute unit the kernel's registers allow (waves per SIMD it is built for)
-            const int by_regs = fewk_waves_per_simd(kw_t, s_log, nw, nw == 8 && kw_t == 26 ? 1 : 0) * 4 / nw;
+            const bool direct = s_log == 4 && (nw == 4 || kw_t == 26);
+            const int by_regs = fewk_waves_per_simd(kw_t, s_log, nw, direct ? 1 : 0) * 4 / nw;
             const int per_cu = by_lds < by_regs ? by_lds : by_regs;
             out->s_log = s_log;
             out->kw = kw_t;
@@ -915,7 +938,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
     } else {
 #define KMX_FEWK_LAUNCH_RM(KW_, SL_, RM_, NW_)                                                             \
     do {                                                                                                  \
-        constexpr int direct_ = (RM_ && NW_ == 8 && KW_ == 26) ? 1 : 0;                                   \
+        constexpr int direct_ = (RM_ && SL_ == 4 && (NW_ == 4 || KW_ == 26)) ? 1 : 0;                     \
         if (sh.lds > 64 * 1024) {                                                                         \
             const hipError_t e = hipFuncSetAttribute(                                                     \
                 reinterpret_cast<const void*>(&lloyd_fewk_kernel<KW_, SL_, RM_, NW_, direct_>),           \
@@ -939,8 +962,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
         KMX_FEWK_REDUCE(FBW_, false, NW_, grid);                           \
     } while (0)
         if (sh.nw == 4 && sh.kw == 8 && sh.s_log == 5) KMX_FEWK_LAUNCH(8, 5, 3, 4);
-        else if (sh.nw == 4 && sh.kw == 16 && sh.s_log == 5) KMX_FEWK_LAUNCH(16, 5, 5, 4);
-        else if (sh.nw == 4 && sh.kw == 32 && sh.s_log == 5) KMX_FEWK_LAUNCH(32, 5, 9, 4);
+        else if (sh.nw == 4 && sh.kw == 16 && sh.s_log == 4) KMX_FEWK_LAUNCH(16, 4, 5, 4);
         else if (sh.nw == 4 && sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4, 9, 4);
         else if (sh.nw == 8 && sh.kw == 26 && sh.s_log == 4) KMX_FEWK_LAUNCH(26, 4, 7, 8);
         else if (sh.nw == 8 && sh.kw == 38 && sh.s_log == 4) KMX_FEWK_LAUNCH(38, 4, 10, 8);
