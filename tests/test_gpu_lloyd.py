@@ -87,6 +87,14 @@ def _small_configs():
         "K32j": lambda: dict(_blob_config(50_001, 128, 16, np.float32, 56), variant=81),
         "K32k": lambda: dict(_blob_config(10_000, 68, 3, np.float32, 57), variant=81),
         "K32l": lambda: dict(_blob_config(30_003, 112, 9, np.float32, 58, skew=True), variant=81),
+        # tiles that arrive in LDS directly (row-major copy, a multiple of 4 features beyond 128): four
+        # waves per workgroup up to 512 features, eight beyond; fewer samples than a tile; rows of
+        # exactly one, two and more than two load instructions of 64 pieces
+        "K32m": lambda: dict(_blob_config(2_501, 384, 6, np.float32, 59), variant=81),
+        "K32n": lambda: dict(_blob_config(9, 640, 4, np.float32, 60), variant=81),
+        "K32o": lambda: dict(_blob_config(4_100, 512, 16, np.float32, 61), variant=81),
+        "K32p": lambda: dict(_blob_config(1_030, 832, 5, np.float32, 62, skew=True), variant=81),
+        "K32q": lambda: dict(_blob_config(777, 256, 11, np.float32, 63), variant=81),
         "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
         # extremes of the tiled product: thousands of features (many passes of the bucketed sums),
         # more clusters than the bucket counts hold in LDS and than the wide path takes
@@ -140,7 +148,7 @@ def _odd_config():
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
                                   "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
                                   "K32a", "K32b", "K32c", "K32d", "K32e", "K32f", "K32g", "K32h", "K32i",
-                                  "K32j", "K32k", "K32l"])
+                                  "K32j", "K32k", "K32l", "K32m", "K32n", "K32o", "K32p", "K32q"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -249,7 +257,7 @@ def test_duplicate_and_identical_centroids_on_every_kernel_family(cuda, name):
                                   # (not K32d: with 1216 features two fp32 evaluations of a score differ by up
                                   # to 2e-6 of its size, more than the near-tie rule's 1e-6 - one label in ten
                                   # iterations of 3002 samples)
-                                  "K32a", "K32b", "K32c", "K32f", "K32i"])
+                                  "K32a", "K32b", "K32c", "K32f", "K32i", "K32m", "K32o", "K32q"])
 def test_lockstep_iterations_match_oracle(cuda, name):
     """Ten iterations, each compared from identical inputs: the oracle repeats every GPU
     iteration from the centroids the GPU started it with (a Lloyd trajectory at tol = 0 is
