@@ -45,20 +45,27 @@ __device__ __forceinline__ void store4(T* __restrict__ row, int64_t i0, int64_t 
 // four consecutive samples (128-bit loads of every feature row); the centroids are staged in
 // LDS when they fit (LDS_CENTROIDS), so that the per-sample gather of the label's centroid
 // does not go through the vector memory pipe.
-// SUM: nothing is written per sample; the workgroup's total goes to partial[blockIdx.x] in fp64
-// (fixed order inside the workgroup, so the result does not depend on timing).
+// SUM: nothing is written per sample; the workgroup's total goes to its slot of `partial` in fp64
+// (fixed order inside the workgroup, so the result does not depend on timing).  With few samples
+// of many features the launch has a second grid dimension and workgroup (x, y) takes the y-th
+// stretch of the features only: a thread that walks hundreds of feature rows alone, with a few
+// hundred threads on the whole device, is a chain of trips to memory.
 template <typename T, bool LDS_CENTROIDS, bool SUM>
 __global__ __launch_bounds__(256) void per_sample_inertia_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight,
     const T* __restrict__ centroids_t, const uint32_t* __restrict__ labels, T* __restrict__ out,
     double* __restrict__ partial, int64_t n, int d, int k, int vec_ok) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* cs = reinterpret_cast<T*>(smem_raw);  // [d * k], same layout as centroids_t
+    T* cs = reinterpret_cast<T*>(smem_raw);  // the workgroup's feature rows of centroids_t, same layout
+    const int f_chunk = (d + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int f_begin = (int)blockIdx.y * f_chunk;
+    const int f_end = f_begin + f_chunk < d ? f_begin + f_chunk : d;
     if (LDS_CENTROIDS) {
-        for (int idx = threadIdx.x; idx < d * k; idx += 256) cs[idx] = centroids_t[idx];
+        for (int idx = threadIdx.x; idx < (f_end - f_begin) * k; idx += 256) cs[idx] = centroids_t[(size_t)f_begin * k + idx];
         __syncthreads();
     }
-    const T* __restrict__ cent = LDS_CENTROIDS ? cs : centroids_t;
+    // (row f of the centroids: cent + f k)
+    const T* __restrict__ cent = LDS_CENTROIDS ? cs - (size_t)f_begin * k : centroids_t;
     const int64_t n_groups = (n + 3) >> 2;
     const int64_t stride = (int64_t)gridDim.x * 256;
     double total = 0.0;
@@ -70,8 +77,8 @@ __global__ __launch_bounds__(256) void per_sample_inertia_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) c[r] = (i0 + r < n) ? labels[i0 + r] : 0u;
         T acc[4] = {T(0), T(0), T(0), T(0)};
-#pragma unroll 2
-        for (int f = 0; f < d; ++f) {
+#pragma unroll 4
+        for (int f = f_begin; f < f_end; ++f) {
             T x[4];
             load4<T>(X_t + (size_t)f * n, i0, n, full, x);
             const T* __restrict__ crow = cent + (size_t)f * k;
@@ -98,7 +105,7 @@ __global__ __launch_bounds__(256) void per_sample_inertia_kernel(
     if constexpr (SUM) {
         __shared__ double wave_part[4];
         total = kmx_block_sum<double>(total, wave_part);
-        if (threadIdx.x == 0) partial[blockIdx.x] = total;
+        if (threadIdx.x == 0) partial[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = total;
     }
 }
 
@@ -332,6 +339,14 @@ __global__ __launch_bounds__(256) void relocate_kernel(
     }
 }
 
+int stream_grid(int64_t n);
+// fp64 partial sums a launch of the summing kernel may write: eight per compute unit, or one per
+// workgroup of its first grid dimension where that is more
+int64_t inertia_partial_slots(int64_t n) {
+    const int64_t a = (int64_t)kmx_num_cus() * 8, b = stream_grid(kmx_cdiv(n, 4));
+    return a > b ? a : b;
+}
+
 int stream_grid(int64_t n) {
     int64_t blocks = kmx_cdiv(n, 256);
     const int64_t cap = (int64_t)kmx_num_cus() * 8;
@@ -361,10 +376,20 @@ static int32_t inertia_launch(const void* X_t, const void* sample_weight, const 
     auto al16 = [](const void* p) { return (((uintptr_t)p) & 15) == 0; };
     const int vec_ok =
         (n % 4 == 0) && al16(X_t) && (sum || al16(out)) && (sample_weight == nullptr || al16(sample_weight));
-    const size_t lds = (size_t)d * k * es;
+    // the sum over few samples of many features: the features split over the second grid dimension
+    // until there are about four workgroups per compute unit (and at least 16 features each)
+    int gy = 1;
+    if (sum) {
+        gy = (int)kmx_cdiv((int64_t)kmx_num_cus() * 4, grid);
+        if (gy > d / 16) gy = d / 16;
+        if ((int64_t)gy * grid > inertia_partial_slots(n)) gy = (int)(inertia_partial_slots(n) / grid);
+        if (gy < 1) gy = 1;
+    }
+    const int f_chunk = (int)kmx_cdiv(d, gy);
+    const size_t lds = (size_t)f_chunk * k * es;
     const bool in_lds = lds <= 48 * 1024;
 #define KMX_INERTIA(T, L, S)                                                                       \
-    hipLaunchKernelGGL((per_sample_inertia_kernel<T, L, S>), dim3(grid), dim3(256), (L) ? lds : 0,  \
+    hipLaunchKernelGGL((per_sample_inertia_kernel<T, L, S>), dim3(grid, gy), dim3(256), (L) ? lds : 0,  \
                        stream, (const T*)X_t, (const T*)sample_weight, (const T*)centroids_t,      \
                        labels, (S) ? nullptr : (T*)out, partial, n, d, k, vec_ok)
 #define KMX_INERTIA_T(T)                                                        \
@@ -379,9 +404,9 @@ static int32_t inertia_launch(const void* X_t, const void* sample_weight, const 
 #undef KMX_INERTIA
     if (sum) {
         if (dtype == KMX_F32)
-            hipLaunchKernelGGL((inertia_total_kernel<float>), dim3(1), dim3(256), 0, stream, partial, grid, (float*)out);
+            hipLaunchKernelGGL((inertia_total_kernel<float>), dim3(1), dim3(256), 0, stream, partial, grid * gy, (float*)out);
         else
-            hipLaunchKernelGGL((inertia_total_kernel<double>), dim3(1), dim3(256), 0, stream, partial, grid, (double*)out);
+            hipLaunchKernelGGL((inertia_total_kernel<double>), dim3(1), dim3(256), 0, stream, partial, grid * gy, (double*)out);
     }
     KMX_LAUNCH_CHECK();
     return KMX_OK;
@@ -402,7 +427,7 @@ int32_t kmx_per_sample_inertia(const void* X_t, const void* sample_weight, const
 
 size_t kmx_inertia_workspace_bytes(int64_t n) {
     if (n <= 0) return 0;
-    return kmx_align256((size_t)stream_grid(kmx_cdiv(n, 4)) * sizeof(double));
+    return kmx_align256((size_t)inertia_partial_slots(n) * sizeof(double));
 }
 
 int32_t kmx_inertia(const void* X_t, const void* sample_weight, const void* centroids_t, const uint32_t* labels,

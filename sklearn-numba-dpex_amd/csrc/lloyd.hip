@@ -1270,6 +1270,9 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
         KMX_LAUNCH_CHECK();
         if (L.variant == KMX_VARIANT_MFMA)
             return kmx_assign_labels_mfma_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
+        // few clusters on wide samples: the products of the labels on the matrix cores, straight from X_t
+        if (L.variant == KMX_VARIANT_FEWK)
+            return kmx_assign_labels_fewk(X_t, centroids_t, ws + L.off_half, labels, n, d, k, stream);
         if (L.variant == KMX_VARIANT_MFMA_WIDE) {
             // with the larger workspace of kmx_assign_workspace_bytes_for: labels screened in fp16
             const size_t extra = kmx_assign_wide_screen_bytes(n, d, k, flags);

@@ -797,6 +797,118 @@ __global__ __launch_bounds__(1024) void fewk_reduce_kernel(const float* __restri
     }
 }
 
+// Labels only (kmx_assign_labels: predict, and the last step of a fit), straight from the
+// feature-major array, with no tile in LDS: for the labels alone the samples are only ever the N
+// side of the products, so a lane's 64- or 128-bit load of SV consecutive samples of one feature IS
+// the B operand of SV matrix instructions - sample block e of a tile holds the samples s0 + SV m + e,
+// m = 0 .. 15 - and the 16 lanes of a feature read one contiguous stretch.  Eight waves share the K
+// steps of a tile of 16 SV samples (centroid values in registers, as in the step above); their
+// partial scores meet in LDS and sixteen threads per sample take the arg-max.
+// (beyond 832 features the centroid values of a wave leave room for one workgroup per compute unit only)
+constexpr int fewk_labels_waves_per_simd(int kw) { return kw <= 26 ? 4 : 2; }
+template <int KW, int SV>
+__global__ __launch_bounds__(512)
+__attribute__((amdgpu_waves_per_eu(fewk_labels_waves_per_simd(KW), fewk_labels_waves_per_simd(KW))))
+void fewk_labels_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
+    uint32_t* __restrict__ labels, int64_t n, int d, int k, int vec_ok) {
+    constexpr int NW = 8, TS = 16 * SV;  // waves, samples per tile
+    constexpr int CH = SV == 4 ? 4 : 8;   // K steps whose loads are in flight together
+    __shared__ __align__(16) float part[NW][SV][256];  // [wave][block][sample m][cluster]
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int g4 = lane >> 4, m16 = lane & 15;
+    const int kw = fewk_kw(d, NW);  // K steps per wave (<= KW)
+    const int ks0 = wave * kw;
+    float ca[KW];
+#pragma unroll
+    for (int s = 0; s < KW; ++s) {
+        const int f = 4 * (ks0 + s) + g4;
+        const bool has = s < kw && f < d && m16 < k;
+        const float v = centroids_t[has ? (size_t)f * k + m16 : (size_t)0];
+        ca[s] = has ? v : 0.0f;
+    }
+    v4f start;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const float hn = half_norms[4 * g4 + r < k ? 4 * g4 + r : 0];
+        start[r] = (wave == 0 && 4 * g4 + r < k) ? -hn : 0.0f;
+    }
+    const int64_t n_tiles = (n + TS - 1) / TS;
+    for (int64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+        const int64_t s0 = t * TS;
+        const bool whole = vec_ok && s0 + TS <= n;  // workgroup-uniform
+        v4f sc[SV];
+#pragma unroll
+        for (int e = 0; e < SV; ++e) sc[e] = start;
+#pragma unroll
+        for (int c0 = 0; c0 < KW; c0 += CH) {
+            if (c0 < kw) {  // wave-uniform (past the wave's share the centroid value is zero)
+                float b[CH][SV];
+#pragma unroll
+                for (int j = 0; j < CH; ++j) {
+                    const int s = c0 + j;
+                    // (a feature past the last one: the row of the last, times a zero centroid value)
+                    const int f = 4 * (ks0 + s) + g4 < d ? 4 * (ks0 + s) + g4 : d - 1;
+                    const float* p = X_t + (size_t)f * n + s0 + SV * m16;
+                    if (s < KW) {
+                        if (whole) {
+                            if constexpr (SV == 4) {
+                                const float4 v = *reinterpret_cast<const float4*>(p);
+                                b[j][0] = v.x; b[j][1] = v.y; b[j][2] = v.z; b[j][3] = v.w;
+                            } else {
+                                const float2 v = *reinterpret_cast<const float2*>(p);
+                                b[j][0] = v.x; b[j][1] = v.y;
+                            }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < SV; ++e) b[j][e] = s0 + SV * m16 + e < n ? p[e] : 0.0f;
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);  // (the loads of the chunk, then its matrix instructions)
+#pragma unroll
+                for (int j = 0; j < CH; ++j)
+                    if (c0 + j < KW)
+#pragma unroll
+                        for (int e = 0; e < SV; ++e)
+                            sc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j < KW ? c0 + j : 0], b[j][e], sc[e], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int e = 0; e < SV; ++e) *reinterpret_cast<v4f*>(&part[wave][e][(m16 << 4) + 4 * g4]) = sc[e];
+        __syncthreads();
+        // sixteen threads per sample, one per cluster: the partial scores of the waves added in wave
+        // order, then the largest score, the lowest index among equals (a score that does not compare,
+        // or a cluster past the last, never wins)
+#pragma unroll
+        for (int rep = 0; rep < (SV * 256) / 512; ++rep) {
+            const int pair = threadIdx.x + 512 * rep;  // block e, sample m, cluster c
+            const int e = pair >> 8, m = (pair >> 4) & 15, c = pair & 15;
+            float best = part[0][e][pair & 255];
+#pragma unroll
+            for (int wv = 1; wv < NW; ++wv) best += part[wv][e][pair & 255];
+            uint32_t bi = (uint32_t)c;
+            if (!(c < k && best > -kmx_inf<float>())) {
+                best = -kmx_inf<float>();
+                bi = 0xffffffffu;
+            }
+#pragma unroll
+            for (int off = 1; off <= 8; off <<= 1) {
+                const float ov = __shfl_xor(best, off, 64);
+                const uint32_t oi = __shfl_xor(bi, off, 64);
+                const bool take = ov > best || (ov == best && oi < bi);
+                best = take ? ov : best;
+                bi = take ? oi : bi;
+            }
+            if (bi == 0xffffffffu) bi = 0u;  // no score compares: the reference's running arg-min keeps 0
+            const int64_t gi = s0 + SV * m + e;
+            if (c == 0 && gi < n) labels[gi] = bi;
+        }
+        __syncthreads();  // the partial scores are read: the next tile may overwrite them
+    }
+}
+
 // Samples per tile (a power of two, 16 .. 64) and workgroups per compute unit.
 struct FewkShape {
     int s_log, kw, nw, per_cu;
@@ -976,5 +1088,37 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
         (void)hipEventRecord(events[2], stream);
         (void)hipEventRecord(events[3], stream);
     }
+    return KMX_OK;
+}
+
+// Labels only for the shapes of this step (kmx_assign_labels), from the feature-major array.
+int32_t kmx_assign_labels_fewk(const void* X_t, const void* centroids_t, const void* half_norms, uint32_t* labels,
+                               int64_t n, int d, int k, hipStream_t stream) {
+    if (!kmx_fewk_supported(d, k)) return KMX_ERR_UNSUPPORTED;
+    // tiles of 64 samples; of 32 while those would not give every compute unit a few tiles
+    const int64_t tiles64 = kmx_cdiv(n, 64);
+    const bool small = tiles64 < (int64_t)8 * kmx_num_cus();
+    const int ts = small ? 32 : 64;
+    const int sv = ts / 16;
+    const int vec_ok = (n % sv == 0) && ((((uintptr_t)X_t) & (size_t)(4 * sv - 1)) == 0);
+    int64_t grid = (int64_t)2 * kmx_num_cus();
+    const int64_t tiles = kmx_cdiv(n, ts);
+    if (grid > tiles) grid = tiles;
+#define KMX_FEWK_LABELS(KW_, SV_)                                                                                     \
+    hipLaunchKernelGGL((fewk_labels_kernel<KW_, SV_>), dim3((unsigned)grid), dim3(512), 0, stream, (const float*)X_t, \
+                       (const float*)centroids_t, (const float*)half_norms, labels, n, d, k, vec_ok)
+    const int kw = fewk_kw(d, 8);
+    if (kw <= 16) {
+        if (small) KMX_FEWK_LABELS(16, 2);
+        else KMX_FEWK_LABELS(16, 4);
+    } else if (kw <= 26) {
+        if (small) KMX_FEWK_LABELS(26, 2);
+        else KMX_FEWK_LABELS(26, 4);
+    } else {
+        if (small) KMX_FEWK_LABELS(38, 2);
+        else KMX_FEWK_LABELS(38, 4);
+    }
+#undef KMX_FEWK_LABELS
+    KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

@@ -484,11 +484,16 @@ def n_samples_differ_cap(X):
     return X.shape[0] // 1000
 
 
-@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a"])
+@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a",
+                                  # few clusters on wide samples: the labels-only matrix-core kernel that reads
+                                  # the feature-major array directly (tiles of 32 and of 64 samples, every width
+                                  # of its centroid registers, n odd, n below a tile) and the inertia summed
+                                  # with the features split over workgroups
+                                  "K32a", "K32b", "K32d", "K32e", "K32f", "K32g", "K32j", "K32m", "K32n", "K32o", "K32p"])
 def test_labels_and_score_paths_on_every_label_kernel(cuda, name):
     """kmx_assign_labels, labels + inertia in one call and the distances on the shapes of the
-    tiled matrix-core product, of the labels-only fp64 matrix-core kernel and of the vector-ALU
-    kernels, against the oracle."""
+    tiled matrix-core product, of the labels-only fp64 matrix-core kernel, of the vector-ALU
+    kernels and of the few-cluster kernels, against the oracle."""
     import torch
 
     from sklearn_numba_dpex_amd.kmeans import drivers
