@@ -229,7 +229,7 @@ int32_t kmx_screen_scores(const void* X_t, const void* centroids_t, float* score
  * samples (vector ALU), 3 = MFMA (fp32) with the centroids resident in LDS, 4 = MFMA (fp32)
  * with samples in registers and centroids streamed (more than 256 clusters), 5 = MFMA (fp64)
  * with the centroids resident in LDS, 6 = labels by a tiled matrix-core product (any shape,
- * fp32 and fp64), 8 = fp32 with up to 16 clusters and 65 .. 1216 features: a tile of samples on chip
+ * fp32 and fp64), 8 = fp32 with up to 16 clusters and 65 .. 1792 features: a tile of samples on chip
  * serves labels and sums on the matrix cores, X read once; accumulation 1 = workgroup-private LDS accumulators, 2 = global sums,
  * 3 = labels only, then sums by a kernel of their own (per bucket of samples sorted by label,
  * or, fp32, straight from the labels into fixed-point accumulators in LDS where those of every

@@ -1,4 +1,4 @@
-// fp32 fused Lloyd step for FEW clusters (k <= 16) on WIDE samples (64 < d <= 1216), reading X
+// fp32 fused Lloyd step for FEW clusters (k <= 16) on WIDE samples (64 < d <= 1792), reading X
 // once per iteration.
 //
 // Replaces, for these shapes, the kernel pair fused_lloyd_single_step
@@ -71,7 +71,7 @@ __host__ __device__ inline FewkLds fewk_lds(int d, int S, int nw, bool two_tiles
 
 // 128-bit pieces of the next tile a thread holds in registers (d * S / 4 values over the threads)
 constexpr int fewk_prefetch(int kw, int s_log, int nw) {
-    if (nw == 8) return kw <= 26 ? 7 : 10;
+    if (nw == 8) return kw <= 26 ? 7 : kw <= 38 ? 10 : 16;
     return (kw <= 8 && s_log == 5) ? 4 : kw <= 16 ? 8 : kw <= 32 ? 10 : kw <= 52 ? 13 : 19;  // ((8, 6): 8)
 }
 
@@ -88,7 +88,7 @@ constexpr int fewk_prefetch(int kw, int s_log, int nw) {
 // (two waves per SIMD - two workgroups of four waves per compute unit - up to 832 features: 256
 // registers; four with tiles of 32 samples of up to 128 features and with eight waves up to 832)
 constexpr int fewk_waves_per_simd(int kw, int s_log, int nw, int direct = 0) {
-    if (nw == 8) return direct == 1 ? 4 : 2;
+    if (nw == 8) return (direct == 1 && kw <= 26) ? 4 : 2;
     if (direct == 1) return 4;
     return (kw <= 8 && s_log == 5) ? 4 : kw <= 52 ? 2 : 1;
 }
@@ -916,11 +916,11 @@ struct FewkShape {
 };
 
 bool fewk_shape(int d, int k, FewkShape* out) {
-    if (d <= 64 || d > 1216 || k < 1 || k > 16) return false;
+    if (d <= 64 || d > 1792 || k < 1 || k > 16) return false;
     // (eight waves per workgroup beyond 512 features)
     const int nw = d > 512 ? 8 : 4;
     const int kw = fewk_kw(d, nw);
-    const int kw_t = nw == 8 ? (kw <= 26 ? 26 : 38) : kw <= 8 ? 8 : kw <= 16 ? 16 : 32;
+    const int kw_t = nw == 8 ? (kw <= 26 ? 26 : kw <= 38 ? 38 : 64) : kw <= 8 ? 8 : kw <= 16 ? 16 : 32;
     // (tiles of 32 samples up to 512 features while two workgroups fit a compute unit, of 16 beyond:
     // the instantiated kernels; measured at 2e6 x 100: tiles of 64 samples, which leave room for two
     // workgroups per compute unit instead of four, are no faster)
@@ -935,7 +935,7 @@ bool fewk_shape(int d, int k, FewkShape* out) {
         if (lds <= cap && pieces <= fewk_prefetch(kw_t, s_log, nw)) {
             const int by_lds = (int)((size_t)160 * 1024 / (lds + 512));
             // workgroups per compute unit the kernel's registers allow (waves per SIMD it is built for)
-            const bool direct = s_log == 4 && (nw == 4 || kw_t == 26);
+            const bool direct = s_log == 4 && (nw == 4 || kw_t != 38);
             const int by_regs = fewk_waves_per_simd(kw_t, s_log, nw, direct ? 1 : 0) * 4 / nw;
             const int per_cu = by_lds < by_regs ? by_lds : by_regs;
             out->s_log = s_log;
@@ -1050,7 +1050,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
     } else {
 #define KMX_FEWK_LAUNCH_RM(KW_, SL_, RM_, NW_)                                                             \
     do {                                                                                                  \
-        constexpr int direct_ = (RM_ && SL_ == 4 && (NW_ == 4 || KW_ == 26)) ? 1 : 0;                     \
+        constexpr int direct_ = (RM_ && SL_ == 4 && (NW_ == 4 || KW_ != 38)) ? 1 : 0;                     \
         if (sh.lds > 64 * 1024) {                                                                         \
             const hipError_t e = hipFuncSetAttribute(                                                     \
                 reinterpret_cast<const void*>(&lloyd_fewk_kernel<KW_, SL_, RM_, NW_, direct_>),           \
@@ -1078,6 +1078,7 @@ int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X
         else if (sh.nw == 4 && sh.kw == 32 && sh.s_log == 4) KMX_FEWK_LAUNCH(32, 4, 9, 4);
         else if (sh.nw == 8 && sh.kw == 26 && sh.s_log == 4) KMX_FEWK_LAUNCH(26, 4, 7, 8);
         else if (sh.nw == 8 && sh.kw == 38 && sh.s_log == 4) KMX_FEWK_LAUNCH(38, 4, 10, 8);
+        else if (sh.nw == 8 && sh.kw == 64 && sh.s_log == 4) KMX_FEWK_LAUNCH(64, 4, 17, 8);
         else return KMX_ERR_UNSUPPORTED;
 #undef KMX_FEWK_LAUNCH_RM
 #undef KMX_FEWK_LAUNCH
@@ -1114,9 +1115,12 @@ int32_t kmx_assign_labels_fewk(const void* X_t, const void* centroids_t, const v
     } else if (kw <= 26) {
         if (small) KMX_FEWK_LABELS(26, 2);
         else KMX_FEWK_LABELS(26, 4);
-    } else {
+    } else if (kw <= 38) {
         if (small) KMX_FEWK_LABELS(38, 2);
         else KMX_FEWK_LABELS(38, 4);
+    } else {
+        if (small) KMX_FEWK_LABELS(64, 2);
+        else KMX_FEWK_LABELS(64, 4);
     }
 #undef KMX_FEWK_LABELS
     KMX_LAUNCH_CHECK();

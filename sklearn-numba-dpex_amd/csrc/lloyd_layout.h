@@ -11,7 +11,7 @@ constexpr int KMX_VARIANT_MFMA = 3;      // fp32 distances on the matrix cores, 
 constexpr int KMX_VARIANT_MFMA_WIDE = 4; // fp32 matrix cores, samples in registers, global sums
 constexpr int KMX_VARIANT_MFMA_F64 = 5;  // fp64 distances on the matrix cores, LDS accumulators
 constexpr int KMX_VARIANT_GEMM = 6;      // labels by a tiled matrix-core product (any shape), bucketed sums
-constexpr int KMX_VARIANT_FEWK = 8;      // fp32, up to 16 clusters, 65 .. 1216 features: a tile of samples in LDS serves labels and sums
+constexpr int KMX_VARIANT_FEWK = 8;      // fp32, up to 16 clusters, 65 .. 1792 features: a tile of samples in LDS serves labels and sums
 
 constexpr int KMX_ACC_LDS = 1;
 constexpr int KMX_ACC_GLOBAL = 2;

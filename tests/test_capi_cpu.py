@@ -131,7 +131,8 @@ def test_kernel_variant_selection():
     assert lib.kmx_lloyd_kernel_variant(100_000, 784, 10, 0, 0) == 81
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 0, 0x1) == 1   # on request: the fused vector-ALU step
     assert lib.kmx_lloyd_kernel_variant(100_000, 784, 10, 0, 0x4) == 63    # or the tiled product with sums per bucket
-    assert lib.kmx_lloyd_kernel_variant(100_000, 1300, 10, 0, 0) == 63     # a tile of such samples does not fit the LDS
+    assert lib.kmx_lloyd_kernel_variant(100_000, 1300, 10, 0, 0) == 81
+    assert lib.kmx_lloyd_kernel_variant(100_000, 1800, 10, 0, 0) == 63     # a tile of such samples does not fit the LDS
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 1, 0) == 1     # fp64: as before
     assert lib.kmx_lloyd_kernel_variant(5_000_000, 14, 127, 0, 0x4) == 63  # the tiled product on request
     assert lib.kmx_lloyd_kernel_variant(0, 3, 5, 0, 0) == -2

@@ -95,6 +95,9 @@ def _small_configs():
         "K32o": lambda: dict(_blob_config(4_100, 512, 16, np.float32, 61), variant=81),
         "K32p": lambda: dict(_blob_config(1_030, 832, 5, np.float32, 62, skew=True), variant=81),
         "K32q": lambda: dict(_blob_config(777, 256, 11, np.float32, 63), variant=81),
+        # the widest samples of this step: one workgroup per compute unit, with and without the row-major copy
+        "K32r": lambda: dict(_blob_config(1_500, 1792, 4, np.float32, 64), variant=81),
+        "K32s": lambda: dict(_blob_config(2_003, 1500, 16, np.float32, 65), variant=81),
         "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
         # extremes of the tiled product: thousands of features (many passes of the bucketed sums),
         # more clusters than the bucket counts hold in LDS and than the wide path takes
@@ -148,7 +151,7 @@ def _odd_config():
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
                                   "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
                                   "K32a", "K32b", "K32c", "K32d", "K32e", "K32f", "K32g", "K32h", "K32i",
-                                  "K32j", "K32k", "K32l", "K32m", "K32n", "K32o", "K32p", "K32q"])
+                                  "K32j", "K32k", "K32l", "K32m", "K32n", "K32o", "K32p", "K32q", "K32r", "K32s"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
     import torch
 
@@ -489,7 +492,7 @@ def n_samples_differ_cap(X):
                                   # the feature-major array directly (tiles of 32 and of 64 samples, every width
                                   # of its centroid registers, n odd, n below a tile) and the inertia summed
                                   # with the features split over workgroups
-                                  "K32a", "K32b", "K32d", "K32e", "K32f", "K32g", "K32j", "K32m", "K32n", "K32o", "K32p"])
+                                  "K32a", "K32b", "K32d", "K32e", "K32f", "K32g", "K32j", "K32m", "K32n", "K32o", "K32p", "K32r", "K32s"])
 def test_labels_and_score_paths_on_every_label_kernel(cuda, name):
     """kmx_assign_labels, labels + inertia in one call and the distances on the shapes of the
     tiled matrix-core product, of the labels-only fp64 matrix-core kernel, of the vector-ALU
