@@ -551,28 +551,46 @@ __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
 }
 
 // Packed (k, dpad) copy of the centroids + half squared norms; optional status reset.
-constexpr int PACK_CLUSTERS = 32;
-template <typename T>
+// LANES feature lanes per cluster (256 / LANES clusters per workgroup): lane g of a cluster takes
+// the features g, g + LANES, ...; 8 lanes, or 64 for wide samples, where eight lanes would each
+// walk a hundred features, a trip to memory per value.
+template <typename T, int LANES>
 __global__ __launch_bounds__(256) void lloyd_pack_kernel(const T* __restrict__ centroids_t,
                                                          T* __restrict__ cpack,
                                                          T* __restrict__ half_norms,
                                                          kmx_lloyd_status* __restrict__ status,
                                                          int d, int k, int dpad, int max_iter,
                                                          double tol) {
-    // 32 clusters x 8 feature lanes per workgroup: lane g of a cluster takes features g, g+8, ...
-    const int g = threadIdx.x & 7;
-    const int c = blockIdx.x * PACK_CLUSTERS + (threadIdx.x >> 3);
+    const int g = threadIdx.x & (LANES - 1);
+    const int c = blockIdx.x * (256 / LANES) + (int)(threadIdx.x / LANES);
     T sq = T(0);
     if (c < k) {
-        for (int f = g; f < dpad; f += 8) {
-            const T v = f < d ? centroids_t[(size_t)f * k + c] : T(0);
-            sq += v * v;
-            cpack[(size_t)c * dpad + f] = v;
+        if constexpr (LANES == 8) {
+            for (int f = g; f < dpad; f += 8) {
+                const T v = f < d ? centroids_t[(size_t)f * k + c] : T(0);
+                sq += v * v;
+                cpack[(size_t)c * dpad + f] = v;
+            }
+        } else {
+            // (eight loads in flight, then their stores)
+            for (int f0 = g; f0 < dpad; f0 += 8 * LANES) {
+                T v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int f = f0 + u * LANES;
+                    v[u] = f < d ? centroids_t[(size_t)f * k + c] : T(0);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int f = f0 + u * LANES;
+                    sq += v[u] * v[u];
+                    if (f < dpad) cpack[(size_t)c * dpad + f] = v[u];
+                }
+            }
         }
     }
-    sq += __shfl_xor(sq, 1, 64);
-    sq += __shfl_xor(sq, 2, 64);
-    sq += __shfl_xor(sq, 4, 64);
+#pragma unroll
+    for (int off = 1; off < LANES; off <<= 1) sq += __shfl_xor(sq, off, 64);
     if (c < k && g == 0) half_norms[c] = sq / T(2);
     if (status != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         status->n_iter = 0;
@@ -587,6 +605,17 @@ __global__ __launch_bounds__(256) void lloyd_pack_kernel(const T* __restrict__ c
         status->reserved[0] = 0;
         status->reserved[1] = 0;
     }
+}
+
+template <typename T>
+static void launch_pack(const void* centroids_t, void* cpack, void* half_norms, kmx_lloyd_status* status, int d, int k,
+                        int dpad, int max_iter, double tol, hipStream_t stream) {
+    if (d >= 256)
+        hipLaunchKernelGGL((lloyd_pack_kernel<T, 64>), dim3((unsigned)kmx_cdiv(k, 4)), dim3(256), 0, stream,
+                           (const T*)centroids_t, (T*)cpack, (T*)half_norms, status, d, k, dpad, max_iter, tol);
+    else
+        hipLaunchKernelGGL((lloyd_pack_kernel<T, 8>), dim3((unsigned)kmx_cdiv(k, 32)), dim3(256), 0, stream,
+                           (const T*)centroids_t, (T*)cpack, (T*)half_norms, status, d, k, dpad, max_iter, tol);
 }
 
 __global__ void fill_zero_bytes_kernel(uint32_t* __restrict__ p, size_t n_words) {
@@ -953,15 +982,10 @@ int32_t kmx_lloyd_init(const kmx_lloyd_plan* plan, void* workspace, size_t works
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
-    const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32)
-        hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
-                           (const float*)centroids_t, (float*)(ws + L.off_cpack),
-                           (float*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
+        launch_pack<float>(centroids_t, ws + L.off_cpack, ws + L.off_half, status, d, k, L.dpad, max_iter, tol, stream);
     else
-        hipLaunchKernelGGL((lloyd_pack_kernel<double>), dim3(grid), dim3(256), 0, stream,
-                           (const double*)centroids_t, (double*)(ws + L.off_cpack),
-                           (double*)(ws + L.off_half), status, d, k, L.dpad, max_iter, tol);
+        launch_pack<double>(centroids_t, ws + L.off_cpack, ws + L.off_half, status, d, k, L.dpad, max_iter, tol, stream);
     KMX_LAUNCH_CHECK();
     if (L.variant == KMX_VARIANT_MFMA || L.variant == KMX_VARIANT_MFMA_WIDE || L.gemm_screen || L.direct_sums ||
         L.screen64 || L.variant == KMX_VARIANT_FEWK) {
@@ -1258,15 +1282,11 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
     if (workspace_bytes < L.off_bucket) return KMX_ERR_WORKSPACE;
     hipStream_t stream = (hipStream_t)stream_;
     char* ws = (char*)workspace;
-    const unsigned grid = (unsigned)kmx_cdiv(k, PACK_CLUSTERS);
     if (dtype == KMX_F32) {
         // labels screened on the fp16 matrix cores: one kernel, straight from the centroids
         if (L.screen || L.screen_labels)
             return kmx_assign_labels_mfma_screen(X_t, centroids_t, labels, n, d, k, L.wgs_per_cu, stream);
-        hipLaunchKernelGGL((lloyd_pack_kernel<float>), dim3(grid), dim3(256), 0, stream,
-                           (const float*)centroids_t, (float*)(ws + L.off_cpack),
-                           (float*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
-                           0.0);
+        launch_pack<float>(centroids_t, ws + L.off_cpack, ws + L.off_half, nullptr, d, k, L.dpad, 0, 0.0, stream);
         KMX_LAUNCH_CHECK();
         if (L.variant == KMX_VARIANT_MFMA)
             return kmx_assign_labels_mfma_f32(L, X_t, centroids_t, labels, ws, n, d, k, stream);
@@ -1299,10 +1319,7 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
                                                          nullptr, n, d, k, stream, absmax, area);
         if (rc != KMX_OK) return rc;
     } else {
-        hipLaunchKernelGGL((lloyd_pack_kernel<double>), dim3(grid), dim3(256), 0, stream,
-                           (const double*)centroids_t, (double*)(ws + L.off_cpack),
-                           (double*)(ws + L.off_half), (kmx_lloyd_status*)nullptr, d, k, L.dpad, 0,
-                           0.0);
+        launch_pack<double>(centroids_t, ws + L.off_cpack, ws + L.off_half, nullptr, d, k, L.dpad, 0, 0.0, stream);
         KMX_LAUNCH_CHECK();
         const int32_t rc = launch_fused<double, ACC_NONE>(L, X_t, nullptr, centroids_t,
                                                           (const double*)(ws + L.off_cpack),
