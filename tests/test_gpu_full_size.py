@@ -238,11 +238,13 @@ def test_large_shapes_off_the_benchmark_configurations(cuda, shape):
     assert all(b <= a * (1 + 1e-6) for a, b in zip(inertias, inertias[1:])), inertias
 
 
-@pytest.mark.parametrize("n,d,k,variant", [(4_300_000, 512, 300, 63), (8_500_000, 256, 512, 42)])
+@pytest.mark.parametrize("n,d,k,variant", [(4_300_000, 512, 300, 63), (8_500_000, 256, 512, 42), (2_800_000, 784, 10, 81)])
 def test_array_past_two_to_the_31_elements(cuda, n, d, k, variant):
-    """4 300 000 x 512 (tiled product + sums per bucket) and 8 500 000 x 256 with 512 clusters (the
+    """4 300 000 x 512 (tiled product + sums per bucket), 8 500 000 x 256 with 512 clusters (the
     wide path: labels screened in fp16, fp32 pass over the uncertified samples, bucketed
-    accumulation) in fp32: 2.2e9 elements, 8.8 GB, generated on the device.  Feature rows from
+    accumulation) and 2 800 000 x 784 with 10 clusters (the few-cluster step: tiles loaded from the
+    row-major copy straight into LDS; its labels-only kernel and the inertia split over the
+    features at the end) in fp32: 2.2e9 elements, 8.8 GB, generated on the device.  Feature rows from
     125 on start more than 2^31 bytes into the array and the last samples of the last row lie
     past element 2^31: three Lloyd iterations through the C ABI (tiled matrix-core labels, sums
     per bucket of samples from the row-major copy), checked through size-independent properties
