@@ -22,7 +22,8 @@
 
 namespace {
 
-constexpr int BUCKET_CHUNK = 1024;       // positions of `order` per workgroup of bucket_sum
+constexpr int BUCKET_CHUNK = 1024;       // positions of `order` per workgroup of bucket_sum (fewer where the
+                                         // array is small: see bucket_sum_chunk)
 constexpr int BUCKET_COUNT_TILE = 2048;  // samples per workgroup and pass of bucket_count
 constexpr int BUCKET_LDS_K = 4096;       // clusters whose counts are gathered in LDS first
 
@@ -130,13 +131,15 @@ template <typename T, bool ROW_MAJOR, int NJ>
 __global__ __launch_bounds__(256) void bucket_sum_kernel(
     const T* __restrict__ X, const T* __restrict__ sample_weight, const int* __restrict__ order,
     const int* __restrict__ offsets, int* __restrict__ counts, T* __restrict__ sums,
-    const kmx_lloyd_status* __restrict__ status, int n, int d, int k) {
+    const kmx_lloyd_status* __restrict__ status, int n, int d, int k, int chunk) {
     if (status->state != KMX_RUNNING) return;
     constexpr int FB = 64 * NJ;  // features per pass
     __shared__ double red[4][FB + 1];
     __shared__ int c_first;
-    const int P0 = blockIdx.x * BUCKET_CHUNK;
-    const int P1 = P0 + BUCKET_CHUNK < n ? P0 + BUCKET_CHUNK : n;
+    // (a chunk of `chunk` positions per workgroup, and the passes over the features dealt out over
+    // the second grid dimension)
+    const int P0 = blockIdx.x * chunk;
+    const int P1 = P0 + chunk < n ? P0 + chunk : n;
     for (int c = blockIdx.x * 256 + threadIdx.x; c < k; c += gridDim.x * 256) counts[c] = 0;
     if (threadIdx.x == 0) c_first = k;
     __syncthreads();
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(256) void bucket_sum_kernel(
     constexpr int U = 4;  // samples in flight per wave
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-    for (int fb = 0; fb < d; fb += FB) {
+    for (int fb = (int)blockIdx.y * FB; fb < d; fb += (int)gridDim.y * FB) {
         size_t col[NJ];   // the lane's features of this pass (clamped: past d the value is dropped)
         bool live[NJ];
 #pragma unroll
@@ -331,10 +334,20 @@ int32_t kmx_lloyd_bucket_sums(const void* X_t, const void* X_rowmajor, const voi
     KMX_LAUNCH_CHECK();
     const int32_t rc = kmx_bucket_order(labels, counts, offsets, ranks, order, n, k, stream);
     if (rc != KMX_OK) return rc;
-    const unsigned ag = (unsigned)kmx_cdiv(n, BUCKET_CHUNK);
+    // With few samples a chunk of 1024 positions per workgroup leaves most compute units without
+    // one (10^5 samples: 98 workgroups): smaller chunks, down to 128 positions, and the passes over
+    // the features side by side, until there are about four workgroups per compute unit.
+    const int64_t want = (int64_t)4 * kmx_num_cus();
+    int chunk = BUCKET_CHUNK;
+    while (chunk > 128 && kmx_cdiv(n, chunk) < want) chunk >>= 1;
+    const unsigned ag = (unsigned)kmx_cdiv(n, chunk);
+    const int fb_features = d <= 64 ? 64 : d <= 128 ? 128 : 256;
+    int64_t gy = kmx_cdiv(want, ag);
+    if (gy > kmx_cdiv(d, fb_features)) gy = kmx_cdiv(d, fb_features);
+    if (gy < 1) gy = 1;
 #define KMX_BUCKET_SUM_NJ(T, RM, XP, NJ_)                                                                \
-    hipLaunchKernelGGL((bucket_sum_kernel<T, RM, NJ_>), dim3(ag), dim3(256), 0, stream, (const T*)(XP), \
-                       (const T*)w, order, offsets, counts, (T*)sums, status, (int)n, d, k)
+    hipLaunchKernelGGL((bucket_sum_kernel<T, RM, NJ_>), dim3(ag, (unsigned)gy), dim3(256), 0, stream,   \
+                       (const T*)(XP), (const T*)w, order, offsets, counts, (T*)sums, status, (int)n, d, k, chunk)
 #define KMX_BUCKET_SUM(T, RM, XP)                      \
     do {                                               \
         if (d <= 64) KMX_BUCKET_SUM_NJ(T, RM, XP, 1);  \
