@@ -909,6 +909,101 @@ void fewk_labels_kernel(
     }
 }
 
+// The same up to 128 features, where a wave holds the centroid values of all features: every wave
+// on tiles of 64 samples of its own, scores complete in its registers - no LDS, no barrier.
+template <int KS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void fewk_labels_wave_kernel(
+    const float* __restrict__ X_t, const float* __restrict__ centroids_t, const float* __restrict__ half_norms,
+    uint32_t* __restrict__ labels, int64_t n, int d, int k, int vec_ok) {
+    constexpr int SV = 4, TS = 16 * SV, CH = 4;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int g4 = lane >> 4, m16 = lane & 15;
+    const int ksteps = (d + 3) >> 2;
+    float ca[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int f = 4 * s + g4;
+        const bool has = f < d && m16 < k;
+        const float v = centroids_t[has ? (size_t)f * k + m16 : (size_t)0];
+        ca[s] = has ? v : 0.0f;
+    }
+    v4f start;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const float hn = half_norms[4 * g4 + r < k ? 4 * g4 + r : 0];
+        start[r] = (4 * g4 + r < k) ? -hn : 0.0f;
+    }
+    const int64_t n_tiles = (n + TS - 1) / TS;
+    for (int64_t t = (int64_t)blockIdx.x * 4 + wave; t < n_tiles; t += (int64_t)gridDim.x * 4) {
+        const int64_t s0 = t * TS;
+        const bool whole = vec_ok && s0 + TS <= n;  // wave-uniform
+        v4f sc[SV];
+#pragma unroll
+        for (int e = 0; e < SV; ++e) sc[e] = start;
+#pragma unroll
+        for (int c0 = 0; c0 < KS; c0 += CH) {
+            if (c0 < ksteps) {  // wave-uniform (past d the centroid values are zero)
+                float b[CH][SV];
+#pragma unroll
+                for (int j = 0; j < CH; ++j) {
+                    const int f = 4 * (c0 + j) + g4 < d ? 4 * (c0 + j) + g4 : d - 1;
+                    const float* p = X_t + (size_t)f * n + s0 + SV * m16;
+                    if (whole) {
+                        const float4 v = *reinterpret_cast<const float4*>(p);
+                        b[j][0] = v.x; b[j][1] = v.y; b[j][2] = v.z; b[j][3] = v.w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < SV; ++e) b[j][e] = s0 + SV * m16 + e < n ? p[e] : 0.0f;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);  // (the loads of the chunk, then its matrix instructions)
+#pragma unroll
+                for (int j = 0; j < CH; ++j)
+                    if (c0 + j < KS)
+#pragma unroll
+                        for (int e = 0; e < SV; ++e)
+                            sc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[c0 + j < KS ? c0 + j : 0], b[j][e], sc[e], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // arg-max of sample SV m16 + e: the lane's clusters 4 g4 + r in increasing order (strict '>'),
+        // then the four lane groups: the largest score, the lowest index among equals
+        uint32_t lab[SV];
+#pragma unroll
+        for (int e = 0; e < SV; ++e) {
+            float best = -kmx_inf<float>();
+            uint32_t bi = 0xffffffffu;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = sc[e][r];
+                if (4 * g4 + r < k && v > best) {
+                    best = v;
+                    bi = (uint32_t)(4 * g4 + r);
+                }
+            }
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const float ov = __shfl_xor(best, off, 64);
+                const uint32_t oi = __shfl_xor(bi, off, 64);
+                const bool take = ov > best || (ov == best && oi < bi);
+                best = take ? ov : best;
+                bi = take ? oi : bi;
+            }
+            lab[e] = bi == 0xffffffffu ? 0u : bi;  // no score compares: the reference's running arg-min keeps 0
+        }
+        if (g4 == 0) {
+            const int64_t gi = s0 + SV * m16;
+            if (whole) {
+                *reinterpret_cast<uint4*>(labels + gi) = make_uint4(lab[0], lab[1], lab[2], lab[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < SV; ++e)
+                    if (gi + e < n) labels[gi + e] = lab[e];
+            }
+        }
+    }
+}
+
 // Samples per tile (a power of two, 16 .. 64) and workgroups per compute unit.
 struct FewkShape {
     int s_log, kw, nw, per_cu;
@@ -1098,6 +1193,16 @@ int32_t kmx_assign_labels_fewk(const void* X_t, const void* centroids_t, const v
     if (!kmx_fewk_supported(d, k)) return KMX_ERR_UNSUPPORTED;
     // tiles of 64 samples; of 32 while those would not give every compute unit a few tiles
     const int64_t tiles64 = kmx_cdiv(n, 64);
+    if (d <= 128 && tiles64 >= (int64_t)16 * kmx_num_cus()) {
+        // every wave on tiles of its own (labels are written 128 bits at a time: 16-byte aligned)
+        const int vec = (n % 4 == 0) && ((((uintptr_t)X_t) & 15) == 0) && ((((uintptr_t)labels) & 15) == 0);
+        int64_t wg = (int64_t)3 * kmx_num_cus();
+        if (wg > kmx_cdiv(tiles64, 4)) wg = kmx_cdiv(tiles64, 4);
+        hipLaunchKernelGGL((fewk_labels_wave_kernel<32>), dim3((unsigned)wg), dim3(256), 0, stream, (const float*)X_t,
+                           (const float*)centroids_t, (const float*)half_norms, labels, n, d, k, vec);
+        KMX_LAUNCH_CHECK();
+        return KMX_OK;
+    }
     const bool small = tiles64 < (int64_t)8 * kmx_num_cus();
     const int ts = small ? 32 : 64;
     const int sv = ts / 16;

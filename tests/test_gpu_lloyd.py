@@ -98,6 +98,8 @@ def _small_configs():
         # the widest samples of this step: one workgroup per compute unit, with and without the row-major copy
         "K32r": lambda: dict(_blob_config(1_500, 1792, 4, np.float32, 64), variant=81),
         "K32s": lambda: dict(_blob_config(2_003, 1500, 16, np.float32, 65), variant=81),
+        # enough samples for the labels-only kernel with a tile per wave, n odd (no 128-bit accesses)
+        "K32t": lambda: dict(_blob_config(270_001, 96, 7, np.float32, 66), variant=81),
         "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
         # extremes of the tiled product: thousands of features (many passes of the bucketed sums),
         # more clusters than the bucket counts hold in LDS and than the wide path takes
@@ -492,7 +494,7 @@ def n_samples_differ_cap(X):
                                   # the feature-major array directly (tiles of 32 and of 64 samples, every width
                                   # of its centroid registers, n odd, n below a tile) and the inertia summed
                                   # with the features split over workgroups
-                                  "K32a", "K32b", "K32d", "K32e", "K32f", "K32g", "K32j", "K32m", "K32n", "K32o", "K32p", "K32r", "K32s"])
+                                  "K32a", "K32b", "K32d", "K32e", "K32f", "K32g", "K32j", "K32m", "K32n", "K32o", "K32p", "K32r", "K32s", "K32t"])
 def test_labels_and_score_paths_on_every_label_kernel(cuda, name):
     """kmx_assign_labels, labels + inertia in one call and the distances on the shapes of the
     tiled matrix-core product, of the labels-only fp64 matrix-core kernel, of the vector-ALU
