@@ -1319,6 +1319,9 @@ int32_t kmx_assign_labels(const void* X_t, const void* centroids_t, uint32_t* la
                                                          nullptr, n, d, k, stream, absmax, area);
         if (rc != KMX_OK) return rc;
     } else {
+        // fp64 inputs of the screened step: the same kernel without the update
+        if (L.screen64)
+            return kmx_assign_labels_mfma_screen_f64(X_t, centroids_t, labels, n, d, k, L.wgs_per_cu, stream);
         launch_pack<double>(centroids_t, ws + L.off_cpack, ws + L.off_half, nullptr, d, k, L.dpad, 0, 0.0, stream);
         KMX_LAUNCH_CHECK();
         const int32_t rc = launch_fused<double, ACC_NONE>(L, X_t, nullptr, centroids_t,

@@ -304,6 +304,8 @@ int32_t kmx_lloyd_iter_mfma_screen_f64(const LloydLayout& L, const void* X_t, co
                                        const uint32_t* labels_prev, uint32_t* labels, void* sizes,
                                        uint32_t* empty_clusters, char* ws, int64_t n, int d, int k,
                                        hipStream_t stream, hipEvent_t* events);
+int32_t kmx_assign_labels_mfma_screen_f64(const void* X_t, const void* centroids_t, uint32_t* labels, int64_t n,
+                                          int d, int k, int wgs_per_cu, hipStream_t stream);
 int32_t kmx_assign_labels_fewk(const void* X_t, const void* centroids_t, const void* half_norms, uint32_t* labels,
                                int64_t n, int d, int k, hipStream_t stream);
 int32_t kmx_lloyd_iter_fewk(const LloydLayout& L, const void* X_t, const void* X_rowmajor, const void* w,

@@ -1821,7 +1821,7 @@ int32_t launch_screen(const void* X_t, const void* w, const void* centroids_t, c
                       double* inertia_partial = nullptr, int* grid_out = nullptr,
                       const LloydTail<TX>* tail = nullptr) {
     constexpr int ES = (int)sizeof(TX);
-    static_assert(ES == 4 || (UPDATE && !INERTIA), "fp64 inputs: the fused step only");
+    static_assert(ES == 4 || !INERTIA, "fp64 inputs: labels and inertia are two calls");
     if (!(ES == 8 ? screen_fits_f64(n, d, k)
                   : (UPDATE ? kmx_mfma_screen_fits(n, d, k) : kmx_mfma_screen_labels_fits(n, d, k))))
         return KMX_ERR_UNSUPPORTED;
@@ -1905,6 +1905,13 @@ int32_t kmx_assign_labels_mfma_screen(const void* X_t, const void* centroids_t, 
                                       int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
     return launch_screen<false>(X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr, nullptr,
                                 nullptr, nullptr, nullptr, n, d, k, wgs_per_cu, stream);
+}
+
+// Labels only on fp64 inputs (the shapes of the fused fp64 step).
+int32_t kmx_assign_labels_mfma_screen_f64(const void* X_t, const void* centroids_t, uint32_t* labels,
+                                          int64_t n, int d, int k, int wgs_per_cu, hipStream_t stream) {
+    return launch_screen<false, false, double>(X_t, nullptr, centroids_t, nullptr, labels, nullptr, nullptr, nullptr,
+                                               nullptr, nullptr, nullptr, n, d, k, wgs_per_cu, stream);
 }
 
 // The same inside the iteration loop (no work once the run's state is terminal).

@@ -489,7 +489,7 @@ def n_samples_differ_cap(X):
     return X.shape[0] // 1000
 
 
-@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a",
+@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "F64h", "F64i", "F64j", "C5", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "R64a", "R32a", "S64a", "S32a",
                                   # few clusters on wide samples: the labels-only matrix-core kernel that reads
                                   # the feature-major array directly (tiles of 32 and of 64 samples, every width
                                   # of its centroid registers, n odd, n below a tile) and the inertia summed

@@ -891,3 +891,16 @@ def test_fp64_certificate_passes_no_label_that_fp64_would_not_give(cuda, d, k, s
     # (most of these samples cannot be certified; with spread centroids a third, smaller centroid is
     # often nearer than the pair whose bisector the sample was put on, and fewer stay uncertain)
     assert rechecked > (n // 4 if spread == 1.0 else n // 20)
+    # the same kernel without the update (kmx_assign_labels on fp64 inputs): the same bar
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    X_t = torch.as_tensor(np.ascontiguousarray(X.T), device=cuda)
+    C_t = torch.as_tensor(np.ascontiguousarray(C.T), device=cuda)
+    assigned = torch.full((n,), -1, dtype=torch.int32, device=cuda)
+    drivers._assign(X_t, C_t, assigned)
+    got = assigned.cpu().numpy().astype(np.int64)
+    bad = np.flatnonzero(got != ref)
+    gap = (dist[bad, got[bad]] - dist[bad, ref[bad]]) / dist[bad].max(axis=1)
+    assert np.all(gap <= 1e-14), f"assign: {bad.size} labels differ, worst relative gap {gap.max():.3e}"
