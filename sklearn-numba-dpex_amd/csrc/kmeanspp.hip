@@ -25,6 +25,8 @@ namespace {
 
 constexpr int TN_MAX = 16;      // n_local_trials = 2 + floor(ln k) <= 16 for k < 1.2e6
 constexpr int CHUNK = 1024;     // samples per workgroup (256 threads x 4)
+constexpr int SPLIT_MIN_D = 64; // from this many features on, few samples are stepped with the
+                                // features split over the four waves of a workgroup
 
 struct KppHeader {
     int32_t best_row;
@@ -35,11 +37,30 @@ struct KppHeader {
 struct KppLayout {
     size_t off_header, off_cand, off_pot, off_cand_rows, off_block_pot, off_rows, total;
     int64_t n_blocks;
+    int chunk;  // samples per block sum: CHUNK, or 64 * split
+    int split;  // 0, or the samples per thread (1, 2, 4) of the feature-split step kernel
 };
 
+// Samples per thread of the feature-split step kernel, 0 when the shape keeps the plain one.
+// With CHUNK samples per workgroup a short, wide array gives the chip a few dozen workgroups
+// that each walk every feature; 64 * split samples per workgroup and a quarter of the features
+// per wave give it thousands of waves.  The block sums stay at most 1 024, which the selection
+// kernel keeps in registers, and the partial distances of 8 trials fit the workgroup's LDS.
+int kpp_split(int64_t n, int d, int n_trials, int dtype) {
+    if (d < SPLIT_MIN_D || n_trials > 8) return 0;
+    if (n <= 65536) return 1;
+    if (n <= 131072) return 2;
+    if (n <= 262144 && dtype == KMX_F32) return 4;
+    return 0;
+}
+
+// The layout, the block sums included, depends on the shape only: calls with either sampler
+// may follow one another on one workspace.
 KppLayout kpp_layout(int64_t n, int d, int n_trials, int dtype) {
     KppLayout L;
-    L.n_blocks = kmx_cdiv(n, CHUNK);
+    L.split = kpp_split(n, d, n_trials, dtype);
+    L.chunk = L.split ? 64 * L.split : CHUNK;
+    L.n_blocks = kmx_cdiv(n, L.chunk);
     L.off_header = 0;
     L.off_cand = 256;
     L.off_pot = 512;
@@ -63,47 +84,6 @@ __device__ __forceinline__ T kpp_sq_acc(T diff, T acc) {
 #pragma clang fp contract(off)
         const T p = diff * diff;
         return acc + p;
-    }
-}
-
-// closest = w * ||x - x_start||^2 into row 0; per-block potential; slot 0 of the outputs.
-template <typename T, bool FUSED>
-__global__ __launch_bounds__(256) void kpp_init_kernel(
-    const T* __restrict__ X_t, const T* __restrict__ sample_weight, int32_t start,
-    T* __restrict__ centers_t, int32_t* __restrict__ center_indices, T* __restrict__ rows,
-    double* __restrict__ block_pot, KppHeader* __restrict__ header, int64_t n, int d, int k) {
-    const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
-    T acc[4] = {T(0), T(0), T(0), T(0)};
-    for (int f = 0; f < d; ++f) {
-        const T* __restrict__ row = X_t + (size_t)f * n;
-        const T sv = row[start];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            if (i0 + r < n) {
-                const T diff = row[i0 + r] - sv;
-                acc[r] = kpp_sq_acc<FUSED>(diff, acc[r]);
-            }
-        }
-    }
-    double pot = 0.0;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        if (i0 + r < n) {
-            const T v = acc[r] * sample_weight[i0 + r];
-            rows[i0 + r] = v;
-            pot += (double)v;
-        }
-    }
-    __shared__ double scratch[4];
-    const double tot = kmx_block_sum<double>(pot, scratch);
-    if (threadIdx.x == 0) block_pot[(size_t)blockIdx.x * TN_MAX] = tot;
-    if (blockIdx.x == 0) {
-        for (int f = threadIdx.x; f < d; f += 256) centers_t[(size_t)f * k] = X_t[(size_t)f * n + start];
-        if (threadIdx.x == 0) {
-            center_indices[0] = start;
-            header->best_row = 0;
-            header->total = 0.0;
-        }
     }
 }
 
@@ -141,18 +121,56 @@ __device__ __forceinline__ void store4(T* __restrict__ row, int64_t i0, int64_t 
     }
 }
 
+// The value lane `src` (a constant) holds, as a wave-uniform scalar.
+template <typename T>
+__device__ __forceinline__ T kpp_readlane(T v, int src) {
+    if constexpr (sizeof(T) == 4) {
+        return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+    } else {
+        const long long b = __double_as_longlong(v);
+        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)b, src);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(b >> 32), src);
+        return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+    }
+}
+
+// The candidates' values of one batch of FB features, fetched with the samples' own loads:
+// lane l of load q asks for feature f0 + l % FB of trial q * (64 / FB) + l / FB (indices
+// clamped to the rows in use), and the feature loop reads each value back from its lane as a
+// scalar.  One scalar load per value, each waited for where it is used, took a round trip
+// per candidate and feature instead.
+template <typename T, int TN, int FB>
+struct KppCandBatch {
+    static constexpr int TPL = 64 / FB;  // trials per load
+    static constexpr int NQ = (TN + TPL - 1) / TPL;
+    T v[NQ];
+    __device__ __forceinline__ void load(const T* __restrict__ cand_rows, int f0, int d, int n_trials, int lane) {
+        const int f = f0 + lane % FB < d ? f0 + lane % FB : d - 1;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int t = q * TPL + lane / FB;
+            v[q] = cand_rows[(size_t)(t < n_trials ? t : n_trials - 1) * d + f];
+        }
+    }
+    __device__ __forceinline__ T get(int t, int j) const { return kpp_readlane<T>(v[t / TPL], (t % TPL) * FB + j); }
+};
+
 // rows[t, i] = min(w_i * ||x_i - x_cand_t||^2, closest_i) and per-block row sums.
-// Candidate rows come from a small (TN, d) buffer through wave-uniform loads (the values sit
-// in SGPRs, no LDS, no barriers in the feature loop); every thread streams 4 consecutive
-// samples of 8 features at a time with 128-bit loads.
-template <typename T, int TN, bool FUSED>
+// Candidate rows come from a small (TN, d) buffer, a batch of features at a time spread over
+// the lanes and read back as scalars (no LDS, no barriers in the feature loop); every thread
+// streams 4 consecutive samples of a batch of features with 128-bit loads.
+// INIT: the first distances instead, closest = w * ||x - x_start||^2 into row 0 with its block
+// sums, and slot 0 of the outputs: one trial whose candidate is sample `start`, no minimum.
+template <typename T, int TN, bool FUSED, bool INIT>
 __global__ __launch_bounds__(256) void kpp_step_kernel(
     const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cand_rows,
-    T* __restrict__ rows, double* __restrict__ block_pot, const KppHeader* __restrict__ header,
-    int64_t n, int d, int n_trials, int vec_ok) {
+    T* __restrict__ rows, double* __restrict__ block_pot, KppHeader* __restrict__ header,
+    int64_t n, int d, int k, int n_trials, int vec_ok, int32_t start, T* __restrict__ centers_t,
+    int32_t* __restrict__ center_indices) {
     __shared__ double wave_pot[4][TN];
     const int64_t i0 = (int64_t)blockIdx.x * CHUNK + threadIdx.x * 4;
-    const int best = header->best_row;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int best = INIT ? 0 : header->best_row;
     // Whether the 128-bit accesses are legal is decided once per workgroup and known at compile
     // time inside the body: with a test per access every load sat in a branch of its own and
     // was waited for before the next one was issued.
@@ -180,27 +198,40 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
             const T* __restrict__ row = X_t + (size_t)f * n;
             load4<T>(row, i0, n, full, xv[j]);
         }
+        KppCandBatch<T, TN, FB> cand;
+        if constexpr (INIT) {
+            const int f = f0 + lane % FB < d ? f0 + lane % FB : d - 1;
+            cand.v[0] = X_t[(size_t)f * n + start];
+        } else {
+            cand.load(cand_rows, f0, d, n_trials, lane);
+        }
         if (f0 + FB >= d) {
             load4<T>(sample_weight, i0, n, full, w);
-            load4<T>(rows + (size_t)best * n, i0, n, full, cl);
+            if constexpr (!INIT) load4<T>(rows + (size_t)best * n, i0, n, full, cl);
         }
+        auto accumulate = [&](auto whole_tag) {
+            constexpr bool whole = decltype(whole_tag)::value;  // all FB features exist
 #pragma unroll
-        for (int t = 0; t < TN; ++t) {
-            if (t < n_trials) {
-                const T* __restrict__ cr = cand_rows + (size_t)t * d + f0;  // wave-uniform
+            for (int t = 0; t < TN; ++t) {
+                if (t < n_trials) {
 #pragma unroll
-                for (int j = 0; j < FB; ++j) {
-                    if (f0 + j < d) {
-                        const T cv = cr[j];
+                    for (int j = 0; j < FB; ++j) {
+                        if (whole || f0 + j < d) {
+                            const T cv = cand.get(t, j);
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const T diff = xv[j][r] - cv;
-                            acc[t][r] = kpp_sq_acc<FUSED>(diff, acc[t][r]);
+                            for (int r = 0; r < 4; ++r) {
+                                const T diff = xv[j][r] - cv;
+                                acc[t][r] = kpp_sq_acc<FUSED>(diff, acc[t][r]);
+                            }
                         }
                     }
                 }
             }
-        }
+        };
+        if (f0 + FB <= d)
+            accumulate(std::true_type{});
+        else
+            accumulate(std::false_type{});
     }
 
     double pot[TN];
@@ -211,14 +242,14 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
             T v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                v[r] = fmin(acc[t][r] * w[r], cl[r]);
+                v[r] = acc[t][r] * w[r];
+                if constexpr (!INIT) v[r] = fmin(v[r], cl[r]);
                 if (i0 + r < n) pot[t] += (double)v[r];
             }
             store4<T>(rows + (size_t)t * n, i0, n, full, v);
         }
     }
     // all row sums of the workgroup with one barrier: waves first, then one thread per trial
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
         if (t < n_trials) {
@@ -236,6 +267,155 @@ __global__ __launch_bounds__(256) void kpp_step_kernel(
         body(std::true_type{});
     else
         body(std::false_type{});
+    if (INIT && blockIdx.x == 0) {
+        for (int f = threadIdx.x; f < d; f += 256) centers_t[(size_t)f * k] = X_t[(size_t)f * n + start];
+        if (threadIdx.x == 0) {
+            center_indices[0] = start;
+            header->best_row = 0;
+            header->total = 0.0;
+        }
+    }
+}
+
+// SPT consecutive values of a row at i0: one access of SPT elements when `full`, else element
+// by element from indices clamped to the array (the caller ignores what lies past n).
+template <typename T, int SPT>
+__device__ __forceinline__ void load_spt(const T* __restrict__ row, int64_t i0, int64_t n, bool full, T (&v)[SPT]) {
+    if (full) {
+        if constexpr (SPT == 1) {
+            v[0] = row[i0];
+        } else if constexpr (SPT == 2) {
+            using V2 = std::conditional_t<sizeof(T) == 4, float2, double2>;
+            const V2 q = *reinterpret_cast<const V2*>(row + i0);
+            v[0] = q.x; v[1] = q.y;
+        } else {
+            load4<T>(row, i0, n, true, v);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < SPT; ++r) v[r] = row[i0 + r < n ? i0 + r : n - 1];
+    }
+}
+
+// The step (or, INIT, the first distances to the starting sample) for few samples of many
+// features.  A workgroup owns 64 * SPT samples; its four waves take the feature batches in
+// turn, every lane streaming SPT consecutive samples, and leave partial squared distances in
+// LDS.  After one barrier wave w finishes trials w, w + 4: the four partial sums added in wave
+// order, weight, minimum with the closest distance so far, the row store and the block sum.
+// The closest distances are read before the barrier: the finishing waves overwrite the row
+// they came from.  LITERAL keeps the reference's roundings (features summed in order, product
+// and sum rounded separately): every wave walks all the features and the first one's sums are
+// used, so that the block sums have one geometry for both samplers.
+template <typename T, int TN, int SPT, bool INIT, bool LITERAL>
+__global__ __launch_bounds__(256) void kpp_step_split_kernel(
+    const T* __restrict__ X_t, const T* __restrict__ sample_weight, const T* __restrict__ cand_rows,
+    T* __restrict__ rows, double* __restrict__ block_pot, KppHeader* __restrict__ header, int64_t n,
+    int d, int k, int n_trials, int vec_ok, int32_t start, T* __restrict__ centers_t,
+    int32_t* __restrict__ center_indices) {
+    constexpr int S = 64 * SPT;
+    __shared__ T part[4][TN][S];
+    // the wave index as a scalar: the feature loop's bounds and the candidates' rows are then
+    // wave-uniform for the compiler as well (scalar loads, no branch per feature)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t base = (int64_t)blockIdx.x * S;
+    const int64_t i0 = base + lane * SPT;
+    const int best = INIT ? 0 : header->best_row;
+
+    // what the finish needs of samples base + r * 64 + lane, requested ahead of the feature loop
+    T w_fin[SPT], cl_fin[SPT];
+#pragma unroll
+    for (int r = 0; r < SPT; ++r) {
+        const int64_t i = base + r * 64 + lane;
+        const int64_t ic = i < n ? i : n - 1;
+        w_fin[r] = sample_weight[ic];
+        cl_fin[r] = INIT ? T(0) : rows[(size_t)best * n + ic];
+    }
+
+    auto body = [&](auto full_tag) {
+        constexpr bool full = decltype(full_tag)::value;
+        T acc[TN][SPT];
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int r = 0; r < SPT; ++r) acc[t][r] = T(0);
+        constexpr int FB = sizeof(T) == 4 ? 16 : 8;
+        for (int f0 = LITERAL ? 0 : wave * FB; f0 < d; f0 += LITERAL ? FB : 4 * FB) {
+            T xv[FB][SPT];
+#pragma unroll
+            for (int j = 0; j < FB; ++j) {
+                const int f = f0 + j < d ? f0 + j : d - 1;  // past the end: a valid row, ignored below
+                load_spt<T, SPT>(X_t + (size_t)f * n, i0, n, full, xv[j]);
+            }
+            // the candidates' rows, or the starting sample's features
+            KppCandBatch<T, TN, FB> cand;
+            if constexpr (INIT) {
+                const int f = f0 + lane % FB < d ? f0 + lane % FB : d - 1;
+                cand.v[0] = X_t[(size_t)f * n + start];
+            } else {
+                cand.load(cand_rows, f0, d, n_trials, lane);
+            }
+            auto accumulate = [&](auto whole_tag) {
+                constexpr bool whole = decltype(whole_tag)::value;  // all FB features exist
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    if (t < n_trials) {
+#pragma unroll
+                        for (int j = 0; j < FB; ++j) {
+                            if (whole || f0 + j < d) {
+                                const T cv = cand.get(t, j);
+#pragma unroll
+                                for (int r = 0; r < SPT; ++r) {
+                                    const T diff = xv[j][r] - cv;
+                                    acc[t][r] = kpp_sq_acc<!LITERAL>(diff, acc[t][r]);
+                                }
+                            }
+                        }
+                    }
+                }
+            };
+            if (f0 + FB <= d)
+                accumulate(std::true_type{});
+            else
+                accumulate(std::false_type{});
+        }
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+            if (t < n_trials)
+#pragma unroll
+                for (int r = 0; r < SPT; ++r) part[wave][t][lane * SPT + r] = acc[t][r];
+    };
+    if (vec_ok && base + S <= n)
+        body(std::true_type{});
+    else
+        body(std::false_type{});
+    __syncthreads();
+
+    for (int t = wave; t < n_trials; t += 4) {
+        double pot = 0.0;
+#pragma unroll
+        for (int r = 0; r < SPT; ++r) {
+            const int sl = r * 64 + lane;
+            const int64_t i = base + sl;
+            if (i < n) {
+                const T dist = LITERAL ? part[0][t][sl]
+                                       : ((part[0][t][sl] + part[1][t][sl]) + part[2][t][sl]) + part[3][t][sl];
+                T v = dist * w_fin[r];
+                if (!INIT) v = fmin(v, cl_fin[r]);
+                rows[(size_t)t * n + i] = v;
+                pot += (double)v;
+            }
+        }
+        const double ws = kmx_wave_sum<double>(pot);
+        if (lane == 0) block_pot[(size_t)blockIdx.x * TN_MAX + t] = ws;
+    }
+    if (INIT && blockIdx.x == 0) {
+        for (int f = threadIdx.x; f < d; f += 256) centers_t[(size_t)f * k] = X_t[(size_t)f * n + start];
+        if (threadIdx.x == 0) {
+            center_indices[0] = start;
+            header->best_row = 0;
+            header->total = 0.0;
+        }
+    }
 }
 
 // Block-wide exclusive scan of one double per thread (256 threads); returns the exclusive
@@ -288,8 +468,8 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     int32_t* __restrict__ cand_out, T* __restrict__ centers_t,
     int32_t* __restrict__ center_indices, const T* __restrict__ rows,
     const double* __restrict__ block_pot, double* __restrict__ potentials,
-    KppHeader* __restrict__ header, T* __restrict__ cand_rows, int64_t n, int64_t n_blocks, int d,
-    int k, int n_trials, int center_slot, int do_select, int do_sample) {
+    KppHeader* __restrict__ header, T* __restrict__ cand_rows, int64_t n, int64_t n_blocks, int chunk,
+    int d, int k, int n_trials, int center_slot, int do_select, int do_sample) {
     __shared__ double wave_tot[4];
     __shared__ double wave_pot[4][TN];
     __shared__ int64_t iscratch[4];
@@ -426,13 +606,14 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     __syncthreads();
     const double prefix = prefix_s;
 
-    // ---- fine level: scan the 1024 samples of block bstar
+    // ---- fine level: scan the samples of block bstar (chunk: a multiple of 4, at most 1024)
     const T* __restrict__ closest = rows + (size_t)best * n;
-    const int64_t j0 = bstar * CHUNK + threadIdx.x * 4;
+    const int64_t j0 = bstar * chunk + threadIdx.x * 4;
+    const bool in_block = (int)threadIdx.x * 4 < chunk;
     double v[4], s = 0.0;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        v[r] = (j0 + r < n) ? (double)closest[j0 + r] : 0.0;
+        v[r] = (in_block && j0 + r < n) ? (double)closest[j0 + r] : 0.0;
         s += v[r];
     }
     double tot2;
@@ -441,11 +622,11 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         c2 += v[r];
-        if (hit == INT64_MAX && j0 + r < n && c2 >= rv) hit = j0 + r;
+        if (hit == INT64_MAX && in_block && j0 + r < n && c2 >= rv) hit = j0 + r;
     }
     int64_t cand = block_min_i64(hit, iscratch);
     if (cand == INT64_MAX) {
-        cand = (bstar + 1) * CHUNK;  // rounding pushed the crossing just past this block
+        cand = (bstar + 1) * chunk;  // rounding pushed the crossing just past this block
     }
     if (cand > n - 1) cand = n - 1;
     if (threadIdx.x == 0) {
@@ -511,7 +692,7 @@ __global__ __launch_bounds__(256) void kpp_sample_literal_kernel(
         rv_sorted[n_trials] = T(0);
         done_s = 0;
     }
-    const int64_t n_chunks = n_blocks;
+    const int64_t n_chunks = (n + CHUNK - 1) / CHUNK;  // the walk's own chunks, not the block sums
     // first chunk
     {
         const int64_t j0 = (int64_t)threadIdx.x * 4;
@@ -620,26 +801,57 @@ int32_t kpp_check(const void* X_t, const void* w, void* ws, size_t ws_bytes, int
 template <typename T>
 void launch_init(const void* X_t, const void* w, int32_t start, void* centers_t, int32_t* idx,
                  const KppPtrs& p, const KppLayout& L, int64_t n, int d, int k, hipStream_t s, bool literal) {
-    if (literal)
-        hipLaunchKernelGGL((kpp_init_kernel<T, false>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
-                           (const T*)X_t, (const T*)w, start, (T*)centers_t, idx, (T*)p.rows,
-                           p.block_pot, p.header, n, d, k);
-    else
-        hipLaunchKernelGGL((kpp_init_kernel<T, true>), dim3((unsigned)L.n_blocks), dim3(256), 0, s,
-                           (const T*)X_t, (const T*)w, start, (T*)centers_t, idx, (T*)p.rows,
-                           p.block_pot, p.header, n, d, k);
+    if (L.split) {
+        const int vec_ok = (n % L.split == 0) && (((uintptr_t)X_t) % 16 == 0);
+#define KMX_KPP_INIT_SPLIT_(SPT, LIT)                                                                 \
+    hipLaunchKernelGGL((kpp_step_split_kernel<T, 1, SPT, true, LIT>), dim3((unsigned)L.n_blocks),    \
+                       dim3(256), 0, s, (const T*)X_t, (const T*)w, (const T*)nullptr, (T*)p.rows,    \
+                       p.block_pot, p.header, n, d, k, 1, vec_ok, start, (T*)centers_t, idx)
+#define KMX_KPP_INIT_SPLIT(SPT) \
+    do { if (literal) KMX_KPP_INIT_SPLIT_(SPT, true); else KMX_KPP_INIT_SPLIT_(SPT, false); } while (0)
+        if (L.split == 1) KMX_KPP_INIT_SPLIT(1);
+        else if (L.split == 2) KMX_KPP_INIT_SPLIT(2);
+        else KMX_KPP_INIT_SPLIT(4);
+#undef KMX_KPP_INIT_SPLIT_
+#undef KMX_KPP_INIT_SPLIT
+        return;
+    }
+    const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0) && (((uintptr_t)w) % 16 == 0) &&
+                       (((uintptr_t)p.rows) % 16 == 0);
+#define KMX_KPP_INIT(FUSED)                                                                          \
+    hipLaunchKernelGGL((kpp_step_kernel<T, 1, FUSED, true>), dim3((unsigned)L.n_blocks), dim3(256), 0, s, \
+                       (const T*)X_t, (const T*)w, (const T*)nullptr, (T*)p.rows, p.block_pot, p.header, \
+                       n, d, k, 1, vec_ok, start, (T*)centers_t, idx)
+    if (literal) KMX_KPP_INIT(false); else KMX_KPP_INIT(true);
+#undef KMX_KPP_INIT
 }
 
 template <typename T>
 void launch_step(const void* X_t, const void* w, const int32_t* cand, const KppPtrs& p,
                  const KppLayout& L, int64_t n, int d, int n_trials, hipStream_t s, bool literal) {
     (void)cand;  // the candidates' rows were copied to p.cand_rows when they were sampled
+    if (L.split) {
+        const int vec_split = (n % L.split == 0) && (((uintptr_t)X_t) % 16 == 0);
+#define KMX_KPP_STEP_SPLIT_(SPT, LIT)                                                                  \
+    hipLaunchKernelGGL((kpp_step_split_kernel<T, 8, SPT, false, LIT>), dim3((unsigned)L.n_blocks),     \
+                       dim3(256), 0, s, (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, \
+                       p.block_pot, p.header, n, d, 0, n_trials, vec_split, 0, (T*)nullptr,            \
+                       (int32_t*)nullptr)
+#define KMX_KPP_STEP_SPLIT(SPT) \
+    do { if (literal) KMX_KPP_STEP_SPLIT_(SPT, true); else KMX_KPP_STEP_SPLIT_(SPT, false); } while (0)
+        if (L.split == 1) KMX_KPP_STEP_SPLIT(1);
+        else if (L.split == 2) KMX_KPP_STEP_SPLIT(2);
+        else KMX_KPP_STEP_SPLIT(4);
+#undef KMX_KPP_STEP_SPLIT
+#undef KMX_KPP_STEP_SPLIT_
+        return;
+    }
     const int vec_ok = (n % 4 == 0) && (((uintptr_t)X_t) % 16 == 0) && (((uintptr_t)w) % 16 == 0) &&
                        (((uintptr_t)p.rows) % 16 == 0);
 #define KMX_KPP_STEP(TN, FUSED)                                                                      \
-    hipLaunchKernelGGL((kpp_step_kernel<T, TN, FUSED>), dim3((unsigned)L.n_blocks), dim3(256), 0, s, \
+    hipLaunchKernelGGL((kpp_step_kernel<T, TN, FUSED, false>), dim3((unsigned)L.n_blocks), dim3(256), 0, s, \
                        (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, p.block_pot,   \
-                       p.header, n, d, n_trials, vec_ok)
+                       p.header, n, d, 0, n_trials, vec_ok, 0, (T*)nullptr, (int32_t*)nullptr)
     if (n_trials <= 8) {
         if (literal) KMX_KPP_STEP(8, false); else KMX_KPP_STEP(8, true);
     } else {
@@ -672,7 +884,7 @@ void launch_select_sample(const void* X_t, const double* uniforms, const int32_t
     hipLaunchKernelGGL((kpp_select_sample_kernel<T, TN>), dim3(grid), dim3(256), 0, s,             \
                        (const T*)X_t, uniforms, cand_prev, cand_next, cand_out, (T*)centers_t, idx, \
                        (const T*)p.rows, p.block_pot, p.potentials, p.header, (T*)p.cand_rows, n,   \
-                       L.n_blocks, d, k, n_trials, slot, do_select, do_sample)
+                       L.n_blocks, L.chunk, d, k, n_trials, slot, do_select, do_sample)
     if (n_trials <= 8)
         KMX_KPP_SELECT(8);
     else

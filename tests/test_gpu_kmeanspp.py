@@ -32,11 +32,20 @@ def _cases():
         "many_trials_f32": (rng.normal(size=(6001, 7)).astype(np.float32), None, 3000, 4),
         # more than 4 x 256 blocks of 1024 samples: the sampler re-reads its block sums
         "many_blocks_f64": (rng.normal(size=(1_100_003, 2)), None, 6, 5),
+        # few samples of many features: the step with the features split over a workgroup's
+        # waves, at 1, 2 and 4 samples per thread, with and without a ragged last block
+        "short_wide_f32": (rng.normal(size=(70_001, 96)).astype(np.float32), None, 6, 7),
+        "short_wide_f64": (rng.normal(size=(100_000, 70)), rng.uniform(0.1, 3.0, 100_000), 5, 8),
+        "short_wide_4_f32": (rng.normal(size=(200_000, 64)).astype(np.float32), None, 7, 9),
+        "short_wide_4_ragged_f32": (rng.normal(size=(140_003, 65)).astype(np.float32), rng.uniform(0.1, 3.0, 140_003), 4, 10),
+        "short_wide_1_f64": (rng.normal(size=(2_049, 333)), None, 12, 12),
     }
 
 
 @pytest.mark.parametrize("sampler", ["scan", "literal"])
-@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32", "many_trials_f32", "many_blocks_f64", "weighted_f32"])
+@pytest.mark.parametrize("name", ["C4", "weighted_f64", "tiny_f32", "wide_f32", "many_trials_f32", "many_blocks_f64", "weighted_f32",
+                                  "short_wide_f32", "short_wide_f64", "short_wide_4_f32", "short_wide_4_ragged_f32",
+                                  "short_wide_1_f64"])
 def test_whole_seeding_matches_oracle(cuda, name, sampler):
     """Both samplers of the library against their counterparts in the oracle: the fp64 scan
     (default) and the reference's running sum in the compute dtype (`KMX_KPP_SAMPLER_LITERAL`)."""
