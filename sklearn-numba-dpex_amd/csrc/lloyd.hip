@@ -444,13 +444,17 @@ __global__ __launch_bounds__(256) void lloyd_reduce_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Finalisation: one thread per cluster, features in order (division, packed copy, half
-// squared norm, squared shift); the last block sums the per-block shifts in block order and
-// runs the convergence test.
+// Finalisation: LANES threads per cluster (256 / LANES clusters per workgroup), lane g on the
+// features g, g + LANES, ... (division, packed copy, half squared norm, squared shift); the lanes
+// meet in LDS in lane order.  8 lanes, or 64 for a few clusters of wide samples, where a
+// workgroup or two of eight-lane clusters would each walk a hundred features, a trip to memory
+// per value.  The last block sums the per-block shifts in block order and runs the convergence
+// test.
 // ------------------------------------------------------------------------------------------
-constexpr int FIN_CLUSTERS = 32;  // clusters per workgroup of the finalisation kernel
+constexpr int fin_lanes(int d, int k) { return (d >= 256 && k <= 128) ? 64 : 8; }
+constexpr int fin_grid(int d, int k) { return (k + 256 / fin_lanes(d, k) - 1) / (256 / fin_lanes(d, k)); }
 
-template <typename T>
+template <typename T, int LANES>
 __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
     const T* __restrict__ old_centroids_t, T* __restrict__ new_centroids_t,
     const T* __restrict__ sizes, T* __restrict__ cpack, T* __restrict__ half_norms,
@@ -459,16 +463,15 @@ __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
     const int state = status->state;
     if (force ? (state != KMX_NEED_RELOCATION && state != KMX_RUNNING) : (state != KMX_RUNNING))
         return;
-    // 32 clusters per workgroup; the 8 thread groups of a cluster take every 8th feature and
-    // meet in LDS (fixed order), so that wide samples do not serialise on one thread
-    const int cl = threadIdx.x & 31, grp = threadIdx.x >> 5;
-    const int c = blockIdx.x * FIN_CLUSTERS + cl;
-    __shared__ T sq_s[8][FIN_CLUSTERS], sh_s[8][FIN_CLUSTERS];
+    constexpr int CPW = 256 / LANES;  // clusters per workgroup
+    const int cl = threadIdx.x & (CPW - 1), grp = threadIdx.x / CPW;
+    const int c = blockIdx.x * CPW + cl;
+    __shared__ T sq_s[LANES][CPW], sh_s[LANES][CPW];
     T sq = T(0), sh = T(0);
     const T sz = c < k ? sizes[c] : T(0);
     if (sz != T(0)) {
 #pragma unroll 4
-        for (int f = grp; f < d; f += 8) {
+        for (int f = grp; f < d; f += LANES) {
             const T nv = new_centroids_t[(size_t)f * k + c] / sz;
             const T df = old_centroids_t[(size_t)f * k + c] - nv;
             sh += df * df;
@@ -476,7 +479,7 @@ __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
             cpack[(size_t)c * dpad + f] = nv;
             new_centroids_t[(size_t)f * k + c] = nv;
         }
-        for (int f = d + grp; f < dpad; f += 8) cpack[(size_t)c * dpad + f] = T(0);
+        for (int f = d + grp; f < dpad; f += LANES) cpack[(size_t)c * dpad + f] = T(0);
     }
     sq_s[grp][cl] = sq;
     sh_s[grp][cl] = sh;
@@ -485,7 +488,7 @@ __global__ __launch_bounds__(256) void lloyd_finalize_kernel(
     if (grp == 0 && sz != T(0)) {
         T sq_t = sq_s[0][cl], sh_t = sh_s[0][cl];
 #pragma unroll
-        for (int g2 = 1; g2 < 8; ++g2) {
+        for (int g2 = 1; g2 < LANES; ++g2) {
             sq_t += sq_s[g2][cl];
             sh_t += sh_s[g2][cl];
         }
@@ -841,9 +844,14 @@ int32_t lloyd_iter_impl(const LloydLayout& L, const void* X_t, const void* X_row
         hipLaunchKernelGGL((lloyd_small_finalize_kernel<T, false>), dim3(1), dim3(256),
                            (size_t)items * sizeof(T), stream, nullptr, nullptr, tail);
     } else {
-        hipLaunchKernelGGL((lloyd_finalize_kernel<T>), dim3((unsigned)kmx_cdiv(k, FIN_CLUSTERS)), dim3(256), 0,
-                           stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
-                           half_norms, shift_partial, status, d, k, L.dpad, 0);
+        if (fin_lanes(d, k) == 64)
+            hipLaunchKernelGGL((lloyd_finalize_kernel<T, 64>), dim3((unsigned)fin_grid(d, k)), dim3(256), 0,
+                               stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
+                               half_norms, shift_partial, status, d, k, L.dpad, 0);
+        else
+            hipLaunchKernelGGL((lloyd_finalize_kernel<T, 8>), dim3((unsigned)fin_grid(d, k)), dim3(256), 0,
+                               stream, (const T*)centroids_t, (T*)new_centroids_t, (const T*)sizes, cpack,
+                               half_norms, shift_partial, status, d, k, L.dpad, 0);
     }
     KMX_LAUNCH_CHECK();
     if (events) (void)hipEventRecord(events[3], stream);
@@ -1178,17 +1186,18 @@ int32_t kmx_lloyd_finalize(const kmx_lloyd_plan* plan, const void* centroids_t,
     char* ws = (char*)workspace;
     auto* status = reinterpret_cast<kmx_lloyd_status*>(ws + L.off_status);
     double* shift_partial = reinterpret_cast<double*>(ws + L.off_shift);
-    const unsigned grid = (unsigned)kmx_cdiv(k, FIN_CLUSTERS);
-    if (dtype == KMX_F32)
-        hipLaunchKernelGGL((lloyd_finalize_kernel<float>), dim3(grid), dim3(256), 0, stream,
-                           (const float*)centroids_t, (float*)new_centroids_t,
-                           (const float*)cluster_sizes, (float*)(ws + L.off_cpack),
-                           (float*)(ws + L.off_half), shift_partial, status, d, k, L.dpad, 1);
-    else
-        hipLaunchKernelGGL((lloyd_finalize_kernel<double>), dim3(grid), dim3(256), 0, stream,
-                           (const double*)centroids_t, (double*)new_centroids_t,
-                           (const double*)cluster_sizes, (double*)(ws + L.off_cpack),
-                           (double*)(ws + L.off_half), shift_partial, status, d, k, L.dpad, 1);
+    const unsigned grid = (unsigned)fin_grid(d, k);
+#define KMX_FINALIZE(T, LANES)                                                                        \
+    hipLaunchKernelGGL((lloyd_finalize_kernel<T, LANES>), dim3(grid), dim3(256), 0, stream,           \
+                       (const T*)centroids_t, (T*)new_centroids_t, (const T*)cluster_sizes,           \
+                       (T*)(ws + L.off_cpack), (T*)(ws + L.off_half), shift_partial, status, d, k,    \
+                       L.dpad, 1)
+    if (dtype == KMX_F32) {
+        if (fin_lanes(d, k) == 64) KMX_FINALIZE(float, 64); else KMX_FINALIZE(float, 8);
+    } else {
+        if (fin_lanes(d, k) == 64) KMX_FINALIZE(double, 64); else KMX_FINALIZE(double, 8);
+    }
+#undef KMX_FINALIZE
     KMX_LAUNCH_CHECK();
     return KMX_OK;
 }

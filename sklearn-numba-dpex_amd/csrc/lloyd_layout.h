@@ -238,7 +238,7 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
     L.off_cpack = L.off_gsum + kmx_align256(items * sizeof(long long));
     L.off_half = L.off_cpack + kmx_align256((size_t)k * L.dpad * s);
     L.off_shift = L.off_half + kmx_align256((size_t)k * s);
-    L.off_bucket = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 32) * sizeof(double));  // one per finalisation workgroup
+    L.off_bucket = L.off_shift + kmx_align256((size_t)kmx_cdiv(k, 4) * sizeof(double));  // one per finalisation workgroup (4 to 32 clusters each)
     // wide matrix-core path: counts (k), offsets (k + 1), sample order (n) and ranks inside the
     // cluster (n) as int32
     // screened path: the counter of samples evaluated in fp32 and its copy for the host (256
