@@ -240,8 +240,11 @@ class KMeansEngine(_EngineBase):
         """scikit-learn's check of the input (check_array(ensure_all_finite=True), as the
         reference's engine runs it: kmeans/engine.py:293-302), taken on the device: one pass at
         memory speed instead of a single-threaded host pass that costs more than the upload.
-        Non-finite data then get scikit-learn's own error from the host copy."""
-        if bool(torch.isfinite(X_t).all()):
+        Non-finite data then get scikit-learn's own error from the host copy.  As in
+        scikit-learn, the sum goes first (one read, nothing written): a NaN or an infinity
+        anywhere makes it non-finite, and so may an overflow of finite values, which the
+        element-wise test then clears."""
+        if bool(torch.isfinite(X_t.sum())) or bool(torch.isfinite(X_t).all()):
             return
         from sklearn.utils.validation import _assert_all_finite
 

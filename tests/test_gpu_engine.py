@@ -466,3 +466,20 @@ def test_non_finite_input_is_refused_like_scikit_learn(cuda, kind, bad):
         with pytest.raises(ValueError) as err:
             call()
         assert str(err.value) == expected
+
+
+def test_finite_input_whose_sum_overflows_is_accepted(cuda):
+    """The check sums the array first; finite values whose sum overflows must still pass."""
+    from sklearn_numba_dpex_amd.kmeans.estimator import KMeans
+
+    X, _ = make_blobs(n_samples=300, random_state=1)
+    X = X.astype(np.float32)
+    km = KMeans(n_clusters=3, n_init=1, random_state=0).fit(X)
+    X_big = X.copy()
+    X_big[5, 0] = X_big[9, 0] = 3e38
+    with np.errstate(over="ignore"):
+        assert not np.isfinite(X_big.sum(dtype=np.float32))
+    keep = np.ones(300, dtype=bool)
+    keep[[5, 9]] = False
+    for arg in (X_big, _as_cuda(X_big, np.float32)):
+        assert_array_equal(_np(km.predict(arg))[keep], _np(km.predict(X))[keep])
