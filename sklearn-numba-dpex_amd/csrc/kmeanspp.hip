@@ -897,7 +897,6 @@ void launch_select_sample(const void* X_t, const double* uniforms, const int32_t
 extern "C" {
 
 size_t kmx_kpp_workspace_bytes(int64_t n, int32_t d, int32_t k, int32_t n_trials, int32_t dtype) {
-    (void)d;
     (void)k;
     if (n <= 0 || n_trials <= 0 || n_trials > TN_MAX || (dtype != KMX_F32 && dtype != KMX_F64))
         return 0;
@@ -1024,7 +1023,6 @@ int32_t kmx_kpp_run(const void* X_t, const void* sample_weight, const double* un
 
 void* kmx_kpp_closest_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
                           int32_t dtype) {
-    (void)d;
     (void)k;
     if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
     // start of the rows; the caller adds best_row * n elements (best_row from the header)
@@ -1033,7 +1031,6 @@ void* kmx_kpp_closest_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int3
 
 double* kmx_kpp_potentials_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
                                int32_t dtype) {
-    (void)d;
     (void)k;
     if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
     return (double*)((char*)workspace + kpp_layout(n, d, n_trials, dtype).off_pot);
@@ -1041,7 +1038,6 @@ double* kmx_kpp_potentials_ptr(void* workspace, int64_t n, int32_t d, int32_t k,
 
 int32_t* kmx_kpp_candidates_ptr(void* workspace, int64_t n, int32_t d, int32_t k, int32_t n_trials,
                                 int32_t dtype) {
-    (void)d;
     (void)k;
     if (!workspace || n <= 0 || n_trials <= 0) return nullptr;
     return (int32_t*)((char*)workspace + kpp_layout(n, d, n_trials, dtype).off_cand);

@@ -36,16 +36,19 @@ constexpr int GK64 = 8;       // features per stage, fp64
 constexpr int GLD32 = GT + 32;  // LDS row length in floats: the two K rows of a wave's read 32 banks apart
 constexpr int GLD64 = GT + 16;  // in doubles: the K rows of a half-wave's read 32 banks apart
 
-// One stage of one operand: rows f0 .. f0 + GK32 - 1 of a feature-major array with `len`
-// columns, columns c0 .. c0 + 127, zero outside the array.  Thread t takes the groups of four
-// columns t and t + 256 (row g / 32, columns 4 (g % 32)).
-__device__ __forceinline__ void stage_load_f32(float4 (&r)[2], const float* __restrict__ base, int64_t len,
+// One stage of one operand: rows f0 .. f0 + 8 L - 1 of a feature-major array with `len`
+// columns, columns c0 .. c0 + 4 GROUPS - 1, zero outside the array.  Thread t takes the groups
+// of four columns t, t + 256, ... (row g / GROUPS, columns 4 (g % GROUPS)); GROUPS = 32 (128
+// columns: the samples, or a tile of 128 centroids) makes a load cover 8 rows, a tile of 32 or
+// 64 centroids 32 or 16.
+template <int L, int GROUPS = 32>
+__device__ __forceinline__ void stage_load_f32(float4 (&r)[L], const float* __restrict__ base, int64_t len,
                                                int64_t c0, int d, int f0, bool vec_ok) {
 #pragma unroll
-    for (int l = 0; l < 2; ++l) {
+    for (int l = 0; l < L; ++l) {
         const int g = threadIdx.x + 256 * l;
-        const int f = f0 + (g >> 5);
-        const int64_t c = c0 + 4 * (g & 31);
+        const int f = f0 + g / GROUPS;
+        const int64_t c = c0 + 4 * (g % GROUPS);
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (f < d) {
             const float* __restrict__ src = base + (size_t)f * (size_t)len + c;
@@ -62,20 +65,23 @@ __device__ __forceinline__ void stage_load_f32(float4 (&r)[2], const float* __re
     }
 }
 
-__device__ __forceinline__ void stage_store_f32(float (*tile)[GLD32], const float4 (&r)[2]) {
+template <int L, int LD, int GROUPS = 32>
+__device__ __forceinline__ void stage_store_f32(float (*tile)[LD], const float4 (&r)[L]) {
 #pragma unroll
-    for (int l = 0; l < 2; ++l) {
+    for (int l = 0; l < L; ++l) {
         const int g = threadIdx.x + 256 * l;
-        *reinterpret_cast<float4*>(&tile[g >> 5][4 * (g & 31)]) = r[l];
+        *reinterpret_cast<float4*>(&tile[g / GROUPS][4 * (g % GROUPS)]) = r[l];
     }
 }
 
 // The same stage for LISTED samples: column c of the tile is sample cols[.] of X_t (gathered,
-// one load per value); a negative index is a column past the end of the list.
-__device__ __forceinline__ void stage_load_listed_f32(float4 (&r)[2], const float* __restrict__ X_t, int64_t n,
-                                                      const int (&cols)[2][4], int d, int f0) {
+// one load per value); a negative index is a column past the end of the list.  (A thread's
+// groups of columns are the same in all its rows.)
+template <int L>
+__device__ __forceinline__ void stage_load_listed_f32(float4 (&r)[L], const float* __restrict__ X_t, int64_t n,
+                                                      const int (&cols)[4], int d, int f0) {
 #pragma unroll
-    for (int l = 0; l < 2; ++l) {
+    for (int l = 0; l < L; ++l) {
         const int g = threadIdx.x + 256 * l;
         const int f = f0 + (g >> 5);
         const bool row_ok = f < d;
@@ -83,8 +89,8 @@ __device__ __forceinline__ void stage_load_listed_f32(float4 (&r)[2], const floa
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const bool ok = row_ok && cols[l][e] >= 0;
-            const float x = row[ok ? cols[l][e] : 0];
+            const bool ok = row_ok && cols[e] >= 0;
+            const float x = row[ok ? cols[e] : 0];
             v[e] = ok ? x : 0.0f;
         }
         r[l] = make_float4(v[0], v[1], v[2], v[3]);
@@ -92,8 +98,10 @@ __device__ __forceinline__ void stage_load_listed_f32(float4 (&r)[2], const floa
 }
 
 // NA: 32-centroid row tiles per pass over the features (4: tiles of 128 centroids; 1 or 2 for
-// up to 32 / 64 clusters, where wider tiles would multiply padding).  A stage always copies 128
-// centroid columns; only the first 32 NA are used.
+// up to 32 / 64 clusters, where wider tiles would multiply padding).  A stage copies the 32 NA
+// centroid columns in use.  With one row tile a stage is 32 features instead of 16: the small
+// centroid tile leaves the LDS for it, and a workgroup has twice the bytes on their way from
+// memory (with few clusters the kernel does little arithmetic per byte and waits for X).
 // LISTED: the samples are list[0 .. *list_count) instead of 0 .. n (what a screened label
 // kernel could not certify); a workgroup without a tile of the list leaves at once.
 template <int NA, bool LISTED = false>
@@ -104,41 +112,48 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
     const int* __restrict__ list = nullptr, const unsigned int* __restrict__ list_count = nullptr) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
     const int64_t n_work = LISTED ? (int64_t)*list_count : n;
-    __shared__ __align__(16) float xs[2][GK32][GLD32];
-    __shared__ __align__(16) float cs[2][GK32][GLD32];
+    constexpr int GK = NA == 1 ? 2 * GK32 : GK32;           // features per stage
+    constexpr int XL = GK / 8;                              // 128-bit loads per thread and stage, samples
+    constexpr int CG = 8 * NA;                              // groups of four columns per centroid row
+    constexpr int CL = GK * CG / 256;                       // loads per thread and stage, centroids
+    constexpr int CLD = 32 * NA + (NA % 2 == 0 ? 32 : 0);   // row length: = 32 mod 64, as GLD32
+    static_assert(GK * CG % 256 == 0 && CLD % 64 == 32, "whole loads per thread; K rows 32 banks apart");
+    __shared__ __align__(16) float xs[2][GK][GLD32];
+    __shared__ __align__(16) float cs[2][GK][CLD];
     __shared__ float hn[GT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, j = lane & 31;
-    const int n_stages = (d + GK32 - 1) / GK32;
+    const int n_stages = (d + GK - 1) / GK;
     const int64_t n_tiles = (n_work + GT - 1) / GT;
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t i0 = tile * GT;
         float best = -kmx_inf<float>();
         int bidx = 0;
-        int cols[2][4];  // LISTED: the samples behind the thread's columns of a stage
+        int cols[4];  // LISTED: the samples behind the thread's columns of a stage
         if constexpr (LISTED) {
 #pragma unroll
-            for (int l = 0; l < 2; ++l)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int64_t slot = i0 + 4 * ((threadIdx.x + 256 * l) & 31) + e;
-                    cols[l][e] = slot < n_work ? list[slot] : -1;
-                }
+            for (int e = 0; e < 4; ++e) {
+                const int64_t slot = i0 + 4 * (threadIdx.x & 31) + e;
+                cols[e] = slot < n_work ? list[slot] : -1;
+            }
         }
-        auto load_x = [&](float4(&r)[2], const int f0) {
-            if constexpr (LISTED) stage_load_listed_f32(r, X_t, n, cols, d, f0);
-            else stage_load_f32(r, X_t, n, i0, d, f0, x_vec != 0);
+        auto load_x = [&](float4(&r)[XL], const int f0) {
+            if constexpr (LISTED) stage_load_listed_f32<XL>(r, X_t, n, cols, d, f0);
+            else stage_load_f32<XL>(r, X_t, n, i0, d, f0, x_vec != 0);
+        };
+        auto load_c = [&](float4(&r)[CL], const int c0, const int f0) {
+            stage_load_f32<CL, CG>(r, centroids_t, k, c0, d, f0, c_vec != 0);
         };
         for (int c0 = 0; c0 < k; c0 += 32 * NA) {
             __syncthreads();  // the previous tile's reads of hn and of the stage buffers are over
             if (threadIdx.x < GT)
                 hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<float>();
-            float4 rx[2], rc[2];
+            float4 rx[XL], rc[CL];
             load_x(rx, 0);
-            stage_load_f32(rc, centroids_t, k, c0, d, 0, c_vec != 0);
-            stage_store_f32(xs[0], rx);
-            stage_store_f32(cs[0], rc);
+            load_c(rc, c0, 0);
+            stage_store_f32<XL, GLD32>(xs[0], rx);
+            stage_store_f32<CL, CLD, CG>(cs[0], rc);
             __syncthreads();
 
             // accumulator register r of lane (j, h): centroid 32 a + 8 (r / 4) + 4 h + r % 4
@@ -151,11 +166,11 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
             for (int st = 0; st < n_stages; ++st) {
                 const int cur = st & 1;
                 if (st + 1 < n_stages) {
-                    load_x(rx, (st + 1) * GK32);
-                    stage_load_f32(rc, centroids_t, k, c0, d, (st + 1) * GK32, c_vec != 0);
+                    load_x(rx, (st + 1) * GK);
+                    load_c(rc, c0, (st + 1) * GK);
                 }
 #pragma unroll
-                for (int s = 0; s < GK32 / 2; ++s) {
+                for (int s = 0; s < GK / 2; ++s) {
                     // lane (j, h) supplies feature 2 s + h of centroid / sample j of the 32
                     const float bf = xs[cur][2 * s + h][32 * wave + j];
                     float af[NA];
@@ -166,8 +181,8 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
                         acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[a], bf, acc[a], 0, 0, 0);
                 }
                 if (st + 1 < n_stages) {
-                    stage_store_f32(xs[cur ^ 1], rx);
-                    stage_store_f32(cs[cur ^ 1], rc);
+                    stage_store_f32<XL, GLD32>(xs[cur ^ 1], rx);
+                    stage_store_f32<CL, CLD, CG>(cs[cur ^ 1], rc);
                 }
                 __syncthreads();
             }
@@ -340,7 +355,8 @@ int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const vo
     int64_t grid = kmx_cdiv(n, GT);
     // workgroups per compute unit: what registers and LDS allow (one workgroup per tile instead
     // measured 4 % slower)
-    const int64_t cap = (int64_t)(dtype == KMX_F32 ? 3 : 2) * kmx_num_cus();
+    // (four with the 64-centroid tile of fp32, whose stages leave the LDS for them)
+    const int64_t cap = (int64_t)(dtype == KMX_F32 ? (k > 32 && k <= 64 ? 4 : 3) : 2) * kmx_num_cus();
     if (grid > cap) grid = cap;
 #define KMX_GEMM_LAUNCH(KERNEL, T)                                                                    \
     hipLaunchKernelGGL(KERNEL, dim3((unsigned)grid), dim3(256), 0, stream, (const T*)X_t,             \
