@@ -209,14 +209,16 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f32_kernel(
     }
 }
 
-// fp64: thread t takes the pairs of columns t and t + 256 (row g / 64, columns 2 (g % 64)).
-__device__ __forceinline__ void stage_load_f64(double2 (&r)[2], const double* __restrict__ base, int64_t len,
+// fp64: thread t takes the pairs of columns t, t + 256, ... (row g / GROUPS, columns
+// 2 (g % GROUPS)); GROUPS = 64 for 128 columns, 16 or 32 for a tile of 32 or 64 centroids.
+template <int L, int GROUPS = 64>
+__device__ __forceinline__ void stage_load_f64(double2 (&r)[L], const double* __restrict__ base, int64_t len,
                                                int64_t c0, int d, int f0, bool vec_ok) {
 #pragma unroll
-    for (int l = 0; l < 2; ++l) {
+    for (int l = 0; l < L; ++l) {
         const int g = threadIdx.x + 256 * l;
-        const int f = f0 + (g >> 6);
-        const int64_t c = c0 + 2 * (g & 63);
+        const int f = f0 + g / GROUPS;
+        const int64_t c = c0 + 2 * (g % GROUPS);
         double2 v = make_double2(0.0, 0.0);
         if (f < d) {
             const double* __restrict__ src = base + (size_t)f * (size_t)len + c;
@@ -231,27 +233,36 @@ __device__ __forceinline__ void stage_load_f64(double2 (&r)[2], const double* __
     }
 }
 
-__device__ __forceinline__ void stage_store_f64(double (*tile)[GLD64], const double2 (&r)[2]) {
+template <int L, int LD, int GROUPS = 64>
+__device__ __forceinline__ void stage_store_f64(double (*tile)[LD], const double2 (&r)[L]) {
 #pragma unroll
-    for (int l = 0; l < 2; ++l) {
+    for (int l = 0; l < L; ++l) {
         const int g = threadIdx.x + 256 * l;
-        *reinterpret_cast<double2*>(&tile[g >> 6][2 * (g & 63)]) = r[l];
+        *reinterpret_cast<double2*>(&tile[g / GROUPS][2 * (g % GROUPS)]) = r[l];
     }
 }
 
 // NA: 16-centroid row tiles per pass (8: tiles of 128 centroids; 2 or 4 for up to 32 / 64 clusters).
+// A stage copies the 16 NA centroid columns in use; with two row tiles it is 16 features instead
+// of 8 (see the fp32 kernel).
 template <int NA>
 __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
     const double* __restrict__ X_t, const double* __restrict__ centroids_t,
     const double* __restrict__ half_norms, uint32_t* __restrict__ labels,
     const kmx_lloyd_status* __restrict__ status, int64_t n, int d, int k, int x_vec, int c_vec) {
     if (status != nullptr && status->state != KMX_RUNNING) return;
-    __shared__ __align__(16) double xs[2][GK64][GLD64];
-    __shared__ __align__(16) double cs[2][GK64][GLD64];
+    constexpr int GK = NA == 2 ? 2 * GK64 : GK64;  // features per stage
+    constexpr int XL = GK / 4;                     // 128-bit loads per thread and stage, samples
+    constexpr int CG = 8 * NA;                     // pairs of columns per centroid row
+    constexpr int CL = GK * CG / 256;              // loads per thread and stage, centroids
+    constexpr int CLD = 16 * NA + 16;              // row length in doubles: = 16 mod 32, as GLD64
+    static_assert(GK * CG % 256 == 0 && CLD % 32 == 16, "whole loads per thread; K rows 32 banks apart");
+    __shared__ __align__(16) double xs[2][GK][GLD64];
+    __shared__ __align__(16) double cs[2][GK][CLD];
     __shared__ double hn[GT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, j = lane & 15;
-    const int n_stages = (d + GK64 - 1) / GK64;
+    const int n_stages = (d + GK - 1) / GK;
     const int64_t n_tiles = (n + GT - 1) / GT;
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -262,11 +273,11 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
             __syncthreads();
             if (threadIdx.x < GT)
                 hn[threadIdx.x] = c0 + (int)threadIdx.x < k ? -half_norms[c0 + threadIdx.x] : -kmx_inf<double>();
-            double2 rx[2], rc[2];
-            stage_load_f64(rx, X_t, n, i0, d, 0, x_vec != 0);
-            stage_load_f64(rc, centroids_t, k, c0, d, 0, c_vec != 0);
-            stage_store_f64(xs[0], rx);
-            stage_store_f64(cs[0], rc);
+            double2 rx[XL], rc[CL];
+            stage_load_f64<XL>(rx, X_t, n, i0, d, 0, x_vec != 0);
+            stage_load_f64<CL, CG>(rc, centroids_t, k, c0, d, 0, c_vec != 0);
+            stage_store_f64<XL, GLD64>(xs[0], rx);
+            stage_store_f64<CL, CLD, CG>(cs[0], rc);
             __syncthreads();
 
             // accumulator r of lane (g, j), row tile a, column tile b: centroid 16 a + g + 4 r of
@@ -284,11 +295,11 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
             for (int st = 0; st < n_stages; ++st) {
                 const int cur = st & 1;
                 if (st + 1 < n_stages) {
-                    stage_load_f64(rx, X_t, n, i0, d, (st + 1) * GK64, x_vec != 0);
-                    stage_load_f64(rc, centroids_t, k, c0, d, (st + 1) * GK64, c_vec != 0);
+                    stage_load_f64<XL>(rx, X_t, n, i0, d, (st + 1) * GK, x_vec != 0);
+                    stage_load_f64<CL, CG>(rc, centroids_t, k, c0, d, (st + 1) * GK, c_vec != 0);
                 }
 #pragma unroll
-                for (int s = 0; s < GK64 / 4; ++s) {
+                for (int s = 0; s < GK / 4; ++s) {
                     // lane (g, j) supplies feature 4 s + g of centroid / sample j of the 16
                     double bf[2];
 #pragma unroll
@@ -302,8 +313,8 @@ __global__ __launch_bounds__(256, 2) void lloyd_gemm_labels_f64_kernel(
                     }
                 }
                 if (st + 1 < n_stages) {
-                    stage_store_f64(xs[cur ^ 1], rx);
-                    stage_store_f64(cs[cur ^ 1], rc);
+                    stage_store_f64<XL, GLD64>(xs[cur ^ 1], rx);
+                    stage_store_f64<CL, CLD, CG>(cs[cur ^ 1], rc);
                 }
                 __syncthreads();
             }
@@ -355,8 +366,8 @@ int32_t kmx_lloyd_gemm_labels(const void* X_t, const void* centroids_t, const vo
     int64_t grid = kmx_cdiv(n, GT);
     // workgroups per compute unit: what registers and LDS allow (one workgroup per tile instead
     // measured 4 % slower)
-    // (four with the 64-centroid tile of fp32, whose stages leave the LDS for them)
-    const int64_t cap = (int64_t)(dtype == KMX_F32 ? (k > 32 && k <= 64 ? 4 : 3) : 2) * kmx_num_cus();
+    // (one more with the narrow centroid tiles, whose stages leave the LDS for it)
+    const int64_t cap = (int64_t)(dtype == KMX_F32 ? (k > 32 && k <= 64 ? 4 : 3) : (k <= 64 ? 3 : 2)) * kmx_num_cus();
     if (grid > cap) grid = cap;
 #define KMX_GEMM_LAUNCH(KERNEL, T)                                                                    \
     hipLaunchKernelGGL(KERNEL, dim3((unsigned)grid), dim3(256), 0, stream, (const T*)X_t,             \
