@@ -45,13 +45,13 @@ struct KppLayout {
 // With CHUNK samples per workgroup a short, wide array gives the chip a few dozen workgroups
 // that each walk every feature; 64 * split samples per workgroup and a quarter of the features
 // per wave give it thousands of waves.  The block sums stay at most 1 024, which the selection
-// kernel keeps in registers, and the partial distances of 8 trials fit the workgroup's LDS.
+// kernel keeps in registers.
 int kpp_split(int64_t n, int d, int n_trials, int dtype) {
-    if (d < SPLIT_MIN_D || n_trials > 8) return 0;
-    if (n <= 65536) return 1;
-    if (n <= 131072) return 2;
-    if (n <= 262144 && dtype == KMX_F32) return 4;
-    return 0;
+    if (d < SPLIT_MIN_D) return 0;
+    // (the partial distances of a workgroup: 4 waves x trials x samples, at most 32 KB)
+    const int most = (dtype == KMX_F32 ? 4 : 2) / (n_trials > 8 ? 2 : 1);
+    const int spt = n <= 65536 ? 1 : n <= 131072 ? 2 : n <= 262144 ? 4 : 8;
+    return spt <= most ? spt : 0;
 }
 
 // The layout, the block sums included, depends on the shape only: calls with either sampler
@@ -811,7 +811,7 @@ void launch_init(const void* X_t, const void* w, int32_t start, void* centers_t,
     do { if (literal) KMX_KPP_INIT_SPLIT_(SPT, true); else KMX_KPP_INIT_SPLIT_(SPT, false); } while (0)
         if (L.split == 1) KMX_KPP_INIT_SPLIT(1);
         else if (L.split == 2) KMX_KPP_INIT_SPLIT(2);
-        else KMX_KPP_INIT_SPLIT(4);
+        else if constexpr (sizeof(T) == 4) KMX_KPP_INIT_SPLIT(4);  // (kpp_split: fp32 only)
 #undef KMX_KPP_INIT_SPLIT_
 #undef KMX_KPP_INIT_SPLIT
         return;
@@ -832,16 +832,22 @@ void launch_step(const void* X_t, const void* w, const int32_t* cand, const KppP
     (void)cand;  // the candidates' rows were copied to p.cand_rows when they were sampled
     if (L.split) {
         const int vec_split = (n % L.split == 0) && (((uintptr_t)X_t) % 16 == 0);
-#define KMX_KPP_STEP_SPLIT_(SPT, LIT)                                                                  \
-    hipLaunchKernelGGL((kpp_step_split_kernel<T, 8, SPT, false, LIT>), dim3((unsigned)L.n_blocks),     \
+#define KMX_KPP_STEP_SPLIT_(TN, SPT, LIT)                                                              \
+    hipLaunchKernelGGL((kpp_step_split_kernel<T, TN, SPT, false, LIT>), dim3((unsigned)L.n_blocks),    \
                        dim3(256), 0, s, (const T*)X_t, (const T*)w, (const T*)p.cand_rows, (T*)p.rows, \
                        p.block_pot, p.header, n, d, 0, n_trials, vec_split, 0, (T*)nullptr,            \
                        (int32_t*)nullptr)
-#define KMX_KPP_STEP_SPLIT(SPT) \
-    do { if (literal) KMX_KPP_STEP_SPLIT_(SPT, true); else KMX_KPP_STEP_SPLIT_(SPT, false); } while (0)
-        if (L.split == 1) KMX_KPP_STEP_SPLIT(1);
-        else if (L.split == 2) KMX_KPP_STEP_SPLIT(2);
-        else KMX_KPP_STEP_SPLIT(4);
+#define KMX_KPP_STEP_SPLIT(TN, SPT) \
+    do { if (literal) KMX_KPP_STEP_SPLIT_(TN, SPT, true); else KMX_KPP_STEP_SPLIT_(TN, SPT, false); } while (0)
+        // (which of these exist is kpp_split's choice: the workgroup's partial distances within 32 KB)
+        if (n_trials <= 8) {
+            if (L.split == 1) KMX_KPP_STEP_SPLIT(8, 1);
+            else if (L.split == 2) KMX_KPP_STEP_SPLIT(8, 2);
+            else if constexpr (sizeof(T) == 4) KMX_KPP_STEP_SPLIT(8, 4);
+        } else {
+            if (L.split == 1) KMX_KPP_STEP_SPLIT(TN_MAX, 1);
+            else if constexpr (sizeof(T) == 4) KMX_KPP_STEP_SPLIT(TN_MAX, 2);
+        }
 #undef KMX_KPP_STEP_SPLIT
 #undef KMX_KPP_STEP_SPLIT_
         return;

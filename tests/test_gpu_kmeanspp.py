@@ -63,8 +63,12 @@ def test_whole_seeding_matches_oracle(cuda, name, sampler):
     assert idx.dtype == np.int32 and np.all((idx >= 0) & (idx < len(X)))
 
 
+# (n, d, local trials): the plain step; then few samples of many features, where a workgroup's
+# waves share the features - more than 8 trials at 2 samples per thread (fp32; fp64 keeps the
+# plain step there) and at 1, and 4 samples per thread (fp32 only)
+@pytest.mark.parametrize("shape", [(10_007, 6, 4), (66_001, 64, 12), (3_001, 70, 10), (140_000, 65, 3)])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-def test_step_kernels_through_c_abi(cuda, dtype):
+def test_step_kernels_through_c_abi(cuda, dtype, shape):
     """init -> sample -> step with the same uniforms as the oracle: candidates, potentials and
     the updated closest-distance array all match."""
     import torch
@@ -73,7 +77,7 @@ def test_step_kernels_through_c_abi(cuda, dtype):
     from sklearn_numba_dpex_amd._capi import lib, ptr
 
     rng = np.random.default_rng(3)
-    n, d, k, tn = 10_007, 6, 8, 4
+    (n, d, tn), k = shape, 8 if shape[0] < 20_000 else 4
     X = rng.normal(size=(n, d)).astype(dtype)
     w = rng.uniform(0.5, 1.5, n).astype(dtype)
     dc = _capi.dtype_code(dtype)
@@ -83,7 +87,7 @@ def test_step_kernels_through_c_abi(cuda, dtype):
     ws_bytes = lib.kmx_kpp_workspace_bytes(n, d, k, tn, dc)
     ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=cuda)
     st = _capi.current_stream()
-    start = 4242
+    start = 4242 % n
     _capi.check(lib.kmx_kpp_init(ptr(X_t), ptr(w_d), start, ptr(centers_t), ptr(indices), ptr(ws), ws_bytes,
                                  n, d, k, tn, dc, 0, st), "kpp_init")
     closest = (((X - X[start]) ** 2).sum(axis=1, dtype=dtype) * w).astype(dtype)
