@@ -464,10 +464,31 @@ def other_shapes():
     fp64 with sums beyond LDS, more than 256 features.  Overlapping blobs (the labels keep
     changing), wall time per iteration over iterations 6-13 of the driver's loop."""
     return [one_shape(*spec) for spec in (("70000 x 784, 10 clusters, fp32", 70_000, 784, 10, np.float32),
+                                          ("70000 x 784, 24 clusters, fp32", 70_000, 784, 24, np.float32),
+                                          ("70000 x 784, 10 clusters, fp64", 70_000, 784, 10, np.float64),
                                           ("2e6 x 100, 10 clusters, fp32", 2_000_000, 100, 10, np.float32),
                                           ("1e6 x 100, 100 clusters, fp64", 1_000_000, 100, 100, np.float64),
                                           ("1e6 x 48, 64 clusters, fp64", 1_000_000, 48, 64, np.float64),
                                           ("1e5 x 300, 300 clusters, fp32", 100_000, 300, 300, np.float32))]
+
+
+def seeding_ms(X, k, reps=3):
+    """Median wall time of a whole kmeans++ seeding (default sampler) of k centres, unit weights."""
+    import torch
+
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    dev = torch.device("cuda:0")
+    X_t = torch.as_tensor(X, device=dev).T.contiguous()
+    w_d = torch.ones(X.shape[0], dtype=X_t.dtype, device=dev)
+    ts = []
+    for rep in range(reps + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        drivers.kmeans_plusplus(X_t, w_d, k, np.random.RandomState(rep))
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t0)
+    return float(np.median(ts[1:])) * 1e3
 
 
 def one_shape(name, n, d, k, dtype, reps=8):
@@ -482,7 +503,7 @@ def one_shape(name, n, d, k, dtype, reps=8):
     kms, variant, wall_ms = gpu_lloyd_step_time(cfg, reps, consecutive=True)
     s = np.dtype(dtype).itemsize
     log(f"[bench] {name}: variant {variant}, {wall_ms:.3f} ms/iter ({time.time() - t0:.1f}s incl. data)")
-    return {"shape": name, "kernel_variant": variant, "ms_per_iter": wall_ms,
+    return {"shape": name, "kernel_variant": variant, "ms_per_iter": wall_ms, "kmeanspp_ms": seeding_ms(X, k),
             "label_and_sum_kernels_ms": float(kms[0]), "reduce_and_finalize_ms": float(kms[1] + kms[2]),
             "TFLOPs": lloyd_flops(n, d, k) / (wall_ms * 1e-3) / 1e12,
             "X_bytes_per_iter_TBs": n * d * s / (wall_ms * 1e-3) / 1e12,
