@@ -197,20 +197,29 @@ __global__ __launch_bounds__(256) void euclidean_distances_reg_kernel(
     }
 }
 
-// Any d: a workgroup owns a tile of DT_S samples x DT_C centroids, a thread a 4 x 8 block of it;
-// the features are staged DT_K at a time through LDS (both arrays are feature-major, as the
+// Any d: a workgroup owns a tile of DT_S samples x DC centroids, a thread a 4 x (DC / 8) block of
+// it; the features are staged DT_K at a time through LDS (both arrays are feature-major, as the
 // tiles: a stage is a copy of rows, 128-bit loads where alignment allows), the next stage's
 // loads in flight during the arithmetic.  Per staged feature a thread reads its four samples
-// and eight centroids from LDS (the centroid reads are broadcasts) and updates 32 sums with a
+// and its centroids from LDS (the centroid reads are broadcasts) and updates its sums with a
 // difference and a fused multiply-add each, features in order: vector-ALU bound.
-constexpr int DT_S = 128, DT_C = 64, DT_K = 16;
+// DC = 64, or 16 for up to 32 clusters: with 10 clusters a tile of 64 is five sixths padding,
+// and the kernel took ten times what reading X takes.
+constexpr int DT_S = 128, DT_C = 64, DT_C_FEW = 16, DT_K = 16;
+
+// 128-bit vectors per thread of a staged tile of COLS columns (fewer vectors than threads: the
+// first threads take one)
+template <typename T, int COLS>
+constexpr int dt_vectors() {
+    return (DT_K * (COLS / (16 / (int)sizeof(T))) + 255) / 256;
+}
 
 template <typename T, int COLS>
 __device__ __forceinline__ void dt_stage_load(T (*regs)[16 / sizeof(T)], const T* __restrict__ base, int64_t len,
                                               int64_t c0, int d, int f0, bool vec_ok) {
     constexpr int V = 16 / sizeof(T);                 // elements per 128-bit vector
     constexpr int PER_ROW = COLS / V;                 // vectors per staged row
-    constexpr int N = DT_K * PER_ROW / 256;           // vectors per thread
+    constexpr int N = dt_vectors<T, COLS>();          // vectors per thread
 #pragma unroll
     for (int l = 0; l < N; ++l) {
         const int g = threadIdx.x + 256 * l;
@@ -218,7 +227,7 @@ __device__ __forceinline__ void dt_stage_load(T (*regs)[16 / sizeof(T)], const T
         const int64_t c = c0 + (int64_t)V * (g % PER_ROW);
 #pragma unroll
         for (int e = 0; e < V; ++e) regs[l][e] = T(0);
-        if (f < d) {
+        if (f < d && g < DT_K * PER_ROW) {
             const T* __restrict__ src = base + (size_t)f * (size_t)len + c;
             if (vec_ok && c + V <= len) {
                 using Vec = typename std::conditional<sizeof(T) == 4, float4, double2>::type;
@@ -242,54 +251,57 @@ template <typename T, int COLS>
 __device__ __forceinline__ void dt_stage_store(T (*tile)[COLS], const T (*regs)[16 / sizeof(T)]) {
     constexpr int V = 16 / sizeof(T);
     constexpr int PER_ROW = COLS / V;
-    constexpr int N = DT_K * PER_ROW / 256;
+    constexpr int N = dt_vectors<T, COLS>();
 #pragma unroll
     for (int l = 0; l < N; ++l) {
         const int g = threadIdx.x + 256 * l;
+        if (g < DT_K * PER_ROW) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) tile[g / PER_ROW][V * (g % PER_ROW) + e] = regs[l][e];
+            for (int e = 0; e < V; ++e) tile[g / PER_ROW][V * (g % PER_ROW) + e] = regs[l][e];
+        }
     }
 }
 
-template <typename T>
+template <typename T, int DC>
 __global__ __launch_bounds__(256) void euclidean_distances_tiled_kernel(
     const T* __restrict__ X_t, const T* __restrict__ centroids_t, T* __restrict__ distances_t,
     int64_t n, int d, int k, int x_vec, int c_vec, int out_vec) {
     constexpr int V = 16 / sizeof(T);
+    constexpr int CT = DC / 8;  // centroids per thread
     __shared__ __align__(16) T xs[DT_K][DT_S];
-    __shared__ __align__(16) T cs[DT_K][DT_C];
+    __shared__ __align__(16) T cs[DT_K][DC];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int64_t i0 = (int64_t)blockIdx.x * DT_S;
-    const int c0 = blockIdx.y * DT_C;
-    T rx[DT_K * DT_S / V / 256][V], rc[DT_K * DT_C / V / 256][V];
-    T acc[8][4];
+    const int c0 = blockIdx.y * DC;
+    T rx[dt_vectors<T, DT_S>()][V], rc[dt_vectors<T, DC>()][V];
+    T acc[CT][4];
 #pragma unroll
-    for (int c = 0; c < 8; ++c)
+    for (int c = 0; c < CT; ++c)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[c][i] = T(0);
 
     dt_stage_load<T, DT_S>(rx, X_t, n, i0, d, 0, x_vec != 0);
-    dt_stage_load<T, DT_C>(rc, centroids_t, k, c0, d, 0, c_vec != 0);
+    dt_stage_load<T, DC>(rc, centroids_t, k, c0, d, 0, c_vec != 0);
     const int n_stages = (d + DT_K - 1) / DT_K;
     for (int st = 0; st < n_stages; ++st) {
         __syncthreads();  // the previous stage's reads are over
         dt_stage_store<T, DT_S>(xs, rx);
-        dt_stage_store<T, DT_C>(cs, rc);
+        dt_stage_store<T, DC>(cs, rc);
         __syncthreads();
         if (st + 1 < n_stages) {
             dt_stage_load<T, DT_S>(rx, X_t, n, i0, d, (st + 1) * DT_K, x_vec != 0);
-            dt_stage_load<T, DT_C>(rc, centroids_t, k, c0, d, (st + 1) * DT_K, c_vec != 0);
+            dt_stage_load<T, DC>(rc, centroids_t, k, c0, d, (st + 1) * DT_K, c_vec != 0);
         }
         // (rows past d hold zeros on both sides: their differences add nothing)
 #pragma unroll
         for (int kk = 0; kk < DT_K; ++kk) {
-            T xv[4], cv[8];
+            T xv[4], cv[CT];
 #pragma unroll
             for (int i = 0; i < 4; ++i) xv[i] = xs[kk][4 * tx + i];
 #pragma unroll
-            for (int c = 0; c < 8; ++c) cv[c] = cs[kk][8 * ty + c];
+            for (int c = 0; c < CT; ++c) cv[c] = cs[kk][CT * ty + c];
 #pragma unroll
-            for (int c = 0; c < 8; ++c)
+            for (int c = 0; c < CT; ++c)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const T diff = cv[c] - xv[i];
@@ -299,8 +311,8 @@ __global__ __launch_bounds__(256) void euclidean_distances_tiled_kernel(
     }
     const int64_t i = i0 + 4 * tx;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        const int cc = c0 + 8 * ty + c;
+    for (int c = 0; c < CT; ++c) {
+        const int cc = c0 + CT * ty + c;
         if (cc >= k) continue;
         T* __restrict__ dst = distances_t + (size_t)cc * (size_t)n + i;
         if (sizeof(T) == 4 && out_vec && i + 4 <= n) {
@@ -482,17 +494,19 @@ int32_t kmx_euclidean_distances(const void* X_t, const void* centroids_t, void* 
                            (const double*)X_t, (const double*)centroids_t, (double*)distances_t, n, d, k, vec_ok,
                            c_chunk);
     } else {
-        const dim3 tgrid((unsigned)kmx_cdiv(n, DT_S), (unsigned)kmx_cdiv(k, DT_C));
+        const int dc = k <= 2 * DT_C_FEW ? DT_C_FEW : DT_C;
+        const dim3 tgrid((unsigned)kmx_cdiv(n, DT_S), (unsigned)kmx_cdiv(k, dc));
         const int per_vec = (int)(16 / es);
         const int x_vec = (n % per_vec == 0) && al16(X_t), c_vec = (k % per_vec == 0) && al16(centroids_t);
-        if (dtype == KMX_F32)
-            hipLaunchKernelGGL((euclidean_distances_tiled_kernel<float>), tgrid, dim3(256), 0, stream,
-                               (const float*)X_t, (const float*)centroids_t, (float*)distances_t, n, d, k, x_vec,
-                               c_vec, vec_ok);
-        else
-            hipLaunchKernelGGL((euclidean_distances_tiled_kernel<double>), tgrid, dim3(256), 0, stream,
-                               (const double*)X_t, (const double*)centroids_t, (double*)distances_t, n, d, k,
-                               x_vec, c_vec, 0);
+#define KMX_DIST_TILED(T, DC, OUT_VEC)                                                                 \
+    hipLaunchKernelGGL((euclidean_distances_tiled_kernel<T, DC>), tgrid, dim3(256), 0, stream,         \
+                       (const T*)X_t, (const T*)centroids_t, (T*)distances_t, n, d, k, x_vec, c_vec, OUT_VEC)
+        if (dtype == KMX_F32) {
+            if (dc == DT_C_FEW) KMX_DIST_TILED(float, DT_C_FEW, vec_ok); else KMX_DIST_TILED(float, DT_C, vec_ok);
+        } else {
+            if (dc == DT_C_FEW) KMX_DIST_TILED(double, DT_C_FEW, 0); else KMX_DIST_TILED(double, DT_C, 0);
+        }
+#undef KMX_DIST_TILED
     }
     KMX_LAUNCH_CHECK();
     return KMX_OK;

@@ -309,7 +309,10 @@ def test_label_helpers(cuda):
 @pytest.mark.parametrize("shape", [(1003, 14, 127, np.float32), (4096, 32, 7, np.float32), (777, 33, 5, np.float32),
                                    (1001, 16, 9, np.float64), (500, 17, 3, np.float64), (1000, 300, 50, np.float32),
                                    (3, 2, 2, np.float64), (1000, 70, 130, np.float64), (1028, 100, 64, np.float32),
-                                   (515, 129, 67, np.float32), (1026, 48, 66, np.float64)])
+                                   (515, 129, 67, np.float32), (1026, 48, 66, np.float64),
+                                   # few clusters of wide samples: centroid tiles of 16 (one, two), then of 64
+                                   (1001, 784, 10, np.float32), (1030, 200, 20, np.float64),
+                                   (1000, 65, 32, np.float32), (1000, 65, 33, np.float32)])
 def test_distances_and_inertia_kernels(cuda, shape):
     import torch
 
