@@ -64,7 +64,7 @@ KppLayout kpp_layout(int64_t n, int d, int n_trials, int dtype) {
     L.off_header = 0;
     L.off_cand = 256;
     L.off_pot = 512;
-    L.off_cand_rows = 768;  // (TN_MAX, d): the candidates' feature rows, read through scalar loads
+    L.off_cand_rows = 768;  // (TN_MAX, d): the candidates' feature rows, read by the step kernel a batch at a time
     L.off_block_pot = L.off_cand_rows + kmx_align256((size_t)TN_MAX * d * kmx_dtype_size(dtype));
     L.off_rows = L.off_block_pot + kmx_align256((size_t)L.n_blocks * TN_MAX * sizeof(double));
     L.total = L.off_rows + kmx_align256((size_t)n_trials * n * kmx_dtype_size(dtype));
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256) void kpp_step_split_kernel(
     constexpr int S = 64 * SPT;
     __shared__ T part[4][TN][S];
     // the wave index as a scalar: the feature loop's bounds and the candidates' rows are then
-    // wave-uniform for the compiler as well (scalar loads, no branch per feature)
+    // wave-uniform for the compiler as well (scalar branches, no lane masks per feature)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t base = (int64_t)blockIdx.x * S;
     const int64_t i0 = base + lane * SPT;
@@ -633,7 +633,7 @@ __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
         cand_next[trial] = (int32_t)cand;
         if (cand_out) cand_out[trial] = (int32_t)cand;
     }
-    // the candidate's feature row, for the step kernel's scalar loads
+    // the candidate's feature row, for the step kernel
     for (int f = threadIdx.x; f < d; f += 256) cand_rows[(size_t)trial * d + f] = X_t[(size_t)f * n + cand];
 }
 
