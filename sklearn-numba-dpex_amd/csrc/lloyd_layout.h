@@ -212,10 +212,15 @@ static inline LloydLayout lloyd_layout(int64_t n, int d, int k, int dtype, uint3
         // fit in LDS, else the tiled product -- then bucketed sums.  Up to 16 clusters with
         // accumulators in LDS: the fused vector-ALU kernels.
         const bool matrix_ok = forced < 0 || forced == KMX_VARIANT_MFMA || forced == KMX_VARIANT_GEMM;
+        // (fp64 beyond 64 features: the streaming kernel reads X twice with a thread per two
+        // samples walking every feature; below a million samples the tiled product + bucketed
+        // sums take 1.0 to 4 times less - 20 000 x 400, k = 10: 0.38 -> 0.09 ms -, above it
+        // 10 to 20 % more)
+        const bool stream_short_f64 = forced < 0 && dtype == KMX_F64 && L.variant == KMX_VARIANT_STREAM && n < 1000000;
         if (forced == KMX_VARIANT_GEMM) {
             L.variant = KMX_VARIANT_GEMM;
             L.acc_mode = KMX_ACC_BUCKET;
-        } else if (matrix_ok && (k > 16 || L.acc_mode == KMX_ACC_GLOBAL)) {
+        } else if (matrix_ok && (k > 16 || L.acc_mode == KMX_ACC_GLOBAL || stream_short_f64)) {
             L.variant = (dtype == KMX_F64 && kmx_mfma_f64_labels_supported(d, k)) ? KMX_VARIANT_MFMA_F64
                                                                                  : KMX_VARIANT_GEMM;
             L.acc_mode = KMX_ACC_BUCKET;

@@ -125,6 +125,10 @@ def test_kernel_variant_selection():
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 256, 1024, 0, 0) == 42  # wide MFMA + global sums
     assert lib.kmx_lloyd_kernel_variant(1_000_000, 300, 1024, 0, 0) == 63  # tiled matrix-core labels + bucketed sums
     assert lib.kmx_lloyd_kernel_variant(1000, 3, 5, 0, 0) == 11           # too few clusters for MFMA
+    # fp64, few clusters of wide samples: streamed twice from a million samples on, else the tiled product
+    assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 1, 0) == 1
+    assert lib.kmx_lloyd_kernel_variant(200_000, 100, 10, 1, 0) == 63
+    assert lib.kmx_lloyd_kernel_variant(200_000, 100, 10, 1, 0x1) == 1
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 64, 0, 0) == 63    # the wide path only beyond 256 clusters
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 300, 0, 0) == 42
     assert lib.kmx_lloyd_kernel_variant(2_000_000, 100, 10, 0, 0) == 81    # few clusters, wide samples: one read of X

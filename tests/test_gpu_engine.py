@@ -415,7 +415,7 @@ def test_numpy_inputs_are_uploaded_through_pinned_staging(cuda):
                                    (6_000, 70, 300, np.float32, 42),
                                    (6_000, 300, 40, np.float32, 63), (6_000, 100, 100, np.float64, 63),
                                    (20_000, 32, 400, np.float64, 53), (20_000, 100, 10, np.float32, 81),
-                                   (20_000, 100, 10, np.float64, 1),
+                                   (20_000, 100, 10, np.float64, 63), (1_000_000, 66, 4, np.float64, 1),
                                    (20_000, 20, 8, np.float64, 11), (1_500, 784, 10, np.float32, 81),
                                    (6_000, 300, 20, np.float32, 63)])
 def test_fit_follows_scikit_learn_on_every_kernel_family(cuda, shape):

@@ -69,7 +69,9 @@ def _small_configs():
         # few clusters: the register-resident and the streaming vector-ALU steps
         "R64a": lambda: dict(_blob_config(5_003, 50, 7, np.float64, 34), variant=11),
         "R32a": lambda: dict(_blob_config(5_003, 40, 8, np.float32, 35), variant=11),
-        "S64a": lambda: dict(_blob_config(5_002, 90, 16, np.float64, 36), variant=1),
+        "S64a": lambda: dict(_blob_config(5_002, 90, 16, np.float64, 36), flags=0x1, variant=1),
+        # (fp64 below a million samples leaves the streaming step to the tiled product by itself)
+        "S64c": lambda: dict(_blob_config(5_002, 90, 16, np.float64, 36), variant=63),
         "S32a": lambda: dict(_blob_config(300_000, 70, 5, np.float32, 37), flags=0x1, variant=1),
         # enough samples for four (fp32) / two (fp64) consecutive samples per thread
         "S32b": lambda: dict(_blob_config(600_000, 70, 5, np.float32, 38), flags=0x1, variant=1),
@@ -102,7 +104,7 @@ def _small_configs():
         "K32s": lambda: dict(_blob_config(2_003, 1500, 16, np.float32, 65), variant=81),
         # enough samples for the labels-only kernel with a tile per wave, n odd (no 128-bit accesses)
         "K32t": lambda: dict(_blob_config(270_001, 96, 7, np.float32, 66), variant=81),
-        "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), variant=1),
+        "S64b": lambda: dict(_blob_config(300_000, 70, 5, np.float64, 39), flags=0x1, variant=1),
         # extremes of the tiled product: thousands of features (many passes of the bucketed sums),
         # more clusters than the bucket counts hold in LDS and than the wide path takes
         "X32a": lambda: dict(_blob_config(1_500, 3_000, 20, np.float32, 40), variant=63),
@@ -153,7 +155,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "B64h", "R64a", "R32a", "S64a", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
+                                  "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "B64h", "R64a", "R32a", "S64a", "S64c", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
                                   "K32a", "K32b", "K32c", "K32d", "K32e", "K32f", "K32g", "K32h", "K32i",
                                   "K32j", "K32k", "K32l", "K32m", "K32n", "K32o", "K32p", "K32q", "K32r", "K32s"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
