@@ -213,7 +213,9 @@ def test_score_path_and_topk_at_full_size(cuda):
                                    (500_000, 300, 300, np.float32, 63), (2_000_000, 100, 10, np.float32, 81),
                                    (2_000_000, 100, 10, np.float64, 1), (300_000, 784, 10, np.float32, 81),
                                    (2_000_000, 48, 64, np.float32, 61), (1_000_000, 64, 128, np.float64, 51),
-                                   (2_000_000, 48, 64, np.float64, 71)])
+                                   (2_000_000, 48, 64, np.float64, 71),
+                                   # the tiled product with centroid tiles of 32 and stages of twice the features
+                                   (1_000_000, 200, 24, np.float32, 63), (500_000, 200, 10, np.float64, 63)])
 def test_large_shapes_off_the_benchmark_configurations(cuda, shape):
     """The same properties on large inputs of the other kernel families: the tiled matrix-core
     product and the fp64 matrix-core labels with bucketed sums, the few-cluster step (per-wave and
