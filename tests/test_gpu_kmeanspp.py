@@ -66,6 +66,27 @@ def test_whole_seeding_matches_oracle(cuda, name, sampler):
 # (n, d, local trials): the plain step; then few samples of many features, where a workgroup's
 # waves share the features - more than 8 trials at 2 samples per thread (fp32; fp64 keeps the
 # plain step there) and at 1, and 4 samples per thread (fp32 only)
+@pytest.mark.parametrize("sampler", ["scan", "literal"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d", [(65_536, 64), (65_537, 64), (131_072, 64), (131_073, 65), (262_144, 64), (262_145, 64),
+                                 (70_000, 63), (1, 64), (63, 64), (65, 80)])
+def test_seeding_at_the_limits_of_the_feature_split_step(cuda, n, d, dtype, sampler):
+    """Sample counts either side of where the step changes its samples per thread (65 536,
+    131 072, 262 144; fp64 stops one earlier), one feature short of the split, and arrays of one
+    sample, of less than a wave and of one more than a wave: indices equal to the oracle's."""
+    from sklearn_numba_dpex_amd.kmeans import drivers
+
+    rng = np.random.default_rng(n + d)
+    X = rng.normal(size=(n, d)).astype(dtype)
+    w = rng.uniform(0.5, 1.5, n).astype(dtype)
+    k = min(3, n)
+    centers_t, idx = drivers.kmeans_plusplus(_dev(X.T, cuda), _dev(w, cuda), k, np.random.RandomState(n % 97), sampler=sampler)
+    seed64 = orng.seed_from_random_state(np.random.RandomState(n % 97))
+    ref_idx = ok.kmeans_plusplus(X, w, k, seed64, sampler="exact" if sampler == "scan" else "literal")[1]
+    np.testing.assert_array_equal(idx.cpu().numpy(), ref_idx)
+    np.testing.assert_array_equal(centers_t.cpu().numpy().T, X[ref_idx])
+
+
 @pytest.mark.parametrize("shape", [(10_007, 6, 4), (66_001, 64, 12), (3_001, 70, 10), (140_000, 65, 3)])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_step_kernels_through_c_abi(cuda, dtype, shape):
