@@ -64,6 +64,15 @@ def _small_configs():
         "B32c": lambda: dict(_blob_config(5_001, 300, 20, np.float32, 31), variant=63),
         "B64f": lambda: dict(_blob_config(4_000, 100, 24, np.float64, 32), variant=63),
         "B64g": lambda: dict(_blob_config(4_003, 90, 50, np.float64, 33), variant=63),
+        # cluster counts either side of where the tiled product widens its centroid tile (32, 64)
+        "B32d": lambda: dict(_blob_config(3_001, 300, 32, np.float32, 68), variant=63),
+        "B32e": lambda: dict(_blob_config(3_001, 300, 33, np.float32, 69), variant=63),
+        "B32f": lambda: dict(_blob_config(2_000, 200, 64, np.float32, 70), variant=63),
+        "B32g": lambda: dict(_blob_config(2_000, 200, 65, np.float32, 71), variant=63),
+        "B64i": lambda: dict(_blob_config(2_001, 150, 32, np.float64, 72), variant=63),
+        "B64j": lambda: dict(_blob_config(2_001, 150, 33, np.float64, 73), variant=63),
+        "B64k": lambda: dict(_blob_config(1_500, 100, 64, np.float64, 74), variant=63),
+        "B64l": lambda: dict(_blob_config(1_500, 100, 65, np.float64, 75), variant=63),
         # few clusters of wide fp64 samples: the finalisation with 64 lanes per cluster
         "B64h": lambda: dict(_blob_config(3_001, 300, 18, np.float64, 67, skew=True), variant=63),
         # few clusters: the register-resident and the streaming vector-ALU steps
@@ -155,7 +164,7 @@ def _odd_config():
 @pytest.mark.parametrize("rowmajor", [False, True])
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C3s", "C3m", "C3w", "C5", "odd", "F64a", "F64b", "F64c",
                                   "M32a", "M32b", "M32c", "C3k", "M32d", "M32e", "M32f", "M32g", "F64d", "F64e", "F64f",
-                                  "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "B64h", "R64a", "R32a", "S64a", "S64c", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
+                                  "F64g", "F64h", "F64e1", "F64h1", "C5f", "F64i", "F64j", "B64a", "B64b", "B32a", "B32b", "B64c", "B64d", "B64e", "C3k2", "B32c", "B64f", "B64g", "B64h", "B32d", "B32e", "B32f", "B32g", "B64i", "B64j", "B64k", "B64l", "R64a", "R32a", "S64a", "S64c", "S32a", "S32b", "S64b", "X32a", "X32b", "X64a", "G32s", "G32t", "G32u",
                                   "K32a", "K32b", "K32c", "K32d", "K32e", "K32f", "K32g", "K32h", "K32i",
                                   "K32j", "K32k", "K32l", "K32m", "K32n", "K32o", "K32p", "K32q", "K32r", "K32s"])
 def test_single_iteration_through_c_abi(cuda, name, rowmajor):
@@ -493,7 +502,7 @@ def n_samples_differ_cap(X):
     return X.shape[0] // 1000
 
 
-@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "F64h", "F64i", "F64j", "C5", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "B64h", "R64a", "R32a", "S64a", "S32a",
+@pytest.mark.parametrize("name", ["C3s", "C3w", "C3k2", "F64d", "F64e", "F64h", "F64i", "F64j", "C5", "B64a", "B64b", "B32a", "B32b", "B64c", "odd", "B32c", "B64f", "B64g", "B64h", "B32d", "B32e", "B32f", "B32g", "B64i", "B64j", "B64k", "B64l", "R64a", "R32a", "S64a", "S32a",
                                   # few clusters on wide samples: the labels-only matrix-core kernel that reads
                                   # the feature-major array directly (tiles of 32 and of 64 samples, every width
                                   # of its centroid registers, n odd, n below a tile) and the inertia summed
