@@ -459,9 +459,8 @@ __device__ __forceinline__ int64_t block_min_i64(int64_t v, int64_t* scratch) {
 //              candidate's feature row for the step kernel.
 // Thread i owns the block sums [i * P, (i + 1) * P); with P <= KPP_OWN they are read once and
 // stay in registers for the row totals, the coarse scan and the search.
-constexpr int KPP_OWN = 4;
-
-template <typename T, int TN>
+// (KPP_OWN = 4 covers a million samples; 8, for up to 8 trials, two million)
+template <typename T, int TN, int KPP_OWN = 4>
 __global__ __launch_bounds__(256) void kpp_select_sample_kernel(
     const T* __restrict__ X_t, const double* __restrict__ uniforms,
     const int32_t* __restrict__ cand_prev, int32_t* __restrict__ cand_next,
@@ -886,15 +885,18 @@ void launch_select_sample(const void* X_t, const double* uniforms, const int32_t
     // one workgroup per trial when sampling, one more when a selection is recorded
     const unsigned grid = (do_sample ? (unsigned)n_trials : 0u) + (do_select ? 1u : 0u);
     if (grid == 0) return;
-#define KMX_KPP_SELECT(TN)                                                                        \
-    hipLaunchKernelGGL((kpp_select_sample_kernel<T, TN>), dim3(grid), dim3(256), 0, s,             \
+#define KMX_KPP_SELECT(...)                                                                       \
+    hipLaunchKernelGGL((kpp_select_sample_kernel<T, __VA_ARGS__>), dim3(grid), dim3(256), 0, s,    \
                        (const T*)X_t, uniforms, cand_prev, cand_next, cand_out, (T*)centers_t, idx, \
                        (const T*)p.rows, p.block_pot, p.potentials, p.header, (T*)p.cand_rows, n,   \
                        L.n_blocks, L.chunk, d, k, n_trials, slot, do_select, do_sample)
-    if (n_trials <= 8)
-        KMX_KPP_SELECT(8);
-    else
+    if (n_trials <= 8) {
+        // (more than four block sums per thread: eight in registers rather than re-read)
+        if (L.n_blocks > 4 * 256 && L.n_blocks <= 8 * 256) KMX_KPP_SELECT(8, 8);
+        else KMX_KPP_SELECT(8);
+    } else {
         KMX_KPP_SELECT(TN_MAX);
+    }
 #undef KMX_KPP_SELECT
 }
 
